@@ -1,0 +1,1184 @@
+// TEST INFRASTRUCTURE ONLY -- CPU restatement of the HCCL per-rank data path.
+//
+// This file is the checker the HIP library is compared against.  It is never linked into, loaded
+// by, or called from the product library; only tests, the smoke check and the CPU-baseline leg of
+// the benchmark may use it.
+//
+// What it restates (paths relative to the reference tree; ALG = src/domain/collective_communication/
+// algorithm, TPL = ALG/base/alg_template, EXE = ALG/impl/coll_executor):
+//   slice plans      TPL/temp_all_reduce/all_reduce_ring.cc:119-130, TPL/recursive_halvingdoubling_base.cc:23-94,
+//                    EXE/coll_comm_executor.cc:1681-1721 (piece cut used for the mesh streams)
+//   chunk loops      EXE/coll_all_reduce/coll_all_reduce_executor.cc:86-93,155-272,
+//                    EXE/coll_reduce_scatter/coll_reduce_scatter_executor.cc:83-90,118-245,
+//                    EXE/coll_all_gather/coll_all_gather_executor.cc:79-87,109-193
+//   ring             TPL/temp_reduce_scatter/reduce_scatter_ring.cc:89-297, TPL/temp_all_gather/all_gather_ring.cc:51-171,
+//                    TPL/temp_all_reduce/all_reduce_ring.cc:32-53,143-191
+//   mesh             TPL/temp_reduce_scatter/reduce_scatter_mesh.cc:57-203, TPL/temp_all_gather/all_gather_mesh.cc:91-253,
+//                    EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240, EXE/coll_comm_executor.cc:1458-1574
+//   halving-doubling TPL/temp_all_reduce/all_reduce_recursive_hd.cc:33-302,
+//                    TPL/temp_reduce_scatter/reduce_scatter_halving_doubling.cc:67-238,
+//                    TPL/temp_all_gather/all_gather_halving_doubling.cc:43-196
+//   pairwise         TPL/temp_alltoallv/alltoallv_pairwise.cc:75-282, ALG/impl/operator/alltoall_operator.cc:49-72
+//
+// Method: every template is restated as the per-rank program it issues (send / receive-and-reduce /
+// receive-and-copy / local copy), one virtual process per rank (per rank and stream for the mesh),
+// and the programs are run by a message-passing machine with FIFO mailboxes.  A message is a
+// snapshot of the sender's bytes at send time ("snapshot" mode) or a pointer into the sender's
+// buffer ("direct" mode, which is what an inline-reduce link does; it is valid because no template
+// rewrites a range after sending it, and the tests check both modes agree).
+//
+// Parity status.  The reference ships no tests, golden vectors or fixtures for this path, and its
+// leaf arithmetic (Reducer / Sender / Transport) is in closed libraries, so every function here is
+// pinned by mathematics only: closed-form reduction chains and trees, order-independent integer
+// results, permutation closed forms for gather / all-to-all, and hand-derived slice-plan vectors
+// (tests/golden).  Assumptions that only a run of the closed reference could confirm -- PARITY
+// UNPINNED for these: the slice alignment constant (128 bytes), the element sizes, the direction of
+// ForwardRank / BackwardRank (forced by all_gather_ring.cc:130-163), the piece cut of
+// PrepareSliceMeshStreams (taken equal to coll_comm_executor.cc:1681-1721), the operand order and
+// the NaN / signed-zero behaviour inside the closed Reducer, and the accumulation width for
+// fp16 / bf16 (here: fp32, rounded to nearest-even after every stored step).
+#include <algorithm>
+#include <atomic>
+#include <condition_variable>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <functional>
+#include <map>
+#include <mutex>
+#include <thread>
+#include <tuple>
+#include <vector>
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------
+// Types (values follow inc/hccl/hccl_types.h:58-87)
+// ------------------------------------------------------------------------------------------------
+enum { DT_INT8 = 0, DT_INT16 = 1, DT_INT32 = 2, DT_FP16 = 3, DT_FP32 = 4, DT_INT64 = 5, DT_UINT64 = 6,
+       DT_UINT8 = 7, DT_UINT16 = 8, DT_UINT32 = 9, DT_FP64 = 10, DT_BF16 = 11, DT_INT128 = 12 };
+enum { OP_SUM = 0, OP_PROD = 1, OP_MAX = 2, OP_MIN = 3 };
+enum { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2 };
+
+size_t DtSize(int dt)
+{
+    static const size_t table[] = {1, 2, 4, 2, 4, 8, 8, 1, 2, 4, 8, 2, 16, 1, 1, 1};
+    return (dt >= 0 && dt < 16) ? table[dt] : 0;
+}
+
+struct Slice { uint64_t off; uint64_t size; };
+
+// ------------------------------------------------------------------------------------------------
+// 16-bit float conversions (round to nearest even; NaN stays NaN, quiet bit set)
+// ------------------------------------------------------------------------------------------------
+inline uint32_t F2U(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
+inline float U2F(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+
+inline float Bf16ToF32(uint16_t b) { return U2F(static_cast<uint32_t>(b) << 16); }
+inline uint16_t F32ToBf16(float f)
+{
+    uint32_t u = F2U(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        return static_cast<uint16_t>((u >> 16) | 0x0040u);
+    }
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return static_cast<uint16_t>(u >> 16);
+}
+
+inline float Fp16ToF32(uint16_t h)
+{
+    uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    if (exp == 0) {
+        if (man == 0) {
+            return U2F(sign);
+        }
+        // subnormal half: value = man * 2^-24
+        float v = static_cast<float>(man) * 5.9604644775390625e-08f;
+        return U2F(F2U(v) | sign);
+    }
+    if (exp == 31) {
+        return U2F(sign | 0x7f800000u | (man << 13));
+    }
+    return U2F(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+inline uint16_t F32ToFp16(float f)
+{
+    uint32_t u = F2U(f);
+    uint16_t sign = static_cast<uint16_t>((u >> 16) & 0x8000u);
+    uint32_t abs = u & 0x7fffffffu;
+    if (abs > 0x7f800000u) {
+        return static_cast<uint16_t>(sign | 0x7e00u | ((abs >> 13) & 0x3ffu));
+    }
+    if (abs >= 0x47800000u) {  // >= 65536 -> inf (65520 rounds to inf below through the normal path)
+        return static_cast<uint16_t>(sign | 0x7c00u);
+    }
+    if (abs < 0x38800000u) {   // below the smallest normal half (2^-14): subnormal or zero
+        if (abs < 0x33000000u) {  // < 2^-25 rounds to zero (2^-25 itself ties to even = 0)
+            return sign;
+        }
+        // value = m * 2^-24 with m in [0.5, 1024); round m to nearest even integer
+        uint32_t e = abs >> 23;
+        uint32_t m = (abs & 0x7fffffu) | 0x800000u;
+        uint32_t shift = 126u - e;          // e in [102,112] -> shift in [14,24]
+        uint32_t q = m >> shift;
+        uint32_t rem = m & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1u);
+        if (rem > half || (rem == half && (q & 1u))) {
+            q++;
+        }
+        return static_cast<uint16_t>(sign | q);
+    }
+    uint32_t lsb = (abs >> 13) & 1u;
+    abs += 0xfffu + lsb;
+    uint32_t h = (abs - 0x38000000u) >> 13;
+    if (h >= 0x7c00u) {
+        h = 0x7c00u;
+    }
+    return static_cast<uint16_t>(sign | h);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Element reduction: dst = a (+) b, where a is the local operand and b the received one.
+//   sum / prod : integers wrap modulo 2^n (computed unsigned); floats use one IEEE operation
+//   max        : (b > a) ? b : a          min : (b < a) ? b : a
+// fp16 / bf16 operands are widened to fp32, combined, and rounded back (max / min keep the bits of
+// the chosen operand).
+// ------------------------------------------------------------------------------------------------
+template <typename T, typename U> inline T IntOp(int op, T a, T b)
+{
+    switch (op) {
+        case OP_SUM: return static_cast<T>(static_cast<U>(static_cast<U>(a) + static_cast<U>(b)));
+        case OP_PROD: return static_cast<T>(static_cast<U>(static_cast<U>(a) * static_cast<U>(b)));
+        case OP_MAX: return (b > a) ? b : a;
+        default: return (b < a) ? b : a;
+    }
+}
+// 16-bit unsigned products promote to int and could overflow it: multiply in 32-bit unsigned.
+template <> inline int16_t IntOp<int16_t, uint16_t>(int op, int16_t a, int16_t b)
+{
+    switch (op) {
+        case OP_SUM: return static_cast<int16_t>(static_cast<uint16_t>(static_cast<uint32_t>(static_cast<uint16_t>(a)) + static_cast<uint16_t>(b)));
+        case OP_PROD: return static_cast<int16_t>(static_cast<uint16_t>(static_cast<uint32_t>(static_cast<uint16_t>(a)) * static_cast<uint16_t>(b)));
+        case OP_MAX: return (b > a) ? b : a;
+        default: return (b < a) ? b : a;
+    }
+}
+template <> inline uint16_t IntOp<uint16_t, uint16_t>(int op, uint16_t a, uint16_t b)
+{
+    switch (op) {
+        case OP_SUM: return static_cast<uint16_t>(static_cast<uint32_t>(a) + b);
+        case OP_PROD: return static_cast<uint16_t>(static_cast<uint32_t>(a) * b);
+        case OP_MAX: return (b > a) ? b : a;
+        default: return (b < a) ? b : a;
+    }
+}
+template <typename T> inline T FloatOp(int op, T a, T b)
+{
+    switch (op) {
+        case OP_SUM: return a + b;
+        case OP_PROD: return a * b;
+        case OP_MAX: return (b > a) ? b : a;
+        default: return (b < a) ? b : a;
+    }
+}
+template <typename T, typename F> void LoopT(void *dst, const void *a, const void *b, size_t n, F f)
+{
+    T *d = static_cast<T *>(dst);
+    const T *x = static_cast<const T *>(a);
+    const T *y = static_cast<const T *>(b);
+    for (size_t i = 0; i < n; i++) {
+        d[i] = f(x[i], y[i]);
+    }
+}
+
+int ReduceElems(int dt, int op, void *dst, const void *a, const void *b, size_t n)
+{
+    switch (dt) {
+        case DT_INT8: LoopT<int8_t>(dst, a, b, n, [op](int8_t x, int8_t y) { return IntOp<int8_t, uint8_t>(op, x, y); }); return 0;
+        case DT_UINT8: LoopT<uint8_t>(dst, a, b, n, [op](uint8_t x, uint8_t y) { return IntOp<uint8_t, uint8_t>(op, x, y); }); return 0;
+        case DT_INT16: LoopT<int16_t>(dst, a, b, n, [op](int16_t x, int16_t y) { return IntOp<int16_t, uint16_t>(op, x, y); }); return 0;
+        case DT_UINT16: LoopT<uint16_t>(dst, a, b, n, [op](uint16_t x, uint16_t y) { return IntOp<uint16_t, uint16_t>(op, x, y); }); return 0;
+        case DT_INT32: LoopT<int32_t>(dst, a, b, n, [op](int32_t x, int32_t y) { return IntOp<int32_t, uint32_t>(op, x, y); }); return 0;
+        case DT_UINT32: LoopT<uint32_t>(dst, a, b, n, [op](uint32_t x, uint32_t y) { return IntOp<uint32_t, uint32_t>(op, x, y); }); return 0;
+        case DT_INT64: LoopT<int64_t>(dst, a, b, n, [op](int64_t x, int64_t y) { return IntOp<int64_t, uint64_t>(op, x, y); }); return 0;
+        case DT_UINT64: LoopT<uint64_t>(dst, a, b, n, [op](uint64_t x, uint64_t y) { return IntOp<uint64_t, uint64_t>(op, x, y); }); return 0;
+        case DT_FP32: LoopT<float>(dst, a, b, n, [op](float x, float y) { return FloatOp<float>(op, x, y); }); return 0;
+        case DT_FP64: LoopT<double>(dst, a, b, n, [op](double x, double y) { return FloatOp<double>(op, x, y); }); return 0;
+        case DT_FP16:
+            LoopT<uint16_t>(dst, a, b, n, [op](uint16_t x, uint16_t y) -> uint16_t {
+                float fx = Fp16ToF32(x), fy = Fp16ToF32(y);
+                if (op == OP_SUM) return F32ToFp16(fx + fy);
+                if (op == OP_PROD) return F32ToFp16(fx * fy);
+                if (op == OP_MAX) return (fy > fx) ? y : x;
+                return (fy < fx) ? y : x;
+            });
+            return 0;
+        case DT_BF16:
+            LoopT<uint16_t>(dst, a, b, n, [op](uint16_t x, uint16_t y) -> uint16_t {
+                float fx = Bf16ToF32(x), fy = Bf16ToF32(y);
+                if (op == OP_SUM) return F32ToBf16(fx + fy);
+                if (op == OP_PROD) return F32ToBf16(fx * fy);
+                if (op == OP_MAX) return (fy > fx) ? y : x;
+                return (fy < fx) ? y : x;
+            });
+            return 0;
+        default: return -1;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Thread pool: splits one byte range into element-aligned pieces (per-element order unchanged, so
+// the result does not depend on the thread count).
+// ------------------------------------------------------------------------------------------------
+class Pool {
+public:
+    explicit Pool(int n) : n_(n < 1 ? 1 : n)
+    {
+        for (int i = 1; i < n_; i++) {
+            workers_.emplace_back([this, i] { Work(i); });
+        }
+    }
+    ~Pool()
+    {
+        {
+            std::lock_guard<std::mutex> g(m_);
+            stop_ = true;
+            gen_++;
+        }
+        cv_.notify_all();
+        for (auto &t : workers_) {
+            t.join();
+        }
+    }
+    int Threads() const { return n_; }
+    // fn(begin, end) over [0, total) cut into n_ pieces of a multiple of `grain`.
+    void Run(uint64_t total, uint64_t grain, const std::function<void(uint64_t, uint64_t)> &fn)
+    {
+        if (n_ == 1 || total < (1u << 16)) {
+            fn(0, total);
+            return;
+        }
+        uint64_t units = (total + grain - 1) / grain;
+        uint64_t per = (units + n_ - 1) / n_ * grain;
+        {
+            std::lock_guard<std::mutex> g(m_);
+            fn_ = &fn;
+            total_ = total;
+            per_ = per;
+            pending_ = n_ - 1;
+            gen_++;
+        }
+        cv_.notify_all();
+        Piece(0);
+        std::unique_lock<std::mutex> g(m_);
+        done_.wait(g, [this] { return pending_ == 0; });
+    }
+
+private:
+    void Piece(int i)
+    {
+        uint64_t b = std::min<uint64_t>(total_, per_ * i);
+        uint64_t e = std::min<uint64_t>(total_, per_ * (i + 1));
+        if (e > b) {
+            (*fn_)(b, e);
+        }
+    }
+    void Work(int i)
+    {
+        uint64_t seen = 0;
+        for (;;) {
+            {
+                std::unique_lock<std::mutex> g(m_);
+                cv_.wait(g, [&] { return gen_ != seen; });
+                seen = gen_;
+                if (stop_) {
+                    return;
+                }
+            }
+            Piece(i);
+            {
+                std::lock_guard<std::mutex> g(m_);
+                pending_--;
+            }
+            done_.notify_one();
+        }
+    }
+    int n_;
+    std::vector<std::thread> workers_;
+    std::mutex m_;
+    std::condition_variable cv_, done_;
+    const std::function<void(uint64_t, uint64_t)> *fn_ = nullptr;
+    uint64_t total_ = 0, per_ = 0, gen_ = 0;
+    int pending_ = 0;
+    bool stop_ = false;
+};
+
+// ------------------------------------------------------------------------------------------------
+// Slice and chunk plans
+// ------------------------------------------------------------------------------------------------
+uint64_t RoundUp(uint64_t v, uint64_t d) { return d == 0 ? v : (v + d - 1) / d * d; }
+
+// all_reduce_ring.cc:119-130 (same rule: coll_all_reduce_executor.cc:330-360).
+std::vector<Slice> RingSlices(uint64_t total, uint32_t p, uint64_t align)
+{
+    std::vector<Slice> s(p);
+    uint64_t per = RoundUp((total + (p - 1)) / p, align);
+    uint64_t residue = total;
+    for (uint32_t i = 0; i < p; i++) {
+        s[i].size = (residue > per) ? per : residue;
+        s[i].off = total - residue;
+        residue -= s[i].size;
+    }
+    return s;
+}
+
+// recursive_halvingdoubling_base.cc:23-37.
+void RhdParams(uint32_t p, uint32_t *block, uint32_t *part1)
+{
+    uint32_t round = 0;
+    while ((1u << round) <= p) {
+        round++;
+    }
+    if (round >= 1) {
+        round--;
+    }
+    *block = 1u << round;
+    *part1 = (p - *block) * 2;
+}
+
+// recursive_halvingdoubling_base.cc:64-94.
+std::vector<Slice> RhdSlices(uint64_t bytes, uint32_t block, uint64_t align)
+{
+    std::vector<Slice> s(block);
+    uint64_t per = bytes / block;
+    if (bytes % block != 0) {
+        per++;
+    }
+    per = RoundUp(per, align);
+    uint64_t left = bytes;
+    uint32_t i = 0;
+    while (left > 0) {
+        s[i].size = per < left ? per : left;
+        s[i].off = bytes - left;
+        left -= s[i].size;
+        i++;
+    }
+    while (i < block) {
+        s[i].off = bytes;
+        s[i].size = 0;
+        i++;
+    }
+    return s;
+}
+
+// coll_comm_executor.cc:1681-1721: cut every rank slice into n pieces, left to right.
+std::vector<std::vector<Slice>> CutPieces(const std::vector<Slice> &slices, uint32_t n, uint64_t align)
+{
+    // result[piece][rank]
+    std::vector<std::vector<Slice>> out(n, std::vector<Slice>(slices.size()));
+    for (size_t r = 0; r < slices.size(); r++) {
+        uint64_t size = slices[r].size, start = slices[r].off;
+        uint32_t k = 0;
+        if (size > 0 && n != 0) {
+            uint64_t per = RoundUp((size + n - 1) / n, align);
+            uint64_t residue = size;
+            while (residue > 0) {
+                uint64_t cur = per < residue ? per : residue;
+                out[k][r] = Slice{start + size - residue, cur};
+                residue -= cur;
+                k++;
+            }
+        }
+        while (k < n) {
+            out[k][r] = Slice{start, 0};
+            k++;
+        }
+    }
+    return out;
+}
+
+// Elements per loop iteration of the executor-level chunk loops.
+//   AllReduce       : cclBytes / unit                                 (coll_all_reduce_executor.cc:86-93)
+//   ReduceScatter   : cclBytes / p / ALIGN * ALIGN / unit             (coll_reduce_scatter_executor.cc:83-90)
+//   AllGather       : cclBytes / p / ALIGN * ALIGN / unit             (coll_all_gather_executor.cc:79-87)
+uint64_t MaxCountPerLoop(int kind, uint64_t cclBytes, uint32_t p, uint64_t unit, uint64_t align)
+{
+    if (kind == 0) {
+        return cclBytes / unit;
+    }
+    return cclBytes / p / align * align / unit;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Message-passing machine
+// ------------------------------------------------------------------------------------------------
+enum ActKind { SEND, RECV_REDUCE, RECV_COPY, LOCAL_COPY, LOCAL_REDUCE };
+enum BufId { B_IN = 0, B_OUT = 1 };
+
+struct Action {
+    ActKind kind;
+    int peer;        // other rank (SEND / RECV_*)
+    int chan;        // FIFO channel between the two ranks (stream index for the mesh)
+    int dstBuf; uint64_t dstOff;
+    int srcBuf; uint64_t srcOff;   // SEND: payload; RECV_REDUCE / LOCAL_*: local operand
+    uint64_t len;
+};
+
+struct Proc {
+    int rank;
+    std::vector<Action> prog;
+    size_t pc = 0;
+};
+
+struct Msg {
+    std::vector<uint8_t> snap;
+    const uint8_t *ptr = nullptr;
+    uint64_t len = 0;
+};
+
+struct Machine {
+    int p = 0;
+    int dt = 0, op = 0;
+    bool direct = false;
+    Pool *pool = nullptr;
+    std::vector<uint8_t *> buf[2];   // buf[B_IN][rank], buf[B_OUT][rank]
+    std::vector<Proc> procs;
+    std::map<std::tuple<int, int, int>, std::deque<Msg>> box;   // (src, dst, chan)
+    uint64_t bytesTouched = 0;
+
+    uint8_t *At(int rank, int b, uint64_t off) { return buf[b][rank] + off; }
+
+    void Copy(uint8_t *dst, const uint8_t *src, uint64_t len)
+    {
+        if (len == 0 || dst == src) {
+            return;
+        }
+        pool->Run(len, 64, [&](uint64_t b, uint64_t e) { std::memmove(dst + b, src + b, e - b); });
+        bytesTouched += 2 * len;
+    }
+    void Reduce(uint8_t *dst, const uint8_t *a, const uint8_t *b, uint64_t len)
+    {
+        if (len == 0) {
+            return;
+        }
+        uint64_t u = DtSize(dt);
+        pool->Run(len, 64, [&](uint64_t s, uint64_t e) { ReduceElems(dt, op, dst + s, a + s, b + s, (e - s) / u); });
+        bytesTouched += 3 * len;
+    }
+
+    // Runs every process to completion; returns 0, or -1 on deadlock.
+    int Run()
+    {
+        bool progress = true;
+        size_t live = 0;
+        for (auto &pr : procs) {
+            live += pr.prog.empty() ? 0 : 1;
+        }
+        while (live > 0 && progress) {
+            progress = false;
+            for (auto &pr : procs) {
+                while (pr.pc < pr.prog.size()) {
+                    const Action &a = pr.prog[pr.pc];
+                    if (a.kind == SEND) {
+                        Msg m;
+                        m.len = a.len;
+                        if (direct) {
+                            m.ptr = At(pr.rank, a.srcBuf, a.srcOff);
+                        } else {
+                            const uint8_t *s = At(pr.rank, a.srcBuf, a.srcOff);
+                            m.snap.assign(s, s + a.len);
+                        }
+                        box[std::make_tuple(pr.rank, a.peer, a.chan)].push_back(std::move(m));
+                    } else if (a.kind == RECV_REDUCE || a.kind == RECV_COPY) {
+                        auto &q = box[std::make_tuple(a.peer, pr.rank, a.chan)];
+                        if (q.empty()) {
+                            break;
+                        }
+                        Msg m = std::move(q.front());
+                        q.pop_front();
+                        if (m.len != a.len) {
+                            std::fprintf(stderr, "oracle: message length mismatch %llu vs %llu\n",
+                                (unsigned long long)m.len, (unsigned long long)a.len);
+                            return -2;
+                        }
+                        const uint8_t *payload = direct ? m.ptr : m.snap.data();
+                        if (a.kind == RECV_REDUCE) {
+                            Reduce(At(pr.rank, a.dstBuf, a.dstOff), At(pr.rank, a.srcBuf, a.srcOff), payload, a.len);
+                        } else {
+                            Copy(At(pr.rank, a.dstBuf, a.dstOff), payload, a.len);
+                        }
+                    } else if (a.kind == LOCAL_COPY) {
+                        Copy(At(pr.rank, a.dstBuf, a.dstOff), At(pr.rank, a.srcBuf, a.srcOff), a.len);
+                    } else {
+                        Reduce(At(pr.rank, a.dstBuf, a.dstOff), At(pr.rank, a.dstBuf, a.dstOff),
+                            At(pr.rank, a.srcBuf, a.srcOff), a.len);
+                    }
+                    pr.pc++;
+                    progress = true;
+                    if (pr.pc == pr.prog.size()) {
+                        live--;
+                    }
+                }
+            }
+        }
+        procs.clear();
+        for (auto &kv : box) {
+            if (!kv.second.empty()) {
+                return -3;   // undelivered message: the programs do not match up
+            }
+        }
+        box.clear();
+        return live == 0 ? 0 : -1;
+    }
+};
+
+inline Action MkSend(int peer, int chan, int b, uint64_t off, uint64_t len)
+{
+    return Action{SEND, peer, chan, 0, 0, b, off, len};
+}
+inline Action MkRecvReduce(int peer, int chan, int dstB, uint64_t dstOff, int srcB, uint64_t srcOff, uint64_t len)
+{
+    return Action{RECV_REDUCE, peer, chan, dstB, dstOff, srcB, srcOff, len};
+}
+inline Action MkRecvCopy(int peer, int chan, int dstB, uint64_t dstOff, uint64_t len)
+{
+    return Action{RECV_COPY, peer, chan, dstB, dstOff, 0, 0, len};
+}
+inline Action MkLocalCopy(int dstB, uint64_t dstOff, int srcB, uint64_t srcOff, uint64_t len)
+{
+    return Action{LOCAL_COPY, -1, 0, dstB, dstOff, srcB, srcOff, len};
+}
+
+// ------------------------------------------------------------------------------------------------
+// Per-rank programs of the templates.  `inB` / `outB` say which machine buffer plays the template's
+// inputMem_ / outputMem_.
+// ------------------------------------------------------------------------------------------------
+
+// ReduceScatterRing::RunReduceScatter, reduce_scatter_ring.cc:179-297 (one segment per rank).
+void ProgReduceScatterRing(std::vector<Action> &pg, uint32_t r, uint32_t p, int inB, int outB,
+    const std::vector<Slice> &in, const std::vector<Slice> &out)
+{
+    if (p == 1) {
+        // reduce_scatter_ring.cc:102-107: whole-buffer copy when input and output differ
+        if (inB != outB) {
+            pg.push_back(MkLocalCopy(outB, out[0].off, inB, in[0].off, in[0].size));
+        }
+        return;
+    }
+    uint32_t left = (r + p - 1) % p, right = (r + 1) % p;
+    uint32_t rx = (r + p - 2) % p;
+    uint32_t tx = (r + p - 1) % p;
+    pg.push_back(MkSend(right, 0, inB, in[tx].off, in[tx].size));
+    for (uint32_t i = 0; i < p - 2; i++) {
+        pg.push_back(MkRecvReduce(left, 0, inB, in[rx].off, inB, in[rx].off, in[rx].size));
+        rx = (rx + p - 1) % p;
+        tx = (tx + p - 1) % p;
+        pg.push_back(MkSend(right, 0, inB, in[tx].off, in[tx].size));
+    }
+    // last transfer: result goes to the template's output at the output slice of this rank
+    pg.push_back(MkRecvReduce(left, 0, outB, out[r].off, inB, in[r].off, in[r].size));
+}
+
+// AllGatherRing::RunAsync + RunAllGather, all_gather_ring.cc:51-171.
+void ProgAllGatherRing(std::vector<Action> &pg, uint32_t r, uint32_t p, int inB, int outB,
+    const std::vector<Slice> &outSl, const std::vector<Slice> &inSl)
+{
+    if (p == 1) {
+        if (inB != outB) {
+            pg.push_back(MkLocalCopy(outB, outSl[0].off, inB, inSl[0].off, outSl[0].size));
+        }
+        return;
+    }
+    uint32_t left = (r + p - 1) % p, right = (r + 1) % p;
+    if (inB != outB) {
+        pg.push_back(MkLocalCopy(outB, outSl[r].off, inB, inSl[r].off, outSl[r].size));
+    }
+    uint32_t rx = (r + p - 1) % p;   // ForwordRank(rank, p, 1)
+    uint32_t tx = r;
+    for (uint32_t i = 0; i + 1 < p; i++) {
+        pg.push_back(MkSend(right, 0, outB, outSl[tx].off, outSl[tx].size));
+        pg.push_back(MkRecvCopy(left, 0, outB, outSl[rx].off, outSl[rx].size));
+        tx = (tx + p - 1) % p;
+        rx = (rx + p - 1) % p;
+    }
+}
+
+// ReduceScatterMesh::RunReduceScatter for one stream, reduce_scatter_mesh.cc:57-124.
+void ProgReduceScatterMeshStream(std::vector<Action> &pg, uint32_t r, uint32_t p, uint32_t stream, int inB,
+    const std::vector<Slice> &sl)
+{
+    for (uint32_t round = 1; round < p; round++) {
+        uint32_t order = (round + stream - 1) % (p - 1);
+        uint32_t src = (r + p - (order + 1)) % p;   // ForwardRank(r, p, order + 1)
+        uint32_t dst = (r + (order + 1)) % p;       // BackwardRank(r, p, order + 1)
+        pg.push_back(MkSend(dst, static_cast<int>(stream), inB, sl[dst].off, sl[dst].size));
+        pg.push_back(MkRecvReduce(src, static_cast<int>(stream), inB, sl[r].off, inB, sl[r].off, sl[r].size));
+    }
+}
+
+// AllGatherMesh::RunAllGather, all_gather_mesh.cc:91-145 (one channel per round).
+void ProgAllGatherMesh(std::vector<Action> &pg, uint32_t r, uint32_t p, int outB, const std::vector<Slice> &sl)
+{
+    for (uint32_t round = 1; round < p; round++) {
+        uint32_t peer = (r + round) % p;
+        uint32_t from = (r + p - round) % p;
+        // rank r sends its slice to r+round and receives slice (r-round) from r-round on the same round
+        pg.push_back(MkSend(peer, static_cast<int>(round), outB, sl[r].off, sl[r].size));
+        pg.push_back(MkRecvCopy(from, static_cast<int>(round), outB, sl[from].off, sl[from].size));
+    }
+}
+
+// ReduceScatterHalvingDoubling::RunReduceScatter, reduce_scatter_halving_doubling.cc:67-91,193-238.
+// q = rank inside the block, rankOf[q] = real rank.
+void ProgReduceScatterHd(std::vector<Action> &pg, uint32_t q, uint32_t block, const std::vector<uint32_t> &rankOf,
+    int inB, int outB, const std::vector<Slice> &sl)
+{
+    uint32_t steps = 0;
+    while ((1u << steps) < block) {
+        steps++;
+    }
+    auto sum = [&](uint32_t first, uint32_t n) {
+        uint64_t s = 0;
+        for (uint32_t i = first; i < first + n; i++) {
+            s += sl[i].size;
+        }
+        return s;
+    };
+    Slice lastRx{0, 0};
+    for (uint32_t step = 0; step < steps; step++) {
+        uint32_t mask = 1u << (steps - step - 1);
+        uint32_t peer = q ^ mask;
+        uint32_t txId = peer & ~(mask - 1);
+        uint32_t rxId = q & ~(mask - 1);
+        Slice tx{sl[txId].off, sum(txId, mask)};
+        Slice rx{sl[rxId].off, sum(rxId, mask)};
+        pg.push_back(MkSend(static_cast<int>(rankOf[peer]), 0, inB, tx.off, tx.size));
+        pg.push_back(MkRecvReduce(static_cast<int>(rankOf[peer]), 0, inB, rx.off, inB, rx.off, rx.size));
+        lastRx = rx;
+    }
+    if (steps > 0) {
+        pg.push_back(MkLocalCopy(outB, lastRx.off, inB, lastRx.off, lastRx.size));
+    }
+}
+
+// AllGatherHalvingDoubling::RunAllGather, all_gather_halving_doubling.cc:43-66,158-196.
+void ProgAllGatherHd(std::vector<Action> &pg, uint32_t q, uint32_t block, const std::vector<uint32_t> &rankOf,
+    int outB, const std::vector<Slice> &sl)
+{
+    uint32_t steps = 0;
+    while ((1u << steps) < block) {
+        steps++;
+    }
+    auto sum = [&](uint32_t first, uint32_t n) {
+        uint64_t s = 0;
+        for (uint32_t i = first; i < first + n; i++) {
+            s += sl[i].size;
+        }
+        return s;
+    };
+    for (uint32_t step = 0; step < steps; step++) {
+        uint32_t mask = 1u << step;
+        uint32_t peer = q ^ mask;
+        uint32_t txId = q & ~(mask - 1);
+        uint32_t rxId = peer & ~(mask - 1);
+        pg.push_back(MkSend(static_cast<int>(rankOf[peer]), 0, outB, sl[txId].off, sum(txId, mask)));
+        pg.push_back(MkRecvCopy(static_cast<int>(rankOf[peer]), 0, outB, sl[rxId].off, sum(rxId, mask)));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Template-level collectives on machine buffers of `bytes` bytes each
+// ------------------------------------------------------------------------------------------------
+
+// AllReduceRing::RunAsync, all_reduce_ring.cc:32-53: RS(in, in, scratch=out) then AG(in, out).
+int RunAllReduceRing(Machine &m, uint64_t bytes, uint64_t align)
+{
+    uint32_t p = m.p;
+    if (p == 1) {
+        m.Copy(m.buf[B_OUT][0], m.buf[B_IN][0], bytes);
+        return 0;
+    }
+    std::vector<Slice> sl = RingSlices(bytes, p, align);
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        ProgReduceScatterRing(pr.prog, r, p, B_IN, B_IN, sl, sl);
+        ProgAllGatherRing(pr.prog, r, p, B_IN, B_OUT, sl, sl);
+        m.procs.push_back(std::move(pr));
+    }
+    return m.Run();
+}
+
+// CollAllReduceMeshExecutor::KernelRun, deterministic branch (coll_all_reduce_mesh_executor.cc:95-240).
+int RunAllReduceMesh(Machine &m, uint64_t bytes, uint64_t align)
+{
+    uint32_t p = m.p;
+    if (p == 1) {
+        m.Copy(m.buf[B_OUT][0], m.buf[B_IN][0], bytes);
+        return 0;
+    }
+    std::vector<Slice> sl = RingSlices(bytes, p, align);
+    if (p > 2) {
+        std::vector<std::vector<Slice>> pieces = CutPieces(sl, p - 1, align);
+        for (uint32_t t = 0; t < p - 1; t++) {
+            for (uint32_t r = 0; r < p; r++) {
+                Proc pr;
+                pr.rank = r;
+                ProgReduceScatterMeshStream(pr.prog, r, p, t, B_IN, pieces[t]);
+                m.procs.push_back(std::move(pr));
+            }
+        }
+    } else {
+        for (uint32_t r = 0; r < p; r++) {
+            Proc pr;
+            pr.rank = r;
+            ProgReduceScatterMeshStream(pr.prog, r, p, 0, B_IN, sl);
+            m.procs.push_back(std::move(pr));
+        }
+    }
+    int rc = m.Run();
+    if (rc != 0) {
+        return rc;
+    }
+    // one server: the level-1 all-reduce is a copy of the own slice from input to output
+    for (uint32_t r = 0; r < p; r++) {
+        m.Copy(m.At(r, B_OUT, sl[r].off), m.At(r, B_IN, sl[r].off), sl[r].size);
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        ProgAllGatherMesh(pr.prog, r, p, B_OUT, sl);
+        m.procs.push_back(std::move(pr));
+    }
+    return m.Run();
+}
+
+// AllReduceRecursiveHalvingDoubling::RunAsync, all_reduce_recursive_hd.cc:33-302.
+int RunAllReduceRhd(Machine &m, uint64_t bytes, uint64_t align)
+{
+    uint32_t p = m.p;
+    if (p == 1) {
+        m.Copy(m.buf[B_OUT][0], m.buf[B_IN][0], bytes);
+        return 0;
+    }
+    uint32_t block, part1;
+    RhdParams(p, &block, &part1);
+    std::vector<Slice> sl = RhdSlices(bytes, block, align);
+    std::vector<uint32_t> rankOf(block);
+    for (uint32_t i = 0; i < p; i++) {
+        if (i < part1 && (i % 2) == 1) {
+            continue;
+        }
+        uint32_t q = (i < part1) ? i / 2 : i - part1 / 2;
+        rankOf[q] = i;
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        bool inPart1 = r < part1;
+        if (inPart1 && (r % 2) == 1) {
+            // fold: send the whole input to the even neighbour; unfold: receive the whole output
+            pr.prog.push_back(MkSend(static_cast<int>(r - 1), 1, B_IN, 0, bytes));
+            pr.prog.push_back(MkRecvCopy(static_cast<int>(r - 1), 1, B_OUT, 0, bytes));
+        } else {
+            if (inPart1) {
+                pr.prog.push_back(MkRecvReduce(static_cast<int>(r + 1), 1, B_IN, 0, B_IN, 0, bytes));
+            }
+            uint32_t q = inPart1 ? r / 2 : r - part1 / 2;
+            ProgReduceScatterHd(pr.prog, q, block, rankOf, B_IN, B_OUT, sl);
+            ProgAllGatherHd(pr.prog, q, block, rankOf, B_OUT, sl);
+            if (inPart1) {
+                pr.prog.push_back(MkSend(static_cast<int>(r + 1), 1, B_OUT, 0, bytes));
+            }
+        }
+        m.procs.push_back(std::move(pr));
+    }
+    int rc = m.Run();
+    // block == 1 cannot happen for p >= 2 (block >= 2); with block == 2^0 there would be no copy to out.
+    return rc;
+}
+
+int RunAllReduceTemplate(Machine &m, int algo, uint64_t bytes, uint64_t align)
+{
+    switch (algo) {
+        case ALGO_RING: return RunAllReduceRing(m, bytes, align);
+        case ALGO_MESH: return RunAllReduceMesh(m, bytes, align);
+        case ALGO_RHD: return RunAllReduceRhd(m, bytes, align);
+        default: return -10;
+    }
+}
+
+}  // namespace
+
+// ================================================================================================
+// C entry points (ctypes)
+// ================================================================================================
+extern "C" {
+
+uint64_t orc_dtype_size(int dt) { return DtSize(dt); }
+
+void orc_ring_slices(uint64_t total, uint32_t p, uint64_t align, uint64_t *off, uint64_t *size)
+{
+    std::vector<Slice> s = RingSlices(total, p, align);
+    for (uint32_t i = 0; i < p; i++) {
+        off[i] = s[i].off;
+        size[i] = s[i].size;
+    }
+}
+
+void orc_rhd_params(uint32_t p, uint32_t *block, uint32_t *part1) { RhdParams(p, block, part1); }
+
+void orc_rhd_slices(uint64_t bytes, uint32_t block, uint64_t align, uint64_t *off, uint64_t *size)
+{
+    std::vector<Slice> s = RhdSlices(bytes, block, align);
+    for (uint32_t i = 0; i < block; i++) {
+        off[i] = s[i].off;
+        size[i] = s[i].size;
+    }
+}
+
+// pieces laid out [piece][rank]
+void orc_cut_pieces(uint32_t nslices, const uint64_t *offIn, const uint64_t *sizeIn, uint32_t n, uint64_t align,
+    uint64_t *off, uint64_t *size)
+{
+    std::vector<Slice> s(nslices);
+    for (uint32_t i = 0; i < nslices; i++) {
+        s[i] = Slice{offIn[i], sizeIn[i]};
+    }
+    auto out = CutPieces(s, n, align);
+    for (uint32_t k = 0; k < n; k++) {
+        for (uint32_t r = 0; r < nslices; r++) {
+            off[k * nslices + r] = out[k][r].off;
+            size[k * nslices + r] = out[k][r].size;
+        }
+    }
+}
+
+// kind: 0 all-reduce, 1 reduce-scatter, 2 all-gather.  Writes up to maxChunks chunk counts.
+uint32_t orc_chunk_plan(int kind, uint64_t count, uint64_t unit, uint32_t p, uint64_t cclBytes, uint64_t align,
+    uint32_t maxChunks, uint64_t *counts)
+{
+    uint64_t maxPer = MaxCountPerLoop(kind, cclBytes, p, unit, align);
+    if (maxPer == 0) {
+        return 0;
+    }
+    uint32_t n = 0;
+    for (uint64_t left = count; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        if (n < maxChunks) {
+            counts[n] = cur;
+        }
+        n++;
+        left -= cur;
+    }
+    return n;
+}
+
+int orc_reduce(int dt, int op, void *dst, const void *a, const void *b, uint64_t n)
+{
+    return ReduceElems(dt, op, dst, a, b, n);
+}
+
+void orc_f32_to_bf16(const float *src, uint16_t *dst, uint64_t n) { for (uint64_t i = 0; i < n; i++) dst[i] = F32ToBf16(src[i]); }
+void orc_bf16_to_f32(const uint16_t *src, float *dst, uint64_t n) { for (uint64_t i = 0; i < n; i++) dst[i] = Bf16ToF32(src[i]); }
+void orc_f32_to_fp16(const float *src, uint16_t *dst, uint64_t n) { for (uint64_t i = 0; i < n; i++) dst[i] = F32ToFp16(src[i]); }
+void orc_fp16_to_f32(const uint16_t *src, float *dst, uint64_t n) { for (uint64_t i = 0; i < n; i++) dst[i] = Fp16ToF32(src[i]); }
+
+// flags: bit0 = direct (pointer) messages instead of snapshots,
+//        bit1 = run the templates on the caller's buffers (no CCL staging copies; `in` is clobbered)
+// Returns 0 on success.  `touched` (optional) receives the bytes read + written by all ranks.
+int orc_allreduce(int algo, uint32_t p, void **in, void **out, uint64_t count, int dt, int op,
+    uint64_t cclBytes, uint64_t align, int flags, int threads, uint64_t *touched)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || cclBytes < unit) {
+        return -20;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.op = op;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    bool zero = (flags & 2) != 0;
+    uint64_t maxPer = MaxCountPerLoop(0, cclBytes, p, unit, align);
+    uint64_t stage = std::min<uint64_t>(count, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn, cclOut;
+    if (!zero) {
+        cclIn.assign(p, std::vector<uint8_t>(stage));
+        cclOut.assign(p, std::vector<uint8_t>(stage));
+    }
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            if (zero) {
+                m.buf[B_IN][r] = static_cast<uint8_t *>(in[r]) + offset;
+                m.buf[B_OUT][r] = static_cast<uint8_t *>(out[r]) + offset;
+            } else {
+                m.buf[B_IN][r] = cclIn[r].data();
+                m.buf[B_OUT][r] = cclOut[r].data();
+                m.Copy(m.buf[B_IN][r], static_cast<uint8_t *>(in[r]) + offset, bytes);
+            }
+        }
+        int rc = RunAllReduceTemplate(m, algo, bytes, align);
+        if (rc != 0) {
+            return rc;
+        }
+        if (!zero) {
+            for (uint32_t r = 0; r < p; r++) {
+                m.Copy(static_cast<uint8_t *>(out[r]) + offset, m.buf[B_OUT][r], bytes);
+            }
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    if (touched) {
+        *touched = m.bytesTouched;
+    }
+    return 0;
+}
+
+// in[r]: p * recvCount elements, out[r]: recvCount elements.  Ring only at this level
+// (coll_reduce_scatter_comm_executor.cc:196-209); mesh uses the same slices with the mesh template.
+int orc_reducescatter(int algo, uint32_t p, void **in, void **out, uint64_t recvCount, int dt, int op,
+    uint64_t cclBytes, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0) {
+        return -20;
+    }
+    uint64_t maxPer = MaxCountPerLoop(1, cclBytes, p, unit, align);
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.op = op;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    uint64_t stage = std::min<uint64_t>(recvCount, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage * p)), cclOut(p, std::vector<uint8_t>(stage));
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_IN][r] = cclIn[r].data();
+        m.buf[B_OUT][r] = cclOut[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = recvCount; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            for (uint32_t i = 0; i < p; i++) {
+                m.Copy(m.buf[B_IN][r] + bytes * i, static_cast<uint8_t *>(in[r]) + recvCount * unit * i + offset, bytes);
+            }
+        }
+        std::vector<Slice> sl(p);
+        for (uint32_t i = 0; i < p; i++) {
+            sl[i] = Slice{bytes * i, bytes};
+        }
+        if (p > 1) {
+            if (algo == ALGO_RING) {
+                for (uint32_t r = 0; r < p; r++) {
+                    Proc pr;
+                    pr.rank = r;
+                    ProgReduceScatterRing(pr.prog, r, p, B_IN, B_IN, sl, sl);
+                    m.procs.push_back(std::move(pr));
+                }
+            } else if (algo == ALGO_MESH) {
+                uint32_t nstream = p > 2 ? p - 1 : 1;
+                std::vector<std::vector<Slice>> pieces = CutPieces(sl, nstream, align);
+                for (uint32_t t = 0; t < nstream; t++) {
+                    for (uint32_t r = 0; r < p; r++) {
+                        Proc pr;
+                        pr.rank = r;
+                        ProgReduceScatterMeshStream(pr.prog, r, p, t, B_IN, pieces[t]);
+                        m.procs.push_back(std::move(pr));
+                    }
+                }
+            } else {
+                return -10;
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            m.Copy(m.buf[B_OUT][r], m.buf[B_IN][r] + bytes * r, bytes);
+            m.Copy(static_cast<uint8_t *>(out[r]) + offset, m.buf[B_OUT][r], bytes);
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
+// in[r]: sendCount elements, out[r]: p * sendCount elements.
+int orc_allgather(int algo, uint32_t p, void **in, void **out, uint64_t sendCount, int dt,
+    uint64_t cclBytes, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0) {
+        return -20;
+    }
+    uint64_t maxPer = MaxCountPerLoop(2, cclBytes, p, unit, align);
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.op = 0;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    uint64_t stage = std::min<uint64_t>(sendCount, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage)), cclOut(p, std::vector<uint8_t>(stage * p));
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_IN][r] = cclIn[r].data();
+        m.buf[B_OUT][r] = cclOut[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = sendCount; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        std::vector<Slice> outSl(p), inSl(p);
+        for (uint32_t i = 0; i < p; i++) {
+            outSl[i] = Slice{bytes * i, bytes};
+            inSl[i] = Slice{(p > 1) ? 0 : bytes * i, bytes};   // input smaller than output -> offset 0
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            m.Copy(m.buf[B_IN][r], static_cast<uint8_t *>(in[r]) + offset, bytes);
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            Proc pr;
+            pr.rank = r;
+            if (algo == ALGO_RING || p == 1) {
+                ProgAllGatherRing(pr.prog, r, p, B_IN, B_OUT, outSl, inSl);
+            } else if (algo == ALGO_MESH) {
+                pr.prog.push_back(MkLocalCopy(B_OUT, outSl[r].off, B_IN, inSl[r].off, bytes));
+                ProgAllGatherMesh(pr.prog, r, p, B_OUT, outSl);
+            } else {
+                return -10;
+            }
+            m.procs.push_back(std::move(pr));
+        }
+        int rc = m.Run();
+        if (rc != 0) {
+            return rc;
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            for (uint32_t i = 0; i < p; i++) {
+                m.Copy(static_cast<uint8_t *>(out[r]) + sendCount * unit * i + offset, m.buf[B_OUT][r] + bytes * i, bytes);
+            }
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
+// PairWise all-to-all-v.  counts / displs are p x p row-major tables in elements: row r is what
+// rank r passed to HcclAlltoAllV.  Returns 1 if the send / receive tables are not symmetric
+// (alltoall_operator.cc:49-72), 0 on success.
+// scratchBytes > 0 selects the BCopy piecewise transfer (alltoallv_pairwise.cc:112-189); 0 = ZCopy.
+int orc_alltoallv(uint32_t p, void **send, const uint64_t *sendCounts, const uint64_t *sdispls,
+    void **recv, const uint64_t *recvCounts, const uint64_t *rdispls, int dt, uint64_t scratchBytes, int flags,
+    int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0) {
+        return -20;
+    }
+    for (uint32_t i = 0; i < p; i++) {
+        for (uint32_t j = 0; j < p; j++) {
+            if (sendCounts[i * p + j] != recvCounts[j * p + i]) {
+                return 1;
+            }
+        }
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_IN][r] = static_cast<uint8_t *>(send[r]);
+        m.buf[B_OUT][r] = static_cast<uint8_t *>(recv[r]);
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        // LocalCopy, alltoallv_pairwise.cc:99-110
+        pr.prog.push_back(MkLocalCopy(B_OUT, rdispls[r * p + r] * unit, B_IN, sdispls[r * p + r] * unit,
+            sendCounts[r * p + r] * unit));
+        for (uint32_t i = 1; i < p; i++) {
+            uint32_t prev = (r + p - i) % p, next = (r + i) % p;
+            uint64_t sendBytes = sendCounts[r * p + next] * unit, recvBytes = recvCounts[r * p + prev] * unit;
+            uint64_t sOff = sdispls[r * p + next] * unit, rOff = rdispls[r * p + prev] * unit;
+            if (scratchBytes == 0) {
+                pr.prog.push_back(MkSend(static_cast<int>(next), 0, B_IN, sOff, sendBytes));
+                pr.prog.push_back(MkRecvCopy(static_cast<int>(prev), 0, B_OUT, rOff, recvBytes));
+            } else {
+                uint64_t sTimes = (sendBytes + scratchBytes - 1) / scratchBytes;
+                uint64_t rTimes = (recvBytes + scratchBytes - 1) / scratchBytes;
+                for (uint64_t t = 0; t < std::max(sTimes, rTimes); t++) {
+                    if (t < sTimes) {
+                        uint64_t cur = std::min(scratchBytes, sendBytes - t * scratchBytes);
+                        pr.prog.push_back(MkSend(static_cast<int>(next), 0, B_IN, sOff + t * scratchBytes, cur));
+                    }
+                    if (t < rTimes) {
+                        uint64_t cur = std::min(scratchBytes, recvBytes - t * scratchBytes);
+                        pr.prog.push_back(MkRecvCopy(static_cast<int>(prev), 0, B_OUT, rOff + t * scratchBytes, cur));
+                    }
+                }
+            }
+        }
+        m.procs.push_back(std::move(pr));
+    }
+    return m.Run();
+}
+
+// ---- synthetic data ------------------------------------------------------------------------------
+static inline uint64_t SplitMix(uint64_t x)
+{
+    x += 0x9e3779b97f4a7c15ull;
+    x = (x ^ (x >> 30)) * 0xbf58476d1ce4e5b9ull;
+    x = (x ^ (x >> 27)) * 0x94d049bb133111ebull;
+    return x ^ (x >> 31);
+}
+
+// x[i] = (u32 >> 8) * 2^-23 - 1  in [-1, 1), counter-based on (seed, rank, i).
+void orc_fill_uniform_f32(float *dst, uint64_t n, uint64_t seed, uint32_t rank, int threads)
+{
+    Pool pool(threads);
+    uint64_t key = seed ^ (static_cast<uint64_t>(rank) << 32);
+    pool.Run(n, 16, [&](uint64_t b, uint64_t e) {
+        for (uint64_t i = b; i < e; i++) {
+            uint32_t u = static_cast<uint32_t>(SplitMix(key + i * 0x2545f4914f6cdd1dull) >> 32);
+            dst[i] = static_cast<float>(u >> 8) * 1.1920928955078125e-07f - 1.0f;
+        }
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,212 @@
+"""ctypes front end of the CPU checker (oracle/hccl_oracle.cc).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the cpu_baseline
+leg of bench.py.  The product library never loads it.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libhccl_oracle.so")
+
+# HcclDataType / HcclReduceOp values (inc/hccl/hccl_types.h:58-87 of the reference).
+INT8, INT16, INT32, FP16, FP32, INT64, UINT64, UINT8, UINT16, UINT32, FP64, BF16 = range(12)
+SUM, PROD, MAX, MIN = range(4)
+RING, MESH, RHD = range(3)
+DIRECT = 1        # flags bit0: messages are pointers, not snapshots
+ZERO_STAGING = 2  # flags bit1: templates run on the caller's buffers (input clobbered)
+
+# numpy carrier type per HcclDataType (fp16 / bf16 travel as raw uint16 bit patterns)
+NP_CARRIER = {
+    INT8: np.int8, INT16: np.int16, INT32: np.int32, FP16: np.uint16, FP32: np.float32, INT64: np.int64,
+    UINT64: np.uint64, UINT8: np.uint8, UINT16: np.uint16, UINT32: np.uint32, FP64: np.float64, BF16: np.uint16,
+}
+
+
+def build(force=False):
+    """Compile the checker with g++ (a few seconds)."""
+    src = os.path.join(_HERE, "hccl_oracle.cc")
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libhccl_oracle.so"], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        u64, u32, i32, vp = ctypes.c_uint64, ctypes.c_uint32, ctypes.c_int, ctypes.c_void_p
+        pu64 = ctypes.POINTER(ctypes.c_uint64)
+        L.orc_dtype_size.restype = u64
+        L.orc_dtype_size.argtypes = [i32]
+        L.orc_ring_slices.argtypes = [u64, u32, u64, pu64, pu64]
+        L.orc_rhd_params.argtypes = [u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]
+        L.orc_rhd_slices.argtypes = [u64, u32, u64, pu64, pu64]
+        L.orc_cut_pieces.argtypes = [u32, pu64, pu64, u32, u64, pu64, pu64]
+        L.orc_chunk_plan.restype = u32
+        L.orc_chunk_plan.argtypes = [i32, u64, u64, u32, u64, u64, u32, pu64]
+        L.orc_reduce.argtypes = [i32, i32, vp, vp, vp, u64]
+        for name in ("orc_f32_to_bf16", "orc_bf16_to_f32", "orc_f32_to_fp16", "orc_fp16_to_f32"):
+            getattr(L, name).argtypes = [vp, vp, u64]
+        L.orc_allreduce.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64, i32, i32, pu64]
+        L.orc_reducescatter.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64, i32, i32]
+        L.orc_allgather.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, u64, u64, i32, i32]
+        L.orc_alltoallv.argtypes = [u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, u64, i32, i32]
+        L.orc_fill_uniform_f32.argtypes = [vp, u64, u64, u32, i32]
+        _lib = L
+    return _lib
+
+
+DEFAULT_CCL_BYTES = 200 << 20   # HCCL_COMM_DEFAULT_BUFFSIZE MiB (inc/hccl/hccl_types.h:112)
+DEFAULT_ALIGN = 128
+
+
+def dtype_size(dt):
+    return int(lib().orc_dtype_size(dt))
+
+
+def _u64arr(n):
+    return (ctypes.c_uint64 * n)()
+
+
+def ring_slices(total, p, align=DEFAULT_ALIGN):
+    off, size = _u64arr(p), _u64arr(p)
+    lib().orc_ring_slices(total, p, align, off, size)
+    return list(off), list(size)
+
+
+def rhd_params(p):
+    b, q = ctypes.c_uint32(), ctypes.c_uint32()
+    lib().orc_rhd_params(p, ctypes.byref(b), ctypes.byref(q))
+    return b.value, q.value
+
+
+def rhd_slices(total, block, align=DEFAULT_ALIGN):
+    off, size = _u64arr(block), _u64arr(block)
+    lib().orc_rhd_slices(total, block, align, off, size)
+    return list(off), list(size)
+
+
+def cut_pieces(offs, sizes, n, align=DEFAULT_ALIGN):
+    k = len(offs)
+    oi, si = _u64arr(k), _u64arr(k)
+    oi[:] = offs
+    si[:] = sizes
+    oo, so = _u64arr(k * n), _u64arr(k * n)
+    lib().orc_cut_pieces(k, oi, si, n, align, oo, so)
+    return [[(oo[t * k + r], so[t * k + r]) for r in range(k)] for t in range(n)]
+
+
+def chunk_plan(kind, count, unit, p, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN):
+    buf = _u64arr(4096)
+    n = lib().orc_chunk_plan(kind, count, unit, p, ccl_bytes, align, 4096, buf)
+    return [int(buf[i]) for i in range(min(n, 4096))]
+
+
+def _ptrs(arrs):
+    a = (ctypes.c_void_p * len(arrs))()
+    for i, x in enumerate(arrs):
+        assert x.flags["C_CONTIGUOUS"]
+        a[i] = x.ctypes.data
+    return a
+
+
+def reduce(dt, op, a, b):
+    out = np.empty_like(a)
+    rc = lib().orc_reduce(dt, op, out.ctypes.data, a.ctypes.data, b.ctypes.data, a.size)
+    assert rc == 0
+    return out
+
+
+def f32_to_bf16(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().orc_f32_to_bf16(x.ctypes.data, out.ctypes.data, x.size)
+    return out
+
+
+def bf16_to_f32(x):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    out = np.empty(x.shape, dtype=np.float32)
+    lib().orc_bf16_to_f32(x.ctypes.data, out.ctypes.data, x.size)
+    return out
+
+
+def f32_to_fp16(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().orc_f32_to_fp16(x.ctypes.data, out.ctypes.data, x.size)
+    return out
+
+
+def fp16_to_f32(x):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    out = np.empty(x.shape, dtype=np.float32)
+    lib().orc_fp16_to_f32(x.ctypes.data, out.ctypes.data, x.size)
+    return out
+
+
+def allreduce(ins, dt, op, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1,
+              outs=None, return_touched=False):
+    """ins: list of p equal-length numpy arrays (carrier dtype).  Returns the p outputs."""
+    p = len(ins)
+    if outs is None:
+        outs = [np.empty_like(x) for x in ins]
+    touched = ctypes.c_uint64(0)
+    rc = lib().orc_allreduce(algo, p, _ptrs(ins), _ptrs(outs), ins[0].size, dt, op, ccl_bytes, align, flags, threads,
+                             ctypes.byref(touched))
+    if rc != 0:
+        raise RuntimeError("oracle allreduce failed rc=%d" % rc)
+    return (outs, touched.value) if return_touched else outs
+
+
+def reducescatter(ins, dt, op, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1):
+    p = len(ins)
+    assert ins[0].size % p == 0
+    n = ins[0].size // p
+    outs = [np.empty(n, dtype=ins[0].dtype) for _ in range(p)]
+    rc = lib().orc_reducescatter(algo, p, _ptrs(ins), _ptrs(outs), n, dt, op, ccl_bytes, align, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle reducescatter failed rc=%d" % rc)
+    return outs
+
+
+def allgather(ins, dt, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1):
+    p = len(ins)
+    n = ins[0].size
+    outs = [np.empty(n * p, dtype=ins[0].dtype) for _ in range(p)]
+    rc = lib().orc_allgather(algo, p, _ptrs(ins), _ptrs(outs), n, dt, ccl_bytes, align, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle allgather failed rc=%d" % rc)
+    return outs
+
+
+def alltoallv(sends, send_counts, sdispls, recvs, recv_counts, rdispls, dt, scratch_bytes=0, flags=0, threads=1):
+    """counts / displs: (p, p) uint64 arrays, row r = rank r's arguments.  recvs are written in place.
+    Returns 0, or 1 when the send / receive tables are not symmetric."""
+    p = len(sends)
+    sc = np.ascontiguousarray(send_counts, dtype=np.uint64)
+    sd = np.ascontiguousarray(sdispls, dtype=np.uint64)
+    rc_ = np.ascontiguousarray(recv_counts, dtype=np.uint64)
+    rd = np.ascontiguousarray(rdispls, dtype=np.uint64)
+    pu64 = ctypes.POINTER(ctypes.c_uint64)
+    rc = lib().orc_alltoallv(p, _ptrs(sends), sc.ctypes.data_as(pu64), sd.ctypes.data_as(pu64), _ptrs(recvs),
+                             rc_.ctypes.data_as(pu64), rd.ctypes.data_as(pu64), dt, scratch_bytes, flags, threads)
+    if rc not in (0, 1):
+        raise RuntimeError("oracle alltoallv failed rc=%d" % rc)
+    return rc
+
+
+def fill_uniform_f32(n, seed, rank, threads=1, out=None):
+    if out is None:
+        out = np.empty(n, dtype=np.float32)
+    lib().orc_fill_uniform_f32(out.ctypes.data, n, seed, rank, threads)
+    return out

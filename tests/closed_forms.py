@@ -1,0 +1,204 @@
+"""Independent closed forms used to pin the CPU checker and the HIP library.
+
+Nothing here shares code with oracle/hccl_oracle.cc or with the product: element arithmetic comes
+from numpy / torch, schedules are written as the reduction chains and trees the templates imply.
+"""
+import numpy as np
+import torch
+
+INT8, INT16, INT32, FP16, FP32, INT64, UINT64, UINT8, UINT16, UINT32, FP64, BF16 = range(12)
+SUM, PROD, MAX, MIN = range(4)
+
+CARRIER = {
+    INT8: np.int8, INT16: np.int16, INT32: np.int32, FP16: np.uint16, FP32: np.float32, INT64: np.int64,
+    UINT64: np.uint64, UINT8: np.uint8, UINT16: np.uint16, UINT32: np.uint32, FP64: np.float64, BF16: np.uint16,
+}
+UNSIGNED_VIEW = {INT8: np.uint8, INT16: np.uint16, INT32: np.uint32, INT64: np.uint64,
+                 UINT8: np.uint8, UINT16: np.uint16, UINT32: np.uint32, UINT64: np.uint64}
+INT_TYPES = tuple(UNSIGNED_VIEW)
+ALL_TYPES = tuple(CARRIER)
+
+
+def bf16_bits_to_f32(bits):
+    return torch.from_numpy(bits.astype(np.int16)).view(torch.bfloat16).to(torch.float32).numpy()
+
+
+def f32_to_bf16_bits(x):
+    t = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(torch.bfloat16)
+    return t.view(torch.int16).numpy().astype(np.uint16)
+
+
+def widen(dt, x):
+    if dt == FP16:
+        return x.view(np.float16).astype(np.float32)
+    if dt == BF16:
+        return bf16_bits_to_f32(x)
+    return x
+
+
+def narrow(dt, x):
+    if dt == FP16:
+        with np.errstate(over="ignore"):
+            return x.astype(np.float16).view(np.uint16)
+    if dt == BF16:
+        return f32_to_bf16_bits(x)
+    return x
+
+
+def combine(dt, op, a, b):
+    """a (+) b with a the local operand, b the received one; carrier arrays in, carrier array out."""
+    with np.errstate(over="ignore", invalid="ignore"):
+        if dt in INT_TYPES:
+            if op in (SUM, PROD):
+                ua, ub = a.view(UNSIGNED_VIEW[dt]), b.view(UNSIGNED_VIEW[dt])
+                r = (ua + ub) if op == SUM else (ua * ub)
+                return r.astype(UNSIGNED_VIEW[dt]).view(CARRIER[dt])
+            return np.where(b > a, b, a) if op == MAX else np.where(b < a, b, a)
+        fa, fb = widen(dt, a), widen(dt, b)
+        if op == SUM:
+            return narrow(dt, fa + fb)
+        if op == PROD:
+            return narrow(dt, fa * fb)
+        pick = (fb > fa) if op == MAX else (fb < fa)
+        return np.where(pick, b, a)
+
+
+def slice_plan(total, n, align):
+    per = -(-total // n)
+    per = -(-per // align) * align
+    out, residue = [], total
+    for _ in range(n):
+        size = min(per, residue)
+        out.append((total - residue, size))
+        residue -= size
+    return out
+
+
+def ring_chain(dt, op, xs, s):
+    """Ring reduce-scatter result for slice s: x[s] (+) (x[s-1] (+) (... (x[s+2] (+) x[s+1])))."""
+    p = len(xs)
+    acc = xs[(s + 1) % p]
+    for j in range(2, p + 1):
+        acc = combine(dt, op, xs[(s + j) % p], acc)
+    return acc
+
+
+def ring_allreduce(dt, op, ins, unit, ccl_bytes, align):
+    p = len(ins)
+    n = ins[0].size
+    if p == 1:
+        return [ins[0].copy()]
+    out = np.empty_like(ins[0])
+    max_per = ccl_bytes // unit
+    base = 0
+    while base < n:
+        cur = min(n - base, max_per)
+        for s, (off, size) in enumerate(slice_plan(cur * unit, p, align)):
+            lo, hi = base + off // unit, base + (off + size) // unit
+            if hi > lo:
+                out[lo:hi] = ring_chain(dt, op, [x[lo:hi] for x in ins], s)
+        base += cur
+    return [out.copy() for _ in range(p)]
+
+
+def mesh_chain(dt, op, xs, r, t):
+    """Deterministic mesh reduce-scatter, piece t of slice r: x[r] (+) x[r-1-((0+t)%(p-1))] (+) ... left to right."""
+    p = len(xs)
+    acc = xs[r]
+    for rnd in range(1, p):
+        order = (rnd + t - 1) % (p - 1)
+        acc = combine(dt, op, acc, xs[(r - (order + 1)) % p])
+    return acc
+
+
+def mesh_allreduce(dt, op, ins, unit, ccl_bytes, align):
+    p = len(ins)
+    n = ins[0].size
+    if p == 1:
+        return [ins[0].copy()]
+    out = np.empty_like(ins[0])
+    max_per = ccl_bytes // unit
+    base = 0
+    nstream = p - 1 if p > 2 else 1
+    while base < n:
+        cur = min(n - base, max_per)
+        for r, (off, size) in enumerate(slice_plan(cur * unit, p, align)):
+            if size == 0:
+                continue
+            for t, (poff, psize) in enumerate(slice_plan(size, nstream, align)):
+                lo, hi = base + (off + poff) // unit, base + (off + poff + psize) // unit
+                if hi > lo:
+                    out[lo:hi] = mesh_chain(dt, op, [x[lo:hi] for x in ins], r, t)
+        base += cur
+    return [out.copy() for _ in range(p)]
+
+
+def rhd_params(p):
+    block = 1
+    while block * 2 <= p:
+        block *= 2
+    return block, 2 * (p - block)
+
+
+def rhd_tree(dt, op, xs, q, block, part1):
+    """Value held by block rank q for its own slice after the halving phase."""
+    def leaf(b):
+        if 2 * b < part1:
+            return combine(dt, op, xs[2 * b], xs[2 * b + 1])
+        return xs[b + part1 // 2]
+
+    steps = block.bit_length() - 1
+
+    def v(b, s):
+        if s == 0:
+            return leaf(b)
+        mask = block >> s
+        return combine(dt, op, v(b, s - 1), v(b ^ mask, s - 1))
+
+    return v(q, steps)
+
+
+def rhd_allreduce(dt, op, ins, unit, ccl_bytes, align):
+    p = len(ins)
+    n = ins[0].size
+    if p == 1:
+        return [ins[0].copy()]
+    block, part1 = rhd_params(p)
+    out = np.empty_like(ins[0])
+    max_per = ccl_bytes // unit
+    base = 0
+    while base < n:
+        cur = min(n - base, max_per)
+        for q, (off, size) in enumerate(slice_plan(cur * unit, block, align)):
+            lo, hi = base + off // unit, base + (off + size) // unit
+            if hi > lo:
+                out[lo:hi] = rhd_tree(dt, op, [x[lo:hi] for x in ins], q, block, part1)
+        base += cur
+    return [out.copy() for _ in range(p)]
+
+
+def naive_reduce(dt, op, xs):
+    acc = xs[0]
+    for x in xs[1:]:
+        acc = combine(dt, op, acc, x)
+    return acc
+
+
+def random_input(dt, n, rng, small=False):
+    """Carrier array of n random elements; `small` keeps floats integer-valued so sums are exact."""
+    if dt in (FP32, FP64):
+        if small:
+            return rng.integers(-64, 65, n).astype(CARRIER[dt])
+        return rng.uniform(-1.0, 1.0, n).astype(CARRIER[dt])
+    if dt == FP16:
+        v = rng.integers(-8, 9, n).astype(np.float32) if small else rng.standard_normal(n).astype(np.float32)
+        return v.astype(np.float16).view(np.uint16)
+    if dt == BF16:
+        v = rng.integers(-8, 9, n).astype(np.float32) if small else rng.standard_normal(n).astype(np.float32)
+        return f32_to_bf16_bits(v)
+    if dt == INT64:
+        return rng.integers(-(1 << 40), (1 << 40), n, dtype=np.int64)
+    if dt == UINT64:
+        return rng.integers(0, 1 << 63, n, dtype=np.uint64)
+    info = np.iinfo(CARRIER[dt])
+    return rng.integers(info.min, int(info.max) + 1, n, dtype=np.int64).astype(CARRIER[dt])

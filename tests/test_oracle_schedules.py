@@ -1,0 +1,273 @@
+"""Pins the checker's schedules (message-passing restatement) against closed forms that do not share
+code with it: reduction chains / trees evaluated with numpy + torch arithmetic, order-independent
+integer results, and permutation closed forms."""
+import numpy as np
+import pytest
+
+import closed_forms as cf
+from closed_forms import (ALL_TYPES, BF16, FP16, FP32, FP64, INT8, INT32, INT64, INT_TYPES, MAX, MIN, PROD, SUM)
+
+RING, MESH, RHD = 0, 1, 2
+OPS = (SUM, PROD, MAX, MIN)
+
+
+def test_element_ops_match_numpy_and_torch(orc):
+    rng = np.random.default_rng(1)
+    for dt in ALL_TYPES:
+        a = cf.random_input(dt, 4099, rng)
+        b = cf.random_input(dt, 4099, rng)
+        for op in OPS:
+            got = orc.reduce(dt, op, a, b)
+            want = cf.combine(dt, op, a, b)
+            if dt in (FP16, BF16, FP32, FP64):
+                both_nan = np.isnan(cf.widen(dt, got).astype(np.float64)) & np.isnan(cf.widen(dt, want).astype(np.float64))
+                assert np.array_equal(got[~both_nan], want[~both_nan]), (dt, op)
+            else:
+                assert np.array_equal(got, want), (dt, op)
+
+
+def test_half_conversions_exhaustive(orc):
+    # every fp16 bit pattern widens exactly as numpy does, and narrows back to itself
+    bits = np.arange(65536, dtype=np.uint16)
+    f = orc.fp16_to_f32(bits)
+    ref = bits.view(np.float16).astype(np.float32)
+    ok = ~np.isnan(ref)
+    assert np.array_equal(f[ok].view(np.uint32), ref[ok].view(np.uint32))
+    assert np.array_equal(orc.f32_to_fp16(f)[ok], bits[ok])
+    # every bf16 bit pattern likewise (torch is the independent converter)
+    fb = orc.bf16_to_f32(bits)
+    refb = cf.bf16_bits_to_f32(bits)
+    okb = ~np.isnan(refb)
+    assert np.array_equal(fb[okb].view(np.uint32), refb[okb].view(np.uint32))
+    assert np.array_equal(orc.f32_to_bf16(fb)[okb], bits[okb])
+
+
+def test_narrowing_rounds_to_nearest_even(orc):
+    rng = np.random.default_rng(2)
+    x = np.concatenate([
+        rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 200000).astype(np.float32),
+        np.array([65504.0, 65519.9, 65520.0, 70000.0, 2.0 ** -24, 2.0 ** -25, 1.5 * 2.0 ** -25, 2.0 ** -14,
+                  6.1e-5, 5.96e-8, 2.98e-8, 0.0, -0.0, np.inf, -np.inf], dtype=np.float32)])
+    with np.errstate(over="ignore"):
+        assert np.array_equal(orc.f32_to_fp16(x), x.astype(np.float16).view(np.uint16))
+    assert np.array_equal(orc.f32_to_bf16(x), cf.f32_to_bf16_bits(x))
+    # halfway cases for bf16: 1 + 2^-8 ties to even (1.0), 1 + 3*2^-8 ties to 1 + 2^-6
+    t = np.array([1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8], dtype=np.float32)
+    assert list(orc.f32_to_bf16(t)) == [0x3f80, 0x3f82]
+
+
+def _inputs(dt, p, n, seed, small=False):
+    rng = np.random.default_rng(seed)
+    return [cf.random_input(dt, n, rng, small) for _ in range(p)]
+
+
+def _eq(dt, got, want):
+    if dt in (FP16, BF16, FP32, FP64):
+        g, w = cf.widen(dt, got).astype(np.float64), cf.widen(dt, want).astype(np.float64)
+        nn = np.isnan(g) & np.isnan(w)
+        return np.array_equal(got[~nn], want[~nn])
+    return np.array_equal(got, want)
+
+
+CLOSED = {RING: cf.ring_allreduce, MESH: cf.mesh_allreduce, RHD: cf.rhd_allreduce}
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+def test_allreduce_fp32_sum_matches_closed_form_all_p(orc, algo):
+    # fp32 sum is order-sensitive: only the right chain / tree reproduces these bits
+    for p in range(1, 34):
+        n = 257 + 3 * p
+        ins = _inputs(FP32, p, n, 100 + p)
+        for align in (4, 128):
+            got = orc.allreduce(ins, FP32, SUM, algo=algo, align=align)
+            want = CLOSED[algo](FP32, SUM, ins, 4, 200 << 20, align)
+            for r in range(p):
+                assert np.array_equal(got[r], want[r]), (algo, p, align, r)
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("dt", ALL_TYPES)
+def test_allreduce_all_types_ops_match_closed_form(orc, algo, dt):
+    unit = orc.dtype_size(dt)
+    for p in (2, 3, 5, 8, 12):
+        for op in OPS:
+            ins = _inputs(dt, p, 1000, 7 * p + op)
+            got = orc.allreduce(ins, dt, op, algo=algo)
+            want = CLOSED[algo](dt, op, ins, unit, 200 << 20, 128)
+            for r in range(p):
+                assert _eq(dt, got[r], want[r]), (algo, dt, p, op, r)
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+def test_allreduce_chunked_matches_closed_form(orc, algo):
+    # CCL buffer smaller than the payload: the chunk loop restarts the slice plan per chunk
+    p, n = 8, 5000
+    ins = _inputs(FP32, p, n, 5)
+    for ccl in (4096, 4100, 1 << 14):
+        got = orc.allreduce(ins, FP32, SUM, algo=algo, ccl_bytes=ccl)
+        want = CLOSED[algo](FP32, SUM, ins, 4, ccl, 128)
+        for r in range(p):
+            assert np.array_equal(got[r], want[r]), (algo, ccl, r)
+
+
+def test_ring_order_sensitive_known_answer(orc):
+    # p = 4, one element per slice (align 4): slice 0 must be x0 + (x3 + (x2 + x1)).
+    # With x1 = 2^24, x2 = 1, x3 = -2^24, x0 = 1: (2^24 + 1) = 2^24 in fp32, then -2^24 -> 0, then +1 -> 1.
+    # A left-to-right sum x0+x1+x2+x3 gives 0 + ... = (1+2^24)=2^24, +1 = 2^24, -2^24 = 0.
+    big = np.float32(2.0 ** 24)
+    xs = [np.array([1, 0, 0, 0], np.float32), np.array([big, 0, 0, 0], np.float32),
+          np.array([1, 0, 0, 0], np.float32), np.array([-big, 0, 0, 0], np.float32)]
+    got = orc.allreduce(xs, FP32, SUM, algo=RING, align=4)
+    assert got[0][0] == np.float32(1.0)
+    assert all(np.array_equal(got[0], g) for g in got)
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("dt", INT_TYPES)
+def test_integer_results_are_schedule_independent(orc, algo, dt):
+    for p in (2, 3, 7, 8, 16, 24):
+        for op in OPS:
+            ins = _inputs(dt, p, 777, p + 31 * op)
+            got = orc.allreduce(ins, dt, op, algo=algo)
+            want = cf.naive_reduce(dt, op, ins)
+            for r in range(p):
+                assert np.array_equal(got[r], want), (algo, dt, p, op)
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+def test_exact_float_sums_equal_integer_sums(orc, algo):
+    for dt in (FP32, FP16, BF16, FP64):
+        for p in (3, 8, 24):
+            ins = _inputs(dt, p, 513, p, small=True)
+            got = orc.allreduce(ins, dt, SUM, algo=algo)
+            exact = sum(cf.widen(dt, x).astype(np.float64) for x in ins)
+            assert np.array_equal(cf.widen(dt, got[0]).astype(np.float64), exact), (algo, dt, p)
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+def test_modes_agree(orc, algo):
+    # snapshot vs pointer messages, staged vs zero-staging, 1 vs 4 threads, in-place vs out-of-place
+    p, n = 6, 70001
+    ins = _inputs(FP32, p, n, 9)
+    base = orc.allreduce(ins, FP32, SUM, algo=algo)
+    for flags in (orc.DIRECT, orc.ZERO_STAGING, orc.DIRECT | orc.ZERO_STAGING):
+        for threads in (1, 4):
+            work = [x.copy() for x in ins]
+            got = orc.allreduce(work, FP32, SUM, algo=algo, flags=flags, threads=threads)
+            for r in range(p):
+                assert np.array_equal(got[r], base[r]), (algo, flags, threads)
+            if not flags & orc.ZERO_STAGING:
+                assert all(np.array_equal(w, x) for w, x in zip(work, ins))   # staged mode leaves inputs alone
+    work = [x.copy() for x in ins]
+    got = orc.allreduce(work, FP32, SUM, algo=algo, outs=work)                 # in place
+    for r in range(p):
+        assert np.array_equal(got[r], base[r])
+
+
+def test_zero_staging_byte_count_matches_formula(orc):
+    # ring all-reduce out-of-place touches (5p - 3) * S bytes when slices are equal
+    p, n = 8, 1 << 16
+    ins = _inputs(FP32, p, n, 3)
+    _, touched = orc.allreduce([x.copy() for x in ins], FP32, SUM, flags=orc.DIRECT | orc.ZERO_STAGING, return_touched=True)
+    assert touched == (5 * p - 3) * n * 4
+
+
+@pytest.mark.parametrize("algo", [RING, MESH])
+def test_reducescatter_matches_chain(orc, algo):
+    for dt in (FP32, BF16, INT8, INT64):
+        unit = orc.dtype_size(dt)
+        for p in (1, 2, 3, 8):
+            n = 333
+            for op in OPS:
+                ins = _inputs(dt, p, n * p, p + op)
+                for ccl in (200 << 20, 128 * p * 2):
+                    got = orc.reducescatter(ins, dt, op, algo=algo, ccl_bytes=ccl)
+                    for r in range(p):
+                        xs = [x[r * n:(r + 1) * n] for x in ins]
+                        if p == 1:
+                            want = xs[0]
+                        elif algo == RING:
+                            want = cf.ring_chain(dt, op, xs, r)
+                        else:
+                            want = np.empty_like(xs[0])
+                            # the piece cut restarts in every chunk of the loop
+                            max_per = ccl // p // 128 * 128 // unit
+                            nstream = p - 1 if p > 2 else 1
+                            base = 0
+                            while base < n:
+                                cur = min(max_per, n - base)
+                                for t, (po, ps) in enumerate(cf.slice_plan(cur * unit, nstream, 128)):
+                                    lo, hi = base + po // unit, base + (po + ps) // unit
+                                    if hi > lo:
+                                        want[lo:hi] = cf.mesh_chain(dt, op, [x[lo:hi] for x in xs], r, t)
+                                base += cur
+                        assert _eq(dt, got[r], want), (algo, dt, p, op, ccl, r)
+
+
+@pytest.mark.parametrize("algo", [RING, MESH])
+def test_allgather_is_the_permutation(orc, algo):
+    for dt in (INT8, FP16, INT32, INT64):
+        for p in (1, 2, 5, 8, 16):
+            n = 301
+            ins = _inputs(dt, p, n, p)
+            for ccl in (200 << 20, 128 * p * 2):
+                got = orc.allgather(ins, dt, algo=algo, ccl_bytes=ccl)
+                want = np.concatenate(ins)
+                for r in range(p):
+                    assert np.array_equal(got[r], want), (algo, dt, p, ccl)
+
+
+def _a2av_case(p, seed, max_count=300):
+    rng = np.random.default_rng(seed)
+    cnt = rng.integers(0, max_count, (p, p)).astype(np.uint64)
+    cnt[rng.random((p, p)) < 0.15] = 0
+    sdis = np.zeros((p, p), np.uint64)
+    rdis = np.zeros((p, p), np.uint64)
+    send_len, recv_len = [], []
+    for r in range(p):
+        pos = 0
+        for j in rng.permutation(p):               # destinations laid out in a shuffled order, with gaps
+            pos += int(rng.integers(0, 17))
+            sdis[r, j] = pos
+            pos += int(cnt[r, j])
+        send_len.append(pos + 5)
+        pos = 0
+        for i in rng.permutation(p):
+            pos += int(rng.integers(0, 17))
+            rdis[r, i] = pos
+            pos += int(cnt[i, r])
+        recv_len.append(pos + 5)
+    return cnt, sdis, cnt.T.copy(), rdis, send_len, recv_len
+
+
+def test_alltoallv_is_the_permutation(orc):
+    for p in (1, 2, 3, 8, 16):
+        cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, p)
+        sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+        for scratch in (0, 64, 1000):
+            recvs = [np.full(n, -1, np.int32) for n in rl]
+            assert orc.alltoallv(sends, cnt, sdis, recvs, rcnt, rdis, INT32, scratch_bytes=scratch) == 0
+            for j in range(p):
+                want = np.full(rl[j], -1, np.int32)
+                for i in range(p):
+                    c = int(cnt[i, j])
+                    want[int(rdis[j, i]):int(rdis[j, i]) + c] = sends[i][int(sdis[i, j]):int(sdis[i, j]) + c]
+                assert np.array_equal(recvs[j], want), (p, scratch, j)
+
+
+def test_alltoallv_rejects_asymmetric_tables(orc):
+    p = 4
+    cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 1)
+    rcnt = rcnt.copy()
+    rcnt[2, 1] += 1
+    sends = [np.zeros(n + 8, np.int32) for n in sl]
+    recvs = [np.zeros(n + 8, np.int32) for n in rl]
+    assert orc.alltoallv(sends, cnt, sdis, recvs, rcnt, rdis, INT32) == 1
+
+
+def test_uniform_fill_is_counter_based(orc):
+    a = orc.fill_uniform_f32(100000, 42, 3, threads=1)
+    b = orc.fill_uniform_f32(100000, 42, 3, threads=4)
+    c = orc.fill_uniform_f32(100000, 42, 4)
+    assert np.array_equal(a, b) and not np.array_equal(a, c)
+    assert a.min() >= -1.0 and a.max() < 1.0 and abs(float(a.mean())) < 0.01
