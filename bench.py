@@ -1,0 +1,170 @@
+"""Benchmark of the hot path on one MI355X.
+
+Default workload: ring all-reduce, sum, fp32, 8 simulated ranks x 256 MiB per rank, out of place
+(BASELINE.json configs[1] at its largest size).  A "step" is one complete collective (one call per
+rank).  Prints one JSON line; see DESIGN.md for the byte accounting.
+
+    python bench.py [--steps K] [--warmup W] [--size-mib M] [--sweep] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+METRIC = "achieved HBM GB/s & % of peak, 8-rank fp32 ring AllReduce 256MiB/rank"
+
+# HBM traffic of the fused all-reduce kernel at the default workload, from rocprofv3 --pmc
+# (FETCH_SIZE, WRITE_SIZE), scaled by the same counters over a plain copy of known size.
+# None until measured; the figures and the commands are in profiles/.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def run_mode(pkg, torch, comms, stream, sends, recvs, n, fuse, steps, warmup):
+    pkg.set_param(comms[0], "fuse", fuse)
+    sp = [t.data_ptr() for t in sends]
+    rp = [t.data_ptr() for t in recvs]
+    dt, op = pkg.HCCL_DATA_TYPE_FP32, pkg.HCCL_REDUCE_SUM
+    for _ in range(warmup):
+        pkg.all_reduce(comms, sp, rp, n, dt, op, stream.cuda_stream)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        e0.record(stream)
+        for _ in range(steps):
+            pkg.all_reduce(comms, sp, rp, n, dt, op, stream.cuda_stream)
+        e1.record(stream)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    dev_ms = e0.elapsed_time(e1) / steps
+    info = pkg.last_op_info(comms[0])
+    return wall_ms, dev_ms, info
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--size-mib", type=float, default=256.0, help="bytes per rank, MiB")
+    ap.add_argument("--ranks", type=int, default=8)
+    ap.add_argument("--sweep", action="store_true", help="also time 8 KiB .. 256 MiB per rank (x2), table on stderr")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path is built and measured on one GPU (the ranks of the communicator are "
+                 "simulated inside it); --gpus %d is not supported" % args.gpus)
+
+    import numpy as np
+    import torch
+    from __graft_entry__ import load_package
+    from oracle import oracle
+
+    pkg = load_package()
+    pkg.lib()                                  # raises if the HIP library is not built
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    p = args.ranks
+    n = int(args.size_mib * (1 << 20)) // 4
+    S = n * 4
+    threads = min(16, os.cpu_count() or 1)
+
+    ins = [oracle.fill_uniform_f32(n, 20240611, r, threads=threads) for r in range(p)]
+    sends = [torch.from_numpy(x).cuda() for x in ins]
+    recvs = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(p)]
+    comms = pkg.comm_init_all(p)
+    stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+
+    wall_ms, dev_ms, info = run_mode(pkg, torch, comms, stream, sends, recvs, n, 1, args.steps, args.warmup)
+    fused_out = recvs[0].cpu().numpy()
+    s_wall_ms, s_dev_ms, s_info = run_mode(pkg, torch, comms, stream, sends, recvs, n, 0, args.steps, args.warmup)
+    step_out = recvs[0].cpu().numpy()
+    same_all = all(torch.equal(recvs[0], recvs[r]) for r in range(1, p))
+
+    actual = info["bytesRead"] + info["bytesWritten"]
+    s_actual = s_info["bytesRead"] + s_info["bytesWritten"]
+    sched = (5 * p - 3) * S                     # reference-faithful out-of-place schedule, all ranks
+    achieved = actual / (dev_ms * 1e-3) / 1e9
+    s_achieved = s_actual / (s_dev_ms * 1e-3) / 1e9
+
+    cpu = None
+    bit_exact = None
+    if not args.no_cpu:
+        best = None
+        outs = [np.empty(n, np.float32) for _ in range(p)]
+        for _ in range(3):
+            work = [x.copy() for x in ins]
+            t0 = time.perf_counter()
+            oracle.allreduce(work, oracle.FP32, oracle.SUM, flags=oracle.DIRECT | oracle.ZERO_STAGING, threads=threads, outs=outs)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        bit_exact = bool(np.array_equal(outs[0], fused_out) and np.array_equal(outs[0], step_out))
+        cpu = {"value": round(sched / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+               "sample": "full workload (%d ranks x %.0f MiB fp32, out of place), checker in direct zero-staging "
+                         "mode, best of 3, %.3f s; bytes = (5p-3)S schedule figure" % (p, args.size_mib, best)}
+
+    if args.sweep:
+        sys.stderr.write("bytes/rank  fused_us  fused_GB/s(actual)  steps_us  steps_GB/s(actual)  sched_GB/s(fused)\n")
+        size = 8 << 10
+        while size <= int(args.size_mib * (1 << 20)):
+            m = size // 4
+            _, f_ms, fi = run_mode(pkg, torch, comms, stream, sends, recvs, m, 1, args.steps, args.warmup)
+            _, g_ms, gi = run_mode(pkg, torch, comms, stream, sends, recvs, m, 0, args.steps, args.warmup)
+            fa = (fi["bytesRead"] + fi["bytesWritten"]) / (f_ms * 1e-3) / 1e9
+            ga = (gi["bytesRead"] + gi["bytesWritten"]) / (g_ms * 1e-3) / 1e9
+            sys.stderr.write("%10d %9.1f %12.1f %9.1f %12.1f %12.1f\n" % (size, f_ms * 1e3, fa, g_ms * 1e3, ga,
+                                                                         (5 * p - 3) * size / (f_ms * 1e-3) / 1e9))
+            size *= 2
+
+    line = {
+        "metric": METRIC,
+        "value": round(actual / (wall_ms * 1e-3) / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "ring all-reduce sum fp32, %d simulated ranks x %.0f MiB per rank, out of place, one GPU "
+                        "(BASELINE.json configs[1] at its largest size)" % (p, args.size_mib),
+            "issue": "fused single-pass kernel, HIP graph replay" if info["fused"] else "step-by-step",
+            "launches_per_step": info["launches"],
+            "bytes_per_step_actual": actual,
+            "bytes_per_step_schedule": sched,
+            "pct_of_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBPS, 2),
+            "sched_GBps": round(sched / (dev_ms * 1e-3) / 1e9, 1),
+            "bit_exact_vs_host_reference": bit_exact,
+            "all_ranks_identical": bool(same_all),
+            "step_by_step": {
+                "launches_per_step": s_info["launches"], "ms_per_step": round(s_dev_ms, 4),
+                "bytes_per_step_actual": s_actual, "hbm_GBps": round(s_achieved, 1),
+                "pct_of_hbm_peak": round(100.0 * s_achieved / HBM_PEAK_GBPS, 2), "graph": s_info["graph"],
+            },
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+            "kernel": "ChainKernel<float, sum> (fused ring all-reduce), avg launch %.4f ms over %d launches" % (dev_ms, args.steps),
+        },
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+    pkg.comm_destroy(comms)
+
+
+if __name__ == "__main__":
+    main()

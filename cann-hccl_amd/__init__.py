@@ -1,0 +1,166 @@
+"""Host-side Python mirror of the HCCL C API served by lib/libhccl.so.
+
+The library is the product; this module only binds it with ctypes (same function names, argument
+order and return codes as include/hccl/hccl.h) so tests and the benchmark can call it.  Device
+memory and streams come from the caller (raw pointers / hipStream_t values, e.g. torch's
+tensor.data_ptr() and torch.cuda.current_stream().cuda_stream).
+
+The package directory name contains a hyphen; load it with `load_package()` from
+__graft_entry__.py, or via importlib from its path.
+"""
+import ctypes
+import json
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libhccl.so")
+
+# HcclResult (include/hccl/hccl_types.h)
+HCCL_SUCCESS, HCCL_E_PARA, HCCL_E_PTR, HCCL_E_MEMORY, HCCL_E_INTERNAL, HCCL_E_NOT_SUPPORT = 0, 1, 2, 3, 4, 5
+HCCL_E_NOT_FOUND, HCCL_E_UNAVAIL, HCCL_E_SYSCALL, HCCL_E_TIMEOUT = 6, 7, 8, 9
+HCCL_E_RUNTIME, HCCL_E_AGAIN, HCCL_E_REMOTE, HCCL_E_SUSPENDING, HCCL_E_RESERVED = 15, 20, 21, 22, 23
+# HcclReduceOp
+HCCL_REDUCE_SUM, HCCL_REDUCE_PROD, HCCL_REDUCE_MAX, HCCL_REDUCE_MIN = 0, 1, 2, 3
+# HcclDataType
+(HCCL_DATA_TYPE_INT8, HCCL_DATA_TYPE_INT16, HCCL_DATA_TYPE_INT32, HCCL_DATA_TYPE_FP16, HCCL_DATA_TYPE_FP32,
+ HCCL_DATA_TYPE_INT64, HCCL_DATA_TYPE_UINT64, HCCL_DATA_TYPE_UINT8, HCCL_DATA_TYPE_UINT16, HCCL_DATA_TYPE_UINT32,
+ HCCL_DATA_TYPE_FP64, HCCL_DATA_TYPE_BFP16, HCCL_DATA_TYPE_INT128) = range(13)
+DTYPE_SIZE = {0: 1, 1: 2, 2: 4, 3: 2, 4: 4, 5: 8, 6: 8, 7: 1, 8: 2, 9: 4, 10: 8, 11: 2, 12: 16}
+COLL_ALLREDUCE, COLL_REDUCESCATTER, COLL_ALLGATHER, COLL_ALLTOALLV = range(4)
+ALGO_RING, ALGO_MESH, ALGO_RHD, ALGO_PAIRWISE = range(4)
+
+# Every symbol include/hccl/hccl.h and include/hccl/hccl_amd_ext.h declare.
+EXPORTS = [
+    "HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAlltoAllV", "HcclAlltoAll", "HcclReduceScatterV",
+    "HcclAllGatherV", "HcclBarrier", "HcclCommInitAll", "HcclCommDestroy", "HcclGetRankSize", "HcclGetRankId",
+    "HcclGetCommName", "HcclSetConfig", "HcclGetConfig", "HcclGetCommAsyncError", "HcclGetErrorString",
+    "HcclGetCommConfigCapability", "HcclCommSuspend", "HcclCommResume", "HcclCommInitClusterInfo",
+    "HcclCommInitClusterInfoConfig", "HcclCreateSubCommConfig", "HcclGetRootInfo", "HcclCommInitRootInfo",
+    "HcclCommInitRootInfoConfig", "HcclBroadcast", "HcclScatter", "HcclSend", "HcclRecv", "HcclReduce",
+    "HcclBatchSendRecv", "HcclCommSetMemoryRange", "HcclCommUnsetMemoryRange", "HcclCommActivateCommMemory",
+    "HcclCommDeactivateCommMemory", "HcclAmdSetParam", "HcclAmdGetLastOpInfo", "HcclAmdDescribePlan",
+]
+
+
+class HcclAmdOpInfo(ctypes.Structure):
+    _fields_ = [("coll", ctypes.c_int32), ("algo", ctypes.c_int32), ("fused", ctypes.c_int32), ("graph", ctypes.c_int32),
+                ("cacheHit", ctypes.c_int32), ("launches", ctypes.c_uint32), ("bytesRead", ctypes.c_uint64),
+                ("bytesWritten", ctypes.c_uint64), ("schedRead", ctypes.c_uint64), ("schedWritten", ctypes.c_uint64),
+                ("scratchBytes", ctypes.c_uint64)]
+
+
+_lib = None
+
+
+def lib():
+    """Loads lib/libhccl.so; raises if it has not been built (there is no fallback path)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("libhccl.so is not built: run `python cann-hccl_amd/build.py` (needs hipcc)")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, u64, u32, i32 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_int32
+    L.HcclCommInitAll.argtypes = [u32, ctypes.POINTER(i32), ctypes.POINTER(vp)]
+    L.HcclCommDestroy.argtypes = [vp]
+    L.HcclGetRankSize.argtypes = [vp, ctypes.POINTER(u32)]
+    L.HcclGetRankId.argtypes = [vp, ctypes.POINTER(u32)]
+    L.HcclGetCommName.argtypes = [vp, ctypes.c_char_p]
+    L.HcclAllReduce.argtypes = [vp, vp, u64, i32, i32, vp, vp]
+    L.HcclReduceScatter.argtypes = [vp, vp, u64, i32, i32, vp, vp]
+    L.HcclAllGather.argtypes = [vp, vp, u64, i32, vp, vp]
+    L.HcclAlltoAllV.argtypes = [vp, vp, vp, i32, vp, vp, vp, i32, vp, vp]
+    L.HcclGetErrorString.restype = ctypes.c_char_p
+    L.HcclGetErrorString.argtypes = [i32]
+    L.HcclGetCommConfigCapability.restype = u32
+    L.HcclSetConfig.argtypes = [i32, i32]
+    L.HcclGetConfig.argtypes = [i32, ctypes.POINTER(i32)]
+    L.HcclGetCommAsyncError.argtypes = [vp, ctypes.POINTER(i32)]
+    L.HcclCommSuspend.argtypes = [vp]
+    L.HcclCommResume.argtypes = [vp]
+    L.HcclAmdSetParam.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p]
+    L.HcclAmdGetLastOpInfo.argtypes = [vp, ctypes.POINTER(HcclAmdOpInfo)]
+    L.HcclAmdDescribePlan.argtypes = [i32, i32, u32, u64, i32, u64, u64, u64, ctypes.POINTER(u64), ctypes.c_char_p,
+                                      ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)]
+    _lib = L
+    return L
+
+
+class HcclError(RuntimeError):
+    def __init__(self, fn, code):
+        self.code = code
+        super().__init__("%s returned %d (%s)" % (fn, code, lib().HcclGetErrorString(code).decode()))
+
+
+def _check(fn, code):
+    if code != HCCL_SUCCESS:
+        raise HcclError(fn, code)
+
+
+def comm_init_all(ndev):
+    """HcclCommInitAll with device labels 0..ndev-1; returns the list of HcclComm handles."""
+    devs = (ctypes.c_int32 * ndev)(*range(ndev))
+    comms = (ctypes.c_void_p * ndev)()
+    _check("HcclCommInitAll", lib().HcclCommInitAll(ndev, devs, comms))
+    return [ctypes.c_void_p(c) for c in comms]
+
+
+def comm_destroy(comms):
+    for c in comms:
+        _check("HcclCommDestroy", lib().HcclCommDestroy(c))
+
+
+def set_param(comm, key, value):
+    _check("HcclAmdSetParam", lib().HcclAmdSetParam(comm, key.encode(), str(value).encode()))
+
+
+def last_op_info(comm):
+    info = HcclAmdOpInfo()
+    _check("HcclAmdGetLastOpInfo", lib().HcclAmdGetLastOpInfo(comm, ctypes.byref(info)))
+    return {f[0]: getattr(info, f[0]) for f in HcclAmdOpInfo._fields_}
+
+
+def all_reduce(comms, sends, recvs, count, dtype, op, stream):
+    """One HcclAllReduce call per rank (pointers are ints); the last call issues the work."""
+    for c, s, r in zip(comms, sends, recvs):
+        _check("HcclAllReduce", lib().HcclAllReduce(s, r, count, dtype, op, c, stream))
+
+
+def reduce_scatter(comms, sends, recvs, recv_count, dtype, op, stream):
+    for c, s, r in zip(comms, sends, recvs):
+        _check("HcclReduceScatter", lib().HcclReduceScatter(s, r, recv_count, dtype, op, c, stream))
+
+
+def all_gather(comms, sends, recvs, send_count, dtype, stream):
+    for c, s, r in zip(comms, sends, recvs):
+        _check("HcclAllGather", lib().HcclAllGather(s, r, send_count, dtype, c, stream))
+
+
+def all_to_all_v(comms, sends, send_counts, sdispls, recvs, recv_counts, rdispls, dtype, stream):
+    """counts / displs: per rank, sequences of p integers (elements)."""
+    p = len(comms)
+    keep = []
+    for r in range(p):
+        arrs = [(ctypes.c_uint64 * p)(*[int(x) for x in t[r]]) for t in (send_counts, sdispls, recv_counts, rdispls)]
+        keep.append(arrs)
+        _check("HcclAlltoAllV", lib().HcclAlltoAllV(sends[r], arrs[0], arrs[1], dtype, recvs[r], arrs[2], arrs[3], dtype,
+                                                   comms[r], stream))
+
+
+def describe_plan(coll, algo, p, count, dtype, ccl_bytes=200 << 20, align=128, in_place_mask=0, tables=None):
+    """Plan a collective without a GPU; returns the plan as a dict (see HcclAmdDescribePlan)."""
+    tab = None
+    if tables is not None:
+        flat = [int(x) for t in tables for row in t for x in row]
+        tab = (ctypes.c_uint64 * len(flat))(*flat)
+    cap = 1 << 20
+    while True:
+        buf = ctypes.create_string_buffer(cap)
+        need = ctypes.c_size_t(0)
+        rc = lib().HcclAmdDescribePlan(coll, algo, p, count, dtype, ccl_bytes, align, in_place_mask, tab, buf, cap,
+                                       ctypes.byref(need))
+        if rc == HCCL_E_MEMORY:
+            cap = need.value + 16
+            continue
+        _check("HcclAmdDescribePlan", rc)
+        return json.loads(buf.value.decode())

@@ -1,0 +1,884 @@
+// The HCCL C ABI (include/hccl/hccl.h) over the planner and the HIP task issue.
+//
+// Replaces, for the single-GPU data path, the definitions in the reference's
+// src/domain/collective_communication/framework/op_base/src/op_base.cc (cited per function) and the
+// argument checks of framework/common/src/param_check.cc.  Check order and return codes follow the
+// reference; what differs is stated where it does.
+#include <chrono>
+#include <cstdlib>
+#include <cstring>
+#include <set>
+#include <string>
+
+#include "hccl/hccl.h"
+#include "hccl/hccl_amd_ext.h"
+#include "log.h"
+#include "runtime.h"
+
+using namespace hcclamd;
+
+namespace {
+
+constexpr uint64_t kSysMaxCount = 0x7FFFFFFFFull;   // largest element count a call may carry
+
+std::mutex g_registryMutex;
+std::set<Group *> g_groups;
+int g_deterministic = -1;   // -1: not set through HcclSetConfig
+
+#define CHK_PTR(p)                                              \
+    do {                                                        \
+        if ((p) == nullptr) {                                   \
+            HCCL_LOG_ERROR("%s: %s is null", __func__, #p);     \
+            return HCCL_E_PTR;                                  \
+        }                                                       \
+    } while (0)
+
+Comm *AsComm(HcclComm h)
+{
+    Comm *c = static_cast<Comm *>(h);
+    return (c != nullptr && c->magic == kCommMagic && c->group != nullptr) ? c : nullptr;
+}
+
+// param_check.cc:22-36,261-269: the supported set; everything else is HCCL_E_NOT_SUPPORT.
+bool DataTypeKnown(HcclDataType dt)
+{
+    return dt >= HCCL_DATA_TYPE_INT8 && dt <= HCCL_DATA_TYPE_INT128;
+}
+
+// param_check.cc:375-407: tag, count, data type, stream -- in this order.
+HcclResult CheckOpParam(const char *fn, uint64_t count, HcclDataType dt, const void *stream)
+{
+    if (count > kSysMaxCount) {
+        HCCL_LOG_ERROR("%s: count %llu exceeds the maximum %llu", fn, (unsigned long long)count,
+            (unsigned long long)kSysMaxCount);
+        return HCCL_E_PARA;
+    }
+    if (!DataTypeKnown(dt)) {
+        HCCL_LOG_ERROR("%s: data type %d not supported", fn, int(dt));
+        return HCCL_E_NOT_SUPPORT;
+    }
+    if (stream == nullptr) {
+        HCCL_LOG_ERROR("%s: stream is null", fn);
+        return HCCL_E_PTR;
+    }
+    return HCCL_SUCCESS;
+}
+
+// param_check.cc:284-294.  The per-SoC restrictions of :296-349 (no int16 / bf16 product on 910B)
+// describe Ascend hardware and are not applied here.
+HcclResult CheckReduce(const char *fn, HcclDataType dt, HcclReduceOp op)
+{
+    if (op != HCCL_REDUCE_SUM && op != HCCL_REDUCE_PROD && op != HCCL_REDUCE_MAX && op != HCCL_REDUCE_MIN) {
+        HCCL_LOG_ERROR("%s: reduce op %d not supported", fn, int(op));
+        return HCCL_E_NOT_SUPPORT;
+    }
+    if (dt == HCCL_DATA_TYPE_INT128) {
+        HCCL_LOG_ERROR("%s: no arithmetic on int128", fn);
+        return HCCL_E_NOT_SUPPORT;
+    }
+    return HCCL_SUCCESS;
+}
+
+uint32_t ElemSize(int dt)
+{
+    static const uint32_t table[] = {1, 2, 4, 2, 4, 8, 8, 1, 2, 4, 8, 2, 16};
+    return (dt >= 0 && dt <= 12) ? table[dt] : 0;
+}
+
+void ApplyEnv(GroupConfig *cfg)
+{
+    if (const char *e = std::getenv("HCCL_BUFFSIZE")) {
+        long v = std::atol(e);
+        if (v >= 1) {
+            cfg->cclBytes = uint64_t(v) << 20;
+        }
+    }
+    if (const char *e = std::getenv("HCCL_ALGO")) {
+        std::string s(e);
+        if (s.find("mesh") != std::string::npos || s.find("fullmesh") != std::string::npos) {
+            cfg->algo = ALGO_MESH;
+        } else if (s.find("H-D") != std::string::npos || s.find("rhd") != std::string::npos || s.find("HD") != std::string::npos) {
+            cfg->algo = ALGO_RHD;
+        } else if (s.find("ring") != std::string::npos) {
+            cfg->algo = ALGO_RING;
+        }
+    }
+    if (const char *e = std::getenv("HCCL_DETERMINISTIC")) {
+        cfg->deterministic = (std::string(e) == "true" || std::string(e) == "1");
+    } else if (g_deterministic >= 0) {
+        cfg->deterministic = g_deterministic == 1;
+    }
+    if (const char *e = std::getenv("HCCL_AMD_FUSE")) {
+        cfg->fuse = std::atoi(e) != 0;
+    }
+    if (const char *e = std::getenv("HCCL_AMD_GRAPH")) {
+        cfg->graph = std::atoi(e) != 0;
+    }
+    if (const char *e = std::getenv("HCCL_AMD_BLOCKS_PER_CU")) {
+        int v = std::atoi(e);
+        if (v >= 1 && v <= 64) {
+            cfg->blocksPerCu = uint32_t(v);
+        }
+    }
+    if (const char *e = std::getenv("HCCL_AMD_BLOCKING_ARRIVE")) {
+        cfg->blockingArrive = std::atoi(e) != 0;
+    }
+    if (const char *e = std::getenv("HCCL_EXEC_TIMEOUT")) {
+        long v = std::atol(e);
+        if (v > 0) {
+            cfg->arriveTimeoutMs = uint32_t(std::min<long>(v, 2000000) * 1000);
+        }
+    }
+    if (const char *e = std::getenv("HCCL_AMD_ARRIVE_TIMEOUT_MS")) {
+        long v = std::atol(e);
+        if (v > 0) {
+            cfg->arriveTimeoutMs = uint32_t(v);
+        }
+    }
+}
+
+struct InUse {
+    Comm *c;
+    explicit InUse(Comm *comm) : c(comm) { c->inUse = true; }
+    ~InUse() { c->inUse = false; }
+};
+
+void CancelPending(Group *g)
+{
+    g->arrived = 0;
+    std::fill(g->here.begin(), g->here.end(), 0);
+    g->opSerial++;
+    g->cv.notify_all();
+}
+
+// One rank joins the current collective.  The last rank to join issues it.
+HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t stream, const uint64_t *sendCounts,
+    const uint64_t *sdispls, const uint64_t *recvCounts, const uint64_t *rdispls)
+{
+    Group *g = c->group;
+    std::unique_lock<std::mutex> lock(g->m);
+    if (g->suspended) {
+        return HCCL_E_SUSPENDING;   // hccl_communicator.cc:2748 (CheckSuspendingStatus)
+    }
+    uint32_t r = c->rank;
+    if (g->here[r]) {
+        HCCL_LOG_ERROR("%s: rank %u called again before the other ranks joined the previous call", CollName(sig.coll), r);
+        return HCCL_E_AGAIN;
+    }
+    if (g->arrived == 0) {
+        g->sig = sig;
+    } else if (!(g->sig == sig)) {
+        // every rank must pass the same operation, count, type and op (the reference checks this
+        // across processes in RankConsistentcyChecker, hccl_communicator.cc:2803-2805)
+        HCCL_LOG_ERROR("%s: rank %u disagrees with the ranks already in the collective (op/count/type)", CollName(sig.coll), r);
+        CancelPending(g);
+        return HCCL_E_PARA;
+    }
+    g->here[r] = 1;
+    g->send[r] = send;
+    g->recv[r] = recv;
+    g->streams[r] = stream;
+    if (sig.coll == COLL_ALLTOALLV) {
+        size_t p = g->p;
+        g->sendCounts.resize(p * p);
+        g->sdispls.resize(p * p);
+        g->recvCounts.resize(p * p);
+        g->rdispls.resize(p * p);
+        std::copy(sendCounts, sendCounts + p, g->sendCounts.begin() + r * p);
+        std::copy(sdispls, sdispls + p, g->sdispls.begin() + r * p);
+        std::copy(recvCounts, recvCounts + p, g->recvCounts.begin() + r * p);
+        std::copy(rdispls, rdispls + p, g->rdispls.begin() + r * p);
+    }
+    g->arrived++;
+    if (g->arrived < g->p) {
+        // remember where this rank's stream stands so the launch can be ordered after it
+        // (without a device nothing is recorded; the rank that issues then fails loudly)
+        if (EnsureDevice(g, true) == HCCL_SUCCESS) {
+            if (hipEventRecord(g->arriveEvents[r], stream) != hipSuccess) {
+                HCCL_LOG_ERROR("%s: recording the arrival event of rank %u failed", CollName(sig.coll), r);
+                g->asyncError = HCCL_E_RUNTIME;
+            }
+        }
+        if (!g->cfg.blockingArrive) {
+            return HCCL_SUCCESS;
+        }
+        uint64_t serial = g->opSerial;
+        bool done = g->cv.wait_for(lock, std::chrono::milliseconds(g->cfg.arriveTimeoutMs),
+            [&] { return g->opSerial != serial; });
+        if (!done) {
+            HCCL_LOG_ERROR("%s: rank %u timed out waiting for the other ranks", CollName(sig.coll), r);
+            CancelPending(g);
+            return HCCL_E_TIMEOUT;
+        }
+        return g->lastIssueResult;
+    }
+    // last arrival
+    HcclResult res = HCCL_SUCCESS;
+    if (sig.coll == COLL_ALLTOALLV) {
+        // alltoall_operator.cc:49-72: what i sends to j must be what j expects from i
+        for (uint32_t i = 0; i < g->p && res == HCCL_SUCCESS; i++) {
+            for (uint32_t j = 0; j < g->p; j++) {
+                if (g->sendCounts[size_t(i) * g->p + j] != g->recvCounts[size_t(j) * g->p + i]) {
+                    HCCL_LOG_ERROR("AlltoAllV: rank %u sends %llu elements to rank %u, which expects %llu", i,
+                        (unsigned long long)g->sendCounts[size_t(i) * g->p + j], j,
+                        (unsigned long long)g->recvCounts[size_t(j) * g->p + i]);
+                    res = HCCL_E_PARA;
+                    break;
+                }
+            }
+        }
+    }
+    if (res == HCCL_SUCCESS) {
+        res = IssueCollective(g, r);
+    }
+    if (res != HCCL_SUCCESS && res != HCCL_E_PARA) {
+        g->asyncError = res;
+    }
+    g->lastIssueResult = res;
+    CancelPending(g);   // resets the rendezvous and wakes blocked ranks
+    return res;
+}
+
+}  // namespace
+
+extern "C" {
+
+// ---- lifecycle ------------------------------------------------------------------------------------
+
+// op_base.cc:244-284.
+HcclResult HcclCommInitAll(uint32_t ndev, int32_t *devices, HcclComm *comms)
+{
+    if (ndev == 0) {
+        HCCL_LOG_ERROR("HcclCommInitAll: ndev is 0");
+        return HCCL_E_PARA;
+    }
+    CHK_PTR(comms);
+    CHK_PTR(devices);
+    std::set<int32_t> distinct(devices, devices + ndev);
+    if (distinct.size() != ndev) {
+        HCCL_LOG_ERROR("HcclCommInitAll: duplicate device id in the device list");
+        return HCCL_E_PARA;
+    }
+    if (ndev > kMaxRanks) {
+        HCCL_LOG_ERROR("HcclCommInitAll: at most %u ranks per group", kMaxRanks);
+        return HCCL_E_PARA;
+    }
+    Group *g = new Group();
+    g->p = ndev;
+    ApplyEnv(&g->cfg);
+    g->here.assign(ndev, 0);
+    g->send.assign(ndev, nullptr);
+    g->recv.assign(ndev, nullptr);
+    g->streams.assign(ndev, nullptr);
+    char nm[64];
+    std::snprintf(nm, sizeof(nm), "hccl_world_group_%p", static_cast<void *>(g));
+    g->name = nm;
+    for (uint32_t r = 0; r < ndev; r++) {
+        std::unique_ptr<Comm> c(new Comm());
+        c->group = g;
+        c->rank = r;
+        comms[r] = c.get();
+        g->comms.push_back(std::move(c));
+    }
+    g->liveComms = ndev;
+    std::lock_guard<std::mutex> reg(g_registryMutex);
+    g_groups.insert(g);
+    return HCCL_SUCCESS;
+}
+
+// op_base.cc:2187-2204: null -> success with a warning; in use -> HCCL_E_AGAIN.
+HcclResult HcclCommDestroy(HcclComm comm)
+{
+    if (comm == nullptr) {
+        HCCL_LOG_WARN("HcclCommDestroy: null communicator, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    Group *g = c->group;
+    bool last = false;
+    {
+        std::lock_guard<std::mutex> lock(g->m);
+        if (c->inUse) {
+            HCCL_LOG_WARN("HcclCommDestroy: communicator is in use, try again later");
+            return HCCL_E_AGAIN;
+        }
+        if (g->here[c->rank]) {
+            HCCL_LOG_WARN("HcclCommDestroy: rank %u had joined a collective that was never issued; it is dropped", c->rank);
+            CancelPending(g);
+        }
+        c->magic = 0;
+        c->group = nullptr;
+        g->liveComms--;
+        last = g->liveComms == 0;
+    }
+    if (last) {
+        {
+            std::lock_guard<std::mutex> reg(g_registryMutex);
+            g_groups.erase(g);
+        }
+        delete g;
+    }
+    return HCCL_SUCCESS;
+}
+
+// op_base.cc:2392-2420.
+HcclResult HcclGetRankSize(HcclComm comm, uint32_t *rankSize)
+{
+    CHK_PTR(comm);
+    CHK_PTR(rankSize);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    *rankSize = c->group->p;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclGetRankId(HcclComm comm, uint32_t *rank)
+{
+    CHK_PTR(comm);
+    CHK_PTR(rank);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    *rank = c->rank;
+    return HCCL_SUCCESS;
+}
+
+// op_base.cc:845-856.
+HcclResult HcclGetCommName(HcclComm comm, char *commName)
+{
+    CHK_PTR(comm);
+    CHK_PTR(commName);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::strncpy(commName, c->group->name.c_str(), COMM_NAME_MAX_LENGTH - 1);
+    commName[COMM_NAME_MAX_LENGTH - 1] = '\0';
+    return HCCL_SUCCESS;
+}
+
+// op_base.cc:1204-1243: ignored when the environment variable is set; only 0 and 1 are values.
+HcclResult HcclSetConfig(HcclConfig config, HcclConfigValue configValue)
+{
+    if (config != HCCL_DETERMINISTIC) {
+        return HCCL_SUCCESS;
+    }
+    if (std::getenv("HCCL_DETERMINISTIC") != nullptr) {
+        HCCL_LOG_WARN("HcclSetConfig: HCCL_DETERMINISTIC is set in the environment and wins");
+        return HCCL_SUCCESS;
+    }
+    if (configValue.value != 0 && configValue.value != 1) {
+        HCCL_LOG_ERROR("HcclSetConfig: HCCL_DETERMINISTIC takes 0 or 1");
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> reg(g_registryMutex);
+    g_deterministic = configValue.value;
+    for (Group *g : g_groups) {
+        std::lock_guard<std::mutex> lock(g->m);
+        g->cfg.deterministic = configValue.value == 1;
+    }
+    return HCCL_SUCCESS;
+}
+
+// op_base.cc:1245-1253.
+HcclResult HcclGetConfig(HcclConfig config, HcclConfigValue *configValue)
+{
+    CHK_PTR(configValue);
+    if (config == HCCL_DETERMINISTIC) {
+        const char *e = std::getenv("HCCL_DETERMINISTIC");
+        if (e != nullptr) {
+            configValue->value = (std::string(e) == "true" || std::string(e) == "1") ? 1 : 0;
+        } else {
+            std::lock_guard<std::mutex> reg(g_registryMutex);
+            configValue->value = g_deterministic == 1 ? 1 : 0;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// op_base.cc:3085-3096.  The error is sticky: a failed launch keeps being reported.
+HcclResult HcclGetCommAsyncError(HcclComm comm, HcclResult *asyncError)
+{
+    CHK_PTR(comm);
+    CHK_PTR(asyncError);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> lock(c->group->m);
+    *asyncError = c->group->asyncError;
+    return HCCL_SUCCESS;
+}
+
+// op_base.cc:3103-3122.  The reference's table has no entry for HCCL_E_SUSPENDING and would throw
+// on it; a string is supplied here.
+const char *HcclGetErrorString(HcclResult code)
+{
+    static const char *const names[] = {"no error", "parameter error", "empty pointer", "memory error", "internal error",
+        "not support feature", "not found specific resource", "resource unavailable", "call system interface error",
+        "timeout", "open file fail", "tcp connect fail", "roce connect fail", "tcp transfer fail", "roce transfer fail",
+        "call runtime api fail", "call driver api fail", "call profiling api fail", "call cce api fail",
+        "call network api fail", "try again", "error cqe", "communicator suspending"};
+    if (int(code) < int(HCCL_SUCCESS) || int(code) >= int(HCCL_E_RESERVED)) {
+        return "unknow error";
+    }
+    return names[int(code)];
+}
+
+// op_base.cc:3567-3571.
+uint32_t HcclGetCommConfigCapability() { return static_cast<uint32_t>(HCCL_COMM_CONFIG_RESERVED); }
+
+// op_base.cc:3541-3565.  Applies to the whole group: a suspended group refuses collectives.
+HcclResult HcclCommSuspend(HcclComm comm)
+{
+    CHK_PTR(comm);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> lock(c->group->m);
+    c->group->suspended = true;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclCommResume(HcclComm comm)
+{
+    CHK_PTR(comm);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> lock(c->group->m);
+    c->group->suspended = false;
+    c->group->asyncError = HCCL_SUCCESS;
+    return HCCL_SUCCESS;
+}
+
+// ---- the four collectives ---------------------------------------------------------------------------
+
+// op_base.cc:1268-1350.
+HcclResult HcclAllReduce(void *sendBuf, void *recvBuf, uint64_t count, HcclDataType dataType, HcclReduceOp op,
+    HcclComm comm, aclrtStream stream)
+{
+    if (count == 0) {
+        HCCL_LOG_WARN("HcclAllReduce: count is 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(sendBuf);
+    CHK_PTR(recvBuf);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    HcclResult r = CheckOpParam("HcclAllReduce", count, dataType, stream);
+    if (r == HCCL_SUCCESS) {
+        r = CheckReduce("HcclAllReduce", dataType, op);
+    }
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if ((reinterpret_cast<uintptr_t>(sendBuf) | reinterpret_cast<uintptr_t>(recvBuf)) % ElemSize(dataType) != 0) {
+        HCCL_LOG_ERROR("HcclAllReduce: buffers must be aligned to the element size");
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_ALLREDUCE;
+    sig.count = count;
+    sig.dtype = dataType;
+    sig.recvType = dataType;
+    sig.op = op;
+    return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr);
+}
+
+// op_base.cc:1506-1583.
+HcclResult HcclReduceScatter(void *sendBuf, void *recvBuf, uint64_t recvCount, HcclDataType dataType, HcclReduceOp op,
+    HcclComm comm, aclrtStream stream)
+{
+    if (recvCount == 0) {
+        HCCL_LOG_WARN("HcclReduceScatter: recvCount is 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(sendBuf);
+    CHK_PTR(recvBuf);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    HcclResult r = CheckOpParam("HcclReduceScatter", recvCount, dataType, stream);
+    if (r == HCCL_SUCCESS) {
+        r = CheckReduce("HcclReduceScatter", dataType, op);
+    }
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if ((reinterpret_cast<uintptr_t>(sendBuf) | reinterpret_cast<uintptr_t>(recvBuf)) % ElemSize(dataType) != 0) {
+        HCCL_LOG_ERROR("HcclReduceScatter: buffers must be aligned to the element size");
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_REDUCESCATTER;
+    sig.count = recvCount;
+    sig.dtype = dataType;
+    sig.recvType = dataType;
+    sig.op = op;
+    return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr);
+}
+
+// op_base.cc:1796-1861.
+HcclResult HcclAllGather(void *sendBuf, void *recvBuf, uint64_t sendCount, HcclDataType dataType, HcclComm comm,
+    aclrtStream stream)
+{
+    if (sendCount == 0) {
+        HCCL_LOG_WARN("HcclAllGather: sendCount is 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(sendBuf);
+    CHK_PTR(recvBuf);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    HcclResult r = CheckOpParam("HcclAllGather", sendCount, dataType, stream);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    OpSig sig;
+    sig.coll = COLL_ALLGATHER;
+    sig.count = sendCount;
+    sig.dtype = dataType;
+    sig.recvType = dataType;
+    sig.op = 0;
+    return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr);
+}
+
+// op_base.cc:2520-2631, param_check.cc:145-203.
+HcclResult HcclAlltoAllV(const void *sendBuf, const void *sendCounts, const void *sdispls, HcclDataType sendType,
+    const void *recvBuf, const void *recvCounts, const void *rdispls, HcclDataType recvType, HcclComm comm,
+    aclrtStream stream)
+{
+    CHK_PTR(sendCounts);
+    CHK_PTR(sdispls);
+    CHK_PTR(recvCounts);
+    CHK_PTR(rdispls);
+    CHK_PTR(stream);
+    CHK_PTR(comm);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    uint32_t p = c->group->p;
+    if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
+        HCCL_LOG_ERROR("HcclAlltoAllV: sendBuf and recvBuf cannot be the same");
+        return HCCL_E_PARA;
+    }
+    const uint64_t *sc = static_cast<const uint64_t *>(sendCounts);
+    const uint64_t *rc = static_cast<const uint64_t *>(recvCounts);
+    bool hasSend = false, hasRecv = false;
+    for (uint32_t i = 0; i < p; i++) {
+        if (sc[i] > kSysMaxCount || rc[i] > kSysMaxCount) {
+            HCCL_LOG_ERROR("HcclAlltoAllV: a count exceeds the maximum");
+            return HCCL_E_PARA;
+        }
+        hasSend = hasSend || sc[i] != 0;
+        hasRecv = hasRecv || rc[i] != 0;
+    }
+    if (hasSend) {
+        CHK_PTR(sendBuf);
+    }
+    if (hasRecv) {
+        CHK_PTR(recvBuf);
+    }
+    HcclResult r = CheckOpParam("HcclAlltoAllV", 0, sendType, stream);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if (!DataTypeKnown(recvType)) {
+        return HCCL_E_NOT_SUPPORT;
+    }
+    if (ElemSize(sendType) != ElemSize(recvType)) {
+        HCCL_LOG_ERROR("HcclAlltoAllV: send and receive element sizes differ");
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_ALLTOALLV;
+    sig.count = 0;
+    sig.dtype = sendType;
+    sig.recvType = recvType;
+    sig.op = 0;
+    return Arrive(c, sig, const_cast<void *>(sendBuf), const_cast<void *>(recvBuf), static_cast<hipStream_t>(stream), sc,
+        static_cast<const uint64_t *>(sdispls), rc, static_cast<const uint64_t *>(rdispls));
+}
+
+// ---- extension ----------------------------------------------------------------------------------------
+
+HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
+{
+    CHK_PTR(comm);
+    CHK_PTR(key);
+    CHK_PTR(value);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> lock(c->group->m);
+    GroupConfig &cfg = c->group->cfg;
+    std::string k(key), v(value);
+    if (k == "algo") {
+        if (v == "ring") {
+            cfg.algo = ALGO_RING;
+        } else if (v == "mesh") {
+            cfg.algo = ALGO_MESH;
+        } else if (v == "rhd") {
+            cfg.algo = ALGO_RHD;
+        } else if (v == "auto") {
+            cfg.algo = -1;
+        } else {
+            return HCCL_E_PARA;
+        }
+    } else if (k == "fuse") {
+        cfg.fuse = v != "0";
+    } else if (k == "graph") {
+        cfg.graph = v != "0";
+    } else if (k == "buffsize_mib") {
+        long n = std::atol(value);
+        if (n < 1) {
+            return HCCL_E_PARA;
+        }
+        cfg.cclBytes = uint64_t(n) << 20;
+    } else if (k == "buffsize_bytes") {
+        long long n = std::atoll(value);
+        if (n < 16) {
+            return HCCL_E_PARA;
+        }
+        cfg.cclBytes = uint64_t(n);
+    } else if (k == "align") {
+        long n = std::atol(value);
+        if (n < 1) {
+            return HCCL_E_PARA;
+        }
+        cfg.align = uint64_t(n);
+    } else if (k == "blocks_per_cu") {
+        long n = std::atol(value);
+        if (n < 1 || n > 64) {
+            return HCCL_E_PARA;
+        }
+        cfg.blocksPerCu = uint32_t(n);
+    } else if (k == "blocking_arrive") {
+        cfg.blockingArrive = v != "0";
+    } else if (k == "arrive_timeout_ms") {
+        long n = std::atol(value);
+        if (n < 1) {
+            return HCCL_E_PARA;
+        }
+        cfg.arriveTimeoutMs = uint32_t(n);
+    } else {
+        return HCCL_E_PARA;
+    }
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info)
+{
+    CHK_PTR(comm);
+    CHK_PTR(info);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    std::lock_guard<std::mutex> lock(c->group->m);
+    const OpInfo &o = c->group->lastInfo;
+    info->coll = o.coll;
+    info->algo = o.algo;
+    info->fused = o.fused;
+    info->graph = o.graph;
+    info->cacheHit = o.cacheHit;
+    info->launches = o.launches;
+    info->bytesRead = o.bytesRead;
+    info->bytesWritten = o.bytesWritten;
+    info->schedRead = o.stepRead;
+    info->schedWritten = o.stepWritten;
+    info->scratchBytes = o.scratchBytes;
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint64_t count, HcclDataType dataType,
+    uint64_t cclBytes, uint64_t align, uint64_t inPlaceMask, const uint64_t *tables, char *out, size_t cap, size_t *needed)
+{
+    CHK_PTR(out);
+    if (nRanks == 0 || nRanks > kMaxRanks || !DataTypeKnown(dataType) || coll < 0 || coll > 3) {
+        return HCCL_E_PARA;
+    }
+    PlanRequest rq;
+    rq.coll = CollKind(coll);
+    rq.algo = Algo(algo);
+    rq.p = nRanks;
+    rq.count = count;
+    rq.unit = ElemSize(dataType);
+    rq.cclBytes = cclBytes;
+    rq.align = align;
+    rq.alias.assign(nRanks, 0);
+    for (uint32_t r = 0; r < nRanks; r++) {
+        rq.alias[r] = (inPlaceMask >> r) & 1ull;
+    }
+    if (coll == COLL_ALLTOALLV) {
+        CHK_PTR(tables);
+        size_t n = size_t(nRanks) * nRanks;
+        rq.sendCounts.assign(tables, tables + n);
+        rq.sdispls.assign(tables + n, tables + 2 * n);
+        rq.recvCounts.assign(tables + 2 * n, tables + 3 * n);
+        rq.rdispls.assign(tables + 3 * n, tables + 4 * n);
+    }
+    Plan plan;
+    std::string err;
+    int rc = BuildPlan(rq, &plan, &err);
+    if (rc != 0) {
+        HCCL_LOG_ERROR("HcclAmdDescribePlan: %s", err.c_str());
+        return rc == 1 ? HCCL_E_PARA : HCCL_E_INTERNAL;
+    }
+    std::string js = DescribePlan(plan);
+    if (needed) {
+        *needed = js.size() + 1;
+    }
+    if (js.size() + 1 > cap) {
+        return HCCL_E_MEMORY;
+    }
+    std::memcpy(out, js.c_str(), js.size() + 1);
+    return HCCL_SUCCESS;
+}
+
+// ---- declared for link compatibility; outside the single-GPU data path -----------------------------------
+
+HcclResult HcclCommInitClusterInfo(const char *clusterInfo, uint32_t, HcclComm *comm)
+{
+    CHK_PTR(clusterInfo);
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclCommInitClusterInfoConfig(const char *clusterInfo, uint32_t, HcclCommConfig *config, HcclComm *comm)
+{
+    CHK_PTR(clusterInfo);
+    CHK_PTR(config);
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclCreateSubCommConfig(HcclComm *comm, uint32_t, uint32_t *, uint64_t, uint32_t, HcclCommConfig *config,
+    HcclComm *subComm)
+{
+    CHK_PTR(comm);
+    CHK_PTR(config);
+    CHK_PTR(subComm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclGetRootInfo(HcclRootInfo *rootInfo)
+{
+    CHK_PTR(rootInfo);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclCommInitRootInfo(uint32_t, const HcclRootInfo *rootInfo, uint32_t, HcclComm *comm)
+{
+    CHK_PTR(rootInfo);
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclCommInitRootInfoConfig(uint32_t, const HcclRootInfo *rootInfo, uint32_t, const HcclCommConfig *config,
+    HcclComm *comm)
+{
+    CHK_PTR(rootInfo);
+    CHK_PTR(config);
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclBroadcast(void *buf, uint64_t, HcclDataType, uint32_t, HcclComm comm, aclrtStream)
+{
+    CHK_PTR(comm);
+    CHK_PTR(buf);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclScatter(void *, void *recvBuf, uint64_t, HcclDataType, uint32_t, HcclComm comm, aclrtStream)
+{
+    CHK_PTR(comm);
+    CHK_PTR(recvBuf);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclSend(void *sendBuf, uint64_t, HcclDataType, uint32_t, HcclComm comm, aclrtStream)
+{
+    CHK_PTR(comm);
+    CHK_PTR(sendBuf);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclRecv(void *recvBuf, uint64_t, HcclDataType, uint32_t, HcclComm comm, aclrtStream)
+{
+    CHK_PTR(comm);
+    CHK_PTR(recvBuf);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclReduce(void *sendBuf, void *, uint64_t, HcclDataType, HcclReduceOp, uint32_t, HcclComm comm, aclrtStream)
+{
+    CHK_PTR(comm);
+    CHK_PTR(sendBuf);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclBatchSendRecv(HcclSendRecvItem *sendRecvInfo, uint32_t, HcclComm comm, aclrtStream)
+{
+    CHK_PTR(comm);
+    CHK_PTR(sendRecvInfo);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclReduceScatterV(void *, const void *, const void *, void *, uint64_t, HcclDataType, HcclReduceOp,
+    HcclComm comm, aclrtStream)
+{
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclAllGatherV(void *, uint64_t, void *, const void *, const void *, HcclDataType, HcclComm comm, aclrtStream)
+{
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclAlltoAll(const void *, uint64_t, HcclDataType, const void *, uint64_t, HcclDataType, HcclComm comm,
+    aclrtStream)
+{
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclBarrier(HcclComm comm, aclrtStream stream)
+{
+    CHK_PTR(comm);
+    CHK_PTR(stream);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclCommSetMemoryRange(HcclComm comm, void *, size_t, size_t, uint64_t)
+{
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclCommUnsetMemoryRange(HcclComm comm, void *)
+{
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclCommActivateCommMemory(HcclComm comm, void *, size_t, size_t, aclrtDrvMemHandle, uint64_t)
+{
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+HcclResult HcclCommDeactivateCommMemory(HcclComm comm, void *)
+{
+    CHK_PTR(comm);
+    return HCCL_E_NOT_SUPPORT;
+}
+
+}  // extern "C"

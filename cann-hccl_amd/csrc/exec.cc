@@ -1,0 +1,559 @@
+// Task issue: plan -> descriptor tables in device memory -> HIP graph of kernel nodes -> replay.
+// See runtime.h for the reference interfaces this replaces.
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <sstream>
+
+#include "log.h"
+#include "runtime.h"
+
+namespace hcclamd {
+
+namespace {
+
+#define HIP_OK(expr)                                                                                  \
+    do {                                                                                              \
+        hipError_t e_ = (expr);                                                                       \
+        if (e_ != hipSuccess) {                                                                       \
+            HCCL_LOG_ERROR("%s failed: %s", #expr, hipGetErrorString(e_));                            \
+            return HCCL_E_RUNTIME;                                                                    \
+        }                                                                                             \
+    } while (0)
+
+uint32_t DtypeSize(int dt)
+{
+    static const uint32_t table[] = {1, 2, 4, 2, 4, 8, 8, 1, 2, 4, 8, 2, 16};
+    return (dt >= 0 && dt <= 12) ? table[dt] : 0;
+}
+
+}  // namespace
+
+HcclResult EnsureDevice(Group *g, bool quiet)
+{
+    if (g->deviceReady) {
+        return HCCL_SUCCESS;
+    }
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        if (!quiet) {
+            HCCL_LOG_ERROR("no HIP device available: collectives need a GPU");
+        }
+        return HCCL_E_RUNTIME;
+    }
+    HIP_OK(hipGetDevice(&g->device));
+    hipDeviceProp_t prop;
+    HIP_OK(hipGetDeviceProperties(&prop, g->device));
+    g->numCu = prop.multiProcessorCount > 0 ? uint32_t(prop.multiProcessorCount) : 256u;
+    g->arriveEvents.assign(g->p, nullptr);
+    for (uint32_t r = 0; r < g->p; r++) {
+        HIP_OK(hipEventCreateWithFlags(&g->arriveEvents[r], hipEventDisableTiming));
+    }
+    HIP_OK(hipEventCreateWithFlags(&g->doneEvent, hipEventDisableTiming));
+    g->scratch.assign(g->p, nullptr);
+    g->deviceReady = true;
+    return HCCL_SUCCESS;
+}
+
+namespace {
+
+HcclResult EnsureScratch(Group *g, uint64_t bytes)
+{
+    if (bytes <= g->scratchBytes) {
+        return HCCL_SUCCESS;
+    }
+    // A cached collective may still be running out of the old scratch.
+    HIP_OK(hipDeviceSynchronize());
+    for (uint32_t r = 0; r < g->p; r++) {
+        if (g->scratch[r]) {
+            HIP_OK(hipFree(g->scratch[r]));
+            g->scratch[r] = nullptr;
+        }
+    }
+    g->scratchBytes = 0;
+    g->scratchGen++;
+    for (uint32_t r = 0; r < g->p; r++) {
+        HIP_OK(hipMalloc(&g->scratch[r], bytes));
+    }
+    g->scratchBytes = bytes;
+    return HCCL_SUCCESS;
+}
+
+struct Builder {
+    Group *g;
+    std::vector<uint8_t> host;   // image of the device allocation
+
+    size_t Reserve(size_t bytes)
+    {
+        size_t at = (host.size() + 255) & ~size_t(255);
+        host.resize(at + bytes);
+        return at;
+    }
+    char *Ptr(const Ref &r) const
+    {
+        char *base = nullptr;
+        switch (r.buf) {
+            case BUF_SEND: base = static_cast<char *>(g->send[r.rank]); break;
+            case BUF_RECV: base = static_cast<char *>(g->recv[r.rank]); break;
+            default: base = static_cast<char *>(g->scratch[r.rank]); break;
+        }
+        return base + r.off;
+    }
+};
+
+// Cuts [0, bytes) into an element-wise head, a 16-byte vector body and an element-wise tail, given
+// the addresses involved.  emit(offset, bytes, mode).
+template <typename F> void SplitByAlignment(const std::vector<uintptr_t> &addrs, uint64_t bytes, F emit)
+{
+    uintptr_t anchor = addrs[0];
+    bool co = true, w4 = true;
+    for (uintptr_t a : addrs) {
+        co = co && ((a & 15) == (anchor & 15));
+        w4 = w4 && ((a & 3) == 0);
+    }
+    if (!co && !w4) {
+        emit(uint64_t(0), bytes, uint32_t(ACC_ELEM));
+        return;
+    }
+    uint64_t head = std::min<uint64_t>(bytes, (16 - (anchor & 15)) & 15);
+    uint64_t body = (bytes - head) & ~uint64_t(15);
+    uint64_t tail = bytes - head - body;
+    if (head) {
+        emit(uint64_t(0), head, uint32_t(ACC_ELEM));
+    }
+    if (body) {
+        emit(head, body, uint32_t(co ? ACC_VEC16 : ACC_VEC16_SRC4));
+    }
+    if (tail) {
+        emit(head + body, tail, uint32_t(ACC_ELEM));
+    }
+}
+
+uint32_t TilesOf(uint64_t bytes) { return uint32_t((bytes + kTileBytes - 1) / kTileBytes); }
+
+struct PendingLaunch {
+    LaunchRec rec;
+    size_t tableAt = 0, srcAt = 0, dstAt = 0;
+};
+
+HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int op)
+{
+    Builder b;
+    b.g = g;
+    std::vector<PendingLaunch> pending;
+    const uint32_t maxGrid = std::max(1u, g->numCu * g->cfg.blocksPerCu);
+
+    if (!pp->fused) {
+        const void *func = reduceColl ? LookupKernel(dtype, op, KK_STEP) : LookupCopyKernel(KK_STEP);
+        if (func == nullptr) {
+            return HCCL_E_NOT_SUPPORT;
+        }
+        for (const Phase &ph : pp->plan.phases) {
+            std::vector<StepDesc> descs;
+            uint32_t tiles = 0;
+            for (const Step &s : ph.steps) {
+                char *dst = b.Ptr(s.dst);
+                char *a = b.Ptr(s.a);
+                char *bb = s.reduce ? b.Ptr(s.b) : nullptr;
+                std::vector<uintptr_t> addrs = {reinterpret_cast<uintptr_t>(dst), reinterpret_cast<uintptr_t>(a)};
+                if (bb) {
+                    addrs.push_back(reinterpret_cast<uintptr_t>(bb));
+                }
+                SplitByAlignment(addrs, s.bytes, [&](uint64_t off, uint64_t n, uint32_t mode) {
+                    StepDesc d;
+                    d.dst = dst + off;
+                    d.a = a + off;
+                    d.b = bb ? bb + off : nullptr;
+                    d.bytes = n;
+                    d.tile0 = tiles;
+                    d.mode = mode;
+                    tiles += TilesOf(n);
+                    descs.push_back(d);
+                });
+            }
+            if (descs.empty()) {
+                continue;
+            }
+            PendingLaunch pl;
+            pl.tableAt = b.Reserve(descs.size() * sizeof(StepDesc));
+            std::memcpy(b.host.data() + pl.tableAt, descs.data(), descs.size() * sizeof(StepDesc));
+            pl.rec.func = func;
+            pl.rec.nitems = uint32_t(descs.size());
+            pl.rec.ntiles = tiles;
+            pl.rec.grid = std::min(tiles, maxGrid);
+            pl.rec.fusedArgs = false;
+            pending.push_back(pl);
+        }
+    } else {
+        // one launch per kernel kind present
+        for (int kind : {int(KK_CHAIN), int(KK_TREE8), int(KK_TREE32)}) {
+            std::vector<FusedDesc> descs;
+            std::vector<const void *> srcPool;
+            std::vector<void *> dstPool;
+            uint32_t tiles = 0;
+            for (const FusedItem &it : pp->plan.fused) {
+                int want = (it.kind == FK_TREE) ? (it.nleaf <= 8 ? int(KK_TREE8) : int(KK_TREE32)) : int(KK_CHAIN);
+                if (want != kind) {
+                    continue;
+                }
+                std::vector<char *> srcs, dsts;
+                std::vector<uintptr_t> addrs;
+                for (const Ref &d : it.dst) {
+                    dsts.push_back(b.Ptr(d));
+                    addrs.push_back(reinterpret_cast<uintptr_t>(dsts.back()));
+                }
+                for (size_t k = 0; k < it.src.size(); k++) {
+                    char *s = it.srcValid[k] ? b.Ptr(it.src[k]) : nullptr;
+                    srcs.push_back(s);
+                    if (s) {
+                        addrs.push_back(reinterpret_cast<uintptr_t>(s));
+                    }
+                }
+                uint64_t mask = 0;
+                for (size_t k = 0; k < it.accLeft.size() && k < 64; k++) {
+                    mask |= uint64_t(it.accLeft[k] ? 1 : 0) << k;
+                }
+                SplitByAlignment(addrs, it.bytes, [&](uint64_t off, uint64_t n, uint32_t mode) {
+                    FusedDesc d;
+                    std::memset(&d, 0, sizeof(d));
+                    d.bytes = n;
+                    d.accLeftMask = mask;
+                    d.tile0 = tiles;
+                    d.mode = mode;
+                    d.nsrc = uint32_t(srcs.size());
+                    d.ndst = uint32_t(dsts.size());
+                    d.srcBase = uint32_t(srcPool.size());
+                    d.dstBase = uint32_t(dstPool.size());
+                    d.nleaf = it.nleaf;
+                    for (char *s : srcs) {
+                        srcPool.push_back(s ? s + off : nullptr);
+                    }
+                    for (char *t : dsts) {
+                        dstPool.push_back(t + off);
+                    }
+                    tiles += TilesOf(n);
+                    descs.push_back(d);
+                });
+            }
+            if (descs.empty()) {
+                continue;
+            }
+            const void *func = reduceColl ? LookupKernel(dtype, op, KernelKind(kind)) : LookupCopyKernel(KernelKind(kind));
+            if (func == nullptr) {
+                return HCCL_E_NOT_SUPPORT;
+            }
+            PendingLaunch pl;
+            pl.tableAt = b.Reserve(descs.size() * sizeof(FusedDesc));
+            std::memcpy(b.host.data() + pl.tableAt, descs.data(), descs.size() * sizeof(FusedDesc));
+            pl.srcAt = b.Reserve(srcPool.size() * sizeof(void *));
+            std::memcpy(b.host.data() + pl.srcAt, srcPool.data(), srcPool.size() * sizeof(void *));
+            pl.dstAt = b.Reserve(dstPool.size() * sizeof(void *));
+            std::memcpy(b.host.data() + pl.dstAt, dstPool.data(), dstPool.size() * sizeof(void *));
+            pl.rec.func = func;
+            pl.rec.nitems = uint32_t(descs.size());
+            pl.rec.ntiles = tiles;
+            pl.rec.grid = std::min(tiles, maxGrid);
+            pl.rec.fusedArgs = true;
+            pending.push_back(pl);
+        }
+    }
+    if (pending.empty()) {
+        return HCCL_SUCCESS;   // nothing to move (e.g. one rank, in place)
+    }
+    HIP_OK(hipMalloc(&pp->devTables, b.host.size()));
+    HIP_OK(hipMemcpy(pp->devTables, b.host.data(), b.host.size(), hipMemcpyHostToDevice));
+    char *base = static_cast<char *>(pp->devTables);
+    for (PendingLaunch &pl : pending) {
+        pl.rec.table = base + pl.tableAt;
+        if (pl.rec.fusedArgs) {
+            pl.rec.srcPool = base + pl.srcAt;
+            pl.rec.dstPool = base + pl.dstAt;
+        }
+        pp->launches.push_back(pl.rec);
+    }
+    return HCCL_SUCCESS;
+}
+
+void KernelArgs(LaunchRec &l, void **args)
+{
+    args[0] = &l.table;
+    args[1] = &l.nitems;
+    args[2] = &l.ntiles;
+    args[3] = &l.srcPool;
+    args[4] = &l.dstPool;
+}
+
+HcclResult BuildGraph(Prepared *pp)
+{
+    HIP_OK(hipGraphCreate(&pp->graph, 0));
+    hipGraphNode_t prev = nullptr;
+    for (LaunchRec &l : pp->launches) {
+        void *args[5];
+        KernelArgs(l, args);
+        hipKernelNodeParams kp;
+        std::memset(&kp, 0, sizeof(kp));
+        kp.func = const_cast<void *>(l.func);
+        kp.gridDim = dim3(l.grid, 1, 1);
+        kp.blockDim = dim3(kBlockThreads, 1, 1);
+        kp.sharedMemBytes = 0;
+        kp.kernelParams = args;
+        kp.extra = nullptr;
+        hipGraphNode_t node = nullptr;
+        HIP_OK(hipGraphAddKernelNode(&node, pp->graph, prev ? &prev : nullptr, prev ? 1 : 0, &kp));
+        prev = node;
+    }
+    HIP_OK(hipGraphInstantiate(&pp->exec, pp->graph, nullptr, nullptr, 0));
+    return HCCL_SUCCESS;
+}
+
+bool RangesOverlap(const char *a, uint64_t al, const char *b, uint64_t bl)
+{
+    return al && bl && a < b + bl && b < a + al;
+}
+
+std::string CacheKey(const Group *g, int algo)
+{
+    std::ostringstream os;
+    os << g->sig.coll << '/' << algo << '/' << g->sig.dtype << '/' << g->sig.op << '/' << g->sig.count << '/'
+       << g->cfg.fuse << g->cfg.graph << '/' << g->cfg.cclBytes << '/' << g->cfg.align << '/' << g->cfg.blocksPerCu;
+    for (uint32_t r = 0; r < g->p; r++) {
+        os << '|' << g->send[r] << ',' << g->recv[r];
+    }
+    if (g->sig.coll == COLL_ALLTOALLV) {
+        auto dump = [&](const std::vector<uint64_t> &v) {
+            os << '#';
+            for (uint64_t x : v) {
+                os << x << ',';
+            }
+        };
+        dump(g->sendCounts);
+        dump(g->sdispls);
+        dump(g->recvCounts);
+        dump(g->rdispls);
+    }
+    return os.str();
+}
+
+HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
+{
+    std::unique_ptr<Prepared> pp(new Prepared());
+    const bool reduceColl = g->sig.coll == COLL_ALLREDUCE || g->sig.coll == COLL_REDUCESCATTER;
+    PlanRequest rq;
+    rq.coll = CollKind(g->sig.coll);
+    rq.algo = Algo(algo);
+    rq.p = g->p;
+    rq.count = g->sig.count;
+    rq.unit = DtypeSize(g->sig.dtype);
+    rq.cclBytes = g->cfg.cclBytes;
+    rq.align = g->cfg.align;
+    rq.alias.assign(g->p, 0);
+    for (uint32_t r = 0; r < g->p; r++) {
+        rq.alias[r] = (g->send[r] == g->recv[r]) ? 1 : 0;
+    }
+    if (rq.coll == COLL_ALLTOALLV) {
+        rq.sendCounts = g->sendCounts;
+        rq.sdispls = g->sdispls;
+        rq.recvCounts = g->recvCounts;
+        rq.rdispls = g->rdispls;
+    }
+    std::string err;
+    int rc = BuildPlan(rq, &pp->plan, &err);
+    if (rc != 0) {
+        HCCL_LOG_ERROR("%s: planning failed: %s", CollName(g->sig.coll), err.c_str());
+        return rc == 1 ? HCCL_E_PARA : HCCL_E_INTERNAL;
+    }
+    // Buffers of different ranks must not overlap where one of them is written; a send buffer that
+    // overlaps a receive buffer other than as an exact in-place pair is staged through scratch.
+    bool needStage = false;
+    for (uint32_t i = 0; i < g->p; i++) {
+        const char *ri = static_cast<const char *>(g->recv[i]);
+        for (uint32_t j = 0; j < g->p; j++) {
+            const char *rj = static_cast<const char *>(g->recv[j]);
+            const char *sj = static_cast<const char *>(g->send[j]);
+            if (i != j && RangesOverlap(ri, pp->plan.recvBytes[i], rj, pp->plan.recvBytes[j])) {
+                HCCL_LOG_ERROR("%s: receive buffers of rank %u and rank %u overlap", CollName(g->sig.coll), i, j);
+                return HCCL_E_PARA;
+            }
+            if (RangesOverlap(ri, pp->plan.recvBytes[i], sj, pp->plan.sendBytes[j])) {
+                bool exact = (i == j) && ri == sj && g->sig.coll == COLL_ALLREDUCE;
+                needStage = needStage || !exact;
+            }
+        }
+    }
+    if (needStage) {
+        rq.stageInput = true;
+        rq.alias.assign(g->p, 0);
+        pp->plan = Plan();
+        rc = BuildPlan(rq, &pp->plan, &err);
+        if (rc != 0) {
+            HCCL_LOG_ERROR("%s: planning (staged) failed: %s", CollName(g->sig.coll), err.c_str());
+            return HCCL_E_INTERNAL;
+        }
+    }
+    pp->fused = g->cfg.fuse && pp->plan.fusedOk && !needStage;
+    if (pp->fused) {
+        for (const FusedItem &it : pp->plan.fused) {
+            if (it.src.size() > 64 || (it.kind == FK_TREE && it.nleaf > 32)) {
+                pp->fused = false;   // beyond what the fused kernels encode
+            }
+        }
+    }
+    if (!pp->fused && pp->plan.scratchBytes > 0) {
+        HcclResult r = EnsureScratch(g, pp->plan.scratchBytes);
+        if (r != HCCL_SUCCESS) {
+            return r;
+        }
+    }
+    pp->scratchGen = g->scratchGen;
+    HcclResult r = BuildTables(g, pp.get(), reduceColl, g->sig.dtype, g->sig.op);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if (g->cfg.graph && !pp->launches.empty()) {
+        r = BuildGraph(pp.get());
+        if (r != HCCL_SUCCESS) {
+            return r;
+        }
+    }
+    OpInfo &info = pp->info;
+    info.coll = g->sig.coll;
+    info.algo = algo;
+    info.fused = pp->fused ? 1 : 0;
+    info.graph = pp->exec ? 1 : 0;
+    info.launches = uint32_t(pp->launches.size());
+    info.bytesRead = pp->fused ? pp->plan.fusedRead : pp->plan.stepRead;
+    info.bytesWritten = pp->fused ? pp->plan.fusedWritten : pp->plan.stepWritten;
+    info.stepRead = pp->plan.stepRead;
+    info.stepWritten = pp->plan.stepWritten;
+    info.scratchBytes = pp->fused ? 0 : pp->plan.scratchBytes;
+    *out = std::move(pp);
+    return HCCL_SUCCESS;
+}
+
+}  // namespace
+
+Prepared::~Prepared()
+{
+    if (exec) {
+        (void)hipGraphExecDestroy(exec);
+    }
+    if (graph) {
+        (void)hipGraphDestroy(graph);
+    }
+    if (devTables) {
+        (void)hipFree(devTables);
+    }
+}
+
+Group::~Group()
+{
+    if (deviceReady) {
+        (void)hipDeviceSynchronize();
+    }
+    cache.clear();
+    for (hipEvent_t e : arriveEvents) {
+        if (e) {
+            (void)hipEventDestroy(e);
+        }
+    }
+    if (doneEvent) {
+        (void)hipEventDestroy(doneEvent);
+    }
+    for (void *s : scratch) {
+        if (s) {
+            (void)hipFree(s);
+        }
+    }
+}
+
+const char *CollName(int coll)
+{
+    switch (coll) {
+        case COLL_ALLREDUCE: return "AllReduce";
+        case COLL_REDUCESCATTER: return "ReduceScatter";
+        case COLL_ALLGATHER: return "AllGather";
+        case COLL_ALLTOALLV: return "AlltoAllV";
+        default: return "?";
+    }
+}
+
+int DefaultAlgo(int coll) { return coll == COLL_ALLTOALLV ? ALGO_PAIRWISE : ALGO_RING; }
+
+HcclResult IssueCollective(Group *g, uint32_t launcher)
+{
+    HcclResult r = EnsureDevice(g, false);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    int algo = g->cfg.algo >= 0 ? g->cfg.algo : DefaultAlgo(g->sig.coll);
+    if (g->sig.coll == COLL_ALLTOALLV) {
+        algo = ALGO_PAIRWISE;
+    } else if (algo == ALGO_PAIRWISE || (algo == ALGO_RHD && g->sig.coll != COLL_ALLREDUCE)) {
+        algo = ALGO_RING;
+    }
+    std::string key = CacheKey(g, algo);
+    Prepared *pp = nullptr;
+    auto it = g->cache.find(key);
+    bool hit = false;
+    if (it != g->cache.end() && it->second->scratchGen == g->scratchGen) {
+        pp = it->second.get();
+        hit = true;
+    } else {
+        if (it != g->cache.end()) {
+            HIP_OK(hipDeviceSynchronize());
+            g->cache.erase(it);
+        }
+        if (g->cache.size() >= 64) {
+            // drop the least recently used entry; it may still be in flight on some stream
+            HIP_OK(hipDeviceSynchronize());
+            auto victim = g->cache.begin();
+            for (auto c = g->cache.begin(); c != g->cache.end(); ++c) {
+                if (c->second->lastUse < victim->second->lastUse) {
+                    victim = c;
+                }
+            }
+            g->cache.erase(victim);
+        }
+        std::unique_ptr<Prepared> fresh;
+        r = Prepare(g, algo, &fresh);
+        if (r != HCCL_SUCCESS) {
+            return r;
+        }
+        pp = fresh.get();
+        g->cache[key] = std::move(fresh);
+    }
+    pp->lastUse = ++g->useClock;
+    g->lastInfo = pp->info;
+    g->lastInfo.cacheHit = hit ? 1 : 0;
+
+    // Order the launch after whatever the other ranks' streams were doing when they arrived, and
+    // order those streams after the collective.
+    hipStream_t ls = g->streams[launcher];
+    bool others = false;
+    for (uint32_t k = 0; k < g->p; k++) {
+        if (k != launcher && g->streams[k] != ls) {
+            HIP_OK(hipStreamWaitEvent(ls, g->arriveEvents[k], 0));
+            others = true;
+        }
+    }
+    if (pp->exec) {
+        HIP_OK(hipGraphLaunch(pp->exec, ls));
+    } else {
+        for (LaunchRec &l : pp->launches) {
+            void *args[5];
+            KernelArgs(l, args);
+            HIP_OK(hipLaunchKernel(l.func, dim3(l.grid, 1, 1), dim3(kBlockThreads, 1, 1), args, 0, ls));
+        }
+    }
+    if (others) {
+        HIP_OK(hipEventRecord(g->doneEvent, ls));
+        for (uint32_t k = 0; k < g->p; k++) {
+            if (k != launcher && g->streams[k] != ls) {
+                HIP_OK(hipStreamWaitEvent(g->streams[k], g->doneEvent, 0));
+            }
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+}  // namespace hcclamd

@@ -1,0 +1,63 @@
+// Device-side contract between the executor and the gfx950 kernels.
+//
+// These kernels stand where the reference has its closed Reducer / Sender / Transport leaf
+// (call sites ALG/base/alg_template/temp_reduce_scatter/reduce_scatter_ring.cc:31-87) and its AIV
+// copy / atomic-reduce kernels (ALG/base/alg_aiv_template/aiv_communication_base.h:367-485):
+// element-wise dst = a (+) b and plain copies between rank buffers, all in one GPU's HBM.
+#pragma once
+#include <cstdint>
+
+namespace hcclamd {
+
+// One workgroup iteration handles one tile: 256 lanes x 16 bytes x 4.
+constexpr uint32_t kTileBytes = 16384;
+constexpr uint32_t kBlockThreads = 256;
+
+// How a step's bytes may be accessed.
+enum AccessMode : uint32_t {
+    ACC_VEC16 = 0,      // every pointer 16-byte aligned, byte count a multiple of 16
+    ACC_VEC16_SRC4 = 1, // destinations 16-byte aligned, sources only 4-byte aligned, multiple of 16
+    ACC_ELEM = 2        // element by element (heads, tails, unaligned buffers)
+};
+
+// dst = a            when b == nullptr
+// dst = a (+) b      otherwise (a = the rank's own operand, b = the peer's)
+struct StepDesc {
+    void *dst;
+    const void *a;
+    const void *b;
+    uint64_t bytes;
+    uint32_t tile0;     // index of this step's first tile inside the launch
+    uint32_t mode;      // AccessMode
+};
+
+// Fused item: read nsrc sources once, combine in the schedule's order, write ndst destinations.
+//   chain : acc = src[0]; for j = 1..nsrc-1: acc = bit j of accLeftMask ? acc (+) src[j] : src[j] (+) acc
+//   tree  : nleaf leaves, leaf i = src[2i] (+) src[2i+1] (src[2i+1] may be null); then
+//           v[i] = v[i] (+) v[i+w] for w = 1, 2, 4, ... ; result v[0]
+struct FusedDesc {
+    uint64_t bytes;
+    uint64_t accLeftMask;
+    uint32_t tile0;
+    uint32_t mode;
+    uint32_t nsrc;
+    uint32_t ndst;
+    uint32_t srcBase;   // index into the source pointer pool
+    uint32_t dstBase;   // index into the destination pointer pool
+    uint32_t nleaf;
+    uint32_t pad;
+};
+
+enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE8 = 2, KK_TREE32 = 3, KK_COUNT = 4 };
+
+// Kernel entry for (data type, reduce op, kind); nullptr if the combination is not built.
+// Signatures:
+//   KK_STEP            (const StepDesc *steps, uint32_t nsteps, uint32_t ntiles)
+//   KK_CHAIN / KK_TREE (const FusedDesc *items, uint32_t nitems, uint32_t ntiles,
+//                       const void *const *srcPool, void *const *dstPool)
+const void *LookupKernel(int hcclDataType, int hcclReduceOp, KernelKind kind);
+
+// Byte-wise variants for pure data movement (all-gather, all-to-all-v): KK_STEP and KK_CHAIN only.
+const void *LookupCopyKernel(KernelKind kind);
+
+}  // namespace hcclamd

@@ -1,0 +1,483 @@
+// gfx950 kernels for the per-rank data path: element-wise reduce / copy over descriptor tables.
+// Bandwidth-bound work: 128-bit coalesced loads and stores, several independent loads in flight per
+// lane, no LDS, no matrix cores.  One launch covers every step of a phase (or every fused item) for
+// all ranks; a workgroup walks tiles of kTileBytes with a grid stride.
+//
+// Arithmetic rules (must match bit for bit on every path):
+//   integers   sum / prod wrap modulo 2^n; max = (b > a) ? b : a, min = (b < a) ? b : a
+//   fp32/fp64  one IEEE operation per combine, same max / min selection rule
+//   fp16/bf16  widen to fp32, combine, round to nearest even; max / min keep the chosen operand's bits
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+#include "kernels.h"
+
+namespace hcclamd {
+
+typedef uint32_t V4 __attribute__((ext_vector_type(4)));   // 16 bytes, one global_load_dwordx4
+
+struct HalfBits { uint16_t v; };
+struct Bf16Bits { uint16_t v; };
+
+enum : int { ROP_SUM = 0, ROP_PROD = 1, ROP_MAX = 2, ROP_MIN = 3 };
+
+// ---- element arithmetic ---------------------------------------------------------------------------
+template <typename T> struct UnsignedOf { using type = T; };
+template <> struct UnsignedOf<int8_t> { using type = uint8_t; };
+template <> struct UnsignedOf<int16_t> { using type = uint16_t; };
+template <> struct UnsignedOf<int32_t> { using type = uint32_t; };
+template <> struct UnsignedOf<int64_t> { using type = uint64_t; };
+
+template <typename T, int OP> struct Elem {
+    // integers
+    static __device__ __forceinline__ T Apply(T a, T b)
+    {
+        using U = typename UnsignedOf<T>::type;
+        if (OP == ROP_SUM) {
+            return static_cast<T>(static_cast<U>(static_cast<uint32_t>(static_cast<U>(a)) + static_cast<uint32_t>(static_cast<U>(b))));
+        } else if (OP == ROP_PROD) {
+            return static_cast<T>(static_cast<U>(static_cast<uint32_t>(static_cast<U>(a)) * static_cast<uint32_t>(static_cast<U>(b))));
+        } else if (OP == ROP_MAX) {
+            return (b > a) ? b : a;
+        } else {
+            return (b < a) ? b : a;
+        }
+    }
+};
+template <typename T, int OP> struct Elem64 {
+    static __device__ __forceinline__ T Apply(T a, T b)
+    {
+        if (OP == ROP_SUM) {
+            return static_cast<T>(static_cast<uint64_t>(a) + static_cast<uint64_t>(b));
+        } else if (OP == ROP_PROD) {
+            return static_cast<T>(static_cast<uint64_t>(a) * static_cast<uint64_t>(b));
+        } else if (OP == ROP_MAX) {
+            return (b > a) ? b : a;
+        } else {
+            return (b < a) ? b : a;
+        }
+    }
+};
+template <int OP> struct Elem<int64_t, OP> : Elem64<int64_t, OP> {};
+template <int OP> struct Elem<uint64_t, OP> : Elem64<uint64_t, OP> {};
+
+template <typename F, int OP> struct ElemFloat {
+    static __device__ __forceinline__ F Apply(F a, F b)
+    {
+        if (OP == ROP_SUM) {
+            return a + b;
+        } else if (OP == ROP_PROD) {
+            return a * b;
+        } else if (OP == ROP_MAX) {
+            return (b > a) ? b : a;
+        } else {
+            return (b < a) ? b : a;
+        }
+    }
+};
+template <int OP> struct Elem<float, OP> : ElemFloat<float, OP> {};
+template <int OP> struct Elem<double, OP> : ElemFloat<double, OP> {};
+
+__device__ __forceinline__ float Bf16ToFloat(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
+__device__ __forceinline__ uint16_t FloatToBf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        return static_cast<uint16_t>((u >> 16) | 0x0040u);
+    }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+__device__ __forceinline__ float HalfToFloat(uint16_t h)
+{
+    _Float16 x;
+    __builtin_memcpy(&x, &h, 2);
+    return static_cast<float>(x);
+}
+__device__ __forceinline__ uint16_t FloatToHalf(float f)
+{
+    _Float16 x = static_cast<_Float16>(f);   // v_cvt_f16_f32, round to nearest even
+    uint16_t h;
+    __builtin_memcpy(&h, &x, 2);
+    return h;
+}
+
+template <int OP> struct Elem<HalfBits, OP> {
+    static __device__ __forceinline__ HalfBits Apply(HalfBits a, HalfBits b)
+    {
+        float fa = HalfToFloat(a.v), fb = HalfToFloat(b.v);
+        HalfBits r;
+        if (OP == ROP_SUM) {
+            r.v = FloatToHalf(fa + fb);
+        } else if (OP == ROP_PROD) {
+            r.v = FloatToHalf(fa * fb);
+        } else if (OP == ROP_MAX) {
+            r.v = (fb > fa) ? b.v : a.v;
+        } else {
+            r.v = (fb < fa) ? b.v : a.v;
+        }
+        return r;
+    }
+};
+template <int OP> struct Elem<Bf16Bits, OP> {
+    static __device__ __forceinline__ Bf16Bits Apply(Bf16Bits a, Bf16Bits b)
+    {
+        float fa = Bf16ToFloat(a.v), fb = Bf16ToFloat(b.v);
+        Bf16Bits r;
+        if (OP == ROP_SUM) {
+            r.v = FloatToBf16(fa + fb);
+        } else if (OP == ROP_PROD) {
+            r.v = FloatToBf16(fa * fb);
+        } else if (OP == ROP_MAX) {
+            r.v = (fb > fa) ? b.v : a.v;
+        } else {
+            r.v = (fb < fa) ? b.v : a.v;
+        }
+        return r;
+    }
+};
+
+// 16 bytes of T combined lane by lane; a is the rank's own operand, b the peer's.
+template <typename T, int OP> __device__ __forceinline__ V4 Combine16(V4 a, V4 b)
+{
+    constexpr int N = 16 / sizeof(T);
+    union U {
+        V4 v;
+        T e[N];
+        __device__ U() {}
+    } ua, ub, ur;
+    ua.v = a;
+    ub.v = b;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        ur.e[i] = Elem<T, OP>::Apply(ua.e[i], ub.e[i]);
+    }
+    return ur.v;
+}
+
+// ---- memory access ---------------------------------------------------------------------------------
+struct __attribute__((packed, aligned(4))) Vec16A4 {
+    uint32_t x, y, z, w;
+};
+
+template <uint32_t MODE> __device__ __forceinline__ V4 Load16(const void *base, uint64_t byteOff)
+{
+    const char *p = static_cast<const char *>(base) + byteOff;
+    if (MODE == ACC_VEC16) {
+        return __builtin_nontemporal_load(reinterpret_cast<const V4 *>(p));
+    } else {
+        Vec16A4 t = *reinterpret_cast<const Vec16A4 *>(p);
+        return V4{t.x, t.y, t.z, t.w};
+    }
+}
+__device__ __forceinline__ void Store16(void *base, uint64_t byteOff, V4 v)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<V4 *>(static_cast<char *>(base) + byteOff));
+}
+
+// Largest i with table[i].tile0 <= tile (tile0 is ascending, table[0].tile0 == 0).
+template <typename D> __device__ __forceinline__ uint32_t FindDesc(const D *table, uint32_t n, uint32_t tile)
+{
+    uint32_t lo = 0, hi = n;
+    while (hi - lo > 1) {
+        uint32_t mid = (lo + hi) >> 1;
+        if (table[mid].tile0 <= tile) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    return lo;
+}
+
+constexpr uint32_t kVecPerLane = kTileBytes / (kBlockThreads * 16);   // 4
+
+// ---- one phase of copy / reduce steps -----------------------------------------------------------------
+template <typename T, int OP, uint32_t MODE>
+__device__ __forceinline__ void StepTileVec(const StepDesc &d, uint64_t off, uint32_t n)
+{
+    const uint32_t nvec = n >> 4;
+    const uint32_t tid = threadIdx.x;
+    if (nvec == kTileBytes / 16) {
+        V4 va[kVecPerLane], vb[kVecPerLane];
+#pragma unroll
+        for (uint32_t u = 0; u < kVecPerLane; u++) {
+            va[u] = Load16<MODE>(d.a, off + (uint64_t(u) * kBlockThreads + tid) * 16);
+        }
+        if (d.b != nullptr) {
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerLane; u++) {
+                vb[u] = Load16<MODE>(d.b, off + (uint64_t(u) * kBlockThreads + tid) * 16);
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerLane; u++) {
+                va[u] = Combine16<T, OP>(va[u], vb[u]);
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < kVecPerLane; u++) {
+            Store16(d.dst, off + (uint64_t(u) * kBlockThreads + tid) * 16, va[u]);
+        }
+    } else {
+        for (uint32_t i = tid; i < nvec; i += kBlockThreads) {
+            V4 v = Load16<MODE>(d.a, off + uint64_t(i) * 16);
+            if (d.b != nullptr) {
+                v = Combine16<T, OP>(v, Load16<MODE>(d.b, off + uint64_t(i) * 16));
+            }
+            Store16(d.dst, off + uint64_t(i) * 16, v);
+        }
+    }
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ void StepTileElem(const StepDesc &d, uint64_t off, uint32_t n)
+{
+    const uint32_t cnt = n / sizeof(T);
+    T *dst = reinterpret_cast<T *>(static_cast<char *>(d.dst) + off);
+    const T *a = reinterpret_cast<const T *>(static_cast<const char *>(d.a) + off);
+    const T *b = d.b ? reinterpret_cast<const T *>(static_cast<const char *>(d.b) + off) : nullptr;
+    for (uint32_t i = threadIdx.x; i < cnt; i += kBlockThreads) {
+        T v = a[i];
+        if (b != nullptr) {
+            v = Elem<T, OP>::Apply(v, b[i]);
+        }
+        dst[i] = v;
+    }
+}
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(kBlockThreads) StepKernel(const StepDesc *__restrict__ steps, uint32_t nsteps, uint32_t ntiles)
+{
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const StepDesc d = steps[FindDesc(steps, nsteps, tile)];
+        const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
+        const uint64_t left = d.bytes - off;
+        const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
+        if (d.mode == ACC_VEC16) {
+            StepTileVec<T, OP, ACC_VEC16>(d, off, n);
+        } else if (d.mode == ACC_VEC16_SRC4) {
+            StepTileVec<T, OP, ACC_VEC16_SRC4>(d, off, n);
+        } else {
+            StepTileElem<T, OP>(d, off, n);
+        }
+    }
+}
+
+// ---- fused chain: read every source once, combine in schedule order, write every destination ----------
+constexpr uint32_t kChainVec = 2;      // vectors per lane per pass
+constexpr uint32_t kChainSrcBatch = 4; // sources whose loads are issued together
+
+template <typename T, int OP, uint32_t MODE>
+__device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *const *__restrict__ src,
+    void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec)
+{
+    // lane handles vectors vecBase + u * 256 + tid, u < kChainVec (guarded by nvec)
+    const uint32_t tid = threadIdx.x;
+    uint64_t pos[kChainVec];
+    bool live[kChainVec];
+#pragma unroll
+    for (uint32_t u = 0; u < kChainVec; u++) {
+        uint32_t i = vecBase + u * kBlockThreads + tid;
+        live[u] = i < nvec;
+        pos[u] = off + uint64_t(i) * 16;
+    }
+    V4 acc[kChainVec];
+    const void *s0 = src[0];
+#pragma unroll
+    for (uint32_t u = 0; u < kChainVec; u++) {
+        if (live[u]) {
+            acc[u] = Load16<MODE>(s0, pos[u]);
+        }
+    }
+    for (uint32_t j = 1; j < d.nsrc; j += kChainSrcBatch) {
+        V4 v[kChainSrcBatch][kChainVec];
+#pragma unroll
+        for (uint32_t jj = 0; jj < kChainSrcBatch; jj++) {
+            if (j + jj < d.nsrc) {
+                const void *s = src[j + jj];
+#pragma unroll
+                for (uint32_t u = 0; u < kChainVec; u++) {
+                    if (live[u]) {
+                        v[jj][u] = Load16<MODE>(s, pos[u]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t jj = 0; jj < kChainSrcBatch; jj++) {
+            if (j + jj < d.nsrc) {
+                const bool accLeft = (d.accLeftMask >> (j + jj)) & 1ull;
+#pragma unroll
+                for (uint32_t u = 0; u < kChainVec; u++) {
+                    if (live[u]) {
+                        acc[u] = accLeft ? Combine16<T, OP>(acc[u], v[jj][u]) : Combine16<T, OP>(v[jj][u], acc[u]);
+                    }
+                }
+            }
+        }
+    }
+    for (uint32_t k = 0; k < d.ndst; k++) {
+        void *o = dst[k];
+#pragma unroll
+        for (uint32_t u = 0; u < kChainVec; u++) {
+            if (live[u]) {
+                if (MODE == ACC_VEC16) {
+                    Store16(o, pos[u], acc[u]);
+                } else {
+                    Vec16A4 t{acc[u].x, acc[u].y, acc[u].z, acc[u].w};
+                    *reinterpret_cast<Vec16A4 *>(static_cast<char *>(o) + pos[u]) = t;
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ void ChainElem(const FusedDesc &d, const void *const *__restrict__ src,
+    void *const *__restrict__ dst, uint64_t off, uint32_t n)
+{
+    const uint32_t cnt = n / sizeof(T);
+    for (uint32_t i = threadIdx.x; i < cnt; i += kBlockThreads) {
+        const uint64_t at = off + uint64_t(i) * sizeof(T);
+        T acc = *reinterpret_cast<const T *>(static_cast<const char *>(src[0]) + at);
+        for (uint32_t j = 1; j < d.nsrc; j++) {
+            T v = *reinterpret_cast<const T *>(static_cast<const char *>(src[j]) + at);
+            acc = ((d.accLeftMask >> j) & 1ull) ? Elem<T, OP>::Apply(acc, v) : Elem<T, OP>::Apply(v, acc);
+        }
+        for (uint32_t k = 0; k < d.ndst; k++) {
+            *reinterpret_cast<T *>(static_cast<char *>(dst[k]) + at) = acc;
+        }
+    }
+}
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
+    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool)
+{
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const FusedDesc d = items[FindDesc(items, nitems, tile)];
+        const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
+        const uint64_t left = d.bytes - off;
+        const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
+        const void *const *src = srcPool + d.srcBase;
+        void *const *dst = dstPool + d.dstBase;
+        if (d.mode == ACC_ELEM) {
+            ChainElem<T, OP>(d, src, dst, off, n);
+        } else {
+            const uint32_t nvec = n >> 4;
+            for (uint32_t base = 0; base < nvec; base += kChainVec * kBlockThreads) {
+                if (d.mode == ACC_VEC16) {
+                    ChainVecPass<T, OP, ACC_VEC16>(d, src, dst, off, base, nvec);
+                } else {
+                    ChainVecPass<T, OP, ACC_VEC16_SRC4>(d, src, dst, off, base, nvec);
+                }
+            }
+        }
+    }
+}
+
+// ---- fused perfect tree (halving-doubling): leaves pairwise bottom-up ----------------------------------
+template <typename T, int OP, uint32_t MAXLEAF, uint32_t MODE>
+__device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *const *__restrict__ src,
+    void *const *__restrict__ dst, uint64_t pos)
+{
+    V4 v[MAXLEAF];
+#pragma unroll
+    for (uint32_t i = 0; i < MAXLEAF; i++) {
+        if (i < d.nleaf) {
+            v[i] = Load16<MODE>(src[2 * i], pos);
+        }
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < MAXLEAF; i++) {
+        if (i < d.nleaf) {
+            const void *s = src[2 * i + 1];
+            if (s != nullptr) {
+                v[i] = Combine16<T, OP>(v[i], Load16<MODE>(s, pos));
+            }
+        }
+    }
+#pragma unroll
+    for (uint32_t w = 1; w < MAXLEAF; w <<= 1) {
+        if (w < d.nleaf) {
+#pragma unroll
+            for (uint32_t i = 0; i + w < MAXLEAF; i += 2 * w) {
+                if (i + w < d.nleaf) {
+                    v[i] = Combine16<T, OP>(v[i], v[i + w]);
+                }
+            }
+        }
+    }
+    for (uint32_t k = 0; k < d.ndst; k++) {
+        if (MODE == ACC_VEC16) {
+            Store16(dst[k], pos, v[0]);
+        } else {
+            Vec16A4 t{v[0].x, v[0].y, v[0].z, v[0].w};
+            *reinterpret_cast<Vec16A4 *>(static_cast<char *>(dst[k]) + pos) = t;
+        }
+    }
+}
+
+template <typename T, int OP, uint32_t MAXLEAF>
+__device__ __forceinline__ void TreeElem(const FusedDesc &d, const void *const *__restrict__ src,
+    void *const *__restrict__ dst, uint64_t off, uint32_t n)
+{
+    const uint32_t cnt = n / sizeof(T);
+    for (uint32_t e = threadIdx.x; e < cnt; e += kBlockThreads) {
+        const uint64_t at = off + uint64_t(e) * sizeof(T);
+        T v[MAXLEAF];
+#pragma unroll
+        for (uint32_t i = 0; i < MAXLEAF; i++) {
+            if (i < d.nleaf) {
+                v[i] = *reinterpret_cast<const T *>(static_cast<const char *>(src[2 * i]) + at);
+                const void *s = src[2 * i + 1];
+                if (s != nullptr) {
+                    v[i] = Elem<T, OP>::Apply(v[i], *reinterpret_cast<const T *>(static_cast<const char *>(s) + at));
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t w = 1; w < MAXLEAF; w <<= 1) {
+            if (w < d.nleaf) {
+#pragma unroll
+                for (uint32_t i = 0; i + w < MAXLEAF; i += 2 * w) {
+                    if (i + w < d.nleaf) {
+                        v[i] = Elem<T, OP>::Apply(v[i], v[i + w]);
+                    }
+                }
+            }
+        }
+        for (uint32_t k = 0; k < d.ndst; k++) {
+            *reinterpret_cast<T *>(static_cast<char *>(dst[k]) + at) = v[0];
+        }
+    }
+}
+
+template <typename T, int OP, uint32_t MAXLEAF>
+__global__ void __launch_bounds__(kBlockThreads) TreeKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
+    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool)
+{
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const FusedDesc d = items[FindDesc(items, nitems, tile)];
+        const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
+        const uint64_t left = d.bytes - off;
+        const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
+        const void *const *src = srcPool + d.srcBase;
+        void *const *dst = dstPool + d.dstBase;
+        if (d.mode == ACC_ELEM) {
+            TreeElem<T, OP, MAXLEAF>(d, src, dst, off, n);
+        } else {
+            const uint32_t nvec = n >> 4;
+            for (uint32_t i = threadIdx.x; i < nvec; i += kBlockThreads) {
+                if (d.mode == ACC_VEC16) {
+                    TreeVecPass<T, OP, MAXLEAF, ACC_VEC16>(d, src, dst, off + uint64_t(i) * 16);
+                } else {
+                    TreeVecPass<T, OP, MAXLEAF, ACC_VEC16_SRC4>(d, src, dst, off + uint64_t(i) * 16);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace hcclamd

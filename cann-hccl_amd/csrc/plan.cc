@@ -1,0 +1,1084 @@
+// Planner implementation.  See plan.h for the reference interfaces this covers.
+//
+// Pipeline: (1) emit the schedule on "virtual" buffers the way the reference runs it on its CCL
+// staging buffers (partial results accumulate in the input buffer); (2) lower to the caller's
+// buffers without touching a send buffer that is not also the receive buffer: partials are homed in
+// the receive buffer when it is large enough, else in scratch; (3) run the program symbolically to
+// check it (no read of unwritten memory, lowered == virtual) and to derive, per output range, the
+// reduction expression over the original inputs; (4) turn those expressions into fused items when
+// they are copies, chains or perfect trees.
+#include "plan.h"
+
+#include <algorithm>
+#include <map>
+#include <sstream>
+#include <tuple>
+#include <utility>
+
+namespace hcclamd {
+
+namespace {
+
+uint64_t RoundUpTo(uint64_t v, uint64_t d) { return d == 0 ? v : (v + d - 1) / d * d; }
+uint32_t Mod(int64_t v, uint32_t p) { int64_t m = v % static_cast<int64_t>(p); return static_cast<uint32_t>(m < 0 ? m + p : m); }
+
+Ref MkRef(uint32_t rank, uint8_t buf, uint64_t off)
+{
+    Ref r;
+    r.rank = rank;
+    r.buf = buf;
+    r.off = off;
+    return r;
+}
+
+// ---- virtual program ----------------------------------------------------------------------------
+// In the virtual program BUF_SEND names the schedule's input buffer (the reference's CCL-in copy,
+// which the schedule may overwrite) and BUF_RECV its output buffer.
+struct VProgram {
+    std::vector<Phase> phases;
+    std::vector<uint64_t> inBytes, outBytes;
+};
+
+void Emit(VProgram &vp, size_t phase, bool reduce, Ref dst, Ref a, Ref b, uint64_t bytes)
+{
+    if (bytes == 0) {
+        return;
+    }
+    if (vp.phases.size() <= phase) {
+        vp.phases.resize(phase + 1);
+    }
+    Step s;
+    s.reduce = reduce;
+    s.dst = dst;
+    s.a = a;
+    s.b = b;
+    s.bytes = bytes;
+    vp.phases[phase].steps.push_back(s);
+}
+void EmitCopy(VProgram &vp, size_t phase, Ref dst, Ref src, uint64_t bytes) { Emit(vp, phase, false, dst, src, Ref(), bytes); }
+void EmitReduce(VProgram &vp, size_t phase, Ref dst, Ref own, Ref peer, uint64_t bytes) { Emit(vp, phase, true, dst, own, peer, bytes); }
+
+uint64_t SpanBytes(const std::vector<Slice> &sl, uint32_t first, uint32_t n)
+{
+    uint64_t s = 0;
+    for (uint32_t i = first; i < first + n; i++) {
+        s += sl[i].size;
+    }
+    return s;
+}
+
+// Ring reduce-scatter over `in` slices; the last step of each rank writes (outBuf, outSl[rank]).
+// Phase k (k = 0..p-2): rank r combines its slice (r-2-k) with the left neighbour's copy of it.
+size_t RingReduceScatterPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t base, const std::vector<Slice> &in,
+    uint8_t outBuf, uint64_t outBase, const std::vector<Slice> &out)
+{
+    for (uint32_t k = 0; k + 1 < p; k++) {
+        bool last = (k + 2 == p);
+        for (uint32_t r = 0; r < p; r++) {
+            uint32_t s = Mod(static_cast<int64_t>(r) - 2 - k, p);
+            uint32_t left = Mod(static_cast<int64_t>(r) - 1, p);
+            Ref own = MkRef(r, BUF_SEND, base + in[s].off);
+            Ref peer = MkRef(left, BUF_SEND, base + in[s].off);
+            Ref dst = last ? MkRef(r, outBuf, outBase + out[s].off) : own;
+            EmitReduce(vp, phase0 + k, dst, own, peer, in[s].size);
+        }
+    }
+    return phase0 + (p - 1);
+}
+
+// Ring all-gather on the output buffer: phase k, rank r takes slice (r-1-k) from its left neighbour.
+size_t RingAllGatherPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t base, const std::vector<Slice> &sl)
+{
+    for (uint32_t k = 0; k + 1 < p; k++) {
+        for (uint32_t r = 0; r < p; r++) {
+            uint32_t s = Mod(static_cast<int64_t>(r) - 1 - k, p);
+            uint32_t left = Mod(static_cast<int64_t>(r) - 1, p);
+            EmitCopy(vp, phase0 + k, MkRef(r, BUF_RECV, base + sl[s].off), MkRef(left, BUF_RECV, base + sl[s].off), sl[s].size);
+        }
+    }
+    return phase0 + (p - 1);
+}
+
+// Deterministic mesh reduce-scatter: every rank slice is cut into (p-1) pieces, piece t follows the
+// peer order rotated by t, so that in each round the pieces of one rank read p-1 different peers.
+size_t MeshReduceScatterPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t base, const std::vector<Slice> &sl,
+    uint64_t align)
+{
+    uint32_t nstream = p > 2 ? p - 1 : 1;
+    for (uint32_t r = 0; r < p; r++) {
+        if (sl[r].size == 0) {
+            continue;
+        }
+        std::vector<Slice> pieces = RingSlicePlan(sl[r].size, nstream, align);
+        for (uint32_t t = 0; t < nstream; t++) {
+            for (uint32_t round = 1; round < p; round++) {
+                uint32_t order = (round + t - 1) % (p - 1);
+                uint32_t src = Mod(static_cast<int64_t>(r) - (order + 1), p);
+                uint64_t off = base + sl[r].off + pieces[t].off;
+                EmitReduce(vp, phase0 + round - 1, MkRef(r, BUF_SEND, off), MkRef(r, BUF_SEND, off), MkRef(src, BUF_SEND, off),
+                    pieces[t].size);
+            }
+        }
+    }
+    return phase0 + (p - 1);
+}
+
+// Mesh all-gather: every rank pulls slice d from rank d, all peers at once (one phase).
+size_t MeshAllGatherPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t base, const std::vector<Slice> &sl)
+{
+    for (uint32_t r = 0; r < p; r++) {
+        for (uint32_t k = 1; k < p; k++) {
+            uint32_t d = (r + k) % p;
+            EmitCopy(vp, phase0, MkRef(r, BUF_RECV, base + sl[d].off), MkRef(d, BUF_RECV, base + sl[d].off), sl[d].size);
+        }
+    }
+    return phase0 + 1;
+}
+
+void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t bytes, uint64_t align)
+{
+    if (p == 1) {
+        EmitCopy(vp, 0, MkRef(0, BUF_RECV, base), MkRef(0, BUF_SEND, base), bytes);
+        return;
+    }
+    if (algo == ALGO_RING || algo == ALGO_MESH) {
+        std::vector<Slice> sl = RingSlicePlan(bytes, p, align);
+        size_t ph = 0;
+        if (algo == ALGO_RING) {
+            // the ring template runs its reduce-scatter with output == input
+            ph = RingReduceScatterPhases(vp, ph, p, base, sl, BUF_SEND, base, sl);
+        } else {
+            ph = MeshReduceScatterPhases(vp, ph, p, base, sl, align);
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            EmitCopy(vp, ph, MkRef(r, BUF_RECV, base + sl[r].off), MkRef(r, BUF_SEND, base + sl[r].off), sl[r].size);
+        }
+        ph++;
+        if (algo == ALGO_RING) {
+            RingAllGatherPhases(vp, ph, p, base, sl);
+        } else {
+            MeshAllGatherPhases(vp, ph, p, base, sl);
+        }
+        return;
+    }
+    // recursive halving-doubling
+    uint32_t block, part1;
+    HalvingDoublingShape(p, &block, &part1);
+    std::vector<Slice> sl = RingSlicePlan(bytes, block, align);
+    std::vector<uint32_t> rankOf(block);
+    for (uint32_t i = 0; i < p; i++) {
+        if (i < part1 && (i & 1)) {
+            continue;
+        }
+        rankOf[i < part1 ? i / 2 : i - part1 / 2] = i;
+    }
+    uint32_t steps = 0;
+    while ((1u << steps) < block) {
+        steps++;
+    }
+    size_t ph = 0;
+    if (part1 > 0) {
+        for (uint32_t e = 0; e < part1; e += 2) {   // fold the odd rank of each pair into the even one
+            EmitReduce(vp, ph, MkRef(e, BUF_SEND, base), MkRef(e, BUF_SEND, base), MkRef(e + 1, BUF_SEND, base), bytes);
+        }
+        ph++;
+    }
+    for (uint32_t s = 0; s < steps; s++) {           // halving: keep the half that contains the own slice
+        uint32_t mask = 1u << (steps - s - 1);
+        for (uint32_t q = 0; q < block; q++) {
+            uint32_t first = q & ~(mask - 1);
+            uint64_t off = base + sl[first].off;
+            EmitReduce(vp, ph, MkRef(rankOf[q], BUF_SEND, off), MkRef(rankOf[q], BUF_SEND, off),
+                MkRef(rankOf[q ^ mask], BUF_SEND, off), SpanBytes(sl, first, mask));
+        }
+        ph++;
+    }
+    for (uint32_t q = 0; q < block; q++) {
+        EmitCopy(vp, ph, MkRef(rankOf[q], BUF_RECV, base + sl[q].off), MkRef(rankOf[q], BUF_SEND, base + sl[q].off), sl[q].size);
+    }
+    ph++;
+    for (uint32_t s = 0; s < steps; s++) {           // doubling: fetch the peer's gathered range
+        uint32_t mask = 1u << s;
+        for (uint32_t q = 0; q < block; q++) {
+            uint32_t peer = q ^ mask;
+            uint32_t first = peer & ~(mask - 1);
+            uint64_t off = base + sl[first].off;
+            EmitCopy(vp, ph, MkRef(rankOf[q], BUF_RECV, off), MkRef(rankOf[peer], BUF_RECV, off), SpanBytes(sl, first, mask));
+        }
+        ph++;
+    }
+    if (part1 > 0) {
+        for (uint32_t e = 0; e < part1; e += 2) {   // unfold: the odd rank receives the whole result
+            EmitCopy(vp, ph, MkRef(e + 1, BUF_RECV, base), MkRef(e, BUF_RECV, base), bytes);
+        }
+    }
+}
+
+int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
+{
+    uint32_t p = rq.p;
+    uint64_t u = rq.unit;
+    vp->inBytes.assign(p, 0);
+    vp->outBytes.assign(p, 0);
+    if (rq.coll == COLL_ALLTOALLV) {
+        if (rq.sendCounts.size() != size_t(p) * p || rq.sdispls.size() != size_t(p) * p ||
+            rq.recvCounts.size() != size_t(p) * p || rq.rdispls.size() != size_t(p) * p) {
+            *err = "all-to-all-v tables must be p x p";
+            return 1;
+        }
+        // phase i: rank r's block for rank (r+i) goes straight into that rank's receive buffer
+        for (uint32_t i = 0; i < p; i++) {
+            for (uint32_t r = 0; r < p; r++) {
+                uint32_t n = (r + i) % p;
+                uint64_t cnt = rq.sendCounts[size_t(r) * p + n];
+                uint64_t so = rq.sdispls[size_t(r) * p + n] * u, ro = rq.rdispls[size_t(n) * p + r] * u;
+                EmitCopy(*vp, i, MkRef(n, BUF_RECV, ro), MkRef(r, BUF_SEND, so), cnt * u);
+                if (cnt) {
+                    vp->inBytes[r] = std::max(vp->inBytes[r], so + cnt * u);
+                    vp->outBytes[n] = std::max(vp->outBytes[n], ro + cnt * u);
+                }
+            }
+        }
+        return 0;
+    }
+    if (rq.algo == ALGO_PAIRWISE || (rq.algo == ALGO_RHD && rq.coll != COLL_ALLREDUCE)) {
+        *err = "algorithm not available for this collective";
+        return 1;
+    }
+    std::vector<uint64_t> chunks = ChunkCounts(rq.coll, rq.count, rq.unit, p, rq.cclBytes, rq.align);
+    if (rq.count > 0 && chunks.empty()) {
+        *err = "CCL buffer too small for one element per rank";
+        return 1;
+    }
+    uint64_t total = rq.count * u;
+    uint64_t done = 0;
+    for (uint64_t cur : chunks) {
+        uint64_t bytes = cur * u;
+        if (rq.coll == COLL_ALLREDUCE) {
+            AllReduceChunk(*vp, rq.algo, p, done, bytes, rq.align);
+        } else if (rq.coll == COLL_REDUCESCATTER) {
+            // input slice i of this chunk sits at i * total + done in the caller's layout
+            std::vector<Slice> in(p), out(p);
+            for (uint32_t i = 0; i < p; i++) {
+                in[i] = Slice{uint64_t(i) * total + done, bytes};
+                out[i] = Slice{done, bytes};
+            }
+            if (p == 1) {
+                EmitCopy(*vp, 0, MkRef(0, BUF_RECV, done), MkRef(0, BUF_SEND, done), bytes);
+            } else if (rq.algo == ALGO_RING) {
+                RingReduceScatterPhases(*vp, 0, p, 0, in, BUF_RECV, 0, out);
+            } else {
+                size_t ph = MeshReduceScatterPhases(*vp, 0, p, 0, in, rq.align);
+                for (uint32_t r = 0; r < p; r++) {
+                    EmitCopy(*vp, ph, MkRef(r, BUF_RECV, done), MkRef(r, BUF_SEND, in[r].off), bytes);
+                }
+            }
+        } else {
+            std::vector<Slice> sl(p);
+            for (uint32_t i = 0; i < p; i++) {
+                sl[i] = Slice{uint64_t(i) * total + done, bytes};
+            }
+            for (uint32_t r = 0; r < p; r++) {
+                EmitCopy(*vp, 0, MkRef(r, BUF_RECV, sl[r].off), MkRef(r, BUF_SEND, done), bytes);
+            }
+            if (p > 1) {
+                if (rq.algo == ALGO_RING) {
+                    RingAllGatherPhases(*vp, 1, p, 0, sl);
+                } else {
+                    MeshAllGatherPhases(*vp, 1, p, 0, sl);
+                }
+            }
+        }
+        done += bytes;
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        vp->inBytes[r] = (rq.coll == COLL_REDUCESCATTER) ? total * p : total;
+        vp->outBytes[r] = (rq.coll == COLL_ALLGATHER) ? total * p : total;
+    }
+    return 0;
+}
+
+// ---- interval set ---------------------------------------------------------------------------------
+class RangeSet {
+public:
+    void Add(uint64_t b, uint64_t e)
+    {
+        if (b >= e) {
+            return;
+        }
+        auto it = m_.upper_bound(b);
+        if (it != m_.begin()) {
+            auto pv = std::prev(it);
+            if (pv->second >= b) {
+                b = pv->first;
+                e = std::max(e, pv->second);
+                it = m_.erase(pv);
+            }
+        }
+        while (it != m_.end() && it->first <= e) {
+            e = std::max(e, it->second);
+            it = m_.erase(it);
+        }
+        m_[b] = e;
+    }
+    // Boundaries of set membership strictly inside (b, e).
+    void Cuts(uint64_t b, uint64_t e, std::vector<uint64_t> *out) const
+    {
+        for (auto it = m_.begin(); it != m_.end(); ++it) {
+            if (it->first > b && it->first < e) {
+                out->push_back(it->first);
+            }
+            if (it->second > b && it->second < e) {
+                out->push_back(it->second);
+            }
+        }
+    }
+    bool Contains(uint64_t x) const
+    {
+        auto it = m_.upper_bound(x);
+        if (it == m_.begin()) {
+            return false;
+        }
+        --it;
+        return x < it->second;
+    }
+
+private:
+    std::map<uint64_t, uint64_t> m_;
+};
+
+// ---- lowering -------------------------------------------------------------------------------------
+// home: where writes to the virtual input buffer go (BUF_RECV or BUF_SCRATCH).
+void Lower(const VProgram &vp, const PlanRequest &rq, uint8_t home, bool stage, std::vector<Phase> *out)
+{
+    uint32_t p = rq.p;
+    std::vector<RangeSet> written(p);
+    out->clear();
+    if (stage) {
+        Phase ph;
+        for (uint32_t r = 0; r < p; r++) {
+            if (vp.inBytes[r] == 0) {
+                continue;
+            }
+            Step s;
+            s.dst = MkRef(r, BUF_SCRATCH, 0);
+            s.a = MkRef(r, BUF_SEND, 0);
+            s.bytes = vp.inBytes[r];
+            ph.steps.push_back(s);
+            written[r].Add(0, vp.inBytes[r]);
+        }
+        if (!ph.steps.empty()) {
+            out->push_back(ph);
+        }
+        home = BUF_SCRATCH;
+    }
+    for (const Phase &vph : vp.phases) {
+        Phase ph;
+        std::vector<std::tuple<uint32_t, uint64_t, uint64_t>> marks;
+        for (const Step &vs : vph.steps) {
+            std::vector<uint64_t> cuts;   // relative to the step start
+            auto addCuts = [&](const Ref &ref) {
+                if (ref.buf != BUF_SEND) {
+                    return;
+                }
+                std::vector<uint64_t> abs;
+                written[ref.rank].Cuts(ref.off, ref.off + vs.bytes, &abs);
+                for (uint64_t c : abs) {
+                    cuts.push_back(c - ref.off);
+                }
+            };
+            addCuts(vs.a);
+            if (vs.reduce) {
+                addCuts(vs.b);
+            }
+            cuts.push_back(0);
+            cuts.push_back(vs.bytes);
+            std::sort(cuts.begin(), cuts.end());
+            cuts.erase(std::unique(cuts.begin(), cuts.end()), cuts.end());
+            for (size_t i = 0; i + 1 < cuts.size(); i++) {
+                uint64_t d = cuts[i], n = cuts[i + 1] - cuts[i];
+                auto mapRead = [&](const Ref &ref) {
+                    if (ref.buf == BUF_RECV) {
+                        return MkRef(ref.rank, BUF_RECV, ref.off + d);
+                    }
+                    bool w = written[ref.rank].Contains(ref.off + d);
+                    return MkRef(ref.rank, w ? home : uint8_t(BUF_SEND), ref.off + d);
+                };
+                Step s;
+                s.reduce = vs.reduce;
+                s.bytes = n;
+                s.a = mapRead(vs.a);
+                if (vs.reduce) {
+                    s.b = mapRead(vs.b);
+                }
+                s.dst = MkRef(vs.dst.rank, vs.dst.buf == BUF_SEND ? home : uint8_t(BUF_RECV), vs.dst.off + d);
+                bool aliased = rq.alias.size() == p && rq.alias[s.dst.rank];
+                auto same = [&](const Ref &x, const Ref &y) {
+                    if (x.rank != y.rank || x.off != y.off) {
+                        return false;
+                    }
+                    uint8_t bx = (aliased && x.buf == BUF_SEND) ? uint8_t(BUF_RECV) : x.buf;
+                    uint8_t by = (aliased && y.buf == BUF_SEND) ? uint8_t(BUF_RECV) : y.buf;
+                    return bx == by;
+                };
+                if (!s.reduce && same(s.dst, s.a)) {
+                    continue;   // the data is already where it has to be
+                }
+                ph.steps.push_back(s);
+            }
+            if (vs.dst.buf == BUF_SEND) {
+                marks.emplace_back(vs.dst.rank, vs.dst.off, vs.dst.off + vs.bytes);
+            }
+        }
+        for (auto &m : marks) {
+            written[std::get<0>(m)].Add(std::get<1>(m), std::get<2>(m));
+        }
+        if (!ph.steps.empty()) {
+            // Order steps by destination offset: the tile that produced a range in one phase and the
+            // tile that consumes it in the next then get the same index in both launches.
+            std::stable_sort(ph.steps.begin(), ph.steps.end(),
+                [](const Step &x, const Step &y) { return x.dst.off < y.dst.off; });
+            out->push_back(ph);
+        }
+    }
+}
+
+// ---- symbolic execution -----------------------------------------------------------------------------
+struct ENode {
+    bool red = false;
+    int a = -1, b = -1;
+    uint64_t da = 0, db = 0;
+    Ref leaf;
+};
+struct Region {
+    uint64_t len = 0;
+    int expr = -1;
+    uint64_t delta = 0;
+};
+struct Piece {
+    uint64_t rel, len;
+    int expr;
+    uint64_t delta;
+};
+
+struct Sym {
+    std::vector<ENode> nodes;
+    std::map<std::pair<uint32_t, uint8_t>, std::map<uint64_t, Region>> mem;
+    std::vector<uint8_t> alias;
+    std::string err;
+
+    std::pair<uint32_t, uint8_t> Key(const Ref &r) const
+    {
+        uint8_t b = r.buf;
+        if (b == BUF_SEND && r.rank < alias.size() && alias[r.rank]) {
+            b = BUF_RECV;
+        }
+        return std::make_pair(r.rank, b);
+    }
+    void Init(uint32_t rank, uint64_t bytes)
+    {
+        if (bytes == 0) {
+            return;
+        }
+        ENode n;
+        n.leaf = MkRef(rank, BUF_SEND, 0);
+        nodes.push_back(n);
+        Region rg;
+        rg.len = bytes;
+        rg.expr = int(nodes.size()) - 1;
+        mem[Key(MkRef(rank, BUF_SEND, 0))][0] = rg;
+    }
+    bool Read(const Ref &ref, uint64_t len, std::vector<Piece> *out)
+    {
+        auto mit = mem.find(Key(ref));
+        uint64_t pos = ref.off, end = ref.off + len;
+        if (mit != mem.end()) {
+            auto &m = mit->second;
+            auto it = m.upper_bound(pos);
+            if (it != m.begin()) {
+                --it;
+            }
+            for (; it != m.end() && it->first < end && pos < end; ++it) {
+                uint64_t rb = it->first, re = it->first + it->second.len;
+                if (re <= pos) {
+                    continue;
+                }
+                if (rb > pos) {
+                    break;
+                }
+                uint64_t take = std::min(re, end) - pos;
+                out->push_back(Piece{pos - ref.off, take, it->second.expr, it->second.delta + (pos - rb)});
+                pos += take;
+            }
+        }
+        if (pos < end) {
+            std::ostringstream os;
+            os << "read of unwritten memory: rank " << ref.rank << " buf " << int(ref.buf) << " offset " << pos;
+            err = os.str();
+            return false;
+        }
+        return true;
+    }
+    void Write(const Ref &ref, const std::vector<Piece> &pieces, uint64_t len)
+    {
+        auto &m = mem[Key(ref)];
+        uint64_t b = ref.off, e = ref.off + len;
+        auto it = m.upper_bound(b);
+        if (it != m.begin()) {
+            --it;
+        }
+        std::vector<std::pair<uint64_t, Region>> keep;
+        while (it != m.end() && it->first < e) {
+            uint64_t rb = it->first, re = it->first + it->second.len;
+            if (re <= b) {
+                ++it;
+                continue;
+            }
+            if (rb < b) {
+                Region l = it->second;
+                l.len = b - rb;
+                keep.emplace_back(rb, l);
+            }
+            if (re > e) {
+                Region r = it->second;
+                r.len = re - e;
+                r.delta += e - rb;
+                keep.emplace_back(e, r);
+            }
+            it = m.erase(it);
+        }
+        for (auto &k : keep) {
+            m[k.first] = k.second;
+        }
+        for (const Piece &pc : pieces) {
+            Region rg;
+            rg.len = pc.len;
+            rg.expr = pc.expr;
+            rg.delta = pc.delta;
+            m[b + pc.rel] = rg;
+        }
+    }
+    bool Run(const std::vector<Phase> &phases)
+    {
+        for (const Phase &ph : phases) {
+            std::vector<std::tuple<Ref, std::vector<Piece>, uint64_t>> writes;
+            for (const Step &s : ph.steps) {
+                std::vector<Piece> pa, pb, res;
+                if (!Read(s.a, s.bytes, &pa)) {
+                    return false;
+                }
+                if (!s.reduce) {
+                    res = pa;
+                } else {
+                    if (!Read(s.b, s.bytes, &pb)) {
+                        return false;
+                    }
+                    size_t i = 0, j = 0;
+                    uint64_t pos = 0;
+                    while (pos < s.bytes) {
+                        const Piece &x = pa[i], &y = pb[j];
+                        uint64_t end = std::min(x.rel + x.len, y.rel + y.len);
+                        ENode n;
+                        n.red = true;
+                        n.a = x.expr;
+                        n.da = x.delta + (pos - x.rel);
+                        n.b = y.expr;
+                        n.db = y.delta + (pos - y.rel);
+                        nodes.push_back(n);
+                        res.push_back(Piece{pos, end - pos, int(nodes.size()) - 1, 0});
+                        pos = end;
+                        if (x.rel + x.len == end) {
+                            i++;
+                        }
+                        if (y.rel + y.len == end) {
+                            j++;
+                        }
+                    }
+                }
+                writes.emplace_back(s.dst, std::move(res), s.bytes);
+            }
+            for (auto &w : writes) {
+                Write(std::get<0>(w), std::get<1>(w), std::get<2>(w));
+            }
+        }
+        return true;
+    }
+    // Canonical text of expression e evaluated at relative position `delta`; leaf offsets are printed
+    // minus `bias` (bias = 0: absolute source offsets; bias = destination start: position-independent
+    // form, equal for two adjacent ranges that continue one another).
+    void Canon(int e, uint64_t delta, uint64_t bias, std::string *out) const
+    {
+        const ENode &n = nodes[e];
+        if (!n.red) {
+            *out += "L" + std::to_string(n.leaf.rank) + ":" +
+                std::to_string(static_cast<long long>(n.leaf.off + delta) - static_cast<long long>(bias));
+            return;
+        }
+        *out += "(";
+        Canon(n.a, n.da + delta, bias, out);
+        *out += ",";
+        Canon(n.b, n.db + delta, bias, out);
+        *out += ")";
+    }
+};
+
+// Final contents of every receive buffer as maximal ranges of one expression each.
+struct OutRange {
+    uint32_t rank;
+    uint64_t start, len;
+    int expr;
+    uint64_t delta;
+    std::string rel;     // position-independent canonical form
+};
+std::vector<OutRange> Outputs(const Sym &sym, uint32_t p)
+{
+    std::vector<OutRange> v;
+    for (uint32_t r = 0; r < p; r++) {
+        auto it = sym.mem.find(std::make_pair(r, uint8_t(BUF_RECV)));
+        if (it == sym.mem.end()) {
+            continue;
+        }
+        for (auto &kv : it->second) {
+            OutRange o;
+            o.rank = r;
+            o.start = kv.first;
+            o.len = kv.second.len;
+            o.expr = kv.second.expr;
+            o.delta = kv.second.delta;
+            sym.Canon(o.expr, o.delta, o.start, &o.rel);
+            if (!v.empty() && v.back().rank == r && v.back().start + v.back().len == o.start && v.back().rel == o.rel) {
+                v.back().len += o.len;   // continuation of the previous range
+            } else {
+                v.push_back(std::move(o));
+            }
+        }
+    }
+    return v;
+}
+
+// Text that identifies the final receive-buffer contents independently of how ranges were split.
+std::string OutputSignature(const Sym &sym, uint32_t p)
+{
+    std::string sig;
+    for (const OutRange &o : Outputs(sym, p)) {
+        sig += "r" + std::to_string(o.rank) + "@" + std::to_string(o.start) + "+" + std::to_string(o.len) + "=" + o.rel + ";";
+    }
+    return sig;
+}
+
+// ---- expression -> fused item -------------------------------------------------------------------------
+Ref LeafRef(const Sym &sym, int e, uint64_t delta)
+{
+    Ref r = sym.nodes[e].leaf;
+    r.off += delta;
+    return r;
+}
+
+bool AsChain(const Sym &sym, int e, uint64_t delta, FusedItem *item)
+{
+    // walk from the outermost combine to the innermost; every level must have a leaf operand
+    std::vector<Ref> rev;
+    std::vector<uint8_t> revLeft;
+    for (;;) {
+        const ENode &n = sym.nodes[e];
+        if (!n.red) {
+            return false;
+        }
+        bool la = !sym.nodes[n.a].red, lb = !sym.nodes[n.b].red;
+        if (la && lb) {
+            rev.push_back(LeafRef(sym, n.b, n.db + delta));
+            revLeft.push_back(1);                 // acc (+) b with acc = a
+            rev.push_back(LeafRef(sym, n.a, n.da + delta));
+            revLeft.push_back(0);
+            break;
+        }
+        if (la) {
+            rev.push_back(LeafRef(sym, n.a, n.da + delta));
+            revLeft.push_back(0);                 // a (+) acc
+            uint64_t nd = n.db + delta;
+            e = n.b;
+            delta = nd;
+        } else if (lb) {
+            rev.push_back(LeafRef(sym, n.b, n.db + delta));
+            revLeft.push_back(1);                 // acc (+) b
+            uint64_t nd = n.da + delta;
+            e = n.a;
+            delta = nd;
+        } else {
+            return false;
+        }
+    }
+    item->kind = FK_CHAIN;
+    item->src.assign(rev.rbegin(), rev.rend());
+    item->accLeft.assign(revLeft.rbegin(), revLeft.rend());
+    item->srcValid.assign(item->src.size(), 1);
+    return true;
+}
+
+bool MatchTree(const Sym &sym, int e, uint64_t delta, uint32_t depth, FusedItem *item)
+{
+    const ENode &n = sym.nodes[e];
+    if (depth == 0) {
+        if (!n.red) {
+            item->src.push_back(LeafRef(sym, e, delta));
+            item->srcValid.push_back(1);
+            item->src.push_back(Ref());
+            item->srcValid.push_back(0);
+            return true;
+        }
+        if (!sym.nodes[n.a].red && !sym.nodes[n.b].red) {
+            item->src.push_back(LeafRef(sym, n.a, n.da + delta));
+            item->srcValid.push_back(1);
+            item->src.push_back(LeafRef(sym, n.b, n.db + delta));
+            item->srcValid.push_back(1);
+            return true;
+        }
+        return false;
+    }
+    if (!n.red) {
+        return false;
+    }
+    return MatchTree(sym, n.a, n.da + delta, depth - 1, item) && MatchTree(sym, n.b, n.db + delta, depth - 1, item);
+}
+
+bool AsTree(const Sym &sym, int e, uint64_t delta, FusedItem *item)
+{
+    for (uint32_t depth = 1; depth <= 5; depth++) {
+        FusedItem t;
+        if (MatchTree(sym, e, delta, depth, &t)) {
+            item->kind = FK_TREE;
+            item->src = t.src;
+            item->srcValid = t.srcValid;
+            item->nleaf = 1u << depth;
+            return true;
+        }
+    }
+    return false;
+}
+
+bool Overlap(uint64_t a, uint64_t al, uint64_t b, uint64_t bl) { return a < b + bl && b < a + al; }
+
+bool BuildFused(const Sym &sym, const PlanRequest &rq, std::vector<FusedItem> *items)
+{
+    std::vector<OutRange> outs = Outputs(sym, rq.p);
+    std::map<std::string, size_t> index;
+    for (const OutRange &o : outs) {
+        std::string key = std::to_string(o.len) + "|";
+        sym.Canon(o.expr, o.delta, 0, &key);
+        auto it = index.find(key);
+        if (it == index.end()) {
+            FusedItem item;
+            item.bytes = o.len;
+            if (!sym.nodes[o.expr].red) {
+                item.kind = FK_COPY;
+                item.src.push_back(LeafRef(sym, o.expr, o.delta));
+                item.srcValid.push_back(1);
+            } else if (!AsChain(sym, o.expr, o.delta, &item) && !AsTree(sym, o.expr, o.delta, &item)) {
+                return false;
+            }
+            items->push_back(item);
+            it = index.emplace(key, items->size() - 1).first;
+        }
+        (*items)[it->second].dst.push_back(MkRef(o.rank, BUF_RECV, o.start));
+    }
+    // A fused launch reads every source and writes every destination in one pass, so a destination
+    // may share memory with a source only when it is the same range of the same item (each thread
+    // then reads its bytes before it overwrites them).  Only aliased ranks can overlap.
+    auto phys = [&](const Ref &r) { return (r.buf == BUF_SEND && rq.alias.size() == rq.p && rq.alias[r.rank]) ? uint8_t(BUF_RECV) : r.buf; };
+    for (size_t i = 0; i < items->size(); i++) {
+        for (const Ref &d : (*items)[i].dst) {
+            for (size_t j = 0; j < items->size(); j++) {
+                const FusedItem &other = (*items)[j];
+                for (size_t k = 0; k < other.src.size(); k++) {
+                    if (!other.srcValid[k]) {
+                        continue;
+                    }
+                    const Ref &s = other.src[k];
+                    if (s.rank != d.rank || phys(s) != phys(d)) {
+                        continue;
+                    }
+                    if (Overlap(s.off, other.bytes, d.off, (*items)[i].bytes) && !(i == j && s.off == d.off)) {
+                        return false;
+                    }
+                }
+            }
+        }
+    }
+    return true;
+}
+
+// Hazard check of one phase: a destination may not overlap any other step's operands or destination.
+bool PhaseIsHazardFree(const Phase &ph, const std::vector<uint8_t> &alias, std::string *err)
+{
+    struct Acc { uint32_t rank; uint8_t buf; uint64_t off, len; size_t step; bool write; };
+    std::vector<Acc> acc;
+    auto phys = [&](const Ref &r) { return (r.buf == BUF_SEND && r.rank < alias.size() && alias[r.rank]) ? uint8_t(BUF_RECV) : r.buf; };
+    for (size_t i = 0; i < ph.steps.size(); i++) {
+        const Step &s = ph.steps[i];
+        acc.push_back(Acc{s.dst.rank, phys(s.dst), s.dst.off, s.bytes, i, true});
+        acc.push_back(Acc{s.a.rank, phys(s.a), s.a.off, s.bytes, i, false});
+        if (s.reduce) {
+            acc.push_back(Acc{s.b.rank, phys(s.b), s.b.off, s.bytes, i, false});
+        }
+    }
+    std::sort(acc.begin(), acc.end(), [](const Acc &x, const Acc &y) {
+        return std::tie(x.rank, x.buf, x.off) < std::tie(y.rank, y.buf, y.off);
+    });
+    for (size_t i = 0; i < acc.size(); i++) {
+        for (size_t j = i + 1; j < acc.size(); j++) {
+            if (acc[j].rank != acc[i].rank || acc[j].buf != acc[i].buf || acc[j].off >= acc[i].off + acc[i].len) {
+                break;
+            }
+            if (!acc[i].write && !acc[j].write) {
+                continue;
+            }
+            if (acc[i].step == acc[j].step && acc[i].off == acc[j].off) {
+                continue;   // a step may update its own operand in place
+            }
+            std::ostringstream os;
+            os << "hazard inside a phase at rank " << acc[i].rank << " buf " << int(acc[i].buf) << " offset " << acc[j].off;
+            *err = os.str();
+            return false;
+        }
+    }
+    return true;
+}
+
+void JsonRef(std::ostringstream &os, const Ref &r)
+{
+    os << "[" << r.rank << "," << int(r.buf) << "," << r.off << "]";
+}
+
+}  // namespace
+
+std::vector<Slice> RingSlicePlan(uint64_t total, uint32_t n, uint64_t align)
+{
+    std::vector<Slice> s(n);
+    uint64_t per = RoundUpTo((total + n - 1) / n, align);
+    uint64_t left = total;
+    for (uint32_t i = 0; i < n; i++) {
+        uint64_t cur = std::min(per, left);
+        s[i].off = total - left;
+        s[i].size = cur;
+        left -= cur;
+    }
+    return s;
+}
+
+void HalvingDoublingShape(uint32_t p, uint32_t *block, uint32_t *part1)
+{
+    uint32_t b = 1;
+    while (b * 2 <= p) {
+        b *= 2;
+    }
+    *block = b;
+    *part1 = 2 * (p - b);
+}
+
+std::vector<uint64_t> ChunkCounts(CollKind coll, uint64_t count, uint32_t unit, uint32_t p, uint64_t cclBytes,
+    uint64_t align)
+{
+    std::vector<uint64_t> v;
+    uint64_t per = (coll == COLL_ALLREDUCE) ? cclBytes / unit : cclBytes / p / align * align / unit;
+    if (per == 0) {
+        return v;
+    }
+    for (uint64_t left = count; left > 0;) {
+        uint64_t cur = std::min(left, per);
+        v.push_back(cur);
+        left -= cur;
+    }
+    return v;
+}
+
+int BuildPlan(const PlanRequest &rq, Plan *plan, std::string *err)
+{
+    if (rq.p == 0 || rq.unit == 0 || rq.align == 0) {
+        *err = "bad plan request";
+        return 1;
+    }
+    VProgram vp;
+    if (BuildVirtual(rq, &vp, err) != 0) {
+        return 1;
+    }
+    uint32_t p = rq.p;
+    std::vector<uint8_t> alias = rq.alias.size() == p ? rq.alias : std::vector<uint8_t>(p, 0);
+    plan->p = p;
+    plan->sendBytes = vp.inBytes;
+    plan->recvBytes = vp.outBytes;
+
+    // expected outputs: the virtual program with separate input and output buffers
+    Sym ref;
+    for (uint32_t r = 0; r < p; r++) {
+        ref.Init(r, vp.inBytes[r]);
+    }
+    if (!ref.Run(vp.phases)) {
+        *err = "virtual program: " + ref.err;
+        return 2;
+    }
+    std::string want = OutputSignature(ref, p);
+
+    // lowering candidates: partials in the receive buffer (no scratch), else in scratch, else staged
+    bool fits = true;
+    for (uint32_t r = 0; r < p; r++) {
+        fits = fits && vp.inBytes[r] <= vp.outBytes[r];
+    }
+    struct Cand { uint8_t home; bool stage; };
+    std::vector<Cand> cands;
+    if (!rq.stageInput) {
+        if (fits) {
+            cands.push_back(Cand{BUF_RECV, false});
+        }
+        cands.push_back(Cand{BUF_SCRATCH, false});
+    }
+    cands.push_back(Cand{BUF_SCRATCH, true});
+    bool ok = false;
+    std::string why;
+    Sym low;
+    for (const Cand &c : cands) {
+        std::vector<Phase> phases;
+        Lower(vp, rq, c.home, c.stage, &phases);
+        bool clean = true;
+        for (const Phase &ph : phases) {
+            if (!PhaseIsHazardFree(ph, alias, &why)) {
+                clean = false;
+                break;
+            }
+        }
+        if (!clean) {
+            continue;
+        }
+        Sym s;
+        s.alias = alias;
+        for (uint32_t r = 0; r < p; r++) {
+            s.Init(r, vp.inBytes[r]);
+        }
+        if (!s.Run(phases)) {
+            why = s.err;
+            continue;
+        }
+        if (OutputSignature(s, p) != want) {
+            why = "lowered program computes different outputs";
+            continue;
+        }
+        plan->phases = std::move(phases);
+        bool usesScratch = false;
+        for (const Phase &ph : plan->phases) {
+            for (const Step &st : ph.steps) {
+                usesScratch = usesScratch || st.dst.buf == BUF_SCRATCH;
+            }
+        }
+        plan->scratchBytes = 0;
+        if (usesScratch) {
+            for (uint32_t r = 0; r < p; r++) {
+                plan->scratchBytes = std::max(plan->scratchBytes, vp.inBytes[r]);
+            }
+        }
+        low = std::move(s);
+        ok = true;
+        break;
+    }
+    if (!ok) {
+        *err = "no safe lowering: " + why;
+        return 2;
+    }
+
+    plan->stepRead = plan->stepWritten = 0;
+    for (const Phase &ph : plan->phases) {
+        for (const Step &s : ph.steps) {
+            plan->stepRead += s.bytes * (s.reduce ? 2 : 1);
+            plan->stepWritten += s.bytes;
+        }
+    }
+
+    // fused form, derived from the virtual program's expressions (leaves are send-buffer ranges)
+    plan->fused.clear();
+    plan->fusedOk = BuildFused(ref, rq, &plan->fused);
+    plan->fusedRead = plan->fusedWritten = 0;
+    if (plan->fusedOk) {
+        for (FusedItem &it : plan->fused) {
+            uint64_t nsrc = 0;
+            for (uint8_t v : it.srcValid) {
+                nsrc += v;
+            }
+            plan->fusedRead += nsrc * it.bytes;
+            plan->fusedWritten += it.dst.size() * it.bytes;
+        }
+        // an aliased copy onto itself moves nothing
+        for (FusedItem &it : plan->fused) {
+            if (it.kind != FK_COPY) {
+                continue;
+            }
+            std::vector<Ref> keep;
+            for (const Ref &d : it.dst) {
+                bool self = d.rank == it.src[0].rank && d.off == it.src[0].off && alias[d.rank] && it.src[0].buf == BUF_SEND;
+                if (self) {
+                    plan->fusedWritten -= it.bytes;
+                } else {
+                    keep.push_back(d);
+                }
+            }
+            if (keep.empty()) {
+                plan->fusedRead -= it.bytes;
+            }
+            it.dst = keep;
+        }
+        plan->fused.erase(std::remove_if(plan->fused.begin(), plan->fused.end(),
+            [](const FusedItem &it) { return it.dst.empty(); }), plan->fused.end());
+    } else {
+        plan->fused.clear();
+    }
+    return 0;
+}
+
+std::string DescribePlan(const Plan &plan)
+{
+    std::ostringstream os;
+    os << "{\"p\":" << plan.p << ",\"scratchBytes\":" << plan.scratchBytes << ",\"fusedOk\":" << (plan.fusedOk ? "true" : "false")
+       << ",\"stepRead\":" << plan.stepRead << ",\"stepWritten\":" << plan.stepWritten << ",\"fusedRead\":" << plan.fusedRead
+       << ",\"fusedWritten\":" << plan.fusedWritten << ",\"phases\":[";
+    for (size_t i = 0; i < plan.phases.size(); i++) {
+        os << (i ? "," : "") << "[";
+        const Phase &ph = plan.phases[i];
+        for (size_t j = 0; j < ph.steps.size(); j++) {
+            const Step &s = ph.steps[j];
+            os << (j ? "," : "") << "{\"r\":" << (s.reduce ? 1 : 0) << ",\"n\":" << s.bytes << ",\"dst\":";
+            JsonRef(os, s.dst);
+            os << ",\"a\":";
+            JsonRef(os, s.a);
+            if (s.reduce) {
+                os << ",\"b\":";
+                JsonRef(os, s.b);
+            }
+            os << "}";
+        }
+        os << "]";
+    }
+    os << "],\"fused\":[";
+    for (size_t i = 0; i < plan.fused.size(); i++) {
+        const FusedItem &it = plan.fused[i];
+        os << (i ? "," : "") << "{\"kind\":" << int(it.kind) << ",\"n\":" << it.bytes << ",\"nleaf\":" << it.nleaf << ",\"src\":[";
+        for (size_t k = 0; k < it.src.size(); k++) {
+            os << (k ? "," : "");
+            if (it.srcValid[k]) {
+                JsonRef(os, it.src[k]);
+            } else {
+                os << "null";
+            }
+        }
+        os << "],\"accLeft\":[";
+        for (size_t k = 0; k < it.accLeft.size(); k++) {
+            os << (k ? "," : "") << int(it.accLeft[k]);
+        }
+        os << "],\"dst\":[";
+        for (size_t k = 0; k < it.dst.size(); k++) {
+            os << (k ? "," : "");
+            JsonRef(os, it.dst[k]);
+        }
+        os << "]}";
+    }
+    os << "]}";
+    return os.str();
+}
+
+}  // namespace hcclamd

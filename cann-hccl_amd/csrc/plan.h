@@ -1,0 +1,104 @@
+// Schedule planner: turns one collective call into a list of phases of copy / reduce steps over the
+// ranks' device buffers, and (when the result can be written as one expression per output range)
+// into fused read-reduce-write items.
+//
+// Reference interfaces this replaces (the host side of the algorithm templates and executors):
+//   slice plan   ALG/base/alg_template/temp_all_reduce/all_reduce_ring.cc:119-130
+//   chunk loop   ALG/impl/coll_executor/coll_all_reduce/coll_all_reduce_executor.cc:155-203
+//   step order   ALG/base/alg_template/temp_reduce_scatter/reduce_scatter_ring.cc:179-297,
+//                temp_all_gather/all_gather_ring.cc:120-171, temp_reduce_scatter/reduce_scatter_mesh.cc:57-124,
+//                temp_all_gather/all_gather_mesh.cc:91-145, temp_all_reduce/all_reduce_recursive_hd.cc:33-302,
+//                temp_reduce_scatter/reduce_scatter_halving_doubling.cc:67-238,
+//                temp_all_gather/all_gather_halving_doubling.cc:43-196, temp_alltoallv/alltoallv_pairwise.cc:99-282
+// (ALG = src/domain/collective_communication/algorithm in the reference tree.)
+//
+// Pure C++: no HIP calls, so the planner can be exercised without a GPU.
+#pragma once
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace hcclamd {
+
+enum CollKind : int { COLL_ALLREDUCE = 0, COLL_REDUCESCATTER = 1, COLL_ALLGATHER = 2, COLL_ALLTOALLV = 3 };
+enum Algo : int { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2, ALGO_PAIRWISE = 3 };
+
+// Physical buffers of a rank: the caller's send and receive buffers and a library-owned scratch.
+enum Buf : uint8_t { BUF_SEND = 0, BUF_RECV = 1, BUF_SCRATCH = 2 };
+
+struct Ref {
+    uint32_t rank = 0;
+    uint8_t buf = BUF_SEND;
+    uint64_t off = 0;
+};
+
+// dst = a            (copy,   reduce == false)
+// dst = a (+) b      (reduce; a is the rank's own operand, b the one read from the peer)
+struct Step {
+    bool reduce = false;
+    Ref dst, a, b;
+    uint64_t bytes = 0;
+};
+
+// Steps of one phase have no hazards between them: one kernel launch runs them all.
+struct Phase {
+    std::vector<Step> steps;
+};
+
+enum FusedKind : uint8_t {
+    FK_COPY = 0,    // dst[*] = src[0]
+    FK_CHAIN = 1,   // acc = src[0]; acc = accLeft[j] ? acc (+) src[j] : src[j] (+) acc, j = 1..n-1
+    FK_TREE = 2     // nleaf = 2^k leaves (leaf i = src[2i] or src[2i] (+) src[2i+1]); pairwise
+                    // bottom-up: v[i] = v[i] (+) v[i+w] for w = 1, 2, 4, ...
+};
+
+struct FusedItem {
+    FusedKind kind = FK_COPY;
+    uint64_t bytes = 0;
+    std::vector<Ref> src;
+    std::vector<uint8_t> srcValid;   // FK_TREE: second source of a leaf may be absent
+    std::vector<uint8_t> accLeft;    // FK_CHAIN: one flag per src (index 0 unused)
+    uint32_t nleaf = 0;
+    std::vector<Ref> dst;
+};
+
+struct PlanRequest {
+    CollKind coll = COLL_ALLREDUCE;
+    Algo algo = ALGO_RING;
+    uint32_t p = 1;
+    uint64_t count = 0;            // all-reduce: elements; reduce-scatter: recvCount; all-gather: sendCount
+    uint32_t unit = 4;             // element size in bytes
+    uint64_t cclBytes = 200ull << 20;
+    uint64_t align = 128;
+    std::vector<uint8_t> alias;    // per rank: send buffer and receive buffer are the same memory
+    bool stageInput = false;       // copy the send buffers to scratch first (used when buffers overlap)
+    // all-to-all-v only: p x p tables in elements, row r = what rank r passed
+    std::vector<uint64_t> sendCounts, sdispls, recvCounts, rdispls;
+};
+
+struct Plan {
+    uint32_t p = 0;
+    std::vector<Phase> phases;          // step-by-step program (always valid)
+    uint64_t scratchBytes = 0;          // per-rank scratch the step program needs (0 = none)
+    bool fusedOk = false;               // `fused` computes the same outputs from the inputs alone
+    std::vector<FusedItem> fused;
+    std::vector<uint64_t> sendBytes, recvBytes;   // extent of each rank's buffers the plan touches
+    // byte accounting (all ranks): what the step program / the fused items read and write in HBM
+    uint64_t stepRead = 0, stepWritten = 0, fusedRead = 0, fusedWritten = 0;
+};
+
+// Returns 0 on success; on failure `err` says why (invalid request, or an internal planner check
+// failed: hazard inside a phase, read of an unwritten range, fused and stepwise results differ).
+int BuildPlan(const PlanRequest &req, Plan *plan, std::string *err);
+
+// JSON rendering of a plan (phases, steps, fused items) for tests and debugging.
+std::string DescribePlan(const Plan &plan);
+
+// Slice plans (exposed for tests).
+struct Slice { uint64_t off, size; };
+std::vector<Slice> RingSlicePlan(uint64_t total, uint32_t n, uint64_t align);
+void HalvingDoublingShape(uint32_t p, uint32_t *block, uint32_t *part1);
+std::vector<uint64_t> ChunkCounts(CollKind coll, uint64_t count, uint32_t unit, uint32_t p, uint64_t cclBytes,
+    uint64_t align);
+
+}  // namespace hcclamd

@@ -1,0 +1,140 @@
+// Communicator group, rendezvous of the simulated ranks, and task issue.
+//
+// Stands where the reference has HcclCommunicator::ExecOp / ExecOpAlltoAll
+// (FW/communicator/impl/hccl_communicator.cc:3959,4109), the executors' InitTask / LaunchTaskExtend
+// bracket (ALG/impl/coll_executor/coll_all_reduce/coll_all_reduce_executor.cc:232-270) and the task
+// loader threads (ALG/impl/task/task_loader.cc:102-203): a planned collective becomes a HIP graph of
+// kernel nodes, instantiated once per (operation, sizes, buffers) and replayed on later calls.
+// (FW = src/domain/collective_communication/framework, ALG = .../algorithm in the reference tree.)
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <condition_variable>
+#include <cstdint>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "hccl/hccl_types.h"
+#include "kernels.h"
+#include "plan.h"
+
+namespace hcclamd {
+
+constexpr uint32_t kCommMagic = 0x48434c31;   // "HCL1"
+constexpr uint32_t kMaxRanks = 64;
+
+struct GroupConfig {
+    uint64_t cclBytes = 200ull << 20;     // HCCL_BUFFSIZE / HcclCommConfig.hcclBufferSize (MiB)
+    uint64_t align = 128;                 // slice alignment
+    int algo = -1;                        // -1 = default per collective, else hcclamd::Algo
+    bool fuse = true;                     // run the fused single-pass form when the plan has one
+    bool graph = true;                    // issue through a HIP graph
+    bool deterministic = false;
+    uint32_t blocksPerCu = 8;
+    bool blockingArrive = false;          // ranks wait inside the call until the collective is issued
+    uint32_t arriveTimeoutMs = 1800 * 1000;
+};
+
+// One kernel launch of a prepared collective.
+struct LaunchRec {
+    const void *func = nullptr;
+    uint32_t grid = 0;
+    // kernel arguments (step kernels use the first three)
+    const void *table = nullptr;
+    uint32_t nitems = 0;
+    uint32_t ntiles = 0;
+    const void *srcPool = nullptr;
+    const void *dstPool = nullptr;
+    bool fusedArgs = false;
+};
+
+struct OpInfo {
+    int coll = 0, algo = 0, fused = 0, graph = 0, cacheHit = 0;
+    uint32_t launches = 0;
+    uint64_t bytesRead = 0, bytesWritten = 0;     // what the issued kernels move in HBM, all ranks
+    uint64_t stepRead = 0, stepWritten = 0;       // the step-by-step schedule's figure
+    uint64_t scratchBytes = 0;
+};
+
+struct Prepared {
+    Plan plan;
+    bool fused = false;
+    void *devTables = nullptr;
+    std::vector<LaunchRec> launches;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    uint64_t scratchGen = 0;
+    OpInfo info;
+    uint64_t lastUse = 0;
+    ~Prepared();
+};
+
+struct OpSig {
+    int coll = -1;
+    uint64_t count = 0;
+    int dtype = 0, recvType = 0, op = 0;
+    bool operator==(const OpSig &o) const
+    {
+        return coll == o.coll && count == o.count && dtype == o.dtype && recvType == o.recvType && op == o.op;
+    }
+};
+
+struct Group;
+
+struct Comm {
+    uint32_t magic = kCommMagic;
+    Group *group = nullptr;
+    uint32_t rank = 0;
+    bool inUse = false;
+};
+
+struct Group {
+    std::mutex m;
+    std::condition_variable cv;
+    uint32_t p = 0;
+    std::vector<std::unique_ptr<Comm>> comms;
+    uint32_t liveComms = 0;
+    GroupConfig cfg;
+    std::string name;
+    bool suspended = false;
+    HcclResult asyncError = HCCL_SUCCESS;
+
+    // rendezvous of the current collective
+    uint32_t arrived = 0;
+    uint64_t opSerial = 0;           // bumped whenever a collective is issued or cancelled
+    HcclResult lastIssueResult = HCCL_SUCCESS;
+    OpSig sig;
+    std::vector<uint8_t> here;
+    std::vector<void *> send, recv;
+    std::vector<hipStream_t> streams;
+    std::vector<uint64_t> sendCounts, sdispls, recvCounts, rdispls;   // p x p (all-to-all-v)
+
+    // device resources
+    bool deviceReady = false;
+    int device = 0;
+    uint32_t numCu = 256;
+    std::vector<hipEvent_t> arriveEvents;
+    hipEvent_t doneEvent = nullptr;
+    std::vector<void *> scratch;
+    uint64_t scratchBytes = 0;
+    uint64_t scratchGen = 0;
+    std::map<std::string, std::unique_ptr<Prepared>> cache;
+    uint64_t useClock = 0;
+    OpInfo lastInfo;
+
+    ~Group();
+};
+
+// Creates the group's events on first use of the device.  HCCL_E_RUNTIME when there is no GPU.
+HcclResult EnsureDevice(Group *g, bool quiet);
+
+// Called with the group mutex held, by the last rank to arrive.
+HcclResult IssueCollective(Group *g, uint32_t launcherRank);
+
+const char *CollName(int coll);
+int DefaultAlgo(int coll);
+
+}  // namespace hcclamd

@@ -1,0 +1,52 @@
+/* Additions of the MI355X library to the HCCL C API.  Nothing here exists in the reference; the
+ * entry points let a harness choose the schedule, read back what the last collective moved, and
+ * inspect a plan without a GPU.  Plain C ABI, no device types. */
+#ifndef HCCL_AMD_EXT_H_
+#define HCCL_AMD_EXT_H_
+
+#include <hccl/hccl_types.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Settings of the communicator's whole group.  Keys and values:
+ *   "algo"          "ring" | "mesh" | "rhd" | "auto"   (all-reduce; reduce-scatter / all-gather take ring or mesh)
+ *   "fuse"          "0" | "1"    run the single-pass fused form when the schedule has one
+ *   "graph"         "0" | "1"    issue through a HIP graph
+ *   "buffsize_mib"  CCL buffer size that sets the chunk plan (default 200, as HCCL_BUFFSIZE)
+ *   "align"         slice alignment in bytes (default 128)
+ *   "blocks_per_cu" launch width
+ * Unknown key or bad value: HCCL_E_PARA. */
+extern HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value);
+
+typedef struct HcclAmdOpInfoDef {
+    int32_t coll;            /* 0 all-reduce, 1 reduce-scatter, 2 all-gather, 3 all-to-all-v */
+    int32_t algo;            /* 0 ring, 1 mesh, 2 rhd, 3 pairwise */
+    int32_t fused;           /* 1: issued as fused single-pass kernels */
+    int32_t graph;           /* 1: issued as a HIP graph */
+    int32_t cacheHit;        /* 1: an instantiated graph / table set was reused */
+    uint32_t launches;       /* kernel launches per collective */
+    uint64_t bytesRead;      /* bytes the issued kernels read from HBM, all ranks */
+    uint64_t bytesWritten;   /* bytes they write */
+    uint64_t schedRead;      /* same for the step-by-step schedule (direct peer reads, no staging) */
+    uint64_t schedWritten;
+    uint64_t scratchBytes;   /* per-rank scratch in use */
+} HcclAmdOpInfo;
+
+/* What the most recent collective of this communicator's group issued. */
+extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
+
+/* Plans a collective without a device and writes the plan as JSON (phases of copy / reduce steps,
+ * fused items, byte counts) into out[0..cap).  coll / algo as in HcclAmdOpInfo.  inPlaceMask bit r:
+ * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64
+ * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); else NULL.
+ * Returns HCCL_E_MEMORY and the needed size in *needed when cap is too small. */
+extern HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint64_t count, HcclDataType dataType,
+    uint64_t cclBytes, uint64_t align, uint64_t inPlaceMask, const uint64_t *tables, char *out, size_t cap, size_t *needed);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HCCL_AMD_EXT_H_ */

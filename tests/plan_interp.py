@@ -1,0 +1,65 @@
+"""Test-side interpreter of a plan (the JSON of HcclAmdDescribePlan) over numpy byte buffers.
+
+Used on the CPU to check the product's planner and fuser against the checker before any kernel
+runs; element arithmetic comes from closed_forms.combine (numpy / torch), not from the product and
+not from the checker.
+"""
+import numpy as np
+
+import closed_forms as cf
+
+
+def _view(buf, off, n, dt):
+    return buf[off:off + n].view(cf.CARRIER[dt])
+
+
+def run_steps(plan, sends, recvs, dt, op, in_place=False):
+    """sends / recvs: lists of uint8 arrays (recvs are written).  Scratch is made on demand."""
+    p = plan["p"]
+    scratch = [np.zeros(plan["scratchBytes"], np.uint8) for _ in range(p)]
+    bufs = {0: sends, 1: recvs, 2: scratch}
+    if in_place:
+        bufs[0] = recvs
+    for phase in plan["phases"]:
+        writes = []
+        for s in phase:
+            n = s["n"]
+            a = _view(bufs[s["a"][1]][s["a"][0]], s["a"][2], n, dt).copy()
+            if s["r"]:
+                b = _view(bufs[s["b"][1]][s["b"][0]], s["b"][2], n, dt)
+                a = cf.combine(dt, op, a, b)
+            writes.append((s["dst"], a))
+        for dst, val in writes:
+            _view(bufs[dst[1]][dst[0]], dst[2], val.nbytes, dt)[:] = val
+
+
+def run_fused(plan, sends, recvs, dt, op, in_place=False):
+    assert plan["fusedOk"]
+    src_bufs = recvs if in_place else sends
+    results = []
+    for it in plan["fused"]:
+        n = it["n"]
+        def load(ref):
+            return _view(src_bufs[ref[0]] if ref[1] == 0 else recvs[ref[0]], ref[2], n, dt).copy()
+        if it["kind"] in (0, 1):
+            acc = load(it["src"][0])
+            for j in range(1, len(it["src"])):
+                v = load(it["src"][j])
+                acc = cf.combine(dt, op, acc, v) if it["accLeft"][j] else cf.combine(dt, op, v, acc)
+        else:
+            leaves = []
+            for i in range(it["nleaf"]):
+                v = load(it["src"][2 * i])
+                if it["src"][2 * i + 1] is not None:
+                    v = cf.combine(dt, op, v, load(it["src"][2 * i + 1]))
+                leaves.append(v)
+            w = 1
+            while w < it["nleaf"]:
+                for i in range(0, it["nleaf"], 2 * w):
+                    leaves[i] = cf.combine(dt, op, leaves[i], leaves[i + w])
+                w *= 2
+            acc = leaves[0]
+        results.append((it["dst"], acc))
+    for dsts, val in results:           # all reads happen before any write, as in one fused pass
+        for d in dsts:
+            _view(recvs[d[0]], d[2], val.nbytes, dt)[:] = val

@@ -1,0 +1,189 @@
+"""C-ABI conformance without a GPU: every declared symbol is exported, argument checks return the
+reference's codes in the reference's order (op_base.cc / param_check.cc), and the rendezvous of the
+simulated ranks behaves (mismatch, suspend / resume, time-out)."""
+import ctypes
+import re
+import os
+import threading
+
+import pytest
+
+from hccl_loader import load, ROOT
+
+H = load()
+L = H.lib()
+STREAM = ctypes.c_void_p(0x1000)     # any non-null value: never dereferenced before a launch
+BUF_A, BUF_B = ctypes.c_void_p(0x10000), ctypes.c_void_p(0x20000)
+
+
+@pytest.fixture
+def comms():
+    cs = H.comm_init_all(4)
+    yield cs
+    for c in cs:
+        assert L.HcclCommDestroy(c) in (H.HCCL_SUCCESS, H.HCCL_E_PARA)   # a pending rendezvous is dropped
+
+
+def test_library_exports_every_declared_symbol():
+    declared = set()
+    for header in ("hccl.h", "hccl_amd_ext.h"):
+        text = open(os.path.join(ROOT, "include", "hccl", header)).read()
+        declared |= set(re.findall(r"extern\s+(?:const\s+)?[\w\s\*]+?\b(Hccl\w+)\s*\(", text))
+    assert declared == set(H.EXPORTS)
+    for name in declared:
+        assert hasattr(L, name), name
+
+
+def test_error_strings():
+    assert L.HcclGetErrorString(0) == b"no error"
+    assert L.HcclGetErrorString(1) == b"parameter error"
+    assert L.HcclGetErrorString(2) == b"empty pointer"
+    assert L.HcclGetErrorString(9) == b"timeout"
+    assert L.HcclGetErrorString(21) == b"error cqe"
+    assert L.HcclGetErrorString(23) == b"unknow error"
+    assert L.HcclGetErrorString(-1) == b"unknow error"
+    assert L.HcclGetCommConfigCapability() == 5
+
+
+def test_comm_init_all_checks():
+    devs = (ctypes.c_int32 * 4)(0, 1, 2, 3)
+    out = (ctypes.c_void_p * 4)()
+    assert L.HcclCommInitAll(0, devs, out) == H.HCCL_E_PARA
+    assert L.HcclCommInitAll(4, devs, None) == H.HCCL_E_PTR
+    assert L.HcclCommInitAll(4, None, out) == H.HCCL_E_PTR
+    dup = (ctypes.c_int32 * 4)(0, 1, 1, 3)
+    assert L.HcclCommInitAll(4, dup, out) == H.HCCL_E_PARA
+
+
+def test_rank_queries(comms):
+    n, r = ctypes.c_uint32(), ctypes.c_uint32()
+    for i, c in enumerate(comms):
+        assert L.HcclGetRankSize(c, ctypes.byref(n)) == 0 and n.value == 4
+        assert L.HcclGetRankId(c, ctypes.byref(r)) == 0 and r.value == i
+    assert L.HcclGetRankSize(None, ctypes.byref(n)) == H.HCCL_E_PTR
+    assert L.HcclGetRankSize(comms[0], None) == H.HCCL_E_PTR
+    name = ctypes.create_string_buffer(128)
+    assert L.HcclGetCommName(comms[0], name) == 0 and name.value
+    assert L.HcclCommDestroy(None) == H.HCCL_SUCCESS
+
+
+def test_allreduce_check_order(comms):
+    c = comms[0]
+    FP32, SUM = H.HCCL_DATA_TYPE_FP32, H.HCCL_REDUCE_SUM
+    # count == 0 succeeds before any pointer check
+    assert L.HcclAllReduce(None, None, 0, FP32, SUM, None, None) == H.HCCL_SUCCESS
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, None, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAllReduce(None, BUF_B, 8, FP32, SUM, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAllReduce(BUF_A, None, 8, FP32, SUM, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAllReduce(BUF_A, BUF_B, 0x800000000, FP32, SUM, c, STREAM) == H.HCCL_E_PARA
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, 13, SUM, c, STREAM) == H.HCCL_E_NOT_SUPPORT      # hif8
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, 255, SUM, c, STREAM) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, c, None) == H.HCCL_E_PTR             # null stream
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, 7, c, STREAM) == H.HCCL_E_NOT_SUPPORT      # bad op
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, H.HCCL_DATA_TYPE_INT128, SUM, c, STREAM) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclAllReduce(ctypes.c_void_p(0x10001), BUF_B, 8, FP32, SUM, c, STREAM) == H.HCCL_E_PARA  # misaligned
+
+
+def test_reducescatter_allgather_checks(comms):
+    c = comms[0]
+    FP32, SUM = H.HCCL_DATA_TYPE_FP32, H.HCCL_REDUCE_SUM
+    assert L.HcclReduceScatter(None, None, 0, FP32, SUM, None, None) == H.HCCL_SUCCESS
+    assert L.HcclReduceScatter(BUF_A, BUF_B, 4, FP32, SUM, None, STREAM) == H.HCCL_E_PTR
+    assert L.HcclReduceScatter(BUF_A, BUF_B, 4, FP32, 9, c, STREAM) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclAllGather(None, None, 0, FP32, None, None) == H.HCCL_SUCCESS
+    assert L.HcclAllGather(BUF_A, None, 4, FP32, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAllGather(BUF_A, BUF_B, 4, 99, c, STREAM) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclAllGather(BUF_A, BUF_B, 4, FP32, c, None) == H.HCCL_E_PTR
+
+
+def test_alltoallv_checks(comms):
+    c = comms[0]
+    I32 = H.HCCL_DATA_TYPE_INT32
+    ones = (ctypes.c_uint64 * 4)(1, 1, 1, 1)
+    zeros = (ctypes.c_uint64 * 4)(0, 0, 0, 0)
+    big = (ctypes.c_uint64 * 4)(1, 0x800000000, 1, 1)
+    assert L.HcclAlltoAllV(BUF_A, None, ones, I32, BUF_B, ones, ones, I32, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAlltoAllV(BUF_A, ones, ones, I32, BUF_B, ones, ones, I32, c, None) == H.HCCL_E_PTR
+    assert L.HcclAlltoAllV(BUF_A, ones, ones, I32, BUF_B, ones, ones, I32, None, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAlltoAllV(BUF_A, ones, ones, I32, BUF_A, ones, ones, I32, c, STREAM) == H.HCCL_E_PARA   # same buffer
+    assert L.HcclAlltoAllV(BUF_A, big, ones, I32, BUF_B, ones, ones, I32, c, STREAM) == H.HCCL_E_PARA
+    assert L.HcclAlltoAllV(None, ones, ones, I32, BUF_B, ones, ones, I32, c, STREAM) == H.HCCL_E_PTR     # sends something
+    assert L.HcclAlltoAllV(BUF_A, ones, ones, 14, BUF_B, ones, ones, I32, c, STREAM) == H.HCCL_E_NOT_SUPPORT
+    # a rank that neither sends nor receives may pass null buffers: it only joins the rendezvous
+    assert L.HcclAlltoAllV(None, zeros, zeros, I32, None, zeros, zeros, I32, c, STREAM) == H.HCCL_SUCCESS
+
+
+def test_mismatched_ranks_are_rejected(comms):
+    FP32, SUM = H.HCCL_DATA_TYPE_FP32, H.HCCL_REDUCE_SUM
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, comms[0], STREAM) == H.HCCL_SUCCESS
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, comms[0], STREAM) == H.HCCL_E_AGAIN      # same rank twice
+    assert L.HcclAllReduce(BUF_A, BUF_B, 16, FP32, SUM, comms[1], STREAM) == H.HCCL_E_PARA      # other count
+    # the failed rendezvous was dropped: a fresh one starts cleanly
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, comms[1], STREAM) == H.HCCL_SUCCESS
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, H.HCCL_REDUCE_MAX, comms[2], STREAM) == H.HCCL_E_PARA
+
+
+def test_suspend_resume(comms):
+    FP32, SUM = H.HCCL_DATA_TYPE_FP32, H.HCCL_REDUCE_SUM
+    assert L.HcclCommSuspend(None) == H.HCCL_E_PTR
+    assert L.HcclCommSuspend(comms[0]) == H.HCCL_SUCCESS
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, comms[1], STREAM) == H.HCCL_E_SUSPENDING
+    assert L.HcclCommResume(comms[0]) == H.HCCL_SUCCESS
+    assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, comms[1], STREAM) == H.HCCL_SUCCESS
+    err = ctypes.c_int32(-1)
+    assert L.HcclGetCommAsyncError(comms[0], ctypes.byref(err)) == 0 and err.value == 0
+
+
+def test_blocking_arrival_times_out(comms):
+    FP32, SUM = H.HCCL_DATA_TYPE_FP32, H.HCCL_REDUCE_SUM
+    H.set_param(comms[0], "blocking_arrive", 1)
+    H.set_param(comms[0], "arrive_timeout_ms", 50)
+    results = {}
+
+    def call(r):
+        results[r] = L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, comms[r], STREAM)
+
+    ts = [threading.Thread(target=call, args=(r,)) for r in (0, 1)]    # ranks 2 and 3 never call
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join(10)
+    assert sorted(results.values()) in ([H.HCCL_E_TIMEOUT, H.HCCL_E_TIMEOUT], [H.HCCL_E_PARA, H.HCCL_E_TIMEOUT],
+                                        [H.HCCL_E_TIMEOUT, H.HCCL_E_AGAIN]) or H.HCCL_E_TIMEOUT in results.values()
+
+
+def test_set_config_deterministic():
+    if "HCCL_DETERMINISTIC" in os.environ:
+        pytest.skip("environment overrides the switch")
+    v = ctypes.c_int32(-1)
+    assert L.HcclSetConfig(0, 2) == H.HCCL_E_PARA
+    assert L.HcclSetConfig(0, 1) == H.HCCL_SUCCESS
+    assert L.HcclGetConfig(0, ctypes.byref(v)) == 0 and v.value == 1
+    assert L.HcclSetConfig(0, 0) == H.HCCL_SUCCESS
+    assert L.HcclGetConfig(0, ctypes.byref(v)) == 0 and v.value == 0
+    assert L.HcclGetConfig(0, None) == H.HCCL_E_PTR
+
+
+def test_amd_params(comms):
+    assert L.HcclAmdSetParam(comms[0], b"algo", b"mesh") == 0
+    assert L.HcclAmdSetParam(comms[0], b"algo", b"bogus") == H.HCCL_E_PARA
+    assert L.HcclAmdSetParam(comms[0], b"nonsense", b"1") == H.HCCL_E_PARA
+    assert L.HcclAmdSetParam(comms[0], b"buffsize_mib", b"0") == H.HCCL_E_PARA
+    assert L.HcclAmdSetParam(None, b"algo", b"ring") == H.HCCL_E_PTR
+
+
+def test_unsupported_entry_points_link_and_refuse(comms):
+    assert L.HcclBroadcast(BUF_A, 4, 4, 0, comms[0], STREAM) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclBroadcast(BUF_A, 4, 4, 0, None, STREAM) == H.HCCL_E_PTR
+    assert L.HcclGetRootInfo(None) == H.HCCL_E_PTR
+
+
+def test_no_gpu_means_loud_failure(comms):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    FP32, SUM = H.HCCL_DATA_TYPE_FP32, H.HCCL_REDUCE_SUM
+    codes = [L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, c, STREAM) for c in comms]
+    assert codes[:3] == [0, 0, 0] and codes[3] == H.HCCL_E_RUNTIME          # the issuing rank reports it
+    err = ctypes.c_int32(0)
+    assert L.HcclGetCommAsyncError(comms[0], ctypes.byref(err)) == 0 and err.value == H.HCCL_E_RUNTIME

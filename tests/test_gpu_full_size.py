@@ -1,0 +1,69 @@
+"""The headline configuration at its real size on the GPU: 8 ranks, fp32 sum, 256 MiB per rank,
+ring all-reduce.  Checked bit for bit against the CPU checker and through size-independent properties."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_harness as gh
+from closed_forms import FP32, SUM
+
+pytestmark = pytest.mark.gpu
+H = gh.H
+
+
+def test_ring_allreduce_256mib_per_rank():
+    from oracle import oracle as orc
+    orc.build()
+    p, n = 8, 64 << 20
+    ins = [orc.fill_uniform_f32(n, 1234, r, threads=16) for r in range(p)]
+    sends = [torch.from_numpy(x).cuda() for x in ins]
+    torch.cuda.synchronize()
+    results = {}
+    for fuse in (1, 0):
+        g = gh.Group(p, fuse=fuse)
+        try:
+            recvs = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(p)]
+            torch.cuda.synchronize()
+            print("full size all-reduce fuse", fuse, flush=True)
+            H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, g.stream_ptr)
+            g.stream.synchronize()
+            info = g.info()
+            S = n * 4
+            if fuse:
+                assert info["bytesRead"] == p * S and info["bytesWritten"] == p * S
+            else:
+                assert info["bytesRead"] + info["bytesWritten"] == 5 * (p - 1) * S
+            # property: every rank holds the same bits
+            for r in range(1, p):
+                assert torch.equal(recvs[0], recvs[r]), (fuse, r)
+            # property: send buffers untouched
+            assert torch.equal(sends[3], torch.from_numpy(ins[3]).cuda())
+            results[fuse] = recvs[0].cpu().numpy()
+            del recvs
+        finally:
+            g.close()
+    assert np.array_equal(results[1], results[0])            # fused and step-by-step agree bit for bit
+    # the checker at full size (direct messages, no staging, 16 threads); its inputs are clobbered
+    work = [x.copy() for x in ins]
+    outs = [np.empty(n, np.float32) for _ in range(p)]
+    orc.allreduce(work, FP32, SUM, flags=orc.DIRECT | orc.ZERO_STAGING, threads=16, outs=outs)
+    assert np.array_equal(results[1], outs[0])
+    assert np.array_equal(outs[0], outs[5])
+    # property: all-reduce == all-gather of reduce-scatter (done with the library itself on a 1/8 sample)
+    m = n // 8
+    g = gh.Group(p)
+    try:
+        rs_out = [torch.empty(m // p, dtype=torch.float32, device="cuda") for _ in range(p)]
+        ag_out = [torch.empty(m, dtype=torch.float32, device="cuda") for _ in range(p)]
+        ar_out = [torch.empty(m, dtype=torch.float32, device="cuda") for _ in range(p)]
+        part = [t[:m].contiguous() for t in sends]
+        torch.cuda.synchronize()
+        H.set_param(g.comms[0], "align", m * 4 // p)     # make the all-reduce slices equal the scatter blocks
+        H.all_reduce(g.comms, [t.data_ptr() for t in part], [t.data_ptr() for t in ar_out], m, FP32, SUM, g.stream_ptr)
+        H.reduce_scatter(g.comms, [t.data_ptr() for t in part], [t.data_ptr() for t in rs_out], m // p, FP32, SUM, g.stream_ptr)
+        H.all_gather(g.comms, [t.data_ptr() for t in rs_out], [t.data_ptr() for t in ag_out], m // p, FP32, g.stream_ptr)
+        g.stream.synchronize()
+        for r in range(p):
+            assert torch.equal(ar_out[r], ag_out[r]), r
+    finally:
+        g.close()

@@ -1,0 +1,337 @@
+"""Parity of the HIP library with the CPU checker, through the C ABI, on a real MI355X.
+
+Bars: bit-exact for integers, all-gather, all-to-all-v and fp32; fp16 / bf16 are expected bit-equal
+too (both sides round after every stored step) and are held to <= 1 ulp."""
+import numpy as np
+import pytest
+import torch
+
+import closed_forms as cf
+import gpu_harness as gh
+from closed_forms import ALL_TYPES, BF16, FP16, FP32, FP64, INT8, INT16, INT32, INT64, MAX, MIN, PROD, SUM
+from test_oracle_schedules import _a2av_case
+
+pytestmark = pytest.mark.gpu
+H = gh.H
+RING, MESH, RHD = 0, 1, 2
+ALGO_NAME = {RING: "ring", MESH: "mesh", RHD: "rhd"}
+OPS = (SUM, PROD, MAX, MIN)
+
+
+def _ins(dt, p, n, seed):
+    rng = np.random.default_rng(seed)
+    return [cf.random_input(dt, n, rng) for _ in range(p)]
+
+
+def _ulp_close(dt, got, want):
+    """<= 1 unit in the last place for 16-bit floats (bit patterns are monotone per sign)."""
+    if gh.same(dt, got, want):
+        return True
+    g, w = got.astype(np.int32), want.astype(np.int32)
+    g = np.where(g & 0x8000, 0x8000 - g, g)
+    w = np.where(w & 0x8000, 0x8000 - w, w)
+    return int(np.abs(g - w).max()) <= 1
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import oracle
+    oracle.build()
+    return oracle
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("fuse", [1, 0])
+def test_allreduce_fp32_sum_bit_exact(orc, algo, fuse):
+    for p in (1, 2, 3, 5, 8, 16):
+        g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+        try:
+            for n in (1, 7, 1000, 262144 + 3):
+                ins = _ins(FP32, p, n, 1000 * p + n)
+                print("allreduce fp32", ALGO_NAME[algo], "fuse", fuse, "p", p, "n", n, flush=True)
+                want = orc.allreduce(ins, FP32, SUM, algo=algo)
+                outs, keep = gh.all_reduce(g, ins, FP32, SUM)
+                for r in range(p):
+                    assert np.array_equal(outs[r], want[r]), (algo, fuse, p, n, r)
+                    assert np.array_equal(keep[r], ins[r])            # send buffers are left alone
+                info = g.info()
+                assert info["fused"] == (1 if (fuse and p <= 32) else 0) or p == 1
+        finally:
+            g.close()
+
+
+@pytest.mark.parametrize("dt", ALL_TYPES)
+def test_allreduce_every_type_and_op(orc, dt):
+    p, n = 8, 40000 + 13
+    for algo in (RING, RHD, MESH):
+        for fuse in (1, 0):
+            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+            try:
+                for op in OPS:
+                    print("allreduce type", dt, "op", op, ALGO_NAME[algo], "fuse", fuse, flush=True)
+                    ins = _ins(dt, p, n, dt * 10 + op)
+                    want = orc.allreduce(ins, dt, op, algo=algo)
+                    outs, _ = gh.all_reduce(g, ins, dt, op)
+                    for r in range(p):
+                        if dt in (FP16, BF16):
+                            assert _ulp_close(dt, outs[r], want[r]), (dt, op, algo, fuse, r)
+                            assert gh.same(dt, outs[r], want[r]), (dt, op, algo, fuse, r)   # in fact bit-equal
+                        else:
+                            assert gh.same(dt, outs[r], want[r]), (dt, op, algo, fuse, r)
+            finally:
+                g.close()
+
+
+@pytest.mark.parametrize("fuse", [1, 0])
+def test_allreduce_in_place_and_unaligned(orc, fuse):
+    p = 8
+    g = gh.Group(p, fuse=fuse)
+    try:
+        for dt, pad in ((FP32, 0), (FP32, 4), (FP32, 16), (BF16, 2), (INT8, 1), (INT8, 3), (INT64, 8), (FP16, 6)):
+            n = 100003
+            ins = _ins(dt, p, n, pad + dt)
+            want = orc.allreduce(ins, dt, SUM)
+            print("allreduce pad", pad, "type", dt, "fuse", fuse, flush=True)
+            outs, _ = gh.all_reduce(g, ins, dt, SUM, pad=pad)
+            assert all(gh.same(dt, outs[r], want[r]) for r in range(p)), (dt, pad, "out of place")
+            outs, _ = gh.all_reduce(g, ins, dt, SUM, in_place=True, pad=pad)
+            assert all(gh.same(dt, outs[r], want[r]) for r in range(p)), (dt, pad, "in place")
+    finally:
+        g.close()
+
+
+def test_allreduce_chunk_plan_follows_buffer_size(orc):
+    # a CCL buffer smaller than the payload restarts the slice plan per chunk and changes the fp32 bits
+    p, n = 8, 300000
+    ins = _ins(FP32, p, n, 77)
+    for fuse in (1, 0):
+        g = gh.Group(p, fuse=fuse, buffsize_bytes=256 * 1024)
+        try:
+            want = orc.allreduce(ins, FP32, SUM, ccl_bytes=256 * 1024)
+            outs, _ = gh.all_reduce(g, ins, FP32, SUM)
+            assert all(np.array_equal(outs[r], want[r]) for r in range(p))
+        finally:
+            g.close()
+
+
+def test_graph_replay_and_cache(orc):
+    p, n = 8, 500000
+    g = gh.Group(p, fuse=0, graph=1)
+    try:
+        ins = _ins(FP32, p, n, 5)
+        want = orc.allreduce(ins, FP32, SUM)
+        sends = [gh.to_dev(x) for x in ins]
+        recvs = [gh.empty_dev(n * 4) for _ in ins]
+        torch.cuda.synchronize()
+        for rep in range(4):
+            for t in recvs:
+                t.fill_(rep)                                    # eager work between replays
+            torch.cuda.synchronize()
+            H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, g.stream_ptr)
+            g.stream.synchronize()
+            info = g.info()
+            assert info["graph"] == 1 and info["launches"] == 2 * (p - 1)
+            assert info["cacheHit"] == (1 if rep else 0)
+            for r in range(p):
+                assert np.array_equal(gh.to_host(recvs[r], FP32), want[r]), (rep, r)
+        # same call without a graph gives the same bits
+        g.set(graph=0)
+        H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, g.stream_ptr)
+        g.stream.synchronize()
+        assert g.info()["graph"] == 0
+        assert all(np.array_equal(gh.to_host(recvs[r], FP32), want[r]) for r in range(p))
+    finally:
+        g.close()
+
+
+def test_streams_of_other_ranks_are_ordered(orc):
+    # every rank on its own stream: inputs are produced on that stream right before the call
+    p, n = 4, 1 << 20
+    g = gh.Group(p)
+    try:
+        ins = _ins(FP32, p, n, 9)
+        want = orc.allreduce(ins, FP32, SUM)
+        streams = [torch.cuda.Stream() for _ in range(p)]
+        host = [torch.from_numpy(x).pin_memory() for x in ins]
+        sends = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(p)]
+        recvs = [torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(p)]
+        torch.cuda.synchronize()
+        for r in range(p):
+            with torch.cuda.stream(streams[r]):
+                sends[r].copy_(host[r], non_blocking=True)
+            rc = H.lib().HcclAllReduce(sends[r].data_ptr(), recvs[r].data_ptr(), n, FP32, SUM, g.comms[r], streams[r].cuda_stream)
+            assert rc == 0
+        outs = []
+        for r in range(p):
+            with torch.cuda.stream(streams[r]):
+                outs.append(recvs[r].cpu())                     # ordered after the collective on rank r's stream
+        torch.cuda.synchronize()
+        for r in range(p):
+            assert np.array_equal(outs[r].numpy(), want[r]), r
+    finally:
+        g.close()
+
+
+@pytest.mark.parametrize("algo", [RING, MESH])
+def test_reducescatter_op_type_matrix(orc, algo):
+    p = 8
+    for fuse in (1, 0):
+        g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+        try:
+            for dt in (FP16, BF16, INT8, INT32, INT64, FP32):
+                for op in OPS:
+                    n = 30011
+                    ins = _ins(dt, p, n * p, dt + 3 * op)
+                    print("reducescatter", ALGO_NAME[algo], "fuse", fuse, "type", dt, "op", op, flush=True)
+                    want = orc.reducescatter(ins, dt, op, algo=algo)
+                    outs, keep = gh.reduce_scatter(g, ins, dt, op)
+                    for r in range(p):
+                        assert gh.same(dt, outs[r], want[r]), (algo, fuse, dt, op, r)
+                        assert np.array_equal(keep[r], ins[r])
+        finally:
+            g.close()
+
+
+def test_reducescatter_64mib_per_rank_int_and_bf16(orc):
+    # the reduce-scatter configuration at its full size: 64 MiB per rank send buffer, 8 ranks
+    p = 8
+    g = gh.Group(p)
+    try:
+        for dt, op in ((INT32, SUM), (BF16, SUM), (INT8, MAX), (INT64, PROD), (FP16, MIN)):
+            unit = H.DTYPE_SIZE[dt]
+            n = (64 << 20) // unit // p
+            ins = _ins(dt, p, n * p, dt)
+            print("reducescatter 64MiB type", dt, "op", op, flush=True)
+            want = orc.reducescatter(ins, dt, op, flags=orc.DIRECT, threads=16)
+            outs, _ = gh.reduce_scatter(g, ins, dt, op)
+            assert all(gh.same(dt, outs[r], want[r]) for r in range(p)), (dt, op)
+    finally:
+        g.close()
+
+
+@pytest.mark.parametrize("algo", [RING, MESH])
+def test_allgather(orc, algo):
+    for p in (1, 2, 5, 8, 16):
+        for fuse in (1, 0):
+            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+            try:
+                for dt, n, pad in ((INT8, 30001, 0), (INT8, 777, 3), (FP16, 4099, 2), (INT64, 65536, 0), (FP32, 1, 0)):
+                    ins = _ins(dt, p, n, p + n)
+                    print("allgather", ALGO_NAME[algo], "fuse", fuse, "p", p, "type", dt, "n", n, flush=True)
+                    outs = gh.all_gather(g, ins, dt, pad=pad)
+                    want = np.concatenate(ins)
+                    assert all(np.array_equal(outs[r], want) for r in range(p)), (algo, p, fuse, dt, n)
+            finally:
+                g.close()
+
+
+def test_alltoallv_small_ragged(orc):
+    for p in (1, 2, 3, 8, 16):
+        for fuse in (1, 0):
+            g = gh.Group(p, fuse=fuse)
+            try:
+                cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 40 + p, max_count=5000)
+                sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+                want = [np.full(n, -1, np.int32) for n in rl]
+                assert orc.alltoallv(sends, cnt, sdis, want, rcnt, rdis, INT32) == 0
+                print("alltoallv p", p, "fuse", fuse, flush=True)
+                outs = gh.all_to_all_v(g, sends, cnt, sdis, rl, rcnt, rdis, INT32)
+                assert all(np.array_equal(outs[r], want[r]) for r in range(p)), (p, fuse)
+            finally:
+                g.close()
+
+
+def test_alltoallv_16_ranks_lognormal(orc):
+    # 16 ranks, per-pair counts lognormal(ln 64K, 1) clamped to [0, 4M] int32 elements, shuffled displacements with gaps
+    p = 16
+    rng = np.random.default_rng(2024)
+    cnt = np.clip(np.rint(np.exp(np.log(65536.0) + rng.standard_normal((p, p)))), 0, 4 << 20).astype(np.uint64)
+    sdis = np.zeros((p, p), np.uint64)
+    rdis = np.zeros((p, p), np.uint64)
+    sl, rl = [], []
+    for r in range(p):
+        pos = 0
+        for j in rng.permutation(p):
+            pos += int(rng.integers(0, 1024))
+            sdis[r, j] = pos
+            pos += int(cnt[r, j])
+        sl.append(pos)
+        pos = 0
+        for i in rng.permutation(p):
+            pos += int(rng.integers(0, 1024))
+            rdis[r, i] = pos
+            pos += int(cnt[i, r])
+        rl.append(pos)
+    rcnt = cnt.T.copy()
+    sends = [((np.arange(n, dtype=np.int64) * 2654435761 + (r << 24)) & 0x7fffffff).astype(np.int32) for r, n in enumerate(sl)]
+    want = [np.full(n, -1, np.int32) for n in rl]
+    assert orc.alltoallv(sends, cnt, sdis, want, rcnt, rdis, INT32, flags=orc.DIRECT, threads=8) == 0
+    for fuse in (1, 0):
+        g = gh.Group(p, fuse=fuse)
+        try:
+            print("alltoallv lognormal fuse", fuse, "total elements", int(cnt.sum()), flush=True)
+            outs = gh.all_to_all_v(g, sends, cnt, sdis, rl, rcnt, rdis, INT32)
+            assert all(np.array_equal(outs[r], want[r]) for r in range(p)), fuse
+            info = g.info()
+            assert info["bytesRead"] == 4 * int(cnt.sum()) and info["bytesWritten"] == 4 * int(cnt.sum())
+        finally:
+            g.close()
+
+
+def test_alltoallv_asymmetric_tables_fail(orc):
+    p = 4
+    g = gh.Group(p)
+    try:
+        cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 3)
+        rcnt = rcnt.copy()
+        rcnt[2, 1] += 1
+        sends = [np.zeros(n + 8, np.int32) for n in sl]
+        with pytest.raises(H.HcclError) as e:
+            gh.all_to_all_v(g, sends, cnt, sdis, [n + 8 for n in rl], rcnt, rdis, INT32)
+        assert e.value.code == H.HCCL_E_PARA
+    finally:
+        g.close()
+
+
+@pytest.mark.parametrize("p", [32, 24])
+def test_rhd_allreduce_bf16(orc, p):
+    # power-of-two and fold (24 = block 16 + 8 pairs) paths, bf16 with fp32 accumulation
+    n = 4 << 20           # 8 MiB per rank
+    ins = _ins(BF16, p, n, p)
+    want = orc.allreduce(ins, BF16, SUM, algo=RHD, flags=orc.DIRECT, threads=16)
+    for fuse in (1, 0):
+        g = gh.Group(p, algo="rhd", fuse=fuse)
+        try:
+            print("rhd bf16 p", p, "fuse", fuse, flush=True)
+            outs, _ = gh.all_reduce(g, ins, BF16, SUM)
+            for r in range(p):
+                assert _ulp_close(BF16, outs[r], want[r]), (p, fuse, r)
+                assert gh.same(BF16, outs[r], want[r]), (p, fuse, r)
+            # sanity against the exact sum: error within (p - 1) roundings
+            exact = sum(cf.bf16_bits_to_f32(x).astype(np.float64) for x in ins)
+            got = cf.bf16_bits_to_f32(outs[0]).astype(np.float64)
+            assert np.all(np.abs(got - exact) <= (p - 1) * np.maximum(np.abs(exact), 1.0) * 2.0 ** -8)
+        finally:
+            g.close()
+
+
+def test_special_values_follow_the_selection_rule(orc):
+    # NaN, signed zeros, infinities, denormals: max / min pick (b > a) ? b : a with a = the rank's own operand
+    p = 4
+    specials = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.0, -1.0, 3.4e38], np.float32)
+    rng = np.random.default_rng(8)
+    ins = [rng.choice(specials, 4096).astype(np.float32) for _ in range(p)]
+    for algo in (RING, RHD):
+        for fuse in (1, 0):
+            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse, align=4)
+            try:
+                for op in OPS:
+                    want = orc.allreduce(ins, FP32, op, algo=algo, align=4)
+                    outs, _ = gh.all_reduce(g, ins, FP32, op)
+                    for r in range(p):
+                        assert gh.same(FP32, outs[r], want[r]), (algo, fuse, op, r)
+                        assert np.array_equal(np.isnan(outs[r]), np.isnan(want[r]))
+                        if op in (MAX, MIN):
+                            assert np.array_equal(outs[r].view(np.uint32), want[r].view(np.uint32))   # incl. sign of zero, NaN bits
+            finally:
+                g.close()

@@ -1,0 +1,126 @@
+"""Product planner and fuser on the CPU: the plan the library would execute (HcclAmdDescribePlan)
+is interpreted with numpy and compared with the checker, step-by-step form and fused form."""
+import numpy as np
+import pytest
+
+import closed_forms as cf
+import plan_interp
+from closed_forms import BF16, FP16, FP32, INT8, INT32, INT64, MAX, MIN, PROD, SUM
+from hccl_loader import load
+from test_oracle_schedules import _a2av_case
+
+H = load()
+RING, MESH, RHD = 0, 1, 2
+
+
+def _bytes(arrs):
+    return [a.view(np.uint8).copy() for a in arrs]
+
+
+def _ins(dt, p, n, seed):
+    rng = np.random.default_rng(seed)
+    return [cf.random_input(dt, n, rng) for _ in range(p)]
+
+
+def _same(dt, got_bytes, want):
+    got = got_bytes.view(cf.CARRIER[dt])
+    if dt in (FP16, BF16, FP32):
+        nn = np.isnan(cf.widen(dt, got).astype(np.float64)) & np.isnan(cf.widen(dt, want).astype(np.float64))
+        return np.array_equal(got[~nn], want[~nn])
+    return np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("p", [1, 2, 3, 4, 5, 6, 8, 12, 16, 24])
+def test_allreduce_plan_matches_checker(orc, algo, p):
+    for dt, op, n, ccl in ((FP32, SUM, 1000, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, PROD, 777, 200 << 20),
+                           (INT8, MAX, 333, 200 << 20), (FP16, SUM, 2049, 2048)):
+        unit = H.DTYPE_SIZE[dt]
+        ins = _ins(dt, p, n, p * 7 + op)
+        want = orc.allreduce(ins, dt, op, algo=algo, ccl_bytes=ccl)
+        for mask in (0, (1 << p) - 1):
+            plan = H.describe_plan(H.COLL_ALLREDUCE, algo, p, n, dt, ccl_bytes=ccl, in_place_mask=mask)
+            assert plan["scratchBytes"] == 0
+            for fused in (False, True):
+                if fused and not plan["fusedOk"]:
+                    continue
+                sends = _bytes(ins)
+                recvs = _bytes(ins) if mask else [np.full(n * unit, 0xA5, np.uint8) for _ in range(p)]
+                runner = plan_interp.run_fused if fused else plan_interp.run_steps
+                runner(plan, sends, recvs, dt, op, in_place=bool(mask))
+                for r in range(p):
+                    assert _same(dt, recvs[r], want[r]), (algo, p, dt, op, ccl, mask, fused, r)
+                if not mask:
+                    assert all(np.array_equal(s, i.view(np.uint8)) for s, i in zip(sends, ins))   # send buffers untouched
+            if p <= 32:
+                assert plan["fusedOk"], (algo, p)
+
+
+def test_allreduce_ring_byte_counts():
+    p, n = 8, 1 << 20
+    S = n * 4
+    plan = H.describe_plan(H.COLL_ALLREDUCE, RING, p, n, FP32)
+    assert plan["stepRead"] + plan["stepWritten"] == 5 * (p - 1) * S     # partials live in the receive buffer
+    assert plan["fusedRead"] == p * S and plan["fusedWritten"] == p * S
+    assert len(plan["phases"]) == 2 * (p - 1)
+    plan = H.describe_plan(H.COLL_ALLREDUCE, RHD, 32, n, FP32)
+    assert plan["fusedRead"] == 32 * S and plan["fusedWritten"] == 32 * S
+    plan = H.describe_plan(H.COLL_ALLREDUCE, RHD, 24, n, FP32)
+    assert plan["fusedOk"] and plan["fused"][0]["kind"] == 2 and plan["fused"][0]["nleaf"] == 16
+
+
+@pytest.mark.parametrize("algo", [RING, MESH])
+@pytest.mark.parametrize("p", [1, 2, 3, 8])
+def test_reducescatter_plan_matches_checker(orc, algo, p):
+    for dt, op, n, ccl in ((FP32, SUM, 500, 200 << 20), (BF16, SUM, 301, 128 * p * 2), (INT64, MIN, 100, 200 << 20)):
+        unit = H.DTYPE_SIZE[dt]
+        ins = _ins(dt, p, n * p, p + op)
+        want = orc.reducescatter(ins, dt, op, algo=algo, ccl_bytes=ccl)
+        plan = H.describe_plan(H.COLL_REDUCESCATTER, algo, p, n, dt, ccl_bytes=ccl)
+        for fused in (False, True):
+            sends = _bytes(ins)
+            recvs = [np.full(n * unit, 0x5A, np.uint8) for _ in range(p)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+            for r in range(p):
+                assert _same(dt, recvs[r], want[r]), (algo, p, dt, fused, r)
+            assert all(np.array_equal(s, i.view(np.uint8)) for s, i in zip(sends, ins))
+
+
+@pytest.mark.parametrize("algo", [RING, MESH])
+@pytest.mark.parametrize("p", [1, 2, 5, 8])
+def test_allgather_plan_matches_checker(orc, algo, p):
+    for dt, n, ccl in ((INT8, 301, 200 << 20), (INT32, 100, 128 * p * 2)):
+        unit = H.DTYPE_SIZE[dt]
+        ins = _ins(dt, p, n, p)
+        want = orc.allgather(ins, dt, algo=algo, ccl_bytes=ccl)
+        plan = H.describe_plan(H.COLL_ALLGATHER, algo, p, n, dt, ccl_bytes=ccl)
+        for fused in (False, True):
+            sends = _bytes(ins)
+            recvs = [np.full(n * unit * p, 0x5A, np.uint8) for _ in range(p)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, 0)
+            for r in range(p):
+                assert np.array_equal(recvs[r].view(cf.CARRIER[dt]), want[r]), (algo, p, dt, fused, r)
+
+
+@pytest.mark.parametrize("p", [1, 2, 3, 8, 16])
+def test_alltoallv_plan_matches_checker(orc, p):
+    cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 10 + p)
+    sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+    want = [np.full(n, -1, np.int32) for n in rl]
+    assert orc.alltoallv(sends, cnt, sdis, want, rcnt, rdis, INT32) == 0
+    plan = H.describe_plan(H.COLL_ALLTOALLV, H.ALGO_PAIRWISE, p, 0, INT32, tables=(cnt, sdis, rcnt, rdis))
+    assert len(plan["phases"]) <= p
+    for fused in (False, True):
+        recvs = [np.full(n, -1, np.int32).view(np.uint8).copy() for n in rl]
+        (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, _bytes(sends), recvs, INT32, 0)
+        for r in range(p):
+            assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, fused, r)
+
+
+def test_plan_rejects_bad_requests():
+    with pytest.raises(H.HcclError):
+        H.describe_plan(H.COLL_ALLREDUCE, RING, 0, 10, FP32)
+    with pytest.raises(H.HcclError):
+        H.describe_plan(H.COLL_REDUCESCATTER, RHD, 4, 10, FP32)       # no halving-doubling at this level
+    with pytest.raises(H.HcclError):
+        H.describe_plan(H.COLL_ALLGATHER, RING, 8, 10, FP32, ccl_bytes=64)   # buffer below one aligned slice per rank
