@@ -59,6 +59,14 @@ def lib():
         return _lib
     if not os.path.exists(LIB_PATH):
         raise RuntimeError("libhccl.so is not built: run `python cann-hccl_amd/build.py` (needs hipcc)")
+    # Streams and device pointers handed to the library must belong to the HIP runtime the library
+    # itself uses.  PyTorch ships its own libamdhip64 (same soname): when it is loaded first the
+    # dynamic linker shares it with libhccl.so, the other way round the process ends up with two
+    # runtimes.  So load PyTorch's first whenever PyTorch is installed.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = ctypes.CDLL(LIB_PATH)
     vp, u64, u32, i32 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_int32
     L.HcclCommInitAll.argtypes = [u32, ctypes.POINTER(i32), ctypes.POINTER(vp)]
