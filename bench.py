@@ -58,6 +58,11 @@ def main():
     ap.add_argument("--ranks", type=int, default=8)
     ap.add_argument("--sweep", action="store_true", help="also time 8 KiB .. 256 MiB per rank (x2), table on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain 1 GiB int32 copy (one-rank all-reduce, out of place) three times, so that a "
+                         "counter profile of this command holds a copy of known size to scale FETCH_SIZE / WRITE_SIZE by")
+    ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
+                    help="library setting for the run (see HcclAmdSetParam), e.g. --set blocks_per_cu=4")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is built and measured on one GPU (the ranks of the communicator are "
@@ -82,6 +87,9 @@ def main():
     recvs = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(p)]
     comms = pkg.comm_init_all(p)
     stream = torch.cuda.Stream()
+    for kv in args.set:
+        k, v = kv.split("=", 1)
+        pkg.set_param(comms[0], k, v)
     torch.cuda.synchronize()
 
     wall_ms, dev_ms, info = run_mode(pkg, torch, comms, stream, sends, recvs, n, 1, args.steps, args.warmup)
@@ -111,6 +119,20 @@ def main():
         cpu = {"value": round(sched / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
                "sample": "full workload (%d ranks x %.0f MiB fp32, out of place), checker in direct zero-staging "
                          "mode, best of 3, %.3f s; bytes = (5p-3)S schedule figure" % (p, args.size_mib, best)}
+
+    if args.calibrate:
+        one = pkg.comm_init_all(1)
+        m = 256 << 20
+        src = torch.ones(m, dtype=torch.int32, device="cuda")
+        dst = torch.zeros(m, dtype=torch.int32, device="cuda")
+        torch.cuda.synchronize()
+        for _ in range(3):
+            pkg.all_reduce(one, [src.data_ptr()], [dst.data_ptr()], m, pkg.HCCL_DATA_TYPE_INT32, pkg.HCCL_REDUCE_SUM,
+                           stream.cuda_stream)
+        stream.synchronize()
+        assert bool(torch.equal(src, dst))
+        pkg.comm_destroy(one)
+        del src, dst
 
     if args.sweep:
         sys.stderr.write("bytes/rank  fused_us  fused_GB/s(actual)  steps_us  steps_GB/s(actual)  sched_GB/s(fused)\n")

@@ -191,14 +191,6 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
     }
     g->arrived++;
     if (g->arrived < g->p) {
-        // remember where this rank's stream stands so the launch can be ordered after it
-        // (without a device nothing is recorded; the rank that issues then fails loudly)
-        if (EnsureDevice(g, true) == HCCL_SUCCESS) {
-            if (hipEventRecord(g->arriveEvents[r], stream) != hipSuccess) {
-                HCCL_LOG_ERROR("%s: recording the arrival event of rank %u failed", CollName(sig.coll), r);
-                g->asyncError = HCCL_E_RUNTIME;
-            }
-        }
         if (!g->cfg.blockingArrive) {
             return HCCL_SUCCESS;
         }
@@ -672,7 +664,7 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         cfg.align = uint64_t(n);
     } else if (k == "blocks_per_cu") {
         long n = std::atol(value);
-        if (n < 1 || n > 64) {
+        if (n < 0 || n > 64) {
             return HCCL_E_PARA;
         }
         cfg.blocksPerCu = uint32_t(n);

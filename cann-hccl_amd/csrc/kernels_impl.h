@@ -265,36 +265,49 @@ __global__ void __launch_bounds__(kBlockThreads) StepKernel(const StepDesc *__re
 }
 
 // ---- fused chain: read every source once, combine in schedule order, write every destination ----------
-constexpr uint32_t kChainVec = 2;      // vectors per lane per pass
-constexpr uint32_t kChainSrcBatch = 4; // sources whose loads are issued together
+constexpr uint32_t kChainVec = 4;      // vectors per lane per pass
+constexpr uint32_t kChainSrcBatch = 8; // sources whose loads are issued together
 
-template <typename T, int OP, uint32_t MODE>
+// Operand order changes the bits only where the combine is not commutative bit for bit:
+// floating max / min (NaN and signed zero follow the selection rule).
+template <typename T, int OP> struct OrderMatters { static constexpr bool value = false; };
+template <int OP> struct OrderMatters<float, OP> { static constexpr bool value = (OP == ROP_MAX || OP == ROP_MIN); };
+template <int OP> struct OrderMatters<double, OP> { static constexpr bool value = (OP == ROP_MAX || OP == ROP_MIN); };
+template <int OP> struct OrderMatters<HalfBits, OP> { static constexpr bool value = (OP == ROP_MAX || OP == ROP_MIN); };
+template <int OP> struct OrderMatters<Bf16Bits, OP> { static constexpr bool value = (OP == ROP_MAX || OP == ROP_MIN); };
+
+template <uint32_t MODE> __device__ __forceinline__ void StoreAny16(void *base, uint64_t pos, V4 v)
+{
+    if (MODE == ACC_VEC16) {
+        Store16(base, pos, v);
+    } else {
+        Vec16A4 t{v.x, v.y, v.z, v.w};
+        *reinterpret_cast<Vec16A4 *>(static_cast<char *>(base) + pos) = t;
+    }
+}
+
+// One pass over kChainVec * 256 vectors starting at vector vecBase of the tile.
+// FULL: every lane has all its vectors inside the tile (no per-lane guards).
+template <typename T, int OP, uint32_t MODE, bool FULL>
 __device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *const *__restrict__ src,
     void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec)
 {
-    // lane handles vectors vecBase + u * 256 + tid, u < kChainVec (guarded by nvec)
     const uint32_t tid = threadIdx.x;
     uint64_t pos[kChainVec];
     bool live[kChainVec];
 #pragma unroll
     for (uint32_t u = 0; u < kChainVec; u++) {
         uint32_t i = vecBase + u * kBlockThreads + tid;
-        live[u] = i < nvec;
+        live[u] = FULL || i < nvec;
         pos[u] = off + uint64_t(i) * 16;
     }
     V4 acc[kChainVec];
-    const void *s0 = src[0];
-#pragma unroll
-    for (uint32_t u = 0; u < kChainVec; u++) {
-        if (live[u]) {
-            acc[u] = Load16<MODE>(s0, pos[u]);
-        }
-    }
-    for (uint32_t j = 1; j < d.nsrc; j += kChainSrcBatch) {
+    const uint32_t nsrc = d.nsrc;
+    for (uint32_t j = 0; j < nsrc; j += kChainSrcBatch) {
         V4 v[kChainSrcBatch][kChainVec];
 #pragma unroll
         for (uint32_t jj = 0; jj < kChainSrcBatch; jj++) {
-            if (j + jj < d.nsrc) {
+            if (j + jj < nsrc) {
                 const void *s = src[j + jj];
 #pragma unroll
                 for (uint32_t u = 0; u < kChainVec; u++) {
@@ -306,28 +319,31 @@ __device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *con
         }
 #pragma unroll
         for (uint32_t jj = 0; jj < kChainSrcBatch; jj++) {
-            if (j + jj < d.nsrc) {
-                const bool accLeft = (d.accLeftMask >> (j + jj)) & 1ull;
+            if (j + jj < nsrc) {
+                if (j + jj == 0) {
 #pragma unroll
-                for (uint32_t u = 0; u < kChainVec; u++) {
-                    if (live[u]) {
-                        acc[u] = accLeft ? Combine16<T, OP>(acc[u], v[jj][u]) : Combine16<T, OP>(v[jj][u], acc[u]);
+                    for (uint32_t u = 0; u < kChainVec; u++) {
+                        acc[u] = v[0][u];
+                    }
+                } else {
+                    const bool accLeft = OrderMatters<T, OP>::value && ((d.accLeftMask >> (j + jj)) & 1ull);
+#pragma unroll
+                    for (uint32_t u = 0; u < kChainVec; u++) {
+                        if (live[u]) {
+                            acc[u] = accLeft ? Combine16<T, OP>(acc[u], v[jj][u]) : Combine16<T, OP>(v[jj][u], acc[u]);
+                        }
                     }
                 }
             }
         }
     }
-    for (uint32_t k = 0; k < d.ndst; k++) {
+    const uint32_t ndst = d.ndst;
+    for (uint32_t k = 0; k < ndst; k++) {
         void *o = dst[k];
 #pragma unroll
         for (uint32_t u = 0; u < kChainVec; u++) {
             if (live[u]) {
-                if (MODE == ACC_VEC16) {
-                    Store16(o, pos[u], acc[u]);
-                } else {
-                    Vec16A4 t{acc[u].x, acc[u].y, acc[u].z, acc[u].w};
-                    *reinterpret_cast<Vec16A4 *>(static_cast<char *>(o) + pos[u]) = t;
-                }
+                StoreAny16<MODE>(o, pos[u], acc[u]);
             }
         }
     }
@@ -366,11 +382,18 @@ __global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__
             ChainElem<T, OP>(d, src, dst, off, n);
         } else {
             const uint32_t nvec = n >> 4;
-            for (uint32_t base = 0; base < nvec; base += kChainVec * kBlockThreads) {
-                if (d.mode == ACC_VEC16) {
-                    ChainVecPass<T, OP, ACC_VEC16>(d, src, dst, off, base, nvec);
-                } else {
-                    ChainVecPass<T, OP, ACC_VEC16_SRC4>(d, src, dst, off, base, nvec);
+            constexpr uint32_t kPass = kChainVec * kBlockThreads;
+            uint32_t base = 0;
+            if (d.mode == ACC_VEC16) {
+                for (; base + kPass <= nvec; base += kPass) {
+                    ChainVecPass<T, OP, ACC_VEC16, true>(d, src, dst, off, base, nvec);
+                }
+                if (base < nvec) {
+                    ChainVecPass<T, OP, ACC_VEC16, false>(d, src, dst, off, base, nvec);
+                }
+            } else {
+                for (; base < nvec; base += kPass) {
+                    ChainVecPass<T, OP, ACC_VEC16_SRC4, false>(d, src, dst, off, base, nvec);
                 }
             }
         }

@@ -15,6 +15,7 @@
 #include <memory>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "hccl/hccl_types.h"
@@ -33,7 +34,7 @@ struct GroupConfig {
     bool fuse = true;                     // run the fused single-pass form when the plan has one
     bool graph = true;                    // issue through a HIP graph
     bool deterministic = false;
-    uint32_t blocksPerCu = 8;
+    uint32_t blocksPerCu = 0;             // workgroups per CU; 0 = per-kernel default
     bool blockingArrive = false;          // ranks wait inside the call until the collective is issued
     uint32_t arriveTimeoutMs = 1800 * 1000;
 };
@@ -121,7 +122,7 @@ struct Group {
     std::vector<void *> scratch;
     uint64_t scratchBytes = 0;
     uint64_t scratchGen = 0;
-    std::map<std::string, std::unique_ptr<Prepared>> cache;
+    std::unordered_map<std::string, std::unique_ptr<Prepared>> cache;
     uint64_t useClock = 0;
     OpInfo lastInfo;
 
