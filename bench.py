@@ -20,8 +20,9 @@ METRIC = "achieved HBM GB/s & % of peak, 8-rank fp32 ring AllReduce 256MiB/rank"
 
 # HBM traffic of the fused all-reduce kernel at the default workload, from rocprofv3 --pmc
 # (FETCH_SIZE, WRITE_SIZE), scaled by the same counters over a plain copy of known size.
-# None until measured; the figures and the commands are in profiles/.
-MEASURED_TRAFFIC_BYTES = None
+# Valid for the default workload only (8 ranks x 256 MiB); the figures and the commands are in
+# profiles/ChainKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt.
+MEASURED_TRAFFIC_BYTES = 4295754000
 
 
 def run_mode(pkg, torch, comms, stream, sends, recvs, n, fuse, steps, warmup):
@@ -179,7 +180,8 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES if (p == 8 and args.size_mib == 256.0 and not args.set) else None,
             "kernel": "ChainKernel<float, sum> (fused ring all-reduce), avg launch %.4f ms over %d launches" % (dev_ms, args.steps),
         },
         "cpu_baseline": cpu,
