@@ -50,6 +50,128 @@ def run_mode(pkg, torch, comms, stream, sends, recvs, n, fuse, steps, warmup):
     return wall_ms, dev_ms, info
 
 
+def time_calls(torch, stream, call, steps, warmup):
+    for _ in range(warmup):
+        call()
+    stream.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(steps):
+        call()
+    e1.record(stream)
+    stream.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def run_suite(pkg, torch, steps, warmup, only="", settings=()):
+    """The other configurations of BASELINE.json (reduce-scatter op x type matrix, 16-rank all-to-all-v,
+    halving-doubling all-reduce in bf16 at 32 and 24 ranks, all-gather), fused and step-by-step: a table on stderr."""
+    import numpy as np
+    stream = torch.cuda.Stream()
+    out = sys.stderr
+    out.write("%-46s %-6s %9s %10s %9s %8s\n" % ("configuration", "mode", "launches", "time_us", "GB/s", "%peak"))
+
+    def report(name, comms, call):
+        if only and only not in name:
+            return
+        for kv in settings:
+            k, v = kv.split("=", 1)
+            pkg.set_param(comms[0], k, v)
+        for fuse in (1, 0):
+            pkg.set_param(comms[0], "fuse", fuse)
+            ms = time_calls(torch, stream, call, steps, warmup)
+            info = pkg.last_op_info(comms[0])
+            moved = info["bytesRead"] + info["bytesWritten"]
+            gbps = moved / (ms * 1e-3) / 1e9
+            out.write("%-46s %-6s %9d %10.1f %9.1f %8.1f\n" % (name, "fused" if info["fused"] else "steps", info["launches"],
+                                                              ms * 1e3, gbps, 100 * gbps / HBM_PEAK_GBPS))
+
+    dtypes = {"fp16": (pkg.HCCL_DATA_TYPE_FP16, torch.float16), "bf16": (pkg.HCCL_DATA_TYPE_BFP16, torch.bfloat16),
+              "int8": (pkg.HCCL_DATA_TYPE_INT8, torch.int8), "int32": (pkg.HCCL_DATA_TYPE_INT32, torch.int32),
+              "int64": (pkg.HCCL_DATA_TYPE_INT64, torch.int64), "fp32": (pkg.HCCL_DATA_TYPE_FP32, torch.float32)}
+    ops = {"sum": 0, "prod": 1, "max": 2, "min": 3}
+
+    def rand(n, tdt):
+        if tdt.is_floating_point:
+            return torch.randn(n, dtype=torch.float32, device="cuda").to(tdt)
+        if tdt == torch.int64:
+            return torch.randint(-(1 << 40), 1 << 40, (n,), dtype=tdt, device="cuda")
+        info = torch.iinfo(tdt)
+        return torch.randint(info.min, info.max, (n,), dtype=tdt, device="cuda")
+
+    # reduce-scatter, 8 ranks, 64 MiB per rank send buffer
+    p = 8
+    comms = pkg.comm_init_all(p)
+    for tname in ("fp16", "bf16", "int8", "int32", "int64"):
+        hdt, tdt = dtypes[tname]
+        unit = pkg.DTYPE_SIZE[hdt]
+        n = (64 << 20) // unit // p
+        sends = [rand(n * p, tdt) for _ in range(p)]
+        recvs = [torch.empty(n, dtype=tdt, device="cuda") for _ in range(p)]
+        sp, rp = [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs]
+        torch.cuda.synchronize()
+        for oname, op in ops.items():
+            report("reduce-scatter ring p=8 64MiB/rank %s %s" % (tname, oname), comms,
+                   lambda: pkg.reduce_scatter(comms, sp, rp, n, hdt, op, stream.cuda_stream))
+        del sends, recvs
+    # all-gather, 8 ranks, 32 MiB per rank in, 256 MiB per rank out
+    n = (32 << 20)
+    sends = [rand(n, torch.int8) for _ in range(p)]
+    recvs = [torch.empty(n * p, dtype=torch.int8, device="cuda") for _ in range(p)]
+    sp, rp = [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs]
+    torch.cuda.synchronize()
+    report("all-gather ring p=8 32MiB/rank in", comms,
+           lambda: pkg.all_gather(comms, sp, rp, n, pkg.HCCL_DATA_TYPE_INT8, stream.cuda_stream))
+    del sends, recvs
+    pkg.comm_destroy(comms)
+
+    # all-to-all-v, 16 ranks, lognormal counts
+    p = 16
+    rng = np.random.default_rng(2024)
+    cnt = np.clip(np.rint(np.exp(np.log(65536.0) + rng.standard_normal((p, p)))), 0, 4 << 20).astype(np.uint64)
+    sdis, rdis = np.zeros((p, p), np.uint64), np.zeros((p, p), np.uint64)
+    sl, rl = [], []
+    for r in range(p):
+        pos = 0
+        for j in rng.permutation(p):
+            pos += int(rng.integers(0, 1024))
+            sdis[r, j] = pos
+            pos += int(cnt[r, j])
+        sl.append(pos)
+        pos = 0
+        for i in rng.permutation(p):
+            pos += int(rng.integers(0, 1024))
+            rdis[r, i] = pos
+            pos += int(cnt[i, r])
+        rl.append(pos)
+    comms = pkg.comm_init_all(p)
+    sends = [rand(max(x, 1), torch.int32) for x in sl]
+    recvs = [torch.empty(max(x, 1), dtype=torch.int32, device="cuda") for x in rl]
+    sp, rp = [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs]
+    torch.cuda.synchronize()
+    tables = pkg.a2av_tables(cnt, sdis, cnt.T.copy(), rdis)
+    report("all-to-all-v pairwise p=16 int32 lognormal (%.0f MB)" % (4 * cnt.sum() / 1e6), comms,
+           lambda: pkg.all_to_all_v(comms, sp, None, None, rp, None, None, pkg.HCCL_DATA_TYPE_INT32, stream.cuda_stream,
+                                    tables=tables))
+    del sends, recvs
+    pkg.comm_destroy(comms)
+
+    # halving-doubling all-reduce, bf16, 128 MiB per rank, 32 and 24 ranks
+    for p in (32, 24):
+        comms = pkg.comm_init_all(p)
+        pkg.set_param(comms[0], "algo", "rhd")
+        n = (128 << 20) // 2
+        sends = [rand(n, torch.bfloat16) for _ in range(p)]
+        recvs = [torch.empty(n, dtype=torch.bfloat16, device="cuda") for _ in range(p)]
+        sp, rp = [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs]
+        torch.cuda.synchronize()
+        report("all-reduce rhd p=%d bf16 sum 128MiB/rank" % p, comms,
+               lambda: pkg.all_reduce(comms, sp, rp, n, pkg.HCCL_DATA_TYPE_BFP16, 0, stream.cuda_stream))
+        del sends, recvs
+        pkg.comm_destroy(comms)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -59,6 +181,8 @@ def main():
     ap.add_argument("--ranks", type=int, default=8)
     ap.add_argument("--sweep", action="store_true", help="also time 8 KiB .. 256 MiB per rank (x2), table on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--suite-filter", default="", help="with --suite: only configurations whose name contains this")
+    ap.add_argument("--suite", action="store_true", help="time the other BASELINE.json configurations (table on stderr) and exit")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 1 GiB int32 copy (one-rank all-reduce, out of place) three times, so that a "
                          "counter profile of this command holds a copy of known size to scale FETCH_SIZE / WRITE_SIZE by")
@@ -78,6 +202,9 @@ def main():
     pkg.lib()                                  # raises if the HIP library is not built
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+    if args.suite:
+        run_suite(pkg, torch, args.steps, args.warmup, args.suite_filter, args.set)
+        return
     p = args.ranks
     n = int(args.size_mib * (1 << 20)) // 4
     S = n * 4

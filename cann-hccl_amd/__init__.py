@@ -144,15 +144,21 @@ def all_gather(comms, sends, recvs, send_count, dtype, stream):
         _check("HcclAllGather", lib().HcclAllGather(s, r, send_count, dtype, c, stream))
 
 
-def all_to_all_v(comms, sends, send_counts, sdispls, recvs, recv_counts, rdispls, dtype, stream):
-    """counts / displs: per rank, sequences of p integers (elements)."""
-    p = len(comms)
-    keep = []
-    for r in range(p):
-        arrs = [(ctypes.c_uint64 * p)(*[int(x) for x in t[r]]) for t in (send_counts, sdispls, recv_counts, rdispls)]
-        keep.append(arrs)
-        _check("HcclAlltoAllV", lib().HcclAlltoAllV(sends[r], arrs[0], arrs[1], dtype, recvs[r], arrs[2], arrs[3], dtype,
-                                                   comms[r], stream))
+def a2av_tables(send_counts, sdispls, recv_counts, rdispls):
+    """Per rank, the four host uint64[p] arrays HcclAlltoAllV takes (build once, reuse across calls)."""
+    p = len(send_counts)
+    return [[(ctypes.c_uint64 * p)(*[int(x) for x in t[r]]) for t in (send_counts, sdispls, recv_counts, rdispls)]
+            for r in range(p)]
+
+
+def all_to_all_v(comms, sends, send_counts, sdispls, recvs, recv_counts, rdispls, dtype, stream, tables=None):
+    """counts / displs: per rank, sequences of p integers (elements); or pass tables=a2av_tables(...)."""
+    if tables is None:
+        tables = a2av_tables(send_counts, sdispls, recv_counts, rdispls)
+    fn = lib().HcclAlltoAllV
+    for r, c in enumerate(comms):
+        t = tables[r]
+        _check("HcclAlltoAllV", fn(sends[r], t[0], t[1], dtype, recvs[r], t[2], t[3], dtype, c, stream))
 
 
 def describe_plan(coll, algo, p, count, dtype, ccl_bytes=200 << 20, align=128, in_place_mask=0, tables=None):

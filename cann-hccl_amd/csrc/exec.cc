@@ -141,10 +141,29 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
     Builder b;
     b.g = g;
     std::vector<PendingLaunch> pending;
-    // Launch width: streaming kernels on this part run best with few, fat workgroups (measured on
-    // MI355X at 8 ranks x 256 MiB: 1 per CU for the fused 8 -> 8 shape, 2 per CU for the step kernel).
+    // Launch width.  Streaming kernels on this part run best with few, fat workgroups as long as a
+    // lane keeps enough memory operations in flight: 1 workgroup per CU when an item touches 8 or
+    // more streams (sources + destinations), more when it touches fewer (measured on MI355X: 8 -> 8
+    // all-reduce and 1 -> 8 all-gather best at 1 per CU, the 2 -> 1 step kernel at 2 per CU).
     const uint32_t stepGrid = std::max(1u, g->numCu * (g->cfg.blocksPerCu ? g->cfg.blocksPerCu : 2u));
-    const uint32_t fusedGrid = std::max(1u, g->numCu * (g->cfg.blocksPerCu ? g->cfg.blocksPerCu : 1u));
+    uint32_t fusedPerCu = g->cfg.blocksPerCu;
+    if (fusedPerCu == 0) {
+        double streamBytes = 0, bytes = 0;
+        for (const FusedItem &it : pp->plan.fused) {
+            uint32_t nsrc = 0;
+            for (uint8_t v : it.srcValid) {
+                nsrc += v;
+            }
+            streamBytes += double(nsrc + it.dst.size()) * double(it.bytes);
+            bytes += double(it.bytes);
+        }
+        double streams = bytes > 0 ? streamBytes / bytes : 2.0;   // loads + stores per lane and vector
+        fusedPerCu = streams >= 8.0 ? 1u : (streams >= 3.0 ? 2u : 4u);
+    }
+    // the tree kernel does log2(p) levels of arithmetic per vector: it needs a second wave per SIMD
+    // to overlap that with memory (measured: 32-rank bf16 all-reduce 2.17 ms at 1 per CU, 1.69 ms at 2)
+    const uint32_t treeGrid = std::max(1u, g->numCu * (g->cfg.blocksPerCu ? g->cfg.blocksPerCu : 2u));
+    const uint32_t fusedGrid = std::max(1u, g->numCu * fusedPerCu);
 
     if (!pp->fused) {
         const void *func = reduceColl ? LookupKernel(dtype, op, KK_STEP) : LookupCopyKernel(KK_STEP);
@@ -189,13 +208,13 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
         }
     } else {
         // one launch per kernel kind present
-        for (int kind : {int(KK_CHAIN), int(KK_TREE8), int(KK_TREE32)}) {
+        for (int kind : {int(KK_CHAIN), int(KK_TREE)}) {
             std::vector<FusedDesc> descs;
             std::vector<const void *> srcPool;
             std::vector<void *> dstPool;
             uint32_t tiles = 0;
             for (const FusedItem &it : pp->plan.fused) {
-                int want = (it.kind == FK_TREE) ? (it.nleaf <= 8 ? int(KK_TREE8) : int(KK_TREE32)) : int(KK_CHAIN);
+                int want = (it.kind == FK_TREE) ? int(KK_TREE) : int(KK_CHAIN);
                 if (want != kind) {
                     continue;
                 }
@@ -255,7 +274,7 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
             pl.rec.func = func;
             pl.rec.nitems = uint32_t(descs.size());
             pl.rec.ntiles = tiles;
-            pl.rec.grid = std::min(tiles, fusedGrid);
+            pl.rec.grid = std::min(tiles, kind == int(KK_TREE) ? treeGrid : fusedGrid);
             pl.rec.fusedArgs = true;
             pending.push_back(pl);
         }

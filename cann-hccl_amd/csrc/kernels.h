@@ -48,7 +48,7 @@ struct FusedDesc {
     uint32_t pad;
 };
 
-enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE8 = 2, KK_TREE32 = 3, KK_COUNT = 4 };
+enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_COUNT = 3 };
 
 // Kernel entry for (data type, reduce op, kind); nullptr if the combination is not built.
 // Signatures:

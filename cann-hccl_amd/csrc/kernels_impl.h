@@ -139,22 +139,114 @@ template <int OP> struct Elem<Bf16Bits, OP> {
 };
 
 // 16 bytes of T combined lane by lane; a is the rank's own operand, b the peer's.
-template <typename T, int OP> __device__ __forceinline__ V4 Combine16(V4 a, V4 b)
-{
-    constexpr int N = 16 / sizeof(T);
-    union U {
-        V4 v;
-        T e[N];
-        __device__ U() {}
-    } ua, ub, ur;
-    ua.v = a;
-    ub.v = b;
+template <typename T, int OP> struct Combiner {
+    static __device__ __forceinline__ V4 Apply(V4 a, V4 b)
+    {
+        constexpr int N = 16 / sizeof(T);
+        union U {
+            V4 v;
+            T e[N];
+            __device__ U() {}
+        } ua, ub, ur;
+        ua.v = a;
+        ub.v = b;
 #pragma unroll
-    for (int i = 0; i < N; i++) {
-        ur.e[i] = Elem<T, OP>::Apply(ua.e[i], ub.e[i]);
+        for (int i = 0; i < N; i++) {
+            ur.e[i] = Elem<T, OP>::Apply(ua.e[i], ub.e[i]);
+        }
+        return ur.v;
     }
-    return ur.v;
+};
+
+// Narrow types work on whole 32-bit words with packed 16-bit instructions (v_pk_*_u16 / _i16) and the
+// hardware bf16 conversion (v_cvt_pk_bf16_f32, round to nearest even), a fraction of the instructions
+// that element-by-element extraction costs; the results are the same bits.
+typedef short S2 __attribute__((ext_vector_type(2)));
+typedef unsigned short U2 __attribute__((ext_vector_type(2)));
+typedef float F2 __attribute__((ext_vector_type(2)));
+typedef __bf16 B2 __attribute__((ext_vector_type(2)));
+
+template <typename To, typename From> __device__ __forceinline__ To BitCast(From f)
+{
+    static_assert(sizeof(To) == sizeof(From), "size");
+    To t;
+    __builtin_memcpy(&t, &f, sizeof(To));
+    return t;
 }
+
+template <bool SIGNED, int OP> __device__ __forceinline__ uint32_t Pk16(uint32_t a, uint32_t b)
+{
+    if (OP == ROP_SUM) {
+        return BitCast<uint32_t>(U2(BitCast<U2>(a) + BitCast<U2>(b)));
+    } else if (OP == ROP_PROD) {
+        return BitCast<uint32_t>(U2(BitCast<U2>(a) * BitCast<U2>(b)));
+    } else if (SIGNED) {
+        S2 x = BitCast<S2>(a), y = BitCast<S2>(b);
+        return BitCast<uint32_t>(OP == ROP_MAX ? __builtin_elementwise_max(x, y) : __builtin_elementwise_min(x, y));
+    } else {
+        U2 x = BitCast<U2>(a), y = BitCast<U2>(b);
+        return BitCast<uint32_t>(OP == ROP_MAX ? __builtin_elementwise_max(x, y) : __builtin_elementwise_min(x, y));
+    }
+}
+
+template <bool SIGNED, int OP> __device__ __forceinline__ uint32_t Pk8(uint32_t a, uint32_t b)
+{
+    if (OP == ROP_SUM) {
+        // add the low 7 bits of every byte, then fix the top bits without carrying across bytes
+        return ((a & 0x7f7f7f7fu) + (b & 0x7f7f7f7fu)) ^ ((a ^ b) & 0x80808080u);
+    } else if (OP == ROP_PROD) {
+        uint32_t even = Pk16<false, ROP_PROD>(a & 0x00ff00ffu, b & 0x00ff00ffu) & 0x00ff00ffu;
+        uint32_t odd = Pk16<false, ROP_PROD>((a >> 8) & 0x00ff00ffu, (b >> 8) & 0x00ff00ffu) & 0x00ff00ffu;
+        return even | (odd << 8);
+    } else {
+        // a byte moved to the top of a 16-bit lane compares like the byte itself
+        uint32_t even = Pk16<SIGNED, OP>((a << 8) & 0xff00ff00u, (b << 8) & 0xff00ff00u);
+        uint32_t odd = Pk16<SIGNED, OP>(a & 0xff00ff00u, b & 0xff00ff00u);
+        return ((even >> 8) & 0x00ff00ffu) | odd;
+    }
+}
+
+template <int OP> __device__ __forceinline__ uint32_t PkBf16(uint32_t a, uint32_t b)
+{
+    const uint32_t aLo = a << 16, aHi = a & 0xffff0000u, bLo = b << 16, bHi = b & 0xffff0000u;
+    const float faLo = __uint_as_float(aLo), faHi = __uint_as_float(aHi);
+    const float fbLo = __uint_as_float(bLo), fbHi = __uint_as_float(bHi);
+    if (OP == ROP_SUM || OP == ROP_PROD) {
+        F2 r;
+        r.x = (OP == ROP_SUM) ? faLo + fbLo : faLo * fbLo;
+        r.y = (OP == ROP_SUM) ? faHi + fbHi : faHi * fbHi;
+        return BitCast<uint32_t>(__builtin_convertvector(r, B2));
+    } else {
+        const bool pickLo = (OP == ROP_MAX) ? (fbLo > faLo) : (fbLo < faLo);
+        const bool pickHi = (OP == ROP_MAX) ? (fbHi > faHi) : (fbHi < faHi);
+        return ((pickHi ? bHi : aHi)) | ((pickLo ? bLo : aLo) >> 16);
+    }
+}
+
+#define HCCL_WORDWISE_COMBINER(TYPE, EXPR)                                  \
+    template <int OP> struct Combiner<TYPE, OP> {                           \
+        static __device__ __forceinline__ V4 Apply(V4 a, V4 b)              \
+        {                                                                   \
+            V4 r;                                                           \
+            r.x = EXPR(a.x, b.x);                                           \
+            r.y = EXPR(a.y, b.y);                                           \
+            r.z = EXPR(a.z, b.z);                                           \
+            r.w = EXPR(a.w, b.w);                                           \
+            return r;                                                       \
+        }                                                                   \
+    };
+#define HCCL_EXPR_I16(x, y) Pk16<true, OP>(x, y)
+#define HCCL_EXPR_U16(x, y) Pk16<false, OP>(x, y)
+#define HCCL_EXPR_I8(x, y) Pk8<true, OP>(x, y)
+#define HCCL_EXPR_U8(x, y) Pk8<false, OP>(x, y)
+#define HCCL_EXPR_BF16(x, y) PkBf16<OP>(x, y)
+HCCL_WORDWISE_COMBINER(int16_t, HCCL_EXPR_I16)
+HCCL_WORDWISE_COMBINER(uint16_t, HCCL_EXPR_U16)
+HCCL_WORDWISE_COMBINER(int8_t, HCCL_EXPR_I8)
+HCCL_WORDWISE_COMBINER(uint8_t, HCCL_EXPR_U8)
+HCCL_WORDWISE_COMBINER(Bf16Bits, HCCL_EXPR_BF16)
+
+template <typename T, int OP> __device__ __forceinline__ V4 Combine16(V4 a, V4 b) { return Combiner<T, OP>::Apply(a, b); }
 
 // ---- memory access ---------------------------------------------------------------------------------
 struct __attribute__((packed, aligned(4))) Vec16A4 {
@@ -401,57 +493,77 @@ __global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__
 }
 
 // ---- fused perfect tree (halving-doubling): leaves pairwise bottom-up ----------------------------------
-template <typename T, int OP, uint32_t MAXLEAF, uint32_t MODE>
-__device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *const *__restrict__ src,
-    void *const *__restrict__ dst, uint64_t pos)
+// v[i] = v[i] (+) v[i+w] for w = 1, 2, 4, ... is evaluated group by group: the first three levels
+// inside groups of 8 consecutive leaves (8 loads in flight, one result kept per group), the remaining
+// levels over the group results.  Same association as the flat loop, a quarter of the registers.
+constexpr uint32_t kTreeGroup = 8;
+constexpr uint32_t kTreeMaxGroups = 4;   // up to 32 leaves
+
+template <typename T, int OP, uint32_t MODE>
+__device__ __forceinline__ V4 TreeValue(const FusedDesc &d, const void *const *__restrict__ src, uint64_t pos)
 {
-    V4 v[MAXLEAF];
+    const uint32_t nleaf = d.nleaf;
+    const uint32_t ngroups = (nleaf + kTreeGroup - 1) / kTreeGroup;   // 1, or a power of two
+    // Pending left operands of the upper levels (a binary counter over the groups seen so far).
+    V4 l0 = {0, 0, 0, 0}, l1 = {0, 0, 0, 0};
+    V4 x = {0, 0, 0, 0};
+    // Kept as a loop on purpose: unrolled, the compiler hoists every group's loads to the top and
+    // the register count (and with it the number of resident waves) is back to the flat version's.
+#pragma nounroll
+    for (uint32_t gi = 0; gi < ngroups; gi++) {
+        const void *const *gs = src + 2 * gi * kTreeGroup;
+        const uint32_t left = nleaf - gi * kTreeGroup;   // leaves in this and later groups
+        V4 v[kTreeGroup];
 #pragma unroll
-    for (uint32_t i = 0; i < MAXLEAF; i++) {
-        if (i < d.nleaf) {
-            v[i] = Load16<MODE>(src[2 * i], pos);
-        }
-    }
-#pragma unroll
-    for (uint32_t i = 0; i < MAXLEAF; i++) {
-        if (i < d.nleaf) {
-            const void *s = src[2 * i + 1];
-            if (s != nullptr) {
-                v[i] = Combine16<T, OP>(v[i], Load16<MODE>(s, pos));
+        for (uint32_t i = 0; i < kTreeGroup; i++) {
+            if (i < left) {
+                v[i] = Load16<MODE>(gs[2 * i], pos);
             }
         }
-    }
 #pragma unroll
-    for (uint32_t w = 1; w < MAXLEAF; w <<= 1) {
-        if (w < d.nleaf) {
+        for (uint32_t i = 0; i < kTreeGroup; i++) {
+            if (i < left) {
+                const void *s = gs[2 * i + 1];
+                if (s != nullptr) {
+                    v[i] = Combine16<T, OP>(v[i], Load16<MODE>(s, pos));
+                }
+            }
+        }
 #pragma unroll
-            for (uint32_t i = 0; i + w < MAXLEAF; i += 2 * w) {
-                if (i + w < d.nleaf) {
+        for (uint32_t w = 1; w < kTreeGroup; w <<= 1) {
+#pragma unroll
+            for (uint32_t i = 0; i + w < kTreeGroup; i += 2 * w) {
+                if (i + w < left) {
                     v[i] = Combine16<T, OP>(v[i], v[i + w]);
                 }
             }
         }
-    }
-    for (uint32_t k = 0; k < d.ndst; k++) {
-        if (MODE == ACC_VEC16) {
-            Store16(dst[k], pos, v[0]);
+        x = v[0];
+        if ((gi & 1u) == 0) {
+            l0 = x;
         } else {
-            Vec16A4 t{v[0].x, v[0].y, v[0].z, v[0].w};
-            *reinterpret_cast<Vec16A4 *>(static_cast<char *>(dst[k]) + pos) = t;
+            x = Combine16<T, OP>(l0, x);
+            if ((gi & 2u) == 0) {
+                l1 = x;
+            } else {
+                x = Combine16<T, OP>(l1, x);
+            }
         }
     }
+    return x;
 }
 
-template <typename T, int OP, uint32_t MAXLEAF>
+template <typename T, int OP>
 __device__ __forceinline__ void TreeElem(const FusedDesc &d, const void *const *__restrict__ src,
     void *const *__restrict__ dst, uint64_t off, uint32_t n)
 {
+    constexpr uint32_t kMax = kTreeGroup * kTreeMaxGroups;
     const uint32_t cnt = n / sizeof(T);
     for (uint32_t e = threadIdx.x; e < cnt; e += kBlockThreads) {
         const uint64_t at = off + uint64_t(e) * sizeof(T);
-        T v[MAXLEAF];
+        T v[kMax];
 #pragma unroll
-        for (uint32_t i = 0; i < MAXLEAF; i++) {
+        for (uint32_t i = 0; i < kMax; i++) {
             if (i < d.nleaf) {
                 v[i] = *reinterpret_cast<const T *>(static_cast<const char *>(src[2 * i]) + at);
                 const void *s = src[2 * i + 1];
@@ -461,10 +573,10 @@ __device__ __forceinline__ void TreeElem(const FusedDesc &d, const void *const *
             }
         }
 #pragma unroll
-        for (uint32_t w = 1; w < MAXLEAF; w <<= 1) {
+        for (uint32_t w = 1; w < kMax; w <<= 1) {
             if (w < d.nleaf) {
 #pragma unroll
-                for (uint32_t i = 0; i + w < MAXLEAF; i += 2 * w) {
+                for (uint32_t i = 0; i + w < kMax; i += 2 * w) {
                     if (i + w < d.nleaf) {
                         v[i] = Elem<T, OP>::Apply(v[i], v[i + w]);
                     }
@@ -477,7 +589,7 @@ __device__ __forceinline__ void TreeElem(const FusedDesc &d, const void *const *
     }
 }
 
-template <typename T, int OP, uint32_t MAXLEAF>
+template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) TreeKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool)
 {
@@ -489,14 +601,21 @@ __global__ void __launch_bounds__(kBlockThreads) TreeKernel(const FusedDesc *__r
         const void *const *src = srcPool + d.srcBase;
         void *const *dst = dstPool + d.dstBase;
         if (d.mode == ACC_ELEM) {
-            TreeElem<T, OP, MAXLEAF>(d, src, dst, off, n);
+            TreeElem<T, OP>(d, src, dst, off, n);
         } else {
             const uint32_t nvec = n >> 4;
             for (uint32_t i = threadIdx.x; i < nvec; i += kBlockThreads) {
+                const uint64_t pos = off + uint64_t(i) * 16;
                 if (d.mode == ACC_VEC16) {
-                    TreeVecPass<T, OP, MAXLEAF, ACC_VEC16>(d, src, dst, off + uint64_t(i) * 16);
+                    V4 r = TreeValue<T, OP, ACC_VEC16>(d, src, pos);
+                    for (uint32_t k = 0; k < d.ndst; k++) {
+                        Store16(dst[k], pos, r);
+                    }
                 } else {
-                    TreeVecPass<T, OP, MAXLEAF, ACC_VEC16_SRC4>(d, src, dst, off + uint64_t(i) * 16);
+                    V4 r = TreeValue<T, OP, ACC_VEC16_SRC4>(d, src, pos);
+                    for (uint32_t k = 0; k < d.ndst; k++) {
+                        StoreAny16<ACC_VEC16_SRC4>(dst[k], pos, r);
+                    }
                 }
             }
         }
