@@ -78,6 +78,10 @@ def lib():
     L.HcclReduceScatter.argtypes = [vp, vp, u64, i32, i32, vp, vp]
     L.HcclAllGather.argtypes = [vp, vp, u64, i32, vp, vp]
     L.HcclAlltoAllV.argtypes = [vp, vp, vp, i32, vp, vp, vp, i32, vp, vp]
+    L.HcclAlltoAll.argtypes = [vp, u64, i32, vp, u64, i32, vp, vp]
+    L.HcclReduceScatterV.argtypes = [vp, vp, vp, vp, u64, i32, i32, vp, vp]
+    L.HcclAllGatherV.argtypes = [vp, u64, vp, vp, vp, i32, vp, vp]
+    L.HcclBarrier.argtypes = [vp, vp]
     L.HcclGetErrorString.restype = ctypes.c_char_p
     L.HcclGetErrorString.argtypes = [i32]
     L.HcclGetCommConfigCapability.restype = u32
@@ -144,6 +148,32 @@ def all_gather(comms, sends, recvs, send_count, dtype, stream):
         _check("HcclAllGather", lib().HcclAllGather(s, r, send_count, dtype, c, stream))
 
 
+def all_to_all(comms, sends, recvs, count, dtype, stream):
+    for c, s, r in zip(comms, sends, recvs):
+        _check("HcclAlltoAll", lib().HcclAlltoAll(s, count, dtype, r, count, dtype, c, stream))
+
+
+def reduce_scatter_v(comms, sends, counts, displs, recvs, dtype, op, stream):
+    p = len(comms)
+    c = (ctypes.c_uint64 * p)(*[int(x) for x in counts])
+    d = (ctypes.c_uint64 * p)(*[int(x) for x in displs])
+    for r in range(p):
+        _check("HcclReduceScatterV", lib().HcclReduceScatterV(sends[r], c, d, recvs[r], int(counts[r]), dtype, op, comms[r], stream))
+
+
+def all_gather_v(comms, sends, recvs, counts, displs, dtype, stream):
+    p = len(comms)
+    c = (ctypes.c_uint64 * p)(*[int(x) for x in counts])
+    d = (ctypes.c_uint64 * p)(*[int(x) for x in displs])
+    for r in range(p):
+        _check("HcclAllGatherV", lib().HcclAllGatherV(sends[r], int(counts[r]), recvs[r], c, d, dtype, comms[r], stream))
+
+
+def barrier(comms, stream):
+    for c in comms:
+        _check("HcclBarrier", lib().HcclBarrier(c, stream))
+
+
 def a2av_tables(send_counts, sdispls, recv_counts, rdispls):
     """Per rank, the four host uint64[p] arrays HcclAlltoAllV takes (build once, reuse across calls)."""
     p = len(send_counts)
@@ -164,7 +194,10 @@ def all_to_all_v(comms, sends, send_counts, sdispls, recvs, recv_counts, rdispls
 def describe_plan(coll, algo, p, count, dtype, ccl_bytes=200 << 20, align=128, in_place_mask=0, tables=None):
     """Plan a collective without a GPU; returns the plan as a dict (see HcclAmdDescribePlan)."""
     tab = None
-    if tables is not None:
+    if tables is not None and coll != COLL_ALLTOALLV:
+        flat = [int(x) for t in tables for x in t]          # (counts, displs)
+        tab = (ctypes.c_uint64 * len(flat))(*flat)
+    elif tables is not None:
         flat = [int(x) for t in tables for row in t for x in row]
         tab = (ctypes.c_uint64 * len(flat))(*flat)
     cap = 1 << 20

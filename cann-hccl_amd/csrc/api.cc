@@ -9,6 +9,7 @@
 #include <cstring>
 #include <set>
 #include <string>
+#include <vector>
 
 #include "hccl/hccl.h"
 #include "hccl/hccl_amd_ext.h"
@@ -153,7 +154,8 @@ void CancelPending(Group *g)
 
 // One rank joins the current collective.  The last rank to join issues it.
 HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t stream, const uint64_t *sendCounts,
-    const uint64_t *sdispls, const uint64_t *recvCounts, const uint64_t *rdispls)
+    const uint64_t *sdispls, const uint64_t *recvCounts, const uint64_t *rdispls, const uint64_t *vCounts = nullptr,
+    const uint64_t *vDispls = nullptr)
 {
     Group *g = c->group;
     std::unique_lock<std::mutex> lock(g->m);
@@ -165,9 +167,19 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
         HCCL_LOG_ERROR("%s: rank %u called again before the other ranks joined the previous call", CollName(sig.coll), r);
         return HCCL_E_AGAIN;
     }
+    bool tablesDiffer = false;
+    if (sig.variable && g->arrived > 0 && g->sig.variable) {
+        for (uint32_t i = 0; i < g->p; i++) {
+            tablesDiffer = tablesDiffer || g->vCounts[i] != vCounts[i] || g->vDispls[i] != vDispls[i];
+        }
+    }
     if (g->arrived == 0) {
         g->sig = sig;
-    } else if (!(g->sig == sig)) {
+        if (sig.variable) {
+            g->vCounts.assign(vCounts, vCounts + g->p);
+            g->vDispls.assign(vDispls, vDispls + g->p);
+        }
+    } else if (!(g->sig == sig) || tablesDiffer) {
         // every rank must pass the same operation, count, type and op (the reference checks this
         // across processes in RankConsistentcyChecker, hccl_communicator.cc:2803-2805)
         HCCL_LOG_ERROR("%s: rank %u disagrees with the ranks already in the collective (op/count/type)", CollName(sig.coll), r);
@@ -614,6 +626,200 @@ HcclResult HcclAlltoAllV(const void *sendBuf, const void *sendCounts, const void
         static_cast<const uint64_t *>(sdispls), rc, static_cast<const uint64_t *>(rdispls));
 }
 
+// ---- siblings that run through the same schedules and kernels -----------------------------------------
+
+// op_base.cc:1585-1718.  Ring / mesh / halving-doubling reduce-scatter over the caller's block table;
+// every rank must pass the same table and recvCount == sendCounts[rank].
+HcclResult HcclReduceScatterV(void *sendBuf, const void *sendCounts, const void *sendDispls, void *recvBuf,
+    uint64_t recvCount, HcclDataType dataType, HcclReduceOp op, HcclComm comm, aclrtStream stream)
+{
+    CHK_PTR(sendCounts);
+    CHK_PTR(sendDispls);
+    CHK_PTR(comm);
+    if (recvCount > 0) {
+        CHK_PTR(recvBuf);
+    }
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    HcclResult r = CheckOpParam("HcclReduceScatterV", recvCount, dataType, stream);
+    if (r == HCCL_SUCCESS) {
+        r = CheckReduce("HcclReduceScatterV", dataType, op);
+    }
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    const uint64_t *counts = static_cast<const uint64_t *>(sendCounts);
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < c->group->p; i++) {
+        if (counts[i] > kSysMaxCount) {
+            HCCL_LOG_ERROR("HcclReduceScatterV: sendCounts[%u] exceeds the maximum", i);
+            return HCCL_E_PARA;
+        }
+        total += counts[i];
+    }
+    if (total == 0) {
+        HCCL_LOG_WARN("HcclReduceScatterV: nothing to reduce");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(sendBuf);
+    if (counts[c->rank] != recvCount) {
+        HCCL_LOG_ERROR("HcclReduceScatterV: recvCount %llu differs from sendCounts[rank] %llu",
+            (unsigned long long)recvCount, (unsigned long long)counts[c->rank]);
+        return HCCL_E_PARA;
+    }
+    uint32_t unit = ElemSize(dataType);
+    if (reinterpret_cast<uintptr_t>(sendBuf) % unit != 0 || (recvBuf && reinterpret_cast<uintptr_t>(recvBuf) % unit != 0)) {
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_REDUCESCATTER;
+    sig.count = 0;
+    sig.dtype = dataType;
+    sig.recvType = dataType;
+    sig.op = op;
+    sig.variable = 1;
+    return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr, counts,
+        static_cast<const uint64_t *>(sendDispls));
+}
+
+// op_base.cc:1863-1972.  sendCount must equal recvCounts[rank]; every rank passes the same table.
+HcclResult HcclAllGatherV(void *sendBuf, uint64_t sendCount, void *recvBuf, const void *recvCounts, const void *recvDispls,
+    HcclDataType dataType, HcclComm comm, aclrtStream stream)
+{
+    CHK_PTR(recvCounts);
+    CHK_PTR(recvDispls);
+    CHK_PTR(comm);
+    if (sendCount > 0) {
+        CHK_PTR(sendBuf);
+    }
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    HcclResult r = CheckOpParam("HcclAllGatherV", sendCount, dataType, stream);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    const uint64_t *counts = static_cast<const uint64_t *>(recvCounts);
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < c->group->p; i++) {
+        if (counts[i] > kSysMaxCount) {
+            HCCL_LOG_ERROR("HcclAllGatherV: recvCounts[%u] exceeds the maximum", i);
+            return HCCL_E_PARA;
+        }
+        total += counts[i];
+    }
+    if (total == 0) {
+        HCCL_LOG_WARN("HcclAllGatherV: nothing to gather");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(recvBuf);
+    if (counts[c->rank] != sendCount) {
+        HCCL_LOG_ERROR("HcclAllGatherV: sendCount %llu differs from recvCounts[rank] %llu", (unsigned long long)sendCount,
+            (unsigned long long)counts[c->rank]);
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_ALLGATHER;
+    sig.count = 0;
+    sig.dtype = dataType;
+    sig.recvType = dataType;
+    sig.op = 0;
+    sig.variable = 1;
+    return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr, counts,
+        static_cast<const uint64_t *>(recvDispls));
+}
+
+// op_base.cc:2422-2518: the uniform all-to-all is the pairwise schedule with equal blocks.
+HcclResult HcclAlltoAll(const void *sendBuf, uint64_t sendCount, HcclDataType sendType, const void *recvBuf,
+    uint64_t recvCount, HcclDataType recvType, HcclComm comm, aclrtStream stream)
+{
+    if (sendCount == 0 && recvCount == 0) {
+        HCCL_LOG_WARN("HcclAlltoAll: both counts are 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(sendBuf);
+    CHK_PTR(recvBuf);
+    if (sendCount != recvCount) {
+        HCCL_LOG_ERROR("HcclAlltoAll: sendCount and recvCount differ");
+        return HCCL_E_PARA;
+    }
+    if (sendType != recvType) {
+        HCCL_LOG_ERROR("HcclAlltoAll: sendType and recvType differ");
+        return HCCL_E_PARA;
+    }
+    CHK_PTR(stream);
+    CHK_PTR(comm);
+    if (sendBuf == recvBuf) {
+        HCCL_LOG_ERROR("HcclAlltoAll: sendBuf and recvBuf cannot be the same");
+        return HCCL_E_PARA;
+    }
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    HcclResult r = CheckOpParam("HcclAlltoAll", 0, sendType, stream);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if (sendCount > kSysMaxCount) {
+        return HCCL_E_PARA;
+    }
+    uint32_t p = c->group->p;
+    std::vector<uint64_t> counts(p, sendCount), displs(p);
+    for (uint32_t i = 0; i < p; i++) {
+        displs[i] = uint64_t(i) * sendCount;
+    }
+    OpSig sig;
+    sig.coll = COLL_ALLTOALLV;
+    sig.dtype = sendType;
+    sig.recvType = recvType;
+    return Arrive(c, sig, const_cast<void *>(sendBuf), const_cast<void *>(recvBuf), static_cast<hipStream_t>(stream),
+        counts.data(), displs.data(), counts.data(), displs.data());
+}
+
+// op_base.cc:1353-1431: an all-reduce (fp32 sum) of a few elements on buffers the group owns.
+HcclResult HcclBarrier(HcclComm comm, aclrtStream stream)
+{
+    CHK_PTR(comm);
+    CHK_PTR(stream);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    Group *g = c->group;
+    constexpr uint64_t kBarrierCount = 8;   // elements per rank; the value is never read back
+    constexpr uint64_t kSlot = 256;         // bytes between buffers
+    {
+        std::lock_guard<std::mutex> lock(g->m);
+        HcclResult r = EnsureDevice(g, false);
+        if (r != HCCL_SUCCESS) {
+            return r;
+        }
+        if (g->barrierMem == nullptr) {
+            if (hipMalloc(&g->barrierMem, 2 * kSlot * g->p) != hipSuccess ||
+                hipMemset(g->barrierMem, 0, 2 * kSlot * g->p) != hipSuccess) {
+                return HCCL_E_RUNTIME;
+            }
+        }
+    }
+    char *base = static_cast<char *>(g->barrierMem);
+    OpSig sig;
+    sig.coll = COLL_ALLREDUCE;
+    sig.count = kBarrierCount;
+    sig.dtype = HCCL_DATA_TYPE_FP32;
+    sig.recvType = HCCL_DATA_TYPE_FP32;
+    sig.op = HCCL_REDUCE_SUM;
+    return Arrive(c, sig, base + kSlot * (2 * c->rank), base + kSlot * (2 * c->rank + 1), static_cast<hipStream_t>(stream),
+        nullptr, nullptr, nullptr, nullptr);
+}
+
 // ---- extension ----------------------------------------------------------------------------------------
 
 HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
@@ -733,6 +939,10 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         rq.recvCounts.assign(tables + 2 * n, tables + 3 * n);
         rq.rdispls.assign(tables + 3 * n, tables + 4 * n);
     }
+    if ((coll == COLL_REDUCESCATTER || coll == COLL_ALLGATHER) && tables != nullptr) {
+        rq.vCounts.assign(tables, tables + nRanks);
+        rq.vDispls.assign(tables + nRanks, tables + 2 * size_t(nRanks));
+    }
     Plan plan;
     std::string err;
     int rc = BuildPlan(rq, &plan, &err);
@@ -827,29 +1037,6 @@ HcclResult HcclBatchSendRecv(HcclSendRecvItem *sendRecvInfo, uint32_t, HcclComm 
 {
     CHK_PTR(comm);
     CHK_PTR(sendRecvInfo);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclReduceScatterV(void *, const void *, const void *, void *, uint64_t, HcclDataType, HcclReduceOp,
-    HcclComm comm, aclrtStream)
-{
-    CHK_PTR(comm);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclAllGatherV(void *, uint64_t, void *, const void *, const void *, HcclDataType, HcclComm comm, aclrtStream)
-{
-    CHK_PTR(comm);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclAlltoAll(const void *, uint64_t, HcclDataType, const void *, uint64_t, HcclDataType, HcclComm comm,
-    aclrtStream)
-{
-    CHK_PTR(comm);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclBarrier(HcclComm comm, aclrtStream stream)
-{
-    CHK_PTR(comm);
-    CHK_PTR(stream);
     return HCCL_E_NOT_SUPPORT;
 }
 HcclResult HcclCommSetMemoryRange(HcclComm comm, void *, size_t, size_t, uint64_t)

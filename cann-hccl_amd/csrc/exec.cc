@@ -338,6 +338,11 @@ std::string CacheKey(const Group *g, int algo)
     // raw bytes of everything the prepared tables depend on
     std::string key;
     auto put = [&](const void *p, size_t n) { key.append(static_cast<const char *>(p), n); };
+    if (g->sig.variable) {
+        put(g->vCounts.data(), g->vCounts.size() * 8);
+        put(g->vDispls.data(), g->vDispls.size() * 8);
+        key.push_back('v');
+    }
     uint64_t head[10] = {uint64_t(g->sig.coll), uint64_t(algo), uint64_t(g->sig.dtype), uint64_t(g->sig.op), g->sig.count,
         uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1), g->cfg.cclBytes, g->cfg.align, g->cfg.blocksPerCu, g->p};
     put(head, sizeof(head));
@@ -367,6 +372,10 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
     rq.alias.assign(g->p, 0);
     for (uint32_t r = 0; r < g->p; r++) {
         rq.alias[r] = (g->send[r] == g->recv[r]) ? 1 : 0;
+    }
+    if (g->sig.variable) {
+        rq.vCounts = g->vCounts;
+        rq.vDispls = g->vDispls;
     }
     if (rq.coll == COLL_ALLTOALLV) {
         rq.sendCounts = g->sendCounts;
@@ -483,6 +492,9 @@ Group::~Group()
             (void)hipFree(s);
         }
     }
+    if (barrierMem) {
+        (void)hipFree(barrierMem);
+    }
 }
 
 const char *CollName(int coll)
@@ -507,7 +519,7 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     int algo = g->cfg.algo >= 0 ? g->cfg.algo : DefaultAlgo(g->sig.coll);
     if (g->sig.coll == COLL_ALLTOALLV) {
         algo = ALGO_PAIRWISE;
-    } else if (algo == ALGO_PAIRWISE || (algo == ALGO_RHD && g->sig.coll != COLL_ALLREDUCE)) {
+    } else if (algo == ALGO_PAIRWISE) {
         algo = ALGO_RING;
     }
     std::string key = CacheKey(g, algo);

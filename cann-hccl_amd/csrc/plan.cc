@@ -214,6 +214,112 @@ void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t
     }
 }
 
+// Halving-doubling shape shared by the standalone reduce-scatter / all-gather variants: block rank b
+// below part1/2 stands for the rank pair (2b, 2b+1) and owns both their slices, the others own one.
+struct HdShape {
+    uint32_t block = 1, part1 = 0, steps = 0;
+    std::vector<uint32_t> rankOf;                  // block rank -> real rank
+    std::vector<std::vector<uint32_t>> owned;      // block rank -> user slices it ends up with
+};
+
+HdShape MakeHdShape(uint32_t p)
+{
+    HdShape h;
+    HalvingDoublingShape(p, &h.block, &h.part1);
+    h.rankOf.assign(h.block, 0);
+    h.owned.assign(h.block, {});
+    for (uint32_t i = 0; i < p; i++) {
+        if (i < h.part1 && (i & 1)) {
+            continue;
+        }
+        h.rankOf[i < h.part1 ? i / 2 : i - h.part1 / 2] = i;
+    }
+    for (uint32_t b = 0; b < h.block; b++) {
+        if (2 * b < h.part1) {
+            h.owned[b] = {2 * b, 2 * b + 1};
+        } else {
+            h.owned[b] = {b + h.part1 / 2};
+        }
+    }
+    while ((1u << h.steps) < h.block) {
+        h.steps++;
+    }
+    return h;
+}
+
+// Standalone recursive halving-doubling reduce-scatter (reduce_scatter_recursive_hd.cc:33-254) over
+// user slices in[i]; every rank ends with its reduced slice in (BUF_RECV, outOff).
+void RhdReduceScatterChunk(VProgram &vp, uint32_t p, const std::vector<Slice> &in, uint64_t outOff)
+{
+    HdShape h = MakeHdShape(p);
+    size_t ph = 0;
+    if (h.part1 > 0) {
+        for (uint32_t e = 0; e < h.part1; e += 2) {
+            for (uint32_t i = 0; i < p; i++) {
+                EmitReduce(vp, ph, MkRef(e, BUF_SEND, in[i].off), MkRef(e, BUF_SEND, in[i].off), MkRef(e + 1, BUF_SEND, in[i].off),
+                    in[i].size);
+            }
+        }
+        ph++;
+    }
+    for (uint32_t s = 0; s < h.steps; s++) {
+        uint32_t mask = 1u << (h.steps - s - 1);
+        for (uint32_t q = 0; q < h.block; q++) {
+            uint32_t first = q & ~(mask - 1);
+            for (uint32_t b = first; b < first + mask; b++) {
+                for (uint32_t u : h.owned[b]) {
+                    EmitReduce(vp, ph, MkRef(h.rankOf[q], BUF_SEND, in[u].off), MkRef(h.rankOf[q], BUF_SEND, in[u].off),
+                        MkRef(h.rankOf[q ^ mask], BUF_SEND, in[u].off), in[u].size);
+                }
+            }
+        }
+        ph++;
+    }
+    if (h.part1 > 0) {   // the even rank of a pair hands the odd rank its slice
+        for (uint32_t e = 0; e < h.part1; e += 2) {
+            EmitCopy(vp, ph, MkRef(e + 1, BUF_SEND, in[e + 1].off), MkRef(e, BUF_SEND, in[e + 1].off), in[e + 1].size);
+        }
+        ph++;
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        EmitCopy(vp, ph, MkRef(r, BUF_RECV, outOff), MkRef(r, BUF_SEND, in[r].off), in[r].size);
+    }
+}
+
+// Standalone recursive halving-doubling all-gather (all_gather_recursive_hd.cc:26-238) on the output
+// buffer; phase0 is the first phase after the ranks copied their own block in.
+void RhdAllGatherChunk(VProgram &vp, size_t phase0, uint32_t p, const std::vector<Slice> &sl)
+{
+    HdShape h = MakeHdShape(p);
+    size_t ph = phase0;
+    if (h.part1 > 0) {
+        for (uint32_t e = 0; e < h.part1; e += 2) {
+            EmitCopy(vp, ph, MkRef(e, BUF_RECV, sl[e + 1].off), MkRef(e + 1, BUF_RECV, sl[e + 1].off), sl[e + 1].size);
+        }
+        ph++;
+    }
+    for (uint32_t s = 0; s < h.steps; s++) {
+        uint32_t mask = 1u << s;
+        for (uint32_t q = 0; q < h.block; q++) {
+            uint32_t peer = q ^ mask;
+            uint32_t first = peer & ~(mask - 1);
+            for (uint32_t b = first; b < first + mask; b++) {
+                for (uint32_t u : h.owned[b]) {
+                    EmitCopy(vp, ph, MkRef(h.rankOf[q], BUF_RECV, sl[u].off), MkRef(h.rankOf[peer], BUF_RECV, sl[u].off), sl[u].size);
+                }
+            }
+        }
+        ph++;
+    }
+    if (h.part1 > 0) {
+        for (uint32_t e = 0; e < h.part1; e += 2) {
+            for (uint32_t i = 0; i < p; i++) {
+                EmitCopy(vp, ph, MkRef(e + 1, BUF_RECV, sl[i].off), MkRef(e, BUF_RECV, sl[i].off), sl[i].size);
+            }
+        }
+    }
+}
+
 int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
 {
     uint32_t p = rq.p;
@@ -241,9 +347,65 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
         }
         return 0;
     }
-    if (rq.algo == ALGO_PAIRWISE || (rq.algo == ALGO_RHD && rq.coll != COLL_ALLREDUCE)) {
+    if (rq.algo == ALGO_PAIRWISE) {
         *err = "algorithm not available for this collective";
         return 1;
+    }
+    if (!rq.vCounts.empty()) {
+        // variable block sizes: the same schedules over explicit slices, one pass (the slice a rank
+        // ends up with is the same whatever the chunking, so no chunk loop is needed)
+        if (rq.vCounts.size() != p || rq.vDispls.size() != p || rq.coll == COLL_ALLREDUCE) {
+            *err = "variable-count tables must have p entries";
+            return 1;
+        }
+        std::vector<Slice> sl(p);
+        uint64_t extent = 0;
+        for (uint32_t i = 0; i < p; i++) {
+            sl[i] = Slice{rq.vDispls[i] * u, rq.vCounts[i] * u};
+            if (sl[i].size) {
+                extent = std::max(extent, sl[i].off + sl[i].size);
+            }
+        }
+        if (rq.coll == COLL_REDUCESCATTER) {
+            std::vector<Slice> out(p);
+            for (uint32_t i = 0; i < p; i++) {
+                out[i] = Slice{0, sl[i].size};
+            }
+            if (p == 1) {
+                EmitCopy(*vp, 0, MkRef(0, BUF_RECV, 0), MkRef(0, BUF_SEND, sl[0].off), sl[0].size);
+            } else if (rq.algo == ALGO_RING) {
+                RingReduceScatterPhases(*vp, 0, p, 0, sl, BUF_RECV, 0, out);
+            } else if (rq.algo == ALGO_RHD) {
+                RhdReduceScatterChunk(*vp, p, sl, 0);
+            } else {
+                size_t ph = MeshReduceScatterPhases(*vp, 0, p, 0, sl, rq.align);
+                for (uint32_t r = 0; r < p; r++) {
+                    EmitCopy(*vp, ph, MkRef(r, BUF_RECV, 0), MkRef(r, BUF_SEND, sl[r].off), sl[r].size);
+                }
+            }
+            for (uint32_t r = 0; r < p; r++) {
+                vp->inBytes[r] = extent;
+                vp->outBytes[r] = sl[r].size;
+            }
+        } else {
+            for (uint32_t r = 0; r < p; r++) {
+                EmitCopy(*vp, 0, MkRef(r, BUF_RECV, sl[r].off), MkRef(r, BUF_SEND, 0), sl[r].size);
+            }
+            if (p > 1) {
+                if (rq.algo == ALGO_RING) {
+                    RingAllGatherPhases(*vp, 1, p, 0, sl);
+                } else if (rq.algo == ALGO_RHD) {
+                    RhdAllGatherChunk(*vp, 1, p, sl);
+                } else {
+                    MeshAllGatherPhases(*vp, 1, p, 0, sl);
+                }
+            }
+            for (uint32_t r = 0; r < p; r++) {
+                vp->inBytes[r] = sl[r].size;
+                vp->outBytes[r] = extent;
+            }
+        }
+        return 0;
     }
     std::vector<uint64_t> chunks = ChunkCounts(rq.coll, rq.count, rq.unit, p, rq.cclBytes, rq.align);
     if (rq.count > 0 && chunks.empty()) {
@@ -267,6 +429,8 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                 EmitCopy(*vp, 0, MkRef(0, BUF_RECV, done), MkRef(0, BUF_SEND, done), bytes);
             } else if (rq.algo == ALGO_RING) {
                 RingReduceScatterPhases(*vp, 0, p, 0, in, BUF_RECV, 0, out);
+            } else if (rq.algo == ALGO_RHD) {
+                RhdReduceScatterChunk(*vp, p, in, done);
             } else {
                 size_t ph = MeshReduceScatterPhases(*vp, 0, p, 0, in, rq.align);
                 for (uint32_t r = 0; r < p; r++) {
@@ -284,6 +448,8 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             if (p > 1) {
                 if (rq.algo == ALGO_RING) {
                     RingAllGatherPhases(*vp, 1, p, 0, sl);
+                } else if (rq.algo == ALGO_RHD) {
+                    RhdAllGatherChunk(*vp, 1, p, sl);
                 } else {
                     MeshAllGatherPhases(*vp, 1, p, 0, sl);
                 }

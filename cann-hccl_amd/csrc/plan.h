@@ -74,6 +74,9 @@ struct PlanRequest {
     bool stageInput = false;       // copy the send buffers to scratch first (used when buffers overlap)
     // all-to-all-v only: p x p tables in elements, row r = what rank r passed
     std::vector<uint64_t> sendCounts, sdispls, recvCounts, rdispls;
+    // reduce-scatter-v / all-gather-v: per-rank block counts and displacements in elements (p entries
+    // each, the same on every rank).  Empty = the uniform collective described by `count`.
+    std::vector<uint64_t> vCounts, vDispls;
 };
 
 struct Plan {

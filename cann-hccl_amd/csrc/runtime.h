@@ -77,9 +77,11 @@ struct OpSig {
     int coll = -1;
     uint64_t count = 0;
     int dtype = 0, recvType = 0, op = 0;
+    int variable = 0;                // 1: reduce-scatter-v / all-gather-v (block tables instead of a count)
     bool operator==(const OpSig &o) const
     {
-        return coll == o.coll && count == o.count && dtype == o.dtype && recvType == o.recvType && op == o.op;
+        return coll == o.coll && count == o.count && dtype == o.dtype && recvType == o.recvType && op == o.op &&
+            variable == o.variable;
     }
 };
 
@@ -112,6 +114,7 @@ struct Group {
     std::vector<void *> send, recv;
     std::vector<hipStream_t> streams;
     std::vector<uint64_t> sendCounts, sdispls, recvCounts, rdispls;   // p x p (all-to-all-v)
+    std::vector<uint64_t> vCounts, vDispls;                           // p (reduce-scatter-v / all-gather-v)
 
     // device resources
     bool deviceReady = false;
@@ -120,6 +123,7 @@ struct Group {
     std::vector<hipEvent_t> arriveEvents;
     hipEvent_t doneEvent = nullptr;
     std::vector<void *> scratch;
+    void *barrierMem = nullptr;       // 2 x p small buffers for HcclBarrier's all-reduce
     uint64_t scratchBytes = 0;
     uint64_t scratchGen = 0;
     std::unordered_map<std::string, std::unique_ptr<Prepared>> cache;

@@ -41,7 +41,8 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
 /* Plans a collective without a device and writes the plan as JSON (phases of copy / reduce steps,
  * fused items, byte counts) into out[0..cap).  coll / algo as in HcclAmdOpInfo.  inPlaceMask bit r:
  * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64
- * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); else NULL.
+ * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); for the variable-count
+ * reduce-scatter / all-gather, tables points to 2*p uint64 (block counts, block displacements); else NULL.
  * Returns HCCL_E_MEMORY and the needed size in *needed when cap is too small. */
 extern HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint64_t count, HcclDataType dataType,
     uint64_t cclBytes, uint64_t align, uint64_t inPlaceMask, const uint64_t *tables, char *out, size_t cap, size_t *needed);

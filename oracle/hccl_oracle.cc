@@ -16,6 +16,7 @@
 //   mesh             TPL/temp_reduce_scatter/reduce_scatter_mesh.cc:57-203, TPL/temp_all_gather/all_gather_mesh.cc:91-253,
 //                    EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240, EXE/coll_comm_executor.cc:1458-1574
 //   halving-doubling TPL/temp_all_reduce/all_reduce_recursive_hd.cc:33-302,
+//                    TPL/temp_reduce_scatter/reduce_scatter_recursive_hd.cc:33-254, TPL/temp_all_gather/all_gather_recursive_hd.cc:26-238,
 //                    TPL/temp_reduce_scatter/reduce_scatter_halving_doubling.cc:67-238,
 //                    TPL/temp_all_gather/all_gather_halving_doubling.cc:43-196
 //   pairwise         TPL/temp_alltoallv/alltoallv_pairwise.cc:75-282, ALG/impl/operator/alltoall_operator.cc:49-72
@@ -805,6 +806,31 @@ int RunAllReduceRhd(Machine &m, uint64_t bytes, uint64_t align)
     return rc;
 }
 
+// Block-rank map and block slices of the standalone recursive halving-doubling reduce-scatter /
+// all-gather: block ranks below part1/2 own two consecutive rank slices
+// (reduce_scatter_recursive_hd.cc:86-110, all_gather_recursive_hd.cc:69-90).
+void RhdBlockLayout(uint32_t p, uint64_t bytes, uint32_t *block, uint32_t *part1, std::vector<uint32_t> *rankOf,
+    std::vector<Slice> *blockSlices)
+{
+    RhdParams(p, block, part1);
+    rankOf->assign(*block, 0);
+    for (uint32_t i = 0; i < p; i++) {
+        if (i < *part1 && (i % 2) == 1) {
+            continue;
+        }
+        (*rankOf)[(i < *part1) ? i / 2 : i - *part1 / 2] = i;
+    }
+    blockSlices->assign(*block, Slice{0, 0});
+    uint32_t half = *part1 / 2;
+    for (uint32_t b = 0; b < *block; b++) {
+        if (b < half) {
+            (*blockSlices)[b] = Slice{uint64_t(b) * 2 * bytes, 2 * bytes};
+        } else {
+            (*blockSlices)[b] = Slice{uint64_t(b) * bytes + uint64_t(half) * bytes, bytes};
+        }
+    }
+}
+
 int RunAllReduceTemplate(Machine &m, int algo, uint64_t bytes, uint64_t align)
 {
     switch (algo) {
@@ -1010,6 +1036,30 @@ int orc_reducescatter(int algo, uint32_t p, void **in, void **out, uint64_t recv
                         m.procs.push_back(std::move(pr));
                     }
                 }
+            } else if (algo == ALGO_RHD) {
+                // ReduceScatterRecursiveHalvingDoubling::RunAsync, reduce_scatter_recursive_hd.cc:33-254
+                uint32_t block, part1;
+                std::vector<uint32_t> rankOf;
+                std::vector<Slice> bsl;
+                RhdBlockLayout(p, bytes, &block, &part1, &rankOf, &bsl);
+                for (uint32_t r = 0; r < p; r++) {
+                    Proc pr;
+                    pr.rank = r;
+                    if (r < part1 && (r % 2) == 1) {
+                        pr.prog.push_back(MkSend(static_cast<int>(r - 1), 1, B_IN, 0, bytes * p));
+                        pr.prog.push_back(MkRecvCopy(static_cast<int>(r - 1), 1, B_IN, bytes * r, bytes));
+                    } else {
+                        if (r < part1) {
+                            pr.prog.push_back(MkRecvReduce(static_cast<int>(r + 1), 1, B_IN, 0, B_IN, 0, bytes * p));
+                        }
+                        uint32_t q = (r < part1) ? r / 2 : r - part1 / 2;
+                        ProgReduceScatterHd(pr.prog, q, block, rankOf, B_IN, B_IN, bsl);
+                        if (r < part1) {
+                            pr.prog.push_back(MkSend(static_cast<int>(r + 1), 1, B_IN, bytes * (r + 1), bytes));
+                        }
+                    }
+                    m.procs.push_back(std::move(pr));
+                }
             } else {
                 return -10;
             }
@@ -1075,6 +1125,26 @@ int orc_allgather(int algo, uint32_t p, void **in, void **out, uint64_t sendCoun
             } else if (algo == ALGO_MESH) {
                 pr.prog.push_back(MkLocalCopy(B_OUT, outSl[r].off, B_IN, inSl[r].off, bytes));
                 ProgAllGatherMesh(pr.prog, r, p, B_OUT, outSl);
+            } else if (algo == ALGO_RHD) {
+                // AllGatherRecursiveHalvingDoubling::RunAsync, all_gather_recursive_hd.cc:26-238
+                uint32_t block, part1;
+                std::vector<uint32_t> rankOf;
+                std::vector<Slice> bsl;
+                RhdBlockLayout(p, bytes, &block, &part1, &rankOf, &bsl);
+                pr.prog.push_back(MkLocalCopy(B_OUT, outSl[r].off, B_IN, inSl[r].off, bytes));
+                if (r < part1 && (r % 2) == 1) {
+                    pr.prog.push_back(MkSend(static_cast<int>(r - 1), 1, B_OUT, bytes * r, bytes));
+                    pr.prog.push_back(MkRecvCopy(static_cast<int>(r - 1), 1, B_OUT, 0, bytes * p));
+                } else {
+                    if (r < part1) {
+                        pr.prog.push_back(MkRecvCopy(static_cast<int>(r + 1), 1, B_OUT, bytes * (r + 1), bytes));
+                    }
+                    uint32_t q = (r < part1) ? r / 2 : r - part1 / 2;
+                    ProgAllGatherHd(pr.prog, q, block, rankOf, B_OUT, bsl);
+                    if (r < part1) {
+                        pr.prog.push_back(MkSend(static_cast<int>(r + 1), 1, B_OUT, 0, bytes * p));
+                    }
+                }
             } else {
                 return -10;
             }
@@ -1093,6 +1163,118 @@ int orc_allgather(int algo, uint32_t p, void **in, void **out, uint64_t sendCoun
         left -= cur;
     }
     return 0;
+}
+
+// Variable-count reduce-scatter: every rank's `in` holds the blocks {displs[i], counts[i]} (elements);
+// rank r receives the reduction of block r.  The templates run over these explicit slices
+// (reduce_scatter_ring.cc:179-297 takes any slice list; mesh and halving-doubling likewise).
+int orc_reducescatter_v(int algo, uint32_t p, void **in, void **out, const uint64_t *counts, const uint64_t *displs,
+    int dt, int op, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0) {
+        return -20;
+    }
+    std::vector<Slice> sl(p);
+    uint64_t extent = 0;
+    for (uint32_t i = 0; i < p; i++) {
+        sl[i] = Slice{displs[i] * unit, counts[i] * unit};
+        if (sl[i].size) {
+            extent = std::max(extent, sl[i].off + sl[i].size);
+        }
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.op = op;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    std::vector<std::vector<uint8_t>> work(p, std::vector<uint8_t>(extent));
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_IN][r] = work[r].data();
+        m.buf[B_OUT][r] = static_cast<uint8_t *>(out[r]);
+        m.Copy(work[r].data(), static_cast<uint8_t *>(in[r]), extent);
+    }
+    if (p > 1) {
+        if (algo == ALGO_RING) {
+            for (uint32_t r = 0; r < p; r++) {
+                Proc pr;
+                pr.rank = r;
+                ProgReduceScatterRing(pr.prog, r, p, B_IN, B_IN, sl, sl);
+                m.procs.push_back(std::move(pr));
+            }
+        } else if (algo == ALGO_MESH) {
+            uint32_t nstream = p > 2 ? p - 1 : 1;
+            std::vector<std::vector<Slice>> pieces = CutPieces(sl, nstream, align);
+            for (uint32_t t = 0; t < nstream; t++) {
+                for (uint32_t r = 0; r < p; r++) {
+                    Proc pr;
+                    pr.rank = r;
+                    ProgReduceScatterMeshStream(pr.prog, r, p, t, B_IN, pieces[t]);
+                    m.procs.push_back(std::move(pr));
+                }
+            }
+        } else {
+            return -10;
+        }
+        int rc = m.Run();
+        if (rc != 0) {
+            return rc;
+        }
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        m.Copy(static_cast<uint8_t *>(out[r]), work[r].data() + sl[r].off, sl[r].size);
+    }
+    return 0;
+}
+
+// Variable-count all-gather: rank r contributes counts[r] elements, every rank's `out` receives block i
+// at displs[i].
+int orc_allgather_v(int algo, uint32_t p, void **in, void **out, const uint64_t *counts, const uint64_t *displs, int dt,
+    int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0) {
+        return -20;
+    }
+    std::vector<Slice> sl(p), inSl(p);
+    for (uint32_t i = 0; i < p; i++) {
+        sl[i] = Slice{displs[i] * unit, counts[i] * unit};
+        inSl[i] = Slice{0, counts[i] * unit};
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_IN][r] = static_cast<uint8_t *>(in[r]);
+        m.buf[B_OUT][r] = static_cast<uint8_t *>(out[r]);
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        if (algo == ALGO_RING || p == 1) {
+            if (p == 1) {
+                pr.prog.push_back(MkLocalCopy(B_OUT, sl[0].off, B_IN, 0, sl[0].size));
+            } else {
+                ProgAllGatherRing(pr.prog, r, p, B_IN, B_OUT, sl, inSl);
+            }
+        } else if (algo == ALGO_MESH) {
+            pr.prog.push_back(MkLocalCopy(B_OUT, sl[r].off, B_IN, 0, sl[r].size));
+            ProgAllGatherMesh(pr.prog, r, p, B_OUT, sl);
+        } else {
+            return -10;
+        }
+        m.procs.push_back(std::move(pr));
+    }
+    return m.Run();
 }
 
 // PairWise all-to-all-v.  counts / displs are p x p row-major tables in elements: row r is what

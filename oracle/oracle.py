@@ -59,6 +59,8 @@ def lib():
         L.orc_allreduce.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64, i32, i32, pu64]
         L.orc_reducescatter.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64, i32, i32]
         L.orc_allgather.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, u64, u64, i32, i32]
+        L.orc_reducescatter_v.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), pu64, pu64, i32, i32, u64, i32, i32]
+        L.orc_allgather_v.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), pu64, pu64, i32, i32, i32]
         L.orc_alltoallv.argtypes = [u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, u64, i32, i32]
         L.orc_fill_uniform_f32.argtypes = [vp, u64, u64, u32, i32]
         _lib = L
@@ -186,6 +188,31 @@ def allgather(ins, dt, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALI
     rc = lib().orc_allgather(algo, p, _ptrs(ins), _ptrs(outs), n, dt, ccl_bytes, align, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle allgather failed rc=%d" % rc)
+    return outs
+
+
+def reducescatter_v(ins, counts, displs, dt, op, algo=RING, align=DEFAULT_ALIGN, flags=0, threads=1):
+    """ins: p arrays holding the blocks {displs[i], counts[i]}; returns p arrays, rank r gets block r reduced."""
+    p = len(ins)
+    c, d = _u64arr(p), _u64arr(p)
+    c[:] = [int(x) for x in counts]
+    d[:] = [int(x) for x in displs]
+    outs = [np.empty(int(counts[r]), dtype=ins[0].dtype) for r in range(p)]
+    rc = lib().orc_reducescatter_v(algo, p, _ptrs(ins), _ptrs(outs), c, d, dt, op, align, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle reducescatter_v failed rc=%d" % rc)
+    return outs
+
+
+def allgather_v(ins, counts, displs, out_len, dt, algo=RING, flags=0, threads=1, fill=0):
+    p = len(ins)
+    c, d = _u64arr(p), _u64arr(p)
+    c[:] = [int(x) for x in counts]
+    d[:] = [int(x) for x in displs]
+    outs = [np.full(out_len, fill, dtype=ins[0].dtype) for _ in range(p)]
+    rc = lib().orc_allgather_v(algo, p, _ptrs(ins), _ptrs(outs), c, d, dt, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle allgather_v failed rc=%d" % rc)
     return outs
 
 

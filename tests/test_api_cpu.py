@@ -113,6 +113,39 @@ def test_alltoallv_checks(comms):
     assert L.HcclAlltoAllV(None, zeros, zeros, I32, None, zeros, zeros, I32, c, STREAM) == H.HCCL_SUCCESS
 
 
+def test_sibling_entry_checks(comms):
+    c = comms[0]
+    I32, SUM = H.HCCL_DATA_TYPE_INT32, H.HCCL_REDUCE_SUM
+    ones = (ctypes.c_uint64 * 4)(1, 1, 1, 1)
+    zeros = (ctypes.c_uint64 * 4)(0, 0, 0, 0)
+    # HcclAlltoAll (op_base.cc:2422): both counts 0 -> success first; then buffers, equal counts / types, stream, comm
+    assert L.HcclAlltoAll(None, 0, I32, None, 0, I32, None, None) == H.HCCL_SUCCESS
+    assert L.HcclAlltoAll(None, 4, I32, BUF_B, 4, I32, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAlltoAll(BUF_A, 4, I32, BUF_B, 8, I32, c, STREAM) == H.HCCL_E_PARA
+    assert L.HcclAlltoAll(BUF_A, 4, I32, BUF_B, 4, H.HCCL_DATA_TYPE_FP32, c, STREAM) == H.HCCL_E_PARA
+    assert L.HcclAlltoAll(BUF_A, 4, I32, BUF_B, 4, I32, c, None) == H.HCCL_E_PTR
+    assert L.HcclAlltoAll(BUF_A, 4, I32, BUF_A, 4, I32, c, STREAM) == H.HCCL_E_PARA
+    # HcclReduceScatterV (op_base.cc:1585)
+    assert L.HcclReduceScatterV(BUF_A, None, ones, BUF_B, 1, I32, SUM, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclReduceScatterV(BUF_A, ones, ones, None, 1, I32, SUM, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclReduceScatterV(BUF_A, zeros, zeros, None, 0, I32, SUM, c, STREAM) == H.HCCL_SUCCESS   # nothing to reduce
+    assert L.HcclReduceScatterV(None, ones, ones, BUF_B, 1, I32, SUM, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclReduceScatterV(BUF_A, ones, ones, BUF_B, 2, I32, SUM, c, STREAM) == H.HCCL_E_PARA       # recvCount != sendCounts[rank]
+    assert L.HcclReduceScatterV(BUF_A, ones, ones, BUF_B, 1, I32, 9, c, STREAM) == H.HCCL_E_NOT_SUPPORT
+    # HcclAllGatherV (op_base.cc:1863)
+    assert L.HcclAllGatherV(BUF_A, 1, BUF_B, None, ones, I32, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAllGatherV(None, 1, BUF_B, ones, ones, I32, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAllGatherV(None, 0, None, zeros, zeros, I32, c, STREAM) == H.HCCL_SUCCESS
+    assert L.HcclAllGatherV(BUF_A, 2, BUF_B, ones, ones, I32, c, STREAM) == H.HCCL_E_PARA
+    # HcclBarrier (op_base.cc:1353)
+    assert L.HcclBarrier(None, STREAM) == H.HCCL_E_PTR
+    assert L.HcclBarrier(c, None) == H.HCCL_E_PTR
+    # ranks that pass different block tables do not form a collective
+    twos = (ctypes.c_uint64 * 4)(2, 1, 1, 1)
+    assert L.HcclReduceScatterV(BUF_A, ones, ones, BUF_B, 1, I32, SUM, comms[1], STREAM) == H.HCCL_SUCCESS
+    assert L.HcclReduceScatterV(BUF_A, twos, ones, BUF_B, 1, I32, SUM, comms[2], STREAM) == H.HCCL_E_PARA
+
+
 def test_mismatched_ranks_are_rejected(comms):
     FP32, SUM = H.HCCL_DATA_TYPE_FP32, H.HCCL_REDUCE_SUM
     assert L.HcclAllReduce(BUF_A, BUF_B, 8, FP32, SUM, comms[0], STREAM) == H.HCCL_SUCCESS

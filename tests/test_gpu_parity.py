@@ -172,9 +172,9 @@ def test_streams_of_other_ranks_are_ordered(orc):
         g.close()
 
 
-@pytest.mark.parametrize("algo", [RING, MESH])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
 def test_reducescatter_op_type_matrix(orc, algo):
-    p = 8
+    p = 8 if algo != RHD else 6
     for fuse in (1, 0):
         g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
         try:
@@ -209,9 +209,9 @@ def test_reducescatter_64mib_per_rank_int_and_bf16(orc):
         g.close()
 
 
-@pytest.mark.parametrize("algo", [RING, MESH])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
 def test_allgather(orc, algo):
-    for p in (1, 2, 5, 8, 16):
+    for p in (1, 2, 5, 8, 12):
         for fuse in (1, 0):
             g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
             try:
@@ -335,5 +335,107 @@ def test_special_values_follow_the_selection_rule(orc):
                         assert np.array_equal(np.isnan(outs[r]), np.isnan(want[r]))
                         if op in (MAX, MIN):
                             assert np.array_equal(outs[r].view(np.uint32), want[r].view(np.uint32))   # incl. sign of zero, NaN bits
+            finally:
+                g.close()
+
+
+def _v_case(p, seed, scale):
+    rng = np.random.default_rng(seed)
+    counts = rng.integers(0, scale, p)
+    counts[rng.random(p) < 0.2] = 0
+    displs, pos = np.zeros(p, np.int64), 0
+    for i in rng.permutation(p):
+        pos += int(rng.integers(0, 9))
+        displs[i] = pos
+        pos += int(counts[i])
+    return counts, displs, pos + 3
+
+
+@pytest.mark.parametrize("algo", [RING, MESH])
+def test_reducescatter_v(orc, algo):
+    for p in (1, 3, 8):
+        for fuse in (1, 0):
+            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+            try:
+                for dt, op, scale in ((FP32, SUM, 50000), (BF16, SUM, 3000), (INT8, MIN, 70000)):
+                    counts, displs, extent = _v_case(p, p + dt, scale)
+                    ins = _ins(dt, p, extent, 3 * p + dt)
+                    want = orc.reducescatter_v(ins, counts, displs, dt, op, algo=algo)
+                    sends = [gh.to_dev(x) for x in ins]
+                    recvs = [gh.empty_dev(max(int(counts[r]), 1) * H.DTYPE_SIZE[dt]) for r in range(p)]
+                    torch.cuda.synchronize()
+                    print("reducescatter_v", ALGO_NAME[algo], "p", p, "fuse", fuse, "type", dt, flush=True)
+                    H.reduce_scatter_v(g.comms, [t.data_ptr() for t in sends], counts, displs, [t.data_ptr() for t in recvs],
+                                       dt, op, g.stream_ptr)
+                    g.stream.synchronize()
+                    for r in range(p):
+                        got = gh.to_host(recvs[r], dt)[:int(counts[r])]
+                        assert gh.same(dt, got, want[r]), (algo, p, fuse, dt, r)
+            finally:
+                g.close()
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+def test_allgather_v(orc, algo):
+    for p in (1, 3, 6, 8):
+        for fuse in (1, 0):
+            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+            try:
+                counts, displs, extent = _v_case(p, 7 * p, 40000)
+                ins = [np.arange(int(counts[r]), dtype=np.int32) + (r << 20) for r in range(p)]
+                want = np.full(extent, -1, np.int32)
+                for r in range(p):
+                    want[displs[r]:displs[r] + counts[r]] = ins[r]
+                sends = [gh.to_dev(x if x.size else np.zeros(1, np.int32)) for x in ins]
+                recvs = [gh.to_dev(np.full(extent, -1, np.int32)) for _ in range(p)]
+                torch.cuda.synchronize()
+                print("allgather_v", ALGO_NAME[algo], "p", p, "fuse", fuse, flush=True)
+                H.all_gather_v(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], counts, displs, INT32,
+                               g.stream_ptr)
+                g.stream.synchronize()
+                for r in range(p):
+                    assert np.array_equal(gh.to_host(recvs[r], INT32), want), (algo, p, fuse, r)
+            finally:
+                g.close()
+
+
+def test_alltoall_uniform_and_barrier(orc):
+    for p in (1, 4, 8):
+        g = gh.Group(p)
+        try:
+            n = 4099
+            sends_np = [(np.arange(n * p, dtype=np.int32) + (r << 24)) for r in range(p)]
+            sends = [gh.to_dev(x) for x in sends_np]
+            recvs = [gh.to_dev(np.full(n * p, -1, np.int32)) for _ in range(p)]
+            torch.cuda.synchronize()
+            H.all_to_all(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, INT32, g.stream_ptr)
+            H.barrier(g.comms, g.stream_ptr)
+            H.barrier(g.comms, g.stream_ptr)
+            g.stream.synchronize()
+            for j in range(p):
+                want = np.concatenate([sends_np[i][j * n:(j + 1) * n] for i in range(p)])
+                assert np.array_equal(gh.to_host(recvs[j], INT32), want), (p, j)
+        finally:
+            g.close()
+
+
+def test_special_values_16bit(orc):
+    # bf16 / fp16 specials through the hardware conversions: infinities, overflow to infinity, denormals, ties
+    p = 4
+    rng = np.random.default_rng(11)
+    bf = np.array([0x0000, 0x8000, 0x7f80, 0xff80, 0x7f7f, 0xff7f, 0x0001, 0x8001, 0x007f, 0x3f80, 0xbf80, 0x3f81, 0x4000,
+                   0x7f00, 0x0080, 0x3b80], np.uint16)
+    hf = np.array([0x0000, 0x8000, 0x7c00, 0xfc00, 0x7bff, 0xfbff, 0x0001, 0x8001, 0x03ff, 0x3c00, 0xbc00, 0x3c01, 0x4000,
+                   0x7800, 0x0400, 0x1400], np.uint16)
+    for dt, table in ((BF16, bf), (FP16, hf)):
+        ins = [rng.choice(table, 8192).astype(np.uint16) for _ in range(p)]
+        for fuse in (1, 0):
+            g = gh.Group(p, fuse=fuse, align=2)
+            try:
+                for op in OPS:
+                    want = orc.allreduce(ins, dt, op, align=2)
+                    outs, _ = gh.all_reduce(g, ins, dt, op)
+                    for r in range(p):
+                        assert gh.same(dt, outs[r], want[r]), (dt, fuse, op, r)
             finally:
                 g.close()

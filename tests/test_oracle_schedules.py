@@ -172,6 +172,33 @@ def test_zero_staging_byte_count_matches_formula(orc):
     assert touched == (5 * p - 3) * n * 4
 
 
+def test_reducescatter_rhd_matches_tree(orc):
+    # standalone recursive halving-doubling reduce-scatter: rank r's block is the halving tree of the
+    # block rank that owns it (a pair of ranks shares one block rank in the fold part)
+    for dt in (FP32, BF16, INT32):
+        for p in (1, 2, 3, 5, 6, 8, 12, 24):
+            n = 211
+            for op in (SUM, MAX):
+                ins = _inputs(dt, p, n * p, 3 * p + op)
+                for ccl in (200 << 20, 128 * p * 2):
+                    got = orc.reducescatter(ins, dt, op, algo=RHD, ccl_bytes=ccl)
+                    block, part1 = cf.rhd_params(p)
+                    for r in range(p):
+                        xs = [x[r * n:(r + 1) * n] for x in ins]
+                        q = r // 2 if r < part1 else r - part1 // 2
+                        want = xs[0] if p == 1 else cf.rhd_tree(dt, op, xs, q, block, part1)
+                        assert _eq(dt, got[r], want), (dt, p, op, ccl, r)
+
+
+def test_allgather_rhd_is_the_permutation(orc):
+    for p in (1, 2, 3, 5, 6, 8, 12, 24):
+        ins = _inputs(INT32, p, 97, p)
+        for ccl in (200 << 20, 128 * p * 2):
+            got = orc.allgather(ins, INT32, algo=RHD, ccl_bytes=ccl)
+            want = np.concatenate(ins)
+            assert all(np.array_equal(g, want) for g in got), (p, ccl)
+
+
 @pytest.mark.parametrize("algo", [RING, MESH])
 def test_reducescatter_matches_chain(orc, algo):
     for dt in (FP32, BF16, INT8, INT64):

@@ -69,8 +69,8 @@ def test_allreduce_ring_byte_counts():
     assert plan["fusedOk"] and plan["fused"][0]["kind"] == 2 and plan["fused"][0]["nleaf"] == 16
 
 
-@pytest.mark.parametrize("algo", [RING, MESH])
-@pytest.mark.parametrize("p", [1, 2, 3, 8])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("p", [1, 2, 3, 6, 8, 12])
 def test_reducescatter_plan_matches_checker(orc, algo, p):
     for dt, op, n, ccl in ((FP32, SUM, 500, 200 << 20), (BF16, SUM, 301, 128 * p * 2), (INT64, MIN, 100, 200 << 20)):
         unit = H.DTYPE_SIZE[dt]
@@ -86,8 +86,8 @@ def test_reducescatter_plan_matches_checker(orc, algo, p):
             assert all(np.array_equal(s, i.view(np.uint8)) for s, i in zip(sends, ins))
 
 
-@pytest.mark.parametrize("algo", [RING, MESH])
-@pytest.mark.parametrize("p", [1, 2, 5, 8])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("p", [1, 2, 5, 6, 8, 12])
 def test_allgather_plan_matches_checker(orc, algo, p):
     for dt, n, ccl in ((INT8, 301, 200 << 20), (INT32, 100, 128 * p * 2)):
         unit = H.DTYPE_SIZE[dt]
@@ -121,6 +121,63 @@ def test_plan_rejects_bad_requests():
     with pytest.raises(H.HcclError):
         H.describe_plan(H.COLL_ALLREDUCE, RING, 0, 10, FP32)
     with pytest.raises(H.HcclError):
-        H.describe_plan(H.COLL_REDUCESCATTER, RHD, 4, 10, FP32)       # no halving-doubling at this level
+        H.describe_plan(H.COLL_REDUCESCATTER, H.ALGO_PAIRWISE, 4, 10, FP32)   # pairwise is an all-to-all schedule
     with pytest.raises(H.HcclError):
         H.describe_plan(H.COLL_ALLGATHER, RING, 8, 10, FP32, ccl_bytes=64)   # buffer below one aligned slice per rank
+
+
+def _v_case(p, seed):
+    rng = np.random.default_rng(seed)
+    counts = rng.integers(0, 400, p)
+    counts[rng.random(p) < 0.2] = 0
+    displs, pos = np.zeros(p, np.int64), 0
+    for i in rng.permutation(p):                 # blocks in shuffled order with gaps
+        pos += int(rng.integers(0, 9))
+        displs[i] = pos
+        pos += int(counts[i])
+    return counts, displs, pos + 3
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("p", [1, 2, 3, 6, 8])
+def test_reducescatter_v_plan_matches_checker(orc, algo, p):
+    for dt, op in ((FP32, SUM), (INT32, MAX)):
+        unit = H.DTYPE_SIZE[dt]
+        counts, displs, extent = _v_case(p, 5 * p + op)
+        ins = _ins(dt, p, extent, p)
+        plan = H.describe_plan(H.COLL_REDUCESCATTER, algo, p, 0, dt, tables=(counts, displs))
+        if algo == RHD:
+            # the checker has no variable-count halving-doubling; the tree closed form pins it
+            block, part1 = cf.rhd_params(p)
+            want = []
+            for r in range(p):
+                xs = [x[displs[r]:displs[r] + counts[r]] for x in ins]
+                q = r // 2 if r < part1 else r - part1 // 2
+                want.append(xs[0] if p == 1 else cf.rhd_tree(dt, op, xs, q, block, part1))
+        else:
+            want = orc.reducescatter_v(ins, counts, displs, dt, op, algo=algo)
+        for fused in (False, True):
+            sends = _bytes(ins)
+            recvs = [np.full(int(counts[r]) * unit, 0x5A, np.uint8) for r in range(p)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+            for r in range(p):
+                assert _same(dt, recvs[r], want[r]), (algo, p, dt, fused, r)
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("p", [1, 2, 5, 6, 8])
+def test_allgather_v_plan_matches_checker(orc, algo, p):
+    counts, displs, extent = _v_case(p, 9 * p)
+    ins = [np.arange(int(counts[r]), dtype=np.int32) + (r << 16) for r in range(p)]
+    want = np.full(extent, 0x5A5A5A5A, np.int32)
+    for r in range(p):
+        want[displs[r]:displs[r] + counts[r]] = ins[r]
+    if algo != RHD:
+        got = orc.allgather_v(ins, counts, displs, extent, INT32, algo=algo, fill=0x5A5A5A5A)
+        assert all(np.array_equal(g, want) for g in got)
+    plan = H.describe_plan(H.COLL_ALLGATHER, algo, p, 0, INT32, tables=(counts, displs))
+    for fused in (False, True):
+        recvs = [np.full(extent * 4, 0x5A, np.uint8) for _ in range(p)]
+        (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, _bytes(ins), recvs, INT32, 0)
+        for r in range(p):
+            assert np.array_equal(recvs[r].view(np.int32), want), (algo, p, fused, r)
