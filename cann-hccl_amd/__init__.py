@@ -26,7 +26,7 @@ HCCL_REDUCE_SUM, HCCL_REDUCE_PROD, HCCL_REDUCE_MAX, HCCL_REDUCE_MIN = 0, 1, 2, 3
  HCCL_DATA_TYPE_INT64, HCCL_DATA_TYPE_UINT64, HCCL_DATA_TYPE_UINT8, HCCL_DATA_TYPE_UINT16, HCCL_DATA_TYPE_UINT32,
  HCCL_DATA_TYPE_FP64, HCCL_DATA_TYPE_BFP16, HCCL_DATA_TYPE_INT128) = range(13)
 DTYPE_SIZE = {0: 1, 1: 2, 2: 4, 3: 2, 4: 4, 5: 8, 6: 8, 7: 1, 8: 2, 9: 4, 10: 8, 11: 2, 12: 16}
-COLL_ALLREDUCE, COLL_REDUCESCATTER, COLL_ALLGATHER, COLL_ALLTOALLV = range(4)
+COLL_ALLREDUCE, COLL_REDUCESCATTER, COLL_ALLGATHER, COLL_ALLTOALLV, COLL_BROADCAST, COLL_REDUCE, COLL_SCATTER = range(7)
 ALGO_RING, ALGO_MESH, ALGO_RHD, ALGO_PAIRWISE = range(4)
 
 # Every symbol include/hccl/hccl.h and include/hccl/hccl_amd_ext.h declare.
@@ -82,6 +82,9 @@ def lib():
     L.HcclReduceScatterV.argtypes = [vp, vp, vp, vp, u64, i32, i32, vp, vp]
     L.HcclAllGatherV.argtypes = [vp, u64, vp, vp, vp, i32, vp, vp]
     L.HcclBarrier.argtypes = [vp, vp]
+    L.HcclBroadcast.argtypes = [vp, u64, i32, u32, vp, vp]
+    L.HcclReduce.argtypes = [vp, vp, u64, i32, i32, u32, vp, vp]
+    L.HcclScatter.argtypes = [vp, vp, u64, i32, u32, vp, vp]
     L.HcclGetErrorString.restype = ctypes.c_char_p
     L.HcclGetErrorString.argtypes = [i32]
     L.HcclGetCommConfigCapability.restype = u32
@@ -167,6 +170,22 @@ def all_gather_v(comms, sends, recvs, counts, displs, dtype, stream):
     d = (ctypes.c_uint64 * p)(*[int(x) for x in displs])
     for r in range(p):
         _check("HcclAllGatherV", lib().HcclAllGatherV(sends[r], int(counts[r]), recvs[r], c, d, dtype, comms[r], stream))
+
+
+def broadcast(comms, bufs, count, dtype, root, stream):
+    for c, b in zip(comms, bufs):
+        _check("HcclBroadcast", lib().HcclBroadcast(b, count, dtype, root, c, stream))
+
+
+def reduce(comms, sends, recvs, count, dtype, op, root, stream):
+    for c, s, r in zip(comms, sends, recvs):
+        _check("HcclReduce", lib().HcclReduce(s, r, count, dtype, op, root, c, stream))
+
+
+def scatter(comms, sends, recvs, recv_count, dtype, root, stream):
+    """sends[r] may be None / 0 for ranks other than the root."""
+    for c, s, r in zip(comms, sends, recvs):
+        _check("HcclScatter", lib().HcclScatter(s, r, recv_count, dtype, root, c, stream))
 
 
 def barrier(comms, stream):

@@ -820,6 +820,114 @@ HcclResult HcclBarrier(HcclComm comm, aclrtStream stream)
         nullptr, nullptr, nullptr, nullptr);
 }
 
+// ---- rooted collectives ---------------------------------------------------------------------------------
+
+// op_base.cc:1433-1504.  Ring broadcast; buf is the source on the root and the destination elsewhere.
+HcclResult HcclBroadcast(void *buf, uint64_t count, HcclDataType dataType, uint32_t root, HcclComm comm, aclrtStream stream)
+{
+    if (count == 0) {
+        HCCL_LOG_WARN("HcclBroadcast: count is 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(buf);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    HcclResult r = CheckOpParam("HcclBroadcast", count, dataType, stream);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if (root >= c->group->p) {   // param_check.cc:351-359
+        HCCL_LOG_ERROR("HcclBroadcast: root %u is out of range", root);
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_BROADCAST;
+    sig.count = count;
+    sig.dtype = dataType;
+    sig.recvType = dataType;
+    sig.root = root;
+    return Arrive(c, sig, buf, buf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr);
+}
+
+// op_base.cc:2737-2814.  Ring reduce towards the root; recvBuf is written on the root only.
+HcclResult HcclReduce(void *sendBuf, void *recvBuf, uint64_t count, HcclDataType dataType, HcclReduceOp op, uint32_t root,
+    HcclComm comm, aclrtStream stream)
+{
+    if (count == 0) {
+        HCCL_LOG_WARN("HcclReduce: count is 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(sendBuf);
+    CHK_PTR(recvBuf);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    HcclResult r = CheckOpParam("HcclReduce", count, dataType, stream);
+    if (r == HCCL_SUCCESS) {
+        r = CheckReduce("HcclReduce", dataType, op);
+    }
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if (root >= c->group->p) {
+        HCCL_LOG_ERROR("HcclReduce: root %u is out of range", root);
+        return HCCL_E_PARA;
+    }
+    if ((reinterpret_cast<uintptr_t>(sendBuf) | reinterpret_cast<uintptr_t>(recvBuf)) % ElemSize(dataType) != 0) {
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_REDUCE;
+    sig.count = count;
+    sig.dtype = dataType;
+    sig.recvType = dataType;
+    sig.op = op;
+    sig.root = root;
+    return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr);
+}
+
+// op_base.cc:1720-1794.  The root's sendBuf holds p blocks of recvCount elements; rank i receives block i.
+HcclResult HcclScatter(void *sendBuf, void *recvBuf, uint64_t recvCount, HcclDataType dataType, uint32_t root, HcclComm comm,
+    aclrtStream stream)
+{
+    if (recvCount == 0) {
+        HCCL_LOG_WARN("HcclScatter: recvCount is 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(recvBuf);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    if (c->rank == root) {
+        CHK_PTR(sendBuf);
+    }
+    HcclResult r = CheckOpParam("HcclScatter", recvCount, dataType, stream);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if (root >= c->group->p) {
+        HCCL_LOG_ERROR("HcclScatter: root %u is out of range", root);
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_SCATTER;
+    sig.count = recvCount;
+    sig.dtype = dataType;
+    sig.recvType = dataType;
+    sig.root = root;
+    return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr);
+}
+
 // ---- extension ----------------------------------------------------------------------------------------
 
 HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
@@ -916,12 +1024,17 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
     uint64_t cclBytes, uint64_t align, uint64_t inPlaceMask, const uint64_t *tables, char *out, size_t cap, size_t *needed)
 {
     CHK_PTR(out);
-    if (nRanks == 0 || nRanks > kMaxRanks || !DataTypeKnown(dataType) || coll < 0 || coll > 3) {
+    if (nRanks == 0 || nRanks > kMaxRanks || !DataTypeKnown(dataType) || coll < 0 || coll > 6) {
         return HCCL_E_PARA;
     }
     PlanRequest rq;
     rq.coll = CollKind(coll);
-    rq.algo = Algo(algo);
+    if (coll >= COLL_BROADCAST) {
+        rq.root = uint32_t(algo);   // rooted collectives have one schedule each; the argument carries the root
+        rq.algo = ALGO_RING;
+    } else {
+        rq.algo = Algo(algo);
+    }
     rq.p = nRanks;
     rq.count = count;
     rq.unit = ElemSize(dataType);
@@ -1003,18 +1116,6 @@ HcclResult HcclCommInitRootInfoConfig(uint32_t, const HcclRootInfo *rootInfo, ui
     CHK_PTR(comm);
     return HCCL_E_NOT_SUPPORT;
 }
-HcclResult HcclBroadcast(void *buf, uint64_t, HcclDataType, uint32_t, HcclComm comm, aclrtStream)
-{
-    CHK_PTR(comm);
-    CHK_PTR(buf);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclScatter(void *, void *recvBuf, uint64_t, HcclDataType, uint32_t, HcclComm comm, aclrtStream)
-{
-    CHK_PTR(comm);
-    CHK_PTR(recvBuf);
-    return HCCL_E_NOT_SUPPORT;
-}
 HcclResult HcclSend(void *sendBuf, uint64_t, HcclDataType, uint32_t, HcclComm comm, aclrtStream)
 {
     CHK_PTR(comm);
@@ -1025,12 +1126,6 @@ HcclResult HcclRecv(void *recvBuf, uint64_t, HcclDataType, uint32_t, HcclComm co
 {
     CHK_PTR(comm);
     CHK_PTR(recvBuf);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclReduce(void *sendBuf, void *, uint64_t, HcclDataType, HcclReduceOp, uint32_t, HcclComm comm, aclrtStream)
-{
-    CHK_PTR(comm);
-    CHK_PTR(sendBuf);
     return HCCL_E_NOT_SUPPORT;
 }
 HcclResult HcclBatchSendRecv(HcclSendRecvItem *sendRecvInfo, uint32_t, HcclComm comm, aclrtStream)

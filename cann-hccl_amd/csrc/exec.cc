@@ -344,7 +344,8 @@ std::string CacheKey(const Group *g, int algo)
         key.push_back('v');
     }
     uint64_t head[10] = {uint64_t(g->sig.coll), uint64_t(algo), uint64_t(g->sig.dtype), uint64_t(g->sig.op), g->sig.count,
-        uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1), g->cfg.cclBytes, g->cfg.align, g->cfg.blocksPerCu, g->p};
+        uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1) | (uint64_t(g->sig.root) << 8), g->cfg.cclBytes, g->cfg.align,
+        g->cfg.blocksPerCu, g->p};
     put(head, sizeof(head));
     put(g->send.data(), g->send.size() * sizeof(void *));
     put(g->recv.data(), g->recv.size() * sizeof(void *));
@@ -360,12 +361,13 @@ std::string CacheKey(const Group *g, int algo)
 HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
 {
     std::unique_ptr<Prepared> pp(new Prepared());
-    const bool reduceColl = g->sig.coll == COLL_ALLREDUCE || g->sig.coll == COLL_REDUCESCATTER;
+    const bool reduceColl = g->sig.coll == COLL_ALLREDUCE || g->sig.coll == COLL_REDUCESCATTER || g->sig.coll == COLL_REDUCE;
     PlanRequest rq;
     rq.coll = CollKind(g->sig.coll);
     rq.algo = Algo(algo);
     rq.p = g->p;
     rq.count = g->sig.count;
+    rq.root = g->sig.root;
     rq.unit = DtypeSize(g->sig.dtype);
     rq.cclBytes = g->cfg.cclBytes;
     rq.align = g->cfg.align;
@@ -402,7 +404,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
                 return HCCL_E_PARA;
             }
             if (RangesOverlap(ri, pp->plan.recvBytes[i], sj, pp->plan.sendBytes[j])) {
-                bool exact = (i == j) && ri == sj && g->sig.coll == COLL_ALLREDUCE;
+                bool exact = (i == j) && ri == sj && (g->sig.coll == COLL_ALLREDUCE || g->sig.coll == COLL_BROADCAST);
                 needStage = needStage || !exact;
             }
         }
@@ -504,6 +506,9 @@ const char *CollName(int coll)
         case COLL_REDUCESCATTER: return "ReduceScatter";
         case COLL_ALLGATHER: return "AllGather";
         case COLL_ALLTOALLV: return "AlltoAllV";
+        case COLL_BROADCAST: return "Broadcast";
+        case COLL_REDUCE: return "Reduce";
+        case COLL_SCATTER: return "Scatter";
         default: return "?";
     }
 }
@@ -519,6 +524,8 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     int algo = g->cfg.algo >= 0 ? g->cfg.algo : DefaultAlgo(g->sig.coll);
     if (g->sig.coll == COLL_ALLTOALLV) {
         algo = ALGO_PAIRWISE;
+    } else if (g->sig.coll >= COLL_BROADCAST) {
+        algo = ALGO_RING;   // one schedule each: ring broadcast, ring reduce, mesh scatter
     } else if (algo == ALGO_PAIRWISE) {
         algo = ALGO_RING;
     }

@@ -347,6 +347,71 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
         }
         return 0;
     }
+    if (rq.coll == COLL_BROADCAST || rq.coll == COLL_REDUCE || rq.coll == COLL_SCATTER) {
+        if (rq.root >= p) {
+            *err = "root out of range";
+            return 1;
+        }
+        const uint32_t R = rq.root;
+        uint64_t total = rq.count * u;
+        if (rq.coll == COLL_SCATTER) {
+            // mesh scatter (scatter_mesh.cc:46-160): the root hands rank i block i, all at once
+            for (uint32_t r = 0; r < p; r++) {
+                EmitCopy(*vp, 0, MkRef(r, BUF_RECV, 0), MkRef(R, BUF_SEND, uint64_t(r) * total), total);
+                vp->outBytes[r] = total;
+            }
+            vp->inBytes[R] = total * p;
+            return 0;
+        }
+        uint64_t per = (rq.coll == COLL_BROADCAST || rq.coll == COLL_REDUCE) ? rq.cclBytes / u : 0;
+        if (per == 0) {
+            *err = "CCL buffer too small";
+            return 1;
+        }
+        uint64_t done = 0;
+        for (uint64_t left = rq.count; left > 0;) {
+            uint64_t cur = std::min(left, per), bytes = cur * u;
+            if (rq.coll == COLL_BROADCAST) {
+                // ring broadcast (broadcast_ring.cc:24-160): the chunk is cut into p slices that travel
+                // root -> root+1 -> ... -> root-1 as a pipeline; slice j reaches distance d in phase j+d-1
+                uint64_t sizeAvg = ((cur + p - 1) / p) * u;
+                uint64_t slice = RoundUpTo(sizeAvg, rq.align);
+                for (uint32_t j = 0; j < p && p > 1; j++) {
+                    uint64_t off = std::min<uint64_t>(uint64_t(j) * slice, bytes);
+                    uint64_t n = std::min<uint64_t>(slice, bytes - off);
+                    for (uint32_t d = 1; d < p; d++) {
+                        uint32_t r = (R + d) % p, prev = (R + d - 1) % p;
+                        Ref src = (d == 1) ? MkRef(R, BUF_SEND, done + off) : MkRef(prev, BUF_RECV, done + off);
+                        EmitCopy(*vp, j + d - 1, MkRef(r, BUF_RECV, done + off), src, n);
+                    }
+                }
+            } else {
+                // ring reduce (reduce_ring.cc:29-154): the whole chunk walks root+1 -> ... -> root, each
+                // rank combining its own data with what arrives; the root writes its output
+                if (p == 1) {
+                    EmitCopy(*vp, 0, MkRef(0, BUF_RECV, done), MkRef(0, BUF_SEND, done), bytes);
+                }
+                for (uint32_t d = 2; d <= p && p > 1; d++) {
+                    uint32_t r = (R + d) % p, prev = (R + d - 1) % p;
+                    Ref own = MkRef(r, BUF_SEND, done);
+                    Ref dst = (d == p) ? MkRef(R, BUF_RECV, done) : own;
+                    EmitReduce(*vp, d - 2, dst, own, MkRef(prev, BUF_SEND, done), bytes);
+                }
+            }
+            done += bytes;
+            left -= cur;
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            if (rq.coll == COLL_BROADCAST) {
+                vp->inBytes[r] = (r == R) ? total : 0;
+                vp->outBytes[r] = (r == R) ? 0 : total;
+            } else {
+                vp->inBytes[r] = total;
+                vp->outBytes[r] = (r == R) ? total : 0;
+            }
+        }
+        return 0;
+    }
     if (rq.algo == ALGO_PAIRWISE) {
         *err = "algorithm not available for this collective";
         return 1;
@@ -823,10 +888,18 @@ std::vector<OutRange> Outputs(const Sym &sym, uint32_t p)
 }
 
 // Text that identifies the final receive-buffer contents independently of how ranges were split.
-std::string OutputSignature(const Sym &sym, uint32_t p)
+// Ranges of an in-place rank that still hold their original bytes (never written) are left out: the
+// same memory seen as "send buffer" is not an output.
+std::string OutputSignature(const Sym &sym, uint32_t p, const std::vector<uint8_t> &alias)
 {
     std::string sig;
     for (const OutRange &o : Outputs(sym, p)) {
+        const ENode &n = sym.nodes[o.expr];
+        bool untouched = !n.red && n.leaf.rank == o.rank && n.leaf.buf == BUF_SEND && n.leaf.off + o.delta == o.start &&
+            o.rank < alias.size() && alias[o.rank];
+        if (untouched) {
+            continue;
+        }
         sig += "r" + std::to_string(o.rank) + "@" + std::to_string(o.start) + "+" + std::to_string(o.len) + "=" + o.rel + ";";
     }
     return sig;
@@ -1082,7 +1155,7 @@ int BuildPlan(const PlanRequest &rq, Plan *plan, std::string *err)
         *err = "virtual program: " + ref.err;
         return 2;
     }
-    std::string want = OutputSignature(ref, p);
+    std::string want = OutputSignature(ref, p, alias);
 
     // lowering candidates: partials in the receive buffer (no scratch), else in scratch, else staged
     bool fits = true;
@@ -1123,7 +1196,7 @@ int BuildPlan(const PlanRequest &rq, Plan *plan, std::string *err)
             why = s.err;
             continue;
         }
-        if (OutputSignature(s, p) != want) {
+        if (OutputSignature(s, p, alias) != want) {
             why = "lowered program computes different outputs";
             continue;
         }

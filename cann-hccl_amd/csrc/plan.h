@@ -9,7 +9,8 @@
 //                temp_all_gather/all_gather_ring.cc:120-171, temp_reduce_scatter/reduce_scatter_mesh.cc:57-124,
 //                temp_all_gather/all_gather_mesh.cc:91-145, temp_all_reduce/all_reduce_recursive_hd.cc:33-302,
 //                temp_reduce_scatter/reduce_scatter_halving_doubling.cc:67-238,
-//                temp_all_gather/all_gather_halving_doubling.cc:43-196, temp_alltoallv/alltoallv_pairwise.cc:99-282
+//                temp_all_gather/all_gather_halving_doubling.cc:43-196, temp_alltoallv/alltoallv_pairwise.cc:99-282,
+//                temp_broadcast/broadcast_ring.cc:24-160, temp_reduce/reduce_ring.cc:29-154, temp_scatter/scatter_mesh.cc:46-160
 // (ALG = src/domain/collective_communication/algorithm in the reference tree.)
 //
 // Pure C++: no HIP calls, so the planner can be exercised without a GPU.
@@ -20,7 +21,10 @@
 
 namespace hcclamd {
 
-enum CollKind : int { COLL_ALLREDUCE = 0, COLL_REDUCESCATTER = 1, COLL_ALLGATHER = 2, COLL_ALLTOALLV = 3 };
+enum CollKind : int {
+    COLL_ALLREDUCE = 0, COLL_REDUCESCATTER = 1, COLL_ALLGATHER = 2, COLL_ALLTOALLV = 3,
+    COLL_BROADCAST = 4, COLL_REDUCE = 5, COLL_SCATTER = 6
+};
 enum Algo : int { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2, ALGO_PAIRWISE = 3 };
 
 // Physical buffers of a rank: the caller's send and receive buffers and a library-owned scratch.
@@ -67,6 +71,7 @@ struct PlanRequest {
     Algo algo = ALGO_RING;
     uint32_t p = 1;
     uint64_t count = 0;            // all-reduce: elements; reduce-scatter: recvCount; all-gather: sendCount
+    uint32_t root = 0;             // broadcast / reduce / scatter
     uint32_t unit = 4;             // element size in bytes
     uint64_t cclBytes = 200ull << 20;
     uint64_t align = 128;

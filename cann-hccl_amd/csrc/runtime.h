@@ -78,10 +78,11 @@ struct OpSig {
     uint64_t count = 0;
     int dtype = 0, recvType = 0, op = 0;
     int variable = 0;                // 1: reduce-scatter-v / all-gather-v (block tables instead of a count)
+    uint32_t root = 0;               // broadcast / reduce / scatter
     bool operator==(const OpSig &o) const
     {
         return coll == o.coll && count == o.count && dtype == o.dtype && recvType == o.recvType && op == o.op &&
-            variable == o.variable;
+            variable == o.variable && root == o.root;
     }
 };
 

@@ -22,7 +22,7 @@ extern "C" {
 extern HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value);
 
 typedef struct HcclAmdOpInfoDef {
-    int32_t coll;            /* 0 all-reduce, 1 reduce-scatter, 2 all-gather, 3 all-to-all-v */
+    int32_t coll;            /* 0 all-reduce, 1 reduce-scatter, 2 all-gather, 3 all-to-all-v, 4 broadcast, 5 reduce, 6 scatter */
     int32_t algo;            /* 0 ring, 1 mesh, 2 rhd, 3 pairwise */
     int32_t fused;           /* 1: issued as fused single-pass kernels */
     int32_t graph;           /* 1: issued as a HIP graph */
@@ -39,7 +39,8 @@ typedef struct HcclAmdOpInfoDef {
 extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
 
 /* Plans a collective without a device and writes the plan as JSON (phases of copy / reduce steps,
- * fused items, byte counts) into out[0..cap).  coll / algo as in HcclAmdOpInfo.  inPlaceMask bit r:
+ * fused items, byte counts) into out[0..cap).  coll / algo as in HcclAmdOpInfo; for the rooted
+ * collectives (coll 4 broadcast, 5 reduce, 6 scatter) the algo argument carries the root rank.  inPlaceMask bit r:
  * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64
  * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); for the variable-count
  * reduce-scatter / all-gather, tables points to 2*p uint64 (block counts, block displacements); else NULL.

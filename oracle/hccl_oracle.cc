@@ -20,6 +20,8 @@
 //                    TPL/temp_reduce_scatter/reduce_scatter_halving_doubling.cc:67-238,
 //                    TPL/temp_all_gather/all_gather_halving_doubling.cc:43-196
 //   pairwise         TPL/temp_alltoallv/alltoallv_pairwise.cc:75-282, ALG/impl/operator/alltoall_operator.cc:49-72
+//   rooted           TPL/temp_broadcast/broadcast_ring.cc:24-160, TPL/temp_reduce/reduce_ring.cc:29-154,
+//                    TPL/temp_scatter/scatter_mesh.cc:46-160
 //
 // Method: every template is restated as the per-rank program it issues (send / receive-and-reduce /
 // receive-and-copy / local copy), one virtual process per rank (per rank and stream for the mesh),
@@ -1271,6 +1273,170 @@ int orc_allgather_v(int algo, uint32_t p, void **in, void **out, const uint64_t 
             ProgAllGatherMesh(pr.prog, r, p, B_OUT, sl);
         } else {
             return -10;
+        }
+        m.procs.push_back(std::move(pr));
+    }
+    return m.Run();
+}
+
+// Ring broadcast (broadcast_ring.cc:24-160) with the executor's chunk loop: buf[root] is the source,
+// every other buf receives it.  Slices of one chunk travel root -> root+1 -> ... -> root-1.
+int orc_broadcast(uint32_t p, void **buf, uint64_t count, int dt, uint32_t root, uint64_t cclBytes, uint64_t align,
+    int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0 && p > 1;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            m.buf[B_IN][r] = static_cast<uint8_t *>(buf[r]) + offset;
+            m.buf[B_OUT][r] = static_cast<uint8_t *>(buf[r]) + offset;
+        }
+        uint64_t sizeAvg = ((cur + p - 1) / p) * unit;
+        uint64_t per = RoundUp(sizeAvg, align);
+        for (uint32_t r = 0; r < p; r++) {
+            Proc pr;
+            pr.rank = r;
+            uint32_t left_ = (r + p - 1) % p, right = (r + 1) % p;
+            uint64_t residue = bytes;
+            for (uint32_t round = 0; round < p; round++) {
+                uint64_t n = residue > per ? per : residue;
+                uint64_t at = bytes - residue;
+                if (r == root) {
+                    pr.prog.push_back(MkSend(static_cast<int>(right), 0, B_IN, at, n));
+                } else {
+                    pr.prog.push_back(MkRecvCopy(static_cast<int>(left_), 0, B_OUT, at, n));
+                    if (right != root) {
+                        pr.prog.push_back(MkSend(static_cast<int>(right), 0, B_OUT, at, n));
+                    }
+                }
+                residue -= n;
+            }
+            m.procs.push_back(std::move(pr));
+        }
+        int rc = m.Run();
+        if (rc != 0) {
+            return rc;
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
+// Ring reduce (reduce_ring.cc:29-154) with the executor's chunk loop; out[root] receives the result.
+// Inputs are staged (the schedule accumulates in its input buffer).
+int orc_reduce_to_root(uint32_t p, void **in, void *outRoot, uint64_t count, int dt, int op, uint32_t root, uint64_t cclBytes,
+    int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.op = op;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    uint64_t stage = std::min<uint64_t>(count, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage)), cclOut(p, std::vector<uint8_t>(stage));
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_IN][r] = cclIn[r].data();
+        m.buf[B_OUT][r] = cclOut[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            m.Copy(m.buf[B_IN][r], static_cast<uint8_t *>(in[r]) + offset, bytes);
+        }
+        if (p == 1) {
+            m.Copy(m.buf[B_OUT][0], m.buf[B_IN][0], bytes);
+        } else {
+            for (uint32_t r = 0; r < p; r++) {
+                Proc pr;
+                pr.rank = r;
+                uint32_t left_ = (r + p - 1) % p, right = (r + 1) % p;
+                if (r == root) {
+                    pr.prog.push_back(MkRecvReduce(static_cast<int>(left_), 0, B_OUT, 0, B_IN, 0, bytes));
+                } else if (left_ == root) {
+                    pr.prog.push_back(MkSend(static_cast<int>(right), 0, B_IN, 0, bytes));
+                } else {
+                    pr.prog.push_back(MkRecvReduce(static_cast<int>(left_), 0, B_IN, 0, B_IN, 0, bytes));
+                    pr.prog.push_back(MkSend(static_cast<int>(right), 0, B_IN, 0, bytes));
+                }
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        m.Copy(static_cast<uint8_t *>(outRoot) + offset, m.buf[B_OUT][root], bytes);
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
+// Mesh scatter (scatter_mesh.cc:46-160): in (on the root) holds p blocks of `count` elements.
+int orc_scatter(uint32_t p, const void *inRoot, void **out, uint64_t count, int dt, uint32_t root, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t bytes = count * unit;
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    m.buf[B_IN].assign(p, nullptr);
+    m.buf[B_OUT].resize(p);
+    m.buf[B_IN][root] = static_cast<uint8_t *>(const_cast<void *>(inRoot));
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_OUT][r] = static_cast<uint8_t *>(out[r]);
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        if (r == root) {
+            for (uint32_t d = 0; d < p; d++) {
+                if (d == root) {
+                    pr.prog.push_back(MkLocalCopy(B_OUT, 0, B_IN, bytes * d, bytes));
+                } else {
+                    pr.prog.push_back(MkSend(static_cast<int>(d), 0, B_IN, bytes * d, bytes));
+                }
+            }
+        } else {
+            pr.prog.push_back(MkRecvCopy(static_cast<int>(root), 0, B_OUT, 0, bytes));
         }
         m.procs.push_back(std::move(pr));
     }

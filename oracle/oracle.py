@@ -61,6 +61,9 @@ def lib():
         L.orc_allgather.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, u64, u64, i32, i32]
         L.orc_reducescatter_v.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), pu64, pu64, i32, i32, u64, i32, i32]
         L.orc_allgather_v.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), pu64, pu64, i32, i32, i32]
+        L.orc_broadcast.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
+        L.orc_reduce_to_root.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, i32, i32]
+        L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
         L.orc_alltoallv.argtypes = [u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, u64, i32, i32]
         L.orc_fill_uniform_f32.argtypes = [vp, u64, u64, u32, i32]
         _lib = L
@@ -213,6 +216,31 @@ def allgather_v(ins, counts, displs, out_len, dt, algo=RING, flags=0, threads=1,
     rc = lib().orc_allgather_v(algo, p, _ptrs(ins), _ptrs(outs), c, d, dt, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle allgather_v failed rc=%d" % rc)
+    return outs
+
+
+def broadcast(bufs, dt, root, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1):
+    """bufs: p equal-length arrays, written in place: every array becomes bufs[root]."""
+    rc = lib().orc_broadcast(len(bufs), _ptrs(bufs), bufs[0].size, dt, root, ccl_bytes, align, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle broadcast failed rc=%d" % rc)
+    return bufs
+
+
+def reduce_to_root(ins, dt, op, root, ccl_bytes=DEFAULT_CCL_BYTES, flags=0, threads=1):
+    out = np.empty_like(ins[0])
+    rc = lib().orc_reduce_to_root(len(ins), _ptrs(ins), out.ctypes.data, ins[0].size, dt, op, root, ccl_bytes, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle reduce failed rc=%d" % rc)
+    return out
+
+
+def scatter(src, p, dt, root, flags=0, threads=1):
+    n = src.size // p
+    outs = [np.empty(n, dtype=src.dtype) for _ in range(p)]
+    rc = lib().orc_scatter(p, src.ctypes.data, _ptrs(outs), n, dt, root, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle scatter failed rc=%d" % rc)
     return outs
 
 

@@ -206,9 +206,28 @@ def test_amd_params(comms):
 
 
 def test_unsupported_entry_points_link_and_refuse(comms):
-    assert L.HcclBroadcast(BUF_A, 4, 4, 0, comms[0], STREAM) == H.HCCL_E_NOT_SUPPORT
-    assert L.HcclBroadcast(BUF_A, 4, 4, 0, None, STREAM) == H.HCCL_E_PTR
+    assert L.HcclSend(BUF_A, 4, 4, 1, comms[0], STREAM) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclSend(BUF_A, 4, 4, 1, None, STREAM) == H.HCCL_E_PTR
     assert L.HcclGetRootInfo(None) == H.HCCL_E_PTR
+
+
+def test_rooted_entry_checks(comms):
+    c = comms[0]
+    FP32, SUM = H.HCCL_DATA_TYPE_FP32, H.HCCL_REDUCE_SUM
+    assert L.HcclBroadcast(None, 0, FP32, 0, None, None) == H.HCCL_SUCCESS                  # count 0 first
+    assert L.HcclBroadcast(BUF_A, 4, FP32, 0, None, STREAM) == H.HCCL_E_PTR
+    assert L.HcclBroadcast(None, 4, FP32, 0, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclBroadcast(BUF_A, 4, FP32, 0, c, None) == H.HCCL_E_PTR
+    assert L.HcclBroadcast(BUF_A, 4, FP32, 4, c, STREAM) == H.HCCL_E_PARA                    # root out of range
+    assert L.HcclReduce(None, None, 0, FP32, SUM, 0, None, None) == H.HCCL_SUCCESS
+    assert L.HcclReduce(BUF_A, None, 4, FP32, SUM, 0, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclReduce(BUF_A, BUF_B, 4, FP32, 8, 0, c, STREAM) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclReduce(BUF_A, BUF_B, 4, FP32, SUM, 9, c, STREAM) == H.HCCL_E_PARA
+    assert L.HcclScatter(None, BUF_B, 0, FP32, 0, c, STREAM) == H.HCCL_SUCCESS
+    assert L.HcclScatter(None, None, 4, FP32, 0, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclScatter(None, BUF_B, 4, FP32, 0, c, STREAM) == H.HCCL_E_PTR                 # rank 0 is the root: needs sendBuf
+    assert L.HcclScatter(None, BUF_B, 4, FP32, 1, c, STREAM) == H.HCCL_SUCCESS               # not the root: joins
+    assert L.HcclScatter(BUF_A, BUF_B, 4, FP32, 2, comms[1], STREAM) == H.HCCL_E_PARA        # ranks disagree on the root
 
 
 def test_no_gpu_means_loud_failure(comms):

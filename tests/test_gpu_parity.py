@@ -439,3 +439,82 @@ def test_special_values_16bit(orc):
                         assert gh.same(dt, outs[r], want[r]), (dt, fuse, op, r)
             finally:
                 g.close()
+
+
+def test_broadcast_reduce_scatter_rooted(orc):
+    for p in (1, 3, 8):
+        for fuse in (1, 0):
+            g = gh.Group(p, fuse=fuse)
+            try:
+                for root in sorted({0, p - 1}):
+                    print("rooted p", p, "fuse", fuse, "root", root, flush=True)
+                    # broadcast
+                    n = 70001
+                    bufs_np = _ins(FP32, p, n, 90 + p)
+                    bufs = [gh.to_dev(x) for x in bufs_np]
+                    torch.cuda.synchronize()
+                    H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, FP32, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(bufs[r], FP32), bufs_np[root]), ("bcast", p, fuse, root, r)
+                    # reduce
+                    for dt, op in ((FP32, SUM), (BF16, SUM), (INT16, MAX)):
+                        ins = _ins(dt, p, n, 91 + p + dt)
+                        want = orc.reduce_to_root(ins, dt, op, root)
+                        sends = [gh.to_dev(x) for x in ins]
+                        recvs = [gh.empty_dev(n * H.DTYPE_SIZE[dt], fill=0x33) for _ in range(p)]
+                        torch.cuda.synchronize()
+                        H.reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, op, root, g.stream_ptr)
+                        g.stream.synchronize()
+                        assert gh.same(dt, gh.to_host(recvs[root], dt), want), ("reduce", p, fuse, root, dt)
+                        for r in range(p):
+                            assert np.array_equal(gh.to_host(sends[r], dt), ins[r])
+                            if r != root:
+                                assert bool((recvs[r] == 0x33).all())
+                    # scatter
+                    src = np.arange(n * p, dtype=np.int32) * 3 + 1
+                    sends = [gh.to_dev(src) if r == root else None for r in range(p)]
+                    recvs = [gh.empty_dev(n * 4) for _ in range(p)]
+                    torch.cuda.synchronize()
+                    H.scatter(g.comms, [t.data_ptr() if t is not None else None for t in sends], [t.data_ptr() for t in recvs],
+                              n, INT32, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(recvs[r], INT32), src[r * n:(r + 1) * n]), ("scatter", p, fuse, root, r)
+            finally:
+                g.close()
+
+
+def test_one_thread_per_rank_blocking_arrival(orc):
+    # the reference's model: every rank on its own thread and stream; calls return once the collective is issued
+    import threading
+    p, n = 8, 1 << 18
+    ins = _ins(FP32, p, n, 123)
+    want = orc.allreduce(ins, FP32, SUM)
+    g = gh.Group(p, blocking_arrive=1, arrive_timeout_ms=20000)
+    try:
+        sends = [gh.to_dev(x) for x in ins]
+        recvs = [gh.empty_dev(n * 4) for _ in range(p)]
+        streams = [torch.cuda.Stream() for _ in range(p)]
+        torch.cuda.synchronize()
+        codes = [None] * p
+
+        def work(r):
+            for _ in range(3):
+                codes[r] = H.lib().HcclAllReduce(sends[r].data_ptr(), recvs[r].data_ptr(), n, FP32, SUM, g.comms[r],
+                                                 streams[r].cuda_stream)
+                if codes[r] != 0:
+                    return
+            streams[r].synchronize()
+
+        ts = [threading.Thread(target=work, args=(r,)) for r in range(p)]
+        for t in ts:
+            t.start()
+        for t in ts:
+            t.join(60)
+        assert codes == [0] * p
+        torch.cuda.synchronize()
+        for r in range(p):
+            assert np.array_equal(gh.to_host(recvs[r], FP32), want[r]), r
+    finally:
+        g.close()

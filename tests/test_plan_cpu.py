@@ -181,3 +181,47 @@ def test_allgather_v_plan_matches_checker(orc, algo, p):
         (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, _bytes(ins), recvs, INT32, 0)
         for r in range(p):
             assert np.array_equal(recvs[r].view(np.int32), want), (algo, p, fused, r)
+
+
+@pytest.mark.parametrize("p", [1, 2, 3, 5, 8])
+def test_rooted_plans_match_checker(orc, p):
+    rng = np.random.default_rng(p)
+    for root in sorted({0, p - 1, p // 2}):
+        # broadcast (in place on every rank), two chunk settings
+        n = 1003
+        for ccl in (200 << 20, 1024):
+            bufs = _ins(INT32, p, n, 50 + p)
+            want = orc.broadcast([b.copy() for b in bufs], INT32, root, ccl_bytes=ccl)
+            plan = H.describe_plan(H.COLL_BROADCAST, root, p, n, INT32, ccl_bytes=ccl, in_place_mask=(1 << p) - 1)
+            for fused in (False, True):
+                mem = _bytes(bufs)
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, mem, mem, INT32, 0, in_place=True)
+                for r in range(p):
+                    assert np.array_equal(mem[r].view(np.int32), want[r]), ("bcast", p, root, ccl, fused, r)
+        # reduce to the root: ring chain x_root (+) (x_{root-1} (+) ( ... (x_{root+2} (+) x_{root+1})))
+        for dt, op in ((FP32, SUM), (BF16, PROD), (INT8, MIN)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n, 60 + p + dt)
+            want = orc.reduce_to_root(ins, dt, op, root, ccl_bytes=2048)
+            chain = cf.ring_chain(dt, op, ins, root) if p > 1 else ins[0]
+            assert _same(dt, want.view(np.uint8), chain)
+            plan = H.describe_plan(H.COLL_REDUCE, root, p, n, dt, ccl_bytes=2048)
+            for fused in (False, True):
+                sends = _bytes(ins)
+                recvs = [np.full(n * unit, 0x77, np.uint8) for _ in range(p)]
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+                assert _same(dt, recvs[root], want), ("reduce", p, root, dt, fused)
+                for r in range(p):
+                    assert np.array_equal(sends[r], ins[r].view(np.uint8))
+                    if r != root:
+                        assert np.all(recvs[r] == 0x77)              # only the root's output is written
+        # scatter
+        src = rng.integers(0, 1 << 30, n * p).astype(np.int32)
+        want = orc.scatter(src, p, INT32, root)
+        plan = H.describe_plan(H.COLL_SCATTER, root, p, n, INT32)
+        for fused in (False, True):
+            sends = [src.view(np.uint8).copy() if r == root else np.zeros(0, np.uint8) for r in range(p)]
+            recvs = [np.zeros(n * 4, np.uint8) for _ in range(p)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, INT32, 0)
+            for r in range(p):
+                assert np.array_equal(recvs[r].view(np.int32), want[r]) and np.array_equal(want[r], src[r * n:(r + 1) * n])
