@@ -49,6 +49,11 @@ class HcclAmdOpInfo(ctypes.Structure):
                 ("scratchBytes", ctypes.c_uint64)]
 
 
+class HcclSendRecvItem(ctypes.Structure):
+    _fields_ = [("sendRecvType", ctypes.c_int32), ("buf", ctypes.c_void_p), ("count", ctypes.c_uint64),
+                ("dataType", ctypes.c_int32), ("remoteRank", ctypes.c_uint32)]
+
+
 _lib = None
 
 
@@ -85,6 +90,9 @@ def lib():
     L.HcclBroadcast.argtypes = [vp, u64, i32, u32, vp, vp]
     L.HcclReduce.argtypes = [vp, vp, u64, i32, i32, u32, vp, vp]
     L.HcclScatter.argtypes = [vp, vp, u64, i32, u32, vp, vp]
+    L.HcclSend.argtypes = [vp, u64, i32, u32, vp, vp]
+    L.HcclRecv.argtypes = [vp, u64, i32, u32, vp, vp]
+    L.HcclBatchSendRecv.argtypes = [ctypes.POINTER(HcclSendRecvItem), u32, vp, vp]
     L.HcclGetErrorString.restype = ctypes.c_char_p
     L.HcclGetErrorString.argtypes = [i32]
     L.HcclGetCommConfigCapability.restype = u32
@@ -186,6 +194,26 @@ def scatter(comms, sends, recvs, recv_count, dtype, root, stream):
     """sends[r] may be None / 0 for ranks other than the root."""
     for c, s, r in zip(comms, sends, recvs):
         _check("HcclScatter", lib().HcclScatter(s, r, recv_count, dtype, root, c, stream))
+
+
+def send(comm, buf, count, dtype, dest, stream):
+    _check("HcclSend", lib().HcclSend(buf, count, dtype, dest, comm, stream))
+
+
+def recv(comm, buf, count, dtype, src, stream):
+    _check("HcclRecv", lib().HcclRecv(buf, count, dtype, src, comm, stream))
+
+
+def batch_send_recv(comm, items, stream):
+    """items: list of (is_send, buf, count, dtype, remote_rank)."""
+    arr = (HcclSendRecvItem * len(items))()
+    for i, (is_send, buf, count, dtype, remote) in enumerate(items):
+        arr[i].sendRecvType = 0 if is_send else 1
+        arr[i].buf = buf
+        arr[i].count = count
+        arr[i].dataType = dtype
+        arr[i].remoteRank = remote
+    _check("HcclBatchSendRecv", lib().HcclBatchSendRecv(arr, len(items), comm, stream))
 
 
 def barrier(comms, stream):

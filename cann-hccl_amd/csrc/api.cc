@@ -168,18 +168,18 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
         return HCCL_E_AGAIN;
     }
     bool tablesDiffer = false;
-    if (sig.variable && g->arrived > 0 && g->sig.variable) {
+    if (sig.variable && g->arrived > 0 && g->pend.sig.variable) {
         for (uint32_t i = 0; i < g->p; i++) {
-            tablesDiffer = tablesDiffer || g->vCounts[i] != vCounts[i] || g->vDispls[i] != vDispls[i];
+            tablesDiffer = tablesDiffer || g->pend.vCounts[i] != vCounts[i] || g->pend.vDispls[i] != vDispls[i];
         }
     }
     if (g->arrived == 0) {
-        g->sig = sig;
+        g->pend.sig = sig;
         if (sig.variable) {
-            g->vCounts.assign(vCounts, vCounts + g->p);
-            g->vDispls.assign(vDispls, vDispls + g->p);
+            g->pend.vCounts.assign(vCounts, vCounts + g->p);
+            g->pend.vDispls.assign(vDispls, vDispls + g->p);
         }
-    } else if (!(g->sig == sig) || tablesDiffer) {
+    } else if (!(g->pend.sig == sig) || tablesDiffer) {
         // every rank must pass the same operation, count, type and op (the reference checks this
         // across processes in RankConsistentcyChecker, hccl_communicator.cc:2803-2805)
         HCCL_LOG_ERROR("%s: rank %u disagrees with the ranks already in the collective (op/count/type)", CollName(sig.coll), r);
@@ -187,19 +187,19 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
         return HCCL_E_PARA;
     }
     g->here[r] = 1;
-    g->send[r] = send;
-    g->recv[r] = recv;
-    g->streams[r] = stream;
+    g->pend.send[r] = send;
+    g->pend.recv[r] = recv;
+    g->pend.streams[r] = stream;
     if (sig.coll == COLL_ALLTOALLV) {
         size_t p = g->p;
-        g->sendCounts.resize(p * p);
-        g->sdispls.resize(p * p);
-        g->recvCounts.resize(p * p);
-        g->rdispls.resize(p * p);
-        std::copy(sendCounts, sendCounts + p, g->sendCounts.begin() + r * p);
-        std::copy(sdispls, sdispls + p, g->sdispls.begin() + r * p);
-        std::copy(recvCounts, recvCounts + p, g->recvCounts.begin() + r * p);
-        std::copy(rdispls, rdispls + p, g->rdispls.begin() + r * p);
+        g->pend.sendCounts.resize(p * p);
+        g->pend.sdispls.resize(p * p);
+        g->pend.recvCounts.resize(p * p);
+        g->pend.rdispls.resize(p * p);
+        std::copy(sendCounts, sendCounts + p, g->pend.sendCounts.begin() + r * p);
+        std::copy(sdispls, sdispls + p, g->pend.sdispls.begin() + r * p);
+        std::copy(recvCounts, recvCounts + p, g->pend.recvCounts.begin() + r * p);
+        std::copy(rdispls, rdispls + p, g->pend.rdispls.begin() + r * p);
     }
     g->arrived++;
     if (g->arrived < g->p) {
@@ -222,10 +222,10 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
         // alltoall_operator.cc:49-72: what i sends to j must be what j expects from i
         for (uint32_t i = 0; i < g->p && res == HCCL_SUCCESS; i++) {
             for (uint32_t j = 0; j < g->p; j++) {
-                if (g->sendCounts[size_t(i) * g->p + j] != g->recvCounts[size_t(j) * g->p + i]) {
+                if (g->pend.sendCounts[size_t(i) * g->p + j] != g->pend.recvCounts[size_t(j) * g->p + i]) {
                     HCCL_LOG_ERROR("AlltoAllV: rank %u sends %llu elements to rank %u, which expects %llu", i,
-                        (unsigned long long)g->sendCounts[size_t(i) * g->p + j], j,
-                        (unsigned long long)g->recvCounts[size_t(j) * g->p + i]);
+                        (unsigned long long)g->pend.sendCounts[size_t(i) * g->p + j], j,
+                        (unsigned long long)g->pend.recvCounts[size_t(j) * g->p + i]);
                     res = HCCL_E_PARA;
                     break;
                 }
@@ -233,6 +233,7 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
         }
     }
     if (res == HCCL_SUCCESS) {
+        g->ctx = &g->pend;
         res = IssueCollective(g, r);
     }
     if (res != HCCL_SUCCESS && res != HCCL_E_PARA) {
@@ -240,6 +241,60 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
     }
     g->lastIssueResult = res;
     CancelPending(g);   // resets the rendezvous and wakes blocked ranks
+    return res;
+}
+
+// A send meets its receive (or the other way round): the later of the two calls issues the copy on
+// its stream, ordered after the earlier caller's stream and before whatever that stream runs next.
+HcclResult PointToPoint(Comm *c, bool isSend, void *buf, uint64_t count, HcclDataType dataType, uint32_t other,
+    hipStream_t stream)
+{
+    Group *g = c->group;
+    std::unique_lock<std::mutex> lock(g->m);
+    if (g->suspended) {
+        return HCCL_E_SUSPENDING;
+    }
+    if (other >= g->p) {
+        HCCL_LOG_ERROR("send / receive: rank %u is out of range", other);
+        return HCCL_E_PARA;
+    }
+    uint32_t src = isSend ? c->rank : other, dst = isSend ? other : c->rank;
+    auto &queue = g->p2p[std::make_pair(src, dst)];
+    if (queue.empty() || queue.front().isSend == isSend) {
+        P2PPending pnd;
+        pnd.isSend = isSend;
+        pnd.buf = buf;
+        pnd.count = count;
+        pnd.dtype = dataType;
+        pnd.stream = stream;
+        queue.push_back(pnd);
+        return HCCL_SUCCESS;
+    }
+    P2PPending match = queue.front();
+    queue.pop_front();
+    if (match.count != count || match.dtype != int(dataType)) {
+        HCCL_LOG_ERROR("send / receive between rank %u and rank %u disagree on count or type", src, dst);
+        return HCCL_E_PARA;
+    }
+    OpCtx ctx;
+    ctx.sig.coll = COLL_SENDRECV;
+    ctx.sig.count = count;
+    ctx.sig.dtype = dataType;
+    ctx.sig.recvType = dataType;
+    ctx.sig.root = src;
+    ctx.sig.peer = dst;
+    ctx.send.assign(g->p, nullptr);
+    ctx.recv.assign(g->p, nullptr);
+    ctx.streams.assign(g->p, stream);
+    ctx.send[src] = isSend ? buf : match.buf;
+    ctx.recv[dst] = isSend ? match.buf : buf;
+    ctx.streams[other] = match.stream;
+    g->ctx = &ctx;
+    HcclResult res = IssueCollective(g, c->rank);
+    g->ctx = &g->pend;
+    if (res != HCCL_SUCCESS && res != HCCL_E_PARA) {
+        g->asyncError = res;
+    }
     return res;
 }
 
@@ -271,9 +326,9 @@ HcclResult HcclCommInitAll(uint32_t ndev, int32_t *devices, HcclComm *comms)
     g->p = ndev;
     ApplyEnv(&g->cfg);
     g->here.assign(ndev, 0);
-    g->send.assign(ndev, nullptr);
-    g->recv.assign(ndev, nullptr);
-    g->streams.assign(ndev, nullptr);
+    g->pend.send.assign(ndev, nullptr);
+    g->pend.recv.assign(ndev, nullptr);
+    g->pend.streams.assign(ndev, nullptr);
     char nm[64];
     std::snprintf(nm, sizeof(nm), "hccl_world_group_%p", static_cast<void *>(g));
     g->name = nm;
@@ -312,6 +367,9 @@ HcclResult HcclCommDestroy(HcclComm comm)
         if (g->here[c->rank]) {
             HCCL_LOG_WARN("HcclCommDestroy: rank %u had joined a collective that was never issued; it is dropped", c->rank);
             CancelPending(g);
+        }
+        for (auto it = g->p2p.begin(); it != g->p2p.end();) {   // unmatched sends / receives of this rank
+            it = (it->first.first == c->rank || it->first.second == c->rank) ? g->p2p.erase(it) : std::next(it);
         }
         c->magic = 0;
         c->group = nullptr;
@@ -928,6 +986,98 @@ HcclResult HcclScatter(void *sendBuf, void *recvBuf, uint64_t recvCount, HcclDat
     return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr);
 }
 
+// ---- point to point -----------------------------------------------------------------------------------------
+
+// op_base.cc:1974-2054.
+HcclResult HcclSend(void *sendBuf, uint64_t count, HcclDataType dataType, uint32_t destRank, HcclComm comm, aclrtStream stream)
+{
+    if (count == 0) {
+        HCCL_LOG_WARN("HcclSend: count is 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(sendBuf);
+    CHK_PTR(stream);
+    if (count > kSysMaxCount) {
+        return HCCL_E_PARA;
+    }
+    if (!DataTypeKnown(dataType)) {
+        return HCCL_E_NOT_SUPPORT;
+    }
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    return PointToPoint(c, true, sendBuf, count, dataType, destRank, static_cast<hipStream_t>(stream));
+}
+
+// op_base.cc:2056-2135.
+HcclResult HcclRecv(void *recvBuf, uint64_t count, HcclDataType dataType, uint32_t srcRank, HcclComm comm, aclrtStream stream)
+{
+    if (count == 0) {
+        HCCL_LOG_WARN("HcclRecv: count is 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(recvBuf);
+    CHK_PTR(stream);
+    if (count > kSysMaxCount) {
+        return HCCL_E_PARA;
+    }
+    if (!DataTypeKnown(dataType)) {
+        return HCCL_E_NOT_SUPPORT;
+    }
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    return PointToPoint(c, false, recvBuf, count, dataType, srcRank, static_cast<hipStream_t>(stream));
+}
+
+// op_base.cc:3428-3509: every item is a send or a receive of this rank.
+HcclResult HcclBatchSendRecv(HcclSendRecvItem *sendRecvInfo, uint32_t itemNum, HcclComm comm, aclrtStream stream)
+{
+    CHK_PTR(comm);
+    CHK_PTR(stream);
+    CHK_PTR(sendRecvInfo);
+    if (itemNum == 0) {
+        HCCL_LOG_WARN("HcclBatchSendRecv: no items");
+        return HCCL_SUCCESS;
+    }
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    for (uint32_t i = 0; i < itemNum; i++) {
+        const HcclSendRecvItem &it = sendRecvInfo[i];
+        CHK_PTR(it.buf);
+        if (it.count > kSysMaxCount) {
+            return HCCL_E_PARA;
+        }
+        if (!DataTypeKnown(it.dataType)) {
+            return HCCL_E_NOT_SUPPORT;
+        }
+        if (it.sendRecvType != HCCL_SEND && it.sendRecvType != HCCL_RECV) {
+            return HCCL_E_PARA;
+        }
+    }
+    for (uint32_t i = 0; i < itemNum; i++) {
+        const HcclSendRecvItem &it = sendRecvInfo[i];
+        if (it.count == 0) {
+            continue;
+        }
+        HcclResult r = PointToPoint(c, it.sendRecvType == HCCL_SEND, it.buf, it.count, it.dataType, it.remoteRank,
+            static_cast<hipStream_t>(stream));
+        if (r != HCCL_SUCCESS) {
+            return r;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
 // ---- extension ----------------------------------------------------------------------------------------
 
 HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
@@ -1114,24 +1264,6 @@ HcclResult HcclCommInitRootInfoConfig(uint32_t, const HcclRootInfo *rootInfo, ui
     CHK_PTR(rootInfo);
     CHK_PTR(config);
     CHK_PTR(comm);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclSend(void *sendBuf, uint64_t, HcclDataType, uint32_t, HcclComm comm, aclrtStream)
-{
-    CHK_PTR(comm);
-    CHK_PTR(sendBuf);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclRecv(void *recvBuf, uint64_t, HcclDataType, uint32_t, HcclComm comm, aclrtStream)
-{
-    CHK_PTR(comm);
-    CHK_PTR(recvBuf);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclBatchSendRecv(HcclSendRecvItem *sendRecvInfo, uint32_t, HcclComm comm, aclrtStream)
-{
-    CHK_PTR(comm);
-    CHK_PTR(sendRecvInfo);
     return HCCL_E_NOT_SUPPORT;
 }
 HcclResult HcclCommSetMemoryRange(HcclComm comm, void *, size_t, size_t, uint64_t)

@@ -93,8 +93,8 @@ struct Builder {
     {
         char *base = nullptr;
         switch (r.buf) {
-            case BUF_SEND: base = static_cast<char *>(g->send[r.rank]); break;
-            case BUF_RECV: base = static_cast<char *>(g->recv[r.rank]); break;
+            case BUF_SEND: base = static_cast<char *>(g->ctx->send[r.rank]); break;
+            case BUF_RECV: base = static_cast<char *>(g->ctx->recv[r.rank]); break;
             default: base = static_cast<char *>(g->scratch[r.rank]); break;
         }
         return base + r.off;
@@ -338,22 +338,22 @@ std::string CacheKey(const Group *g, int algo)
     // raw bytes of everything the prepared tables depend on
     std::string key;
     auto put = [&](const void *p, size_t n) { key.append(static_cast<const char *>(p), n); };
-    if (g->sig.variable) {
-        put(g->vCounts.data(), g->vCounts.size() * 8);
-        put(g->vDispls.data(), g->vDispls.size() * 8);
+    if (g->ctx->sig.variable) {
+        put(g->ctx->vCounts.data(), g->ctx->vCounts.size() * 8);
+        put(g->ctx->vDispls.data(), g->ctx->vDispls.size() * 8);
         key.push_back('v');
     }
-    uint64_t head[10] = {uint64_t(g->sig.coll), uint64_t(algo), uint64_t(g->sig.dtype), uint64_t(g->sig.op), g->sig.count,
-        uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1) | (uint64_t(g->sig.root) << 8), g->cfg.cclBytes, g->cfg.align,
+    uint64_t head[10] = {uint64_t(g->ctx->sig.coll), uint64_t(algo), uint64_t(g->ctx->sig.dtype), uint64_t(g->ctx->sig.op), g->ctx->sig.count,
+        uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1) | (uint64_t(g->ctx->sig.root) << 8) | (uint64_t(g->ctx->sig.peer) << 20), g->cfg.cclBytes, g->cfg.align,
         g->cfg.blocksPerCu, g->p};
     put(head, sizeof(head));
-    put(g->send.data(), g->send.size() * sizeof(void *));
-    put(g->recv.data(), g->recv.size() * sizeof(void *));
-    if (g->sig.coll == COLL_ALLTOALLV) {
-        put(g->sendCounts.data(), g->sendCounts.size() * 8);
-        put(g->sdispls.data(), g->sdispls.size() * 8);
-        put(g->recvCounts.data(), g->recvCounts.size() * 8);
-        put(g->rdispls.data(), g->rdispls.size() * 8);
+    put(g->ctx->send.data(), g->ctx->send.size() * sizeof(void *));
+    put(g->ctx->recv.data(), g->ctx->recv.size() * sizeof(void *));
+    if (g->ctx->sig.coll == COLL_ALLTOALLV) {
+        put(g->ctx->sendCounts.data(), g->ctx->sendCounts.size() * 8);
+        put(g->ctx->sdispls.data(), g->ctx->sdispls.size() * 8);
+        put(g->ctx->recvCounts.data(), g->ctx->recvCounts.size() * 8);
+        put(g->ctx->rdispls.data(), g->ctx->rdispls.size() * 8);
     }
     return key;
 }
@@ -361,50 +361,51 @@ std::string CacheKey(const Group *g, int algo)
 HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
 {
     std::unique_ptr<Prepared> pp(new Prepared());
-    const bool reduceColl = g->sig.coll == COLL_ALLREDUCE || g->sig.coll == COLL_REDUCESCATTER || g->sig.coll == COLL_REDUCE;
+    const bool reduceColl = g->ctx->sig.coll == COLL_ALLREDUCE || g->ctx->sig.coll == COLL_REDUCESCATTER || g->ctx->sig.coll == COLL_REDUCE;
     PlanRequest rq;
-    rq.coll = CollKind(g->sig.coll);
+    rq.coll = CollKind(g->ctx->sig.coll);
     rq.algo = Algo(algo);
     rq.p = g->p;
-    rq.count = g->sig.count;
-    rq.root = g->sig.root;
-    rq.unit = DtypeSize(g->sig.dtype);
+    rq.count = g->ctx->sig.count;
+    rq.root = g->ctx->sig.root;
+    rq.peer = g->ctx->sig.peer;
+    rq.unit = DtypeSize(g->ctx->sig.dtype);
     rq.cclBytes = g->cfg.cclBytes;
     rq.align = g->cfg.align;
     rq.alias.assign(g->p, 0);
     for (uint32_t r = 0; r < g->p; r++) {
-        rq.alias[r] = (g->send[r] == g->recv[r]) ? 1 : 0;
+        rq.alias[r] = (g->ctx->send[r] == g->ctx->recv[r]) ? 1 : 0;
     }
-    if (g->sig.variable) {
-        rq.vCounts = g->vCounts;
-        rq.vDispls = g->vDispls;
+    if (g->ctx->sig.variable) {
+        rq.vCounts = g->ctx->vCounts;
+        rq.vDispls = g->ctx->vDispls;
     }
     if (rq.coll == COLL_ALLTOALLV) {
-        rq.sendCounts = g->sendCounts;
-        rq.sdispls = g->sdispls;
-        rq.recvCounts = g->recvCounts;
-        rq.rdispls = g->rdispls;
+        rq.sendCounts = g->ctx->sendCounts;
+        rq.sdispls = g->ctx->sdispls;
+        rq.recvCounts = g->ctx->recvCounts;
+        rq.rdispls = g->ctx->rdispls;
     }
     std::string err;
     int rc = BuildPlan(rq, &pp->plan, &err);
     if (rc != 0) {
-        HCCL_LOG_ERROR("%s: planning failed: %s", CollName(g->sig.coll), err.c_str());
+        HCCL_LOG_ERROR("%s: planning failed: %s", CollName(g->ctx->sig.coll), err.c_str());
         return rc == 1 ? HCCL_E_PARA : HCCL_E_INTERNAL;
     }
     // Buffers of different ranks must not overlap where one of them is written; a send buffer that
     // overlaps a receive buffer other than as an exact in-place pair is staged through scratch.
     bool needStage = false;
     for (uint32_t i = 0; i < g->p; i++) {
-        const char *ri = static_cast<const char *>(g->recv[i]);
+        const char *ri = static_cast<const char *>(g->ctx->recv[i]);
         for (uint32_t j = 0; j < g->p; j++) {
-            const char *rj = static_cast<const char *>(g->recv[j]);
-            const char *sj = static_cast<const char *>(g->send[j]);
+            const char *rj = static_cast<const char *>(g->ctx->recv[j]);
+            const char *sj = static_cast<const char *>(g->ctx->send[j]);
             if (i != j && RangesOverlap(ri, pp->plan.recvBytes[i], rj, pp->plan.recvBytes[j])) {
-                HCCL_LOG_ERROR("%s: receive buffers of rank %u and rank %u overlap", CollName(g->sig.coll), i, j);
+                HCCL_LOG_ERROR("%s: receive buffers of rank %u and rank %u overlap", CollName(g->ctx->sig.coll), i, j);
                 return HCCL_E_PARA;
             }
             if (RangesOverlap(ri, pp->plan.recvBytes[i], sj, pp->plan.sendBytes[j])) {
-                bool exact = (i == j) && ri == sj && (g->sig.coll == COLL_ALLREDUCE || g->sig.coll == COLL_BROADCAST);
+                bool exact = (i == j) && ri == sj && (g->ctx->sig.coll == COLL_ALLREDUCE || g->ctx->sig.coll == COLL_BROADCAST);
                 needStage = needStage || !exact;
             }
         }
@@ -415,7 +416,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         pp->plan = Plan();
         rc = BuildPlan(rq, &pp->plan, &err);
         if (rc != 0) {
-            HCCL_LOG_ERROR("%s: planning (staged) failed: %s", CollName(g->sig.coll), err.c_str());
+            HCCL_LOG_ERROR("%s: planning (staged) failed: %s", CollName(g->ctx->sig.coll), err.c_str());
             return HCCL_E_INTERNAL;
         }
     }
@@ -434,7 +435,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         }
     }
     pp->scratchGen = g->scratchGen;
-    HcclResult r = BuildTables(g, pp.get(), reduceColl, g->sig.dtype, g->sig.op);
+    HcclResult r = BuildTables(g, pp.get(), reduceColl, g->ctx->sig.dtype, g->ctx->sig.op);
     if (r != HCCL_SUCCESS) {
         return r;
     }
@@ -446,7 +447,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         }
     }
     OpInfo &info = pp->info;
-    info.coll = g->sig.coll;
+    info.coll = g->ctx->sig.coll;
     info.algo = algo;
     info.fused = pp->fused ? 1 : 0;
     info.graph = pp->exec ? 1 : 0;
@@ -509,6 +510,7 @@ const char *CollName(int coll)
         case COLL_BROADCAST: return "Broadcast";
         case COLL_REDUCE: return "Reduce";
         case COLL_SCATTER: return "Scatter";
+        case COLL_SENDRECV: return "Send/Recv";
         default: return "?";
     }
 }
@@ -521,10 +523,10 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     if (r != HCCL_SUCCESS) {
         return r;
     }
-    int algo = g->cfg.algo >= 0 ? g->cfg.algo : DefaultAlgo(g->sig.coll);
-    if (g->sig.coll == COLL_ALLTOALLV) {
+    int algo = g->cfg.algo >= 0 ? g->cfg.algo : DefaultAlgo(g->ctx->sig.coll);
+    if (g->ctx->sig.coll == COLL_ALLTOALLV) {
         algo = ALGO_PAIRWISE;
-    } else if (g->sig.coll >= COLL_BROADCAST) {
+    } else if (g->ctx->sig.coll >= COLL_BROADCAST) {
         algo = ALGO_RING;   // one schedule each: ring broadcast, ring reduce, mesh scatter
     } else if (algo == ALGO_PAIRWISE) {
         algo = ALGO_RING;
@@ -566,18 +568,18 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
 
     // Order the launch after everything queued so far on the other ranks' streams, and order those
     // streams after the collective.  Ranks that share the launcher's stream need nothing.
-    hipStream_t ls = g->streams[launcher];
+    hipStream_t ls = g->ctx->streams[launcher];
     bool others = false;
     for (uint32_t k = 0; k < g->p; k++) {
-        if (k == launcher || g->streams[k] == ls) {
+        if (k == launcher || g->ctx->streams[k] == ls) {
             continue;
         }
         bool seen = false;
         for (uint32_t q = 0; q < k; q++) {
-            seen = seen || (q != launcher && g->streams[q] == g->streams[k]);
+            seen = seen || (q != launcher && g->ctx->streams[q] == g->ctx->streams[k]);
         }
         if (!seen) {
-            HIP_OK(hipEventRecord(g->arriveEvents[k], g->streams[k]));
+            HIP_OK(hipEventRecord(g->arriveEvents[k], g->ctx->streams[k]));
             HIP_OK(hipStreamWaitEvent(ls, g->arriveEvents[k], 0));
         }
         others = true;
@@ -594,8 +596,8 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     if (others) {
         HIP_OK(hipEventRecord(g->doneEvent, ls));
         for (uint32_t k = 0; k < g->p; k++) {
-            if (k != launcher && g->streams[k] != ls) {
-                HIP_OK(hipStreamWaitEvent(g->streams[k], g->doneEvent, 0));
+            if (k != launcher && g->ctx->streams[k] != ls) {
+                HIP_OK(hipStreamWaitEvent(g->ctx->streams[k], g->doneEvent, 0));
             }
         }
     }

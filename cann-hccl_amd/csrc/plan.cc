@@ -347,6 +347,17 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
         }
         return 0;
     }
+    if (rq.coll == COLL_SENDRECV) {
+        // one block from the sender's buffer to the receiver's (send_receive.cc: TxAsync / RxAsync pair)
+        if (rq.root >= p || rq.peer >= p) {
+            *err = "send / receive rank out of range";
+            return 1;
+        }
+        EmitCopy(*vp, 0, MkRef(rq.peer, BUF_RECV, 0), MkRef(rq.root, BUF_SEND, 0), rq.count * u);
+        vp->inBytes[rq.root] = rq.count * u;
+        vp->outBytes[rq.peer] = rq.count * u;
+        return 0;
+    }
     if (rq.coll == COLL_BROADCAST || rq.coll == COLL_REDUCE || rq.coll == COLL_SCATTER) {
         if (rq.root >= p) {
             *err = "root out of range";

@@ -23,7 +23,7 @@ namespace hcclamd {
 
 enum CollKind : int {
     COLL_ALLREDUCE = 0, COLL_REDUCESCATTER = 1, COLL_ALLGATHER = 2, COLL_ALLTOALLV = 3,
-    COLL_BROADCAST = 4, COLL_REDUCE = 5, COLL_SCATTER = 6
+    COLL_BROADCAST = 4, COLL_REDUCE = 5, COLL_SCATTER = 6, COLL_SENDRECV = 7
 };
 enum Algo : int { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2, ALGO_PAIRWISE = 3 };
 
@@ -71,7 +71,8 @@ struct PlanRequest {
     Algo algo = ALGO_RING;
     uint32_t p = 1;
     uint64_t count = 0;            // all-reduce: elements; reduce-scatter: recvCount; all-gather: sendCount
-    uint32_t root = 0;             // broadcast / reduce / scatter
+    uint32_t root = 0;             // broadcast / reduce / scatter; send / receive: the sending rank
+    uint32_t peer = 0;             // send / receive: the receiving rank
     uint32_t unit = 4;             // element size in bytes
     uint64_t cclBytes = 200ull << 20;
     uint64_t align = 128;

@@ -10,6 +10,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <condition_variable>
+#include <deque>
 #include <cstdint>
 #include <map>
 #include <memory>
@@ -78,12 +79,31 @@ struct OpSig {
     uint64_t count = 0;
     int dtype = 0, recvType = 0, op = 0;
     int variable = 0;                // 1: reduce-scatter-v / all-gather-v (block tables instead of a count)
+    uint32_t peer = 0;               // send / receive: destination rank (root = source rank)
     uint32_t root = 0;               // broadcast / reduce / scatter
     bool operator==(const OpSig &o) const
     {
         return coll == o.coll && count == o.count && dtype == o.dtype && recvType == o.recvType && op == o.op &&
-            variable == o.variable && root == o.root;
+            variable == o.variable && root == o.root && peer == o.peer;
     }
+};
+
+// Everything one collective needs from its callers.
+struct OpCtx {
+    OpSig sig;
+    std::vector<void *> send, recv;
+    std::vector<hipStream_t> streams;
+    std::vector<uint64_t> sendCounts, sdispls, recvCounts, rdispls;   // p x p (all-to-all-v)
+    std::vector<uint64_t> vCounts, vDispls;                           // p (reduce-scatter-v / all-gather-v)
+};
+
+// A send or receive waiting for its counterpart (matched first-in first-out per (source, destination)).
+struct P2PPending {
+    bool isSend = false;
+    void *buf = nullptr;
+    uint64_t count = 0;
+    int dtype = 0;
+    hipStream_t stream = nullptr;
 };
 
 struct Group;
@@ -110,12 +130,10 @@ struct Group {
     uint32_t arrived = 0;
     uint64_t opSerial = 0;           // bumped whenever a collective is issued or cancelled
     HcclResult lastIssueResult = HCCL_SUCCESS;
-    OpSig sig;
     std::vector<uint8_t> here;
-    std::vector<void *> send, recv;
-    std::vector<hipStream_t> streams;
-    std::vector<uint64_t> sendCounts, sdispls, recvCounts, rdispls;   // p x p (all-to-all-v)
-    std::vector<uint64_t> vCounts, vDispls;                           // p (reduce-scatter-v / all-gather-v)
+    OpCtx pend;                      // what the ranks of the current collective passed
+    OpCtx *ctx = nullptr;            // the operation being issued (the rendezvous, or a matched send / receive)
+    std::map<std::pair<uint32_t, uint32_t>, std::deque<P2PPending>> p2p;
 
     // device resources
     bool deviceReady = false;

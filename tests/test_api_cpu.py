@@ -206,9 +206,24 @@ def test_amd_params(comms):
 
 
 def test_unsupported_entry_points_link_and_refuse(comms):
-    assert L.HcclSend(BUF_A, 4, 4, 1, comms[0], STREAM) == H.HCCL_E_NOT_SUPPORT
-    assert L.HcclSend(BUF_A, 4, 4, 1, None, STREAM) == H.HCCL_E_PTR
     assert L.HcclGetRootInfo(None) == H.HCCL_E_PTR
+    assert L.HcclCommInitClusterInfo(b"ranktable.json", 0, ctypes.byref(ctypes.c_void_p())) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclCommSetMemoryRange(comms[0], BUF_A, 4096, 0, 0) == H.HCCL_E_NOT_SUPPORT
+
+
+def test_send_recv_checks_and_matching(comms):
+    FP32 = H.HCCL_DATA_TYPE_FP32
+    assert L.HcclSend(None, 0, FP32, 1, None, None) == H.HCCL_SUCCESS                       # count 0 first
+    assert L.HcclSend(BUF_A, 4, FP32, 1, None, STREAM) == H.HCCL_E_PTR
+    assert L.HcclSend(None, 4, FP32, 1, comms[0], STREAM) == H.HCCL_E_PTR
+    assert L.HcclSend(BUF_A, 4, FP32, 1, comms[0], None) == H.HCCL_E_PTR
+    assert L.HcclSend(BUF_A, 4, 200, 1, comms[0], STREAM) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclSend(BUF_A, 4, FP32, 7, comms[0], STREAM) == H.HCCL_E_PARA                  # no such rank
+    assert L.HcclRecv(None, 4, FP32, 1, comms[0], STREAM) == H.HCCL_E_PTR
+    assert L.HcclBatchSendRecv(None, 1, comms[0], STREAM) == H.HCCL_E_PTR
+    # a send waits for its receive; a receive that disagrees on the count is refused
+    assert L.HcclSend(BUF_A, 4, FP32, 1, comms[0], STREAM) == H.HCCL_SUCCESS
+    assert L.HcclRecv(BUF_B, 8, FP32, 0, comms[1], STREAM) == H.HCCL_E_PARA
 
 
 def test_rooted_entry_checks(comms):

@@ -518,3 +518,39 @@ def test_one_thread_per_rank_blocking_arrival(orc):
             assert np.array_equal(gh.to_host(recvs[r], FP32), want[r]), r
     finally:
         g.close()
+
+
+def test_send_recv_and_batch():
+    p, n = 4, 250007
+    g = gh.Group(p)
+    try:
+        rng = np.random.default_rng(5)
+        data = [rng.integers(-1000, 1000, n).astype(np.int32) for _ in range(p)]
+        src = [gh.to_dev(x) for x in data]
+        dst = [gh.to_dev(np.zeros(n, np.int32)) for _ in range(p)]
+        streams = [torch.cuda.Stream() for _ in range(p)]
+        torch.cuda.synchronize()
+        # ring shift with plain send / receive, receives posted first on odd ranks
+        for r in range(p):
+            nxt, prv = (r + 1) % p, (r - 1) % p
+            if r % 2:
+                H.recv(g.comms[r], dst[r].data_ptr(), n, INT32, prv, streams[r].cuda_stream)
+                H.send(g.comms[r], src[r].data_ptr(), n, INT32, nxt, streams[r].cuda_stream)
+            else:
+                H.send(g.comms[r], src[r].data_ptr(), n, INT32, nxt, streams[r].cuda_stream)
+                H.recv(g.comms[r], dst[r].data_ptr(), n, INT32, prv, streams[r].cuda_stream)
+        torch.cuda.synchronize()
+        for r in range(p):
+            assert np.array_equal(gh.to_host(dst[r], INT32), data[(r - 1) % p]), r
+        # the same exchange in the other direction as one batch per rank
+        for t in dst:
+            t.zero_()
+        torch.cuda.synchronize()
+        for r in range(p):
+            H.batch_send_recv(g.comms[r], [(True, src[r].data_ptr(), n, INT32, (r - 1) % p),
+                                           (False, dst[r].data_ptr(), n, INT32, (r + 1) % p)], streams[r].cuda_stream)
+        torch.cuda.synchronize()
+        for r in range(p):
+            assert np.array_equal(gh.to_host(dst[r], INT32), data[(r + 1) % p]), r
+    finally:
+        g.close()
