@@ -49,6 +49,57 @@ class HcclAmdOpInfo(ctypes.Structure):
                 ("scratchBytes", ctypes.c_uint64)]
 
 
+class HcclCommConfig(ctypes.Structure):
+    _fields_ = [("reserved", ctypes.c_char * 24), ("hcclBufferSize", ctypes.c_uint32), ("hcclDeterministic", ctypes.c_uint32),
+                ("hcclCommName", ctypes.c_char * 128), ("hcclUdi", ctypes.c_char * 128), ("hcclOpExpansionMode", ctypes.c_uint32),
+                ("hcclRdmaTrafficClass", ctypes.c_uint32), ("hcclRdmaServiceLevel", ctypes.c_uint32)]
+
+
+def comm_config_init():
+    """What the inline HcclCommConfigInit of hccl.h writes."""
+    cfg = HcclCommConfig()
+    hdr = ctypes.cast(ctypes.byref(cfg), ctypes.POINTER(ctypes.c_uint64))
+    hdr[0] = ctypes.sizeof(HcclCommConfig)
+    hdr[1] = 0xf0f0f0f0 | (5 << 32)          # magic word, version
+    hdr[2] = 0
+    cfg.hcclBufferSize = 0xffffffff
+    cfg.hcclDeterministic = 0xffffffff
+    cfg.hcclOpExpansionMode = 0
+    cfg.hcclRdmaTrafficClass = 0xffffffff
+    cfg.hcclRdmaServiceLevel = 0xffffffff
+    return cfg
+
+
+def comm_init_root_info(n_ranks, config=None):
+    """HcclGetRootInfo + one HcclCommInitRootInfo[Config] per rank; returns the handles."""
+    info = ctypes.create_string_buffer(4108)
+    _check("HcclGetRootInfo", lib().HcclGetRootInfo(info))
+    comms = []
+    for r in range(n_ranks):
+        c = ctypes.c_void_p()
+        if config is None:
+            _check("HcclCommInitRootInfo", lib().HcclCommInitRootInfo(n_ranks, info, r, ctypes.byref(c)))
+        else:
+            _check("HcclCommInitRootInfoConfig", lib().HcclCommInitRootInfoConfig(n_ranks, info, r, ctypes.byref(config),
+                                                                                  ctypes.byref(c)))
+        comms.append(c)
+    return comms
+
+
+def create_sub_comm(comms, rank_ids, sub_comm_id, config=None):
+    """HcclCreateSubCommConfig for every member; returns the sub-communicator handles in rank_ids order."""
+    cfg = config or comm_config_init()
+    ids = (ctypes.c_uint32 * len(rank_ids))(*rank_ids)
+    subs = []
+    for pos, r in enumerate(rank_ids):
+        parent = ctypes.c_void_p(comms[r].value)
+        sub = ctypes.c_void_p()
+        _check("HcclCreateSubCommConfig", lib().HcclCreateSubCommConfig(ctypes.byref(parent), len(rank_ids), ids, sub_comm_id,
+                                                                         pos, ctypes.byref(cfg), ctypes.byref(sub)))
+        subs.append(sub)
+    return subs
+
+
 class HcclSendRecvItem(ctypes.Structure):
     _fields_ = [("sendRecvType", ctypes.c_int32), ("buf", ctypes.c_void_p), ("count", ctypes.c_uint64),
                 ("dataType", ctypes.c_int32), ("remoteRank", ctypes.c_uint32)]
@@ -90,6 +141,10 @@ def lib():
     L.HcclBroadcast.argtypes = [vp, u64, i32, u32, vp, vp]
     L.HcclReduce.argtypes = [vp, vp, u64, i32, i32, u32, vp, vp]
     L.HcclScatter.argtypes = [vp, vp, u64, i32, u32, vp, vp]
+    L.HcclGetRootInfo.argtypes = [vp]
+    L.HcclCommInitRootInfo.argtypes = [u32, vp, u32, ctypes.POINTER(vp)]
+    L.HcclCommInitRootInfoConfig.argtypes = [u32, vp, u32, vp, ctypes.POINTER(vp)]
+    L.HcclCreateSubCommConfig.argtypes = [ctypes.POINTER(vp), u32, ctypes.POINTER(u32), u64, u32, vp, ctypes.POINTER(vp)]
     L.HcclSend.argtypes = [vp, u64, i32, u32, vp, vp]
     L.HcclRecv.argtypes = [vp, u64, i32, u32, vp, vp]
     L.HcclBatchSendRecv.argtypes = [ctypes.POINTER(HcclSendRecvItem), u32, vp, vp]

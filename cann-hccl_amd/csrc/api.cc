@@ -7,6 +7,7 @@
 #include <chrono>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <set>
 #include <string>
 #include <vector>
@@ -136,6 +137,123 @@ void ApplyEnv(GroupConfig *cfg)
             cfg->arriveTimeoutMs = uint32_t(v);
         }
     }
+}
+
+// HcclCommConfig loading, as FW/communicator/comm_config.cc:29-178: size-prefixed copy, magic word,
+// fields gated by version (>= 1 buffer size and deterministic, >= 2 name).
+struct ConfigHeader {
+    size_t size;
+    uint32_t magicWord;
+    uint32_t version;
+    uint64_t reserved;
+};
+
+HcclResult LoadCommConfig(const HcclCommConfig *user, GroupConfig *cfg, std::string *name)
+{
+    HcclCommConfig local;
+    std::memset(&local, 0, sizeof(local));   // bytes the caller's (older, smaller) struct does not have stay zero
+    size_t size = *reinterpret_cast<const size_t *>(user);
+    std::memcpy(&local, user, std::min(size, sizeof(local)));
+    const ConfigHeader *h = reinterpret_cast<const ConfigHeader *>(&local);
+    if (h->magicWord != HCCL_COMM_CONFIG_MAGIC_WORD) {
+        HCCL_LOG_ERROR("comm config: bad magic word 0x%x; initialise the struct with HcclCommConfigInit()", h->magicWord);
+        return HCCL_E_PARA;
+    }
+    if (h->version >= 1) {
+        if (local.hcclBufferSize != HCCL_COMM_BUFFSIZE_CONFIG_NOT_SET) {
+            if (local.hcclBufferSize < 1) {
+                HCCL_LOG_ERROR("comm config: hcclBufferSize must be at least 1 (MiB)");
+                return HCCL_E_PARA;
+            }
+            cfg->cclBytes = uint64_t(local.hcclBufferSize) << 20;
+        }
+        if (local.hcclDeterministic != HCCL_COMM_DETERMINISTIC_CONFIG_NOT_SET) {
+            if (local.hcclDeterministic > 1) {
+                HCCL_LOG_ERROR("comm config: hcclDeterministic must be 0 or 1");
+                return HCCL_E_PARA;
+            }
+            cfg->deterministic = local.hcclDeterministic == 1;
+        }
+    }
+    if (h->version >= 2 && local.hcclCommName[0] != '\0') {
+        local.hcclCommName[COMM_NAME_MAX_LENGTH - 1] = '\0';
+        *name = local.hcclCommName;
+    }
+    if (h->version >= 4 && local.hcclOpExpansionMode > 3) {
+        HCCL_LOG_WARN("comm config: unknown hcclOpExpansionMode %u, using the default", local.hcclOpExpansionMode);
+    }
+    return HCCL_SUCCESS;
+}
+
+Group *NewGroup(uint32_t nRanks)
+{
+    Group *g = new Group();
+    g->p = nRanks;
+    ApplyEnv(&g->cfg);
+    g->here.assign(nRanks, 0);
+    g->pend.send.assign(nRanks, nullptr);
+    g->pend.recv.assign(nRanks, nullptr);
+    g->pend.streams.assign(nRanks, nullptr);
+    g->ctx = &g->pend;
+    char nm[64];
+    std::snprintf(nm, sizeof(nm), "hccl_world_group_%p", static_cast<void *>(g));
+    g->name = nm;
+    g->comms.resize(nRanks);
+    return g;
+}
+
+// Groups that are being assembled rank by rank (root-info and sub-communicator creation), by key.
+std::map<std::string, Group *> g_forming;
+uint64_t g_rootInfoSerial = 0;
+
+// Joins rank `rank` to the group forming under `key` (created on first use).
+HcclResult JoinFormingGroup(const std::string &key, uint32_t nRanks, uint32_t rank, const HcclCommConfig *config, HcclComm *out)
+{
+    std::lock_guard<std::mutex> reg(g_registryMutex);
+    Group *g = nullptr;
+    auto it = g_forming.find(key);
+    if (it == g_forming.end()) {
+        if (nRanks > kMaxRanks) {
+            HCCL_LOG_ERROR("at most %u ranks per group", kMaxRanks);
+            return HCCL_E_PARA;
+        }
+        g = NewGroup(nRanks);
+        g->name = key;
+        if (config != nullptr) {
+            HcclResult r = LoadCommConfig(config, &g->cfg, &g->name);
+            if (r != HCCL_SUCCESS) {
+                delete g;
+                return r;
+            }
+        }
+        g_forming[key] = g;
+        g_groups.insert(g);
+    } else {
+        g = it->second;
+        if (g->p != nRanks) {
+            HCCL_LOG_ERROR("rank %u joins with %u ranks, the group was created with %u", rank, nRanks, g->p);
+            return HCCL_E_PARA;
+        }
+    }
+    std::lock_guard<std::mutex> lock(g->m);
+    if (g->comms[rank]) {
+        HCCL_LOG_ERROR("rank %u of this group exists already", rank);
+        return HCCL_E_PARA;
+    }
+    std::unique_ptr<Comm> c(new Comm());
+    c->group = g;
+    c->rank = rank;
+    *out = c.get();
+    g->comms[rank] = std::move(c);
+    g->liveComms++;
+    bool complete = true;
+    for (auto &m : g->comms) {
+        complete = complete && bool(m);
+    }
+    if (complete) {
+        g_forming.erase(key);
+    }
+    return HCCL_SUCCESS;
 }
 
 struct InUse {
@@ -322,22 +440,13 @@ HcclResult HcclCommInitAll(uint32_t ndev, int32_t *devices, HcclComm *comms)
         HCCL_LOG_ERROR("HcclCommInitAll: at most %u ranks per group", kMaxRanks);
         return HCCL_E_PARA;
     }
-    Group *g = new Group();
-    g->p = ndev;
-    ApplyEnv(&g->cfg);
-    g->here.assign(ndev, 0);
-    g->pend.send.assign(ndev, nullptr);
-    g->pend.recv.assign(ndev, nullptr);
-    g->pend.streams.assign(ndev, nullptr);
-    char nm[64];
-    std::snprintf(nm, sizeof(nm), "hccl_world_group_%p", static_cast<void *>(g));
-    g->name = nm;
+    Group *g = NewGroup(ndev);
     for (uint32_t r = 0; r < ndev; r++) {
         std::unique_ptr<Comm> c(new Comm());
         c->group = g;
         c->rank = r;
         comms[r] = c.get();
-        g->comms.push_back(std::move(c));
+        g->comms[r] = std::move(c);
     }
     g->liveComms = ndev;
     std::lock_guard<std::mutex> reg(g_registryMutex);
@@ -380,6 +489,9 @@ HcclResult HcclCommDestroy(HcclComm comm)
         {
             std::lock_guard<std::mutex> reg(g_registryMutex);
             g_groups.erase(g);
+            for (auto it = g_forming.begin(); it != g_forming.end();) {
+                it = (it->second == g) ? g_forming.erase(it) : std::next(it);
+            }
         }
         delete g;
     }
@@ -1078,6 +1190,98 @@ HcclResult HcclBatchSendRecv(HcclSendRecvItem *sendRecvInfo, uint32_t itemNum, H
     return HCCL_SUCCESS;
 }
 
+// ---- communicators assembled rank by rank --------------------------------------------------------------------
+
+// op_base.cc:794-843.  The token names a group that HcclCommInitRootInfo calls of this process join.
+HcclResult HcclGetRootInfo(HcclRootInfo *rootInfo)
+{
+    CHK_PTR(rootInfo);
+    std::lock_guard<std::mutex> reg(g_registryMutex);
+    std::memset(rootInfo->internal, 0, HCCL_ROOT_INFO_BYTES);
+    std::snprintf(rootInfo->internal, 128, "hccl_amd_root_%llu", static_cast<unsigned long long>(++g_rootInfoSerial));
+    return HCCL_SUCCESS;
+}
+
+// op_base.cc:1055-1120.  One call per rank, from any thread of this process; all ranks run on the current GPU.
+HcclResult HcclCommInitRootInfo(uint32_t nRanks, const HcclRootInfo *rootInfo, uint32_t rank, HcclComm *comm)
+{
+    CHK_PTR(rootInfo);
+    if (nRanks == 0) {
+        HCCL_LOG_ERROR("HcclCommInitRootInfo: nRanks must be greater than 0");
+        return HCCL_E_PARA;
+    }
+    if (rank >= nRanks) {
+        HCCL_LOG_ERROR("HcclCommInitRootInfo: rank %u is out of range", rank);
+        return HCCL_E_PARA;
+    }
+    CHK_PTR(comm);
+    std::string key(rootInfo->internal, strnlen(rootInfo->internal, 127));
+    if (key.compare(0, 14, "hccl_amd_root_") != 0) {
+        HCCL_LOG_ERROR("HcclCommInitRootInfo: the root info was not produced by HcclGetRootInfo of this process");
+        return HCCL_E_PARA;
+    }
+    return JoinFormingGroup(key, nRanks, rank, nullptr, comm);
+}
+
+// op_base.cc:1122-1202; configuration rules of comm_config.cc (the first rank's configuration applies).
+HcclResult HcclCommInitRootInfoConfig(uint32_t nRanks, const HcclRootInfo *rootInfo, uint32_t rank,
+    const HcclCommConfig *config, HcclComm *comm)
+{
+    CHK_PTR(rootInfo);
+    if (nRanks == 0 || rank >= nRanks) {
+        return HCCL_E_PARA;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(config);
+    std::string key(rootInfo->internal, strnlen(rootInfo->internal, 127));
+    if (key.compare(0, 14, "hccl_amd_root_") != 0) {
+        return HCCL_E_PARA;
+    }
+    GroupConfig probe;
+    std::string name;
+    HcclResult r = LoadCommConfig(config, &probe, &name);   // every rank's configuration is validated
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    return JoinFormingGroup(key, nRanks, rank, config, comm);
+}
+
+// op_base.cc:730-792.  Every member rank calls with the same rankIds and subCommId; a rank outside the
+// sub-communicator passes rankIds == nullptr and subCommId == 0xFFFFFFFF and gets nothing.
+HcclResult HcclCreateSubCommConfig(HcclComm *comm, uint32_t rankNum, uint32_t *rankIds, uint64_t subCommId,
+    uint32_t subCommRankId, HcclCommConfig *config, HcclComm *subComm)
+{
+    constexpr uint64_t kInvalidSubCommId = 0xFFFFFFFFull;
+    CHK_PTR(subComm);
+    if (rankIds == nullptr && subCommId == kInvalidSubCommId) {
+        return HCCL_SUCCESS;
+    }
+    if (rankIds == nullptr || subCommId == kInvalidSubCommId) {
+        HCCL_LOG_ERROR("HcclCreateSubCommConfig: rankIds and subCommId must both be valid or both be invalid");
+        return HCCL_E_PARA;
+    }
+    if (rankNum == 0 || subCommRankId >= rankNum) {
+        return HCCL_E_PARA;
+    }
+    CHK_PTR(config);
+    CHK_PTR(comm);
+    Comm *parent = AsComm(*comm);
+    if (parent == nullptr) {
+        return HCCL_E_PTR;
+    }
+    if (rankNum > parent->group->p || rankIds[subCommRankId] != parent->rank) {
+        HCCL_LOG_ERROR("HcclCreateSubCommConfig: rankIds[subCommRankId] must be the calling rank");
+        return HCCL_E_PARA;
+    }
+    GroupConfig probe;
+    std::string name;
+    if (LoadCommConfig(config, &probe, &name) != HCCL_SUCCESS) {
+        return HCCL_E_PARA;
+    }
+    std::string key = parent->group->name + "_sub_" + std::to_string(subCommId);
+    return JoinFormingGroup(key, rankNum, subCommRankId, config, subComm);
+}
+
 // ---- extension ----------------------------------------------------------------------------------------
 
 HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
@@ -1235,33 +1439,6 @@ HcclResult HcclCommInitClusterInfo(const char *clusterInfo, uint32_t, HcclComm *
 HcclResult HcclCommInitClusterInfoConfig(const char *clusterInfo, uint32_t, HcclCommConfig *config, HcclComm *comm)
 {
     CHK_PTR(clusterInfo);
-    CHK_PTR(config);
-    CHK_PTR(comm);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclCreateSubCommConfig(HcclComm *comm, uint32_t, uint32_t *, uint64_t, uint32_t, HcclCommConfig *config,
-    HcclComm *subComm)
-{
-    CHK_PTR(comm);
-    CHK_PTR(config);
-    CHK_PTR(subComm);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclGetRootInfo(HcclRootInfo *rootInfo)
-{
-    CHK_PTR(rootInfo);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclCommInitRootInfo(uint32_t, const HcclRootInfo *rootInfo, uint32_t, HcclComm *comm)
-{
-    CHK_PTR(rootInfo);
-    CHK_PTR(comm);
-    return HCCL_E_NOT_SUPPORT;
-}
-HcclResult HcclCommInitRootInfoConfig(uint32_t, const HcclRootInfo *rootInfo, uint32_t, const HcclCommConfig *config,
-    HcclComm *comm)
-{
-    CHK_PTR(rootInfo);
     CHK_PTR(config);
     CHK_PTR(comm);
     return HCCL_E_NOT_SUPPORT;

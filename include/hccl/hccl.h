@@ -124,32 +124,52 @@ inline void HcclCommConfigInit(HcclCommConfig *config)
     config->hcclRdmaServiceLevel = HCCL_COMM_SERVICE_LEVEL_CONFIG_NOT_SET;
 }
 
-/* ---- declared so existing binaries link; outside the single-GPU data path ------------------- */
-/* Cluster bootstrap, rooted collectives, point-to-point and virtual-memory registration need
- * more than one device or are not on the per-rank data path; each returns HCCL_E_NOT_SUPPORT
- * after the reference's own null-pointer checks.  decl inc/hccl/hccl.h:30-92,146,196,270-284,
- * 343,386,446-471. */
-extern HcclResult HcclCommInitClusterInfo(const char *clusterInfo, uint32_t rank, HcclComm *comm);
-extern HcclResult HcclCommInitClusterInfoConfig(const char *clusterInfo, uint32_t rank,
-    HcclCommConfig *config, HcclComm *comm);
-extern HcclResult HcclCreateSubCommConfig(HcclComm *comm, uint32_t rankNum, uint32_t *rankIds,
-    uint64_t subCommId, uint32_t subCommRankId, HcclCommConfig *config, HcclComm *subComm);
-extern HcclResult HcclGetRootInfo(HcclRootInfo *rootInfo);
-extern HcclResult HcclCommInitRootInfo(uint32_t nRanks, const HcclRootInfo *rootInfo, uint32_t rank, HcclComm *comm);
-extern HcclResult HcclCommInitRootInfoConfig(uint32_t nRanks, const HcclRootInfo *rootInfo, uint32_t rank,
-    const HcclCommConfig *config, HcclComm *comm);
+/* ---- rooted collectives and point to point --------------------------------------------------------- */
+
+/* Ring broadcast: buf is the source on the root, the destination elsewhere.
+ * decl inc/hccl/hccl.h:146, impl op_base.cc:1433. */
 extern HcclResult HcclBroadcast(void *buf, uint64_t count, HcclDataType dataType, uint32_t root, HcclComm comm,
     aclrtStream stream);
+/* Ring reduce towards the root; recvBuf is written on the root only.
+ * decl inc/hccl/hccl.h:343, impl op_base.cc:2737. */
+extern HcclResult HcclReduce(void *sendBuf, void *recvBuf, uint64_t count, HcclDataType dataType,
+    HcclReduceOp op, uint32_t root, HcclComm comm, aclrtStream stream);
+/* The root's sendBuf holds p blocks of recvCount elements; rank i receives block i (sendBuf may be
+ * null elsewhere).  decl inc/hccl/hccl.h:196, impl op_base.cc:1720. */
 extern HcclResult HcclScatter(void *sendBuf, void *recvBuf, uint64_t recvCount, HcclDataType dataType, uint32_t root,
     HcclComm comm, aclrtStream stream);
+/* A send completes with the matching receive of the destination rank (first in, first out per pair
+ * of ranks); counts and types must agree.  decl inc/hccl/hccl.h:270 / :284 / :386,
+ * impl op_base.cc:1974 / :2056 / :3428. */
 extern HcclResult HcclSend(void *sendBuf, uint64_t count, HcclDataType dataType, uint32_t destRank,
     HcclComm comm, aclrtStream stream);
 extern HcclResult HcclRecv(void *recvBuf, uint64_t count, HcclDataType dataType, uint32_t srcRank,
     HcclComm comm, aclrtStream stream);
-extern HcclResult HcclReduce(void *sendBuf, void *recvBuf, uint64_t count, HcclDataType dataType,
-    HcclReduceOp op, uint32_t root, HcclComm comm, aclrtStream stream);
 extern HcclResult HcclBatchSendRecv(HcclSendRecvItem *sendRecvInfo, uint32_t itemNum, HcclComm comm,
     aclrtStream stream);
+
+/* ---- communicators assembled rank by rank ---------------------------------------------------------- */
+
+/* HcclGetRootInfo makes a token; nRanks calls of HcclCommInitRootInfo[Config] with that token, one
+ * per rank and all from this process, form one group on the current GPU.  The Config variant reads
+ * hcclBufferSize (MiB), hcclDeterministic and hcclCommName from a struct prepared with
+ * HcclCommConfigInit.  decl inc/hccl/hccl.h:67 / :79 / :92, impl op_base.cc:794 / :1111 / :1192. */
+extern HcclResult HcclGetRootInfo(HcclRootInfo *rootInfo);
+extern HcclResult HcclCommInitRootInfo(uint32_t nRanks, const HcclRootInfo *rootInfo, uint32_t rank, HcclComm *comm);
+extern HcclResult HcclCommInitRootInfoConfig(uint32_t nRanks, const HcclRootInfo *rootInfo, uint32_t rank,
+    const HcclCommConfig *config, HcclComm *comm);
+/* Sub-communicator over the ranks rankIds[0..rankNum) of an existing one; every member calls with
+ * its position subCommRankId.  decl inc/hccl/hccl.h:58, impl op_base.cc:730. */
+extern HcclResult HcclCreateSubCommConfig(HcclComm *comm, uint32_t rankNum, uint32_t *rankIds,
+    uint64_t subCommId, uint32_t subCommRankId, HcclCommConfig *config, HcclComm *subComm);
+
+/* ---- declared so existing binaries link; outside the single-GPU data path ------------------- */
+/* Rank-table bootstrap and virtual-memory registration concern several devices or the Ascend
+ * memory manager; each returns HCCL_E_NOT_SUPPORT after the reference's own null-pointer checks.
+ * decl inc/hccl/hccl.h:30-43,446-471. */
+extern HcclResult HcclCommInitClusterInfo(const char *clusterInfo, uint32_t rank, HcclComm *comm);
+extern HcclResult HcclCommInitClusterInfoConfig(const char *clusterInfo, uint32_t rank,
+    HcclCommConfig *config, HcclComm *comm);
 extern HcclResult HcclCommSetMemoryRange(HcclComm comm, void *baseVirPtr, size_t size, size_t alignment,
     uint64_t flags);
 extern HcclResult HcclCommUnsetMemoryRange(HcclComm comm, void *baseVirPtr);

@@ -206,7 +206,6 @@ def test_amd_params(comms):
 
 
 def test_unsupported_entry_points_link_and_refuse(comms):
-    assert L.HcclGetRootInfo(None) == H.HCCL_E_PTR
     assert L.HcclCommInitClusterInfo(b"ranktable.json", 0, ctypes.byref(ctypes.c_void_p())) == H.HCCL_E_NOT_SUPPORT
     assert L.HcclCommSetMemoryRange(comms[0], BUF_A, 4096, 0, 0) == H.HCCL_E_NOT_SUPPORT
 
@@ -254,3 +253,65 @@ def test_no_gpu_means_loud_failure(comms):
     assert codes[:3] == [0, 0, 0] and codes[3] == H.HCCL_E_RUNTIME          # the issuing rank reports it
     err = ctypes.c_int32(0)
     assert L.HcclGetCommAsyncError(comms[0], ctypes.byref(err)) == 0 and err.value == H.HCCL_E_RUNTIME
+
+
+def test_root_info_init_and_comm_config():
+    assert L.HcclGetRootInfo(None) == H.HCCL_E_PTR
+    comms = H.comm_init_root_info(3)
+    n, r = ctypes.c_uint32(), ctypes.c_uint32()
+    for i, c in enumerate(comms):
+        assert L.HcclGetRankSize(c, ctypes.byref(n)) == 0 and n.value == 3
+        assert L.HcclGetRankId(c, ctypes.byref(r)) == 0 and r.value == i
+    H.comm_destroy(comms)
+    # argument rules (op_base.cc:1055-1110): rank within range, one handle per rank, same size on every rank
+    info = ctypes.create_string_buffer(4108)
+    assert L.HcclGetRootInfo(info) == 0
+    c = ctypes.c_void_p()
+    assert L.HcclCommInitRootInfo(0, info, 0, ctypes.byref(c)) == H.HCCL_E_PARA
+    assert L.HcclCommInitRootInfo(2, info, 2, ctypes.byref(c)) == H.HCCL_E_PARA
+    assert L.HcclCommInitRootInfo(2, None, 0, ctypes.byref(c)) == H.HCCL_E_PTR
+    assert L.HcclCommInitRootInfo(2, info, 0, None) == H.HCCL_E_PTR
+    assert L.HcclCommInitRootInfo(2, info, 0, ctypes.byref(c)) == 0
+    d = ctypes.c_void_p()
+    assert L.HcclCommInitRootInfo(2, info, 0, ctypes.byref(d)) == H.HCCL_E_PARA       # rank 0 exists
+    assert L.HcclCommInitRootInfo(3, info, 1, ctypes.byref(d)) == H.HCCL_E_PARA       # other group size
+    assert L.HcclCommInitRootInfo(2, ctypes.create_string_buffer(4108), 1, ctypes.byref(d)) == H.HCCL_E_PARA   # foreign token
+    assert L.HcclCommDestroy(c) == 0
+    # configuration rules (comm_config.cc:29-178)
+    cfg = H.comm_config_init()
+    cfg.hcclBufferSize = 16
+    cfg.hcclDeterministic = 1
+    cfg.hcclCommName = b"tensor_parallel_0"
+    comms = H.comm_init_root_info(2, cfg)
+    name = ctypes.create_string_buffer(128)
+    assert L.HcclGetCommName(comms[0], name) == 0 and name.value == b"tensor_parallel_0"
+    H.comm_destroy(comms)
+    for field, value in (("hcclBufferSize", 0), ("hcclDeterministic", 2)):
+        bad = H.comm_config_init()
+        setattr(bad, field, value)
+        info = ctypes.create_string_buffer(4108)
+        assert L.HcclGetRootInfo(info) == 0
+        assert L.HcclCommInitRootInfoConfig(2, info, 0, ctypes.byref(bad), ctypes.byref(c)) == H.HCCL_E_PARA
+    raw = H.HcclCommConfig()                                                          # never initialised: no magic word
+    assert L.HcclCommInitRootInfoConfig(2, info, 0, ctypes.byref(raw), ctypes.byref(c)) == H.HCCL_E_PARA
+    assert L.HcclCommInitRootInfoConfig(2, info, 0, None, ctypes.byref(c)) == H.HCCL_E_PTR
+
+
+def test_sub_communicator(comms):
+    subs = H.create_sub_comm(comms, [1, 3], 7)
+    n, r = ctypes.c_uint32(), ctypes.c_uint32()
+    for pos, sc in enumerate(subs):
+        assert L.HcclGetRankSize(sc, ctypes.byref(n)) == 0 and n.value == 2
+        assert L.HcclGetRankId(sc, ctypes.byref(r)) == 0 and r.value == pos
+    H.comm_destroy(subs)
+    cfg = H.comm_config_init()
+    out = ctypes.c_void_p()
+    parent = ctypes.c_void_p(comms[0].value)
+    ids = (ctypes.c_uint32 * 2)(1, 3)
+    # a rank outside the sub-communicator passes no list and the invalid id: nothing happens
+    assert L.HcclCreateSubCommConfig(ctypes.byref(parent), 0, None, 0xFFFFFFFF, 0, ctypes.byref(cfg), ctypes.byref(out)) == 0
+    assert out.value is None
+    assert L.HcclCreateSubCommConfig(ctypes.byref(parent), 2, None, 5, 0, ctypes.byref(cfg), ctypes.byref(out)) == H.HCCL_E_PARA
+    assert L.HcclCreateSubCommConfig(ctypes.byref(parent), 2, ids, 5, 2, ctypes.byref(cfg), ctypes.byref(out)) == H.HCCL_E_PARA
+    assert L.HcclCreateSubCommConfig(ctypes.byref(parent), 2, ids, 5, 0, ctypes.byref(cfg), ctypes.byref(out)) == H.HCCL_E_PARA  # rank 0 is not rankIds[0]
+    assert L.HcclCreateSubCommConfig(ctypes.byref(parent), 2, ids, 5, 0, ctypes.byref(cfg), None) == H.HCCL_E_PTR

@@ -554,3 +554,36 @@ def test_send_recv_and_batch():
             assert np.array_equal(gh.to_host(dst[r], INT32), data[(r + 1) % p]), r
     finally:
         g.close()
+
+
+def test_root_info_comms_config_and_sub_comm(orc):
+    # communicators assembled rank by rank, buffer size from HcclCommConfig (it sets the chunk plan), and a sub-communicator
+    p, n = 8, 300000
+    cfg = H.comm_config_init()
+    cfg.hcclBufferSize = 1                      # 1 MiB: 300000 fp32 = 1.14 MiB -> two chunks
+    comms = H.comm_init_root_info(p, cfg)
+    stream = torch.cuda.Stream()
+    try:
+        ins = _ins(FP32, p, n, 77)
+        want = orc.allreduce(ins, FP32, SUM, ccl_bytes=1 << 20)
+        assert not np.array_equal(want[0], orc.allreduce(ins, FP32, SUM)[0])      # the chunk plan matters for fp32
+        sends = [gh.to_dev(x) for x in ins]
+        recvs = [gh.empty_dev(n * 4) for _ in range(p)]
+        torch.cuda.synchronize()
+        H.all_reduce(comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, stream.cuda_stream)
+        stream.synchronize()
+        for r in range(p):
+            assert np.array_equal(gh.to_host(recvs[r], FP32), want[r]), r
+        members = [1, 2, 5, 6]
+        subs = H.create_sub_comm(comms, members, 3)
+        want = orc.allreduce([ins[r] for r in members], FP32, SUM)
+        H.all_reduce(subs, [sends[r].data_ptr() for r in members], [recvs[r].data_ptr() for r in members], n, FP32, SUM,
+                     stream.cuda_stream)
+        stream.synchronize()
+        for pos, r in enumerate(members):
+            assert np.array_equal(gh.to_host(recvs[r], FP32), want[pos]), r
+        torch.cuda.synchronize()
+        H.comm_destroy(subs)
+    finally:
+        torch.cuda.synchronize()
+        H.comm_destroy(comms)
