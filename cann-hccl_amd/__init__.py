@@ -31,7 +31,7 @@ ALGO_RING, ALGO_MESH, ALGO_RHD, ALGO_PAIRWISE = range(4)
 
 # Every symbol include/hccl/hccl.h and include/hccl/hccl_amd_ext.h declare.
 EXPORTS = [
-    "HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAlltoAllV", "HcclAlltoAll", "HcclReduceScatterV",
+    "HcclAllReduce", "HcclReduceScatter", "HcclAllGather", "HcclAlltoAllV", "HcclAlltoAll", "HcclAlltoAllVC", "HcclReduceScatterV",
     "HcclAllGatherV", "HcclBarrier", "HcclCommInitAll", "HcclCommDestroy", "HcclGetRankSize", "HcclGetRankId",
     "HcclGetCommName", "HcclSetConfig", "HcclGetConfig", "HcclGetCommAsyncError", "HcclGetErrorString",
     "HcclGetCommConfigCapability", "HcclCommSuspend", "HcclCommResume", "HcclCommInitClusterInfo",
@@ -135,6 +135,7 @@ def lib():
     L.HcclAllGather.argtypes = [vp, vp, u64, i32, vp, vp]
     L.HcclAlltoAllV.argtypes = [vp, vp, vp, i32, vp, vp, vp, i32, vp, vp]
     L.HcclAlltoAll.argtypes = [vp, u64, i32, vp, u64, i32, vp, vp]
+    L.HcclAlltoAllVC.argtypes = [vp, vp, i32, vp, i32, vp, vp]
     L.HcclReduceScatterV.argtypes = [vp, vp, vp, vp, u64, i32, i32, vp, vp]
     L.HcclAllGatherV.argtypes = [vp, u64, vp, vp, vp, i32, vp, vp]
     L.HcclBarrier.argtypes = [vp, vp]
@@ -217,6 +218,14 @@ def all_gather(comms, sends, recvs, send_count, dtype, stream):
 def all_to_all(comms, sends, recvs, count, dtype, stream):
     for c, s, r in zip(comms, sends, recvs):
         _check("HcclAlltoAll", lib().HcclAlltoAll(s, count, dtype, r, count, dtype, c, stream))
+
+
+def all_to_all_vc(comms, sends, recvs, matrix, dtype, stream):
+    """matrix[i][j] = elements rank i sends to rank j (the same table goes to every rank)."""
+    p = len(comms)
+    flat = (ctypes.c_uint64 * (p * p))(*[int(matrix[i][j]) for i in range(p) for j in range(p)])
+    for c, s, r in zip(comms, sends, recvs):
+        _check("HcclAlltoAllVC", lib().HcclAlltoAllVC(s, flat, dtype, r, dtype, c, stream))
 
 
 def reduce_scatter_v(comms, sends, counts, displs, recvs, dtype, op, stream):

@@ -953,6 +953,68 @@ HcclResult HcclAlltoAll(const void *sendBuf, uint64_t sendCount, HcclDataType se
         counts.data(), displs.data(), counts.data(), displs.data());
 }
 
+// op_base.cc:2633-2733.  sendCountMatrix is a host array of p x p uint64_t, the same on every rank:
+// entry [i * p + j] = elements rank i sends to rank j.  Blocks are packed back to back on both sides
+// (displacements are running sums, alltoall_operator.cc:74-120); checks as in param_check.cc:205-242.
+HcclResult HcclAlltoAllVC(const void *sendBuf, const void *sendCountMatrix, HcclDataType sendType, const void *recvBuf,
+    HcclDataType recvType, HcclComm comm, aclrtStream stream)
+{
+    CHK_PTR(sendCountMatrix);
+    CHK_PTR(comm);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    const uint32_t p = c->group->p, me = c->rank;
+    if (sendBuf != nullptr && recvBuf != nullptr && sendBuf == recvBuf) {
+        HCCL_LOG_ERROR("HcclAlltoAllVC: sendBuf and recvBuf cannot be the same");
+        return HCCL_E_PARA;
+    }
+    const uint64_t *m = static_cast<const uint64_t *>(sendCountMatrix);
+    std::vector<uint64_t> sc(p), sd(p), rc(p), rd(p);
+    bool hasSend = false, hasRecv = false;
+    uint64_t sAt = 0, rAt = 0;
+    for (uint32_t j = 0; j < p; j++) {
+        sc[j] = m[uint64_t(me) * p + j];
+        rc[j] = m[uint64_t(j) * p + me];
+        if (sc[j] > kSysMaxCount) {
+            HCCL_LOG_ERROR("HcclAlltoAllVC: a count exceeds the maximum");
+            return HCCL_E_PARA;
+        }
+        sd[j] = sAt;
+        rd[j] = rAt;
+        sAt += sc[j];
+        rAt += rc[j];
+        hasSend = hasSend || sc[j] != 0;
+        hasRecv = hasRecv || rc[j] != 0;
+    }
+    if (hasSend) {
+        CHK_PTR(sendBuf);
+    }
+    if (hasRecv) {
+        CHK_PTR(recvBuf);
+    }
+    HcclResult r = CheckOpParam("HcclAlltoAllVC", 0, sendType, stream);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if (!DataTypeKnown(recvType)) {
+        return HCCL_E_NOT_SUPPORT;
+    }
+    if (ElemSize(sendType) != ElemSize(recvType)) {
+        HCCL_LOG_ERROR("HcclAlltoAllVC: send and receive element sizes differ");
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_ALLTOALLV;
+    sig.dtype = sendType;
+    sig.recvType = recvType;
+    // ranks that pass different matrices fail the symmetry check of the rendezvous (HCCL_E_PARA)
+    return Arrive(c, sig, const_cast<void *>(sendBuf), const_cast<void *>(recvBuf), static_cast<hipStream_t>(stream),
+        sc.data(), sd.data(), rc.data(), rd.data());
+}
+
 // op_base.cc:1353-1431: an all-reduce (fp32 sum) of a few elements on buffers the group owns.
 HcclResult HcclBarrier(HcclComm comm, aclrtStream stream)
 {
@@ -1308,6 +1370,8 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         } else {
             return HCCL_E_PARA;
         }
+    } else if (k == "deterministic") {
+        cfg.deterministic = v != "0";
     } else if (k == "fuse") {
         cfg.fuse = v != "0";
     } else if (k == "graph") {

@@ -536,6 +536,13 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     } else if (algo == ALGO_PAIRWISE) {
         algo = ALGO_RING;
     }
+    // coll_all_reduce_mesh_executor.cc:108-112, coll_reduce_scatter_mesh_executor.cc:227-229: without the
+    // deterministic setting the mesh reduce phases run uncut, except for int64 and for products
+    if (algo == ALGO_MESH && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
+        g->ctx->sig.op != HCCL_REDUCE_PROD &&
+        (g->ctx->sig.coll == COLL_ALLREDUCE || g->ctx->sig.coll == COLL_REDUCESCATTER)) {
+        algo = ALGO_MESH_ATOMIC;
+    }
     std::string key = CacheKey(g, algo);
     Prepared *pp = nullptr;
     auto it = g->cache.find(key);

@@ -101,10 +101,14 @@ size_t RingAllGatherPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t bas
 
 // Deterministic mesh reduce-scatter: every rank slice is cut into (p-1) pieces, piece t follows the
 // peer order rotated by t, so that in each round the pieces of one rank read p-1 different peers.
+// Atomic variant (reduce_scatter_mesh_atomic.cc:82-141): no piece cut; stream j of rank r pulls the
+// whole slice r from rank (r+1+j) and accumulates it into the rank's own copy.  The reference lets
+// the p-1 streams race (accumulation in arrival order); here they are taken in stream order, one of
+// the orders the reference can produce.
 size_t MeshReduceScatterPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t base, const std::vector<Slice> &sl,
-    uint64_t align)
+    uint64_t align, bool atomic)
 {
-    uint32_t nstream = p > 2 ? p - 1 : 1;
+    uint32_t nstream = (p > 2 && !atomic) ? p - 1 : 1;
     for (uint32_t r = 0; r < p; r++) {
         if (sl[r].size == 0) {
             continue;
@@ -113,7 +117,7 @@ size_t MeshReduceScatterPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t
         for (uint32_t t = 0; t < nstream; t++) {
             for (uint32_t round = 1; round < p; round++) {
                 uint32_t order = (round + t - 1) % (p - 1);
-                uint32_t src = Mod(static_cast<int64_t>(r) - (order + 1), p);
+                uint32_t src = atomic ? (r + round) % p : Mod(static_cast<int64_t>(r) - (order + 1), p);
                 uint64_t off = base + sl[r].off + pieces[t].off;
                 EmitReduce(vp, phase0 + round - 1, MkRef(r, BUF_SEND, off), MkRef(r, BUF_SEND, off), MkRef(src, BUF_SEND, off),
                     pieces[t].size);
@@ -135,7 +139,7 @@ size_t MeshAllGatherPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t bas
     return phase0 + 1;
 }
 
-void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t bytes, uint64_t align)
+void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t bytes, uint64_t align, bool meshAtomic)
 {
     if (p == 1) {
         EmitCopy(vp, 0, MkRef(0, BUF_RECV, base), MkRef(0, BUF_SEND, base), bytes);
@@ -148,7 +152,7 @@ void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t
             // the ring template runs its reduce-scatter with output == input
             ph = RingReduceScatterPhases(vp, ph, p, base, sl, BUF_SEND, base, sl);
         } else {
-            ph = MeshReduceScatterPhases(vp, ph, p, base, sl, align);
+            ph = MeshReduceScatterPhases(vp, ph, p, base, sl, align, meshAtomic);
         }
         for (uint32_t r = 0; r < p; r++) {
             EmitCopy(vp, ph, MkRef(r, BUF_RECV, base + sl[r].off), MkRef(r, BUF_SEND, base + sl[r].off), sl[r].size);
@@ -454,7 +458,7 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             } else if (rq.algo == ALGO_RHD) {
                 RhdReduceScatterChunk(*vp, p, sl, 0);
             } else {
-                size_t ph = MeshReduceScatterPhases(*vp, 0, p, 0, sl, rq.align);
+                size_t ph = MeshReduceScatterPhases(*vp, 0, p, 0, sl, rq.align, rq.meshAtomic);
                 for (uint32_t r = 0; r < p; r++) {
                     EmitCopy(*vp, ph, MkRef(r, BUF_RECV, 0), MkRef(r, BUF_SEND, sl[r].off), sl[r].size);
                 }
@@ -493,7 +497,7 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
     for (uint64_t cur : chunks) {
         uint64_t bytes = cur * u;
         if (rq.coll == COLL_ALLREDUCE) {
-            AllReduceChunk(*vp, rq.algo, p, done, bytes, rq.align);
+            AllReduceChunk(*vp, rq.algo, p, done, bytes, rq.align, rq.meshAtomic);
         } else if (rq.coll == COLL_REDUCESCATTER) {
             // input slice i of this chunk sits at i * total + done in the caller's layout
             std::vector<Slice> in(p), out(p);
@@ -508,7 +512,7 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             } else if (rq.algo == ALGO_RHD) {
                 RhdReduceScatterChunk(*vp, p, in, done);
             } else {
-                size_t ph = MeshReduceScatterPhases(*vp, 0, p, 0, in, rq.align);
+                size_t ph = MeshReduceScatterPhases(*vp, 0, p, 0, in, rq.align, rq.meshAtomic);
                 for (uint32_t r = 0; r < p; r++) {
                     EmitCopy(*vp, ph, MkRef(r, BUF_RECV, done), MkRef(r, BUF_SEND, in[r].off), bytes);
                 }
@@ -1141,12 +1145,19 @@ std::vector<uint64_t> ChunkCounts(CollKind coll, uint64_t count, uint32_t unit, 
     return v;
 }
 
-int BuildPlan(const PlanRequest &rq, Plan *plan, std::string *err)
+int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
 {
-    if (rq.p == 0 || rq.unit == 0 || rq.align == 0) {
+    if (request.p == 0 || request.unit == 0 || request.align == 0) {
         *err = "bad plan request";
         return 1;
     }
+    PlanRequest normalised;
+    if (request.algo == ALGO_MESH_ATOMIC) {
+        normalised = request;
+        normalised.algo = ALGO_MESH;
+        normalised.meshAtomic = true;
+    }
+    const PlanRequest &rq = request.algo == ALGO_MESH_ATOMIC ? normalised : request;
     VProgram vp;
     if (BuildVirtual(rq, &vp, err) != 0) {
         return 1;

@@ -25,7 +25,9 @@ enum CollKind : int {
     COLL_ALLREDUCE = 0, COLL_REDUCESCATTER = 1, COLL_ALLGATHER = 2, COLL_ALLTOALLV = 3,
     COLL_BROADCAST = 4, COLL_REDUCE = 5, COLL_SCATTER = 6, COLL_SENDRECV = 7
 };
-enum Algo : int { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2, ALGO_PAIRWISE = 3 };
+// ALGO_MESH_ATOMIC: the mesh schedule whose reduce phases skip the piece cut (the reference's
+// non-deterministic variant, taken in stream order); BuildPlan turns it into ALGO_MESH + meshAtomic.
+enum Algo : int { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2, ALGO_PAIRWISE = 3, ALGO_MESH_ATOMIC = 4 };
 
 // Physical buffers of a rank: the caller's send and receive buffers and a library-owned scratch.
 enum Buf : uint8_t { BUF_SEND = 0, BUF_RECV = 1, BUF_SCRATCH = 2 };
@@ -77,6 +79,7 @@ struct PlanRequest {
     uint64_t cclBytes = 200ull << 20;
     uint64_t align = 128;
     std::vector<uint8_t> alias;    // per rank: send buffer and receive buffer are the same memory
+    bool meshAtomic = false;       // mesh reduce phases without the piece cut (the reference's non-deterministic variant)
     bool stageInput = false;       // copy the send buffers to scratch first (used when buffers overlap)
     // all-to-all-v only: p x p tables in elements, row r = what rank r passed
     std::vector<uint64_t> sendCounts, sdispls, recvCounts, rdispls;

@@ -53,6 +53,13 @@ extern HcclResult HcclAlltoAllV(const void *sendBuf, const void *sendCounts, con
 extern HcclResult HcclAlltoAll(const void *sendBuf, uint64_t sendCount, HcclDataType sendType,
     const void *recvBuf, uint64_t recvCount, HcclDataType recvType, HcclComm comm, aclrtStream stream);
 
+/* sendCountMatrix: host array of p x p uint64_t, identical on every rank; entry [i * p + j] is the
+ * number of elements rank i sends to rank j.  Blocks lie back to back in both buffers.  Not in the
+ * reference's public header: declared in its framework header
+ * src/domain/collective_communication/framework/op_base/src/op_base.h:59, impl op_base.cc:2633. */
+extern HcclResult HcclAlltoAllVC(const void *sendBuf, const void *sendCountMatrix, HcclDataType sendType,
+    const void *recvBuf, HcclDataType recvType, HcclComm comm, aclrtStream stream);
+
 /* decl inc/hccl/hccl.h:181, impl op_base.cc:1585. */
 extern HcclResult HcclReduceScatterV(void *sendBuf, const void *sendCounts, const void *sendDispls,
     void *recvBuf, uint64_t recvCount, HcclDataType dataType, HcclReduceOp op, HcclComm comm, aclrtStream stream);

@@ -12,18 +12,23 @@ extern "C" {
 #endif
 
 /* Settings of the communicator's whole group.  Keys and values:
- *   "algo"          "ring" | "mesh" | "rhd" | "auto"   (all-reduce; reduce-scatter / all-gather take ring or mesh)
+ *   "algo"          "ring" | "mesh" | "rhd" | "auto"
+ *   "deterministic" "0" | "1"    as HCCL_DETERMINISTIC; with "0" (the default) the mesh reduce phases of
+ *                                all-reduce / reduce-scatter run without the piece cut (not for int64, not for products)
  *   "fuse"          "0" | "1"    run the single-pass fused form when the schedule has one
  *   "graph"         "0" | "1"    issue through a HIP graph
- *   "buffsize_mib"  CCL buffer size that sets the chunk plan (default 200, as HCCL_BUFFSIZE)
+ *   "buffsize_mib"  CCL buffer size that sets the chunk plan (default 200, as HCCL_BUFFSIZE);
+ *   "buffsize_bytes" the same in bytes (tests of the chunk loop on small inputs)
  *   "align"         slice alignment in bytes (default 128)
- *   "blocks_per_cu" launch width
+ *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
+ *   "blocking_arrive" "0" | "1"  a rank's call waits inside the library until the group is complete
+ *   "arrive_timeout_ms"          limit of that wait (HCCL_E_TIMEOUT)
  * Unknown key or bad value: HCCL_E_PARA. */
 extern HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value);
 
 typedef struct HcclAmdOpInfoDef {
     int32_t coll;            /* 0 all-reduce, 1 reduce-scatter, 2 all-gather, 3 all-to-all-v, 4 broadcast, 5 reduce, 6 scatter */
-    int32_t algo;            /* 0 ring, 1 mesh, 2 rhd, 3 pairwise */
+    int32_t algo;            /* 0 ring, 1 mesh, 2 rhd, 3 pairwise, 4 mesh without the piece cut */
     int32_t fused;           /* 1: issued as fused single-pass kernels */
     int32_t graph;           /* 1: issued as a HIP graph */
     int32_t cacheHit;        /* 1: an instantiated graph / table set was reused */

@@ -14,7 +14,9 @@
 //   ring             TPL/temp_reduce_scatter/reduce_scatter_ring.cc:89-297, TPL/temp_all_gather/all_gather_ring.cc:51-171,
 //                    TPL/temp_all_reduce/all_reduce_ring.cc:32-53,143-191
 //   mesh             TPL/temp_reduce_scatter/reduce_scatter_mesh.cc:57-203, TPL/temp_all_gather/all_gather_mesh.cc:91-253,
-//                    EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240, EXE/coll_comm_executor.cc:1458-1574
+//                    EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240, EXE/coll_comm_executor.cc:1458-1574,
+//                    TPL/temp_reduce_scatter/reduce_scatter_mesh_atomic.cc:82-141 (accumulation order of the racing
+//                    streams fixed to stream order: for floating point the reference itself has no single answer)
 //   halving-doubling TPL/temp_all_reduce/all_reduce_recursive_hd.cc:33-302,
 //                    TPL/temp_reduce_scatter/reduce_scatter_recursive_hd.cc:33-254, TPL/temp_all_gather/all_gather_recursive_hd.cc:26-238,
 //                    TPL/temp_reduce_scatter/reduce_scatter_halving_doubling.cc:67-238,
@@ -64,7 +66,7 @@ namespace {
 enum { DT_INT8 = 0, DT_INT16 = 1, DT_INT32 = 2, DT_FP16 = 3, DT_FP32 = 4, DT_INT64 = 5, DT_UINT64 = 6,
        DT_UINT8 = 7, DT_UINT16 = 8, DT_UINT32 = 9, DT_FP64 = 10, DT_BF16 = 11, DT_INT128 = 12 };
 enum { OP_SUM = 0, OP_PROD = 1, OP_MAX = 2, OP_MIN = 3 };
-enum { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2 };
+enum { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2, ALGO_MESH_ATOMIC = 4 };
 
 size_t DtSize(int dt)
 {
@@ -626,6 +628,23 @@ void ProgReduceScatterMeshStream(std::vector<Action> &pg, uint32_t r, uint32_t p
     }
 }
 
+// ReduceScatterMeshAtomic::RunReduceScatter, reduce_scatter_mesh_atomic.cc:82-141: stream j of rank r
+// pulls slice r of rank (r+1+j) and accumulates it into the rank's own slice r.  The reference lets
+// the p-1 streams race, so its floating-point result depends on arrival order; this restatement
+// takes the streams in index order, which is one of the outcomes the reference can produce.
+// The slices a rank hands out are never written during the phase, so all hand-outs come first.
+void ProgReduceScatterMeshAtomic(std::vector<Action> &pg, uint32_t r, uint32_t p, int inB, const std::vector<Slice> &sl)
+{
+    for (uint32_t j = 0; j + 1 < p; j++) {
+        uint32_t puller = (r + p - 1 - j) % p;   // the rank whose stream j reads from this rank
+        pg.push_back(MkSend(puller, static_cast<int>(j), inB, sl[puller].off, sl[puller].size));
+    }
+    for (uint32_t j = 0; j + 1 < p; j++) {
+        uint32_t remote = (r + 1 + j) % p;
+        pg.push_back(MkRecvReduce(remote, static_cast<int>(j), inB, sl[r].off, inB, sl[r].off, sl[r].size));
+    }
+}
+
 // AllGatherMesh::RunAllGather, all_gather_mesh.cc:91-145 (one channel per round).
 void ProgAllGatherMesh(std::vector<Action> &pg, uint32_t r, uint32_t p, int outB, const std::vector<Slice> &sl)
 {
@@ -720,7 +739,7 @@ int RunAllReduceRing(Machine &m, uint64_t bytes, uint64_t align)
 }
 
 // CollAllReduceMeshExecutor::KernelRun, deterministic branch (coll_all_reduce_mesh_executor.cc:95-240).
-int RunAllReduceMesh(Machine &m, uint64_t bytes, uint64_t align)
+int RunAllReduceMesh(Machine &m, uint64_t bytes, uint64_t align, bool atomic)
 {
     uint32_t p = m.p;
     if (p == 1) {
@@ -728,7 +747,15 @@ int RunAllReduceMesh(Machine &m, uint64_t bytes, uint64_t align)
         return 0;
     }
     std::vector<Slice> sl = RingSlices(bytes, p, align);
-    if (p > 2) {
+    if (atomic) {
+        // non-deterministic branch, coll_all_reduce_mesh_executor.cc:108-113
+        for (uint32_t r = 0; r < p; r++) {
+            Proc pr;
+            pr.rank = r;
+            ProgReduceScatterMeshAtomic(pr.prog, r, p, B_IN, sl);
+            m.procs.push_back(std::move(pr));
+        }
+    } else if (p > 2) {
         std::vector<std::vector<Slice>> pieces = CutPieces(sl, p - 1, align);
         for (uint32_t t = 0; t < p - 1; t++) {
             for (uint32_t r = 0; r < p; r++) {
@@ -837,7 +864,8 @@ int RunAllReduceTemplate(Machine &m, int algo, uint64_t bytes, uint64_t align)
 {
     switch (algo) {
         case ALGO_RING: return RunAllReduceRing(m, bytes, align);
-        case ALGO_MESH: return RunAllReduceMesh(m, bytes, align);
+        case ALGO_MESH: return RunAllReduceMesh(m, bytes, align, false);
+        case ALGO_MESH_ATOMIC: return RunAllReduceMesh(m, bytes, align, true);
         case ALGO_RHD: return RunAllReduceRhd(m, bytes, align);
         default: return -10;
     }
@@ -1027,6 +1055,14 @@ int orc_reducescatter(int algo, uint32_t p, void **in, void **out, uint64_t recv
                     ProgReduceScatterRing(pr.prog, r, p, B_IN, B_IN, sl, sl);
                     m.procs.push_back(std::move(pr));
                 }
+            } else if (algo == ALGO_MESH_ATOMIC) {
+                // coll_reduce_scatter_mesh_executor.cc:227-232
+                for (uint32_t r = 0; r < p; r++) {
+                    Proc pr;
+                    pr.rank = r;
+                    ProgReduceScatterMeshAtomic(pr.prog, r, p, B_IN, sl);
+                    m.procs.push_back(std::move(pr));
+                }
             } else if (algo == ALGO_MESH) {
                 uint32_t nstream = p > 2 ? p - 1 : 1;
                 std::vector<std::vector<Slice>> pieces = CutPieces(sl, nstream, align);
@@ -1206,6 +1242,13 @@ int orc_reducescatter_v(int algo, uint32_t p, void **in, void **out, const uint6
                 Proc pr;
                 pr.rank = r;
                 ProgReduceScatterRing(pr.prog, r, p, B_IN, B_IN, sl, sl);
+                m.procs.push_back(std::move(pr));
+            }
+        } else if (algo == ALGO_MESH_ATOMIC) {
+            for (uint32_t r = 0; r < p; r++) {
+                Proc pr;
+                pr.rank = r;
+                ProgReduceScatterMeshAtomic(pr.prog, r, p, B_IN, sl);
                 m.procs.push_back(std::move(pr));
             }
         } else if (algo == ALGO_MESH) {

@@ -16,6 +16,7 @@ _LIB_PATH = os.path.join(_HERE, "libhccl_oracle.so")
 INT8, INT16, INT32, FP16, FP32, INT64, UINT64, UINT8, UINT16, UINT32, FP64, BF16 = range(12)
 SUM, PROD, MAX, MIN = range(4)
 RING, MESH, RHD = range(3)
+MESH_ATOMIC = 4   # mesh reduce phases without the piece cut, streams in index order
 DIRECT = 1        # flags bit0: messages are pointers, not snapshots
 ZERO_STAGING = 2  # flags bit1: templates run on the caller's buffers (input clobbered)
 

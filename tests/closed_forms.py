@@ -133,6 +133,34 @@ def mesh_allreduce(dt, op, ins, unit, ccl_bytes, align):
     return [out.copy() for _ in range(p)]
 
 
+def mesh_atomic_chain(dt, op, xs, r):
+    """Mesh reduce-scatter without the piece cut, streams taken in index order:
+    ((x[r] (+) x[r+1]) (+) x[r+2]) ... (+) x[r+p-1]."""
+    p = len(xs)
+    acc = xs[r]
+    for j in range(p - 1):
+        acc = combine(dt, op, acc, xs[(r + 1 + j) % p])
+    return acc
+
+
+def mesh_atomic_allreduce(dt, op, ins, unit, ccl_bytes, align):
+    p = len(ins)
+    n = ins[0].size
+    if p == 1:
+        return [ins[0].copy()]
+    out = np.empty_like(ins[0])
+    max_per = ccl_bytes // unit
+    base = 0
+    while base < n:
+        cur = min(n - base, max_per)
+        for r, (off, size) in enumerate(slice_plan(cur * unit, p, align)):
+            lo, hi = base + off // unit, base + (off + size) // unit
+            if hi > lo:
+                out[lo:hi] = mesh_atomic_chain(dt, op, [x[lo:hi] for x in ins], r)
+        base += cur
+    return [out.copy() for _ in range(p)]
+
+
 def rhd_params(p):
     block = 1
     while block * 2 <= p:

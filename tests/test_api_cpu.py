@@ -125,6 +125,18 @@ def test_sibling_entry_checks(comms):
     assert L.HcclAlltoAll(BUF_A, 4, I32, BUF_B, 4, H.HCCL_DATA_TYPE_FP32, c, STREAM) == H.HCCL_E_PARA
     assert L.HcclAlltoAll(BUF_A, 4, I32, BUF_B, 4, I32, c, None) == H.HCCL_E_PTR
     assert L.HcclAlltoAll(BUF_A, 4, I32, BUF_A, 4, I32, c, STREAM) == H.HCCL_E_PARA
+    # HcclAlltoAllVC (op_base.cc:2633, param_check.cc:205-242): 4 x 4 matrix of element counts
+    m1 = (ctypes.c_uint64 * 16)(*([1] * 16))
+    mbig = (ctypes.c_uint64 * 16)(*([0x800000000] * 16))
+    assert L.HcclAlltoAllVC(BUF_A, None, I32, BUF_B, I32, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAlltoAllVC(BUF_A, m1, I32, BUF_B, I32, None, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAlltoAllVC(BUF_A, m1, I32, BUF_A, I32, c, STREAM) == H.HCCL_E_PARA
+    assert L.HcclAlltoAllVC(BUF_A, mbig, I32, BUF_B, I32, c, STREAM) == H.HCCL_E_PARA
+    assert L.HcclAlltoAllVC(None, m1, I32, BUF_B, I32, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAlltoAllVC(BUF_A, m1, I32, None, I32, c, STREAM) == H.HCCL_E_PTR
+    assert L.HcclAlltoAllVC(BUF_A, m1, I32, BUF_B, I32, c, None) == H.HCCL_E_PTR
+    assert L.HcclAlltoAllVC(BUF_A, m1, 14, BUF_B, I32, c, STREAM) == H.HCCL_E_NOT_SUPPORT
+    assert L.HcclAlltoAllVC(BUF_A, m1, I32, BUF_B, 14, c, STREAM) == H.HCCL_E_NOT_SUPPORT
     # HcclReduceScatterV (op_base.cc:1585)
     assert L.HcclReduceScatterV(BUF_A, None, ones, BUF_B, 1, I32, SUM, c, STREAM) == H.HCCL_E_PTR
     assert L.HcclReduceScatterV(BUF_A, ones, ones, None, 1, I32, SUM, c, STREAM) == H.HCCL_E_PTR

@@ -13,8 +13,8 @@ from test_oracle_schedules import _a2av_case
 
 pytestmark = pytest.mark.gpu
 H = gh.H
-RING, MESH, RHD = 0, 1, 2
-ALGO_NAME = {RING: "ring", MESH: "mesh", RHD: "rhd"}
+RING, MESH, RHD, MESH_ATOMIC = 0, 1, 2, 4
+ALGO_NAME = {RING: "ring", MESH: "mesh", RHD: "rhd", MESH_ATOMIC: "mesh"}
 OPS = (SUM, PROD, MAX, MIN)
 
 
@@ -33,6 +33,18 @@ def _ulp_close(dt, got, want):
     return int(np.abs(g - w).max()) <= 1
 
 
+def _group(p, algo, **params):
+    """MESH = the deterministic mesh (piece cut); MESH_ATOMIC = the library's default for the mesh."""
+    return gh.Group(p, algo=ALGO_NAME[algo], deterministic=0 if algo == MESH_ATOMIC else 1, **params)
+
+
+def _expected_algo(algo, dt, op):
+    """The uncut mesh is not used for int64 or for products (coll_all_reduce_mesh_executor.cc:108-112)."""
+    if algo == MESH_ATOMIC and (dt == INT64 or op == PROD):
+        return MESH
+    return algo
+
+
 @pytest.fixture(scope="module")
 def orc():
     from oracle import oracle
@@ -40,11 +52,11 @@ def orc():
     return oracle
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD, MESH_ATOMIC])
 @pytest.mark.parametrize("fuse", [1, 0])
 def test_allreduce_fp32_sum_bit_exact(orc, algo, fuse):
     for p in (1, 2, 3, 5, 8, 16):
-        g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+        g = _group(p, algo, fuse=fuse)
         try:
             for n in (1, 7, 1000, 262144 + 3):
                 ins = _ins(FP32, p, n, 1000 * p + n)
@@ -63,15 +75,16 @@ def test_allreduce_fp32_sum_bit_exact(orc, algo, fuse):
 @pytest.mark.parametrize("dt", ALL_TYPES)
 def test_allreduce_every_type_and_op(orc, dt):
     p, n = 8, 40000 + 13
-    for algo in (RING, RHD, MESH):
+    for algo in (RING, RHD, MESH, MESH_ATOMIC):
         for fuse in (1, 0):
-            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+            g = _group(p, algo, fuse=fuse)
             try:
                 for op in OPS:
                     print("allreduce type", dt, "op", op, ALGO_NAME[algo], "fuse", fuse, flush=True)
                     ins = _ins(dt, p, n, dt * 10 + op)
-                    want = orc.allreduce(ins, dt, op, algo=algo)
+                    want = orc.allreduce(ins, dt, op, algo=_expected_algo(algo, dt, op))
                     outs, _ = gh.all_reduce(g, ins, dt, op)
+                    assert g.info()["algo"] == _expected_algo(algo, dt, op)
                     for r in range(p):
                         if dt in (FP16, BF16):
                             assert _ulp_close(dt, outs[r], want[r]), (dt, op, algo, fuse, r)
@@ -172,18 +185,18 @@ def test_streams_of_other_ranks_are_ordered(orc):
         g.close()
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD, MESH_ATOMIC])
 def test_reducescatter_op_type_matrix(orc, algo):
     p = 8 if algo != RHD else 6
     for fuse in (1, 0):
-        g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+        g = _group(p, algo, fuse=fuse)
         try:
             for dt in (FP16, BF16, INT8, INT32, INT64, FP32):
                 for op in OPS:
                     n = 30011
                     ins = _ins(dt, p, n * p, dt + 3 * op)
                     print("reducescatter", ALGO_NAME[algo], "fuse", fuse, "type", dt, "op", op, flush=True)
-                    want = orc.reducescatter(ins, dt, op, algo=algo)
+                    want = orc.reducescatter(ins, dt, op, algo=_expected_algo(algo, dt, op))
                     outs, keep = gh.reduce_scatter(g, ins, dt, op)
                     for r in range(p):
                         assert gh.same(dt, outs[r], want[r]), (algo, fuse, dt, op, r)
@@ -213,7 +226,7 @@ def test_reducescatter_64mib_per_rank_int_and_bf16(orc):
 def test_allgather(orc, algo):
     for p in (1, 2, 5, 8, 12):
         for fuse in (1, 0):
-            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+            g = _group(p, algo, fuse=fuse)
             try:
                 for dt, n, pad in ((INT8, 30001, 0), (INT8, 777, 3), (FP16, 4099, 2), (INT64, 65536, 0), (FP32, 1, 0)):
                     ins = _ins(dt, p, n, p + n)
@@ -325,7 +338,7 @@ def test_special_values_follow_the_selection_rule(orc):
     ins = [rng.choice(specials, 4096).astype(np.float32) for _ in range(p)]
     for algo in (RING, RHD):
         for fuse in (1, 0):
-            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse, align=4)
+            g = _group(p, algo, fuse=fuse, align=4)
             try:
                 for op in OPS:
                     want = orc.allreduce(ins, FP32, op, algo=algo, align=4)
@@ -351,16 +364,16 @@ def _v_case(p, seed, scale):
     return counts, displs, pos + 3
 
 
-@pytest.mark.parametrize("algo", [RING, MESH])
+@pytest.mark.parametrize("algo", [RING, MESH, MESH_ATOMIC])
 def test_reducescatter_v(orc, algo):
     for p in (1, 3, 8):
         for fuse in (1, 0):
-            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+            g = _group(p, algo, fuse=fuse)
             try:
                 for dt, op, scale in ((FP32, SUM, 50000), (BF16, SUM, 3000), (INT8, MIN, 70000)):
                     counts, displs, extent = _v_case(p, p + dt, scale)
                     ins = _ins(dt, p, extent, 3 * p + dt)
-                    want = orc.reducescatter_v(ins, counts, displs, dt, op, algo=algo)
+                    want = orc.reducescatter_v(ins, counts, displs, dt, op, algo=_expected_algo(algo, dt, op))
                     sends = [gh.to_dev(x) for x in ins]
                     recvs = [gh.empty_dev(max(int(counts[r]), 1) * H.DTYPE_SIZE[dt]) for r in range(p)]
                     torch.cuda.synchronize()
@@ -379,7 +392,7 @@ def test_reducescatter_v(orc, algo):
 def test_allgather_v(orc, algo):
     for p in (1, 3, 6, 8):
         for fuse in (1, 0):
-            g = gh.Group(p, algo=ALGO_NAME[algo], fuse=fuse)
+            g = _group(p, algo, fuse=fuse)
             try:
                 counts, displs, extent = _v_case(p, 7 * p, 40000)
                 ins = [np.arange(int(counts[r]), dtype=np.int32) + (r << 20) for r in range(p)]
@@ -415,6 +428,36 @@ def test_alltoall_uniform_and_barrier(orc):
             for j in range(p):
                 want = np.concatenate([sends_np[i][j * n:(j + 1) * n] for i in range(p)])
                 assert np.array_equal(gh.to_host(recvs[j], INT32), want), (p, j)
+        finally:
+            g.close()
+
+
+def test_alltoallvc_matrix(orc):
+    # one p x p count matrix for every rank; blocks packed back to back (alltoall_operator.cc:74-120)
+    for p in (1, 3, 8):
+        rng = np.random.default_rng(70 + p)
+        m = rng.integers(0, 3000, size=(p, p)).astype(np.uint64)
+        m[rng.integers(0, p), rng.integers(0, p)] = 0
+        sdis = np.zeros((p, p), np.uint64)
+        rdis = np.zeros((p, p), np.uint64)
+        for r in range(p):
+            sdis[r, 1:] = np.cumsum(m[r, :-1])
+            rdis[r, 1:] = np.cumsum(m[:-1, r])
+        sl = [int(m[r].sum()) for r in range(p)]
+        rl = [int(m[:, r].sum()) for r in range(p)]
+        sends_np = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+        want = [np.full(n, -1, np.int32) for n in rl]
+        assert orc.alltoallv(sends_np, m, sdis, want, m.T.copy(), rdis, INT32) == 0
+        g = gh.Group(p)
+        try:
+            print("alltoallvc p", p, flush=True)
+            sends = [gh.to_dev(x) for x in sends_np]
+            recvs = [gh.to_dev(np.full(max(n, 1), -1, np.int32)) for n in rl]
+            torch.cuda.synchronize()
+            H.all_to_all_vc(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], m, INT32, g.stream_ptr)
+            g.stream.synchronize()
+            for r in range(p):
+                assert np.array_equal(gh.to_host(recvs[r], INT32)[:rl[r]], want[r]), (p, r)
         finally:
             g.close()
 

@@ -7,7 +7,7 @@ import pytest
 import closed_forms as cf
 from closed_forms import (ALL_TYPES, BF16, FP16, FP32, FP64, INT8, INT32, INT64, INT_TYPES, MAX, MIN, PROD, SUM)
 
-RING, MESH, RHD = 0, 1, 2
+RING, MESH, RHD, MESH_ATOMIC = 0, 1, 2, 4
 OPS = (SUM, PROD, MAX, MIN)
 
 
@@ -69,10 +69,10 @@ def _eq(dt, got, want):
     return np.array_equal(got, want)
 
 
-CLOSED = {RING: cf.ring_allreduce, MESH: cf.mesh_allreduce, RHD: cf.rhd_allreduce}
+CLOSED = {RING: cf.ring_allreduce, MESH: cf.mesh_allreduce, RHD: cf.rhd_allreduce, MESH_ATOMIC: cf.mesh_atomic_allreduce}
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD, MESH_ATOMIC])
 def test_allreduce_fp32_sum_matches_closed_form_all_p(orc, algo):
     # fp32 sum is order-sensitive: only the right chain / tree reproduces these bits
     for p in range(1, 34):
@@ -85,7 +85,7 @@ def test_allreduce_fp32_sum_matches_closed_form_all_p(orc, algo):
                 assert np.array_equal(got[r], want[r]), (algo, p, align, r)
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD, MESH_ATOMIC])
 @pytest.mark.parametrize("dt", ALL_TYPES)
 def test_allreduce_all_types_ops_match_closed_form(orc, algo, dt):
     unit = orc.dtype_size(dt)
@@ -98,7 +98,7 @@ def test_allreduce_all_types_ops_match_closed_form(orc, algo, dt):
                 assert _eq(dt, got[r], want[r]), (algo, dt, p, op, r)
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD, MESH_ATOMIC])
 def test_allreduce_chunked_matches_closed_form(orc, algo):
     # CCL buffer smaller than the payload: the chunk loop restarts the slice plan per chunk
     p, n = 8, 5000
@@ -122,7 +122,7 @@ def test_ring_order_sensitive_known_answer(orc):
     assert all(np.array_equal(got[0], g) for g in got)
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD, MESH_ATOMIC])
 @pytest.mark.parametrize("dt", INT_TYPES)
 def test_integer_results_are_schedule_independent(orc, algo, dt):
     for p in (2, 3, 7, 8, 16, 24):
@@ -199,7 +199,7 @@ def test_allgather_rhd_is_the_permutation(orc):
             assert all(np.array_equal(g, want) for g in got), (p, ccl)
 
 
-@pytest.mark.parametrize("algo", [RING, MESH])
+@pytest.mark.parametrize("algo", [RING, MESH, MESH_ATOMIC])
 def test_reducescatter_matches_chain(orc, algo):
     for dt in (FP32, BF16, INT8, INT64):
         unit = orc.dtype_size(dt)
@@ -215,6 +215,8 @@ def test_reducescatter_matches_chain(orc, algo):
                             want = xs[0]
                         elif algo == RING:
                             want = cf.ring_chain(dt, op, xs, r)
+                        elif algo == MESH_ATOMIC:
+                            want = cf.mesh_atomic_chain(dt, op, xs, r)
                         else:
                             want = np.empty_like(xs[0])
                             # the piece cut restarts in every chunk of the loop

@@ -10,7 +10,7 @@ from hccl_loader import load
 from test_oracle_schedules import _a2av_case
 
 H = load()
-RING, MESH, RHD = 0, 1, 2
+RING, MESH, RHD, MESH_ATOMIC = 0, 1, 2, 4
 
 
 def _bytes(arrs):
@@ -30,7 +30,7 @@ def _same(dt, got_bytes, want):
     return np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD, MESH_ATOMIC])
 @pytest.mark.parametrize("p", [1, 2, 3, 4, 5, 6, 8, 12, 16, 24])
 def test_allreduce_plan_matches_checker(orc, algo, p):
     for dt, op, n, ccl in ((FP32, SUM, 1000, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, PROD, 777, 200 << 20),
@@ -69,7 +69,7 @@ def test_allreduce_ring_byte_counts():
     assert plan["fusedOk"] and plan["fused"][0]["kind"] == 2 and plan["fused"][0]["nleaf"] == 16
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, RHD])
+@pytest.mark.parametrize("algo", [RING, MESH, RHD, MESH_ATOMIC])
 @pytest.mark.parametrize("p", [1, 2, 3, 6, 8, 12])
 def test_reducescatter_plan_matches_checker(orc, algo, p):
     for dt, op, n, ccl in ((FP32, SUM, 500, 200 << 20), (BF16, SUM, 301, 128 * p * 2), (INT64, MIN, 100, 200 << 20)):
