@@ -249,23 +249,52 @@ HCCL_WORDWISE_COMBINER(Bf16Bits, HCCL_EXPR_BF16)
 template <typename T, int OP> __device__ __forceinline__ V4 Combine16(V4 a, V4 b) { return Combiner<T, OP>::Apply(a, b); }
 
 // ---- memory access ---------------------------------------------------------------------------------
-struct __attribute__((packed, aligned(4))) Vec16A4 {
-    uint32_t x, y, z, w;
-};
+// 16 bytes at an address that is only 4-byte aligned.
+typedef uint32_t V4A4 __attribute__((ext_vector_type(4), aligned(4)));
+
+// Rank buffers are device (global) memory.  The pointers come out of descriptor tables, so the
+// compiler cannot know that and would issue flat accesses, whose completion is counted together
+// with scalar loads (a wait for the next descriptor pointer then also waits for every load in
+// flight).  Casting to the global address space gives global_load / global_store.
+#define HCCL_GLOBAL __attribute__((address_space(1)))
+typedef V4 HCCL_GLOBAL GlobalV4;
+typedef V4A4 HCCL_GLOBAL GlobalV4A4;
 
 template <uint32_t MODE> __device__ __forceinline__ V4 Load16(const void *base, uint64_t byteOff)
 {
     const char *p = static_cast<const char *>(base) + byteOff;
     if (MODE == ACC_VEC16) {
-        return __builtin_nontemporal_load(reinterpret_cast<const V4 *>(p));
+        return __builtin_nontemporal_load((const GlobalV4 *)p);
     } else {
-        Vec16A4 t = *reinterpret_cast<const Vec16A4 *>(p);
+        V4A4 t = *(const GlobalV4A4 *)p;
         return V4{t.x, t.y, t.z, t.w};
     }
 }
 __device__ __forceinline__ void Store16(void *base, uint64_t byteOff, V4 v)
 {
-    __builtin_nontemporal_store(v, reinterpret_cast<V4 *>(static_cast<char *>(base) + byteOff));
+    __builtin_nontemporal_store(v, (GlobalV4 *)(static_cast<char *>(base) + byteOff));
+}
+
+// Element-wise access to global memory (heads, tails, unaligned buffers).
+template <size_t N> struct ElemCarrier;
+template <> struct ElemCarrier<1> { typedef uint8_t type; };
+template <> struct ElemCarrier<2> { typedef uint16_t type; };
+template <> struct ElemCarrier<4> { typedef uint32_t type; };
+template <> struct ElemCarrier<8> { typedef uint64_t type; };
+template <typename T> __device__ __forceinline__ T LoadElem(const void *base, uint64_t byteOff)
+{
+    typedef typename ElemCarrier<sizeof(T)>::type C;
+    C c = *(const C HCCL_GLOBAL *)(static_cast<const char *>(base) + byteOff);
+    T t;
+    __builtin_memcpy(&t, &c, sizeof(T));
+    return t;
+}
+template <typename T> __device__ __forceinline__ void StoreElem(void *base, uint64_t byteOff, T t)
+{
+    typedef typename ElemCarrier<sizeof(T)>::type C;
+    C c;
+    __builtin_memcpy(&c, &t, sizeof(T));
+    *(C HCCL_GLOBAL *)(static_cast<char *>(base) + byteOff) = c;
 }
 
 // Largest i with table[i].tile0 <= tile (tile0 is ascending, table[0].tile0 == 0).
@@ -326,15 +355,13 @@ template <typename T, int OP>
 __device__ __forceinline__ void StepTileElem(const StepDesc &d, uint64_t off, uint32_t n)
 {
     const uint32_t cnt = n / sizeof(T);
-    T *dst = reinterpret_cast<T *>(static_cast<char *>(d.dst) + off);
-    const T *a = reinterpret_cast<const T *>(static_cast<const char *>(d.a) + off);
-    const T *b = d.b ? reinterpret_cast<const T *>(static_cast<const char *>(d.b) + off) : nullptr;
     for (uint32_t i = threadIdx.x; i < cnt; i += kBlockThreads) {
-        T v = a[i];
-        if (b != nullptr) {
-            v = Elem<T, OP>::Apply(v, b[i]);
+        const uint64_t at = off + uint64_t(i) * sizeof(T);
+        T v = LoadElem<T>(d.a, at);
+        if (d.b != nullptr) {
+            v = Elem<T, OP>::Apply(v, LoadElem<T>(d.b, at));
         }
-        dst[i] = v;
+        StoreElem<T>(d.dst, at, v);
     }
 }
 
@@ -373,8 +400,8 @@ template <uint32_t MODE> __device__ __forceinline__ void StoreAny16(void *base, 
     if (MODE == ACC_VEC16) {
         Store16(base, pos, v);
     } else {
-        Vec16A4 t{v.x, v.y, v.z, v.w};
-        *reinterpret_cast<Vec16A4 *>(static_cast<char *>(base) + pos) = t;
+        V4A4 t = {v.x, v.y, v.z, v.w};
+        *(GlobalV4A4 *)(static_cast<char *>(base) + pos) = t;
     }
 }
 
@@ -448,13 +475,13 @@ __device__ __forceinline__ void ChainElem(const FusedDesc &d, const void *const 
     const uint32_t cnt = n / sizeof(T);
     for (uint32_t i = threadIdx.x; i < cnt; i += kBlockThreads) {
         const uint64_t at = off + uint64_t(i) * sizeof(T);
-        T acc = *reinterpret_cast<const T *>(static_cast<const char *>(src[0]) + at);
+        T acc = LoadElem<T>(src[0], at);
         for (uint32_t j = 1; j < d.nsrc; j++) {
-            T v = *reinterpret_cast<const T *>(static_cast<const char *>(src[j]) + at);
+            T v = LoadElem<T>(src[j], at);
             acc = ((d.accLeftMask >> j) & 1ull) ? Elem<T, OP>::Apply(acc, v) : Elem<T, OP>::Apply(v, acc);
         }
         for (uint32_t k = 0; k < d.ndst; k++) {
-            *reinterpret_cast<T *>(static_cast<char *>(dst[k]) + at) = acc;
+            StoreElem<T>(dst[k], at, acc);
         }
     }
 }
@@ -504,12 +531,13 @@ constexpr uint32_t kTreeMaxGroups = 4;   // up to 32 leaves
 constexpr uint32_t kTreeVec = 2;         // vectors per lane per pass
 
 // Evaluates the tree for kTreeVec vectors of one lane (positions pos[u], skipped where !live[u]).
-template <typename T, int OP, uint32_t MODE, bool FULL>
+// G = leaves per group: 8 when the tree has 8 or more leaves, else the leaf count itself (1, 2, 4),
+// so that no group is ever partial and the loads of a group are issued back to back.
+template <typename T, int OP, uint32_t MODE, bool FULL, uint32_t G>
 __device__ __forceinline__ void TreeValue(const FusedDesc &d, const void *const *__restrict__ src,
     const uint64_t (&pos)[kTreeVec], const bool (&live)[kTreeVec], V4 (&x)[kTreeVec])
 {
-    const uint32_t nleaf = d.nleaf;
-    const uint32_t ngroups = (nleaf + kTreeGroup - 1) / kTreeGroup;   // 1, or a power of two
+    const uint32_t ngroups = d.nleaf / G;   // 1, 2 or 4
     // Pending left operands of the upper levels (a binary counter over the groups seen so far).
     V4 l0[kTreeVec], l1[kTreeVec];
 #pragma unroll
@@ -520,44 +548,57 @@ __device__ __forceinline__ void TreeValue(const FusedDesc &d, const void *const 
     // the register count (and with it the number of resident waves) is back to the flat version's.
 #pragma nounroll
     for (uint32_t gi = 0; gi < ngroups; gi++) {
-        const void *const *gs = src + 2 * gi * kTreeGroup;
-        const uint32_t left = nleaf - gi * kTreeGroup;   // leaves in this and later groups
-        V4 v[kTreeGroup][kTreeVec];
+        const void *const *gs = src + 2 * gi * G;
+        V4 v[G][kTreeVec];
 #pragma unroll
-        for (uint32_t i = 0; i < kTreeGroup; i++) {
-            if (i < left) {
-                const void *s = gs[2 * i];
+        for (uint32_t i = 0; i < G; i++) {
+            const void *s = gs[2 * i];
 #pragma unroll
-                for (uint32_t u = 0; u < kTreeVec; u++) {
-                    if (FULL || live[u]) {
-                        v[i][u] = Load16<MODE>(s, pos[u]);
-                    }
+            for (uint32_t u = 0; u < kTreeVec; u++) {
+                if (FULL || live[u]) {
+                    v[i][u] = Load16<MODE>(s, pos[u]);
                 }
             }
         }
+        // second sources of the leaves (folded rank pairs), four leaves at a time: all loads of a
+        // batch first, then the combines
+        constexpr uint32_t B = G >= 4 ? 4 : G;
 #pragma unroll
-        for (uint32_t i = 0; i < kTreeGroup; i++) {
-            if (i < left) {
-                const void *s = gs[2 * i + 1];
-                if (s != nullptr) {
+        for (uint32_t b0 = 0; b0 < G; b0 += B) {
+            V4 w[B][kTreeVec];
+            bool has[B];
+#pragma unroll
+            for (uint32_t i = 0; i < B; i++) {
+                const void *s = gs[2 * (b0 + i) + 1];
+                has[i] = s != nullptr;
+                if (has[i]) {
 #pragma unroll
                     for (uint32_t u = 0; u < kTreeVec; u++) {
                         if (FULL || live[u]) {
-                            v[i][u] = Combine16<T, OP>(v[i][u], Load16<MODE>(s, pos[u]));
+                            w[i][u] = Load16<MODE>(s, pos[u]);
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (uint32_t i = 0; i < B; i++) {
+                if (has[i]) {
+#pragma unroll
+                    for (uint32_t u = 0; u < kTreeVec; u++) {
+                        if (FULL || live[u]) {
+                            v[b0 + i][u] = Combine16<T, OP>(v[b0 + i][u], w[i][u]);
                         }
                     }
                 }
             }
         }
 #pragma unroll
-        for (uint32_t w = 1; w < kTreeGroup; w <<= 1) {
+        for (uint32_t w = 1; w < G; w <<= 1) {
 #pragma unroll
-            for (uint32_t i = 0; i + w < kTreeGroup; i += 2 * w) {
-                if (i + w < left) {
+            for (uint32_t i = 0; i + w < G; i += 2 * w) {
 #pragma unroll
-                    for (uint32_t u = 0; u < kTreeVec; u++) {
-                        v[i][u] = Combine16<T, OP>(v[i][u], v[i + w][u]);
-                    }
+                for (uint32_t u = 0; u < kTreeVec; u++) {
+                    v[i][u] = Combine16<T, OP>(v[i][u], v[i + w][u]);
                 }
             }
         }
@@ -591,7 +632,7 @@ __device__ __forceinline__ void TreeValue(const FusedDesc &d, const void *const 
 }
 
 // One pass over kTreeVec * 256 vectors starting at vector vecBase of the tile.
-template <typename T, int OP, uint32_t MODE, bool FULL>
+template <typename T, int OP, uint32_t MODE, bool FULL, uint32_t G>
 __device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *const *__restrict__ src,
     void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec)
 {
@@ -604,7 +645,7 @@ __device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *cons
         pos[u] = off + uint64_t(i) * 16;
     }
     V4 r[kTreeVec];
-    TreeValue<T, OP, MODE, FULL>(d, src, pos, live, r);
+    TreeValue<T, OP, MODE, FULL, G>(d, src, pos, live, r);
     const uint32_t ndst = d.ndst;
     for (uint32_t k = 0; k < ndst; k++) {
         void *o = dst[k];
@@ -613,6 +654,27 @@ __device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *cons
             if (live[u]) {
                 StoreAny16<MODE>(o, pos[u], r[u]);
             }
+        }
+    }
+}
+
+// All vector passes of one tile.
+template <typename T, int OP, uint32_t G>
+__device__ __forceinline__ void TreeTileVec(const FusedDesc &d, const void *const *__restrict__ src,
+    void *const *__restrict__ dst, uint64_t off, uint32_t nvec)
+{
+    constexpr uint32_t kPass = kTreeVec * kBlockThreads;
+    uint32_t base = 0;
+    if (d.mode == ACC_VEC16) {
+        for (; base + kPass <= nvec; base += kPass) {
+            TreeVecPass<T, OP, ACC_VEC16, true, G>(d, src, dst, off, base, nvec);
+        }
+        if (base < nvec) {
+            TreeVecPass<T, OP, ACC_VEC16, false, G>(d, src, dst, off, base, nvec);
+        }
+    } else {
+        for (; base < nvec; base += kPass) {
+            TreeVecPass<T, OP, ACC_VEC16_SRC4, false, G>(d, src, dst, off, base, nvec);
         }
     }
 }
@@ -629,10 +691,10 @@ __device__ __forceinline__ void TreeElem(const FusedDesc &d, const void *const *
 #pragma unroll
         for (uint32_t i = 0; i < kMax; i++) {
             if (i < d.nleaf) {
-                v[i] = *reinterpret_cast<const T *>(static_cast<const char *>(src[2 * i]) + at);
+                v[i] = LoadElem<T>(src[2 * i], at);
                 const void *s = src[2 * i + 1];
                 if (s != nullptr) {
-                    v[i] = Elem<T, OP>::Apply(v[i], *reinterpret_cast<const T *>(static_cast<const char *>(s) + at));
+                    v[i] = Elem<T, OP>::Apply(v[i], LoadElem<T>(s, at));
                 }
             }
         }
@@ -648,7 +710,7 @@ __device__ __forceinline__ void TreeElem(const FusedDesc &d, const void *const *
             }
         }
         for (uint32_t k = 0; k < d.ndst; k++) {
-            *reinterpret_cast<T *>(static_cast<char *>(dst[k]) + at) = v[0];
+            StoreElem<T>(dst[k], at, v[0]);
         }
     }
 }
@@ -668,19 +730,14 @@ __global__ void __launch_bounds__(kBlockThreads) TreeKernel(const FusedDesc *__r
             TreeElem<T, OP>(d, src, dst, off, n);
         } else {
             const uint32_t nvec = n >> 4;
-            constexpr uint32_t kPass = kTreeVec * kBlockThreads;
-            uint32_t base = 0;
-            if (d.mode == ACC_VEC16) {
-                for (; base + kPass <= nvec; base += kPass) {
-                    TreeVecPass<T, OP, ACC_VEC16, true>(d, src, dst, off, base, nvec);
-                }
-                if (base < nvec) {
-                    TreeVecPass<T, OP, ACC_VEC16, false>(d, src, dst, off, base, nvec);
-                }
+            if (d.nleaf >= kTreeGroup) {
+                TreeTileVec<T, OP, kTreeGroup>(d, src, dst, off, nvec);
+            } else if (d.nleaf == 4) {
+                TreeTileVec<T, OP, 4>(d, src, dst, off, nvec);
+            } else if (d.nleaf == 2) {
+                TreeTileVec<T, OP, 2>(d, src, dst, off, nvec);
             } else {
-                for (; base < nvec; base += kPass) {
-                    TreeVecPass<T, OP, ACC_VEC16_SRC4, false>(d, src, dst, off, base, nvec);
-                }
+                TreeTileVec<T, OP, 1>(d, src, dst, off, nvec);
             }
         }
     }
