@@ -22,7 +22,7 @@ METRIC = "achieved HBM GB/s & % of peak, 8-rank fp32 ring AllReduce 256MiB/rank"
 # (FETCH_SIZE, WRITE_SIZE), scaled by the same counters over a plain copy of known size.
 # Valid for the default workload only (8 ranks x 256 MiB); the figures and the commands are in
 # profiles/ChainKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt.
-MEASURED_TRAFFIC_BYTES = 4295754000
+MEASURED_TRAFFIC_BYTES = 4295456000
 
 
 def run_mode(pkg, torch, comms, stream, sends, recvs, n, fuse, steps, warmup):
@@ -48,6 +48,34 @@ def run_mode(pkg, torch, comms, stream, sends, recvs, n, fuse, steps, warmup):
     dev_ms = e0.elapsed_time(e1) / steps
     info = pkg.last_op_info(comms[0])
     return wall_ms, dev_ms, info
+
+
+def per_launch_times(pkg, torch, comms, stream, sends, recvs, n, fuse, steps):
+    """Median and minimum device time of single collectives (one event pair each), in ms."""
+    pkg.set_param(comms[0], "fuse", fuse)
+    sp = [t.data_ptr() for t in sends]
+    rp = [t.data_ptr() for t in recvs]
+    dt, op = pkg.HCCL_DATA_TYPE_FP32, pkg.HCCL_REDUCE_SUM
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    with torch.cuda.stream(stream):
+        for e0, e1 in pairs:
+            e0.record(stream)
+            pkg.all_reduce(comms, sp, rp, n, dt, op, stream.cuda_stream)
+            e1.record(stream)
+    stream.synchronize()
+    ts = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+    return ts[len(ts) // 2], ts[0]
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def time_calls(torch, stream, call, steps, warmup):
@@ -222,6 +250,7 @@ def main():
 
     wall_ms, dev_ms, info = run_mode(pkg, torch, comms, stream, sends, recvs, n, 1, args.steps, args.warmup)
     fused_out = recvs[0].cpu().numpy()
+    med_ms, min_ms = per_launch_times(pkg, torch, comms, stream, sends, recvs, n, 1, args.steps)
     s_wall_ms, s_dev_ms, s_info = run_mode(pkg, torch, comms, stream, sends, recvs, n, 0, args.steps, args.warmup)
     step_out = recvs[0].cpu().numpy()
     same_all = all(torch.equal(recvs[0], recvs[r]) for r in range(1, p))
@@ -244,9 +273,15 @@ def main():
             dt = time.perf_counter() - t0
             best = dt if best is None else min(best, dt)
         bit_exact = bool(np.array_equal(outs[0], fused_out) and np.array_equal(outs[0], step_out))
+        work = [x.copy() for x in ins]
+        t0 = time.perf_counter()
+        oracle.allreduce(work, oracle.FP32, oracle.SUM, flags=oracle.DIRECT | oracle.ZERO_STAGING, threads=1, outs=outs)
+        single = time.perf_counter() - t0
         cpu = {"value": round(sched / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
                "sample": "full workload (%d ranks x %.0f MiB fp32, out of place), checker in direct zero-staging "
-                         "mode, best of 3, %.3f s; bytes = (5p-3)S schedule figure" % (p, args.size_mib, best)}
+                         "mode, best of 3, %.3f s; bytes = (5p-3)S schedule figure" % (p, args.size_mib, best),
+               "single_thread_value": round(sched / single / 1e9, 3), "single_thread_s": round(single, 3),
+               "cpu_model": cpu_model()}
 
     if args.calibrate:
         one = pkg.comm_init_all(1)
@@ -297,6 +332,8 @@ def main():
             "bytes_per_step_schedule": sched,
             "pct_of_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBPS, 2),
             "sched_GBps": round(sched / (dev_ms * 1e-3) / 1e9, 1),
+            "launch_ms_median": round(med_ms, 4),
+            "launch_ms_min": round(min_ms, 4),
             "bit_exact_vs_host_reference": bit_exact,
             "all_ranks_identical": bool(same_all),
             "step_by_step": {
