@@ -149,7 +149,7 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
     uint32_t fusedPerCu = g->cfg.blocksPerCu;
     if (fusedPerCu == 0) {
         double streamBytes = 0, bytes = 0;
-        for (const FusedItem &it : pp->plan.fused) {
+        for (const FusedItem &it : pp->plan->fused) {
             uint32_t nsrc = 0;
             for (uint8_t v : it.srcValid) {
                 nsrc += v;
@@ -173,7 +173,7 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
         if (func == nullptr) {
             return HCCL_E_NOT_SUPPORT;
         }
-        for (const Phase &ph : pp->plan.phases) {
+        for (const Phase &ph : pp->plan->phases) {
             std::vector<StepDesc> descs;
             uint32_t tiles = 0;
             for (const Step &s : ph.steps) {
@@ -216,7 +216,7 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
             std::vector<const void *> srcPool;
             std::vector<void *> dstPool;
             uint32_t tiles = 0;
-            for (const FusedItem &it : pp->plan.fused) {
+            for (const FusedItem &it : pp->plan->fused) {
                 int want = (it.kind == FK_TREE) ? int(KK_TREE) : int(KK_CHAIN);
                 if (want != kind) {
                     continue;
@@ -361,6 +361,46 @@ std::string CacheKey(const Group *g, int algo)
     return key;
 }
 
+// Planning costs about a millisecond for 8 ranks and tens of milliseconds for 32; a plan depends on
+// the request only (sizes, schedule, which ranks run in place), not on addresses, so a caller that
+// comes back with other buffers gets the plan from here and pays for the pointer tables only.
+int CachedPlan(Group *g, const PlanRequest &rq, std::shared_ptr<const Plan> *out, std::string *err)
+{
+    std::string key;
+    auto put = [&](const void *p, size_t n) { key.append(static_cast<const char *>(p), n); };
+    auto putVec = [&](const std::vector<uint64_t> &v) {
+        uint64_t n = v.size();
+        put(&n, sizeof(n));
+        put(v.data(), v.size() * sizeof(uint64_t));
+    };
+    uint64_t head[10] = {uint64_t(rq.coll), uint64_t(rq.algo), rq.p, rq.count, rq.root, rq.peer, rq.unit, rq.cclBytes, rq.align,
+        uint64_t(rq.meshAtomic) | (uint64_t(rq.stageInput) << 1)};
+    put(head, sizeof(head));
+    put(rq.alias.data(), rq.alias.size());
+    putVec(rq.sendCounts);
+    putVec(rq.sdispls);
+    putVec(rq.recvCounts);
+    putVec(rq.rdispls);
+    putVec(rq.vCounts);
+    putVec(rq.vDispls);
+    auto it = g->planCache.find(key);
+    if (it != g->planCache.end()) {
+        *out = it->second;
+        return 0;
+    }
+    std::shared_ptr<Plan> fresh = std::make_shared<Plan>();
+    int rc = BuildPlan(rq, fresh.get(), err);
+    if (rc != 0) {
+        return rc;
+    }
+    if (g->planCache.size() >= 128) {
+        g->planCache.clear();   // plans in use stay alive through the prepared collectives that hold them
+    }
+    g->planCache[key] = fresh;
+    *out = fresh;
+    return 0;
+}
+
 HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
 {
     std::unique_ptr<Prepared> pp(new Prepared());
@@ -390,7 +430,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         rq.rdispls = g->ctx->rdispls;
     }
     std::string err;
-    int rc = BuildPlan(rq, &pp->plan, &err);
+    int rc = CachedPlan(g, rq, &pp->plan, &err);
     if (rc != 0) {
         HCCL_LOG_ERROR("%s: planning failed: %s", CollName(g->ctx->sig.coll), err.c_str());
         return rc == 1 ? HCCL_E_PARA : HCCL_E_INTERNAL;
@@ -403,11 +443,11 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         for (uint32_t j = 0; j < g->p; j++) {
             const char *rj = static_cast<const char *>(g->ctx->recv[j]);
             const char *sj = static_cast<const char *>(g->ctx->send[j]);
-            if (i != j && RangesOverlap(ri, pp->plan.recvBytes[i], rj, pp->plan.recvBytes[j])) {
+            if (i != j && RangesOverlap(ri, pp->plan->recvBytes[i], rj, pp->plan->recvBytes[j])) {
                 HCCL_LOG_ERROR("%s: receive buffers of rank %u and rank %u overlap", CollName(g->ctx->sig.coll), i, j);
                 return HCCL_E_PARA;
             }
-            if (RangesOverlap(ri, pp->plan.recvBytes[i], sj, pp->plan.sendBytes[j])) {
+            if (RangesOverlap(ri, pp->plan->recvBytes[i], sj, pp->plan->sendBytes[j])) {
                 bool exact = (i == j) && ri == sj && (g->ctx->sig.coll == COLL_ALLREDUCE || g->ctx->sig.coll == COLL_BROADCAST);
                 needStage = needStage || !exact;
             }
@@ -416,23 +456,22 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
     if (needStage) {
         rq.stageInput = true;
         rq.alias.assign(g->p, 0);
-        pp->plan = Plan();
-        rc = BuildPlan(rq, &pp->plan, &err);
+        rc = CachedPlan(g, rq, &pp->plan, &err);
         if (rc != 0) {
             HCCL_LOG_ERROR("%s: planning (staged) failed: %s", CollName(g->ctx->sig.coll), err.c_str());
             return HCCL_E_INTERNAL;
         }
     }
-    pp->fused = g->cfg.fuse && pp->plan.fusedOk && !needStage;
+    pp->fused = g->cfg.fuse && pp->plan->fusedOk && !needStage;
     if (pp->fused) {
-        for (const FusedItem &it : pp->plan.fused) {
+        for (const FusedItem &it : pp->plan->fused) {
             if (it.src.size() > 64 || (it.kind == FK_TREE && it.nleaf > 32)) {
                 pp->fused = false;   // beyond what the fused kernels encode
             }
         }
     }
-    if (!pp->fused && pp->plan.scratchBytes > 0) {
-        HcclResult r = EnsureScratch(g, pp->plan.scratchBytes);
+    if (!pp->fused && pp->plan->scratchBytes > 0) {
+        HcclResult r = EnsureScratch(g, pp->plan->scratchBytes);
         if (r != HCCL_SUCCESS) {
             return r;
         }
@@ -455,11 +494,11 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
     info.fused = pp->fused ? 1 : 0;
     info.graph = pp->exec ? 1 : 0;
     info.launches = uint32_t(pp->launches.size());
-    info.bytesRead = pp->fused ? pp->plan.fusedRead : pp->plan.stepRead;
-    info.bytesWritten = pp->fused ? pp->plan.fusedWritten : pp->plan.stepWritten;
-    info.stepRead = pp->plan.stepRead;
-    info.stepWritten = pp->plan.stepWritten;
-    info.scratchBytes = pp->fused ? 0 : pp->plan.scratchBytes;
+    info.bytesRead = pp->fused ? pp->plan->fusedRead : pp->plan->stepRead;
+    info.bytesWritten = pp->fused ? pp->plan->fusedWritten : pp->plan->stepWritten;
+    info.stepRead = pp->plan->stepRead;
+    info.stepWritten = pp->plan->stepWritten;
+    info.scratchBytes = pp->fused ? 0 : pp->plan->scratchBytes;
     *out = std::move(pp);
     return HCCL_SUCCESS;
 }

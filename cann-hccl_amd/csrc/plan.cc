@@ -1038,22 +1038,48 @@ bool BuildFused(const Sym &sym, const PlanRequest &rq, std::vector<FusedItem> *i
     // A fused launch reads every source and writes every destination in one pass, so a destination
     // may share memory with a source only when it is the same range of the same item (each thread
     // then reads its bytes before it overwrites them).  Only aliased ranks can overlap.
-    auto phys = [&](const Ref &r) { return (r.buf == BUF_SEND && rq.alias.size() == rq.p && rq.alias[r.rank]) ? uint8_t(BUF_RECV) : r.buf; };
+    // Sources are ranges of send buffers and destinations ranges of receive buffers, so only ranks
+    // whose two buffers are the same memory need the check.
+    if (rq.alias.size() != rq.p) {
+        return true;
+    }
+    struct Span {
+        uint64_t off, end;
+        size_t item;
+    };
+    std::vector<std::vector<Span>> srcOf(rq.p);
+    for (size_t j = 0; j < items->size(); j++) {
+        const FusedItem &it = (*items)[j];
+        for (size_t k = 0; k < it.src.size(); k++) {
+            const Ref &sr = it.src[k];
+            if (it.srcValid[k] && sr.buf == BUF_SEND && rq.alias[sr.rank] && it.bytes) {
+                srcOf[sr.rank].push_back(Span{sr.off, sr.off + it.bytes, j});
+            }
+        }
+    }
+    std::vector<std::vector<uint64_t>> maxEnd(rq.p);   // running maximum of Span::end in offset order
+    for (uint32_t r = 0; r < rq.p; r++) {
+        std::sort(srcOf[r].begin(), srcOf[r].end(), [](const Span &x, const Span &y) { return x.off < y.off; });
+        maxEnd[r].resize(srcOf[r].size());
+        uint64_t m = 0;
+        for (size_t i = 0; i < srcOf[r].size(); i++) {
+            m = std::max(m, srcOf[r][i].end);
+            maxEnd[r][i] = m;
+        }
+    }
     for (size_t i = 0; i < items->size(); i++) {
+        const uint64_t len = (*items)[i].bytes;
         for (const Ref &d : (*items)[i].dst) {
-            for (size_t j = 0; j < items->size(); j++) {
-                const FusedItem &other = (*items)[j];
-                for (size_t k = 0; k < other.src.size(); k++) {
-                    if (!other.srcValid[k]) {
-                        continue;
-                    }
-                    const Ref &s = other.src[k];
-                    if (s.rank != d.rank || phys(s) != phys(d)) {
-                        continue;
-                    }
-                    if (Overlap(s.off, other.bytes, d.off, (*items)[i].bytes) && !(i == j && s.off == d.off)) {
-                        return false;
-                    }
+            if (d.buf != BUF_RECV || !rq.alias[d.rank] || len == 0) {
+                continue;
+            }
+            const std::vector<Span> &v = srcOf[d.rank];
+            // candidates start below the destination's end; walk down while anything can still reach it
+            size_t hi = std::lower_bound(v.begin(), v.end(), d.off + len, [](const Span &x, uint64_t e) { return x.off < e; }) -
+                v.begin();
+            for (size_t k = hi; k-- > 0 && maxEnd[d.rank][k] > d.off;) {
+                if (v[k].end > d.off && !(v[k].item == i && v[k].off == d.off)) {
+                    return false;
                 }
             }
         }

@@ -62,7 +62,7 @@ struct OpInfo {
 };
 
 struct Prepared {
-    Plan plan;
+    std::shared_ptr<const Plan> plan;   // shared with the group's plan cache (plans do not depend on addresses)
     bool fused = false;
     void *devTables = nullptr;
     std::vector<LaunchRec> launches;
@@ -146,6 +146,7 @@ struct Group {
     uint64_t scratchBytes = 0;
     uint64_t scratchGen = 0;
     std::unordered_map<std::string, std::unique_ptr<Prepared>> cache;
+    std::unordered_map<std::string, std::shared_ptr<const Plan>> planCache;   // keyed by the plan request
     uint64_t useClock = 0;
     OpInfo lastInfo;
 
