@@ -1448,8 +1448,9 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
     PlanRequest rq;
     rq.coll = CollKind(coll);
     if (coll >= COLL_BROADCAST) {
-        rq.root = uint32_t(algo);   // rooted collectives have one schedule each; the argument carries the root
-        rq.algo = ALGO_RING;
+        // rooted collectives: low 16 bits = root rank, bits 16.. = schedule (0 ring, 1 mesh, 4 mesh uncut)
+        rq.root = uint32_t(algo) & 0xffffu;
+        rq.algo = Algo(uint32_t(algo) >> 16);
     } else {
         rq.algo = Algo(algo);
     }

@@ -568,16 +568,19 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     int algo = g->cfg.algo >= 0 ? g->cfg.algo : DefaultAlgo(g->ctx->sig.coll);
     if (g->ctx->sig.coll == COLL_ALLTOALLV) {
         algo = ALGO_PAIRWISE;
-    } else if (g->ctx->sig.coll >= COLL_BROADCAST) {
-        algo = ALGO_RING;   // one schedule each: ring broadcast, ring reduce, mesh scatter
+    } else if (g->ctx->sig.coll == COLL_BROADCAST || g->ctx->sig.coll == COLL_REDUCE) {
+        algo = (algo == ALGO_MESH) ? ALGO_MESH : ALGO_RING;   // ring or mesh broadcast / reduce
+    } else if (g->ctx->sig.coll >= COLL_SCATTER) {
+        algo = ALGO_RING;   // one schedule each: mesh scatter, direct send / receive
     } else if (algo == ALGO_PAIRWISE) {
         algo = ALGO_RING;
     }
-    // coll_all_reduce_mesh_executor.cc:108-112, coll_reduce_scatter_mesh_executor.cc:227-229: without the
+    // coll_all_reduce_mesh_executor.cc:108-112, coll_reduce_scatter_mesh_executor.cc:227-229,
+    // coll_reduce_mesh_executor.cc:93-97: without the
     // deterministic setting the mesh reduce phases run uncut, except for int64 and for products
     if (algo == ALGO_MESH && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
         g->ctx->sig.op != HCCL_REDUCE_PROD &&
-        (g->ctx->sig.coll == COLL_ALLREDUCE || g->ctx->sig.coll == COLL_REDUCESCATTER)) {
+        (g->ctx->sig.coll == COLL_ALLREDUCE || g->ctx->sig.coll == COLL_REDUCESCATTER || g->ctx->sig.coll == COLL_REDUCE)) {
         algo = ALGO_MESH_ATOMIC;
     }
     std::string key = CacheKey(g, algo);

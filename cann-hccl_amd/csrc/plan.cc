@@ -386,7 +386,40 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
         uint64_t done = 0;
         for (uint64_t left = rq.count; left > 0;) {
             uint64_t cur = std::min(left, per), bytes = cur * u;
-            if (rq.coll == COLL_BROADCAST) {
+            if (rq.coll == COLL_BROADCAST && rq.algo == ALGO_MESH) {
+                // mesh broadcast (coll_broadcast_mesh_executor.cc:59-213): the root scatters slice i to
+                // rank i (scatter_mesh.cc), then a mesh all-gather; slices from GetRankSliceSize
+                // (coll_broadcast_executor.cc:275-306).  The root keeps its data where it is.
+                uint64_t avg = bytes / p + ((cur % p) > 0 ? 1 : 0);
+                uint64_t slice = RoundUpTo(avg, rq.align);
+                std::vector<Slice> sl(p);
+                uint64_t residue = bytes;
+                for (uint32_t i = 0; i < p; i++) {
+                    sl[i].size = std::min(slice, residue);
+                    sl[i].off = sl[i].size == 0 ? 0 : uint64_t(i) * slice;
+                    residue -= sl[i].size;
+                }
+                for (uint32_t r = 0; r < p; r++) {
+                    if (r != R) {
+                        EmitCopy(*vp, 0, MkRef(r, BUF_RECV, done + sl[r].off), MkRef(R, BUF_SEND, done + sl[r].off), sl[r].size);
+                    }
+                }
+                for (uint32_t r = 0; r < p; r++) {
+                    for (uint32_t k = 1; k < p && r != R; k++) {
+                        uint32_t d = (r + k) % p;
+                        Ref src = (d == R) ? MkRef(R, BUF_SEND, done + sl[d].off) : MkRef(d, BUF_RECV, done + sl[d].off);
+                        EmitCopy(*vp, 1, MkRef(r, BUF_RECV, done + sl[d].off), src, sl[d].size);
+                    }
+                }
+            } else if (rq.coll == COLL_REDUCE && rq.algo == ALGO_MESH && p > 1) {
+                // mesh reduce (coll_reduce_mesh_executor.cc:75-194): mesh reduce-scatter over the ring
+                // slice plan, then the root gathers slice r from rank r (gather_mesh.cc:60-170)
+                std::vector<Slice> sl = RingSlicePlan(bytes, p, rq.align);
+                size_t ph = MeshReduceScatterPhases(*vp, 0, p, done, sl, rq.align, rq.meshAtomic);
+                for (uint32_t r = 0; r < p; r++) {
+                    EmitCopy(*vp, ph, MkRef(R, BUF_RECV, done + sl[r].off), MkRef(r, BUF_SEND, done + sl[r].off), sl[r].size);
+                }
+            } else if (rq.coll == COLL_BROADCAST) {
                 // ring broadcast (broadcast_ring.cc:24-160): the chunk is cut into p slices that travel
                 // root -> root+1 -> ... -> root-1 as a pipeline; slice j reaches distance d in phase j+d-1
                 uint64_t sizeAvg = ((cur + p - 1) / p) * u;

@@ -45,7 +45,8 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
 
 /* Plans a collective without a device and writes the plan as JSON (phases of copy / reduce steps,
  * fused items, byte counts) into out[0..cap).  coll / algo as in HcclAmdOpInfo; for the rooted
- * collectives (coll 4 broadcast, 5 reduce, 6 scatter) the algo argument carries the root rank.  inPlaceMask bit r:
+ * collectives (coll 4 broadcast, 5 reduce, 6 scatter) the algo argument carries the root rank in its low 16 bits and the
+ * schedule above them (0 ring, 1 mesh, 4 mesh without the piece cut; reduce only).  inPlaceMask bit r:
  * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64
  * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); for the variable-count
  * reduce-scatter / all-gather, tables points to 2*p uint64 (block counts, block displacements); else NULL.

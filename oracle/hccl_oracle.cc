@@ -23,7 +23,8 @@
 //                    TPL/temp_all_gather/all_gather_halving_doubling.cc:43-196
 //   pairwise         TPL/temp_alltoallv/alltoallv_pairwise.cc:75-282, ALG/impl/operator/alltoall_operator.cc:49-72
 //   rooted           TPL/temp_broadcast/broadcast_ring.cc:24-160, TPL/temp_reduce/reduce_ring.cc:29-154,
-//                    TPL/temp_scatter/scatter_mesh.cc:46-160
+//                    TPL/temp_scatter/scatter_mesh.cc:46-160, TPL/temp_gather/gather_mesh.cc:60-170,
+//                    EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213, EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194
 //
 // Method: every template is restated as the per-rank program it issues (send / receive-and-reduce /
 // receive-and-copy / local copy), one virtual process per rank (per rank and stream for the mesh),
@@ -1382,6 +1383,172 @@ int orc_broadcast(uint32_t p, void **buf, uint64_t count, int dt, uint32_t root,
     }
     return 0;
 }
+
+// Mesh broadcast, CollBroadcastMeshExecutor::KernelRun (EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213)
+// on one server: the root scatters slice i to rank i (TPL/temp_scatter/scatter_mesh.cc:46-160), then a mesh
+// all-gather; slices from GetRankSliceSize (EXE/coll_broadcast/coll_broadcast_executor.cc:275-306).
+int orc_broadcast_mesh(uint32_t p, void **buf, uint64_t count, int dt, uint32_t root, uint64_t cclBytes, uint64_t align,
+    int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0 && p > 1;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            m.buf[B_IN][r] = static_cast<uint8_t *>(buf[r]) + offset;
+            m.buf[B_OUT][r] = static_cast<uint8_t *>(buf[r]) + offset;
+        }
+        uint64_t avg = bytes / p + ((cur % p) > 0 ? 1 : 0);
+        uint64_t per = RoundUp(avg, align);
+        std::vector<Slice> sl(p);
+        uint64_t residue = bytes;
+        for (uint32_t i = 0; i < p; i++) {
+            sl[i].size = per < residue ? per : residue;
+            sl[i].off = sl[i].size == 0 ? 0 : i * per;
+            residue -= sl[i].size;
+        }
+        for (uint32_t r = 0; r < p; r++) {          // stage 0: scatter from the root
+            Proc pr;
+            pr.rank = r;
+            if (r == root) {
+                for (uint32_t d = 0; d < p; d++) {
+                    if (d != root) {
+                        pr.prog.push_back(MkSend(static_cast<int>(d), 0, B_IN, sl[d].off, sl[d].size));
+                    }
+                }
+            } else {
+                pr.prog.push_back(MkRecvCopy(static_cast<int>(root), 0, B_OUT, sl[r].off, sl[r].size));
+            }
+            m.procs.push_back(std::move(pr));
+        }
+        int rc = m.Run();
+        if (rc != 0) {
+            return rc;
+        }
+        for (uint32_t r = 0; r < p; r++) {          // stage 2: all-gather of the slices
+            Proc pr;
+            pr.rank = r;
+            ProgAllGatherMesh(pr.prog, r, p, B_OUT, sl);
+            m.procs.push_back(std::move(pr));
+        }
+        rc = m.Run();
+        if (rc != 0) {
+            return rc;
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
+// Mesh reduce, CollReduceMeshExecutor::KernelRun (EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194) on one
+// server: mesh reduce-scatter (piece cut, or uncut when `atomic`) over the ring slice plan, the own slice
+// copied from input to output, then GatherMesh to the root (TPL/temp_gather/gather_mesh.cc:60-170).
+int orc_reduce_to_root_mesh(uint32_t p, void **in, void *outRoot, uint64_t count, int dt, int op, uint32_t root,
+    uint64_t cclBytes, uint64_t align, int atomic, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.op = op;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    uint64_t stage = std::min<uint64_t>(count, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage)), cclOut(p, std::vector<uint8_t>(stage));
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_IN][r] = cclIn[r].data();
+        m.buf[B_OUT][r] = cclOut[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            m.Copy(m.buf[B_IN][r], static_cast<uint8_t *>(in[r]) + offset, bytes);
+        }
+        if (p == 1) {
+            m.Copy(m.buf[B_OUT][0], m.buf[B_IN][0], bytes);
+        } else {
+            std::vector<Slice> sl = RingSlices(bytes, p, align);
+            if (atomic) {
+                for (uint32_t r = 0; r < p; r++) {
+                    Proc pr;
+                    pr.rank = r;
+                    ProgReduceScatterMeshAtomic(pr.prog, r, p, B_IN, sl);
+                    m.procs.push_back(std::move(pr));
+                }
+            } else {
+                uint32_t nstream = p > 2 ? p - 1 : 1;
+                std::vector<std::vector<Slice>> pieces = CutPieces(sl, nstream, align);
+                for (uint32_t t = 0; t < nstream; t++) {
+                    for (uint32_t r = 0; r < p; r++) {
+                        Proc pr;
+                        pr.rank = r;
+                        ProgReduceScatterMeshStream(pr.prog, r, p, t, B_IN, pieces[t]);
+                        m.procs.push_back(std::move(pr));
+                    }
+                }
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+            for (uint32_t r = 0; r < p; r++) {      // one server: the level-1 reduce is a copy input -> output
+                m.Copy(m.At(r, B_OUT, sl[r].off), m.At(r, B_IN, sl[r].off), sl[r].size);
+            }
+            for (uint32_t r = 0; r < p; r++) {      // gather to the root
+                Proc pr;
+                pr.rank = r;
+                if (r == root) {
+                    for (uint32_t srcRank = 0; srcRank < p; srcRank++) {
+                        if (srcRank != root) {
+                            pr.prog.push_back(MkRecvCopy(static_cast<int>(srcRank), 0, B_OUT, sl[srcRank].off, sl[srcRank].size));
+                        }
+                    }
+                } else {
+                    pr.prog.push_back(MkSend(static_cast<int>(root), 0, B_OUT, sl[r].off, sl[r].size));
+                }
+                m.procs.push_back(std::move(pr));
+            }
+            rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        m.Copy(static_cast<uint8_t *>(outRoot) + offset, m.buf[B_OUT][root], bytes);
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
 
 // Ring reduce (reduce_ring.cc:29-154) with the executor's chunk loop; out[root] receives the result.
 // Inputs are staged (the schedule accumulates in its input buffer).

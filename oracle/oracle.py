@@ -64,6 +64,8 @@ def lib():
         L.orc_allgather_v.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), pu64, pu64, i32, i32, i32]
         L.orc_broadcast.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, i32, i32]
+        L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
+        L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
         L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
         L.orc_alltoallv.argtypes = [u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, u64, i32, i32]
         L.orc_fill_uniform_f32.argtypes = [vp, u64, u64, u32, i32]
@@ -220,17 +222,23 @@ def allgather_v(ins, counts, displs, out_len, dt, algo=RING, flags=0, threads=1,
     return outs
 
 
-def broadcast(bufs, dt, root, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1):
-    """bufs: p equal-length arrays, written in place: every array becomes bufs[root]."""
-    rc = lib().orc_broadcast(len(bufs), _ptrs(bufs), bufs[0].size, dt, root, ccl_bytes, align, flags, threads)
+def broadcast(bufs, dt, root, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1, algo=RING):
+    """bufs: p equal-length arrays, written in place: every array becomes bufs[root].  algo: RING or MESH."""
+    fn = lib().orc_broadcast_mesh if algo == MESH else lib().orc_broadcast
+    rc = fn(len(bufs), _ptrs(bufs), bufs[0].size, dt, root, ccl_bytes, align, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle broadcast failed rc=%d" % rc)
     return bufs
 
 
-def reduce_to_root(ins, dt, op, root, ccl_bytes=DEFAULT_CCL_BYTES, flags=0, threads=1):
+def reduce_to_root(ins, dt, op, root, ccl_bytes=DEFAULT_CCL_BYTES, flags=0, threads=1, algo=RING, align=DEFAULT_ALIGN):
+    """algo: RING, MESH (piece cut) or MESH_ATOMIC (uncut, streams in index order)."""
     out = np.empty_like(ins[0])
-    rc = lib().orc_reduce_to_root(len(ins), _ptrs(ins), out.ctypes.data, ins[0].size, dt, op, root, ccl_bytes, flags, threads)
+    if algo in (MESH, MESH_ATOMIC):
+        rc = lib().orc_reduce_to_root_mesh(len(ins), _ptrs(ins), out.ctypes.data, ins[0].size, dt, op, root, ccl_bytes, align,
+                                           1 if algo == MESH_ATOMIC else 0, flags, threads)
+    else:
+        rc = lib().orc_reduce_to_root(len(ins), _ptrs(ins), out.ctypes.data, ins[0].size, dt, op, root, ccl_bytes, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle reduce failed rc=%d" % rc)
     return out

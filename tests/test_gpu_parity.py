@@ -528,6 +528,41 @@ def test_broadcast_reduce_scatter_rooted(orc):
                 g.close()
 
 
+def test_broadcast_and_reduce_mesh_schedules(orc):
+    n = 70001
+    for p in (3, 8):
+        for algo in (MESH, MESH_ATOMIC):
+            for fuse in (1, 0):
+                g = _group(p, algo, fuse=fuse)
+                try:
+                    root = p - 2
+                    print("rooted mesh p", p, "algo", algo, "fuse", fuse, flush=True)
+                    bufs_np = _ins(INT32, p, n, 190 + p)
+                    bufs = [gh.to_dev(x) for x in bufs_np]
+                    torch.cuda.synchronize()
+                    H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, INT32, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    assert g.info()["algo"] == MESH
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(bufs[r], INT32), bufs_np[root]), ("bcast mesh", p, fuse, r)
+                    for dt, op in ((FP32, SUM), (BF16, SUM), (INT64, SUM), (FP16, PROD)):
+                        ins = _ins(dt, p, n, 191 + p + dt)
+                        want = orc.reduce_to_root(ins, dt, op, root, algo=_expected_algo(algo, dt, op))
+                        sends = [gh.to_dev(x) for x in ins]
+                        recvs = [gh.empty_dev(n * H.DTYPE_SIZE[dt], fill=0x33) for _ in range(p)]
+                        torch.cuda.synchronize()
+                        H.reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, op, root, g.stream_ptr)
+                        g.stream.synchronize()
+                        assert g.info()["algo"] == _expected_algo(algo, dt, op)
+                        assert gh.same(dt, gh.to_host(recvs[root], dt), want), ("reduce mesh", p, algo, fuse, dt)
+                        for r in range(p):
+                            assert np.array_equal(gh.to_host(sends[r], dt), ins[r])
+                            if r != root:
+                                assert bool((recvs[r] == 0x33).all())
+                finally:
+                    g.close()
+
+
 def test_one_thread_per_rank_blocking_arrival(orc):
     # the reference's model: every rank on its own thread and stream; calls return once the collective is issued
     import threading

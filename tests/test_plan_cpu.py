@@ -225,3 +225,43 @@ def test_rooted_plans_match_checker(orc, p):
             (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, INT32, 0)
             for r in range(p):
                 assert np.array_equal(recvs[r].view(np.int32), want[r]) and np.array_equal(want[r], src[r * n:(r + 1) * n])
+
+
+@pytest.mark.parametrize("p", [1, 2, 3, 5, 8])
+def test_rooted_mesh_plans_match_checker(orc, p):
+    # mesh broadcast (scatter + all-gather) and mesh reduce (mesh reduce-scatter + gather to the root)
+    n = 1003
+    for root in sorted({0, p - 1, p // 2}):
+        for ccl, align in ((200 << 20, 128), (1024, 128), (200 << 20, 4)):
+            bufs = _ins(INT32, p, n, 150 + p)
+            want = orc.broadcast([b.copy() for b in bufs], INT32, root, ccl_bytes=ccl, align=align, algo=MESH)
+            assert all(np.array_equal(w, bufs[root]) for w in want)
+            plan = H.describe_plan(H.COLL_BROADCAST, root | (MESH << 16), p, n, INT32, ccl_bytes=ccl, align=align,
+                                   in_place_mask=(1 << p) - 1)
+            if p > 1:
+                assert len(plan["phases"]) == 2
+            for fused in (False, True):
+                mem = _bytes(bufs)
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, mem, mem, INT32, 0, in_place=True)
+                for r in range(p):
+                    assert np.array_equal(mem[r].view(np.int32), want[r]), ("bcast mesh", p, root, ccl, fused, r)
+        for algo in (MESH, MESH_ATOMIC):
+            for dt, op in ((FP32, SUM), (BF16, SUM), (INT8, MIN)):
+                unit = H.DTYPE_SIZE[dt]
+                ins = _ins(dt, p, n, 160 + p + dt)
+                want = orc.reduce_to_root(ins, dt, op, root, ccl_bytes=2048, algo=algo)
+                closed = (cf.mesh_allreduce if algo == MESH else cf.mesh_atomic_allreduce)(dt, op, ins, unit, 2048, 128)[0]
+                assert _same(dt, want.view(np.uint8), closed), ("reduce mesh closed form", p, root, algo, dt)
+                plan = H.describe_plan(H.COLL_REDUCE, root | (algo << 16), p, n, dt, ccl_bytes=2048)
+                for fused in (False, True):
+                    if fused and not plan["fusedOk"]:
+                        continue
+                    sends = _bytes(ins)
+                    recvs = [np.full(n * unit, 0x77, np.uint8) for _ in range(p)]
+                    (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+                    assert _same(dt, recvs[root], want), ("reduce mesh", p, root, algo, dt, fused)
+                    for r in range(p):
+                        assert np.array_equal(sends[r], ins[r].view(np.uint8))
+                        if r != root:
+                            assert np.all(recvs[r] == 0x77)
+                assert plan["fusedOk"]
