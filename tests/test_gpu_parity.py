@@ -528,6 +528,27 @@ def test_broadcast_reduce_scatter_rooted(orc):
                 g.close()
 
 
+def test_order_sensitive_known_answers_on_the_gpu():
+    # hand-derived fp32 sums that differ between ring, the two mesh variants and halving-doubling
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_fp32.json")) as f:
+        kat = json.load(f)
+    xs = [np.array(v, np.float32) for v in kat["inputs"]]
+    p = kat["ranks"]
+    for name, algo in (("ring", RING), ("mesh", MESH), ("mesh_uncut", MESH_ATOMIC), ("rhd", RHD)):
+        for fuse in (1, 0):
+            g = _group(p, algo, fuse=fuse, align=kat["align"])
+            try:
+                print("order KAT", name, "fuse", fuse, flush=True)
+                outs, _ = gh.all_reduce(g, xs, FP32, SUM)
+                for r in range(p):
+                    assert float(outs[r][0]) == kat["expected_element0"][name], (name, fuse, r, float(outs[r][0]))
+                    assert np.array_equal(outs[r][1:], np.zeros(3, np.float32))
+            finally:
+                g.close()
+
+
 def test_broadcast_and_reduce_mesh_schedules(orc):
     n = 70001
     for p in (3, 8):

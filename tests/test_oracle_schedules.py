@@ -300,3 +300,23 @@ def test_uniform_fill_is_counter_based(orc):
     c = orc.fill_uniform_f32(100000, 42, 4)
     assert np.array_equal(a, b) and not np.array_equal(a, c)
     assert a.min() >= -1.0 and a.max() < 1.0 and abs(float(a.mean())) < 0.01
+
+
+def _order_kat():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_fp32.json")) as f:
+        return json.load(f)
+
+
+def test_order_sensitive_known_answers_all_schedules(orc):
+    # one hand-derived input on which ring, both mesh variants and halving-doubling give four different sums
+    kat = _order_kat()
+    xs = [np.array(v, np.float32) for v in kat["inputs"]]
+    for name, algo in (("ring", RING), ("mesh", MESH), ("mesh_uncut", MESH_ATOMIC), ("rhd", RHD)):
+        got = orc.allreduce([x.copy() for x in xs], FP32, SUM, algo=algo, align=kat["align"])
+        assert all(float(g[0]) == kat["expected_element0"][name] for g in got), (name, [float(g[0]) for g in got])
+        assert all(np.array_equal(g[1:], np.zeros(3, np.float32)) for g in got)
+        # and the closed forms agree with the hand derivation
+        want = CLOSED[algo](FP32, SUM, xs, 4, 200 << 20, kat["align"])
+        assert float(want[0][0]) == kat["expected_element0"][name], name

@@ -265,3 +265,20 @@ def test_rooted_mesh_plans_match_checker(orc, p):
                         if r != root:
                             assert np.all(recvs[r] == 0x77)
                 assert plan["fusedOk"]
+
+
+def test_order_sensitive_known_answers_through_the_planner():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_fp32.json")) as f:
+        kat = json.load(f)
+    xs = [np.array(v, np.float32) for v in kat["inputs"]]
+    p = kat["ranks"]
+    for name, algo in (("ring", RING), ("mesh", MESH), ("mesh_uncut", MESH_ATOMIC), ("rhd", RHD)):
+        plan = H.describe_plan(H.COLL_ALLREDUCE, algo, p, 4, FP32, align=kat["align"])
+        for fused in (False, True):
+            sends = _bytes(xs)
+            recvs = [np.full(16, 0xA5, np.uint8) for _ in range(p)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, FP32, SUM)
+            for r in range(p):
+                assert float(recvs[r].view(np.float32)[0]) == kat["expected_element0"][name], (name, fused, r)
