@@ -568,8 +568,10 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     int algo = g->cfg.algo >= 0 ? g->cfg.algo : DefaultAlgo(g->ctx->sig.coll);
     if (g->ctx->sig.coll == COLL_ALLTOALLV) {
         algo = ALGO_PAIRWISE;
-    } else if (g->ctx->sig.coll == COLL_BROADCAST || g->ctx->sig.coll == COLL_REDUCE) {
-        algo = (algo == ALGO_MESH) ? ALGO_MESH : ALGO_RING;   // ring or mesh broadcast / reduce
+    } else if (g->ctx->sig.coll == COLL_REDUCE) {
+        algo = (algo == ALGO_MESH || algo == ALGO_RHD) ? algo : ALGO_RING;   // ring, mesh or halving-doubling reduce
+    } else if (g->ctx->sig.coll == COLL_BROADCAST) {
+        algo = (algo == ALGO_MESH) ? ALGO_MESH : ALGO_RING;   // ring or mesh broadcast
     } else if (g->ctx->sig.coll >= COLL_SCATTER) {
         algo = ALGO_RING;   // one schedule each: mesh scatter, direct send / receive
     } else if (algo == ALGO_PAIRWISE) {

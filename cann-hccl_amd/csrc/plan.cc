@@ -139,6 +139,29 @@ size_t MeshAllGatherPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t bas
     return phase0 + 1;
 }
 
+// Halving steps of the in-block reduce-scatter (reduce_scatter_halving_doubling.cc:67-91,193-238): in
+// step s block rank q keeps the half of its current range that contains its own slice and combines
+// it with the same range of block rank q ^ mask.
+size_t HalvingSteps(VProgram &vp, size_t ph, uint32_t block, const std::vector<uint32_t> &rankOf, uint64_t base,
+    const std::vector<Slice> &sl)
+{
+    uint32_t steps = 0;
+    while ((1u << steps) < block) {
+        steps++;
+    }
+    for (uint32_t s = 0; s < steps; s++) {
+        uint32_t mask = 1u << (steps - s - 1);
+        for (uint32_t q = 0; q < block; q++) {
+            uint32_t first = q & ~(mask - 1);
+            uint64_t off = base + sl[first].off;
+            EmitReduce(vp, ph, MkRef(rankOf[q], BUF_SEND, off), MkRef(rankOf[q], BUF_SEND, off),
+                MkRef(rankOf[q ^ mask], BUF_SEND, off), SpanBytes(sl, first, mask));
+        }
+        ph++;
+    }
+    return ph;
+}
+
 void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t bytes, uint64_t align, bool meshAtomic)
 {
     if (p == 1) {
@@ -187,16 +210,7 @@ void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t
         }
         ph++;
     }
-    for (uint32_t s = 0; s < steps; s++) {           // halving: keep the half that contains the own slice
-        uint32_t mask = 1u << (steps - s - 1);
-        for (uint32_t q = 0; q < block; q++) {
-            uint32_t first = q & ~(mask - 1);
-            uint64_t off = base + sl[first].off;
-            EmitReduce(vp, ph, MkRef(rankOf[q], BUF_SEND, off), MkRef(rankOf[q], BUF_SEND, off),
-                MkRef(rankOf[q ^ mask], BUF_SEND, off), SpanBytes(sl, first, mask));
-        }
-        ph++;
-    }
+    ph = HalvingSteps(vp, ph, block, rankOf, base, sl);
     for (uint32_t q = 0; q < block; q++) {
         EmitCopy(vp, ph, MkRef(rankOf[q], BUF_RECV, base + sl[q].off), MkRef(rankOf[q], BUF_SEND, base + sl[q].off), sl[q].size);
     }
@@ -418,6 +432,32 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                 size_t ph = MeshReduceScatterPhases(*vp, 0, p, done, sl, rq.align, rq.meshAtomic);
                 for (uint32_t r = 0; r < p; r++) {
                     EmitCopy(*vp, ph, MkRef(R, BUF_RECV, done + sl[r].off), MkRef(r, BUF_SEND, done + sl[r].off), sl[r].size);
+                }
+            } else if (rq.coll == COLL_REDUCE && rq.algo == ALGO_RHD && p > 1) {
+                // recursive halving-doubling reduce (reduce_recursive_hd.cc:31-316): in every rank pair of
+                // part one the rank with the root's parity folds its neighbour in (:85-148), the block
+                // runs the halving reduce-scatter (:150-183), and a binomial gather over the output
+                // buffers brings the slices to the root (:236-313).  The gather only forwards finished
+                // slices, so here the root takes each slice from the rank that reduced it.
+                uint32_t block, part1;
+                HalvingDoublingShape(p, &block, &part1);
+                const uint32_t par = (R >= part1 ? 0u : R) % 2;
+                std::vector<uint32_t> rankOf(block);
+                for (uint32_t b = 0; b < block; b++) {
+                    rankOf[b] = b < part1 / 2 ? 2 * b + par : b + part1 / 2;
+                }
+                std::vector<Slice> sl = RingSlicePlan(bytes, block, rq.align);
+                size_t ph = 0;
+                if (part1 > 0) {
+                    for (uint32_t b = 0; b < part1 / 2; b++) {
+                        uint32_t mbr = rankOf[b], other = mbr ^ 1u;
+                        EmitReduce(*vp, ph, MkRef(mbr, BUF_SEND, done), MkRef(mbr, BUF_SEND, done), MkRef(other, BUF_SEND, done), bytes);
+                    }
+                    ph++;
+                }
+                ph = HalvingSteps(*vp, ph, block, rankOf, done, sl);
+                for (uint32_t b = 0; b < block; b++) {
+                    EmitCopy(*vp, ph, MkRef(R, BUF_RECV, done + sl[b].off), MkRef(rankOf[b], BUF_SEND, done + sl[b].off), sl[b].size);
                 }
             } else if (rq.coll == COLL_BROADCAST) {
                 // ring broadcast (broadcast_ring.cc:24-160): the chunk is cut into p slices that travel

@@ -24,7 +24,8 @@
 //   pairwise         TPL/temp_alltoallv/alltoallv_pairwise.cc:75-282, ALG/impl/operator/alltoall_operator.cc:49-72
 //   rooted           TPL/temp_broadcast/broadcast_ring.cc:24-160, TPL/temp_reduce/reduce_ring.cc:29-154,
 //                    TPL/temp_scatter/scatter_mesh.cc:46-160, TPL/temp_gather/gather_mesh.cc:60-170,
-//                    EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213, EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194
+//                    EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213, EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194,
+//                    TPL/temp_reduce/reduce_recursive_hd.cc:31-316
 //
 // Method: every template is restated as the per-rank program it issues (send / receive-and-reduce /
 // receive-and-copy / local copy), one virtual process per rank (per rank and stream for the mesh),
@@ -1451,6 +1452,112 @@ int orc_broadcast_mesh(uint32_t p, void **buf, uint64_t count, int dt, uint32_t 
         if (rc != 0) {
             return rc;
         }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
+// Recursive halving-doubling reduce, ReduceRecursiveHalvingDoubling::RunAsync
+// (TPL/temp_reduce/reduce_recursive_hd.cc:31-316): ReduceInPartOne (:85-148: in each rank pair of part one the
+// rank whose parity is the root's receives), ReduceScatterInBlock (:150-183), GatherInBlock (:236-313: a
+// binomial gather over the output buffers towards the root's block rank).  Chunk loop as for the ring reduce.
+int orc_reduce_to_root_rhd(uint32_t p, void **in, void *outRoot, uint64_t count, int dt, int op, uint32_t root,
+    uint64_t cclBytes, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.op = op;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    uint64_t stage = std::min<uint64_t>(count, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage)), cclOut(p, std::vector<uint8_t>(stage));
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_IN][r] = cclIn[r].data();
+        m.buf[B_OUT][r] = cclOut[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            m.Copy(m.buf[B_IN][r], static_cast<uint8_t *>(in[r]) + offset, bytes);
+        }
+        if (p == 1) {
+            m.Copy(m.buf[B_OUT][0], m.buf[B_IN][0], bytes);
+        } else {
+            uint32_t block, part1;
+            RhdParams(p, &block, &part1);
+            std::vector<Slice> sl = RhdSlices(bytes, block, align);
+            const uint32_t rootFlag = root >= part1 ? 0 : root;
+            auto member = [&](uint32_t r) { return r >= part1 || (r % 2) == (rootFlag % 2); };
+            auto blockRank = [&](uint32_t r) { return r < part1 ? r / 2 : r - part1 / 2; };
+            std::vector<uint32_t> rankOf(block);
+            for (uint32_t r = 0; r < p; r++) {
+                if (member(r)) {
+                    rankOf[blockRank(r)] = r;
+                }
+            }
+            const uint32_t rootQ = root > part1 ? root - part1 / 2 : root / 2;   // as written at :246
+            uint32_t rounds = 0;
+            while ((1u << rounds) < block) {
+                rounds++;
+            }
+            auto sum = [&](uint32_t first, uint32_t n) {
+                uint64_t t = 0;
+                for (uint32_t i = first; i < first + n; i++) {
+                    t += sl[i].size;
+                }
+                return t;
+            };
+            for (uint32_t r = 0; r < p; r++) {
+                Proc pr;
+                pr.rank = r;
+                const uint32_t pairPeer = (r % 2) == 0 ? r + 1 : r - 1;
+                if (!member(r)) {
+                    pr.prog.push_back(MkSend(static_cast<int>(pairPeer), 1, B_IN, 0, bytes));
+                    m.procs.push_back(std::move(pr));
+                    continue;
+                }
+                if (r < part1) {
+                    pr.prog.push_back(MkRecvReduce(static_cast<int>(pairPeer), 1, B_IN, 0, B_IN, 0, bytes));
+                }
+                const uint32_t q = blockRank(r);
+                ProgReduceScatterHd(pr.prog, q, block, rankOf, B_IN, B_OUT, sl);
+                for (uint32_t step = 0; step < rounds; step++) {
+                    const uint32_t mask = 1u << step;
+                    if (step != 0 && (q & (mask - 1)) != (rootQ & (mask - 1))) {
+                        break;
+                    }
+                    const uint32_t peer = q ^ mask;
+                    if ((q & mask) == (rootQ & mask)) {
+                        const uint32_t rxId = peer & ~(mask - 1);
+                        pr.prog.push_back(MkRecvCopy(static_cast<int>(rankOf[peer]), 2, B_OUT, sl[rxId].off, sum(rxId, mask)));
+                    } else {
+                        const uint32_t txId = q & ~(mask - 1);
+                        pr.prog.push_back(MkSend(static_cast<int>(rankOf[peer]), 2, B_OUT, sl[txId].off, sum(txId, mask)));
+                    }
+                }
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        m.Copy(static_cast<uint8_t *>(outRoot) + offset, m.buf[B_OUT][root], bytes);
         offset += bytes;
         left -= cur;
     }

@@ -64,6 +64,7 @@ def lib():
         L.orc_allgather_v.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), pu64, pu64, i32, i32, i32]
         L.orc_broadcast.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, i32, i32]
+        L.orc_reduce_to_root_rhd.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
         L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
@@ -232,11 +233,14 @@ def broadcast(bufs, dt, root, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, 
 
 
 def reduce_to_root(ins, dt, op, root, ccl_bytes=DEFAULT_CCL_BYTES, flags=0, threads=1, algo=RING, align=DEFAULT_ALIGN):
-    """algo: RING, MESH (piece cut) or MESH_ATOMIC (uncut, streams in index order)."""
+    """algo: RING, MESH (piece cut), MESH_ATOMIC (uncut, streams in index order) or RHD."""
     out = np.empty_like(ins[0])
     if algo in (MESH, MESH_ATOMIC):
         rc = lib().orc_reduce_to_root_mesh(len(ins), _ptrs(ins), out.ctypes.data, ins[0].size, dt, op, root, ccl_bytes, align,
                                            1 if algo == MESH_ATOMIC else 0, flags, threads)
+    elif algo == RHD:
+        rc = lib().orc_reduce_to_root_rhd(len(ins), _ptrs(ins), out.ctypes.data, ins[0].size, dt, op, root, ccl_bytes, align,
+                                          flags, threads)
     else:
         rc = lib().orc_reduce_to_root(len(ins), _ptrs(ins), out.ctypes.data, ins[0].size, dt, op, root, ccl_bytes, flags, threads)
     if rc != 0:

@@ -168,11 +168,12 @@ def rhd_params(p):
     return block, 2 * (p - block)
 
 
-def rhd_tree(dt, op, xs, q, block, part1):
-    """Value held by block rank q for its own slice after the halving phase."""
+def rhd_tree(dt, op, xs, q, block, part1, par=0):
+    """Value held by block rank q for its own slice after the halving phase.  par: parity of the rank
+    that stands for a folded pair (0 in the all-reduce; the root's parity in the rooted reduce)."""
     def leaf(b):
         if 2 * b < part1:
-            return combine(dt, op, xs[2 * b], xs[2 * b + 1])
+            return combine(dt, op, xs[2 * b + par], xs[(2 * b + par) ^ 1])
         return xs[b + part1 // 2]
 
     steps = block.bit_length() - 1
@@ -203,6 +204,28 @@ def rhd_allreduce(dt, op, ins, unit, ccl_bytes, align):
                 out[lo:hi] = rhd_tree(dt, op, [x[lo:hi] for x in ins], q, block, part1)
         base += cur
     return [out.copy() for _ in range(p)]
+
+
+def rhd_reduce_to_root(dt, op, ins, unit, ccl_bytes, align, root):
+    """Recursive halving-doubling reduce: the all-reduce tree, with the folded pairs represented by the
+    rank that has the root's parity (rank 0's parity when the root is outside part one)."""
+    p = len(ins)
+    n = ins[0].size
+    if p == 1:
+        return ins[0].copy()
+    block, part1 = rhd_params(p)
+    par = (0 if root >= part1 else root) % 2
+    out = np.empty_like(ins[0])
+    max_per = ccl_bytes // unit
+    base = 0
+    while base < n:
+        cur = min(n - base, max_per)
+        for q, (off, size) in enumerate(slice_plan(cur * unit, block, align)):
+            lo, hi = base + off // unit, base + (off + size) // unit
+            if hi > lo:
+                out[lo:hi] = rhd_tree(dt, op, [x[lo:hi] for x in ins], q, block, part1, par)
+        base += cur
+    return out
 
 
 def naive_reduce(dt, op, xs):

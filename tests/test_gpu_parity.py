@@ -549,10 +549,10 @@ def test_order_sensitive_known_answers_on_the_gpu():
                 g.close()
 
 
-def test_broadcast_and_reduce_mesh_schedules(orc):
+def test_broadcast_and_reduce_mesh_and_rhd_schedules(orc):
     n = 70001
-    for p in (3, 8):
-        for algo in (MESH, MESH_ATOMIC):
+    for p in (3, 8, 6):
+        for algo in (MESH, MESH_ATOMIC, RHD):
             for fuse in (1, 0):
                 g = _group(p, algo, fuse=fuse)
                 try:
@@ -563,7 +563,7 @@ def test_broadcast_and_reduce_mesh_schedules(orc):
                     torch.cuda.synchronize()
                     H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, INT32, root, g.stream_ptr)
                     g.stream.synchronize()
-                    assert g.info()["algo"] == MESH
+                    assert g.info()["algo"] == (RING if algo == RHD else MESH)   # no halving-doubling broadcast: ring
                     for r in range(p):
                         assert np.array_equal(gh.to_host(bufs[r], INT32), bufs_np[root]), ("bcast mesh", p, fuse, r)
                     for dt, op in ((FP32, SUM), (BF16, SUM), (INT64, SUM), (FP16, PROD)):

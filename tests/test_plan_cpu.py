@@ -282,3 +282,28 @@ def test_order_sensitive_known_answers_through_the_planner():
             (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, FP32, SUM)
             for r in range(p):
                 assert float(recvs[r].view(np.float32)[0]) == kat["expected_element0"][name], (name, fused, r)
+
+
+@pytest.mark.parametrize("p", [2, 3, 4, 5, 6, 7, 8, 12, 13, 24])
+def test_reduce_rhd_plan_matches_checker_and_tree(orc, p):
+    n = 1003
+    for root in sorted({0, 1, p - 1, p // 2}):
+        for dt, op, ccl in ((FP32, SUM, 200 << 20), (FP32, SUM, 2048), (BF16, SUM, 200 << 20), (INT8, MIN, 200 << 20)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n, 260 + p + dt)
+            want = orc.reduce_to_root(ins, dt, op, root, ccl_bytes=ccl, algo=RHD)
+            closed = cf.rhd_reduce_to_root(dt, op, ins, unit, ccl, 128, root)
+            assert _same(dt, want.view(np.uint8), closed), ("reduce rhd closed form", p, root, dt, ccl)
+            plan = H.describe_plan(H.COLL_REDUCE, root | (RHD << 16), p, n, dt, ccl_bytes=ccl)
+            for fused in (False, True):
+                if fused and not plan["fusedOk"]:
+                    continue
+                sends = _bytes(ins)
+                recvs = [np.full(n * unit, 0x77, np.uint8) for _ in range(p)]
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+                assert _same(dt, recvs[root], want), ("reduce rhd", p, root, dt, ccl, fused)
+                for r in range(p):
+                    assert np.array_equal(sends[r], ins[r].view(np.uint8))
+                    if r != root:
+                        assert np.all(recvs[r] == 0x77)
+            assert plan["fusedOk"], (p, root)
