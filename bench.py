@@ -94,7 +94,9 @@ def time_calls(torch, stream, call, steps, warmup):
 
 def run_suite(pkg, torch, steps, warmup, only="", settings=()):
     """The other configurations of BASELINE.json (reduce-scatter op x type matrix, 16-rank all-to-all-v,
-    halving-doubling all-reduce in bf16 at 32 and 24 ranks, all-gather), fused and step-by-step: a table on stderr."""
+    halving-doubling all-reduce in bf16 at 32 and 24 ranks, all-gather) and the rest of the API (mesh and
+    halving-doubling all-reduce, rooted collectives, uniform all-to-all, send / receive), fused and step-by-step:
+    a table on stderr."""
     import numpy as np
     stream = torch.cuda.Stream()
     out = sys.stderr
@@ -198,6 +200,43 @@ def run_suite(pkg, torch, steps, warmup, only="", settings=()):
                lambda: pkg.all_reduce(comms, sp, rp, n, pkg.HCCL_DATA_TYPE_BFP16, 0, stream.cuda_stream))
         del sends, recvs
         pkg.comm_destroy(comms)
+
+    # the widened API: mesh / halving-doubling all-reduce, rooted collectives, uniform all-to-all, send / receive
+    p = 8
+    n = (256 << 20) // 4
+    sends = [rand(n, torch.float32) for _ in range(p)]
+    recvs = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(p)]
+    sp, rp = [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs]
+    FP32 = pkg.HCCL_DATA_TYPE_FP32
+    for algo, det in (("mesh", 1), ("mesh", 0), ("rhd", 0)):
+        comms = pkg.comm_init_all(p)
+        pkg.set_param(comms[0], "algo", algo)
+        pkg.set_param(comms[0], "deterministic", det)
+        torch.cuda.synchronize()
+        label = algo + (" (piece cut)" if (algo, det) == ("mesh", 1) else " (uncut)" if algo == "mesh" else "")
+        report("all-reduce %s p=8 fp32 sum 256MiB/rank" % label, comms,
+               lambda: pkg.all_reduce(comms, sp, rp, n, FP32, 0, stream.cuda_stream))
+        for ralgo in (("ring", "mesh", "rhd") if (algo, det) == ("mesh", 0) else ()):
+            pkg.set_param(comms[0], "algo", ralgo)
+            report("reduce %s p=8 fp32 sum 256MiB/rank root 3" % ralgo, comms,
+                   lambda: pkg.reduce(comms, sp, rp, n, FP32, 0, 3, stream.cuda_stream))
+            if ralgo != "rhd":
+                report("broadcast %s p=8 256MiB root 3" % ralgo, comms,
+                       lambda: pkg.broadcast(comms, rp, n, FP32, 3, stream.cuda_stream))
+        pkg.comm_destroy(comms)
+    comms = pkg.comm_init_all(p)
+    m = n // p
+    report("scatter mesh p=8 32MiB/rank root 3", comms,
+           lambda: pkg.scatter(comms, sp, rp, m, FP32, 3, stream.cuda_stream))
+    report("all-to-all uniform p=8 32MiB/pair", comms,
+           lambda: pkg.all_to_all(comms, sp, rp, m, FP32, stream.cuda_stream))
+
+    def sendrecv():
+        pkg.send(comms[1], sp[1], n, FP32, 5, stream.cuda_stream)
+        pkg.recv(comms[5], rp[5], n, FP32, 1, stream.cuda_stream)
+    report("send/recv rank 1 -> 5 256MiB", comms, sendrecv)
+    del sends, recvs
+    pkg.comm_destroy(comms)
 
 
 def main():
