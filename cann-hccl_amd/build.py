@@ -16,6 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libhccl.so")
+ABI_CALLER = os.path.join(LIBDIR, "abi_caller")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
@@ -66,7 +67,24 @@ def build(force=False, jobs=None):
                 sys.stderr.write(out + "\n")
     if force or tasks or _newer(LIB, objs):
         _run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs + ["-lpthread"])
+    build_abi_caller(force)
     return LIB
+
+
+def build_abi_caller(force=False, include_dirs=None, out=None):
+    """Links the C-ABI conformance program (tests/c_abi/caller.cc) against the library.  include_dirs
+    lets a test put another header tree in front of this repository's include/."""
+    src = os.path.join(ROOT, "tests", "c_abi", "caller.cc")
+    out = out or ABI_CALLER
+    if not os.path.exists(src):
+        return None
+    if force or include_dirs or _newer(out, [src, LIB]):
+        inc = []
+        for d in (include_dirs or []) + [os.path.join(ROOT, "include")]:
+            inc += ["-I", d]
+        _run([HIPCC, "-O1", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-Wno-unused-command-line-argument"] + inc +
+             [src, "-L", LIBDIR, "-lhccl", "-Wl,-rpath,$ORIGIN", "-o", out])
+    return out
 
 
 if __name__ == "__main__":

@@ -327,3 +327,21 @@ def test_sub_communicator(comms):
     assert L.HcclCreateSubCommConfig(ctypes.byref(parent), 2, ids, 5, 2, ctypes.byref(cfg), ctypes.byref(out)) == H.HCCL_E_PARA
     assert L.HcclCreateSubCommConfig(ctypes.byref(parent), 2, ids, 5, 0, ctypes.byref(cfg), ctypes.byref(out)) == H.HCCL_E_PARA  # rank 0 is not rankIds[0]
     assert L.HcclCreateSubCommConfig(ctypes.byref(parent), 2, ids, 5, 0, ctypes.byref(cfg), None) == H.HCCL_E_PTR
+
+
+def test_caller_compiles_against_the_reference_header_and_links(tmp_path):
+    """A program written against the reference's own inc/hccl/hccl.h (only acl/acl.h comes from this
+    repository) must compile and link against libhccl.so: same names, same argument lists."""
+    import importlib.util
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("hccl_build", os.path.join(root, "cann-hccl_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    own = build.build_abi_caller(force=True, out=str(tmp_path / "caller_own"))
+    assert os.path.exists(own)
+    ref_inc = "/root/reference/inc"
+    if not os.path.isdir(ref_inc):
+        pytest.skip("reference tree not present on this machine")
+    theirs = build.build_abi_caller(include_dirs=[ref_inc], out=str(tmp_path / "caller_ref"))
+    assert os.path.exists(theirs)

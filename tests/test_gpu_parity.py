@@ -584,6 +584,17 @@ def test_broadcast_and_reduce_mesh_and_rhd_schedules(orc):
                     g.close()
 
 
+def test_compiled_caller_through_the_c_abi():
+    # a C++ program that includes <hccl/hccl.h> and links libhccl.so, built beforehand by cann-hccl_amd/build.py
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "cann-hccl_amd", "lib", "abi_caller")
+    assert os.path.exists(exe), "run cann-hccl_amd/build.py first"
+    print("running", exe, flush=True)
+    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert r.returncode == 0 and "ABI_CALLER_OK" in r.stdout, r.stdout[-2000:]
+
+
 def test_one_thread_per_rank_blocking_arrival(orc):
     # the reference's model: every rank on its own thread and stream; calls return once the collective is issued
     import threading
