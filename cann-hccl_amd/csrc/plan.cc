@@ -780,7 +780,44 @@ struct Piece {
     uint64_t delta;
 };
 
+// Gives equal expressions equal numbers.  The "shape" of an expression is its tree with every leaf
+// offset taken relative to the offset of its leftmost leaf, so that one shape number plus that
+// leftmost offset identifies the expression at any position.  One interner serves all the symbolic
+// runs of a planning pass, which makes shape numbers comparable between them.
+struct Interner {
+    struct Key {
+        int kind, a, b;
+        int64_t diff;
+        bool operator==(const Key &o) const { return kind == o.kind && a == o.a && b == o.b && diff == o.diff; }
+    };
+    struct Hash {
+        size_t operator()(const Key &k) const
+        {
+            uint64_t h = 0x9e3779b97f4a7c15ull;
+            for (uint64_t v : {uint64_t(k.kind), uint64_t(uint32_t(k.a)), uint64_t(uint32_t(k.b)), uint64_t(k.diff)}) {
+                h ^= v + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2);
+            }
+            return size_t(h);
+        }
+    };
+    std::unordered_map<Key, int, Hash> ids;
+    int Get(int kind, int a, int b, int64_t diff)
+    {
+        Key k{kind, a, b, diff};
+        auto it = ids.find(k);
+        if (it != ids.end()) {
+            return it->second;
+        }
+        int id = int(ids.size());
+        ids.emplace(k, id);
+        return id;
+    }
+};
+
 struct Sym {
+    Interner *in = nullptr;
+    mutable std::vector<int> shapeOf;        // per node, -1 = not computed yet
+    mutable std::vector<int64_t> baseOf;     // offset of the node's leftmost leaf at delta 0
     std::vector<ENode> nodes;
     std::map<std::pair<uint32_t, uint8_t>, std::map<uint64_t, Region>> mem;
     std::vector<uint8_t> alias;
@@ -922,22 +959,31 @@ struct Sym {
         }
         return true;
     }
-    // Canonical text of expression e evaluated at relative position `delta`; leaf offsets are printed
-    // minus `bias` (bias = 0: absolute source offsets; bias = destination start: position-independent
-    // form, equal for two adjacent ranges that continue one another).
-    void Canon(int e, uint64_t delta, uint64_t bias, std::string *out) const
+    // Shape number of expression e and the offset of its leftmost leaf (at delta 0), memoised.
+    void Shape(int e, int *shape, int64_t *base) const
     {
-        const ENode &n = nodes[e];
-        if (!n.red) {
-            *out += "L" + std::to_string(n.leaf.rank) + ":" +
-                std::to_string(static_cast<long long>(n.leaf.off + delta) - static_cast<long long>(bias));
-            return;
+        if (shapeOf.size() < nodes.size()) {
+            shapeOf.resize(nodes.size(), -1);
+            baseOf.resize(nodes.size(), 0);
         }
-        *out += "(";
-        Canon(n.a, n.da + delta, bias, out);
-        *out += ",";
-        Canon(n.b, n.db + delta, bias, out);
-        *out += ")";
+        if (shapeOf[e] < 0) {
+            const ENode &n = nodes[e];
+            if (!n.red) {
+                shapeOf[e] = in->Get(0, int(n.leaf.rank), int(n.leaf.buf), 0);
+                baseOf[e] = int64_t(n.leaf.off);
+            } else {
+                int sa, sb;
+                int64_t ba, bb;
+                Shape(n.a, &sa, &ba);
+                Shape(n.b, &sb, &bb);
+                ba += int64_t(n.da);
+                bb += int64_t(n.db);
+                shapeOf[e] = in->Get(1, sa, sb, bb - ba);
+                baseOf[e] = ba;
+            }
+        }
+        *shape = shapeOf[e];
+        *base = baseOf[e];
     }
 };
 
@@ -947,7 +993,9 @@ struct OutRange {
     uint64_t start, len;
     int expr;
     uint64_t delta;
-    std::string rel;     // position-independent canonical form
+    int shape;           // position-independent form: shape number ...
+    int64_t rel;         // ... and leftmost source offset minus the range's own start
+    int64_t abs;         // leftmost source offset
 };
 std::vector<OutRange> Outputs(const Sym &sym, uint32_t p)
 {
@@ -964,8 +1012,12 @@ std::vector<OutRange> Outputs(const Sym &sym, uint32_t p)
             o.len = kv.second.len;
             o.expr = kv.second.expr;
             o.delta = kv.second.delta;
-            sym.Canon(o.expr, o.delta, o.start, &o.rel);
-            if (!v.empty() && v.back().rank == r && v.back().start + v.back().len == o.start && v.back().rel == o.rel) {
+            int64_t base;
+            sym.Shape(o.expr, &o.shape, &base);
+            o.abs = base + int64_t(o.delta);
+            o.rel = o.abs - int64_t(o.start);
+            if (!v.empty() && v.back().rank == r && v.back().start + v.back().len == o.start && v.back().shape == o.shape &&
+                v.back().rel == o.rel) {
                 v.back().len += o.len;   // continuation of the previous range
             } else {
                 v.push_back(std::move(o));
@@ -988,7 +1040,8 @@ std::string OutputSignature(const Sym &sym, uint32_t p, const std::vector<uint8_
         if (untouched) {
             continue;
         }
-        sig += "r" + std::to_string(o.rank) + "@" + std::to_string(o.start) + "+" + std::to_string(o.len) + "=" + o.rel + ";";
+        sig += "r" + std::to_string(o.rank) + "@" + std::to_string(o.start) + "+" + std::to_string(o.len) + "=" +
+            std::to_string(o.shape) + ":" + std::to_string(o.rel) + ";";
     }
     return sig;
 }
@@ -1083,15 +1136,13 @@ bool AsTree(const Sym &sym, int e, uint64_t delta, FusedItem *item)
     return false;
 }
 
-bool Overlap(uint64_t a, uint64_t al, uint64_t b, uint64_t bl) { return a < b + bl && b < a + al; }
 
 bool BuildFused(const Sym &sym, const PlanRequest &rq, std::vector<FusedItem> *items)
 {
     std::vector<OutRange> outs = Outputs(sym, rq.p);
-    std::map<std::string, size_t> index;
+    std::map<std::tuple<uint64_t, int, int64_t>, size_t> index;   // (length, shape, leftmost source offset)
     for (const OutRange &o : outs) {
-        std::string key = std::to_string(o.len) + "|";
-        sym.Canon(o.expr, o.delta, 0, &key);
+        auto key = std::make_tuple(o.len, o.shape, o.abs);
         auto it = index.find(key);
         if (it == index.end()) {
             FusedItem item;
@@ -1268,7 +1319,9 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
     plan->recvBytes = vp.outBytes;
 
     // expected outputs: the virtual program with separate input and output buffers
+    Interner interner;
     Sym ref;
+    ref.in = &interner;
     for (uint32_t r = 0; r < p; r++) {
         ref.Init(r, vp.inBytes[r]);
     }
@@ -1309,6 +1362,7 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
             continue;
         }
         Sym s;
+        s.in = &interner;
         s.alias = alias;
         for (uint32_t r = 0; r < p; r++) {
             s.Init(r, vp.inBytes[r]);

@@ -584,6 +584,27 @@ def test_broadcast_and_reduce_mesh_and_rhd_schedules(orc):
                     g.close()
 
 
+def test_allreduce_at_the_rank_limit(orc):
+    # 64 ranks is the most a group holds: ring / uncut mesh = chains of 64 sources (the fused kernel's limit),
+    # halving-doubling at 48 ranks = 32 leaves of which 16 are folded pairs, at 64 ranks = 32 leaves of two
+    # sources each (the lowest tree level rides in the leaves)
+    n = 20011
+    for p, algo, dt, fused in ((64, RING, FP32, 1), (64, MESH_ATOMIC, BF16, 1), (48, RHD, FP32, 1), (64, RHD, BF16, 1),
+                               (33, MESH, FP32, 1)):
+        ins = _ins(dt, p, n, p + algo)
+        want = orc.allreduce(ins, dt, SUM, algo=algo)
+        g = _group(p, algo)
+        try:
+            print("rank limit p", p, "algo", algo, flush=True)
+            outs, keep = gh.all_reduce(g, ins, dt, SUM)
+            assert g.info()["fused"] == fused, (p, algo, g.info())
+            for r in range(p):
+                assert gh.same(dt, outs[r], want[r]), (p, algo, r)
+                assert np.array_equal(keep[r], ins[r])
+        finally:
+            g.close()
+
+
 def test_compiled_caller_through_the_c_abi():
     # a C++ program that includes <hccl/hccl.h> and links libhccl.so, built beforehand by cann-hccl_amd/build.py
     import os
