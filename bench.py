@@ -253,12 +253,22 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 1 GiB int32 copy (one-rank all-reduce, out of place) three times, so that a "
                          "counter profile of this command holds a copy of known size to scale FETCH_SIZE / WRITE_SIZE by")
+    ap.add_argument("--probe", action="store_true",
+                    help="run the stand-alone memory-bandwidth probe (cann-hccl_amd/lib/hbm_probe: plain kernels, n streams "
+                         "read : m written) and exit; its rates bound what the collectives can reach for the same mix")
     ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
                     help="library setting for the run (see HcclAmdSetParam), e.g. --set blocks_per_cu=4")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is built and measured on one GPU (the ranks of the communicator are "
                  "simulated inside it); --gpus %d is not supported" % args.gpus)
+
+    if args.probe:
+        import subprocess
+        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cann-hccl_amd", "lib", "hbm_probe")
+        if not os.path.exists(exe):
+            sys.exit("bench.py: %s is not built (python cann-hccl_amd/build.py)" % exe)
+        sys.exit(subprocess.run([exe, str(int(args.size_mib))]).returncode)
 
     import numpy as np
     import torch

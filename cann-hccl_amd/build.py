@@ -17,6 +17,7 @@ OBJ = os.path.join(HERE, "build")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libhccl.so")
 ABI_CALLER = os.path.join(LIBDIR, "abi_caller")
+PROBE = os.path.join(LIBDIR, "hbm_probe")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
@@ -68,7 +69,16 @@ def build(force=False, jobs=None):
     if force or tasks or _newer(LIB, objs):
         _run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs + ["-lpthread"])
     build_abi_caller(force)
+    build_probe(force)
     return LIB
+
+
+def build_probe(force=False):
+    """The stand-alone memory-bandwidth probe (csrc/hbm_probe.hip -> lib/hbm_probe)."""
+    src = os.path.join(CSRC, "hbm_probe.hip")
+    if force or _newer(PROBE, [src]):
+        _run([HIPCC, "-O3", "-std=c++17", "-Wno-unused-command-line-argument"] + DEVICE + [src, "-o", PROBE])
+    return PROBE
 
 
 def build_abi_caller(force=False, include_dirs=None, out=None):
