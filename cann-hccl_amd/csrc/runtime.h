@@ -44,10 +44,12 @@ struct GroupConfig {
 struct LaunchRec {
     const void *func = nullptr;
     uint32_t grid = 0;
-    // kernel arguments (step kernels use the first three)
+    // kernel arguments: step kernels take (table, nitems, nwhole, ntiles), fused kernels
+    // (table, nitems, ntiles, srcPool, dstPool)
     const void *table = nullptr;
     uint32_t nitems = 0;
     uint32_t ntiles = 0;
+    uint32_t nwhole = 0;
     const void *srcPool = nullptr;
     const void *dstPool = nullptr;
     bool fusedArgs = false;
