@@ -23,6 +23,9 @@ METRIC = "achieved HBM GB/s & % of peak, 8-rank fp32 ring AllReduce 256MiB/rank"
 # Valid for the default workload only (8 ranks x 256 MiB); the figures and the commands are in
 # profiles/ChainKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt.
 MEASURED_TRAFFIC_BYTES = 4295463000
+# The same for the 14 launches of the step-by-step mode together (traffic between L2 and the fabric per
+# collective); profiles/StepKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt.
+MEASURED_STEP_TRAFFIC_BYTES = 9395242000
 
 
 def run_mode(pkg, torch, comms, stream, sends, recvs, n, fuse, steps, warmup):
@@ -396,6 +399,14 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES if (p == 8 and args.size_mib == 256.0 and not args.set) else None,
             "kernel": "ChainKernel<float, sum> (fused ring all-reduce), avg launch %.4f ms over %d launches" % (dev_ms, args.steps),
+        },
+        # the literal schedule (14 phases of copy / reduce steps replayed from a HIP graph), same workload
+        "roofline_step_by_step": {
+            "bound": "hbm", "achieved": round(s_achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(s_achieved / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_STEP_TRAFFIC_BYTES if (p == 8 and args.size_mib == 256.0 and not args.set) else None,
+            "kernel": "StepKernel<float, sum>, %d launches per collective, %.4f ms per collective over %d graph replays"
+                      % (s_info["launches"], s_dev_ms, args.steps),
         },
         "cpu_baseline": cpu,
     }
