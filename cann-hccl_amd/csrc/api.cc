@@ -1370,6 +1370,16 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         } else {
             return HCCL_E_PARA;
         }
+    } else if (k == "step_stores") {
+        if (v == "auto") {
+            cfg.stepStores = -1;
+        } else if (v == "nt") {
+            cfg.stepStores = 0;
+        } else if (v == "ordinary") {
+            cfg.stepStores = 1;
+        } else {
+            return HCCL_E_PARA;
+        }
     } else if (k == "deterministic") {
         cfg.deterministic = v != "0";
     } else if (k == "fuse") {

@@ -48,11 +48,14 @@ struct FusedDesc {
     uint32_t pad;
 };
 
+// flags of the step kernel
+constexpr uint32_t kStepOrdinaryStores = 1u;   // write-back stores instead of non-temporal ones in the fast loop
+
 enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_COUNT = 3 };
 
 // Kernel entry for (data type, reduce op, kind); nullptr if the combination is not built.
 // Signatures:
-//   KK_STEP            (const StepDesc *steps, uint32_t nsteps, uint32_t nwhole, uint32_t ntiles)
+//   KK_STEP            (const StepDesc *steps, uint32_t nsteps, uint32_t nwhole, uint32_t ntiles, uint32_t flags)
 //                      steps whose tiles are all whole and ACC_VEC16 come first: tiles [0, nwhole)
 //   KK_CHAIN / KK_TREE (const FusedDesc *items, uint32_t nitems, uint32_t ntiles,
 //                       const void *const *srcPool, void *const *dstPool)

@@ -306,9 +306,13 @@ __device__ __forceinline__ V4 StepLoad(const void *base, uint64_t byteOff)
 {
     return Load16<ACC_VEC16>(base, byteOff);
 }
-__device__ __forceinline__ void StepStore(void *base, uint64_t byteOff, V4 v)
+template <bool ORDINARY> __device__ __forceinline__ void StepStore(void *base, uint64_t byteOff, V4 v)
 {
-    *(GlobalV4 *)(static_cast<char *>(base) + byteOff) = v;
+    if (ORDINARY) {
+        *(GlobalV4 *)(static_cast<char *>(base) + byteOff) = v;
+    } else {
+        Store16(base, byteOff, v);
+    }
 }
 
 // Largest i with table[i].tile0 <= tile (tile0 is ascending, table[0].tile0 == 0).
@@ -352,7 +356,7 @@ __device__ __forceinline__ void StepTileVec(const StepDesc &d, uint64_t off, uin
         }
 #pragma unroll
         for (uint32_t u = 0; u < kVecPerLane; u++) {
-            StepStore(d.dst, off + (uint64_t(u) * kBlockThreads + tid) * 16, va[u]);
+            Store16(d.dst, off + (uint64_t(u) * kBlockThreads + tid) * 16, va[u]);
         }
     } else {
         for (uint32_t i = tid; i < nvec; i += kBlockThreads) {
@@ -360,7 +364,7 @@ __device__ __forceinline__ void StepTileVec(const StepDesc &d, uint64_t off, uin
             if (d.b != nullptr) {
                 v = Combine16<T, OP>(v, Load16<MODE>(d.b, off + uint64_t(i) * 16));
             }
-            StepStore(d.dst, off + uint64_t(i) * 16, v);
+            Store16(d.dst, off + uint64_t(i) * 16, v);
         }
     }
 }
@@ -379,6 +383,62 @@ __device__ __forceinline__ void StepTileElem(const StepDesc &d, uint64_t off, ui
     }
 }
 
+// Fast loop of the step kernel over tiles [blockIdx.x, nwhole) with stride gridDim.x: every tile is
+// whole and ACC_VEC16.  The descriptor of the next tile is looked up while the loads of the current
+// one are in flight (the lookup is a chain of dependent scalar loads), and not at all while the next
+// tile still belongs to the current step.  ORDINARY picks the store kind at compile time (a run-time
+// choice per store is folded into one store by the compiler).
+template <typename T, int OP, bool ORDINARY>
+__device__ __forceinline__ void StepWholeTiles(const StepDesc *__restrict__ steps, uint32_t nsteps, uint32_t nwhole, uint32_t ntiles)
+{
+    const uint32_t tid = threadIdx.x;
+    uint32_t tile = blockIdx.x;
+    uint32_t idx = FindDesc(steps, nsteps, tile);
+    StepDesc d = steps[idx];
+    uint32_t dEnd = idx + 1 < nsteps ? steps[idx + 1].tile0 : ntiles;   // first tile past this step
+    for (;;) {
+        const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
+        const uint32_t next = tile + gridDim.x;
+        const bool reduce = d.b != nullptr;
+        V4 va[kVecPerLane], vb[kVecPerLane];
+#pragma unroll
+        for (uint32_t u = 0; u < kVecPerLane; u++) {
+            va[u] = StepLoad(d.a, off + (uint64_t(u) * kBlockThreads + tid) * 16);
+        }
+        if (reduce) {
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerLane; u++) {
+                vb[u] = StepLoad(d.b, off + (uint64_t(u) * kBlockThreads + tid) * 16);
+            }
+        }
+        // keep the loads above where they are: without this the compiler sinks them below the lookup
+        asm volatile("" ::: "memory");
+        StepDesc dn = d;
+        uint32_t dnEnd = dEnd;
+        if (next < nwhole && next >= dEnd) {
+            idx = FindDesc(steps, nsteps, next);
+            dn = steps[idx];
+            dnEnd = idx + 1 < nsteps ? steps[idx + 1].tile0 : ntiles;
+        }
+        if (reduce) {
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerLane; u++) {
+                va[u] = Combine16<T, OP>(va[u], vb[u]);
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < kVecPerLane; u++) {
+            StepStore<ORDINARY>(d.dst, off + (uint64_t(u) * kBlockThreads + tid) * 16, va[u]);
+        }
+        if (next >= nwhole) {
+            break;
+        }
+        tile = next;
+        d = dn;
+        dEnd = dnEnd;
+    }
+}
+
 // Tiles [0, nwhole) belong to steps that are ACC_VEC16 and a whole number of tiles (the host puts
 // those first in the table); tiles [nwhole, ntiles) are everything else: ragged ends, unaligned
 // buffers.  The two get separate loops: with the slow paths in the same loop as the fast one, the
@@ -386,60 +446,16 @@ __device__ __forceinline__ void StepTileElem(const StepDesc &d, uint64_t off, ui
 // wait for the previous iteration's stores before it issues its loads.
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) StepKernel(const StepDesc *__restrict__ steps, uint32_t nsteps, uint32_t nwhole,
-    uint32_t ntiles)
+    uint32_t ntiles, uint32_t flags)
 {
-    const uint32_t tid = threadIdx.x;
-    uint32_t tile = blockIdx.x;
-    if (tile < nwhole) {
-        // The descriptor of the next tile is looked up while the loads of the current one are in
-        // flight (the lookup is a chain of dependent scalar loads), and not at all while the next
-        // tile still belongs to the current step.
-        uint32_t idx = FindDesc(steps, nsteps, tile);
-        StepDesc d = steps[idx];
-        uint32_t dEnd = idx + 1 < nsteps ? steps[idx + 1].tile0 : ntiles;   // first tile past this step
-        for (;;) {
-            const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
-            const uint32_t next = tile + gridDim.x;
-            const bool reduce = d.b != nullptr;
-            V4 va[kVecPerLane], vb[kVecPerLane];
-#pragma unroll
-            for (uint32_t u = 0; u < kVecPerLane; u++) {
-                va[u] = StepLoad(d.a, off + (uint64_t(u) * kBlockThreads + tid) * 16);
-            }
-            if (reduce) {
-#pragma unroll
-                for (uint32_t u = 0; u < kVecPerLane; u++) {
-                    vb[u] = StepLoad(d.b, off + (uint64_t(u) * kBlockThreads + tid) * 16);
-                }
-            }
-            // keep the loads above where they are: without this the compiler sinks them below the lookup
-            asm volatile("" ::: "memory");
-            StepDesc dn = d;
-            uint32_t dnEnd = dEnd;
-            if (next < nwhole && next >= dEnd) {
-                idx = FindDesc(steps, nsteps, next);
-                dn = steps[idx];
-                dnEnd = idx + 1 < nsteps ? steps[idx + 1].tile0 : ntiles;
-            }
-            if (reduce) {
-#pragma unroll
-                for (uint32_t u = 0; u < kVecPerLane; u++) {
-                    va[u] = Combine16<T, OP>(va[u], vb[u]);
-                }
-            }
-#pragma unroll
-            for (uint32_t u = 0; u < kVecPerLane; u++) {
-                StepStore(d.dst, off + (uint64_t(u) * kBlockThreads + tid) * 16, va[u]);
-            }
-            if (next >= nwhole) {
-                break;
-            }
-            tile = next;
-            d = dn;
-            dEnd = dnEnd;
+    if (blockIdx.x < nwhole) {
+        if (flags & kStepOrdinaryStores) {
+            StepWholeTiles<T, OP, true>(steps, nsteps, nwhole, ntiles);
+        } else {
+            StepWholeTiles<T, OP, false>(steps, nsteps, nwhole, ntiles);
         }
     }
-    for (tile = nwhole + blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    for (uint32_t tile = nwhole + blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const StepDesc d = steps[FindDesc(steps, nsteps, tile)];
         const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
         const uint64_t left = d.bytes - off;

@@ -35,6 +35,7 @@ struct GroupConfig {
     bool fuse = true;                     // run the fused single-pass form when the plan has one
     bool graph = true;                    // issue through a HIP graph
     bool deterministic = false;
+    int stepStores = -1;             // step kernel stores: -1 chosen per launch, 0 non-temporal, 1 ordinary
     uint32_t blocksPerCu = 0;             // workgroups per CU; 0 = per-kernel default
     bool blockingArrive = false;          // ranks wait inside the call until the collective is issued
     uint32_t arriveTimeoutMs = 1800 * 1000;
@@ -44,12 +45,13 @@ struct GroupConfig {
 struct LaunchRec {
     const void *func = nullptr;
     uint32_t grid = 0;
-    // kernel arguments: step kernels take (table, nitems, nwhole, ntiles), fused kernels
+    // kernel arguments: step kernels take (table, nitems, nwhole, ntiles, flags), fused kernels
     // (table, nitems, ntiles, srcPool, dstPool)
     const void *table = nullptr;
     uint32_t nitems = 0;
     uint32_t ntiles = 0;
     uint32_t nwhole = 0;
+    uint32_t flags = 0;
     const void *srcPool = nullptr;
     const void *dstPool = nullptr;
     bool fusedArgs = false;

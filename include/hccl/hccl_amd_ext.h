@@ -20,6 +20,8 @@ extern "C" {
  *   "buffsize_mib"  CCL buffer size that sets the chunk plan (default 200, as HCCL_BUFFSIZE);
  *   "buffsize_bytes" the same in bytes (tests of the chunk loop on small inputs)
  *   "align"         slice alignment in bytes (default 128)
+ *   "step_stores"   "auto" | "nt" | "ordinary"   store kind of the step-by-step kernels (non-temporal, or write-back
+ *                                so that the next phase finds the data in the memory-side cache); "auto" decides per collective
  *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
  *   "blocking_arrive" "0" | "1"  a rank's call waits inside the library until the group is complete
  *   "arrive_timeout_ms"          limit of that wait (HCCL_E_TIMEOUT)
