@@ -262,8 +262,10 @@ struct InUse {
     ~InUse() { c->inUse = false; }
 };
 
-void CancelPending(Group *g)
+// Ends the current rendezvous.  Ranks blocked inside their call wake up and return `result`.
+void CancelPending(Group *g, HcclResult result)
 {
+    g->lastIssueResult = result;
     g->arrived = 0;
     std::fill(g->here.begin(), g->here.end(), 0);
     g->opSerial++;
@@ -301,7 +303,7 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
         // every rank must pass the same operation, count, type and op (the reference checks this
         // across processes in RankConsistentcyChecker, hccl_communicator.cc:2803-2805)
         HCCL_LOG_ERROR("%s: rank %u disagrees with the ranks already in the collective (op/count/type)", CollName(sig.coll), r);
-        CancelPending(g);
+        CancelPending(g, HCCL_E_PARA);
         return HCCL_E_PARA;
     }
     g->here[r] = 1;
@@ -329,7 +331,7 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
             [&] { return g->opSerial != serial; });
         if (!done) {
             HCCL_LOG_ERROR("%s: rank %u timed out waiting for the other ranks", CollName(sig.coll), r);
-            CancelPending(g);
+            CancelPending(g, HCCL_E_TIMEOUT);
             return HCCL_E_TIMEOUT;
         }
         return g->lastIssueResult;
@@ -357,8 +359,7 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
     if (res != HCCL_SUCCESS && res != HCCL_E_PARA) {
         g->asyncError = res;
     }
-    g->lastIssueResult = res;
-    CancelPending(g);   // resets the rendezvous and wakes blocked ranks
+    CancelPending(g, res);   // resets the rendezvous and wakes blocked ranks with the result
     return res;
 }
 
@@ -475,7 +476,7 @@ HcclResult HcclCommDestroy(HcclComm comm)
         }
         if (g->here[c->rank]) {
             HCCL_LOG_WARN("HcclCommDestroy: rank %u had joined a collective that was never issued; it is dropped", c->rank);
-            CancelPending(g);
+            CancelPending(g, HCCL_E_PARA);
         }
         for (auto it = g->p2p.begin(); it != g->p2p.end();) {   // unmatched sends / receives of this rank
             it = (it->first.first == c->rank || it->first.second == c->rank) ? g->p2p.erase(it) : std::next(it);
