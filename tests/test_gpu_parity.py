@@ -605,6 +605,29 @@ def test_allreduce_at_the_rank_limit(orc):
             g.close()
 
 
+def test_int128_moves_but_does_not_reduce():
+    # HCCL_DATA_TYPE_INT128 is a 16-byte element: the copying collectives carry it, the reducing ones refuse it
+    p, n = 4, 3001
+    I128 = H.HCCL_DATA_TYPE_INT128
+    rng = np.random.default_rng(128)
+    ins = [rng.integers(0, 256, n * 16, dtype=np.uint8) for _ in range(p)]
+    g = gh.Group(p)
+    try:
+        sends = [gh.to_dev(x) for x in ins]
+        recvs = [gh.empty_dev(n * 16 * p) for _ in range(p)]
+        torch.cuda.synchronize()
+        H.all_gather(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, I128, g.stream_ptr)
+        g.stream.synchronize()
+        want = np.concatenate(ins)
+        for r in range(p):
+            assert np.array_equal(recvs[r].cpu().numpy(), want), r
+        with pytest.raises(H.HcclError) as e:
+            H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, I128, SUM, g.stream_ptr)
+        assert e.value.code == H.HCCL_E_NOT_SUPPORT
+    finally:
+        g.close()
+
+
 def test_compiled_caller_through_the_c_abi():
     # a C++ program that includes <hccl/hccl.h> and links libhccl.so, built beforehand by cann-hccl_amd/build.py
     import os
