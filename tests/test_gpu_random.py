@@ -1,0 +1,131 @@
+"""Seeded random configurations through the C ABI against the CPU checker: ranks, sizes (whole tiles,
+ragged ends, a few elements), types, operations, schedules, misaligned and in-place buffers, fused and
+step-by-step issue.  Every case must match bit for bit (16-bit floats included: both sides round after
+every step)."""
+import numpy as np
+import pytest
+import torch
+
+import closed_forms as cf
+import gpu_harness as gh
+from closed_forms import ALL_TYPES, INT64, PROD
+
+pytestmark = pytest.mark.gpu
+H = gh.H
+RING, MESH, RHD, MESH_ATOMIC = 0, 1, 2, 4
+NAMES = {RING: "ring", MESH: "mesh", RHD: "rhd", MESH_ATOMIC: "mesh"}
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import oracle
+    oracle.build()
+    return oracle
+
+
+def _size(rng):
+    kind = rng.integers(0, 5)
+    if kind == 0:
+        return int(rng.integers(1, 40))                       # a few elements
+    if kind == 1:
+        return int(rng.integers(1, 9)) * 4096 * 8             # whole tiles for every type and rank count up to 8
+    if kind == 2:
+        return int(rng.integers(1, 9)) * 4096 * 8 + int(rng.integers(1, 4096))   # tiles plus a ragged end
+    return int(rng.integers(40, 300000))
+
+
+def _expected(algo, dt, op):
+    return MESH if (algo == MESH_ATOMIC and (dt == INT64 or op == PROD)) else algo
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_allreduce(orc, seed):
+    rng = np.random.default_rng(9000 + seed)
+    for case in range(12):
+        p = int(rng.choice([2, 3, 4, 5, 7, 8, 12, 16]))
+        algo = int(rng.choice([RING, MESH, RHD, MESH_ATOMIC]))
+        dt = int(rng.choice(ALL_TYPES))
+        op = int(rng.integers(0, 4))
+        n = _size(rng)
+        fuse = int(rng.integers(0, 2))
+        in_place = bool(rng.integers(0, 2))
+        unit = H.DTYPE_SIZE[dt]
+        pad = int(rng.choice([0, 0, unit, 16, 4 if unit <= 4 else 8]))
+        ccl = int(rng.choice([200 << 20, 200 << 20, 1 << 16, 3000 * unit]))
+        ins = [cf.random_input(dt, n, rng) for _ in range(p)]
+        want = orc.allreduce(ins, dt, op, algo=_expected(algo, dt, op), ccl_bytes=ccl)
+        print("random allreduce seed", seed, "case", case, "p", p, "algo", algo, "type", dt, "op", op, "n", n, "fuse", fuse,
+              "in place", in_place, "pad", pad, "ccl", ccl, flush=True)
+        g = gh.Group(p, algo=NAMES[algo], deterministic=0 if algo == MESH_ATOMIC else 1, fuse=fuse, buffsize_bytes=ccl)
+        try:
+            outs, keep = gh.all_reduce(g, ins, dt, op, in_place=in_place, pad=pad)
+            for r in range(p):
+                assert gh.same(dt, outs[r], want[r]), (seed, case, r)
+                if keep is not None:
+                    assert np.array_equal(keep[r], ins[r])
+        finally:
+            g.close()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_reducescatter_allgather(orc, seed):
+    rng = np.random.default_rng(9100 + seed)
+    for case in range(10):
+        p = int(rng.choice([2, 3, 4, 6, 8, 12]))
+        algo = int(rng.choice([RING, MESH, RHD, MESH_ATOMIC]))
+        dt = int(rng.choice(ALL_TYPES))
+        op = int(rng.integers(0, 4))
+        n = max(1, _size(rng) // p)
+        fuse = int(rng.integers(0, 2))
+        unit = H.DTYPE_SIZE[dt]
+        pad = int(rng.choice([0, unit, 16]))
+        print("random rs/ag seed", seed, "case", case, "p", p, "algo", algo, "type", dt, "op", op, "n", n, "fuse", fuse, "pad", pad,
+              flush=True)
+        g = gh.Group(p, algo=NAMES[algo], deterministic=0 if algo == MESH_ATOMIC else 1, fuse=fuse)
+        try:
+            ins = [cf.random_input(dt, n * p, rng) for _ in range(p)]
+            want = orc.reducescatter(ins, dt, op, algo=_expected(algo, dt, op))
+            outs, keep = gh.reduce_scatter(g, ins, dt, op, pad=pad)
+            for r in range(p):
+                assert gh.same(dt, outs[r], want[r]), (seed, case, "rs", r)
+                assert np.array_equal(keep[r], ins[r])
+            small = [x[:n] for x in ins]
+            outs = gh.all_gather(g, small, dt, pad=pad)
+            whole = np.concatenate(small)
+            for r in range(p):
+                assert np.array_equal(outs[r], whole), (seed, case, "ag", r)
+        finally:
+            g.close()
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_rooted(orc, seed):
+    rng = np.random.default_rng(9200 + seed)
+    for case in range(8):
+        p = int(rng.choice([2, 3, 5, 8, 12]))
+        algo = int(rng.choice([RING, MESH, RHD, MESH_ATOMIC]))
+        dt = int(rng.choice(ALL_TYPES))
+        op = int(rng.integers(0, 4))
+        n = _size(rng)
+        fuse = int(rng.integers(0, 2))
+        root = int(rng.integers(0, p))
+        print("random rooted seed", seed, "case", case, "p", p, "algo", algo, "type", dt, "op", op, "n", n, "fuse", fuse, "root", root,
+              flush=True)
+        g = gh.Group(p, algo=NAMES[algo], deterministic=0 if algo == MESH_ATOMIC else 1, fuse=fuse)
+        try:
+            ins = [cf.random_input(dt, n, rng) for _ in range(p)]
+            want = orc.reduce_to_root(ins, dt, op, root, algo=_expected(algo, dt, op))
+            sends = [gh.to_dev(x) for x in ins]
+            recvs = [gh.empty_dev(n * H.DTYPE_SIZE[dt], fill=0x33) for _ in range(p)]
+            torch.cuda.synchronize()
+            H.reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, op, root, g.stream_ptr)
+            g.stream.synchronize()
+            assert gh.same(dt, gh.to_host(recvs[root], dt), want), (seed, case, "reduce")
+            bufs = [gh.to_dev(x) for x in ins]
+            torch.cuda.synchronize()
+            H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, dt, root, g.stream_ptr)
+            g.stream.synchronize()
+            for r in range(p):
+                assert np.array_equal(gh.to_host(bufs[r], dt), ins[root]), (seed, case, "broadcast", r)
+        finally:
+            g.close()
