@@ -350,7 +350,8 @@ def main():
         del src, dst
 
     if args.sweep:
-        sys.stderr.write("bytes/rank  fused_us  fused_GB/s(actual)  steps_us  steps_GB/s(actual)  sched_GB/s(fused)\n")
+        sys.stderr.write("bytes/rank  fused_us  fused_GB/s(actual)  steps_us  steps_GB/s(actual)  sched_GB/s(fused)"
+                         "  cpu_us(%d threads)  cpu_sched_GB/s\n" % threads)
         size = 8 << 10
         while size <= int(args.size_mib * (1 << 20)):
             m = size // 4
@@ -358,8 +359,22 @@ def main():
             _, g_ms, gi = run_mode(pkg, torch, comms, stream, sends, recvs, m, 0, args.steps, args.warmup)
             fa = (fi["bytesRead"] + fi["bytesWritten"]) / (f_ms * 1e-3) / 1e9
             ga = (gi["bytesRead"] + gi["bytesWritten"]) / (g_ms * 1e-3) / 1e9
-            sys.stderr.write("%10d %9.1f %12.1f %9.1f %12.1f %12.1f\n" % (size, f_ms * 1e3, fa, g_ms * 1e3, ga,
-                                                                         (5 * p - 3) * size / (f_ms * 1e-3) / 1e9))
+            cpu_us = float("nan")
+            if not args.no_cpu:
+                small = [x[:m] for x in ins]
+                outs = [np.empty(m, np.float32) for _ in range(p)]
+                best = None
+                for _ in range(3):
+                    work = [x.copy() for x in small]
+                    t0 = time.perf_counter()
+                    oracle.allreduce(work, oracle.FP32, oracle.SUM, flags=oracle.DIRECT | oracle.ZERO_STAGING, threads=threads,
+                                     outs=outs)
+                    dt = time.perf_counter() - t0
+                    best = dt if best is None else min(best, dt)
+                cpu_us = best * 1e6
+            sys.stderr.write("%10d %9.1f %12.1f %9.1f %12.1f %12.1f %12.1f %12.1f\n"
+                             % (size, f_ms * 1e3, fa, g_ms * 1e3, ga, (5 * p - 3) * size / (f_ms * 1e-3) / 1e9, cpu_us,
+                                (5 * p - 3) * size / (cpu_us * 1e-6) / 1e9))
             size *= 2
 
     line = {
