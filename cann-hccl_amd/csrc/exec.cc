@@ -670,7 +670,7 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     } else if (g->ctx->sig.coll == COLL_REDUCE) {
         algo = (algo == ALGO_MESH || algo == ALGO_RHD) ? algo : ALGO_RING;   // ring, mesh or halving-doubling reduce
     } else if (g->ctx->sig.coll == COLL_BROADCAST) {
-        algo = (algo == ALGO_MESH) ? ALGO_MESH : ALGO_RING;   // ring or mesh broadcast
+        algo = (algo == ALGO_MESH || algo == ALGO_RHD) ? algo : ALGO_RING;   // ring, mesh or halving-doubling broadcast
     } else if (g->ctx->sig.coll >= COLL_SCATTER) {
         algo = ALGO_RING;   // one schedule each: mesh scatter, direct send / receive
     } else if (algo == ALGO_PAIRWISE) {

@@ -425,6 +425,43 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                         EmitCopy(*vp, 1, MkRef(r, BUF_RECV, done + sl[d].off), src, sl[d].size);
                     }
                 }
+            } else if (rq.coll == COLL_BROADCAST && rq.algo == ALGO_RHD && p > 1) {
+                // recursive halving-doubling broadcast (bcast_recursive_halvingdoubling.cc:21-290): a binomial
+                // tree over the block, whole chunk per hop, widest distance first (:162-203); the block holds
+                // the root and, of every rank pair of part one, the rank with the root's parity (:120-160);
+                // afterwards that rank hands the chunk to its neighbour (:205-262)
+                uint32_t block, part1;
+                HalvingDoublingShape(p, &block, &part1);
+                const uint32_t par = (R < part1 && (R % 2) == 1) ? 1u : 0u;
+                std::vector<uint32_t> rankOf(block);
+                for (uint32_t b = 0; b < block; b++) {
+                    rankOf[b] = b < part1 / 2 ? 2 * b + par : b + part1 / 2;
+                }
+                const uint32_t rootQ = R < part1 ? R / 2 : R - part1 / 2;
+                auto data = [&](uint32_t r) { return r == R ? MkRef(R, BUF_SEND, done) : MkRef(r, BUF_RECV, done); };
+                uint32_t rounds = 0;
+                while ((1u << rounds) < block) {
+                    rounds++;
+                }
+                std::vector<uint8_t> has(block, 0);
+                has[rootQ] = 1;
+                size_t ph = 0;
+                for (uint32_t i = 0; i < rounds; i++, ph++) {
+                    const uint32_t mask = 1u << (rounds - i - 1);
+                    std::vector<uint32_t> got;
+                    for (uint32_t q = 0; q < block; q++) {
+                        if (has[q] && (q & (mask - 1)) == (rootQ & (mask - 1)) && !has[q ^ mask]) {
+                            EmitCopy(*vp, ph, data(rankOf[q ^ mask]), data(rankOf[q]), bytes);
+                            got.push_back(q ^ mask);
+                        }
+                    }
+                    for (uint32_t q : got) {
+                        has[q] = 1;
+                    }
+                }
+                for (uint32_t b = 0; b < part1 / 2; b++) {
+                    EmitCopy(*vp, ph, data(rankOf[b] ^ 1u), data(rankOf[b]), bytes);
+                }
             } else if (rq.coll == COLL_REDUCE && rq.algo == ALGO_MESH && p > 1) {
                 // mesh reduce (coll_reduce_mesh_executor.cc:75-194): mesh reduce-scatter over the ring
                 // slice plan, then the root gathers slice r from rank r (gather_mesh.cc:60-170)

@@ -25,7 +25,7 @@
 //   rooted           TPL/temp_broadcast/broadcast_ring.cc:24-160, TPL/temp_reduce/reduce_ring.cc:29-154,
 //                    TPL/temp_scatter/scatter_mesh.cc:46-160, TPL/temp_gather/gather_mesh.cc:60-170,
 //                    EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213, EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194,
-//                    TPL/temp_reduce/reduce_recursive_hd.cc:31-316
+//                    TPL/temp_reduce/reduce_recursive_hd.cc:31-316, TPL/temp_broadcast/bcast_recursive_halvingdoubling.cc:21-290
 //
 // Method: every template is restated as the per-rank program it issues (send / receive-and-reduce /
 // receive-and-copy / local copy), one virtual process per rank (per rank and stream for the mesh),
@@ -1449,6 +1449,100 @@ int orc_broadcast_mesh(uint32_t p, void **buf, uint64_t count, int dt, uint32_t 
             m.procs.push_back(std::move(pr));
         }
         rc = m.Run();
+        if (rc != 0) {
+            return rc;
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
+// Recursive halving-doubling broadcast, BcastRecursiveHalvingDoubling::RunAsync
+// (TPL/temp_broadcast/bcast_recursive_halvingdoubling.cc:21-290): BroadcastInBlock (:162-203) and the hand-over
+// inside the rank pairs of part one (:205-262); block membership from GetRankIndexInBlock (:138-160).
+int orc_broadcast_rhd(uint32_t p, void **buf, uint64_t count, int dt, uint32_t root, uint64_t cclBytes, uint64_t align,
+    int flags, int threads)
+{
+    (void)align;
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    uint32_t block, part1;
+    RhdParams(p, &block, &part1);
+    const bool rootEven = (root < part1 && (root % 2) == 0) || root >= part1;
+    auto inBlock = [&](uint32_t r) -> int {   // GetRankIndexInBlock
+        if (r >= part1) {
+            return static_cast<int>(r - part1 / 2);
+        }
+        if (rootEven) {
+            return (r % 2) == 0 ? static_cast<int>(r / 2) : -1;
+        }
+        return (r % 2) == 1 ? static_cast<int>((r - 1) / 2) : -1;
+    };
+    auto real = [&](uint32_t q) -> uint32_t {   // GetRankIndexReal
+        if (q < part1 / 2) {
+            return rootEven ? q * 2 : q * 2 + 1;
+        }
+        return part1 / 2 + q;
+    };
+    uint32_t rounds = 0;
+    while ((1u << rounds) < block) {
+        rounds++;
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0 && p > 1;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            m.buf[B_IN][r] = static_cast<uint8_t *>(buf[r]) + offset;
+            m.buf[B_OUT][r] = static_cast<uint8_t *>(buf[r]) + offset;
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            Proc pr;
+            pr.rank = r;
+            int q = inBlock(r);
+            if (q >= 0) {
+                const uint32_t rq = static_cast<uint32_t>(q), rootQ = static_cast<uint32_t>(inBlock(root));
+                bool hasData = r == root;
+                for (uint32_t i = 0; i < rounds; i++) {
+                    const uint32_t mask = 1u << (rounds - i - 1);
+                    const uint32_t peer = real(rq ^ mask);
+                    if ((rq & (mask - 1)) == (rootQ & (mask - 1)) && r != root && !hasData) {
+                        pr.prog.push_back(MkRecvCopy(static_cast<int>(peer), 0, B_IN, 0, bytes));
+                        hasData = true;
+                        continue;
+                    }
+                    if (hasData) {
+                        pr.prog.push_back(MkSend(static_cast<int>(peer), 0, B_IN, 0, bytes));
+                    }
+                }
+            }
+            if (r < part1) {
+                const uint32_t pairPeer = (r % 2) == 0 ? r + 1 : r - 1;
+                const bool sends = ((r % 2) == 0) == rootEven;   // EvenNumberRankProcess / OddNumberRankProcess
+                if (sends) {
+                    pr.prog.push_back(MkSend(static_cast<int>(pairPeer), 1, B_IN, 0, bytes));
+                } else {
+                    pr.prog.push_back(MkRecvCopy(static_cast<int>(pairPeer), 1, B_IN, 0, bytes));
+                }
+            }
+            m.procs.push_back(std::move(pr));
+        }
+        int rc = m.Run();
         if (rc != 0) {
             return rc;
         }

@@ -65,6 +65,7 @@ def lib():
         L.orc_broadcast.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, i32, i32]
         L.orc_reduce_to_root_rhd.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
+        L.orc_broadcast_rhd.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
         L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
@@ -224,8 +225,8 @@ def allgather_v(ins, counts, displs, out_len, dt, algo=RING, flags=0, threads=1,
 
 
 def broadcast(bufs, dt, root, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1, algo=RING):
-    """bufs: p equal-length arrays, written in place: every array becomes bufs[root].  algo: RING or MESH."""
-    fn = lib().orc_broadcast_mesh if algo == MESH else lib().orc_broadcast
+    """bufs: p equal-length arrays, written in place: every array becomes bufs[root].  algo: RING, MESH or RHD."""
+    fn = lib().orc_broadcast_mesh if algo == MESH else lib().orc_broadcast_rhd if algo == RHD else lib().orc_broadcast
     rc = fn(len(bufs), _ptrs(bufs), bufs[0].size, dt, root, ccl_bytes, align, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle broadcast failed rc=%d" % rc)

@@ -563,7 +563,7 @@ def test_broadcast_and_reduce_mesh_and_rhd_schedules(orc):
                     torch.cuda.synchronize()
                     H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, INT32, root, g.stream_ptr)
                     g.stream.synchronize()
-                    assert g.info()["algo"] == (RING if algo == RHD else MESH)   # no halving-doubling broadcast: ring
+                    assert g.info()["algo"] == (RHD if algo == RHD else MESH)
                     for r in range(p):
                         assert np.array_equal(gh.to_host(bufs[r], INT32), bufs_np[root]), ("bcast mesh", p, fuse, r)
                     for dt, op in ((FP32, SUM), (BF16, SUM), (INT64, SUM), (FP16, PROD)):

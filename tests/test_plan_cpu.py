@@ -307,3 +307,21 @@ def test_reduce_rhd_plan_matches_checker_and_tree(orc, p):
                     if r != root:
                         assert np.all(recvs[r] == 0x77)
             assert plan["fusedOk"], (p, root)
+
+
+@pytest.mark.parametrize("p", [2, 3, 4, 5, 6, 7, 8, 12, 13, 24])
+def test_broadcast_rhd_plan_matches_checker(orc, p):
+    n = 1003
+    for root in sorted({0, 1, p - 1, p // 2}):
+        for ccl in (200 << 20, 1024):
+            bufs = _ins(INT32, p, n, 350 + p)
+            want = orc.broadcast([b.copy() for b in bufs], INT32, root, ccl_bytes=ccl, algo=RHD)
+            assert all(np.array_equal(w, bufs[root]) for w in want), (p, root)
+            plan = H.describe_plan(H.COLL_BROADCAST, root | (RHD << 16), p, n, INT32, ccl_bytes=ccl, in_place_mask=(1 << p) - 1)
+            block = 1 << (p.bit_length() - 1)
+            assert len(plan["phases"]) == (block.bit_length() - 1) + (1 if p > block else 0)   # tree depth, plus the pair hand-over
+            for fused in (False, True):
+                mem = _bytes(bufs)
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, mem, mem, INT32, 0, in_place=True)
+                for r in range(p):
+                    assert np.array_equal(mem[r].view(np.int32), want[r]), ("bcast rhd", p, root, ccl, fused, r)
