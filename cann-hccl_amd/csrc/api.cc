@@ -1371,6 +1371,12 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         } else {
             return HCCL_E_PARA;
         }
+    } else if (k == "servers") {
+        long n = std::atol(value);
+        if (n < 1 || uint32_t(n) > c->group->p || c->group->p % uint32_t(n) != 0) {
+            return HCCL_E_PARA;
+        }
+        cfg.servers = uint32_t(n);
     } else if (k == "step_stores") {
         if (v == "auto") {
             cfg.stepStores = -1;
@@ -1462,6 +1468,11 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         // rooted collectives: low 16 bits = root rank, bits 16.. = schedule (0 ring, 1 mesh, 4 mesh uncut)
         rq.root = uint32_t(algo) & 0xffffu;
         rq.algo = Algo(uint32_t(algo) >> 16);
+    } else if (coll == COLL_ALLREDUCE) {
+        // all-reduce: low 8 bits = schedule, bits 8..15 = number of rank groups ("servers") of a two-level schedule
+        rq.algo = Algo(uint32_t(algo) & 0xffu);
+        rq.servers = std::max(1u, (uint32_t(algo) >> 8) & 0xffu);
+        rq.meshAtomic = ((uint32_t(algo) >> 16) & 1u) != 0;   // bit 16: mesh level without the piece cut
     } else {
         rq.algo = Algo(algo);
     }

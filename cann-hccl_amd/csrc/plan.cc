@@ -37,12 +37,24 @@ Ref MkRef(uint32_t rank, uint8_t buf, uint64_t off)
 struct VProgram {
     std::vector<Phase> phases;
     std::vector<uint64_t> inBytes, outBytes;
+    // While a schedule is laid out for a sub-communicator: its ranks (local index -> rank of the whole
+    // group; empty = identity) and the phase its own phase 0 stands for.
+    std::vector<uint32_t> rankMap;
+    size_t phaseBase = 0;
 };
 
 void Emit(VProgram &vp, size_t phase, bool reduce, Ref dst, Ref a, Ref b, uint64_t bytes)
 {
     if (bytes == 0) {
         return;
+    }
+    phase += vp.phaseBase;
+    if (!vp.rankMap.empty()) {
+        dst.rank = vp.rankMap[dst.rank];
+        a.rank = vp.rankMap[a.rank];
+        if (reduce) {
+            b.rank = vp.rankMap[b.rank];
+        }
     }
     if (vp.phases.size() <= phase) {
         vp.phases.resize(phase + 1);
@@ -230,6 +242,44 @@ void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t
             EmitCopy(vp, ph, MkRef(e + 1, BUF_RECV, base), MkRef(e, BUF_RECV, base), bytes);
         }
     }
+}
+
+// Two-level all-reduce of one chunk, CollAllReduceMeshExecutor::KernelRun with several servers
+// (coll_all_reduce_mesh_executor.cc:95-240): `servers` groups of D = p / servers consecutive ranks.
+//   level 0  mesh reduce-scatter inside every group over the ring slice plan for D (:102-118)
+//   level 1  ranks with the same position d in their groups all-reduce slice d among themselves, ring
+//            or recursive halving-doubling, from the input range to the output range (:120-196)
+//   level 0  mesh all-gather of the slices inside every group on the output (:198-236)
+// With one group the middle level is the copy of the own slice and this is the plain mesh all-reduce.
+void TwoLevelAllReduceChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, uint64_t base, uint64_t bytes, uint64_t align,
+    bool meshAtomic)
+{
+    const uint32_t D = p / servers;
+    std::vector<Slice> sl = RingSlicePlan(bytes, D, align);
+    const size_t l1 = D > 1 ? D - 1 : 0;
+    VProgram shape;   // how many phases the level-1 schedule has (it does not depend on the size)
+    AllReduceChunk(shape, level1, servers, 0, uint64_t(servers) * align * 64, align, false);
+    const size_t l2 = l1 + shape.phases.size();
+    for (uint32_t s = 0; s < servers && D > 1; s++) {
+        vp.rankMap.resize(D);
+        for (uint32_t d = 0; d < D; d++) {
+            vp.rankMap[d] = s * D + d;
+        }
+        vp.phaseBase = 0;
+        MeshReduceScatterPhases(vp, 0, D, base, sl, align, meshAtomic);
+        vp.phaseBase = l2;
+        MeshAllGatherPhases(vp, 0, D, base, sl);
+    }
+    for (uint32_t d = 0; d < D; d++) {
+        vp.rankMap.resize(servers);
+        for (uint32_t s = 0; s < servers; s++) {
+            vp.rankMap[s] = s * D + d;
+        }
+        vp.phaseBase = l1;
+        AllReduceChunk(vp, level1, servers, base + sl[d].off, sl[d].size, align, false);
+    }
+    vp.rankMap.clear();
+    vp.phaseBase = 0;
 }
 
 // Halving-doubling shape shared by the standalone reduce-scatter / all-gather variants: block rank b
@@ -606,7 +656,10 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
     uint64_t done = 0;
     for (uint64_t cur : chunks) {
         uint64_t bytes = cur * u;
-        if (rq.coll == COLL_ALLREDUCE) {
+        if (rq.coll == COLL_ALLREDUCE && rq.servers > 1) {
+            TwoLevelAllReduceChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, done, bytes, rq.align,
+                rq.meshAtomic);
+        } else if (rq.coll == COLL_ALLREDUCE) {
             AllReduceChunk(*vp, rq.algo, p, done, bytes, rq.align, rq.meshAtomic);
         } else if (rq.coll == COLL_REDUCESCATTER) {
             // input slice i of this chunk sits at i * total + done in the caller's layout
@@ -1334,7 +1387,7 @@ std::vector<uint64_t> ChunkCounts(CollKind coll, uint64_t count, uint32_t unit, 
 
 int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
 {
-    if (request.p == 0 || request.unit == 0 || request.align == 0) {
+    if (request.p == 0 || request.unit == 0 || request.align == 0 || request.servers == 0 || request.p % request.servers != 0) {
         *err = "bad plan request";
         return 1;
     }

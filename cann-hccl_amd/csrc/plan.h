@@ -79,6 +79,8 @@ struct PlanRequest {
     uint64_t cclBytes = 200ull << 20;
     uint64_t align = 128;
     std::vector<uint8_t> alias;    // per rank: send buffer and receive buffer are the same memory
+    uint32_t servers = 1;          // all-reduce only: > 1 = two levels, `servers` groups of p / servers consecutive ranks
+                                   // (mesh inside a group, `algo` ring or halving-doubling between the groups)
     bool meshAtomic = false;       // mesh reduce phases without the piece cut (the reference's non-deterministic variant)
     bool stageInput = false;       // copy the send buffers to scratch first (used when buffers overlap)
     // all-to-all-v only: p x p tables in elements, row r = what rank r passed

@@ -35,6 +35,7 @@ struct GroupConfig {
     bool fuse = true;                     // run the fused single-pass form when the plan has one
     bool graph = true;                    // issue through a HIP graph
     bool deterministic = false;
+    uint32_t servers = 1;            // all-reduce: > 1 = two-level schedule over `servers` groups of consecutive ranks
     int stepStores = -1;             // step kernel stores: -1 chosen per launch, 0 non-temporal, 1 ordinary
     uint32_t blocksPerCu = 0;             // workgroups per CU; 0 = per-kernel default
     bool blockingArrive = false;          // ranks wait inside the call until the collective is issued

@@ -20,6 +20,8 @@ extern "C" {
  *   "buffsize_mib"  CCL buffer size that sets the chunk plan (default 200, as HCCL_BUFFSIZE);
  *   "buffsize_bytes" the same in bytes (tests of the chunk loop on small inputs)
  *   "align"         slice alignment in bytes (default 128)
+ *   "servers"       number of rank groups for the all-reduce: with n > 1 the p ranks form n groups of p / n
+ *                   consecutive ranks and the two-level schedule runs (mesh inside a group, "algo" ring or rhd between)
  *   "step_stores"   "auto" | "nt" | "ordinary"   store kind of the step-by-step kernels (non-temporal, or write-back
  *                                so that the next phase finds the data in the memory-side cache); "auto" decides per collective
  *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
@@ -48,7 +50,9 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
 /* Plans a collective without a device and writes the plan as JSON (phases of copy / reduce steps,
  * fused items, byte counts) into out[0..cap).  coll / algo as in HcclAmdOpInfo; for the rooted
  * collectives (coll 4 broadcast, 5 reduce, 6 scatter) the algo argument carries the root rank in its low 16 bits and the
- * schedule above them (0 ring, 1 mesh, 4 mesh without the piece cut; reduce only).  inPlaceMask bit r:
+ * schedule above them (0 ring, 1 mesh, 2 rhd, 4 mesh without the piece cut); for the all-reduce (coll 0) bits 8..15 of algo
+ * carry the number of rank groups of the two-level schedule (0 or 1: one level) and bit 16 asks for its mesh level
+ * without the piece cut.  inPlaceMask bit r:
  * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64
  * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); for the variable-count
  * reduce-scatter / all-gather, tables points to 2*p uint64 (block counts, block displacements); else NULL.

@@ -1008,6 +1008,122 @@ int orc_allreduce(int algo, uint32_t p, void **in, void **out, uint64_t count, i
     return 0;
 }
 
+// Two-level all-reduce, CollAllReduceMeshExecutor::KernelRun with several servers
+// (EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240): `servers` groups of D = p / servers consecutive
+// ranks; mesh reduce-scatter inside every group (piece cut, or uncut when `atomic`), then the ranks with the same
+// position in their groups all-reduce their slice among themselves (level1 = ALGO_RING or ALGO_RHD) from the
+// input range to the output range, then a mesh all-gather inside every group.  Chunk loop and staging as in
+// orc_allreduce.
+int orc_allreduce_two_level(int level1, int atomic, uint32_t servers, uint32_t p, void **in, void **out, uint64_t count, int dt,
+    int op, uint64_t cclBytes, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || servers == 0 || p % servers != 0 || cclBytes < unit || (level1 != ALGO_RING && level1 != ALGO_RHD)) {
+        return -20;
+    }
+    const uint32_t D = p / servers;
+    Pool pool(threads);
+    auto machine = [&](uint32_t n) {
+        Machine m;
+        m.p = static_cast<int>(n);
+        m.dt = dt;
+        m.op = op;
+        m.direct = (flags & 1) != 0;
+        m.pool = &pool;
+        m.buf[B_IN].resize(n);
+        m.buf[B_OUT].resize(n);
+        return m;
+    };
+    Machine all = machine(p);
+    uint64_t maxPer = MaxCountPerLoop(0, cclBytes, p, unit, align);
+    uint64_t stage = std::min<uint64_t>(count, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage)), cclOut(p, std::vector<uint8_t>(stage));
+    for (uint32_t r = 0; r < p; r++) {
+        all.buf[B_IN][r] = cclIn[r].data();
+        all.buf[B_OUT][r] = cclOut[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            all.Copy(all.buf[B_IN][r], static_cast<uint8_t *>(in[r]) + offset, bytes);
+        }
+        std::vector<Slice> sl = RingSlices(bytes, D, align);
+        // level 0: reduce-scatter inside every group
+        for (uint32_t s = 0; s < servers && D > 1; s++) {
+            Machine m = machine(D);
+            for (uint32_t d = 0; d < D; d++) {
+                m.buf[B_IN][d] = all.buf[B_IN][s * D + d];
+                m.buf[B_OUT][d] = all.buf[B_OUT][s * D + d];
+            }
+            if (atomic) {
+                for (uint32_t d = 0; d < D; d++) {
+                    Proc pr;
+                    pr.rank = d;
+                    ProgReduceScatterMeshAtomic(pr.prog, d, D, B_IN, sl);
+                    m.procs.push_back(std::move(pr));
+                }
+            } else {
+                uint32_t nstream = D > 2 ? D - 1 : 1;
+                std::vector<std::vector<Slice>> pieces = CutPieces(sl, nstream, align);
+                for (uint32_t t = 0; t < nstream; t++) {
+                    for (uint32_t d = 0; d < D; d++) {
+                        Proc pr;
+                        pr.rank = d;
+                        ProgReduceScatterMeshStream(pr.prog, d, D, t, B_IN, pieces[t]);
+                        m.procs.push_back(std::move(pr));
+                    }
+                }
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        // level 1: all-reduce of slice d among the ranks at position d of every group
+        for (uint32_t d = 0; d < D; d++) {
+            Machine m = machine(servers);
+            for (uint32_t s = 0; s < servers; s++) {
+                m.buf[B_IN][s] = all.buf[B_IN][s * D + d] + sl[d].off;
+                m.buf[B_OUT][s] = all.buf[B_OUT][s * D + d] + sl[d].off;
+            }
+            if (sl[d].size == 0) {
+                continue;
+            }
+            int rc = RunAllReduceTemplate(m, level1, sl[d].size, align);
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        // level 0: all-gather inside every group
+        for (uint32_t s = 0; s < servers && D > 1; s++) {
+            Machine m = machine(D);
+            for (uint32_t d = 0; d < D; d++) {
+                m.buf[B_IN][d] = all.buf[B_IN][s * D + d];
+                m.buf[B_OUT][d] = all.buf[B_OUT][s * D + d];
+            }
+            for (uint32_t d = 0; d < D; d++) {
+                Proc pr;
+                pr.rank = d;
+                ProgAllGatherMesh(pr.prog, d, D, B_OUT, sl);
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            all.Copy(static_cast<uint8_t *>(out[r]) + offset, all.buf[B_OUT][r], bytes);
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
+
 // in[r]: p * recvCount elements, out[r]: recvCount elements.  Ring only at this level
 // (coll_reduce_scatter_comm_executor.cc:196-209); mesh uses the same slices with the mesh template.
 int orc_reducescatter(int algo, uint32_t p, void **in, void **out, uint64_t recvCount, int dt, int op,

@@ -65,6 +65,8 @@ def lib():
         L.orc_broadcast.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, i32, i32]
         L.orc_reduce_to_root_rhd.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
+        L.orc_allreduce_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64,
+                                              i32, i32]
         L.orc_broadcast_rhd.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
@@ -176,6 +178,18 @@ def allreduce(ins, dt, op, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT
     if rc != 0:
         raise RuntimeError("oracle allreduce failed rc=%d" % rc)
     return (outs, touched.value) if return_touched else outs
+
+
+def allreduce_two_level(ins, dt, op, servers, level1=RING, atomic=False, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0,
+                        threads=1):
+    """`servers` groups of consecutive ranks: mesh inside a group (piece cut, or uncut when `atomic`), `level1`
+    (RING or RHD) between the groups."""
+    outs = [np.empty_like(x) for x in ins]
+    rc = lib().orc_allreduce_two_level(level1, 1 if atomic else 0, servers, len(ins), _ptrs(ins), _ptrs(outs), ins[0].size, dt, op,
+                                       ccl_bytes, align, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle two-level allreduce failed rc=%d" % rc)
+    return outs
 
 
 def reducescatter(ins, dt, op, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1):

@@ -228,6 +228,42 @@ def rhd_reduce_to_root(dt, op, ins, unit, ccl_bytes, align, root):
     return out
 
 
+def two_level_allreduce(dt, op, ins, unit, ccl_bytes, align, servers, level1, atomic):
+    """Groups of D = p / servers consecutive ranks: mesh chain inside a group for slice d (per piece when the
+    slice is cut), then the level-1 closed form (ring_allreduce or rhd_allreduce) over the groups' partial
+    results of that slice."""
+    p = len(ins)
+    D = p // servers
+    n = ins[0].size
+    out = np.empty_like(ins[0])
+    max_per = ccl_bytes // unit
+    base = 0
+    while base < n:
+        cur = min(n - base, max_per)
+        for d, (off, size) in enumerate(slice_plan(cur * unit, D, align)):
+            lo, hi = base + off // unit, base + (off + size) // unit
+            if hi <= lo:
+                continue
+            partial = []
+            for s in range(servers):
+                xs = [x[lo:hi] for x in ins[s * D:(s + 1) * D]]
+                if D == 1:
+                    partial.append(xs[0].copy())
+                elif atomic:
+                    partial.append(mesh_atomic_chain(dt, op, xs, d))
+                else:
+                    acc = np.empty_like(xs[0])
+                    nstream = D - 1 if D > 2 else 1
+                    for t, (poff, psize) in enumerate(slice_plan(size, nstream, align)):
+                        a, b = poff // unit, (poff + psize) // unit
+                        if b > a:
+                            acc[a:b] = mesh_chain(dt, op, [x[a:b] for x in xs], d, t)
+                    partial.append(acc)
+            out[lo:hi] = level1(dt, op, partial, unit, 1 << 62, align)[0]
+        base += cur
+    return [out.copy() for _ in range(p)]
+
+
 def naive_reduce(dt, op, xs):
     acc = xs[0]
     for x in xs[1:]:

@@ -628,6 +628,27 @@ def test_int128_moves_but_does_not_reduce():
         g.close()
 
 
+@pytest.mark.parametrize("level1", [RING, RHD])
+def test_two_level_allreduce(orc, level1):
+    # groups of consecutive ranks ("servers"): mesh inside a group, ring or halving-doubling between the groups
+    for servers, D in ((2, 4), (4, 2), (3, 4), (2, 8)):
+        p = servers * D
+        for det in (1, 0):
+            g = gh.Group(p, algo=ALGO_NAME[level1], deterministic=det, servers=servers)
+            try:
+                for dt, op, n in ((FP32, SUM, 300007), (BF16, SUM, 65536 + 5), (INT64, SUM, 10001), (FP16, PROD, 4096)):
+                    atomic = (det == 0) and dt != INT64 and op != PROD
+                    ins = _ins(dt, p, n, 17 * p + n)
+                    want = orc.allreduce_two_level(ins, dt, op, servers, level1=level1, atomic=atomic)
+                    print("two-level", servers, "x", D, "level1", level1, "deterministic", det, "type", dt, flush=True)
+                    for in_place in (False, True):
+                        outs, _ = gh.all_reduce(g, ins, dt, op, in_place=in_place)
+                        for r in range(p):
+                            assert gh.same(dt, outs[r], want[r]), (servers, D, level1, det, dt, in_place, r)
+            finally:
+                g.close()
+
+
 def test_compiled_caller_through_the_c_abi():
     # a C++ program that includes <hccl/hccl.h> and links libhccl.so, built beforehand by cann-hccl_amd/build.py
     import os

@@ -320,3 +320,24 @@ def test_order_sensitive_known_answers_all_schedules(orc):
         # and the closed forms agree with the hand derivation
         want = CLOSED[algo](FP32, SUM, xs, 4, 200 << 20, kat["align"])
         assert float(want[0][0]) == kat["expected_element0"][name], name
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("atomic", [False, True])
+def test_two_level_allreduce_matches_closed_form(orc, level1, atomic):
+    # (servers, ranks per server): mesh inside a server, ring or halving-doubling between servers
+    closed1 = cf.ring_allreduce if level1 == RING else cf.rhd_allreduce
+    for servers, D in ((2, 4), (4, 2), (3, 4), (2, 8), (8, 1), (1, 8), (5, 3), (6, 2)):
+        p = servers * D
+        for dt, op, n, ccl in ((FP32, SUM, 2003, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, SUM, 1501, 200 << 20),
+                               (INT32, MAX, 700, 200 << 20)):
+            ins = _inputs(dt, p, n, 31 * p + n)
+            got = orc.allreduce_two_level(ins, dt, op, servers, level1=level1, atomic=atomic, ccl_bytes=ccl)
+            want = cf.two_level_allreduce(dt, op, ins, orc.dtype_size(dt), ccl, 128, servers, closed1, atomic)
+            for r in range(p):
+                assert _eq(dt, got[r], want[r]), (servers, D, level1, atomic, dt, ccl, r)
+    # one server is the plain mesh all-reduce
+    ins = _inputs(FP32, 8, 4099, 5)
+    a = orc.allreduce_two_level(ins, FP32, SUM, 1, level1=level1, atomic=atomic)
+    b = orc.allreduce(ins, FP32, SUM, algo=MESH_ATOMIC if atomic else MESH)
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))

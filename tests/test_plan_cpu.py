@@ -325,3 +325,27 @@ def test_broadcast_rhd_plan_matches_checker(orc, p):
                 (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, mem, mem, INT32, 0, in_place=True)
                 for r in range(p):
                     assert np.array_equal(mem[r].view(np.int32), want[r]), ("bcast rhd", p, root, ccl, fused, r)
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("shape", [(2, 4), (4, 2), (3, 4), (2, 8), (8, 1), (5, 3)])
+def test_two_level_allreduce_plan_matches_checker(orc, level1, shape):
+    servers, D = shape
+    p = servers * D
+    for atomic in (False, True):
+        for dt, op, n, ccl in ((FP32, SUM, 2003, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, PROD, 777, 200 << 20)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n, 400 + p + n)
+            want = orc.allreduce_two_level(ins, dt, op, servers, level1=level1, atomic=atomic, ccl_bytes=ccl)
+            for mask in (0, (1 << p) - 1):
+                plan = H.describe_plan(H.COLL_ALLREDUCE, level1 | (servers << 8) | (int(atomic) << 16), p, n, dt, ccl_bytes=ccl,
+                                       in_place_mask=mask)
+                assert plan["scratchBytes"] == 0
+                for fused in (False, True):
+                    if fused and not plan["fusedOk"]:
+                        continue
+                    sends = _bytes(ins)
+                    recvs = _bytes(ins) if mask else [np.full(n * unit, 0xA5, np.uint8) for _ in range(p)]
+                    (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op, in_place=bool(mask))
+                    for r in range(p):
+                        assert _same(dt, recvs[r], want[r]), (shape, level1, atomic, dt, ccl, mask, fused, r)
