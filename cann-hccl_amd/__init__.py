@@ -70,6 +70,21 @@ def comm_config_init():
     return cfg
 
 
+def comm_init_cluster_info(rank_table_path, n_ranks, config=None):
+    """One HcclCommInitClusterInfo[Config] per rank of the rank table (a JSON file); returns the handles."""
+    path = str(rank_table_path).encode()
+    comms = []
+    for r in range(n_ranks):
+        c = ctypes.c_void_p()
+        if config is None:
+            _check("HcclCommInitClusterInfo", lib().HcclCommInitClusterInfo(path, r, ctypes.byref(c)))
+        else:
+            _check("HcclCommInitClusterInfoConfig", lib().HcclCommInitClusterInfoConfig(path, r, ctypes.byref(config),
+                                                                                        ctypes.byref(c)))
+        comms.append(c)
+    return comms
+
+
 def comm_init_root_info(n_ranks, config=None):
     """HcclGetRootInfo + one HcclCommInitRootInfo[Config] per rank; returns the handles."""
     info = ctypes.create_string_buffer(4108)
@@ -144,6 +159,8 @@ def lib():
     L.HcclScatter.argtypes = [vp, vp, u64, i32, u32, vp, vp]
     L.HcclGetRootInfo.argtypes = [vp]
     L.HcclCommInitRootInfo.argtypes = [u32, vp, u32, ctypes.POINTER(vp)]
+    L.HcclCommInitClusterInfo.argtypes = [ctypes.c_char_p, u32, ctypes.POINTER(vp)]
+    L.HcclCommInitClusterInfoConfig.argtypes = [ctypes.c_char_p, u32, vp, ctypes.POINTER(vp)]
     L.HcclCommInitRootInfoConfig.argtypes = [u32, vp, u32, vp, ctypes.POINTER(vp)]
     L.HcclCreateSubCommConfig.argtypes = [ctypes.POINTER(vp), u32, ctypes.POINTER(u32), u64, u32, vp, ctypes.POINTER(vp)]
     L.HcclSend.argtypes = [vp, u64, i32, u32, vp, vp]

@@ -25,7 +25,7 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-I", os.path.join(
 # gfx950 only; packed fp32 instructions are switched off for device code
 DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 DTYPES = list(range(12)) + [255]
-HOST_SOURCES = ["plan.cc", "exec.cc", "api.cc", "kernels_table.cc"]
+HOST_SOURCES = ["plan.cc", "ranktable.cc", "exec.cc", "api.cc", "kernels_table.cc"]
 
 
 def _newer(target, deps):

@@ -7,14 +7,17 @@
 #include <chrono>
 #include <cstdlib>
 #include <cstring>
+#include <fstream>
 #include <map>
 #include <set>
+#include <sstream>
 #include <string>
 #include <vector>
 
 #include "hccl/hccl.h"
 #include "hccl/hccl_amd_ext.h"
 #include "log.h"
+#include "ranktable.h"
 #include "runtime.h"
 
 using namespace hcclamd;
@@ -1517,19 +1520,71 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
 
 // ---- declared for link compatibility; outside the single-GPU data path -----------------------------------
 
-HcclResult HcclCommInitClusterInfo(const char *clusterInfo, uint32_t, HcclComm *comm)
+// op_base.cc:465-503, :567-620 (declarations hccl.h:30, :42).  clusterInfo is the path of a rank table; its ranks are
+// the ranks of one group in this process (every one of them makes this call, as for the root-info
+// variant), and its servers become the rank groups of the two-level all-reduce.
+static HcclResult InitFromRankTable(const char *clusterInfo, uint32_t rank, const HcclCommConfig *config, HcclComm *comm)
+{
+    std::ifstream file(clusterInfo);
+    if (!file) {
+        HCCL_LOG_ERROR("HcclCommInitClusterInfo: cannot read the rank table %s", clusterInfo);
+        return HCCL_E_PARA;
+    }
+    std::stringstream text;
+    text << file.rdbuf();
+    RankTable table;
+    std::string err;
+    if (ParseRankTable(text.str(), &table, &err) != 0) {
+        HCCL_LOG_ERROR("HcclCommInitClusterInfo: %s", err.c_str());
+        return HCCL_E_PARA;
+    }
+    if (rank >= table.rankCount) {
+        HCCL_LOG_ERROR("HcclCommInitClusterInfo: rank %u is not in the rank table (%u ranks)", rank, table.rankCount);
+        return HCCL_E_PARA;
+    }
+    // the two-level schedule takes servers of equal size whose ranks are consecutive
+    const size_t perServer = table.servers[0].ranks.size();
+    bool regular = true;
+    for (size_t s = 0; s < table.servers.size(); s++) {
+        regular = regular && table.servers[s].ranks.size() == perServer;
+        for (size_t d = 0; regular && d < perServer; d++) {
+            regular = table.servers[s].ranks[d] == s * perServer + d;
+        }
+    }
+    if (!regular) {
+        HCCL_LOG_ERROR("HcclCommInitClusterInfo: servers must hold equally many ranks, numbered consecutively server by server");
+        return HCCL_E_NOT_SUPPORT;
+    }
+    HcclResult r = JoinFormingGroup(std::string("ranktable:") + clusterInfo, table.rankCount, rank, config, comm);
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    Group *g = AsComm(*comm)->group;
+    std::lock_guard<std::mutex> lock(g->m);
+    g->cfg.servers = uint32_t(table.servers.size());
+    return HCCL_SUCCESS;
+}
+
+HcclResult HcclCommInitClusterInfo(const char *clusterInfo, uint32_t rank, HcclComm *comm)
 {
     CHK_PTR(clusterInfo);
     CHK_PTR(comm);
-    return HCCL_E_NOT_SUPPORT;
+    return InitFromRankTable(clusterInfo, rank, nullptr, comm);
 }
-HcclResult HcclCommInitClusterInfoConfig(const char *clusterInfo, uint32_t, HcclCommConfig *config, HcclComm *comm)
+
+HcclResult HcclCommInitClusterInfoConfig(const char *clusterInfo, uint32_t rank, HcclCommConfig *config, HcclComm *comm)
 {
     CHK_PTR(clusterInfo);
     CHK_PTR(config);
     CHK_PTR(comm);
-    return HCCL_E_NOT_SUPPORT;
+    GroupConfig probe;
+    std::string name;
+    if (LoadCommConfig(config, &probe, &name) != HCCL_SUCCESS) {
+        return HCCL_E_PARA;
+    }
+    return InitFromRankTable(clusterInfo, rank, config, comm);
 }
+
 HcclResult HcclCommSetMemoryRange(HcclComm comm, void *, size_t, size_t, uint64_t)
 {
     CHK_PTR(comm);

@@ -523,7 +523,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         // two levels: mesh inside a group of ranks (uncut under the same conditions as the one-level
         // mesh, coll_all_reduce_mesh_executor.cc:108-112), ring or halving-doubling between the groups
         rq.servers = g->cfg.servers;
-        rq.algo = (algo == ALGO_RING) ? ALGO_RING : ALGO_RHD;
+        rq.algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_RHD;   // halving-doubling unless ring is asked for (:185-191)
         rq.meshAtomic = !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 && g->ctx->sig.op != HCCL_REDUCE_PROD;
     }
     if (g->ctx->sig.variable) {

@@ -170,13 +170,19 @@ extern HcclResult HcclCommInitRootInfoConfig(uint32_t nRanks, const HcclRootInfo
 extern HcclResult HcclCreateSubCommConfig(HcclComm *comm, uint32_t rankNum, uint32_t *rankIds,
     uint64_t subCommId, uint32_t subCommRankId, HcclCommConfig *config, HcclComm *subComm);
 
-/* ---- declared so existing binaries link; outside the single-GPU data path ------------------- */
-/* Rank-table bootstrap and virtual-memory registration concern several devices or the Ascend
- * memory manager; each returns HCCL_E_NOT_SUPPORT after the reference's own null-pointer checks.
- * decl inc/hccl/hccl.h:30-43,446-471. */
+/* Communicator from a rank table: clusterInfo is the path of the JSON file ("server_list" of servers with their
+ * "device" entries "device_id" / "rank_id"; addresses are ignored).  Every rank of the table makes this call
+ * from this process; the group lives on the current GPU.  Servers must hold equally many ranks, numbered
+ * consecutively server by server; with more than one server the all-reduce runs the two-level schedule
+ * (mesh inside a server, ring or halving-doubling between servers).
+ * decl inc/hccl/hccl.h:30 / :42, impl op_base.cc:465 / :567. */
 extern HcclResult HcclCommInitClusterInfo(const char *clusterInfo, uint32_t rank, HcclComm *comm);
 extern HcclResult HcclCommInitClusterInfoConfig(const char *clusterInfo, uint32_t rank,
     HcclCommConfig *config, HcclComm *comm);
+
+/* ---- declared so existing binaries link; outside the single-GPU data path ------------------- */
+/* Virtual-memory registration concerns the Ascend memory manager; each returns HCCL_E_NOT_SUPPORT
+ * after the reference's own null-pointer checks.  decl inc/hccl/hccl.h:446-471. */
 extern HcclResult HcclCommSetMemoryRange(HcclComm comm, void *baseVirPtr, size_t size, size_t alignment,
     uint64_t flags);
 extern HcclResult HcclCommUnsetMemoryRange(HcclComm comm, void *baseVirPtr);

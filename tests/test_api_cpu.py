@@ -237,7 +237,6 @@ def test_amd_params(comms):
 
 
 def test_unsupported_entry_points_link_and_refuse(comms):
-    assert L.HcclCommInitClusterInfo(b"ranktable.json", 0, ctypes.byref(ctypes.c_void_p())) == H.HCCL_E_NOT_SUPPORT
     assert L.HcclCommSetMemoryRange(comms[0], BUF_A, 4096, 0, 0) == H.HCCL_E_NOT_SUPPORT
 
 
@@ -364,3 +363,62 @@ def test_caller_compiles_against_the_reference_header_and_links(tmp_path):
         pytest.skip("reference tree not present on this machine")
     theirs = build.build_abi_caller(include_dirs=[ref_inc], out=str(tmp_path / "caller_ref"))
     assert os.path.exists(theirs)
+
+
+def _rank_table(path, servers, per_server, **edits):
+    import json
+    table = {"server_count": str(servers), "status": "completed", "version": "1.0", "server_list": []}
+    for s in range(servers):
+        devices = [{"device_id": str(d), "device_ip": "192.168.%d.%d" % (s, d), "rank_id": str(s * per_server + d)}
+                   for d in range(per_server)]
+        table["server_list"].append({"server_id": "10.0.0.%d" % (s + 1), "device": devices})
+    table.update(edits)
+    with open(path, "w") as f:
+        json.dump(table, f, indent=1)
+    return str(path).encode()
+
+
+def test_comm_from_rank_table(tmp_path):
+    # HcclCommInitClusterInfo: the rank table's ranks form one group; its servers become the rank groups
+    path = _rank_table(tmp_path / "ranktable.json", 2, 4)
+    comms = []
+    for r in range(8):
+        c = ctypes.c_void_p()
+        assert L.HcclCommInitClusterInfo(path, r, ctypes.byref(c)) == H.HCCL_SUCCESS
+        comms.append(c)
+    n, rank = ctypes.c_uint32(0), ctypes.c_uint32(99)
+    assert L.HcclGetRankSize(comms[5], ctypes.byref(n)) == 0 and n.value == 8
+    assert L.HcclGetRankId(comms[5], ctypes.byref(rank)) == 0 and rank.value == 5
+    extra = ctypes.c_void_p()
+    assert L.HcclCommInitClusterInfo(path, 8, ctypes.byref(extra)) == H.HCCL_E_PARA        # not in the table
+    H.comm_destroy(comms)
+    # with a configuration
+    cfg = H.comm_config_init()
+    cfg.hcclBufferSize = 64
+    comms = []
+    for r in range(8):
+        c = ctypes.c_void_p()
+        assert L.HcclCommInitClusterInfoConfig(path, r, ctypes.byref(cfg), ctypes.byref(c)) == H.HCCL_SUCCESS
+        comms.append(c)
+    H.comm_destroy(comms)
+    # refusals
+    c = ctypes.c_void_p()
+    assert L.HcclCommInitClusterInfo(None, 0, ctypes.byref(c)) == H.HCCL_E_PTR
+    assert L.HcclCommInitClusterInfo(path, 0, None) == H.HCCL_E_PTR
+    assert L.HcclCommInitClusterInfo(str(tmp_path / "missing.json").encode(), 0, ctypes.byref(c)) == H.HCCL_E_PARA
+    bad = tmp_path / "bad.json"
+    bad.write_text("{ not json")
+    assert L.HcclCommInitClusterInfo(str(bad).encode(), 0, ctypes.byref(c)) == H.HCCL_E_PARA
+    wrong_count = _rank_table(tmp_path / "count.json", 2, 4, server_count="3")
+    assert L.HcclCommInitClusterInfo(wrong_count, 0, ctypes.byref(c)) == H.HCCL_E_PARA
+    empty = _rank_table(tmp_path / "empty.json", 2, 4, server_list=[], server_count="0")
+    assert L.HcclCommInitClusterInfo(empty, 0, ctypes.byref(c)) == H.HCCL_E_PARA
+    import json
+    uneven = json.loads(open(tmp_path / "ranktable.json").read())
+    uneven["server_list"][1]["device"].pop()
+    (tmp_path / "uneven.json").write_text(json.dumps(uneven))
+    assert L.HcclCommInitClusterInfo(str(tmp_path / "uneven.json").encode(), 0, ctypes.byref(c)) == H.HCCL_E_NOT_SUPPORT
+    twice = json.loads(open(tmp_path / "ranktable.json").read())
+    twice["server_list"][1]["device"][0]["rank_id"] = "0"
+    (tmp_path / "twice.json").write_text(json.dumps(twice))
+    assert L.HcclCommInitClusterInfo(str(tmp_path / "twice.json").encode(), 0, ctypes.byref(c)) == H.HCCL_E_PARA

@@ -649,6 +649,38 @@ def test_two_level_allreduce(orc, level1):
                 g.close()
 
 
+def test_allreduce_on_a_rank_table_communicator(orc, tmp_path):
+    # 2 servers x 4 devices from a rank table: the all-reduce runs the two-level schedule by itself
+    import json
+    servers, D = 2, 4
+    table = {"server_count": str(servers), "status": "completed", "version": "1.0", "server_list": [
+        {"server_id": "10.0.0.%d" % (s + 1),
+         "device": [{"device_id": str(d), "device_ip": "192.168.%d.%d" % (s, d), "rank_id": str(s * D + d)} for d in range(D)]}
+        for s in range(servers)]}
+    path = tmp_path / "ranktable.json"
+    path.write_text(json.dumps(table))
+    p = servers * D
+    comms = H.comm_init_cluster_info(path, p)
+    stream = torch.cuda.Stream()
+    try:
+        n = 200003
+        ins = _ins(FP32, p, n, 77)
+        for algo, level1 in ((None, RHD), ("ring", RING)):
+            if algo:
+                H.set_param(comms[0], "algo", algo)
+            want = orc.allreduce_two_level(ins, FP32, SUM, servers, level1=level1, atomic=True)
+            sends = [gh.to_dev(x) for x in ins]
+            recvs = [gh.empty_dev(n * 4) for _ in range(p)]
+            torch.cuda.synchronize()
+            H.all_reduce(comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, stream.cuda_stream)
+            stream.synchronize()
+            for r in range(p):
+                assert np.array_equal(gh.to_host(recvs[r], FP32), want[r]), (algo, r)
+    finally:
+        torch.cuda.synchronize()
+        H.comm_destroy(comms)
+
+
 def test_compiled_caller_through_the_c_abi():
     # a C++ program that includes <hccl/hccl.h> and links libhccl.so, built beforehand by cann-hccl_amd/build.py
     import os
