@@ -681,6 +681,38 @@ def test_allreduce_on_a_rank_table_communicator(orc, tmp_path):
         H.comm_destroy(comms)
 
 
+def test_many_shapes_evict_cached_collectives_without_leaking(orc):
+    # more distinct shapes than the library keeps prepared (64): old entries are dropped, results stay right and
+    # device memory returns to where it was
+    p = 4
+    g = gh.Group(p)
+    try:
+        rng = np.random.default_rng(404)
+        base = np.stack([rng.integers(-1000, 1000, 70000).astype(np.int32) for _ in range(p)])
+        sends = [gh.to_dev(base[r]) for r in range(p)]
+        recvs = [gh.empty_dev(70000 * 4) for _ in range(p)]
+        torch.cuda.synchronize()
+        free0 = None
+        for round_ in range(3):
+            for k in range(100):
+                n = 1000 + 577 * k
+                g.set(fuse=k % 2)
+                H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, INT32, SUM, g.stream_ptr)
+                if k % 17 == 0:
+                    g.stream.synchronize()
+                    want = base[:, :n].sum(axis=0, dtype=np.int64).astype(np.int32)
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(recvs[r], INT32)[:n], want), (round_, k, r)
+            torch.cuda.synchronize()
+            free, _ = torch.cuda.mem_get_info()
+            if free0 is None:
+                free0 = free            # after the first round the cache is full
+            else:
+                assert free0 - free < (8 << 20), ("device memory keeps growing", free0, free)
+    finally:
+        g.close()
+
+
 def test_compiled_caller_through_the_c_abi():
     # a C++ program that includes <hccl/hccl.h> and links libhccl.so, built beforehand by cann-hccl_amd/build.py
     import os
