@@ -304,13 +304,14 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
         }
     } else {
         // one launch per kernel kind present
-        for (int kind : {int(KK_CHAIN), int(KK_TREE)}) {
+        for (int kind : {int(KK_CHAIN), int(KK_TREE), int(KK_STACK)}) {
             std::vector<FusedDesc> descs;
             std::vector<const void *> srcPool;
+            std::vector<uint32_t> opPool;      // stack items: one word per source-pool entry
             std::vector<void *> dstPool;
             uint32_t tiles = 0;
             for (const FusedItem &it : pp->plan->fused) {
-                int want = (it.kind == FK_TREE) ? int(KK_TREE) : int(KK_CHAIN);
+                int want = it.kind == FK_TREE ? int(KK_TREE) : (it.kind == FK_STACK ? int(KK_STACK) : int(KK_CHAIN));
                 if (want != kind) {
                     continue;
                 }
@@ -343,8 +344,11 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                     d.srcBase = uint32_t(srcPool.size());
                     d.dstBase = uint32_t(dstPool.size());
                     d.nleaf = it.nleaf;
-                    for (char *s : srcs) {
-                        srcPool.push_back(s ? s + off : nullptr);
+                    for (size_t k = 0; k < srcs.size(); k++) {
+                        srcPool.push_back(srcs[k] ? srcs[k] + off : nullptr);
+                        if (kind == int(KK_STACK)) {
+                            opPool.push_back(k < it.ops.size() ? it.ops[k] : 0u);
+                        }
                     }
                     for (char *t : dsts) {
                         dstPool.push_back(t + off);
@@ -361,8 +365,13 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                 return HCCL_E_NOT_SUPPORT;
             }
             PendingLaunch pl;
-            pl.tableAt = b.Reserve(descs.size() * sizeof(FusedDesc));
+            // the op words of the stack kernel sit right behind its item table
+            pl.tableAt = b.Reserve(descs.size() * sizeof(FusedDesc) + opPool.size() * sizeof(uint32_t));
             std::memcpy(b.host.data() + pl.tableAt, descs.data(), descs.size() * sizeof(FusedDesc));
+            if (!opPool.empty()) {
+                std::memcpy(b.host.data() + pl.tableAt + descs.size() * sizeof(FusedDesc), opPool.data(),
+                    opPool.size() * sizeof(uint32_t));
+            }
             pl.srcAt = b.Reserve(srcPool.size() * sizeof(void *));
             std::memcpy(b.host.data() + pl.srcAt, srcPool.data(), srcPool.size() * sizeof(void *));
             pl.dstAt = b.Reserve(dstPool.size() * sizeof(void *));

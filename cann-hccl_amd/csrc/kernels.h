@@ -35,6 +35,10 @@ struct StepDesc {
 //   chain : acc = src[0]; for j = 1..nsrc-1: acc = bit j of accLeftMask ? acc (+) src[j] : src[j] (+) acc
 //   tree  : nleaf leaves, leaf i = src[2i] (+) src[2i+1] (src[2i+1] may be null); then
 //           v[i] = v[i] (+) v[i+w] for w = 1, 2, 4, ... ; result v[0]
+//   stack : any other expression.  Sources in evaluation order; after pushing src[j] the two topmost
+//           values are folded ops[j] & 7 times, bit 8 + i of ops[j] set = the lower value is the left
+//           operand of fold i.  The launch's op words (one uint32 per source-pool entry, same index)
+//           follow its item table in memory.
 struct FusedDesc {
     uint64_t bytes;
     uint64_t accLeftMask;
@@ -51,13 +55,14 @@ struct FusedDesc {
 // flags of the step kernel
 constexpr uint32_t kStepOrdinaryStores = 1u;   // write-back stores instead of non-temporal ones in the fast loop
 
-enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_COUNT = 3 };
+enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_STACK = 3, KK_COUNT = 4 };
 
 // Kernel entry for (data type, reduce op, kind); nullptr if the combination is not built.
 // Signatures:
 //   KK_STEP            (const StepDesc *steps, uint32_t nsteps, uint32_t nwhole, uint32_t ntiles, uint32_t flags)
 //                      steps whose tiles are all whole and ACC_VEC16 come first: tiles [0, nwhole)
-//   KK_CHAIN / KK_TREE (const FusedDesc *items, uint32_t nitems, uint32_t ntiles,
+//   KK_CHAIN / KK_TREE / KK_STACK
+//                      (const FusedDesc *items, uint32_t nitems, uint32_t ntiles,
 //                       const void *const *srcPool, void *const *dstPool)
 const void *LookupKernel(int hcclDataType, int hcclReduceOp, KernelKind kind);
 

@@ -62,6 +62,7 @@ extern const void *const HCCL_CAT(kKernels_, HCCL_DT_NAME)[2] = {
         reinterpret_cast<const void *>(&StepKernel<DT, OP>),             \
         reinterpret_cast<const void *>(&ChainKernel<DT, OP>),            \
         reinterpret_cast<const void *>(&TreeKernel<DT, OP>),             \
+        reinterpret_cast<const void *>(&StackKernel<DT, OP>),            \
     }
 extern const void *const HCCL_CAT(kKernels_, HCCL_DT_NAME)[4][KK_COUNT] = {
     HCCL_ROW(ROP_SUM), HCCL_ROW(ROP_PROD), HCCL_ROW(ROP_MAX), HCCL_ROW(ROP_MIN),

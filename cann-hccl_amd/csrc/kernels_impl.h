@@ -830,4 +830,181 @@ __global__ void __launch_bounds__(kBlockThreads) TreeKernel(const FusedDesc *__r
     }
 }
 
+// ---- fused general expression: a stack machine over registers -----------------------------------------
+// Handles what is neither a chain nor a perfect tree (a ring or halving-doubling schedule whose
+// operands are themselves mesh chains, for one).  The item's sources come in evaluation order; after
+// source j the two topmost values are folded ops[j] & 7 times, bit 8 + i saying which of the two is
+// the left operand in fold i.  The op words of a launch follow its item table in memory.
+// The stack lives in registers: its depth is a wave-uniform number, so every access goes through a
+// switch with constant indices.  Sources are loaded in batches like the chain kernel's.
+constexpr uint32_t kStackVec = 2;        // vectors per lane per pass
+constexpr uint32_t kStackSrcBatch = 8;
+
+struct StackVal {
+    V4 x[kStackVec];
+};
+
+// The values below the top one are seven separate variables, not an array or a struct: a switch over
+// parts of one object is merged by the compiler into a single access at a computed offset, which
+// moves the object to private memory.
+#define HCCL_STACK_PUT(i, v)          \
+    switch (i) {                      \
+        case 0: b0 = (v); break;      \
+        case 1: b1 = (v); break;      \
+        case 2: b2 = (v); break;      \
+        case 3: b3 = (v); break;      \
+        case 4: b4 = (v); break;      \
+        case 5: b5 = (v); break;      \
+        default: b6 = (v); break;     \
+    }
+#define HCCL_STACK_GET(i, v)          \
+    switch (i) {                      \
+        case 0: (v) = b0; break;      \
+        case 1: (v) = b1; break;      \
+        case 2: (v) = b2; break;      \
+        case 3: (v) = b3; break;      \
+        case 4: (v) = b4; break;      \
+        case 5: (v) = b5; break;      \
+        default: (v) = b6; break;     \
+    }
+
+template <typename T, int OP, uint32_t MODE, bool FULL>
+__device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *const *__restrict__ src,
+    const uint32_t *__restrict__ ops, void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec)
+{
+    uint64_t pos[kStackVec];
+    bool live[kStackVec];
+#pragma unroll
+    for (uint32_t u = 0; u < kStackVec; u++) {
+        uint32_t i = vecBase + u * kBlockThreads + threadIdx.x;
+        live[u] = FULL || i < nvec;
+        pos[u] = off + uint64_t(i) * 16;
+    }
+    StackVal top;
+#pragma unroll
+    for (uint32_t u = 0; u < kStackVec; u++) {
+        top.x[u] = V4{0, 0, 0, 0};
+    }
+    StackVal b0 = top, b1 = top, b2 = top, b3 = top, b4 = top, b5 = top, b6 = top;
+    uint32_t depth = 0;                  // values on the stack, the top one included
+    const uint32_t nsrc = d.nsrc;
+    for (uint32_t j = 0; j < nsrc; j += kStackSrcBatch) {
+        StackVal v[kStackSrcBatch];
+#pragma unroll
+        for (uint32_t jj = 0; jj < kStackSrcBatch; jj++) {
+            if (j + jj < nsrc) {
+                const void *s = src[j + jj];
+#pragma unroll
+                for (uint32_t u = 0; u < kStackVec; u++) {
+                    if (live[u]) {
+                        v[jj].x[u] = Load16<MODE>(s, pos[u]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t jj = 0; jj < kStackSrcBatch; jj++) {
+            if (j + jj < nsrc) {
+                const uint32_t op = ops[j + jj];
+                if (depth > 0) {
+                    HCCL_STACK_PUT(depth - 1, top)
+                }
+                top = v[jj];
+                depth++;
+                const uint32_t nfold = op & 7u;
+#pragma nounroll
+                for (uint32_t f = 0; f < nfold && depth >= 2; f++) {
+                    StackVal under;
+                    HCCL_STACK_GET(depth - 2, under)
+                    const bool underLeft = !OrderMatters<T, OP>::value || ((op >> (8 + f)) & 1u);
+#pragma unroll
+                    for (uint32_t u = 0; u < kStackVec; u++) {
+                        if (live[u]) {
+                            top.x[u] = underLeft ? Combine16<T, OP>(under.x[u], top.x[u]) : Combine16<T, OP>(top.x[u], under.x[u]);
+                        }
+                    }
+                    depth--;
+                }
+            }
+        }
+    }
+    const uint32_t ndst = d.ndst;
+    for (uint32_t k = 0; k < ndst; k++) {
+        void *o = dst[k];
+#pragma unroll
+        for (uint32_t u = 0; u < kStackVec; u++) {
+            if (live[u]) {
+                StoreAny16<MODE>(o, pos[u], top.x[u]);
+            }
+        }
+    }
+}
+
+// Heads, tails and unaligned buffers: the same machine element by element.
+template <typename T, int OP>
+__device__ __forceinline__ void StackElem(const FusedDesc &d, const void *const *__restrict__ src,
+    const uint32_t *__restrict__ ops, void *const *__restrict__ dst, uint64_t off, uint32_t n)
+{
+    const uint32_t cnt = n / sizeof(T);
+    for (uint32_t e = threadIdx.x; e < cnt; e += kBlockThreads) {
+        const uint64_t at = off + uint64_t(e) * sizeof(T);
+        T top = T();
+        T b0 = top, b1 = top, b2 = top, b3 = top, b4 = top, b5 = top, b6 = top;
+        uint32_t depth = 0;
+        for (uint32_t j = 0; j < d.nsrc; j++) {
+            const uint32_t op = ops[j];
+            if (depth > 0) {
+                HCCL_STACK_PUT(depth - 1, top)
+            }
+            top = LoadElem<T>(src[j], at);
+            depth++;
+            const uint32_t nfold = op & 7u;
+            for (uint32_t f = 0; f < nfold && depth >= 2; f++) {
+                T under;
+                HCCL_STACK_GET(depth - 2, under)
+                top = ((op >> (8 + f)) & 1u) ? Elem<T, OP>::Apply(under, top) : Elem<T, OP>::Apply(top, under);
+                depth--;
+            }
+        }
+        for (uint32_t k = 0; k < d.ndst; k++) {
+            StoreElem<T>(dst[k], at, top);
+        }
+    }
+}
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(kBlockThreads) StackKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
+    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool)
+{
+    const uint32_t *opPool = reinterpret_cast<const uint32_t *>(items + nitems);
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const FusedDesc d = items[FindDesc(items, nitems, tile)];
+        const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
+        const uint64_t left = d.bytes - off;
+        const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
+        const void *const *src = srcPool + d.srcBase;
+        const uint32_t *ops = opPool + d.srcBase;
+        void *const *dst = dstPool + d.dstBase;
+        if (d.mode == ACC_ELEM) {
+            StackElem<T, OP>(d, src, ops, dst, off, n);
+        } else {
+            const uint32_t nvec = n >> 4;
+            constexpr uint32_t kPass = kStackVec * kBlockThreads;
+            uint32_t base = 0;
+            if (d.mode == ACC_VEC16) {
+                for (; base + kPass <= nvec; base += kPass) {
+                    StackVecPass<T, OP, ACC_VEC16, true>(d, src, ops, dst, off, base, nvec);
+                }
+                if (base < nvec) {
+                    StackVecPass<T, OP, ACC_VEC16, false>(d, src, ops, dst, off, base, nvec);
+                }
+            } else {
+                for (; base < nvec; base += kPass) {
+                    StackVecPass<T, OP, ACC_VEC16_SRC4, false>(d, src, ops, dst, off, base, nvec);
+                }
+            }
+        }
+    }
+}
+
 }  // namespace hcclamd

@@ -1226,6 +1226,67 @@ bool AsTree(const Sym &sym, int e, uint64_t delta, FusedItem *item)
     return false;
 }
 
+// Any expression as a stack program.  Of the two operands of a combine the one that needs the deeper
+// stack is evaluated first (the classic register-need numbering), which keeps chains at depth 2 and a
+// tree of 2^k equal parts at k + 1 whatever way they lean.
+struct StackForm {
+    const Sym &sym;
+    std::unordered_map<int, uint32_t> need, leaves;
+    explicit StackForm(const Sym &s) : sym(s) {}
+    void Measure(int e)
+    {
+        if (need.count(e)) {
+            return;
+        }
+        const ENode &n = sym.nodes[e];
+        if (!n.red) {
+            need[e] = 1;
+            leaves[e] = 1;
+            return;
+        }
+        Measure(n.a);
+        Measure(n.b);
+        uint32_t na = need[n.a], nb = need[n.b];
+        need[e] = na == nb ? na + 1 : std::max(na, nb);
+        leaves[e] = std::min<uint32_t>(leaves[n.a] + leaves[n.b], 1u << 20);
+    }
+    void Emit(int e, uint64_t delta, FusedItem *item)
+    {
+        const ENode &n = sym.nodes[e];
+        if (!n.red) {
+            item->src.push_back(LeafRef(sym, e, delta));
+            item->srcValid.push_back(1);
+            item->ops.push_back(0);
+            return;
+        }
+        const bool leftFirst = need[n.a] >= need[n.b];
+        if (leftFirst) {
+            Emit(n.a, n.da + delta, item);
+            Emit(n.b, n.db + delta, item);
+        } else {
+            Emit(n.b, n.db + delta, item);
+            Emit(n.a, n.da + delta, item);
+        }
+        uint16_t &op = item->ops.back();
+        const uint32_t k = op & 7u;              // at most depth - 1 folds follow one push
+        op = uint16_t((op & ~7u) | (k + 1) | (leftFirst ? (1u << (8 + k)) : 0u));
+    }
+};
+
+bool AsStack(const Sym &sym, int e, uint64_t delta, FusedItem *item)
+{
+    StackForm f(sym);
+    f.Measure(e);
+    if (f.need[e] > kStackDepth || f.leaves[e] > kStackMaxSrc) {
+        return false;
+    }
+    item->kind = FK_STACK;
+    item->src.clear();
+    item->srcValid.clear();
+    item->ops.clear();
+    f.Emit(e, delta, item);
+    return true;
+}
 
 bool BuildFused(const Sym &sym, const PlanRequest &rq, std::vector<FusedItem> *items)
 {
@@ -1241,7 +1302,8 @@ bool BuildFused(const Sym &sym, const PlanRequest &rq, std::vector<FusedItem> *i
                 item.kind = FK_COPY;
                 item.src.push_back(LeafRef(sym, o.expr, o.delta));
                 item.srcValid.push_back(1);
-            } else if (!AsChain(sym, o.expr, o.delta, &item) && !AsTree(sym, o.expr, o.delta, &item)) {
+            } else if (!AsChain(sym, o.expr, o.delta, &item) && !AsTree(sym, o.expr, o.delta, &item) &&
+                       !AsStack(sym, o.expr, o.delta, &item)) {
                 return false;
             }
             items->push_back(item);
@@ -1573,6 +1635,10 @@ std::string DescribePlan(const Plan &plan)
         os << "],\"accLeft\":[";
         for (size_t k = 0; k < it.accLeft.size(); k++) {
             os << (k ? "," : "") << int(it.accLeft[k]);
+        }
+        os << "],\"ops\":[";
+        for (size_t k = 0; k < it.ops.size(); k++) {
+            os << (k ? "," : "") << int(it.ops[k]);
         }
         os << "],\"dst\":[";
         for (size_t k = 0; k < it.dst.size(); k++) {

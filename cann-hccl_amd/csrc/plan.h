@@ -54,9 +54,16 @@ struct Phase {
 enum FusedKind : uint8_t {
     FK_COPY = 0,    // dst[*] = src[0]
     FK_CHAIN = 1,   // acc = src[0]; acc = accLeft[j] ? acc (+) src[j] : src[j] (+) acc, j = 1..n-1
-    FK_TREE = 2     // nleaf = 2^k leaves (leaf i = src[2i] or src[2i] (+) src[2i+1]); pairwise
+    FK_TREE = 2,    // nleaf = 2^k leaves (leaf i = src[2i] or src[2i] (+) src[2i+1]); pairwise
                     // bottom-up: v[i] = v[i] (+) v[i+w] for w = 1, 2, 4, ...
+    FK_STACK = 3    // any other expression, in stack-machine form: for each source in turn push it, then
+                    // fold the two topmost values ops[j] & 7 times; bit 8 + i of ops[j] set = in fold i the
+                    // lower value is the left operand, clear = the top value is
 };
+
+// Limits of the stack form (what its kernel holds in registers).
+constexpr uint32_t kStackDepth = 8;
+constexpr uint32_t kStackMaxSrc = 64;
 
 struct FusedItem {
     FusedKind kind = FK_COPY;
@@ -64,6 +71,7 @@ struct FusedItem {
     std::vector<Ref> src;
     std::vector<uint8_t> srcValid;   // FK_TREE: second source of a leaf may be absent
     std::vector<uint8_t> accLeft;    // FK_CHAIN: one flag per src (index 0 unused)
+    std::vector<uint16_t> ops;       // FK_STACK: one word per src
     uint32_t nleaf = 0;
     std::vector<Ref> dst;
 };

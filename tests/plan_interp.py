@@ -46,6 +46,18 @@ def run_fused(plan, sends, recvs, dt, op, in_place=False):
             for j in range(1, len(it["src"])):
                 v = load(it["src"][j])
                 acc = cf.combine(dt, op, acc, v) if it["accLeft"][j] else cf.combine(dt, op, v, acc)
+        elif it["kind"] == 3:
+            # stack form: push each source, then fold the two topmost values ops[j] & 7 times
+            stack = []
+            for j, ref in enumerate(it["src"]):
+                stack.append(load(ref))
+                for f in range(it["ops"][j] & 7):
+                    top = stack.pop()
+                    under = stack.pop()
+                    lower_is_left = (it["ops"][j] >> (8 + f)) & 1
+                    stack.append(cf.combine(dt, op, under, top) if lower_is_left else cf.combine(dt, op, top, under))
+            assert len(stack) == 1
+            acc = stack[0]
         else:
             leaves = []
             for i in range(it["nleaf"]):

@@ -641,12 +641,38 @@ def test_two_level_allreduce(orc, level1):
                     ins = _ins(dt, p, n, 17 * p + n)
                     want = orc.allreduce_two_level(ins, dt, op, servers, level1=level1, atomic=atomic)
                     print("two-level", servers, "x", D, "level1", level1, "deterministic", det, "type", dt, flush=True)
-                    for in_place in (False, True):
-                        outs, _ = gh.all_reduce(g, ins, dt, op, in_place=in_place)
-                        for r in range(p):
-                            assert gh.same(dt, outs[r], want[r]), (servers, D, level1, det, dt, in_place, r)
+                    for fuse in (1, 0):
+                        g.set(fuse=fuse)
+                        for in_place in (False, True):
+                            outs, _ = gh.all_reduce(g, ins, dt, op, in_place=in_place)
+                            assert g.info()["fused"] == fuse     # every two-level expression has a fused form
+                            for r in range(p):
+                                assert gh.same(dt, outs[r], want[r]), (servers, D, level1, det, dt, fuse, in_place, r)
             finally:
                 g.close()
+
+
+@pytest.mark.gpu
+def test_two_level_allreduce_operand_order_of_max_min(orc):
+    # NaN payloads and signed zeros show which operand stood left in every combine of the fused form
+    specials = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.0, -1.0, 3.4e38], np.float32)
+    nan2 = np.array([0x7fc00001, 0xffc00002, 0x7fa00003], np.uint32).view(np.float32)
+    pool = np.concatenate([specials, nan2])
+    for servers, D, level1 in ((2, 4, RING), (3, 4, RHD), (4, 4, RHD), (8, 2, RING)):
+        p = servers * D
+        rng = np.random.default_rng(1000 + p)
+        ins = [rng.choice(pool, 20000 + 3).astype(np.float32) for _ in range(p)]
+        g = gh.Group(p, algo=ALGO_NAME[level1], deterministic=1, servers=servers, align=4)
+        try:
+            for op in (MAX, MIN):
+                want = orc.allreduce_two_level(ins, FP32, op, servers, level1=level1, atomic=False, align=4)
+                for fuse in (1, 0):
+                    g.set(fuse=fuse)
+                    outs, _ = gh.all_reduce(g, ins, FP32, op)
+                    for r in range(p):
+                        assert np.array_equal(outs[r].view(np.uint32), want[r].view(np.uint32)), (servers, D, level1, op, fuse, r)
+        finally:
+            g.close()
 
 
 def test_allreduce_on_a_rank_table_communicator(orc, tmp_path):

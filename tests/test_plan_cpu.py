@@ -349,3 +349,29 @@ def test_two_level_allreduce_plan_matches_checker(orc, level1, shape):
                     (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op, in_place=bool(mask))
                     for r in range(p):
                         assert _same(dt, recvs[r], want[r]), (shape, level1, atomic, dt, ccl, mask, fused, r)
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+def test_two_level_fused_stack_form_keeps_operand_order(orc, level1):
+    # every two-level expression has a fused form (a stack program); NaN payloads and signed zeros under
+    # max / min show which operand stood left in each of its combines
+    pool = np.concatenate([np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0], np.float32),
+                           np.array([0x7fc00001, 0xffc00002, 0x7fa00003], np.uint32).view(np.float32)])
+    for servers, D in ((2, 4), (3, 4), (4, 4), (8, 2), (5, 3)):
+        p = servers * D
+        rng = np.random.default_rng(31 * p + level1)
+        ins = [rng.choice(pool, 1501).astype(np.float32) for _ in range(p)]
+        for op in (H.HCCL_REDUCE_MAX, H.HCCL_REDUCE_MIN):
+            want = orc.allreduce_two_level(ins, FP32, op, servers, level1=level1, atomic=False, align=4)
+            plan = H.describe_plan(H.COLL_ALLREDUCE, level1 | (servers << 8), p, 1501, FP32, align=4)
+            assert plan["fusedOk"]
+            kinds = {it["kind"] for it in plan["fused"]}
+            assert kinds <= {2, 3} and (3 in kinds or (level1 == RHD and D == 2))
+            for it in plan["fused"]:
+                if it["kind"] == 3:
+                    assert len(it["src"]) == p and sum(o & 7 for o in it["ops"]) == p - 1
+            sends = _bytes(ins)
+            recvs = [np.full(1501 * 4, 0xA5, np.uint8) for _ in range(p)]
+            plan_interp.run_fused(plan, sends, recvs, FP32, op)
+            for r in range(p):
+                assert np.array_equal(recvs[r].view(np.uint32), want[r].view(np.uint32)), (servers, D, level1, op, r)
