@@ -227,12 +227,13 @@ def run_suite(pkg, torch, steps, warmup, only="", settings=()):
                 report("broadcast %s p=8 256MiB root 3" % ralgo, comms,
                        lambda: pkg.broadcast(comms, rp, n, FP32, 3, stream.cuda_stream))
         pkg.comm_destroy(comms)
-    for servers, level1 in ((2, "ring"), (2, "rhd"), (4, "rhd")):
+    for servers, level0, level1 in ((2, "mesh", "ring"), (2, "mesh", "rhd"), (4, "mesh", "rhd"), (2, "ring", "rhd"), (1, "ring4", "rhd")):
         comms = pkg.comm_init_all(p)
         pkg.set_param(comms[0], "servers", servers)
+        pkg.set_param(comms[0], "level0", level0)
         pkg.set_param(comms[0], "algo", level1)
         torch.cuda.synchronize()
-        report("all-reduce two-level %dx%d mesh+%s fp32 sum 256MiB/rank" % (servers, p // servers, level1), comms,
+        report("all-reduce two-level %dx%d %s+%s fp32 sum 256MiB/rank" % (servers, p // servers, level0, level1), comms,
                lambda: pkg.all_reduce(comms, sp, rp, n, FP32, 0, stream.cuda_stream))
         pkg.comm_destroy(comms)
     comms = pkg.comm_init_all(p)

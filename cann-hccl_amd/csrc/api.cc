@@ -1380,6 +1380,16 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
             return HCCL_E_PARA;
         }
         cfg.servers = uint32_t(n);
+    } else if (k == "level0") {
+        if (v == "mesh") {
+            cfg.level0Rings = 0;
+        } else if (v == "ring") {
+            cfg.level0Rings = 1;
+        } else if (v == "ring4") {
+            cfg.level0Rings = 4;
+        } else {
+            return HCCL_E_PARA;
+        }
     } else if (k == "step_stores") {
         if (v == "auto") {
             cfg.stepStores = -1;
@@ -1476,6 +1486,7 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         rq.algo = Algo(uint32_t(algo) & 0xffu);
         rq.servers = std::max(1u, (uint32_t(algo) >> 8) & 0xffu);
         rq.meshAtomic = ((uint32_t(algo) >> 16) & 1u) != 0;   // bit 16: mesh level without the piece cut
+        rq.level0Rings = (uint32_t(algo) >> 17) & 7u;         // bits 17..19: rings inside a group (0 = mesh, 1, 4)
     } else {
         rq.algo = Algo(algo);
     }

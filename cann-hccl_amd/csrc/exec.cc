@@ -457,7 +457,7 @@ std::string CacheKey(const Group *g, int algo)
     uint64_t head[10] = {uint64_t(g->ctx->sig.coll), uint64_t(algo), uint64_t(g->ctx->sig.dtype), uint64_t(g->ctx->sig.op), g->ctx->sig.count,
         uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1) | (uint64_t(g->ctx->sig.root) << 8) | (uint64_t(g->ctx->sig.peer) << 20), g->cfg.cclBytes, g->cfg.align,
         uint64_t(g->cfg.blocksPerCu) | (uint64_t(uint32_t(g->cfg.stepStores + 1)) << 32) | (uint64_t(g->cfg.servers) << 40) |
-            (uint64_t(g->cfg.deterministic) << 56), g->p};
+            (uint64_t(g->cfg.deterministic) << 56) | (uint64_t(g->cfg.level0Rings) << 57), g->p};
     put(head, sizeof(head));
     put(g->ctx->send.data(), g->ctx->send.size() * sizeof(void *));
     put(g->ctx->recv.data(), g->ctx->recv.size() * sizeof(void *));
@@ -483,7 +483,7 @@ int CachedPlan(Group *g, const PlanRequest &rq, std::shared_ptr<const Plan> *out
         put(v.data(), v.size() * sizeof(uint64_t));
     };
     uint64_t head[10] = {uint64_t(rq.coll), uint64_t(rq.algo), rq.p, rq.count, rq.root, rq.peer, rq.unit, rq.cclBytes, rq.align,
-        uint64_t(rq.meshAtomic) | (uint64_t(rq.stageInput) << 1) | (uint64_t(rq.servers) << 8)};
+        uint64_t(rq.meshAtomic) | (uint64_t(rq.stageInput) << 1) | (uint64_t(rq.servers) << 8) | (uint64_t(rq.level0Rings) << 40)};
     put(head, sizeof(head));
     put(rq.alias.data(), rq.alias.size());
     putVec(rq.sendCounts);
@@ -528,12 +528,16 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
     for (uint32_t r = 0; r < g->p; r++) {
         rq.alias[r] = (g->ctx->send[r] == g->ctx->recv[r]) ? 1 : 0;
     }
-    if (rq.coll == COLL_ALLREDUCE && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
+    const bool fourRings = g->cfg.level0Rings == 4 && g->cfg.servers >= 1 && g->p % g->cfg.servers == 0 && g->p / g->cfg.servers == 8;
+    if (rq.coll == COLL_ALLREDUCE && ((g->cfg.servers > 1 && g->p % g->cfg.servers == 0) || fourRings)) {
         // two levels: mesh inside a group of ranks (uncut under the same conditions as the one-level
-        // mesh, coll_all_reduce_mesh_executor.cc:108-112), ring or halving-doubling between the groups
+        // mesh, coll_all_reduce_mesh_executor.cc:108-112) or ring(s) when the group is set up as a ring
+        // topology (coll_all_reduce_ring_executor.cc:95-135); ring or halving-doubling between the groups
         rq.servers = g->cfg.servers;
         rq.algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_RHD;   // halving-doubling unless ring is asked for (:185-191)
-        rq.meshAtomic = !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 && g->ctx->sig.op != HCCL_REDUCE_PROD;
+        rq.level0Rings = g->cfg.level0Rings == 4 ? (fourRings ? 4u : 1u) : g->cfg.level0Rings;
+        rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
+            g->ctx->sig.op != HCCL_REDUCE_PROD;
     }
     if (g->ctx->sig.variable) {
         rq.vCounts = g->ctx->vCounts;

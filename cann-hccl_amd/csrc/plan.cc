@@ -244,15 +244,26 @@ void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t
     }
 }
 
-// Two-level all-reduce of one chunk, CollAllReduceMeshExecutor::KernelRun with several servers
-// (coll_all_reduce_mesh_executor.cc:95-240): `servers` groups of D = p / servers consecutive ranks.
-//   level 0  mesh reduce-scatter inside every group over the ring slice plan for D (:102-118)
+// Device orders of the four rings of the 8-device ring topology (coll_comm_executor.cc:1595-1606).
+const uint32_t kRingOrders8[4][8] = {
+    {0, 1, 2, 6, 5, 4, 7, 3}, {0, 3, 7, 4, 5, 6, 2, 1}, {0, 2, 3, 1, 5, 7, 6, 4}, {0, 4, 6, 7, 5, 1, 3, 2}};
+
+// Two-level all-reduce of one chunk: `servers` groups of D = p / servers consecutive ranks.
+//   level 0  reduce-scatter inside every group over the ring slice plan for D:
+//            mesh (CollAllReduceMeshExecutor::KernelRun, coll_all_reduce_mesh_executor.cc:102-118), or ring
+//            (CollAllReduceRingExecutor::KernelRun, coll_all_reduce_ring_executor.cc:95-135), the latter over one
+//            ring in rank order or over the four rings of the 8-device topology: every slice is cut into one
+//            part per ring (MutliSegSlicePrepare, coll_comm_executor.cc:1681-1720) and ring k, whose i-th
+//            member is device order[k][i], runs the ring schedule on part k of its members' slices
+//            (PrepareMultiRingSlice, :1761-1833), so that every device still ends with its own slice
 //   level 1  ranks with the same position d in their groups all-reduce slice d among themselves, ring
-//            or recursive halving-doubling, from the input range to the output range (:120-196)
-//   level 0  mesh all-gather of the slices inside every group on the output (:198-236)
-// With one group the middle level is the copy of the own slice and this is the plain mesh all-reduce.
-void TwoLevelAllReduceChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, uint64_t base, uint64_t bytes, uint64_t align,
-    bool meshAtomic)
+//            or recursive halving-doubling, from the input range to the output range
+//            (coll_all_reduce_mesh_executor.cc:120-196, coll_all_reduce_ring_executor.cc:137-225)
+//   level 0  all-gather of the slices inside every group on the output, mesh or the same rings
+//            (coll_all_reduce_mesh_executor.cc:198-236, coll_all_reduce_ring_executor.cc:227-240)
+// With one group the middle level is the copy of the own slice and this is the plain one-level all-reduce.
+void TwoLevelAllReduceChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, uint32_t level0Rings, uint64_t base,
+    uint64_t bytes, uint64_t align, bool meshAtomic)
 {
     const uint32_t D = p / servers;
     std::vector<Slice> sl = RingSlicePlan(bytes, D, align);
@@ -262,13 +273,29 @@ void TwoLevelAllReduceChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t serv
     const size_t l2 = l1 + shape.phases.size();
     for (uint32_t s = 0; s < servers && D > 1; s++) {
         vp.rankMap.resize(D);
-        for (uint32_t d = 0; d < D; d++) {
-            vp.rankMap[d] = s * D + d;
+        if (level0Rings == 0) {
+            for (uint32_t d = 0; d < D; d++) {
+                vp.rankMap[d] = s * D + d;
+            }
+            vp.phaseBase = 0;
+            MeshReduceScatterPhases(vp, 0, D, base, sl, align, meshAtomic);
+            vp.phaseBase = l2;
+            MeshAllGatherPhases(vp, 0, D, base, sl);
+            continue;
         }
-        vp.phaseBase = 0;
-        MeshReduceScatterPhases(vp, 0, D, base, sl, align, meshAtomic);
-        vp.phaseBase = l2;
-        MeshAllGatherPhases(vp, 0, D, base, sl);
+        for (uint32_t k = 0; k < level0Rings; k++) {
+            std::vector<Slice> part(D);
+            for (uint32_t i = 0; i < D; i++) {
+                uint32_t dev = level0Rings > 1 ? kRingOrders8[k][i] : i;
+                vp.rankMap[i] = s * D + dev;
+                std::vector<Slice> cut = RingSlicePlan(sl[dev].size, level0Rings, align);
+                part[i] = Slice{sl[dev].off + cut[k].off, cut[k].size};
+            }
+            vp.phaseBase = 0;
+            RingReduceScatterPhases(vp, 0, D, base, part, BUF_SEND, base, part);
+            vp.phaseBase = l2;
+            RingAllGatherPhases(vp, 0, D, base, part);
+        }
     }
     for (uint32_t d = 0; d < D; d++) {
         vp.rankMap.resize(servers);
@@ -656,9 +683,9 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
     uint64_t done = 0;
     for (uint64_t cur : chunks) {
         uint64_t bytes = cur * u;
-        if (rq.coll == COLL_ALLREDUCE && rq.servers > 1) {
-            TwoLevelAllReduceChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, done, bytes, rq.align,
-                rq.meshAtomic);
+        if (rq.coll == COLL_ALLREDUCE && (rq.servers > 1 || rq.level0Rings > 0)) {
+            TwoLevelAllReduceChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, rq.level0Rings, done, bytes,
+                rq.align, rq.meshAtomic);
         } else if (rq.coll == COLL_ALLREDUCE) {
             AllReduceChunk(*vp, rq.algo, p, done, bytes, rq.align, rq.meshAtomic);
         } else if (rq.coll == COLL_REDUCESCATTER) {
@@ -1451,6 +1478,11 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
 {
     if (request.p == 0 || request.unit == 0 || request.align == 0 || request.servers == 0 || request.p % request.servers != 0) {
         *err = "bad plan request";
+        return 1;
+    }
+    if ((request.level0Rings != 0 && request.level0Rings != 1 && request.level0Rings != 4) ||
+        (request.level0Rings == 4 && request.p / request.servers != 8)) {
+        *err = "level 0 runs as a mesh, one ring, or the four rings of a group of 8 ranks";
         return 1;
     }
     PlanRequest normalised;

@@ -89,6 +89,8 @@ struct PlanRequest {
     std::vector<uint8_t> alias;    // per rank: send buffer and receive buffer are the same memory
     uint32_t servers = 1;          // all-reduce only: > 1 = two levels, `servers` groups of p / servers consecutive ranks
                                    // (mesh inside a group, `algo` ring or halving-doubling between the groups)
+    uint32_t level0Rings = 0;      // two-level all-reduce: 0 = mesh inside a group, 1 = one ring, 4 = the four rings of
+                                   // the 8-device ring topology (groups of 8 ranks only), each on a quarter of every slice
     bool meshAtomic = false;       // mesh reduce phases without the piece cut (the reference's non-deterministic variant)
     bool stageInput = false;       // copy the send buffers to scratch first (used when buffers overlap)
     // all-to-all-v only: p x p tables in elements, row r = what rank r passed

@@ -22,6 +22,9 @@ extern "C" {
  *   "align"         slice alignment in bytes (default 128)
  *   "servers"       number of rank groups for the all-reduce: with n > 1 the p ranks form n groups of p / n
  *                   consecutive ranks and the two-level schedule runs (mesh inside a group, "algo" ring or rhd between)
+ *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce: the mesh schedule
+ *                                (default), one ring in rank order, or -- for groups of 8 ranks, also with one group --
+ *                                the four rings of the 8-device ring topology, each on a quarter of every slice
  *   "step_stores"   "auto" | "nt" | "ordinary"   store kind of the step-by-step kernels (non-temporal, or write-back
  *                                so that the next phase finds the data in the memory-side cache); "auto" decides per collective
  *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
@@ -51,8 +54,8 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
  * fused items, byte counts) into out[0..cap).  coll / algo as in HcclAmdOpInfo; for the rooted
  * collectives (coll 4 broadcast, 5 reduce, 6 scatter) the algo argument carries the root rank in its low 16 bits and the
  * schedule above them (0 ring, 1 mesh, 2 rhd, 4 mesh without the piece cut); for the all-reduce (coll 0) bits 8..15 of algo
- * carry the number of rank groups of the two-level schedule (0 or 1: one level) and bit 16 asks for its mesh level
- * without the piece cut.  inPlaceMask bit r:
+ * carry the number of rank groups of the two-level schedule (0 or 1: one level), bit 16 asks for its mesh level
+ * without the piece cut and bits 17..19 give the rings inside a group (0: mesh, 1, or 4).  inPlaceMask bit r:
  * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64
  * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); for the variable-count
  * reduce-scatter / all-gather, tables points to 2*p uint64 (block counts, block displacements); else NULL.

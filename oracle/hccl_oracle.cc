@@ -15,6 +15,8 @@
 //                    TPL/temp_all_reduce/all_reduce_ring.cc:32-53,143-191
 //   mesh             TPL/temp_reduce_scatter/reduce_scatter_mesh.cc:57-203, TPL/temp_all_gather/all_gather_mesh.cc:91-253,
 //                    EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240, EXE/coll_comm_executor.cc:1458-1574,
+//                    EXE/coll_all_reduce/coll_all_reduce_ring_executor.cc:95-243 with EXE/coll_comm_executor.cc:1595-1606,
+//                    1681-1720,1761-1833 (ring or four rings inside a server),
 //                    TPL/temp_reduce_scatter/reduce_scatter_mesh_atomic.cc:82-141 (accumulation order of the racing
 //                    streams fixed to stream order: for floating point the reference itself has no single answer)
 //   halving-doubling TPL/temp_all_reduce/all_reduce_recursive_hd.cc:33-302,
@@ -41,7 +43,9 @@
 // (tests/golden).  Assumptions that only a run of the closed reference could confirm -- PARITY
 // UNPINNED for these: the slice alignment constant (128 bytes), the element sizes, the direction of
 // ForwardRank / BackwardRank (forced by all_gather_ring.cc:130-163), the piece cut of
-// PrepareSliceMeshStreams (taken equal to coll_comm_executor.cc:1681-1721), the operand order and
+// PrepareSliceMeshStreams (taken equal to coll_comm_executor.cc:1681-1721), the level-0 slice plan of the
+// two-level executors (closed AlgTemplateBase::PrepareSliceData, taken equal to the ring template's
+// all_reduce_ring.cc:119-130, as coll_all_reduce_executor.cc:330-360 does in the open), the operand order and
 // the NaN / signed-zero behaviour inside the closed Reducer, and the accumulation width for
 // fp16 / bf16 (here: fp32, rounded to nearest-even after every stored step).
 #include <algorithm>
@@ -1008,20 +1012,59 @@ int orc_allreduce(int algo, uint32_t p, void **in, void **out, uint64_t count, i
     return 0;
 }
 
-// Two-level all-reduce, CollAllReduceMeshExecutor::KernelRun with several servers
-// (EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240): `servers` groups of D = p / servers consecutive
-// ranks; mesh reduce-scatter inside every group (piece cut, or uncut when `atomic`), then the ranks with the same
-// position in their groups all-reduce their slice among themselves (level1 = ALGO_RING or ALGO_RHD) from the
-// input range to the output range, then a mesh all-gather inside every group.  Chunk loop and staging as in
+// MutliSegSlicePrepare (EXE/coll_comm_executor.cc:1681-1720): every rank slice is cut into ringCount parts of
+// RoundUp(ceil(size / ringCount), align) bytes, the last one shorter; parts that are left get size 0.
+std::vector<std::vector<Slice>> MultiSegSlices(const std::vector<Slice> &dataSegs, uint32_t ringCount, uint64_t align)
+{
+    std::vector<std::vector<Slice>> all;
+    for (const Slice &seg : dataSegs) {
+        std::vector<Slice> one;
+        uint32_t ringIndex = 0;
+        if (seg.size > 0) {
+            uint64_t per = (seg.size + ringCount - 1) / ringCount;
+            per = (per + align - 1) / align * align;
+            uint64_t residue = seg.size;
+            while (residue > 0) {
+                uint64_t sz = per < residue ? per : residue;
+                one.push_back(Slice{seg.off + seg.size - residue, sz});
+                residue -= sz;
+                ringIndex++;
+            }
+        }
+        for (; ringIndex < ringCount; ringIndex++) {
+            one.push_back(Slice{seg.off, 0});
+        }
+        all.push_back(one);
+    }
+    return all;
+}
+
+// PrepareMultiRingSlice with every device on the network list (EXE/coll_comm_executor.cc:1761-1833): ring k
+// visits the devices in order[k]; its member i works on part k of the slice of device order[k][i].
+// Ring orders of the 8-device ring topology: GetRingsOrderByTopoType, :1595-1606.
+const uint32_t kEightDeviceRings[4][8] = {
+    {0, 1, 2, 6, 5, 4, 7, 3}, {0, 3, 7, 4, 5, 6, 2, 1}, {0, 2, 3, 1, 5, 7, 6, 4}, {0, 4, 6, 7, 5, 1, 3, 2}};
+
+// Two-level all-reduce: `servers` groups of D = p / servers consecutive ranks.
+//   level0 = 0 / 1   CollAllReduceMeshExecutor::KernelRun (EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240):
+//                    mesh reduce-scatter inside every group (piece cut, or uncut when 1), mesh all-gather at the end
+//   level0 = 2 / 3   CollAllReduceRingExecutor::KernelRun (EXE/coll_all_reduce/coll_all_reduce_ring_executor.cc:95-243):
+//                    ring reduce-scatter inside every group on the input buffer and ring all-gather on the output,
+//                    over one ring in rank order (2) or the four rings of the 8-device topology (3, D = 8)
+// In between, the ranks with the same position in their groups all-reduce their slice among themselves
+// (level1 = ALGO_RING or ALGO_RHD) from the input range to the output range.  Chunk loop and staging as in
 // orc_allreduce.
-int orc_allreduce_two_level(int level1, int atomic, uint32_t servers, uint32_t p, void **in, void **out, uint64_t count, int dt,
+int orc_allreduce_two_level(int level1, int level0, uint32_t servers, uint32_t p, void **in, void **out, uint64_t count, int dt,
     int op, uint64_t cclBytes, uint64_t align, int flags, int threads)
 {
     uint64_t unit = DtSize(dt);
-    if (unit == 0 || p == 0 || servers == 0 || p % servers != 0 || cclBytes < unit || (level1 != ALGO_RING && level1 != ALGO_RHD)) {
+    if (unit == 0 || p == 0 || servers == 0 || p % servers != 0 || cclBytes < unit || (level1 != ALGO_RING && level1 != ALGO_RHD) ||
+        level0 < 0 || level0 > 3 || (level0 == 3 && p / servers != 8)) {
         return -20;
     }
     const uint32_t D = p / servers;
+    const bool atomic = level0 == 1;
+    const uint32_t ringCount = level0 == 3 ? 4u : 1u;
     Pool pool(threads);
     auto machine = [&](uint32_t n) {
         Machine m;
@@ -1056,6 +1099,31 @@ int orc_allreduce_two_level(int level1, int atomic, uint32_t servers, uint32_t p
             for (uint32_t d = 0; d < D; d++) {
                 m.buf[B_IN][d] = all.buf[B_IN][s * D + d];
                 m.buf[B_OUT][d] = all.buf[B_OUT][s * D + d];
+            }
+            if (level0 >= 2) {
+                // one sub-machine per ring: member i is device order[k][i]
+                std::vector<std::vector<Slice>> segs = MultiSegSlices(sl, ringCount, align);
+                for (uint32_t k = 0; k < ringCount; k++) {
+                    Machine ring = machine(D);
+                    std::vector<Slice> ringSl(D);
+                    for (uint32_t i = 0; i < D; i++) {
+                        uint32_t dev = ringCount > 1 ? kEightDeviceRings[k][i] : i;
+                        ring.buf[B_IN][i] = m.buf[B_IN][dev];
+                        ring.buf[B_OUT][i] = m.buf[B_OUT][dev];
+                        ringSl[i] = segs[dev][k];
+                    }
+                    for (uint32_t i = 0; i < D; i++) {
+                        Proc pr;
+                        pr.rank = i;
+                        ProgReduceScatterRing(pr.prog, i, D, B_IN, B_IN, ringSl, ringSl);
+                        ring.procs.push_back(std::move(pr));
+                    }
+                    int rc = ring.Run();
+                    if (rc != 0) {
+                        return rc;
+                    }
+                }
+                continue;
             }
             if (atomic) {
                 for (uint32_t d = 0; d < D; d++) {
@@ -1102,6 +1170,30 @@ int orc_allreduce_two_level(int level1, int atomic, uint32_t servers, uint32_t p
             for (uint32_t d = 0; d < D; d++) {
                 m.buf[B_IN][d] = all.buf[B_IN][s * D + d];
                 m.buf[B_OUT][d] = all.buf[B_OUT][s * D + d];
+            }
+            if (level0 >= 2) {
+                std::vector<std::vector<Slice>> segs = MultiSegSlices(sl, ringCount, align);
+                for (uint32_t k = 0; k < ringCount; k++) {
+                    Machine ring = machine(D);
+                    std::vector<Slice> ringSl(D);
+                    for (uint32_t i = 0; i < D; i++) {
+                        uint32_t dev = ringCount > 1 ? kEightDeviceRings[k][i] : i;
+                        ring.buf[B_IN][i] = m.buf[B_IN][dev];
+                        ring.buf[B_OUT][i] = m.buf[B_OUT][dev];
+                        ringSl[i] = segs[dev][k];
+                    }
+                    for (uint32_t i = 0; i < D; i++) {
+                        Proc pr;
+                        pr.rank = i;
+                        ProgAllGatherRing(pr.prog, i, D, B_OUT, B_OUT, ringSl, ringSl);
+                        ring.procs.push_back(std::move(pr));
+                    }
+                    int rc = ring.Run();
+                    if (rc != 0) {
+                        return rc;
+                    }
+                }
+                continue;
             }
             for (uint32_t d = 0; d < D; d++) {
                 Proc pr;

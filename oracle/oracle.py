@@ -181,11 +181,13 @@ def allreduce(ins, dt, op, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT
 
 
 def allreduce_two_level(ins, dt, op, servers, level1=RING, atomic=False, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0,
-                        threads=1):
-    """`servers` groups of consecutive ranks: mesh inside a group (piece cut, or uncut when `atomic`), `level1`
-    (RING or RHD) between the groups."""
+                        threads=1, level0="mesh"):
+    """`servers` groups of consecutive ranks; inside a group `level0`: "mesh" (piece cut, or uncut when `atomic`),
+    "ring" (one ring in rank order) or "ring4" (the four rings of the 8-device ring topology, groups of 8);
+    `level1` (RING or RHD) between the groups."""
     outs = [np.empty_like(x) for x in ins]
-    rc = lib().orc_allreduce_two_level(level1, 1 if atomic else 0, servers, len(ins), _ptrs(ins), _ptrs(outs), ins[0].size, dt, op,
+    mode = {"mesh": 1 if atomic else 0, "ring": 2, "ring4": 3}[level0]
+    rc = lib().orc_allreduce_two_level(level1, mode, servers, len(ins), _ptrs(ins), _ptrs(outs), ins[0].size, dt, op,
                                        ccl_bytes, align, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle two-level allreduce failed rc=%d" % rc)

@@ -264,6 +264,44 @@ def two_level_allreduce(dt, op, ins, unit, ccl_bytes, align, servers, level1, at
     return [out.copy() for _ in range(p)]
 
 
+EIGHT_DEVICE_RINGS = ((0, 1, 2, 6, 5, 4, 7, 3), (0, 3, 7, 4, 5, 6, 2, 1), (0, 2, 3, 1, 5, 7, 6, 4), (0, 4, 6, 7, 5, 1, 3, 2))
+
+
+def two_level_ring_allreduce(dt, op, ins, unit, ccl_bytes, align, servers, level1, rings):
+    """Groups of D = p / servers consecutive ranks with ring(s) inside: the slice of device `dev` is cut into one
+    part per ring; part k is the ring chain over the group's ranks taken in ring k's order, at the position
+    of `dev` in that order.  Then the level-1 closed form over the groups' partial results of the slice."""
+    p = len(ins)
+    D = p // servers
+    n = ins[0].size
+    orders = EIGHT_DEVICE_RINGS if rings == 4 else (tuple(range(D)),)
+    out = np.empty_like(ins[0])
+    max_per = ccl_bytes // unit
+    base = 0
+    while base < n:
+        cur = min(n - base, max_per)
+        for dev, (off, size) in enumerate(slice_plan(cur * unit, D, align)):
+            lo, hi = base + off // unit, base + (off + size) // unit
+            if hi <= lo:
+                continue
+            partial = []
+            for s in range(servers):
+                xs = [x[lo:hi] for x in ins[s * D:(s + 1) * D]]
+                if D == 1:
+                    partial.append(xs[0].copy())
+                    continue
+                acc = np.empty_like(xs[0])
+                for k, (poff, psize) in enumerate(slice_plan(size, len(orders), align)):
+                    a, b = poff // unit, (poff + psize) // unit
+                    if b > a:
+                        order = orders[k]
+                        acc[a:b] = ring_chain(dt, op, [xs[order[i]][a:b] for i in range(D)], order.index(dev))
+                partial.append(acc)
+            out[lo:hi] = level1(dt, op, partial, unit, 1 << 62, align)[0]
+        base += cur
+    return [out.copy() for _ in range(p)]
+
+
 def naive_reduce(dt, op, xs):
     acc = xs[0]
     for x in xs[1:]:

@@ -653,6 +653,31 @@ def test_two_level_allreduce(orc, level1):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("level0", ["ring", "ring4"])
+def test_two_level_allreduce_with_rings_inside_a_group(orc, level0):
+    # ring(s) inside a group: one ring in rank order, or the four rings of the 8-device topology on quarters of every slice
+    shapes = ((1, 8), (2, 8)) if level0 == "ring4" else ((2, 4), (4, 2), (3, 4))
+    for servers, D in shapes:
+        p = servers * D
+        for level1 in (RING, RHD):
+            g = gh.Group(p, algo=ALGO_NAME[level1], servers=servers, level0=level0)
+            try:
+                for dt, op, n in ((FP32, SUM, 300007), (BF16, SUM, 65536 + 5), (INT64, SUM, 10001), (FP32, MAX, 999)):
+                    ins = _ins(dt, p, n, 19 * p + n)
+                    want = orc.allreduce_two_level(ins, dt, op, servers, level1=level1, level0=level0)
+                    print("two-level", servers, "x", D, level0, "level1", level1, "type", dt, flush=True)
+                    for fuse in (1, 0):
+                        g.set(fuse=fuse)
+                        for in_place in (False, True):
+                            outs, _ = gh.all_reduce(g, ins, dt, op, in_place=in_place)
+                            assert g.info()["fused"] == fuse
+                            for r in range(p):
+                                assert gh.same(dt, outs[r], want[r]), (servers, D, level0, level1, dt, fuse, in_place, r)
+            finally:
+                g.close()
+
+
+@pytest.mark.gpu
 def test_two_level_allreduce_operand_order_of_max_min(orc):
     # NaN payloads and signed zeros show which operand stood left in every combine of the fused form
     specials = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.0, -1.0, 3.4e38], np.float32)

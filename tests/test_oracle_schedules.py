@@ -341,3 +341,40 @@ def test_two_level_allreduce_matches_closed_form(orc, level1, atomic):
     a = orc.allreduce_two_level(ins, FP32, SUM, 1, level1=level1, atomic=atomic)
     b = orc.allreduce(ins, FP32, SUM, algo=MESH_ATOMIC if atomic else MESH)
     assert all(np.array_equal(x, y) for x, y in zip(a, b))
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("level0", ["ring", "ring4"])
+def test_two_level_allreduce_with_rings_inside_a_server_matches_closed_form(orc, level1, level0):
+    # ring(s) inside a server (one ring in rank order, or the four rings of the 8-device topology, each on its
+    # part of every slice), ring or halving-doubling between servers
+    closed1 = cf.ring_allreduce if level1 == RING else cf.rhd_allreduce
+    shapes = ((1, 8), (2, 8), (3, 8)) if level0 == "ring4" else ((2, 4), (4, 2), (3, 4), (1, 8), (5, 3), (8, 1))
+    rings = 4 if level0 == "ring4" else 1
+    for servers, D in shapes:
+        p = servers * D
+        for dt, op, n, ccl in ((FP32, SUM, 2003, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, SUM, 1501, 200 << 20),
+                               (INT32, MAX, 700, 200 << 20), (FP32, SUM, 100, 200 << 20)):
+            ins = _inputs(dt, p, n, 37 * p + n)
+            got = orc.allreduce_two_level(ins, dt, op, servers, level1=level1, level0=level0, ccl_bytes=ccl)
+            want = cf.two_level_ring_allreduce(dt, op, ins, orc.dtype_size(dt), ccl, 128, servers, closed1, rings)
+            for r in range(p):
+                assert _eq(dt, got[r], want[r]), (servers, D, level1, level0, dt, ccl, r)
+    # one server with one ring is the plain ring all-reduce
+    ins = _inputs(FP32, 8, 4099, 5)
+    a = orc.allreduce_two_level(ins, FP32, SUM, 1, level1=level1, level0="ring")
+    b = orc.allreduce(ins, FP32, SUM, algo=RING)
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+    # four rings: a different association than one ring, visible in fp32 sums of generic data
+    if level0 == "ring4":
+        c = orc.allreduce_two_level(ins, FP32, SUM, 1, level1=level1, level0="ring4")
+        assert not all(np.array_equal(x, y) for x, y in zip(b, c))
+        # every rank holds the same result whatever ring a part went through
+        assert all(np.array_equal(c[0], x) for x in c)
+
+
+def test_multi_ring_parts_of_a_slice():
+    # the cut of one rank slice into one part per ring: RoundUp(ceil(size / rings), 128) each, the last shorter,
+    # left-over rings empty (hand-computed: 1000 B over 4 rings -> 256, 256, 256, 232; 300 B -> 128, 128, 44, 0)
+    assert [s for _, s in cf.slice_plan(1000, 4, 128)] == [256, 256, 256, 232]
+    assert [s for _, s in cf.slice_plan(300, 4, 128)] == [128, 128, 44, 0]

@@ -375,3 +375,29 @@ def test_two_level_fused_stack_form_keeps_operand_order(orc, level1):
             plan_interp.run_fused(plan, sends, recvs, FP32, op)
             for r in range(p):
                 assert np.array_equal(recvs[r].view(np.uint32), want[r].view(np.uint32)), (servers, D, level1, op, r)
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("level0", ["ring", "ring4"])
+def test_two_level_allreduce_with_rings_inside_a_group_matches_checker(orc, level1, level0):
+    rings = 4 if level0 == "ring4" else 1
+    shapes = ((1, 8), (2, 8), (3, 8)) if rings == 4 else ((2, 4), (4, 2), (3, 4), (5, 3))
+    for servers, D in shapes:
+        p = servers * D
+        for dt, op, n, ccl in ((FP32, SUM, 2003, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, PROD, 777, 200 << 20), (FP32, SUM, 60, 200 << 20)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n, 500 + p + n)
+            want = orc.allreduce_two_level(ins, dt, op, servers, level1=level1, level0=level0, ccl_bytes=ccl)
+            for mask in (0, (1 << p) - 1):
+                plan = H.describe_plan(H.COLL_ALLREDUCE, level1 | (servers << 8) | (rings << 17), p, n, dt, ccl_bytes=ccl,
+                                       in_place_mask=mask)
+                assert plan["scratchBytes"] == 0 and plan["fusedOk"]
+                for fused in (False, True):
+                    sends = _bytes(ins)
+                    recvs = _bytes(ins) if mask else [np.full(n * unit, 0xA5, np.uint8) for _ in range(p)]
+                    (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op, in_place=bool(mask))
+                    for r in range(p):
+                        assert _same(dt, recvs[r], want[r]), (servers, D, level1, level0, dt, ccl, mask, fused, r)
+    # groups of another size have no four-ring form
+    with pytest.raises(Exception):
+        H.describe_plan(H.COLL_ALLREDUCE, level1 | (2 << 8) | (4 << 17), 8, 1000, FP32)
