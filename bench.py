@@ -2,7 +2,9 @@
 
 Default workload: ring all-reduce, sum, fp32, 8 simulated ranks x 256 MiB per rank, out of place
 (BASELINE.json configs[1] at its largest size).  A "step" is one complete collective (one call per
-rank).  Prints one JSON line; see DESIGN.md for the byte accounting.
+rank).  Prints one JSON line.  Byte accounting: the fused mode reads every rank's input once and writes
+every rank's output once (2 * p * S bytes per collective); the step-by-step mode moves what the ring
+schedule moves, 5 * (p - 1) * S (3 * S per reduce-scatter phase, 2 * S per all-gather phase).
 
     python bench.py [--steps K] [--warmup W] [--size-mib M] [--sweep] [--no-cpu]
 """
