@@ -1390,6 +1390,14 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         } else {
             return HCCL_E_PARA;
         }
+    } else if (k == "fused_stores") {
+        if (v == "nt") {
+            cfg.fusedStores = 0;
+        } else if (v == "ordinary") {
+            cfg.fusedStores = 1;
+        } else {
+            return HCCL_E_PARA;
+        }
     } else if (k == "step_stores") {
         if (v == "auto") {
             cfg.stepStores = -1;

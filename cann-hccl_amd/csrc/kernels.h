@@ -49,8 +49,11 @@ struct FusedDesc {
     uint32_t srcBase;   // index into the source pointer pool
     uint32_t dstBase;   // index into the destination pointer pool
     uint32_t nleaf;
-    uint32_t pad;
+    uint32_t flags;     // kFusedOrdinaryStores
 };
+
+// flags of a fused item
+constexpr uint32_t kFusedOrdinaryStores = 1u;  // whole passes of the chain kernel store write-back instead of non-temporal
 
 // flags of the step kernel
 constexpr uint32_t kStepOrdinaryStores = 1u;   // write-back stores instead of non-temporal ones in the fast loop

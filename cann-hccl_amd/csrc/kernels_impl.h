@@ -482,10 +482,14 @@ template <int OP> struct OrderMatters<double, OP> { static constexpr bool value 
 template <int OP> struct OrderMatters<HalfBits, OP> { static constexpr bool value = (OP == ROP_MAX || OP == ROP_MIN); };
 template <int OP> struct OrderMatters<Bf16Bits, OP> { static constexpr bool value = (OP == ROP_MAX || OP == ROP_MIN); };
 
-template <uint32_t MODE> __device__ __forceinline__ void StoreAny16(void *base, uint64_t pos, V4 v)
+template <uint32_t MODE, bool ORDINARY = false> __device__ __forceinline__ void StoreAny16(void *base, uint64_t pos, V4 v)
 {
     if (MODE == ACC_VEC16) {
-        Store16(base, pos, v);
+        if (ORDINARY) {
+            *(GlobalV4 *)(static_cast<char *>(base) + pos) = v;
+        } else {
+            Store16(base, pos, v);
+        }
     } else {
         V4A4 t = {v.x, v.y, v.z, v.w};
         *(GlobalV4A4 *)(static_cast<char *>(base) + pos) = t;
@@ -494,7 +498,7 @@ template <uint32_t MODE> __device__ __forceinline__ void StoreAny16(void *base, 
 
 // One pass over kChainVec * 256 vectors starting at vector vecBase of the tile.
 // FULL: every lane has all its vectors inside the tile (no per-lane guards).
-template <typename T, int OP, uint32_t MODE, bool FULL>
+template <typename T, int OP, uint32_t MODE, bool FULL, bool ORDINARY = false>
 __device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *const *__restrict__ src,
     void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec)
 {
@@ -549,7 +553,7 @@ __device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *con
 #pragma unroll
         for (uint32_t u = 0; u < kChainVec; u++) {
             if (live[u]) {
-                StoreAny16<MODE>(o, pos[u], acc[u]);
+                StoreAny16<MODE, ORDINARY>(o, pos[u], acc[u]);
             }
         }
     }
@@ -591,8 +595,16 @@ __global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__
             constexpr uint32_t kPass = kChainVec * kBlockThreads;
             uint32_t base = 0;
             if (d.mode == ACC_VEC16) {
-                for (; base + kPass <= nvec; base += kPass) {
-                    ChainVecPass<T, OP, ACC_VEC16, true>(d, src, dst, off, base, nvec);
+                // the store kind is a compile-time property of the pass (a per-store choice at run time
+                // is merged by the compiler into one plain store)
+                if (d.flags & kFusedOrdinaryStores) {
+                    for (; base + kPass <= nvec; base += kPass) {
+                        ChainVecPass<T, OP, ACC_VEC16, true, true>(d, src, dst, off, base, nvec);
+                    }
+                } else {
+                    for (; base + kPass <= nvec; base += kPass) {
+                        ChainVecPass<T, OP, ACC_VEC16, true, false>(d, src, dst, off, base, nvec);
+                    }
                 }
                 if (base < nvec) {
                     ChainVecPass<T, OP, ACC_VEC16, false>(d, src, dst, off, base, nvec);

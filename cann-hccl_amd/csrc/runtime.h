@@ -38,6 +38,7 @@ struct GroupConfig {
     uint32_t servers = 1;            // all-reduce: > 1 = two-level schedule over `servers` groups of consecutive ranks
     uint32_t level0Rings = 0;        // two-level all-reduce inside a group: 0 = mesh, 1 = one ring, 4 = four rings (groups of 8)
     int stepStores = -1;             // step kernel stores: -1 chosen per launch, 0 non-temporal, 1 ordinary
+    int fusedStores = 0;             // fused chain kernel stores: 0 non-temporal, 1 ordinary
     uint32_t blocksPerCu = 0;             // workgroups per CU; 0 = per-kernel default
     bool blockingArrive = false;          // ranks wait inside the call until the collective is issued
     uint32_t arriveTimeoutMs = 1800 * 1000;

@@ -732,6 +732,22 @@ def test_allreduce_on_a_rank_table_communicator(orc, tmp_path):
         H.comm_destroy(comms)
 
 
+def test_fused_write_back_stores_give_the_same_bits(orc):
+    p = 8
+    g = _group(p, RING, fuse=1, fused_stores="ordinary")
+    try:
+        for dt, op, n in ((FP32, SUM, 1 << 20), (BF16, MAX, 300001), (INT8, SUM, 70001)):
+            ins = _ins(dt, p, n, 23 + n)
+            want = orc.allreduce(ins, dt, op, algo=RING)
+            outs, _ = gh.all_reduce(g, ins, dt, op)
+            assert g.info()["fused"] == 1
+            for r in range(p):
+                assert gh.same(dt, outs[r], want[r]), (dt, op, r)
+    finally:
+        g.close()
+
+
+@pytest.mark.gpu
 def test_many_shapes_evict_cached_collectives_without_leaking(orc):
     # more distinct shapes than the library keeps prepared (64): old entries are dropped, results stay right and
     # device memory returns to where it was
