@@ -826,6 +826,46 @@ def test_one_thread_per_rank_blocking_arrival(orc):
         g.close()
 
 
+def test_two_groups_on_two_host_threads(orc):
+    # independent communicator groups driven from different host threads on their own streams share nothing
+    # but the library's global tables
+    import threading
+    p = 4
+    errors = []
+
+    def drive(seed, algo):
+        try:
+            rng = np.random.default_rng(seed)
+            g = gh.Group(p, algo=ALGO_NAME[algo])
+            try:
+                base = [rng.integers(-50, 50, 120000).astype(np.int32) for _ in range(p)]
+                sends = [gh.to_dev(x) for x in base]
+                recvs = [gh.empty_dev(120000 * 4) for _ in range(p)]
+                g.stream.synchronize()
+                for k in range(40):
+                    n = int(rng.integers(1, 120000))
+                    g.set(fuse=k % 2)
+                    H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, INT32, SUM, g.stream_ptr)
+                    g.stream.synchronize()
+                    want = np.sum([x[:n] for x in base], axis=0, dtype=np.int64).astype(np.int32)
+                    for r in range(p):
+                        if not np.array_equal(gh.to_host(recvs[r], INT32)[:n], want):
+                            errors.append((seed, k, n, r))
+                            return
+            finally:
+                g.close()
+        except Exception as e:   # noqa: BLE001 - reported by the assertion below
+            errors.append((seed, repr(e)))
+
+    ts = [threading.Thread(target=drive, args=(s, a)) for s, a in ((1, RING), (2, MESH), (3, RHD))]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join(100)
+    assert not errors, errors
+    assert not any(t.is_alive() for t in ts)
+
+
 def test_send_recv_and_batch():
     p, n = 4, 250007
     g = gh.Group(p)
