@@ -67,3 +67,45 @@ def test_ring_allreduce_256mib_per_rank():
             assert torch.equal(ar_out[r], ag_out[r]), r
     finally:
         g.close()
+
+
+@pytest.mark.parametrize("p", [32, 24])
+def test_rhd_allreduce_bf16_128mib_per_rank(p):
+    """Recursive halving-doubling all-reduce, bf16 sum, 128 MiB per rank, 32 ranks (power of two) and 24 ranks
+    (block of 16 plus 8 folded pairs): the fused tree kernel and the step-by-step schedule against the
+    checker at full size, bit for bit (fp32 accumulation, one rounding per stored step in all three)."""
+    from closed_forms import BF16
+    from oracle import oracle as orc
+    orc.build()
+    n = 64 << 20                                     # bf16 elements per rank
+    rng = np.random.default_rng(99 + p)
+    # bf16 bit patterns with exponents around 1.0 (no Inf / NaN), every rank a different rotation of one block
+    base = (rng.integers(0, 2, n, dtype=np.uint16) << 15) | (rng.integers(118, 132, n, dtype=np.uint16) << 7) | \
+        rng.integers(0, 128, n, dtype=np.uint16)
+    ins = [np.roll(base, 1237 * r + 1) ^ np.uint16(r & 0x7f) for r in range(p)]
+    sends = [torch.from_numpy(x.view(np.int16)).cuda() for x in ins]
+    torch.cuda.synchronize()
+    results = {}
+    for fuse in (1, 0):
+        g = gh.Group(p, algo="rhd", fuse=fuse)
+        try:
+            recvs = [torch.empty(n, dtype=torch.int16, device="cuda") for _ in range(p)]
+            torch.cuda.synchronize()
+            print("full size rhd all-reduce p", p, "fuse", fuse, flush=True)
+            H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, BF16, SUM, g.stream_ptr)
+            g.stream.synchronize()
+            assert g.info()["fused"] == fuse
+            for r in range(1, p):
+                assert torch.equal(recvs[0], recvs[r]), (fuse, r)      # every rank holds the same bits
+            results[fuse] = recvs[0].cpu().numpy().view(np.uint16)
+            del recvs
+        finally:
+            g.close()
+    assert torch.equal(sends[p - 1], torch.from_numpy(ins[p - 1].view(np.int16)).cuda())   # inputs untouched
+    assert np.array_equal(results[1], results[0])                      # fused and step-by-step agree bit for bit
+    del sends
+    print("checker at full size", flush=True)
+    outs = [np.empty(n, np.uint16) for _ in range(p)]
+    orc.allreduce(ins, BF16, SUM, algo=orc.RHD, flags=orc.DIRECT | orc.ZERO_STAGING, threads=16, outs=outs)   # clobbers ins
+    assert np.array_equal(results[1], outs[0])
+    assert np.array_equal(outs[0], outs[p - 1])
