@@ -402,8 +402,10 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "ring all-reduce sum fp32, %d simulated ranks x %.0f MiB per rank, out of place, one GPU "
-                        "(BASELINE.json configs[1] at its largest size)" % (p, args.size_mib),
+            "workload": "%s all-reduce sum fp32, %d simulated ranks x %.0f MiB per rank, out of place, one GPU%s"
+                        % ({0: "ring", 1: "mesh", 2: "halving-doubling", 4: "mesh"}.get(info["algo"], "?"), p, args.size_mib,
+                           " (BASELINE.json configs[1] at its largest size)" if (p == 8 and args.size_mib == 256.0 and info["algo"] == 0)
+                           else ""),
             "issue": "fused single-pass kernel, HIP graph replay" if info["fused"] else "step-by-step",
             "launches_per_step": info["launches"],
             "bytes_per_step_actual": actual,
@@ -424,7 +426,9 @@ def main():
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES if (p == 8 and args.size_mib == 256.0 and not args.set) else None,
-            "kernel": "ChainKernel<float, sum> (fused ring all-reduce), avg launch %.4f ms over %d launches" % (dev_ms, args.steps),
+            "kernel": "%s<float, sum> (fused %s all-reduce), avg launch %.4f ms over %d launches"
+                      % ("TreeKernel" if info["algo"] == 2 else "ChainKernel", {0: "ring", 1: "mesh", 2: "halving-doubling", 4: "mesh"}
+                         .get(info["algo"], "?"), dev_ms, args.steps),
         },
         # the literal schedule (14 phases of copy / reduce steps replayed from a HIP graph), same workload
         "roofline_step_by_step": {
