@@ -546,6 +546,14 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
             g->ctx->sig.op != HCCL_REDUCE_PROD;
     }
+    if (rq.coll == COLL_REDUCESCATTER && !g->ctx->sig.variable && g->cfg.servers > 1 && g->p % g->cfg.servers == 0 &&
+        g->cfg.level0Rings == 0) {
+        // two levels (coll_reduce_scatter_mesh_executor.cc:128-247): ring or halving-doubling between the
+        // groups first, then the mesh inside a group, uncut under the conditions of :216-218
+        rq.servers = g->cfg.servers;
+        rq.algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_RHD;
+        rq.meshAtomic = !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 && g->ctx->sig.op != HCCL_REDUCE_PROD;
+    }
     if (g->ctx->sig.variable) {
         rq.vCounts = g->ctx->vCounts;
         rq.vDispls = g->ctx->vDispls;

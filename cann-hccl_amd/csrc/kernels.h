@@ -38,7 +38,7 @@ struct StepDesc {
 //   stack : any other expression.  Sources in evaluation order; after pushing src[j] the two topmost
 //           values are folded ops[j] & 7 times, bit 8 + i of ops[j] set = the lower value is the left
 //           operand of fold i.  The launch's op words (one uint32 per source-pool entry, same index)
-//           follow its item table in memory.
+//           follow its item table in memory; nleaf holds the stack depth the program needs.
 struct FusedDesc {
     uint64_t bytes;
     uint64_t accLeftMask;

@@ -849,65 +849,87 @@ __global__ void __launch_bounds__(kBlockThreads) TreeKernel(const FusedDesc *__r
 // the left operand in fold i.  The op words of a launch follow its item table in memory.
 // The stack lives in registers: its depth is a wave-uniform number, so every access goes through a
 // switch with constant indices.  Sources are loaded in batches like the chain kernel's.
-constexpr uint32_t kStackVec = 2;        // vectors per lane per pass
+// Two shapes: expressions that need at most 4 values (a chain of chains, a 4-leaf tree of chains) run
+// with 4 vectors per lane like the chain kernel, deeper ones (up to 8 values) with 2.
+constexpr uint32_t kStackVecShallow = 4;
+constexpr uint32_t kStackVecDeep = 2;
+constexpr uint32_t kStackShallowDepth = 4;
 constexpr uint32_t kStackSrcBatch = 8;
 
-struct StackVal {
-    V4 x[kStackVec];
+template <uint32_t U> struct StackVal {
+    V4 x[U];
 };
 
-// The values below the top one are seven separate variables, not an array or a struct: a switch over
+// The values below the top one are separate variables, not an array or a struct: a switch over
 // parts of one object is merged by the compiler into a single access at a computed offset, which
-// moves the object to private memory.
-#define HCCL_STACK_PUT(i, v)          \
-    switch (i) {                      \
-        case 0: b0 = (v); break;      \
-        case 1: b1 = (v); break;      \
-        case 2: b2 = (v); break;      \
-        case 3: b3 = (v); break;      \
-        case 4: b4 = (v); break;      \
-        case 5: b5 = (v); break;      \
-        default: b6 = (v); break;     \
+// moves the object to private memory.  DEEP is a compile-time constant of the enclosing function;
+// without it only b0..b2 are ever touched and the others cost no registers.
+#define HCCL_STACK_PUT(i, v)              \
+    if (DEEP) {                           \
+        switch (i) {                      \
+            case 0: b0 = (v); break;      \
+            case 1: b1 = (v); break;      \
+            case 2: b2 = (v); break;      \
+            case 3: b3 = (v); break;      \
+            case 4: b4 = (v); break;      \
+            case 5: b5 = (v); break;      \
+            default: b6 = (v); break;     \
+        }                                 \
+    } else {                              \
+        switch (i) {                      \
+            case 0: b0 = (v); break;      \
+            case 1: b1 = (v); break;      \
+            default: b2 = (v); break;     \
+        }                                 \
     }
-#define HCCL_STACK_GET(i, v)          \
-    switch (i) {                      \
-        case 0: (v) = b0; break;      \
-        case 1: (v) = b1; break;      \
-        case 2: (v) = b2; break;      \
-        case 3: (v) = b3; break;      \
-        case 4: (v) = b4; break;      \
-        case 5: (v) = b5; break;      \
-        default: (v) = b6; break;     \
+#define HCCL_STACK_GET(i, v)              \
+    if (DEEP) {                           \
+        switch (i) {                      \
+            case 0: (v) = b0; break;      \
+            case 1: (v) = b1; break;      \
+            case 2: (v) = b2; break;      \
+            case 3: (v) = b3; break;      \
+            case 4: (v) = b4; break;      \
+            case 5: (v) = b5; break;      \
+            default: (v) = b6; break;     \
+        }                                 \
+    } else {                              \
+        switch (i) {                      \
+            case 0: (v) = b0; break;      \
+            case 1: (v) = b1; break;      \
+            default: (v) = b2; break;     \
+        }                                 \
     }
 
-template <typename T, int OP, uint32_t MODE, bool FULL>
+template <typename T, int OP, uint32_t MODE, bool FULL, bool DEEP>
 __device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *const *__restrict__ src,
     const uint32_t *__restrict__ ops, void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec)
 {
-    uint64_t pos[kStackVec];
-    bool live[kStackVec];
+    constexpr uint32_t U = DEEP ? kStackVecDeep : kStackVecShallow;
+    uint64_t pos[U];
+    bool live[U];
 #pragma unroll
-    for (uint32_t u = 0; u < kStackVec; u++) {
+    for (uint32_t u = 0; u < U; u++) {
         uint32_t i = vecBase + u * kBlockThreads + threadIdx.x;
         live[u] = FULL || i < nvec;
         pos[u] = off + uint64_t(i) * 16;
     }
-    StackVal top;
+    StackVal<U> top;
 #pragma unroll
-    for (uint32_t u = 0; u < kStackVec; u++) {
+    for (uint32_t u = 0; u < U; u++) {
         top.x[u] = V4{0, 0, 0, 0};
     }
-    StackVal b0 = top, b1 = top, b2 = top, b3 = top, b4 = top, b5 = top, b6 = top;
+    StackVal<U> b0 = top, b1 = top, b2 = top, b3 = top, b4 = top, b5 = top, b6 = top;
     uint32_t depth = 0;                  // values on the stack, the top one included
     const uint32_t nsrc = d.nsrc;
     for (uint32_t j = 0; j < nsrc; j += kStackSrcBatch) {
-        StackVal v[kStackSrcBatch];
+        StackVal<U> v[kStackSrcBatch];
 #pragma unroll
         for (uint32_t jj = 0; jj < kStackSrcBatch; jj++) {
             if (j + jj < nsrc) {
                 const void *s = src[j + jj];
 #pragma unroll
-                for (uint32_t u = 0; u < kStackVec; u++) {
+                for (uint32_t u = 0; u < U; u++) {
                     if (live[u]) {
                         v[jj].x[u] = Load16<MODE>(s, pos[u]);
                     }
@@ -926,11 +948,11 @@ __device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *con
                 const uint32_t nfold = op & 7u;
 #pragma nounroll
                 for (uint32_t f = 0; f < nfold && depth >= 2; f++) {
-                    StackVal under;
+                    StackVal<U> under;
                     HCCL_STACK_GET(depth - 2, under)
                     const bool underLeft = !OrderMatters<T, OP>::value || ((op >> (8 + f)) & 1u);
 #pragma unroll
-                    for (uint32_t u = 0; u < kStackVec; u++) {
+                    for (uint32_t u = 0; u < U; u++) {
                         if (live[u]) {
                             top.x[u] = underLeft ? Combine16<T, OP>(under.x[u], top.x[u]) : Combine16<T, OP>(top.x[u], under.x[u]);
                         }
@@ -944,7 +966,7 @@ __device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *con
     for (uint32_t k = 0; k < ndst; k++) {
         void *o = dst[k];
 #pragma unroll
-        for (uint32_t u = 0; u < kStackVec; u++) {
+        for (uint32_t u = 0; u < U; u++) {
             if (live[u]) {
                 StoreAny16<MODE>(o, pos[u], top.x[u]);
             }
@@ -960,6 +982,7 @@ __device__ __forceinline__ void StackElem(const FusedDesc &d, const void *const 
     const uint32_t cnt = n / sizeof(T);
     for (uint32_t e = threadIdx.x; e < cnt; e += kBlockThreads) {
         const uint64_t at = off + uint64_t(e) * sizeof(T);
+        constexpr bool DEEP = true;
         T top = T();
         T b0 = top, b1 = top, b2 = top, b3 = top, b4 = top, b5 = top, b6 = top;
         uint32_t depth = 0;
@@ -1001,18 +1024,24 @@ __global__ void __launch_bounds__(kBlockThreads) StackKernel(const FusedDesc *__
             StackElem<T, OP>(d, src, ops, dst, off, n);
         } else {
             const uint32_t nvec = n >> 4;
-            constexpr uint32_t kPass = kStackVec * kBlockThreads;
+            constexpr uint32_t kPassShallow = kStackVecShallow * kBlockThreads, kPassDeep = kStackVecDeep * kBlockThreads;
             uint32_t base = 0;
             if (d.mode == ACC_VEC16) {
-                for (; base + kPass <= nvec; base += kPass) {
-                    StackVecPass<T, OP, ACC_VEC16, true>(d, src, ops, dst, off, base, nvec);
+                // d.nleaf: the stack depth the item needs
+                if (d.nleaf <= kStackShallowDepth) {
+                    for (; base + kPassShallow <= nvec; base += kPassShallow) {
+                        StackVecPass<T, OP, ACC_VEC16, true, false>(d, src, ops, dst, off, base, nvec);
+                    }
+                }
+                for (; base + kPassDeep <= nvec; base += kPassDeep) {
+                    StackVecPass<T, OP, ACC_VEC16, true, true>(d, src, ops, dst, off, base, nvec);
                 }
                 if (base < nvec) {
-                    StackVecPass<T, OP, ACC_VEC16, false>(d, src, ops, dst, off, base, nvec);
+                    StackVecPass<T, OP, ACC_VEC16, false, true>(d, src, ops, dst, off, base, nvec);
                 }
             } else {
-                for (; base < nvec; base += kPass) {
-                    StackVecPass<T, OP, ACC_VEC16_SRC4, false>(d, src, ops, dst, off, base, nvec);
+                for (; base < nvec; base += kPassDeep) {
+                    StackVecPass<T, OP, ACC_VEC16_SRC4, false, true>(d, src, ops, dst, off, base, nvec);
                 }
             }
         }

@@ -343,8 +343,9 @@ HdShape MakeHdShape(uint32_t p)
 }
 
 // Standalone recursive halving-doubling reduce-scatter (reduce_scatter_recursive_hd.cc:33-254) over
-// user slices in[i]; every rank ends with its reduced slice in (BUF_RECV, outOff).
-void RhdReduceScatterChunk(VProgram &vp, uint32_t p, const std::vector<Slice> &in, uint64_t outOff)
+// user slices in[i], in place: every rank ends with its reduced slice where the slice lies in its
+// input buffer.  Returns the phase after the last one used.
+size_t RhdReduceScatterInPlace(VProgram &vp, uint32_t p, const std::vector<Slice> &in)
 {
     HdShape h = MakeHdShape(p);
     size_t ph = 0;
@@ -376,8 +377,62 @@ void RhdReduceScatterChunk(VProgram &vp, uint32_t p, const std::vector<Slice> &i
         }
         ph++;
     }
+    return ph;
+}
+
+// The same with the result copied to (BUF_RECV, outOff).
+void RhdReduceScatterChunk(VProgram &vp, uint32_t p, const std::vector<Slice> &in, uint64_t outOff)
+{
+    size_t ph = RhdReduceScatterInPlace(vp, p, in);
     for (uint32_t r = 0; r < p; r++) {
         EmitCopy(vp, ph, MkRef(r, BUF_RECV, outOff), MkRef(r, BUF_SEND, in[r].off), in[r].size);
+    }
+}
+
+// Two-level reduce-scatter of one chunk, CollReduceScatterMeshExecutor::KernelRun with several servers
+// (coll_reduce_scatter_mesh_executor.cc:128-247): `servers` groups of D = p / servers consecutive ranks;
+// block i of the input (the part for rank i) lies at blockOff[i].
+//   level 1  ranks with the same position in their groups reduce-scatter the whole input among
+//            themselves, ring or recursive halving-doubling, in place: the slice of group s is the D
+//            blocks for the ranks of group s (:141-196)
+//   level 0  mesh reduce-scatter inside every group over those D blocks, in place (:198-238)
+//   then the rank's own block goes to the output (:240-243)
+void TwoLevelReduceScatterChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, const std::vector<uint64_t> &blockOff,
+    uint64_t bytes, uint64_t outOff, uint64_t align, bool meshAtomic)
+{
+    const uint32_t D = p / servers;
+    size_t l1 = 0;
+    for (uint32_t d = 0; d < D && servers > 1; d++) {
+        vp.rankMap.resize(servers);
+        for (uint32_t s = 0; s < servers; s++) {
+            vp.rankMap[s] = s * D + d;
+        }
+        vp.phaseBase = 0;
+        // a group's slice is D separate blocks in the caller's layout: one pass of the schedule per block
+        for (uint32_t k = 0; k < D; k++) {
+            std::vector<Slice> in(servers);
+            for (uint32_t s = 0; s < servers; s++) {
+                in[s] = Slice{blockOff[s * D + k], bytes};
+            }
+            l1 = level1 == ALGO_RING ? RingReduceScatterPhases(vp, 0, servers, 0, in, BUF_SEND, 0, in)
+                                     : RhdReduceScatterInPlace(vp, servers, in);
+        }
+    }
+    size_t l0 = l1;
+    for (uint32_t s = 0; s < servers && D > 1; s++) {
+        vp.rankMap.resize(D);
+        std::vector<Slice> sl(D);
+        for (uint32_t d = 0; d < D; d++) {
+            vp.rankMap[d] = s * D + d;
+            sl[d] = Slice{blockOff[s * D + d], bytes};
+        }
+        vp.phaseBase = l1;
+        l0 = l1 + MeshReduceScatterPhases(vp, 0, D, 0, sl, align, meshAtomic);
+    }
+    vp.rankMap.clear();
+    vp.phaseBase = 0;
+    for (uint32_t r = 0; r < p; r++) {
+        EmitCopy(vp, l0, MkRef(r, BUF_RECV, outOff), MkRef(r, BUF_SEND, blockOff[r]), bytes);
     }
 }
 
@@ -674,7 +729,10 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
         }
         return 0;
     }
-    std::vector<uint64_t> chunks = ChunkCounts(rq.coll, rq.count, rq.unit, p, rq.cclBytes, rq.align);
+    // the two-level reduce-scatter sizes its chunks without rounding to the slice alignment
+    // (CollReduceScatterMeshExecutor::CalcLoopMaxCount, coll_reduce_scatter_mesh_executor.cc:114-119)
+    const bool twoLevelScatter = rq.coll == COLL_REDUCESCATTER && rq.servers > 1;
+    std::vector<uint64_t> chunks = ChunkCounts(rq.coll, rq.count, rq.unit, p, rq.cclBytes, twoLevelScatter ? 1 : rq.align);
     if (rq.count > 0 && chunks.empty()) {
         *err = "CCL buffer too small for one element per rank";
         return 1;
@@ -697,6 +755,13 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             }
             if (p == 1) {
                 EmitCopy(*vp, 0, MkRef(0, BUF_RECV, done), MkRef(0, BUF_SEND, done), bytes);
+            } else if (rq.servers > 1) {
+                std::vector<uint64_t> blockOff(p);
+                for (uint32_t i = 0; i < p; i++) {
+                    blockOff[i] = in[i].off;
+                }
+                TwoLevelReduceScatterChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, blockOff, bytes, done,
+                    rq.align, rq.meshAtomic);
             } else if (rq.algo == ALGO_RING) {
                 RingReduceScatterPhases(*vp, 0, p, 0, in, BUF_RECV, 0, out);
             } else if (rq.algo == ALGO_RHD) {
@@ -1308,6 +1373,7 @@ bool AsStack(const Sym &sym, int e, uint64_t delta, FusedItem *item)
         return false;
     }
     item->kind = FK_STACK;
+    item->nleaf = f.need[e];          // stack depth the program needs
     item->src.clear();
     item->srcValid.clear();
     item->ops.clear();

@@ -72,7 +72,7 @@ struct FusedItem {
     std::vector<uint8_t> srcValid;   // FK_TREE: second source of a leaf may be absent
     std::vector<uint8_t> accLeft;    // FK_CHAIN: one flag per src (index 0 unused)
     std::vector<uint16_t> ops;       // FK_STACK: one word per src
-    uint32_t nleaf = 0;
+    uint32_t nleaf = 0;              // FK_TREE: leaves; FK_STACK: stack depth the program needs
     std::vector<Ref> dst;
 };
 

@@ -1216,6 +1216,35 @@ int orc_allreduce_two_level(int level1, int level0, uint32_t servers, uint32_t p
 }
 
 
+// ReduceScatterRecursiveHalvingDoubling::RunAsync, reduce_scatter_recursive_hd.cc:33-254, on the machine's
+// input buffers (m.p slices of `bytes` bytes each), in place.
+void AddReduceScatterRhdProcs(Machine &m, uint64_t bytes)
+{
+    const uint32_t p = static_cast<uint32_t>(m.p);
+    uint32_t block, part1;
+    std::vector<uint32_t> rankOf;
+    std::vector<Slice> bsl;
+    RhdBlockLayout(p, bytes, &block, &part1, &rankOf, &bsl);
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        if (r < part1 && (r % 2) == 1) {
+            pr.prog.push_back(MkSend(static_cast<int>(r - 1), 1, B_IN, 0, bytes * p));
+            pr.prog.push_back(MkRecvCopy(static_cast<int>(r - 1), 1, B_IN, bytes * r, bytes));
+        } else {
+            if (r < part1) {
+                pr.prog.push_back(MkRecvReduce(static_cast<int>(r + 1), 1, B_IN, 0, B_IN, 0, bytes * p));
+            }
+            uint32_t q = (r < part1) ? r / 2 : r - part1 / 2;
+            ProgReduceScatterHd(pr.prog, q, block, rankOf, B_IN, B_IN, bsl);
+            if (r < part1) {
+                pr.prog.push_back(MkSend(static_cast<int>(r + 1), 1, B_IN, bytes * (r + 1), bytes));
+            }
+        }
+        m.procs.push_back(std::move(pr));
+    }
+}
+
 // in[r]: p * recvCount elements, out[r]: recvCount elements.  Ring only at this level
 // (coll_reduce_scatter_comm_executor.cc:196-209); mesh uses the same slices with the mesh template.
 int orc_reducescatter(int algo, uint32_t p, void **in, void **out, uint64_t recvCount, int dt, int op,
@@ -1285,29 +1314,7 @@ int orc_reducescatter(int algo, uint32_t p, void **in, void **out, uint64_t recv
                     }
                 }
             } else if (algo == ALGO_RHD) {
-                // ReduceScatterRecursiveHalvingDoubling::RunAsync, reduce_scatter_recursive_hd.cc:33-254
-                uint32_t block, part1;
-                std::vector<uint32_t> rankOf;
-                std::vector<Slice> bsl;
-                RhdBlockLayout(p, bytes, &block, &part1, &rankOf, &bsl);
-                for (uint32_t r = 0; r < p; r++) {
-                    Proc pr;
-                    pr.rank = r;
-                    if (r < part1 && (r % 2) == 1) {
-                        pr.prog.push_back(MkSend(static_cast<int>(r - 1), 1, B_IN, 0, bytes * p));
-                        pr.prog.push_back(MkRecvCopy(static_cast<int>(r - 1), 1, B_IN, bytes * r, bytes));
-                    } else {
-                        if (r < part1) {
-                            pr.prog.push_back(MkRecvReduce(static_cast<int>(r + 1), 1, B_IN, 0, B_IN, 0, bytes * p));
-                        }
-                        uint32_t q = (r < part1) ? r / 2 : r - part1 / 2;
-                        ProgReduceScatterHd(pr.prog, q, block, rankOf, B_IN, B_IN, bsl);
-                        if (r < part1) {
-                            pr.prog.push_back(MkSend(static_cast<int>(r + 1), 1, B_IN, bytes * (r + 1), bytes));
-                        }
-                    }
-                    m.procs.push_back(std::move(pr));
-                }
+                AddReduceScatterRhdProcs(m, bytes);
             } else {
                 return -10;
             }
@@ -1319,6 +1326,124 @@ int orc_reducescatter(int algo, uint32_t p, void **in, void **out, uint64_t recv
         for (uint32_t r = 0; r < p; r++) {
             m.Copy(m.buf[B_OUT][r], m.buf[B_IN][r] + bytes * r, bytes);
             m.Copy(static_cast<uint8_t *>(out[r]) + offset, m.buf[B_OUT][r], bytes);
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
+// Two-level reduce-scatter, CollReduceScatterMeshExecutor::KernelRun with several servers
+// (EXE/coll_reduce_scatter/coll_reduce_scatter_mesh_executor.cc:128-247): `servers` groups of D = p / servers
+// consecutive ranks.  First the ranks with the same position in their groups reduce-scatter the whole staged
+// input among themselves (level1 = ALGO_RING or ALGO_RHD; a group's slice is the D blocks for its ranks), in
+// place; then the mesh reduce-scatter inside every group over that slice (piece cut, or uncut when `atomic`);
+// then the rank's block goes to the output.  Chunks of cclBytes / (p * unit) elements (:114-119).
+int orc_reducescatter_two_level(int level1, int atomic, uint32_t servers, uint32_t p, void **in, void **out, uint64_t recvCount,
+    int dt, int op, uint64_t cclBytes, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || servers == 0 || p % servers != 0 || (level1 != ALGO_RING && level1 != ALGO_RHD)) {
+        return -20;
+    }
+    const uint32_t D = p / servers;
+    uint64_t maxPer = cclBytes / (uint64_t(p) * unit);
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    auto machine = [&](uint32_t n) {
+        Machine m;
+        m.p = static_cast<int>(n);
+        m.dt = dt;
+        m.op = op;
+        m.direct = (flags & 1) != 0;
+        m.pool = &pool;
+        m.buf[B_IN].resize(n);
+        m.buf[B_OUT].resize(n);
+        return m;
+    };
+    Machine all = machine(p);
+    uint64_t stage = std::min<uint64_t>(recvCount, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage * p)), cclOut(p, std::vector<uint8_t>(stage));
+    for (uint32_t r = 0; r < p; r++) {
+        all.buf[B_IN][r] = cclIn[r].data();
+        all.buf[B_OUT][r] = cclOut[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = recvCount; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            for (uint32_t i = 0; i < p; i++) {
+                all.Copy(all.buf[B_IN][r] + bytes * i, static_cast<uint8_t *>(in[r]) + recvCount * unit * i + offset, bytes);
+            }
+        }
+        const uint64_t serverSlice = bytes * D;          // inputMem.size() / level1RankSize
+        // level 1: between the groups, for every position d
+        for (uint32_t d = 0; d < D && servers > 1; d++) {
+            Machine m = machine(servers);
+            for (uint32_t s = 0; s < servers; s++) {
+                m.buf[B_IN][s] = all.buf[B_IN][s * D + d];
+                m.buf[B_OUT][s] = all.buf[B_OUT][s * D + d];
+            }
+            if (level1 == ALGO_RING) {
+                std::vector<Slice> sl(servers);
+                for (uint32_t s = 0; s < servers; s++) {
+                    sl[s] = Slice{serverSlice * s, serverSlice};
+                }
+                for (uint32_t s = 0; s < servers; s++) {
+                    Proc pr;
+                    pr.rank = s;
+                    ProgReduceScatterRing(pr.prog, s, servers, B_IN, B_IN, sl, sl);
+                    m.procs.push_back(std::move(pr));
+                }
+            } else {
+                AddReduceScatterRhdProcs(m, serverSlice);
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        // level 0: mesh inside every group, on the group's slice of the input
+        for (uint32_t s = 0; s < servers && D > 1; s++) {
+            Machine m = machine(D);
+            for (uint32_t d = 0; d < D; d++) {
+                m.buf[B_IN][d] = all.buf[B_IN][s * D + d] + serverSlice * s;
+                m.buf[B_OUT][d] = all.buf[B_OUT][s * D + d];
+            }
+            std::vector<Slice> sl(D);
+            for (uint32_t d = 0; d < D; d++) {
+                sl[d] = Slice{bytes * d, bytes};
+            }
+            if (atomic) {
+                for (uint32_t d = 0; d < D; d++) {
+                    Proc pr;
+                    pr.rank = d;
+                    ProgReduceScatterMeshAtomic(pr.prog, d, D, B_IN, sl);
+                    m.procs.push_back(std::move(pr));
+                }
+            } else {
+                uint32_t nstream = D > 2 ? D - 1 : 1;
+                std::vector<std::vector<Slice>> pieces = CutPieces(sl, nstream, align);
+                for (uint32_t t = 0; t < nstream; t++) {
+                    for (uint32_t d = 0; d < D; d++) {
+                        Proc pr;
+                        pr.rank = d;
+                        ProgReduceScatterMeshStream(pr.prog, d, D, t, B_IN, pieces[t]);
+                        m.procs.push_back(std::move(pr));
+                    }
+                }
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            all.Copy(all.buf[B_OUT][r], all.buf[B_IN][r] + bytes * r, bytes);
+            all.Copy(static_cast<uint8_t *>(out[r]) + offset, all.buf[B_OUT][r], bytes);
         }
         offset += bytes;
         left -= cur;

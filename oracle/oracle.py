@@ -67,6 +67,8 @@ def lib():
         L.orc_reduce_to_root_rhd.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
         L.orc_allreduce_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64,
                                               i32, i32]
+        L.orc_reducescatter_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64,
+                                                  i32, i32]
         L.orc_broadcast_rhd.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
@@ -202,6 +204,21 @@ def reducescatter(ins, dt, op, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEF
     rc = lib().orc_reducescatter(algo, p, _ptrs(ins), _ptrs(outs), n, dt, op, ccl_bytes, align, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle reducescatter failed rc=%d" % rc)
+    return outs
+
+
+def reducescatter_two_level(ins, dt, op, servers, level1=RING, atomic=False, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN,
+                            flags=0, threads=1):
+    """`servers` groups of consecutive ranks: `level1` (RING or RHD) between the groups first, then the mesh inside
+    a group (piece cut, or uncut when `atomic`)."""
+    p = len(ins)
+    assert ins[0].size % p == 0
+    n = ins[0].size // p
+    outs = [np.empty(n, dtype=ins[0].dtype) for _ in range(p)]
+    rc = lib().orc_reducescatter_two_level(level1, 1 if atomic else 0, servers, p, _ptrs(ins), _ptrs(outs), n, dt, op,
+                                           ccl_bytes, align, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle two-level reducescatter failed rc=%d" % rc)
     return outs
 
 

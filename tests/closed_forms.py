@@ -302,6 +302,49 @@ def two_level_ring_allreduce(dt, op, ins, unit, ccl_bytes, align, servers, level
     return [out.copy() for _ in range(p)]
 
 
+def two_level_reducescatter(dt, op, ins, unit, ccl_bytes, align, servers, level1, atomic):
+    """Groups of D = p / servers consecutive ranks.  Block j = s * D + d of every input is first reduced over the
+    ranks at one position d' of all groups (level1 "ring": the ring chain for ring slice s; "rhd": the halving
+    tree of the block rank that owns slice s), giving one partial per position; the partials are then reduced
+    by the mesh chain of rank d inside group s (per piece when the block is cut)."""
+    p = len(ins)
+    D = p // servers
+    n = ins[0].size // p
+    max_per = ccl_bytes // (p * unit)
+    block, part1 = rhd_params(servers)
+    outs = []
+    for r in range(p):
+        s, d = divmod(r, D)
+        out = np.empty(n, dtype=ins[0].dtype)
+        base = 0
+        while base < n:
+            cur = min(n - base, max_per)
+            lo = r * n + base
+            partial = []
+            for dd in range(D):
+                xs = [ins[ss * D + dd][lo:lo + cur] for ss in range(servers)]
+                if servers == 1:
+                    partial.append(xs[0])
+                elif level1 == "ring":
+                    partial.append(ring_chain(dt, op, xs, s))
+                else:
+                    q = s // 2 if s < part1 else s - part1 // 2
+                    partial.append(rhd_tree(dt, op, xs, q, block, part1))
+            if D == 1:
+                out[base:base + cur] = partial[0]
+            elif atomic:
+                out[base:base + cur] = mesh_atomic_chain(dt, op, partial, d)
+            else:
+                nstream = D - 1 if D > 2 else 1
+                for t, (poff, psize) in enumerate(slice_plan(cur * unit, nstream, align)):
+                    a, b = poff // unit, (poff + psize) // unit
+                    if b > a:
+                        out[base + a:base + b] = mesh_chain(dt, op, [x[a:b] for x in partial], d, t)
+            base += cur
+        outs.append(out)
+    return outs
+
+
 def naive_reduce(dt, op, xs):
     acc = xs[0]
     for x in xs[1:]:

@@ -678,6 +678,31 @@ def test_two_level_allreduce_with_rings_inside_a_group(orc, level0):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("level1", [RING, RHD])
+def test_two_level_reducescatter(orc, level1):
+    # between the groups first (ring or halving-doubling), then the mesh inside a group
+    for servers, D in ((2, 4), (4, 2), (3, 4)):
+        p = servers * D
+        for det in (1, 0):
+            g = gh.Group(p, algo=ALGO_NAME[level1], deterministic=det, servers=servers)
+            try:
+                for dt, op, n in ((FP32, SUM, 30011), (BF16, SUM, 8192 + 5), (INT64, SUM, 1001), (FP32, MAX, 777)):
+                    atomic = (det == 0) and dt != INT64 and op != PROD
+                    ins = _ins(dt, p, n * p, 29 * p + n)
+                    want = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, atomic=atomic)
+                    print("two-level reduce-scatter", servers, "x", D, "level1", level1, "deterministic", det, "type", dt, flush=True)
+                    for fuse in (1, 0):
+                        g.set(fuse=fuse)
+                        outs, kept = gh.reduce_scatter(g, ins, dt, op)
+                        assert g.info()["fused"] == fuse
+                        for r in range(p):
+                            assert gh.same(dt, outs[r], want[r]), (servers, D, level1, det, dt, fuse, r)
+                            assert np.array_equal(kept[r], ins[r]), "send buffer changed"
+            finally:
+                g.close()
+
+
+@pytest.mark.gpu
 def test_two_level_allreduce_operand_order_of_max_min(orc):
     # NaN payloads and signed zeros show which operand stood left in every combine of the fused form
     specials = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.0, -1.0, 3.4e38], np.float32)

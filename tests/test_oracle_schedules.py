@@ -378,3 +378,24 @@ def test_multi_ring_parts_of_a_slice():
     # left-over rings empty (hand-computed: 1000 B over 4 rings -> 256, 256, 256, 232; 300 B -> 128, 128, 44, 0)
     assert [s for _, s in cf.slice_plan(1000, 4, 128)] == [256, 256, 256, 232]
     assert [s for _, s in cf.slice_plan(300, 4, 128)] == [128, 128, 44, 0]
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("atomic", [False, True])
+def test_two_level_reducescatter_matches_closed_form(orc, level1, atomic):
+    # between the servers first (ring or halving-doubling over the whole input), then the mesh inside a server
+    for servers, D in ((2, 4), (4, 2), (3, 4), (2, 8), (8, 1), (5, 3), (6, 2)):
+        p = servers * D
+        for dt, op, n, ccl in ((FP32, SUM, 211, 200 << 20), (FP32, SUM, 500, 4 * p * 128), (BF16, SUM, 301, 200 << 20),
+                               (INT32, MAX, 70, 200 << 20)):
+            ins = _inputs(dt, p, n * p, 41 * p + n)
+            got = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, atomic=atomic, ccl_bytes=ccl)
+            want = cf.two_level_reducescatter(dt, op, ins, orc.dtype_size(dt), ccl, 128, servers,
+                                              "ring" if level1 == RING else "rhd", atomic)
+            for r in range(p):
+                assert _eq(dt, got[r], want[r]), (servers, D, level1, atomic, dt, ccl, r)
+    # one server is the plain mesh reduce-scatter
+    ins = _inputs(FP32, 8, 8 * 409, 5)
+    a = orc.reducescatter_two_level(ins, FP32, SUM, 1, level1=level1, atomic=atomic)
+    b = orc.reducescatter(ins, FP32, SUM, algo=MESH_ATOMIC if atomic else MESH)
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))

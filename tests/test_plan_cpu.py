@@ -401,3 +401,24 @@ def test_two_level_allreduce_with_rings_inside_a_group_matches_checker(orc, leve
     # groups of another size have no four-ring form
     with pytest.raises(Exception):
         H.describe_plan(H.COLL_ALLREDUCE, level1 | (2 << 8) | (4 << 17), 8, 1000, FP32)
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("shape", [(2, 4), (4, 2), (3, 4), (2, 8), (8, 1), (5, 3)])
+def test_two_level_reducescatter_plan_matches_checker(orc, level1, shape):
+    servers, D = shape
+    p = servers * D
+    for atomic in (False, True):
+        for dt, op, n, ccl in ((FP32, SUM, 211, 200 << 20), (FP32, SUM, 500, 4 * p * 128), (BF16, PROD, 77, 200 << 20)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n * p, 600 + p + n)
+            want = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, atomic=atomic, ccl_bytes=ccl)
+            plan = H.describe_plan(H.COLL_REDUCESCATTER, level1 | (servers << 8) | (int(atomic) << 16), p, n, dt, ccl_bytes=ccl)
+            assert plan["fusedOk"]
+            for fused in (False, True):
+                sends = _bytes(ins)
+                recvs = [np.full(n * unit, 0x5A, np.uint8) for _ in range(p)]
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+                for r in range(p):
+                    assert _same(dt, recvs[r], want[r]), (shape, level1, atomic, dt, ccl, fused, r)
+                assert all(np.array_equal(s_, i.view(np.uint8)) for s_, i in zip(sends, ins))   # inputs stay as they were
