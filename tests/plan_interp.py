@@ -13,13 +13,20 @@ def _view(buf, off, n, dt):
     return buf[off:off + n].view(cf.CARRIER[dt])
 
 
+def _send_side(sends, recvs, in_place):
+    """in_place: True (every rank), False, or a bit mask of the ranks whose two buffers are one."""
+    if in_place is True:
+        return recvs
+    if not in_place:
+        return sends
+    return [recvs[r] if (in_place >> r) & 1 else sends[r] for r in range(len(sends))]
+
+
 def run_steps(plan, sends, recvs, dt, op, in_place=False):
     """sends / recvs: lists of uint8 arrays (recvs are written).  Scratch is made on demand."""
     p = plan["p"]
     scratch = [np.zeros(plan["scratchBytes"], np.uint8) for _ in range(p)]
-    bufs = {0: sends, 1: recvs, 2: scratch}
-    if in_place:
-        bufs[0] = recvs
+    bufs = {0: _send_side(sends, recvs, in_place), 1: recvs, 2: scratch}
     for phase in plan["phases"]:
         writes = []
         for s in phase:
@@ -35,7 +42,7 @@ def run_steps(plan, sends, recvs, dt, op, in_place=False):
 
 def run_fused(plan, sends, recvs, dt, op, in_place=False):
     assert plan["fusedOk"]
-    src_bufs = recvs if in_place else sends
+    src_bufs = _send_side(sends, recvs, in_place)
     results = []
     for it in plan["fused"]:
         n = it["n"]
