@@ -129,3 +129,43 @@ def test_random_rooted(orc, seed):
                 assert np.array_equal(gh.to_host(bufs[r], dt), ins[root]), (seed, case, "broadcast", r)
         finally:
             g.close()
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_allreduce_some_ranks_in_place_and_rank_groups(orc, seed):
+    # a random subset of the ranks passes one buffer for both arguments; half the cases run on rank groups
+    # (two-level schedules, mesh or rings inside a group)
+    rng = np.random.default_rng(9300 + seed)
+    for case in range(10):
+        p = int(rng.choice([4, 6, 8, 12, 16]))
+        dt = int(rng.choice(ALL_TYPES))
+        op = int(rng.integers(0, 4))
+        n = _size(rng)
+        fuse = int(rng.integers(0, 2))
+        mask = int(rng.integers(0, 1 << p))
+        level1 = int(rng.choice([RING, RHD]))
+        servers, level0 = 1, "mesh"
+        if rng.random() < 0.5:
+            servers = int(rng.choice([s for s in range(2, p + 1) if p % s == 0]))
+            level0 = str(rng.choice(["mesh", "ring", "ring4"])) if p // servers == 8 else str(rng.choice(["mesh", "ring"]))
+        ins = [cf.random_input(dt, n, rng) for _ in range(p)]
+        if servers > 1:
+            atomic = level0 == "mesh" and dt != INT64 and op != PROD
+            want = orc.allreduce_two_level(ins, dt, op, servers, level1=level1, atomic=atomic, level0=level0)
+        else:
+            want = orc.allreduce(ins, dt, op, algo=level1)
+        print("random allreduce seed", seed, "case", case, "p", p, "type", dt, "op", op, "n", n, "fuse", fuse, "mask", bin(mask),
+              "servers", servers, level0, "level1", level1, flush=True)
+        g = gh.Group(p, algo=NAMES[level1], fuse=fuse, servers=servers, level0=level0)
+        try:
+            sends = [gh.to_dev(x) for x in ins]
+            recvs = [sends[r] if (mask >> r) & 1 else gh.empty_dev(n * H.DTYPE_SIZE[dt]) for r in range(p)]
+            torch.cuda.synchronize()
+            H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, op, g.stream_ptr)
+            g.stream.synchronize()
+            for r in range(p):
+                assert gh.same(dt, gh.to_host(recvs[r], dt), want[r]), (seed, case, r)
+                if not (mask >> r) & 1:
+                    assert np.array_equal(gh.to_host(sends[r], dt), ins[r]), (seed, case, r, "send buffer changed")
+        finally:
+            g.close()
