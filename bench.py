@@ -244,6 +244,11 @@ def run_suite(pkg, torch, steps, warmup, only="", settings=()):
            lambda: pkg.reduce_scatter(comms, sp, rp, n // p, FP32, 0, stream.cuda_stream))
     pkg.comm_destroy(comms)
     comms = pkg.comm_init_all(p)
+    pkg.set_param(comms[0], "servers", 2)
+    report("reduce two-level 2x4 mesh+rhd fp32 sum 256MiB/rank root 3", comms,
+           lambda: pkg.reduce(comms, sp, rp, n, FP32, 0, 3, stream.cuda_stream))
+    pkg.comm_destroy(comms)
+    comms = pkg.comm_init_all(p)
     m = n // p
     report("scatter mesh p=8 32MiB/rank root 3", comms,
            lambda: pkg.scatter(comms, sp, rp, m, FP32, 3, stream.cuda_stream))

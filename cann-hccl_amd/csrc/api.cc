@@ -1486,9 +1486,14 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
     PlanRequest rq;
     rq.coll = CollKind(coll);
     if (coll >= COLL_BROADCAST) {
-        // rooted collectives: low 16 bits = root rank, bits 16.. = schedule (0 ring, 1 mesh, 4 mesh uncut)
+        // rooted collectives: low 16 bits = root rank, bits 16..19 = schedule (0 ring, 1 mesh, 2 rhd, 4 mesh uncut);
+        // reduce only: bits 20..27 = number of rank groups of the two-level schedule, bit 28 = its mesh level uncut
         rq.root = uint32_t(algo) & 0xffffu;
-        rq.algo = Algo(uint32_t(algo) >> 16);
+        rq.algo = Algo((uint32_t(algo) >> 16) & 0xfu);
+        if (coll == COLL_REDUCE) {
+            rq.servers = std::max(1u, (uint32_t(algo) >> 20) & 0xffu);
+            rq.meshAtomic = ((uint32_t(algo) >> 28) & 1u) != 0;
+        }
     } else if (coll == COLL_ALLREDUCE) {
         // all-reduce: low 8 bits = schedule, bits 8..15 = number of rank groups ("servers") of a two-level schedule
         rq.algo = Algo(uint32_t(algo) & 0xffu);

@@ -470,6 +470,94 @@ void RhdAllGatherChunk(VProgram &vp, size_t phase0, uint32_t p, const std::vecto
     }
 }
 
+// Ring reduce (reduce_ring.cc:29-154) among n ranks of `bytes` bytes at `off` in their input buffers:
+// the data walks root+1 -> ... -> root, every rank combining its own with what arrives; the last
+// combine writes `result` instead of the root's input.  Returns the phase after the last one used.
+size_t RingReducePhases(VProgram &vp, uint32_t n, uint32_t root, uint64_t off, uint64_t bytes, const Ref &result)
+{
+    for (uint32_t d = 2; d <= n; d++) {
+        uint32_t r = (root + d) % n, prev = (root + d - 1) % n;
+        Ref own = MkRef(r, BUF_SEND, off);
+        EmitReduce(vp, d - 2, d == n ? result : own, own, MkRef(prev, BUF_SEND, off), bytes);
+    }
+    return n > 1 ? n - 1 : 0;
+}
+
+// Recursive halving-doubling reduce (reduce_recursive_hd.cc:31-316) among n ranks: in every rank pair
+// of part one the rank with the root's parity folds its neighbour in (:85-148), the block runs the
+// halving reduce-scatter (:150-183), and a binomial gather over the output buffers brings the slices
+// to the root (:236-313).  The gather only forwards finished slices, so here each slice goes from the
+// rank that reduced it straight to `result` (rank and buffer of the destination; its offset is that
+// of the start of the data).  Returns the phase after the last one used.
+size_t RhdReducePhases(VProgram &vp, uint32_t n, uint32_t root, uint64_t off, uint64_t bytes, uint64_t align, const Ref &result)
+{
+    uint32_t block, part1;
+    HalvingDoublingShape(n, &block, &part1);
+    const uint32_t par = (root >= part1 ? 0u : root) % 2;
+    std::vector<uint32_t> rankOf(block);
+    for (uint32_t b = 0; b < block; b++) {
+        rankOf[b] = b < part1 / 2 ? 2 * b + par : b + part1 / 2;
+    }
+    std::vector<Slice> sl = RingSlicePlan(bytes, block, align);
+    size_t ph = 0;
+    if (part1 > 0) {
+        for (uint32_t b = 0; b < part1 / 2; b++) {
+            uint32_t mbr = rankOf[b], other = mbr ^ 1u;
+            EmitReduce(vp, ph, MkRef(mbr, BUF_SEND, off), MkRef(mbr, BUF_SEND, off), MkRef(other, BUF_SEND, off), bytes);
+        }
+        ph++;
+    }
+    ph = HalvingSteps(vp, ph, block, rankOf, off, sl);
+    for (uint32_t b = 0; b < block; b++) {
+        Ref dst = result;
+        dst.off += sl[b].off;
+        EmitCopy(vp, ph, dst, MkRef(rankOf[b], BUF_SEND, off + sl[b].off), sl[b].size);
+    }
+    return ph + 1;
+}
+
+// Two-level reduce of one chunk, CollReduceMeshExecutor::KernelRun with several servers
+// (coll_reduce_mesh_executor.cc:75-194): mesh reduce-scatter inside every group of D = p / servers
+// consecutive ranks (:95-107), the ranks at position d of all groups reduce slice d towards the one
+// in the root's group, ring or recursive halving-doubling (:109-160), and the root gathers the
+// slices inside its group (:164-187).  The level-1 results are written straight to the root's
+// output, which is where the gather would carry them.
+void TwoLevelReduceChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, uint32_t root, uint64_t base, uint64_t bytes,
+    uint64_t align, bool meshAtomic)
+{
+    const uint32_t D = p / servers;
+    const uint32_t rootServer = root / D;
+    std::vector<Slice> sl = RingSlicePlan(bytes, D, align);
+    const size_t l1 = D > 1 ? D - 1 : 0;
+    for (uint32_t s = 0; s < servers && D > 1; s++) {
+        vp.rankMap.resize(D);
+        for (uint32_t d = 0; d < D; d++) {
+            vp.rankMap[d] = s * D + d;
+        }
+        vp.phaseBase = 0;
+        MeshReduceScatterPhases(vp, 0, D, base, sl, align, meshAtomic);
+    }
+    for (uint32_t d = 0; d < D; d++) {
+        // local ranks 0 .. servers-1 are the groups' ranks at position d; one more entry names the root
+        vp.rankMap.resize(servers + 1);
+        for (uint32_t s = 0; s < servers; s++) {
+            vp.rankMap[s] = s * D + d;
+        }
+        vp.rankMap[servers] = root;
+        vp.phaseBase = l1;
+        const Ref result = MkRef(servers, BUF_RECV, base + sl[d].off);
+        if (servers == 1) {
+            EmitCopy(vp, 0, result, MkRef(0, BUF_SEND, base + sl[d].off), sl[d].size);
+        } else if (level1 == ALGO_RING) {
+            RingReducePhases(vp, servers, rootServer, base + sl[d].off, sl[d].size, result);
+        } else {
+            RhdReducePhases(vp, servers, rootServer, base + sl[d].off, sl[d].size, align, result);
+        }
+    }
+    vp.rankMap.clear();
+    vp.phaseBase = 0;
+}
+
 int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
 {
     uint32_t p = rq.p;
@@ -594,6 +682,9 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                 for (uint32_t b = 0; b < part1 / 2; b++) {
                     EmitCopy(*vp, ph, data(rankOf[b] ^ 1u), data(rankOf[b]), bytes);
                 }
+            } else if (rq.coll == COLL_REDUCE && rq.servers > 1 && p > 1) {
+                TwoLevelReduceChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, R, done, bytes, rq.align,
+                    rq.meshAtomic);
             } else if (rq.coll == COLL_REDUCE && rq.algo == ALGO_MESH && p > 1) {
                 // mesh reduce (coll_reduce_mesh_executor.cc:75-194): mesh reduce-scatter over the ring
                 // slice plan, then the root gathers slice r from rank r (gather_mesh.cc:60-170)
@@ -603,31 +694,7 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                     EmitCopy(*vp, ph, MkRef(R, BUF_RECV, done + sl[r].off), MkRef(r, BUF_SEND, done + sl[r].off), sl[r].size);
                 }
             } else if (rq.coll == COLL_REDUCE && rq.algo == ALGO_RHD && p > 1) {
-                // recursive halving-doubling reduce (reduce_recursive_hd.cc:31-316): in every rank pair of
-                // part one the rank with the root's parity folds its neighbour in (:85-148), the block
-                // runs the halving reduce-scatter (:150-183), and a binomial gather over the output
-                // buffers brings the slices to the root (:236-313).  The gather only forwards finished
-                // slices, so here the root takes each slice from the rank that reduced it.
-                uint32_t block, part1;
-                HalvingDoublingShape(p, &block, &part1);
-                const uint32_t par = (R >= part1 ? 0u : R) % 2;
-                std::vector<uint32_t> rankOf(block);
-                for (uint32_t b = 0; b < block; b++) {
-                    rankOf[b] = b < part1 / 2 ? 2 * b + par : b + part1 / 2;
-                }
-                std::vector<Slice> sl = RingSlicePlan(bytes, block, rq.align);
-                size_t ph = 0;
-                if (part1 > 0) {
-                    for (uint32_t b = 0; b < part1 / 2; b++) {
-                        uint32_t mbr = rankOf[b], other = mbr ^ 1u;
-                        EmitReduce(*vp, ph, MkRef(mbr, BUF_SEND, done), MkRef(mbr, BUF_SEND, done), MkRef(other, BUF_SEND, done), bytes);
-                    }
-                    ph++;
-                }
-                ph = HalvingSteps(*vp, ph, block, rankOf, done, sl);
-                for (uint32_t b = 0; b < block; b++) {
-                    EmitCopy(*vp, ph, MkRef(R, BUF_RECV, done + sl[b].off), MkRef(rankOf[b], BUF_SEND, done + sl[b].off), sl[b].size);
-                }
+                RhdReducePhases(*vp, p, R, done, bytes, rq.align, MkRef(R, BUF_RECV, done));
             } else if (rq.coll == COLL_BROADCAST) {
                 // ring broadcast (broadcast_ring.cc:24-160): the chunk is cut into p slices that travel
                 // root -> root+1 -> ... -> root-1 as a pipeline; slice j reaches distance d in phase j+d-1
@@ -648,12 +715,7 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                 if (p == 1) {
                     EmitCopy(*vp, 0, MkRef(0, BUF_RECV, done), MkRef(0, BUF_SEND, done), bytes);
                 }
-                for (uint32_t d = 2; d <= p && p > 1; d++) {
-                    uint32_t r = (R + d) % p, prev = (R + d - 1) % p;
-                    Ref own = MkRef(r, BUF_SEND, done);
-                    Ref dst = (d == p) ? MkRef(R, BUF_RECV, done) : own;
-                    EmitReduce(*vp, d - 2, dst, own, MkRef(prev, BUF_SEND, done), bytes);
-                }
+                RingReducePhases(*vp, p, R, done, bytes, MkRef(R, BUF_RECV, done));
             }
             done += bytes;
             left -= cur;

@@ -1885,6 +1885,87 @@ int orc_broadcast_rhd(uint32_t p, void **buf, uint64_t count, int dt, uint32_t r
     return 0;
 }
 
+// Per-rank programs of ReduceRecursiveHalvingDoubling::RunAsync (TPL/temp_reduce/reduce_recursive_hd.cc:31-316) on the
+// machine's buffers of `bytes` bytes: input accumulates in place, the result ends in the root's output buffer.
+void AddReduceRhdProcs(Machine &m, uint32_t root, uint64_t bytes, uint64_t align)
+{
+    const uint32_t p = static_cast<uint32_t>(m.p);
+    uint32_t block, part1;
+    RhdParams(p, &block, &part1);
+    std::vector<Slice> sl = RhdSlices(bytes, block, align);
+    const uint32_t rootFlag = root >= part1 ? 0 : root;
+    auto member = [&](uint32_t r) { return r >= part1 || (r % 2) == (rootFlag % 2); };
+    auto blockRank = [&](uint32_t r) { return r < part1 ? r / 2 : r - part1 / 2; };
+    std::vector<uint32_t> rankOf(block);
+    for (uint32_t r = 0; r < p; r++) {
+        if (member(r)) {
+            rankOf[blockRank(r)] = r;
+        }
+    }
+    const uint32_t rootQ = root > part1 ? root - part1 / 2 : root / 2;   // as written at :246
+    uint32_t rounds = 0;
+    while ((1u << rounds) < block) {
+        rounds++;
+    }
+    auto sum = [&](uint32_t first, uint32_t n) {
+        uint64_t t = 0;
+        for (uint32_t i = first; i < first + n; i++) {
+            t += sl[i].size;
+        }
+        return t;
+    };
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        const uint32_t pairPeer = (r % 2) == 0 ? r + 1 : r - 1;
+        if (!member(r)) {
+            pr.prog.push_back(MkSend(static_cast<int>(pairPeer), 1, B_IN, 0, bytes));
+            m.procs.push_back(std::move(pr));
+            continue;
+        }
+        if (r < part1) {
+            pr.prog.push_back(MkRecvReduce(static_cast<int>(pairPeer), 1, B_IN, 0, B_IN, 0, bytes));
+        }
+        const uint32_t q = blockRank(r);
+        ProgReduceScatterHd(pr.prog, q, block, rankOf, B_IN, B_OUT, sl);
+        for (uint32_t step = 0; step < rounds; step++) {
+            const uint32_t mask = 1u << step;
+            if (step != 0 && (q & (mask - 1)) != (rootQ & (mask - 1))) {
+                break;
+            }
+            const uint32_t peer = q ^ mask;
+            if ((q & mask) == (rootQ & mask)) {
+                const uint32_t rxId = peer & ~(mask - 1);
+                pr.prog.push_back(MkRecvCopy(static_cast<int>(rankOf[peer]), 2, B_OUT, sl[rxId].off, sum(rxId, mask)));
+            } else {
+                const uint32_t txId = q & ~(mask - 1);
+                pr.prog.push_back(MkSend(static_cast<int>(rankOf[peer]), 2, B_OUT, sl[txId].off, sum(txId, mask)));
+            }
+        }
+        m.procs.push_back(std::move(pr));
+    }
+}
+
+// Per-rank programs of ReduceRing::RunAsync (TPL/temp_reduce/reduce_ring.cc:29-154): the data walks root+1 -> ... -> root.
+void AddReduceRingProcs(Machine &m, uint32_t root, uint64_t bytes)
+{
+    const uint32_t p = static_cast<uint32_t>(m.p);
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        uint32_t left_ = (r + p - 1) % p, right = (r + 1) % p;
+        if (r == root) {
+            pr.prog.push_back(MkRecvReduce(static_cast<int>(left_), 0, B_OUT, 0, B_IN, 0, bytes));
+        } else if (left_ == root) {
+            pr.prog.push_back(MkSend(static_cast<int>(right), 0, B_IN, 0, bytes));
+        } else {
+            pr.prog.push_back(MkRecvReduce(static_cast<int>(left_), 0, B_IN, 0, B_IN, 0, bytes));
+            pr.prog.push_back(MkSend(static_cast<int>(right), 0, B_IN, 0, bytes));
+        }
+        m.procs.push_back(std::move(pr));
+    }
+}
+
 // Recursive halving-doubling reduce, ReduceRecursiveHalvingDoubling::RunAsync
 // (TPL/temp_reduce/reduce_recursive_hd.cc:31-316): ReduceInPartOne (:85-148: in each rank pair of part one the
 // rank whose parity is the root's receives), ReduceScatterInBlock (:150-183), GatherInBlock (:236-313: a
@@ -1925,60 +2006,7 @@ int orc_reduce_to_root_rhd(uint32_t p, void **in, void *outRoot, uint64_t count,
         if (p == 1) {
             m.Copy(m.buf[B_OUT][0], m.buf[B_IN][0], bytes);
         } else {
-            uint32_t block, part1;
-            RhdParams(p, &block, &part1);
-            std::vector<Slice> sl = RhdSlices(bytes, block, align);
-            const uint32_t rootFlag = root >= part1 ? 0 : root;
-            auto member = [&](uint32_t r) { return r >= part1 || (r % 2) == (rootFlag % 2); };
-            auto blockRank = [&](uint32_t r) { return r < part1 ? r / 2 : r - part1 / 2; };
-            std::vector<uint32_t> rankOf(block);
-            for (uint32_t r = 0; r < p; r++) {
-                if (member(r)) {
-                    rankOf[blockRank(r)] = r;
-                }
-            }
-            const uint32_t rootQ = root > part1 ? root - part1 / 2 : root / 2;   // as written at :246
-            uint32_t rounds = 0;
-            while ((1u << rounds) < block) {
-                rounds++;
-            }
-            auto sum = [&](uint32_t first, uint32_t n) {
-                uint64_t t = 0;
-                for (uint32_t i = first; i < first + n; i++) {
-                    t += sl[i].size;
-                }
-                return t;
-            };
-            for (uint32_t r = 0; r < p; r++) {
-                Proc pr;
-                pr.rank = r;
-                const uint32_t pairPeer = (r % 2) == 0 ? r + 1 : r - 1;
-                if (!member(r)) {
-                    pr.prog.push_back(MkSend(static_cast<int>(pairPeer), 1, B_IN, 0, bytes));
-                    m.procs.push_back(std::move(pr));
-                    continue;
-                }
-                if (r < part1) {
-                    pr.prog.push_back(MkRecvReduce(static_cast<int>(pairPeer), 1, B_IN, 0, B_IN, 0, bytes));
-                }
-                const uint32_t q = blockRank(r);
-                ProgReduceScatterHd(pr.prog, q, block, rankOf, B_IN, B_OUT, sl);
-                for (uint32_t step = 0; step < rounds; step++) {
-                    const uint32_t mask = 1u << step;
-                    if (step != 0 && (q & (mask - 1)) != (rootQ & (mask - 1))) {
-                        break;
-                    }
-                    const uint32_t peer = q ^ mask;
-                    if ((q & mask) == (rootQ & mask)) {
-                        const uint32_t rxId = peer & ~(mask - 1);
-                        pr.prog.push_back(MkRecvCopy(static_cast<int>(rankOf[peer]), 2, B_OUT, sl[rxId].off, sum(rxId, mask)));
-                    } else {
-                        const uint32_t txId = q & ~(mask - 1);
-                        pr.prog.push_back(MkSend(static_cast<int>(rankOf[peer]), 2, B_OUT, sl[txId].off, sum(txId, mask)));
-                    }
-                }
-                m.procs.push_back(std::move(pr));
-            }
+            AddReduceRhdProcs(m, root, bytes, align);
             int rc = m.Run();
             if (rc != 0) {
                 return rc;
@@ -2084,6 +2112,138 @@ int orc_reduce_to_root_mesh(uint32_t p, void **in, void *outRoot, uint64_t count
 }
 
 
+// Two-level reduce, CollReduceMeshExecutor::KernelRun with several servers
+// (EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194): `servers` groups of D = p / servers consecutive ranks.
+// Mesh reduce-scatter inside every group over the ring slice plan for D (piece cut, or uncut when `atomic`); the
+// ranks at position d of all groups reduce slice d to the one in the root's group (level1 = ALGO_RING or ALGO_RHD,
+// input range to output range; a copy when there is one group); GatherMesh to the root inside its group.
+int orc_reduce_to_root_two_level(int level1, int atomic, uint32_t servers, uint32_t p, void **in, void *outRoot, uint64_t count,
+    int dt, int op, uint32_t root, uint64_t cclBytes, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p || servers == 0 || p % servers != 0 || (level1 != ALGO_RING && level1 != ALGO_RHD)) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    const uint32_t D = p / servers;
+    const uint32_t rootServer = root / D, rootPos = root % D;
+    Pool pool(threads);
+    auto machine = [&](uint32_t n) {
+        Machine m;
+        m.p = static_cast<int>(n);
+        m.dt = dt;
+        m.op = op;
+        m.direct = (flags & 1) != 0;
+        m.pool = &pool;
+        m.buf[B_IN].resize(n);
+        m.buf[B_OUT].resize(n);
+        return m;
+    };
+    Machine all = machine(p);
+    uint64_t stage = std::min<uint64_t>(count, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage)), cclOut(p, std::vector<uint8_t>(stage));
+    for (uint32_t r = 0; r < p; r++) {
+        all.buf[B_IN][r] = cclIn[r].data();
+        all.buf[B_OUT][r] = cclOut[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            all.Copy(all.buf[B_IN][r], static_cast<uint8_t *>(in[r]) + offset, bytes);
+        }
+        std::vector<Slice> sl = RingSlices(bytes, D, align);
+        for (uint32_t s = 0; s < servers && D > 1; s++) {
+            Machine m = machine(D);
+            for (uint32_t d = 0; d < D; d++) {
+                m.buf[B_IN][d] = all.buf[B_IN][s * D + d];
+                m.buf[B_OUT][d] = all.buf[B_OUT][s * D + d];
+            }
+            if (atomic) {
+                for (uint32_t d = 0; d < D; d++) {
+                    Proc pr;
+                    pr.rank = d;
+                    ProgReduceScatterMeshAtomic(pr.prog, d, D, B_IN, sl);
+                    m.procs.push_back(std::move(pr));
+                }
+            } else {
+                uint32_t nstream = D > 2 ? D - 1 : 1;
+                std::vector<std::vector<Slice>> pieces = CutPieces(sl, nstream, align);
+                for (uint32_t t = 0; t < nstream; t++) {
+                    for (uint32_t d = 0; d < D; d++) {
+                        Proc pr;
+                        pr.rank = d;
+                        ProgReduceScatterMeshStream(pr.prog, d, D, t, B_IN, pieces[t]);
+                        m.procs.push_back(std::move(pr));
+                    }
+                }
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        // level 1: slice d, among the ranks at position d, to the one in the root's group
+        for (uint32_t d = 0; d < D; d++) {
+            if (sl[d].size == 0) {
+                continue;
+            }
+            Machine m = machine(servers);
+            for (uint32_t s = 0; s < servers; s++) {
+                m.buf[B_IN][s] = all.buf[B_IN][s * D + d] + sl[d].off;
+                m.buf[B_OUT][s] = all.buf[B_OUT][s * D + d] + sl[d].off;
+            }
+            if (servers == 1) {
+                m.Copy(m.buf[B_OUT][0], m.buf[B_IN][0], sl[d].size);
+                continue;
+            }
+            if (level1 == ALGO_RING) {
+                AddReduceRingProcs(m, rootServer, sl[d].size);
+            } else {
+                AddReduceRhdProcs(m, rootServer, sl[d].size, align);
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        // gather inside the root's group
+        if (D > 1) {
+            Machine m = machine(D);
+            for (uint32_t d = 0; d < D; d++) {
+                m.buf[B_IN][d] = all.buf[B_IN][rootServer * D + d];
+                m.buf[B_OUT][d] = all.buf[B_OUT][rootServer * D + d];
+            }
+            for (uint32_t d = 0; d < D; d++) {
+                Proc pr;
+                pr.rank = d;
+                if (d == rootPos) {
+                    for (uint32_t srcRank = 0; srcRank < D; srcRank++) {
+                        if (srcRank != rootPos) {
+                            pr.prog.push_back(MkRecvCopy(static_cast<int>(srcRank), 0, B_OUT, sl[srcRank].off, sl[srcRank].size));
+                        }
+                    }
+                } else {
+                    pr.prog.push_back(MkSend(static_cast<int>(rootPos), 0, B_OUT, sl[d].off, sl[d].size));
+                }
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        all.Copy(static_cast<uint8_t *>(outRoot) + offset, all.buf[B_OUT][root], bytes);
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
 // Ring reduce (reduce_ring.cc:29-154) with the executor's chunk loop; out[root] receives the result.
 // Inputs are staged (the schedule accumulates in its input buffer).
 int orc_reduce_to_root(uint32_t p, void **in, void *outRoot, uint64_t count, int dt, int op, uint32_t root, uint64_t cclBytes,
@@ -2122,20 +2282,7 @@ int orc_reduce_to_root(uint32_t p, void **in, void *outRoot, uint64_t count, int
         if (p == 1) {
             m.Copy(m.buf[B_OUT][0], m.buf[B_IN][0], bytes);
         } else {
-            for (uint32_t r = 0; r < p; r++) {
-                Proc pr;
-                pr.rank = r;
-                uint32_t left_ = (r + p - 1) % p, right = (r + 1) % p;
-                if (r == root) {
-                    pr.prog.push_back(MkRecvReduce(static_cast<int>(left_), 0, B_OUT, 0, B_IN, 0, bytes));
-                } else if (left_ == root) {
-                    pr.prog.push_back(MkSend(static_cast<int>(right), 0, B_IN, 0, bytes));
-                } else {
-                    pr.prog.push_back(MkRecvReduce(static_cast<int>(left_), 0, B_IN, 0, B_IN, 0, bytes));
-                    pr.prog.push_back(MkSend(static_cast<int>(right), 0, B_IN, 0, bytes));
-                }
-                m.procs.push_back(std::move(pr));
-            }
+            AddReduceRingProcs(m, root, bytes);
             int rc = m.Run();
             if (rc != 0) {
                 return rc;

@@ -69,6 +69,7 @@ def lib():
                                               i32, i32]
         L.orc_reducescatter_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64,
                                                   i32, i32]
+        L.orc_reduce_to_root_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_rhd.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
@@ -279,6 +280,18 @@ def reduce_to_root(ins, dt, op, root, ccl_bytes=DEFAULT_CCL_BYTES, flags=0, thre
         rc = lib().orc_reduce_to_root(len(ins), _ptrs(ins), out.ctypes.data, ins[0].size, dt, op, root, ccl_bytes, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle reduce failed rc=%d" % rc)
+    return out
+
+
+def reduce_to_root_two_level(ins, dt, op, root, servers, level1=RING, atomic=False, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN,
+                             flags=0, threads=1):
+    """`servers` groups of consecutive ranks: mesh reduce-scatter inside a group (piece cut, or uncut when `atomic`),
+    `level1` (RING or RHD) reduce of every slice towards the root's group, gather to the root inside its group."""
+    out = np.empty_like(ins[0])
+    rc = lib().orc_reduce_to_root_two_level(level1, 1 if atomic else 0, servers, len(ins), _ptrs(ins), out.ctypes.data, ins[0].size,
+                                            dt, op, root, ccl_bytes, align, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle two-level reduce failed rc=%d" % rc)
     return out
 
 

@@ -345,6 +345,48 @@ def two_level_reducescatter(dt, op, ins, unit, ccl_bytes, align, servers, level1
     return outs
 
 
+def two_level_reduce_to_root(dt, op, ins, unit, ccl_bytes, align, servers, level1, atomic, root):
+    """Groups of D = p / servers consecutive ranks: the mesh chain inside every group for slice d (per piece when the
+    slice is cut), then the groups' partial results of that slice reduced towards the root's group: level1 "ring" is
+    the ring chain ending at that group, "rhd" the halving-doubling reduce tree."""
+    p = len(ins)
+    D = p // servers
+    n = ins[0].size
+    root_server = root // D
+    out = np.empty_like(ins[0])
+    max_per = ccl_bytes // unit
+    base = 0
+    while base < n:
+        cur = min(n - base, max_per)
+        for d, (off, size) in enumerate(slice_plan(cur * unit, D, align)):
+            lo, hi = base + off // unit, base + (off + size) // unit
+            if hi <= lo:
+                continue
+            partial = []
+            for s in range(servers):
+                xs = [x[lo:hi] for x in ins[s * D:(s + 1) * D]]
+                if D == 1:
+                    partial.append(xs[0].copy())
+                elif atomic:
+                    partial.append(mesh_atomic_chain(dt, op, xs, d))
+                else:
+                    acc = np.empty_like(xs[0])
+                    nstream = D - 1 if D > 2 else 1
+                    for t, (poff, psize) in enumerate(slice_plan(size, nstream, align)):
+                        a, b = poff // unit, (poff + psize) // unit
+                        if b > a:
+                            acc[a:b] = mesh_chain(dt, op, [x[a:b] for x in xs], d, t)
+                    partial.append(acc)
+            if servers == 1:
+                out[lo:hi] = partial[0]
+            elif level1 == "ring":
+                out[lo:hi] = ring_chain(dt, op, partial, root_server)
+            else:
+                out[lo:hi] = rhd_reduce_to_root(dt, op, partial, unit, 1 << 62, align, root_server)
+        base += cur
+    return out
+
+
 def naive_reduce(dt, op, xs):
     acc = xs[0]
     for x in xs[1:]:

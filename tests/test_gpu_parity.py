@@ -703,6 +703,42 @@ def test_two_level_reducescatter(orc, level1):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("level1", [RING, RHD])
+def test_two_level_reduce_to_root(orc, level1):
+    # mesh inside a group, every slice reduced towards the root's group, gathered by the root
+    for servers, D in ((2, 4), (4, 2), (3, 4)):
+        p = servers * D
+        for det in (1, 0):
+            g = gh.Group(p, algo=ALGO_NAME[level1], deterministic=det, servers=servers)
+            try:
+                for dt, op, n in ((FP32, SUM, 300007), (BF16, SUM, 65536 + 5), (INT64, SUM, 10001)):
+                    atomic = (det == 0) and dt != INT64 and op != PROD
+                    ins = _ins(dt, p, n, 31 * p + n)
+                    for root in (0, D + 1):
+                        want = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, atomic=atomic)
+                        print("two-level reduce", servers, "x", D, "level1", level1, "deterministic", det, "type", dt, "root", root,
+                              flush=True)
+                        for fuse in (1, 0):
+                            g.set(fuse=fuse)
+                            sends = [gh.to_dev(x) for x in ins]
+                            recvs = [gh.empty_dev(n * H.DTYPE_SIZE[dt]) for _ in range(p)]
+                            for t in recvs:
+                                t.fill_(0x77)
+                            torch.cuda.synchronize()
+                            H.reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, op, root,
+                                     g.stream_ptr)
+                            g.stream.synchronize()
+                            assert g.info()["fused"] == fuse
+                            assert gh.same(dt, gh.to_host(recvs[root], dt), want), (servers, D, level1, det, dt, root, fuse)
+                            for r in range(p):
+                                assert np.array_equal(gh.to_host(sends[r], dt), ins[r]), "send buffer changed"
+                                if r != root:
+                                    assert bool((recvs[r] == 0x77).all()), "a rank other than the root was written"
+            finally:
+                g.close()
+
+
+@pytest.mark.gpu
 def test_two_level_allreduce_operand_order_of_max_min(orc):
     # NaN payloads and signed zeros show which operand stood left in every combine of the fused form
     specials = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.0, -1.0, 3.4e38], np.float32)

@@ -399,3 +399,24 @@ def test_two_level_reducescatter_matches_closed_form(orc, level1, atomic):
     a = orc.reducescatter_two_level(ins, FP32, SUM, 1, level1=level1, atomic=atomic)
     b = orc.reducescatter(ins, FP32, SUM, algo=MESH_ATOMIC if atomic else MESH)
     assert all(np.array_equal(x, y) for x, y in zip(a, b))
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("atomic", [False, True])
+def test_two_level_reduce_to_root_matches_closed_form(orc, level1, atomic):
+    # mesh inside a server, then every slice reduced towards the root's server, then gathered to the root
+    for servers, D in ((2, 4), (4, 2), (3, 4), (2, 8), (8, 1), (5, 3), (6, 2), (1, 4)):
+        p = servers * D
+        for dt, op, n, ccl in ((FP32, SUM, 2003, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, SUM, 1501, 200 << 20),
+                               (INT32, MAX, 700, 200 << 20)):
+            ins = _inputs(dt, p, n, 43 * p + n)
+            for root in sorted({0, p - 1, p // 2, (D + 1) % p}):
+                got = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, atomic=atomic, ccl_bytes=ccl)
+                want = cf.two_level_reduce_to_root(dt, op, ins, orc.dtype_size(dt), ccl, 128, servers,
+                                                   "ring" if level1 == RING else "rhd", atomic, root)
+                assert _eq(dt, got, want), (servers, D, level1, atomic, dt, ccl, root)
+    # one server is the plain mesh reduce
+    ins = _inputs(FP32, 8, 4099, 5)
+    a = orc.reduce_to_root_two_level(ins, FP32, SUM, 3, 1, level1=level1, atomic=atomic)
+    b = orc.reduce_to_root(ins, FP32, SUM, 3, algo=MESH_ATOMIC if atomic else MESH)
+    assert np.array_equal(a, b)

@@ -422,3 +422,28 @@ def test_two_level_reducescatter_plan_matches_checker(orc, level1, shape):
                 for r in range(p):
                     assert _same(dt, recvs[r], want[r]), (shape, level1, atomic, dt, ccl, fused, r)
                 assert all(np.array_equal(s_, i.view(np.uint8)) for s_, i in zip(sends, ins))   # inputs stay as they were
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("shape", [(2, 4), (4, 2), (3, 4), (2, 8), (8, 1), (5, 3)])
+def test_two_level_reduce_plan_matches_checker(orc, level1, shape):
+    servers, D = shape
+    p = servers * D
+    for atomic in (False, True):
+        for dt, op, n, ccl in ((FP32, SUM, 2003, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, PROD, 777, 200 << 20)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n, 700 + p + n)
+            for root in sorted({0, p - 1, (D + 1) % p}):
+                want = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, atomic=atomic, ccl_bytes=ccl)
+                plan = H.describe_plan(H.COLL_REDUCE, root | (level1 << 16) | (servers << 20) | (int(atomic) << 28), p, n, dt,
+                                       ccl_bytes=ccl)
+                assert plan["fusedOk"]
+                for fused in (False, True):
+                    sends = _bytes(ins)
+                    recvs = [np.full(n * unit, 0x77, np.uint8) for _ in range(p)]
+                    (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+                    assert _same(dt, recvs[root], want), (shape, level1, atomic, dt, ccl, root, fused)
+                    for r in range(p):
+                        assert np.array_equal(sends[r], ins[r].view(np.uint8))
+                        if r != root:
+                            assert np.all(recvs[r] == 0x77)              # only the root's output is written

@@ -20,7 +20,7 @@ def _case(rng):
     ccl = int(rng.choice([200 << 20, 200 << 20, 4 * p * align, 4096, 4 * int(rng.integers(p, 40 * p))]))
     algo = int(rng.choice([RING, MESH, RHD, MESH_ATOMIC]))
     servers, rings = 1, 0
-    if coll in (H.COLL_ALLREDUCE, H.COLL_REDUCESCATTER) and rng.random() < 0.4:
+    if coll in (H.COLL_ALLREDUCE, H.COLL_REDUCESCATTER, H.COLL_REDUCE) and rng.random() < 0.4:
         servers = int(rng.choice([s for s in range(1, p + 1) if p % s == 0]))
         algo = int(rng.choice([RING, RHD]))
         if coll == H.COLL_ALLREDUCE and rng.random() < 0.4:
@@ -45,6 +45,8 @@ def test_random_plans_compute_the_plain_result(seed):
             word = algo | (servers << 8) if servers > 1 else algo
         elif coll == H.COLL_ALLGATHER:
             word = algo
+        elif coll == H.COLL_REDUCE and servers > 1:
+            word = root | (algo << 16) | (servers << 20)
         else:
             word = root | (algo << 16)
         in_n = n * p if coll == H.COLL_REDUCESCATTER else n
