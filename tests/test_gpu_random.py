@@ -148,6 +148,8 @@ def test_random_allreduce_some_ranks_in_place_and_rank_groups(orc, seed):
         if rng.random() < 0.5:
             servers = int(rng.choice([s for s in range(2, p + 1) if p % s == 0]))
             level0 = str(rng.choice(["mesh", "ring", "ring4"])) if p // servers == 8 else str(rng.choice(["mesh", "ring"]))
+        unit = H.DTYPE_SIZE[dt]
+        pad = int(rng.choice([0, 0, unit, 16, 4 if unit <= 4 else 8]))      # buffers off their natural alignment
         ins = [cf.random_input(dt, n, rng) for _ in range(p)]
         if servers > 1:
             atomic = level0 == "mesh" and dt != INT64 and op != PROD
@@ -155,11 +157,11 @@ def test_random_allreduce_some_ranks_in_place_and_rank_groups(orc, seed):
         else:
             want = orc.allreduce(ins, dt, op, algo=level1)
         print("random allreduce seed", seed, "case", case, "p", p, "type", dt, "op", op, "n", n, "fuse", fuse, "mask", bin(mask),
-              "servers", servers, level0, "level1", level1, flush=True)
+              "servers", servers, level0, "level1", level1, "pad", pad, flush=True)
         g = gh.Group(p, algo=NAMES[level1], fuse=fuse, servers=servers, level0=level0)
         try:
-            sends = [gh.to_dev(x) for x in ins]
-            recvs = [sends[r] if (mask >> r) & 1 else gh.empty_dev(n * H.DTYPE_SIZE[dt]) for r in range(p)]
+            sends = [gh.to_dev(x, pad) for x in ins]
+            recvs = [sends[r] if (mask >> r) & 1 else gh.empty_dev(n * unit, pad if r % 2 else 0) for r in range(p)]
             torch.cuda.synchronize()
             H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, op, g.stream_ptr)
             g.stream.synchronize()
