@@ -280,6 +280,9 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="run the stand-alone memory-bandwidth probe (cann-hccl_amd/lib/hbm_probe: plain kernels, n streams "
                          "read : m written) and exit; its rates bound what the collectives can reach for the same mix")
+    ap.add_argument("--latency", action="store_true",
+                    help="run the compiled small-message timing (cann-hccl_amd/lib/call_latency: issue cost, back-to-back device "
+                         "time and call-to-completion time of 8 KiB ... 4 MiB all-reduces through the C ABI) and exit")
     ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
                     help="library setting for the run (see HcclAmdSetParam), e.g. --set blocks_per_cu=4")
     args = ap.parse_args()
@@ -287,6 +290,13 @@ def main():
         sys.exit("bench.py: this path is built and measured on one GPU (the ranks of the communicator are "
                  "simulated inside it); --gpus %d is not supported" % args.gpus)
 
+    if args.latency:
+        import subprocess
+        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cann-hccl_amd", "lib", "call_latency")
+        if not os.path.exists(exe):
+            sys.exit("bench.py: %s is not built (python cann-hccl_amd/build.py)" % exe)
+        rc = subprocess.run([exe, "1"]).returncode
+        sys.exit(rc or subprocess.run([exe, "0"]).returncode)
     if args.probe:
         import subprocess
         exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cann-hccl_amd", "lib", "hbm_probe")
