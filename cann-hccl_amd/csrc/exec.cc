@@ -735,6 +735,15 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         pp = it->second.get();
         hit = true;
     } else {
+        // Preparing a collective allocates and fills its device tables, which a stream under capture
+        // does not allow: a caller that records collectives into a graph runs each of them once before.
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        HIP_OK(hipStreamIsCapturing(g->ctx->streams[launcher], &capture));
+        if (capture != hipStreamCaptureStatusNone) {
+            HCCL_LOG_ERROR("%s: first use of this collective (sizes, buffers, settings) while its stream is being captured; "
+                "run it once before the capture", CollName(g->ctx->sig.coll));
+            return HCCL_E_NOT_SUPPORT;
+        }
         if (it != g->cache.end()) {
             HIP_OK(hipDeviceSynchronize());
             g->cache.erase(it);
@@ -780,7 +789,14 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         }
         others = true;
     }
+    // A caller may be capturing this stream into a graph of its own.  A graph launched into a
+    // capturing stream is not recorded there (the caller's graph came out empty and replays did
+    // nothing), so the kernels are then launched one by one and become nodes of the caller's graph.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (pp->exec) {
+        HIP_OK(hipStreamIsCapturing(ls, &capture));
+    }
+    if (pp->exec && capture == hipStreamCaptureStatusNone) {
         HIP_OK(hipGraphLaunch(pp->exec, ls));
     } else {
         for (LaunchRec &l : pp->launches) {

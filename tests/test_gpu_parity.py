@@ -927,6 +927,61 @@ def test_two_groups_on_two_host_threads(orc):
     assert not any(t.is_alive() for t in ts)
 
 
+def test_collectives_recorded_into_a_callers_graph(orc):
+    # a caller captures its stream (collectives it has run once before, so nothing needs preparing) and replays
+    # the graph with other work of its own in between; every replay must give the eager result
+    p, n = 8, 100003
+    for fuse in (1, 0):
+        g = gh.Group(p, fuse=fuse)
+        try:
+            rng = np.random.default_rng(50 + fuse)
+            ins = [rng.standard_normal(n).astype(np.float32) for _ in range(p)]
+            sends = [torch.from_numpy(x).cuda() for x in ins]
+            recvs = [torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(p)]
+            gath = [torch.zeros(n * p, dtype=torch.float32, device="cuda") for _ in range(p)]
+            torch.cuda.synchronize()
+
+            def both():
+                H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, g.stream_ptr)
+                H.all_gather(g.comms, [t.data_ptr() for t in recvs], [t.data_ptr() for t in gath], n, FP32, g.stream_ptr)
+
+            both()                                   # first use prepares the tables (not allowed under capture)
+            g.stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(g.stream):
+                graph.capture_begin()
+                try:
+                    both()
+                finally:
+                    graph.capture_end()
+            for replay in range(3):
+                for t in sends:
+                    t.mul_(1.25)                     # the caller's own eager work between replays
+                torch.cuda.synchronize()
+                host = [t.cpu().numpy() for t in sends]
+                want = orc.allreduce(host, FP32, SUM)
+                for t in recvs + gath:
+                    t.zero_()
+                torch.cuda.synchronize()
+                graph.replay()
+                torch.cuda.synchronize()
+                for r in range(p):
+                    assert np.array_equal(recvs[r].cpu().numpy(), want[r]), (fuse, replay, r)
+                    assert np.array_equal(gath[r].cpu().numpy(), np.concatenate(want)), (fuse, replay, r)
+            # a collective the library has not seen yet cannot be prepared while the stream is being captured
+            graph2 = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(g.stream):
+                graph2.capture_begin()
+                try:
+                    codes = [H.lib().HcclAllReduce(sends[r].data_ptr(), recvs[r].data_ptr(), n - 7, FP32, SUM, g.comms[r], g.stream_ptr)
+                             for r in range(p)]
+                finally:
+                    graph2.capture_end()
+            assert codes[:-1] == [0] * (p - 1) and codes[-1] == H.HCCL_E_NOT_SUPPORT
+        finally:
+            g.close()
+
+
 def test_send_recv_and_batch():
     p, n = 4, 250007
     g = gh.Group(p)
