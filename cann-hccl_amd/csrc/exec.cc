@@ -102,7 +102,11 @@ struct Builder {
 };
 
 // Cuts [0, bytes) into an element-wise head, a 16-byte vector body and an element-wise tail, given
-// the addresses involved.  emit(offset, bytes, mode).
+// the addresses involved (the first one is a destination).  emit(offset, bytes, mode).
+// A long body is cut once more so that its main part starts on a 128-byte boundary of the destination:
+// a wave stores 1 KiB at a time, and when those stores straddle memory lines every line is written in
+// two pieces (measured, 8-rank fp32 all-reduce of 256 MiB per rank with all buffers 16 bytes off a
+// 128-byte boundary: 0.97 ms fused against 0.76 ms aligned).
 template <typename F> void SplitByAlignment(const std::vector<uintptr_t> &addrs, uint64_t bytes, F emit)
 {
     uintptr_t anchor = addrs[0];
@@ -122,7 +126,14 @@ template <typename F> void SplitByAlignment(const std::vector<uintptr_t> &addrs,
         emit(uint64_t(0), head, uint32_t(ACC_ELEM));
     }
     if (body) {
-        emit(head, body, uint32_t(co ? ACC_VEC16 : ACC_VEC16_SRC4));
+        const uint32_t mode = co ? ACC_VEC16 : ACC_VEC16_SRC4;
+        const uint64_t lead = (128 - ((anchor + head) & 127)) & 127;     // a multiple of 16
+        if (lead != 0 && body >= 4 * uint64_t(kTileBytes)) {
+            emit(head, lead, mode);
+            emit(head + lead, body - lead, mode);
+        } else {
+            emit(head, body, mode);
+        }
     }
     if (tail) {
         emit(head + body, tail, uint32_t(ACC_ELEM));
