@@ -102,7 +102,9 @@ struct Builder {
 };
 
 // Cuts [0, bytes) into an element-wise head, a 16-byte vector body and an element-wise tail, given
-// the addresses involved (the first one is a destination).  emit(offset, bytes, mode).
+// the addresses involved (the first one is a destination; all are multiples of the element size).
+// The head brings the first destination to a 16-byte boundary; pointers that are then not on one
+// too are accessed with unaligned 128-bit loads and stores (ACC_VEC16_ANY).  emit(offset, bytes, mode).
 // A long body is cut once more so that its main part starts on a 128-byte boundary of the destination:
 // a wave stores 1 KiB at a time, and when those stores straddle memory lines every line is written in
 // two pieces (measured, 8-rank fp32 all-reduce of 256 MiB per rank with all buffers 16 bytes off a
@@ -110,14 +112,9 @@ struct Builder {
 template <typename F> void SplitByAlignment(const std::vector<uintptr_t> &addrs, uint64_t bytes, F emit)
 {
     uintptr_t anchor = addrs[0];
-    bool co = true, w4 = true;
+    bool co = true;
     for (uintptr_t a : addrs) {
         co = co && ((a & 15) == (anchor & 15));
-        w4 = w4 && ((a & 3) == 0);
-    }
-    if (!co && !w4) {
-        emit(uint64_t(0), bytes, uint32_t(ACC_ELEM));
-        return;
     }
     uint64_t head = std::min<uint64_t>(bytes, (16 - (anchor & 15)) & 15);
     uint64_t body = (bytes - head) & ~uint64_t(15);
@@ -126,7 +123,7 @@ template <typename F> void SplitByAlignment(const std::vector<uintptr_t> &addrs,
         emit(uint64_t(0), head, uint32_t(ACC_ELEM));
     }
     if (body) {
-        const uint32_t mode = co ? ACC_VEC16 : ACC_VEC16_SRC4;
+        const uint32_t mode = co ? ACC_VEC16 : ACC_VEC16_ANY;
         const uint64_t lead = (128 - ((anchor + head) & 127)) & 127;     // a multiple of 16
         if (lead != 0 && body >= 4 * uint64_t(kTileBytes)) {
             emit(head, lead, mode);

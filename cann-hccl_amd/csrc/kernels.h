@@ -16,7 +16,7 @@ constexpr uint32_t kBlockThreads = 256;
 // How a step's bytes may be accessed.
 enum AccessMode : uint32_t {
     ACC_VEC16 = 0,      // every pointer 16-byte aligned, byte count a multiple of 16
-    ACC_VEC16_SRC4 = 1, // destinations 16-byte aligned, sources only 4-byte aligned, multiple of 16
+    ACC_VEC16_ANY = 1,  // first destination 16-byte aligned, the other pointers at any element boundary; multiple of 16
     ACC_ELEM = 2        // element by element (heads, tails, unaligned buffers)
 };
 

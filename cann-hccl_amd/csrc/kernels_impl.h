@@ -249,8 +249,9 @@ HCCL_WORDWISE_COMBINER(Bf16Bits, HCCL_EXPR_BF16)
 template <typename T, int OP> __device__ __forceinline__ V4 Combine16(V4 a, V4 b) { return Combiner<T, OP>::Apply(a, b); }
 
 // ---- memory access ---------------------------------------------------------------------------------
-// 16 bytes at an address that is only 4-byte aligned.
-typedef uint32_t V4A4 __attribute__((ext_vector_type(4), aligned(4)));
+// 16 bytes at an address of any alignment: the device runs in unaligned-access mode, so this is still
+// one 128-bit load or store (one that may touch two memory lines).
+typedef uint32_t V4U __attribute__((ext_vector_type(4), aligned(1)));
 
 // Rank buffers are device (global) memory.  The pointers come out of descriptor tables, so the
 // compiler cannot know that and would issue flat accesses, whose completion is counted together
@@ -258,7 +259,7 @@ typedef uint32_t V4A4 __attribute__((ext_vector_type(4), aligned(4)));
 // flight).  Casting to the global address space gives global_load / global_store.
 #define HCCL_GLOBAL __attribute__((address_space(1)))
 typedef V4 HCCL_GLOBAL GlobalV4;
-typedef V4A4 HCCL_GLOBAL GlobalV4A4;
+typedef V4U HCCL_GLOBAL GlobalV4U;
 
 template <uint32_t MODE> __device__ __forceinline__ V4 Load16(const void *base, uint64_t byteOff)
 {
@@ -266,7 +267,7 @@ template <uint32_t MODE> __device__ __forceinline__ V4 Load16(const void *base, 
     if (MODE == ACC_VEC16) {
         return __builtin_nontemporal_load((const GlobalV4 *)p);
     } else {
-        V4A4 t = *(const GlobalV4A4 *)p;
+        V4U t = __builtin_nontemporal_load((const GlobalV4U *)p);
         return V4{t.x, t.y, t.z, t.w};
     }
 }
@@ -462,8 +463,8 @@ __global__ void __launch_bounds__(kBlockThreads) StepKernel(const StepDesc *__re
         const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
         if (d.mode == ACC_VEC16) {
             StepTileVec<T, OP, ACC_VEC16>(d, off, n);
-        } else if (d.mode == ACC_VEC16_SRC4) {
-            StepTileVec<T, OP, ACC_VEC16_SRC4>(d, off, n);
+        } else if (d.mode == ACC_VEC16_ANY) {
+            StepTileVec<T, OP, ACC_VEC16_ANY>(d, off, n);
         } else {
             StepTileElem<T, OP>(d, off, n);
         }
@@ -491,8 +492,8 @@ template <uint32_t MODE, bool ORDINARY = false> __device__ __forceinline__ void 
             Store16(base, pos, v);
         }
     } else {
-        V4A4 t = {v.x, v.y, v.z, v.w};
-        *(GlobalV4A4 *)(static_cast<char *>(base) + pos) = t;
+        V4U t = {v.x, v.y, v.z, v.w};
+        __builtin_nontemporal_store(t, (GlobalV4U *)(static_cast<char *>(base) + pos));
     }
 }
 
@@ -610,8 +611,11 @@ __global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__
                     ChainVecPass<T, OP, ACC_VEC16, false>(d, src, dst, off, base, nvec);
                 }
             } else {
-                for (; base < nvec; base += kPass) {
-                    ChainVecPass<T, OP, ACC_VEC16_SRC4, false>(d, src, dst, off, base, nvec);
+                for (; base + kPass <= nvec; base += kPass) {
+                    ChainVecPass<T, OP, ACC_VEC16_ANY, true>(d, src, dst, off, base, nvec);
+                }
+                if (base < nvec) {
+                    ChainVecPass<T, OP, ACC_VEC16_ANY, false>(d, src, dst, off, base, nvec);
                 }
             }
         }
@@ -773,7 +777,7 @@ __device__ __forceinline__ void TreeTileVec(const FusedDesc &d, const void *cons
         }
     } else {
         for (; base < nvec; base += kPass) {
-            TreeVecPass<T, OP, ACC_VEC16_SRC4, false, G>(d, src, dst, off, base, nvec);
+            TreeVecPass<T, OP, ACC_VEC16_ANY, false, G>(d, src, dst, off, base, nvec);
         }
     }
 }
@@ -1041,7 +1045,7 @@ __global__ void __launch_bounds__(kBlockThreads) StackKernel(const FusedDesc *__
                 }
             } else {
                 for (; base < nvec; base += kPassDeep) {
-                    StackVecPass<T, OP, ACC_VEC16_SRC4, false, true>(d, src, ops, dst, off, base, nvec);
+                    StackVecPass<T, OP, ACC_VEC16_ANY, false, true>(d, src, ops, dst, off, base, nvec);
                 }
             }
         }
