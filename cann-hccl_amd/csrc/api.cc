@@ -1390,6 +1390,12 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         } else {
             return HCCL_E_PARA;
         }
+    } else if (k == "cache_entries") {
+        long n = std::atol(value);
+        if (n < 1 || n > (1 << 20)) {
+            return HCCL_E_PARA;
+        }
+        cfg.cacheEntries = uint32_t(n);
     } else if (k == "fused_stores") {
         if (v == "nt") {
             cfg.fusedStores = 0;

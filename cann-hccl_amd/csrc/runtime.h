@@ -39,6 +39,7 @@ struct GroupConfig {
     uint32_t level0Rings = 0;        // two-level all-reduce inside a group: 0 = mesh, 1 = one ring, 4 = four rings (groups of 8)
     int stepStores = -1;             // step kernel stores: -1 chosen per launch, 0 non-temporal, 1 ordinary
     int fusedStores = 0;             // fused chain kernel stores: 0 non-temporal, 1 ordinary
+    uint32_t cacheEntries = 1024;    // prepared collectives kept (distinct sizes / buffers / settings)
     uint32_t blocksPerCu = 0;             // workgroups per CU; 0 = per-kernel default
     bool blockingArrive = false;          // ranks wait inside the call until the collective is issued
     uint32_t arriveTimeoutMs = 1800 * 1000;
@@ -68,16 +69,29 @@ struct OpInfo {
     uint64_t scratchBytes = 0;
 };
 
+// Device memory for the descriptor tables of the prepared collectives: carved out of a few large
+// allocations, handed back all at once (hipFree waits for the whole device, so it is kept off the
+// path of a caller that cycles through many buffers).
+struct TableArena {
+    struct Chunk {
+        char *base = nullptr;
+        size_t size = 0, used = 0;
+    };
+    std::vector<Chunk> chunks;
+    void *Alloc(size_t bytes);       // nullptr when the device is out of memory
+    void Reset();                    // every block handed out becomes invalid; the first chunk is kept
+    void FreeAll();
+};
+
 struct Prepared {
     std::shared_ptr<const Plan> plan;   // shared with the group's plan cache (plans do not depend on addresses)
     bool fused = false;
-    void *devTables = nullptr;
+    void *devTables = nullptr;        // inside the group's table arena
     std::vector<LaunchRec> launches;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     uint64_t scratchGen = 0;
     OpInfo info;
-    uint64_t lastUse = 0;
     ~Prepared();
 };
 
@@ -152,9 +166,9 @@ struct Group {
     void *barrierMem = nullptr;       // 2 x p small buffers for HcclBarrier's all-reduce
     uint64_t scratchBytes = 0;
     uint64_t scratchGen = 0;
-    std::unordered_map<std::string, std::unique_ptr<Prepared>> cache;
+    std::unordered_map<std::string, std::unique_ptr<Prepared>> cache;   // keyed by request, settings and buffer addresses
+    TableArena arena;
     std::unordered_map<std::string, std::shared_ptr<const Plan>> planCache;   // keyed by the plan request
-    uint64_t useClock = 0;
     OpInfo lastInfo;
 
     ~Group();

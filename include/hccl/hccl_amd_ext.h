@@ -29,6 +29,8 @@ extern "C" {
  *                                so that the next phase finds the data in the memory-side cache); "auto" decides per collective
  *   "fused_stores"  "nt" | "ordinary"   store kind of the fused chain kernel: non-temporal (default), or write-back, which
  *                                keeps a result of up to 256 MB in the memory-side cache for whoever reads it next
+ *   "cache_entries" how many prepared collectives (distinct sizes, buffers, settings) the group keeps (default 1024);
+ *                   when full, the library waits for the device once and starts over
  *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
  *   "blocking_arrive" "0" | "1"  a rank's call waits inside the library until the group is complete
  *   "arrive_timeout_ms"          limit of that wait (HCCL_E_TIMEOUT)

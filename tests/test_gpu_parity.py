@@ -810,10 +810,10 @@ def test_fused_write_back_stores_give_the_same_bits(orc):
 
 @pytest.mark.gpu
 def test_many_shapes_evict_cached_collectives_without_leaking(orc):
-    # more distinct shapes than the library keeps prepared (64): old entries are dropped, results stay right and
-    # device memory returns to where it was
+    # more distinct shapes than the library keeps prepared (set to 48 here): when the table is full it is emptied
+    # and rebuilt, results stay right and device memory does not grow
     p = 4
-    g = gh.Group(p)
+    g = gh.Group(p, cache_entries=48)
     try:
         rng = np.random.default_rng(404)
         base = np.stack([rng.integers(-1000, 1000, 70000).astype(np.int32) for _ in range(p)])
