@@ -234,6 +234,27 @@ def test_amd_params(comms):
     assert L.HcclAmdSetParam(comms[0], b"nonsense", b"1") == H.HCCL_E_PARA
     assert L.HcclAmdSetParam(comms[0], b"buffsize_mib", b"0") == H.HCCL_E_PARA
     assert L.HcclAmdSetParam(None, b"algo", b"ring") == H.HCCL_E_PTR
+    # every documented key takes its documented values and nothing else
+    good = {b"algo": [b"ring", b"mesh", b"rhd", b"auto"], b"deterministic": [b"0", b"1"], b"fuse": [b"0", b"1"],
+            b"graph": [b"0", b"1"], b"buffsize_mib": [b"1", b"200"], b"buffsize_bytes": [b"4096"], b"align": [b"4", b"128"],
+            b"level0": [b"mesh", b"ring", b"ring4"], b"step_stores": [b"auto", b"nt", b"ordinary"],
+            b"fused_stores": [b"nt", b"ordinary"], b"cache_entries": [b"1", b"1024"], b"blocks_per_cu": [b"0", b"2"],
+            b"blocking_arrive": [b"0", b"1"], b"arrive_timeout_ms": [b"1000"]}
+    for key, values in good.items():
+        for v in values:
+            assert L.HcclAmdSetParam(comms[0], key, v) == 0, (key, v)
+    bad = {b"level0": b"star", b"step_stores": b"maybe", b"fused_stores": b"auto", b"cache_entries": b"0", b"align": b"0",
+           b"servers": b"0"}
+    for key, v in bad.items():
+        assert L.HcclAmdSetParam(comms[0], key, v) == H.HCCL_E_PARA, (key, v)
+    p = ctypes.c_uint32(0)
+    assert L.HcclGetRankSize(comms[0], ctypes.byref(p)) == 0
+    assert L.HcclAmdSetParam(comms[0], b"servers", str(p.value).encode()) == 0            # every rank its own group
+    assert L.HcclAmdSetParam(comms[0], b"servers", str(p.value + 1).encode()) == H.HCCL_E_PARA   # does not divide the ranks
+    for key, v in ((b"algo", b"auto"), (b"servers", b"1"), (b"level0", b"mesh"), (b"fuse", b"1"), (b"graph", b"1"),
+                   (b"deterministic", b"0"), (b"step_stores", b"auto"), (b"fused_stores", b"nt"), (b"blocking_arrive", b"0"),
+                   (b"buffsize_mib", b"200"), (b"align", b"128"), (b"blocks_per_cu", b"0"), (b"cache_entries", b"1024")):
+        assert L.HcclAmdSetParam(comms[0], key, v) == 0                                   # back to the defaults
 
 
 def test_unsupported_entry_points_link_and_refuse(comms):
