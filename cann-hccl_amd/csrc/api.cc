@@ -268,7 +268,7 @@ struct InUse {
 // Ends the current rendezvous.  Ranks blocked inside their call wake up and return `result`.
 void CancelPending(Group *g, HcclResult result)
 {
-    g->lastIssueResult = result;
+    g->issueResults[g->opSerial % 8] = result;
     g->arrived = 0;
     std::fill(g->here.begin(), g->here.end(), 0);
     g->opSerial++;
@@ -337,7 +337,7 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
             CancelPending(g, HCCL_E_TIMEOUT);
             return HCCL_E_TIMEOUT;
         }
-        return g->lastIssueResult;
+        return g->issueResults[serial % 8];
     }
     // last arrival
     HcclResult res = HCCL_SUCCESS;

@@ -150,7 +150,9 @@ struct Group {
     // rendezvous of the current collective
     uint32_t arrived = 0;
     uint64_t opSerial = 0;           // bumped whenever a collective is issued or cancelled
-    HcclResult lastIssueResult = HCCL_SUCCESS;
+    // How the most recent rendezvous ended, by serial number modulo the array size: a rank that blocked in
+    // rendezvous n reads entry n even if the other ranks have moved on to n + 1 by the time it wakes.
+    HcclResult issueResults[8] = {};
     std::vector<uint8_t> here;
     OpCtx pend;                      // what the ranks of the current collective passed
     OpCtx *ctx = nullptr;            // the operation being issued (the rendezvous, or a matched send / receive)
