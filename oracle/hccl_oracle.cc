@@ -19,6 +19,9 @@
 //                    1681-1720,1761-1833 (ring or four rings inside a server),
 //                    TPL/temp_reduce_scatter/reduce_scatter_mesh_atomic.cc:82-141 (accumulation order of the racing
 //                    streams fixed to stream order: for floating point the reference itself has no single answer)
+//   two levels       EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240 (several servers),
+//                    EXE/coll_reduce_scatter/coll_reduce_scatter_mesh_executor.cc:114-119,128-247,
+//                    EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194 (several servers)
 //   halving-doubling TPL/temp_all_reduce/all_reduce_recursive_hd.cc:33-302,
 //                    TPL/temp_reduce_scatter/reduce_scatter_recursive_hd.cc:33-254, TPL/temp_all_gather/all_gather_recursive_hd.cc:26-238,
 //                    TPL/temp_reduce_scatter/reduce_scatter_halving_doubling.cc:67-238,
