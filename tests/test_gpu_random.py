@@ -171,3 +171,47 @@ def test_random_allreduce_some_ranks_in_place_and_rank_groups(orc, seed):
                     assert np.array_equal(gh.to_host(sends[r], dt), ins[r]), (seed, case, r, "send buffer changed")
         finally:
             g.close()
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_reducescatter_and_reduce_on_rank_groups(orc, seed):
+    # two-level reduce-scatter and rooted reduce: random group shapes, types, sizes, misaligned buffers, both issue modes
+    rng = np.random.default_rng(9400 + seed)
+    for case in range(8):
+        p = int(rng.choice([4, 6, 8, 12, 16]))
+        servers = int(rng.choice([s for s in range(2, p + 1) if p % s == 0]))
+        level1 = int(rng.choice([RING, RHD]))
+        det = int(rng.integers(0, 2))
+        dt = int(rng.choice(ALL_TYPES))
+        op = int(rng.integers(0, 4))
+        n = max(1, _size(rng) // p)
+        fuse = int(rng.integers(0, 2))
+        root = int(rng.integers(0, p))
+        unit = H.DTYPE_SIZE[dt]
+        pad = int(rng.choice([0, 0, unit, 16]))
+        atomic = det == 0 and dt != INT64 and op != PROD
+        print("random grouped seed", seed, "case", case, "p", p, "servers", servers, "level1", level1, "deterministic", det, "type", dt,
+              "op", op, "n", n, "fuse", fuse, "root", root, "pad", pad, flush=True)
+        g = gh.Group(p, algo=NAMES[level1], deterministic=det, fuse=fuse, servers=servers)
+        try:
+            ins = [cf.random_input(dt, n * p, rng) for _ in range(p)]
+            want = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, atomic=atomic)
+            sends = [gh.to_dev(x, pad) for x in ins]
+            recvs = [gh.empty_dev(n * unit, pad if r % 2 else 0) for r in range(p)]
+            torch.cuda.synchronize()
+            H.reduce_scatter(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, op, g.stream_ptr)
+            g.stream.synchronize()
+            for r in range(p):
+                assert gh.same(dt, gh.to_host(recvs[r], dt), want[r]), (seed, case, "reduce-scatter", r)
+                assert np.array_equal(gh.to_host(sends[r], dt), ins[r]), (seed, case, "send buffer changed", r)
+            want_root = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, atomic=atomic)
+            outs = [gh.empty_dev(n * p * unit, 0 if r % 2 else pad, fill=0x33) for r in range(p)]
+            torch.cuda.synchronize()
+            H.reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in outs], n * p, dt, op, root, g.stream_ptr)
+            g.stream.synchronize()
+            assert gh.same(dt, gh.to_host(outs[root], dt), want_root), (seed, case, "reduce")
+            for r in range(p):
+                if r != root:
+                    assert bool((outs[r] == 0x33).all()), (seed, case, "a rank other than the root was written", r)
+        finally:
+            g.close()
