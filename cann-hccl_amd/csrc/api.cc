@@ -1390,6 +1390,14 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         } else {
             return HCCL_E_PARA;
         }
+    } else if (k == "step_sweep") {
+        if (v == "forward") {
+            cfg.stepSweep = 0;
+        } else if (v == "alternate") {
+            cfg.stepSweep = 1;
+        } else {
+            return HCCL_E_PARA;
+        }
     } else if (k == "cache_entries") {
         long n = std::atol(value);
         if (n < 1 || n > (1 << 20)) {

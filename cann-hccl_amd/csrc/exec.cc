@@ -245,6 +245,7 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
         }
         const bool ordinaryStores = g->cfg.stepStores < 0 ? PreferOrdinaryStores(*pp->plan, g->ctx->send, g->ctx->recv)
                                                           : g->cfg.stepStores == 1;
+        uint32_t launchNo = 0;
         for (const Phase &ph : pp->plan->phases) {
             // whole-tile 16-byte-vector pieces first (the kernel's fast loop), everything else after
             std::vector<StepDesc> whole, ragged;
@@ -276,6 +277,14 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                     }
                 });
             }
+            // Every other launch walks the data the other way round, so that a phase starts with what the
+            // phase before it wrote last (measured, 8-rank fp32 ring all-reduce of 256 MiB per rank: 1.431 ms
+            // against 1.437 ms; running all phases on one 16 ... 128 MiB window of offsets at a time, to keep
+            // the data between phases in the 256 MB memory-side cache, was slower: 1.44 ... 1.81 ms).
+            const bool reverse = g->cfg.stepSweep == 1 && (launchNo & 1u) != 0;
+            if (reverse) {
+                std::reverse(whole.begin(), whole.end());
+            }
             std::vector<StepDesc> descs;
             uint32_t tiles = 0, nwhole = 0;
             for (std::vector<StepDesc> *v : {&whole, &ragged}) {
@@ -306,9 +315,10 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                 grid = g->numCu;
             }
             pl.rec.grid = std::min(tiles, grid);
-            pl.rec.flags = ordinaryStores ? kStepOrdinaryStores : 0u;
+            pl.rec.flags = (ordinaryStores ? kStepOrdinaryStores : 0u) | (reverse ? kStepReverse : 0u);
             pl.rec.fusedArgs = false;
             pending.push_back(pl);
+            launchNo++;
         }
     } else {
         // Fused results are streamed past the caches (non-temporal stores) unless the caller asks for
@@ -476,7 +486,7 @@ std::string CacheKey(const Group *g, int algo)
         uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1) | (uint64_t(g->ctx->sig.root) << 8) | (uint64_t(g->ctx->sig.peer) << 20), g->cfg.cclBytes, g->cfg.align,
         uint64_t(g->cfg.blocksPerCu) | (uint64_t(uint32_t(g->cfg.stepStores + 1)) << 32) | (uint64_t(g->cfg.servers) << 40) |
             (uint64_t(g->cfg.deterministic) << 56) | (uint64_t(g->cfg.level0Rings) << 57) |
-            (uint64_t(uint32_t(g->cfg.fusedStores + 1)) << 60), g->p};
+            (uint64_t(uint32_t(g->cfg.fusedStores + 1)) << 60) | (uint64_t(g->cfg.stepSweep) << 62), g->p};
     put(head, sizeof(head));
     put(g->ctx->send.data(), g->ctx->send.size() * sizeof(void *));
     put(g->ctx->recv.data(), g->ctx->recv.size() * sizeof(void *));

@@ -57,6 +57,7 @@ constexpr uint32_t kFusedOrdinaryStores = 1u;  // whole passes of the chain kern
 
 // flags of the step kernel
 constexpr uint32_t kStepOrdinaryStores = 1u;   // write-back stores instead of non-temporal ones in the fast loop
+constexpr uint32_t kStepReverse = 2u;          // the fast loop walks every step from its last tile to its first
 
 enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_STACK = 3, KK_COUNT = 4 };
 

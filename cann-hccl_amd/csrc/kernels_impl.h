@@ -390,7 +390,8 @@ __device__ __forceinline__ void StepTileElem(const StepDesc &d, uint64_t off, ui
 // tile still belongs to the current step.  ORDINARY picks the store kind at compile time (a run-time
 // choice per store is folded into one store by the compiler).
 template <typename T, int OP, bool ORDINARY>
-__device__ __forceinline__ void StepWholeTiles(const StepDesc *__restrict__ steps, uint32_t nsteps, uint32_t nwhole, uint32_t ntiles)
+__device__ __forceinline__ void StepWholeTiles(const StepDesc *__restrict__ steps, uint32_t nsteps, uint32_t nwhole, uint32_t ntiles,
+    bool reverse)
 {
     const uint32_t tid = threadIdx.x;
     uint32_t tile = blockIdx.x;
@@ -398,7 +399,8 @@ __device__ __forceinline__ void StepWholeTiles(const StepDesc *__restrict__ step
     StepDesc d = steps[idx];
     uint32_t dEnd = idx + 1 < nsteps ? steps[idx + 1].tile0 : ntiles;   // first tile past this step
     for (;;) {
-        const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
+        // whole tiles only, so walking a step backwards is a matter of the index
+        const uint64_t off = uint64_t(reverse ? dEnd - 1 - tile : tile - d.tile0) * kTileBytes;
         const uint32_t next = tile + gridDim.x;
         const bool reduce = d.b != nullptr;
         V4 va[kVecPerLane], vb[kVecPerLane];
@@ -451,9 +453,9 @@ __global__ void __launch_bounds__(kBlockThreads) StepKernel(const StepDesc *__re
 {
     if (blockIdx.x < nwhole) {
         if (flags & kStepOrdinaryStores) {
-            StepWholeTiles<T, OP, true>(steps, nsteps, nwhole, ntiles);
+            StepWholeTiles<T, OP, true>(steps, nsteps, nwhole, ntiles, (flags & kStepReverse) != 0);
         } else {
-            StepWholeTiles<T, OP, false>(steps, nsteps, nwhole, ntiles);
+            StepWholeTiles<T, OP, false>(steps, nsteps, nwhole, ntiles, (flags & kStepReverse) != 0);
         }
     }
     for (uint32_t tile = nwhole + blockIdx.x; tile < ntiles; tile += gridDim.x) {

@@ -39,6 +39,7 @@ struct GroupConfig {
     uint32_t level0Rings = 0;        // two-level all-reduce inside a group: 0 = mesh, 1 = one ring, 4 = four rings (groups of 8)
     int stepStores = -1;             // step kernel stores: -1 chosen per launch, 0 non-temporal, 1 ordinary
     int fusedStores = 0;             // fused chain kernel stores: 0 non-temporal, 1 ordinary
+    int stepSweep = 1;               // step kernel: 0 every phase walks its steps forwards, 1 every other phase backwards
     uint32_t cacheEntries = 1024;    // prepared collectives kept (distinct sizes / buffers / settings)
     uint32_t blocksPerCu = 0;             // workgroups per CU; 0 = per-kernel default
     bool blockingArrive = false;          // ranks wait inside the call until the collective is issued

@@ -27,6 +27,8 @@ extern "C" {
  *                                the four rings of the 8-device ring topology, each on a quarter of every slice
  *   "step_stores"   "auto" | "nt" | "ordinary"   store kind of the step-by-step kernels (non-temporal, or write-back
  *                                so that the next phase finds the data in the memory-side cache); "auto" decides per collective
+ *   "step_sweep"    "alternate" | "forward"   step-by-step kernels: every other launch walks its data backwards (default),
+ *                                or all walk forwards
  *   "fused_stores"  "nt" | "ordinary"   store kind of the fused chain kernel: non-temporal (default), or write-back, which
  *                                keeps a result of up to 256 MB in the memory-side cache for whoever reads it next
  *   "cache_entries" how many prepared collectives (distinct sizes, buffers, settings) the group keeps (default 1024);

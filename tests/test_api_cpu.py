@@ -238,7 +238,7 @@ def test_amd_params(comms):
     good = {b"algo": [b"ring", b"mesh", b"rhd", b"auto"], b"deterministic": [b"0", b"1"], b"fuse": [b"0", b"1"],
             b"graph": [b"0", b"1"], b"buffsize_mib": [b"1", b"200"], b"buffsize_bytes": [b"4096"], b"align": [b"4", b"128"],
             b"level0": [b"mesh", b"ring", b"ring4"], b"step_stores": [b"auto", b"nt", b"ordinary"],
-            b"fused_stores": [b"nt", b"ordinary"], b"cache_entries": [b"1", b"1024"], b"blocks_per_cu": [b"0", b"2"],
+            b"fused_stores": [b"nt", b"ordinary"], b"step_sweep": [b"forward", b"alternate"], b"cache_entries": [b"1", b"1024"], b"blocks_per_cu": [b"0", b"2"],
             b"blocking_arrive": [b"0", b"1"], b"arrive_timeout_ms": [b"1000"]}
     for key, values in good.items():
         for v in values:
@@ -252,7 +252,7 @@ def test_amd_params(comms):
     assert L.HcclAmdSetParam(comms[0], b"servers", str(p.value).encode()) == 0            # every rank its own group
     assert L.HcclAmdSetParam(comms[0], b"servers", str(p.value + 1).encode()) == H.HCCL_E_PARA   # does not divide the ranks
     for key, v in ((b"algo", b"auto"), (b"servers", b"1"), (b"level0", b"mesh"), (b"fuse", b"1"), (b"graph", b"1"),
-                   (b"deterministic", b"0"), (b"step_stores", b"auto"), (b"fused_stores", b"nt"), (b"blocking_arrive", b"0"),
+                   (b"deterministic", b"0"), (b"step_stores", b"auto"), (b"fused_stores", b"nt"), (b"step_sweep", b"alternate"), (b"blocking_arrive", b"0"),
                    (b"buffsize_mib", b"200"), (b"align", b"128"), (b"blocks_per_cu", b"0"), (b"cache_entries", b"1024")):
         assert L.HcclAmdSetParam(comms[0], key, v) == 0                                   # back to the defaults
 
