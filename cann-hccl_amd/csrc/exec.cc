@@ -451,8 +451,7 @@ HcclResult BuildGraph(Prepared *pp)
     for (LaunchRec &l : pp->launches) {
         void *args[5];
         KernelArgs(l, args);
-        hipKernelNodeParams kp;
-        std::memset(&kp, 0, sizeof(kp));
+        hipKernelNodeParams kp = {};
         kp.func = const_cast<void *>(l.func);
         kp.gridDim = dim3(l.grid, 1, 1);
         kp.blockDim = dim3(kBlockThreads, 1, 1);
