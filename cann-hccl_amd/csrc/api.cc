@@ -197,6 +197,7 @@ Group *NewGroup(uint32_t nRanks)
     g->pend.send.assign(nRanks, nullptr);
     g->pend.recv.assign(nRanks, nullptr);
     g->pend.streams.assign(nRanks, nullptr);
+    g->pend.recorded.assign(nRanks, 0);
     g->ctx = &g->pend;
     char nm[64];
     std::snprintf(nm, sizeof(nm), "hccl_world_group_%p", static_cast<void *>(g));
@@ -313,6 +314,16 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
     g->pend.send[r] = send;
     g->pend.recv[r] = recv;
     g->pend.streams[r] = stream;
+    g->pend.recorded[r] = 0;
+    if (g->cfg.blockingArrive && g->deviceReady && g->arrived + 1 < g->p) {
+        // This rank is going to wait inside its call: it marks its stream now, on its own thread, so that
+        // the rank that issues the collective only has to make its stream wait for the markers.
+        if (hipEventRecord(g->arriveEvents[r], stream) == hipSuccess) {
+            g->pend.recorded[r] = 1;
+        } else {
+            (void)hipGetLastError();
+        }
+    }
     if (sig.coll == COLL_ALLTOALLV) {
         size_t p = g->p;
         g->pend.sendCounts.resize(p * p);
@@ -337,7 +348,16 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
             CancelPending(g, HCCL_E_TIMEOUT);
             return HCCL_E_TIMEOUT;
         }
-        return g->issueResults[serial % 8];
+        const HcclResult res = g->issueResults[serial % 8];
+        // what follows on this rank's stream comes after the collective
+        const bool wait = res == HCCL_SUCCESS && g->doneRecorded[serial % 8] && g->launchStreams[serial % 8] != stream;
+        hipEvent_t doneEvent = g->doneEvent;
+        lock.unlock();
+        if (wait && hipStreamWaitEvent(stream, doneEvent, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            return HCCL_E_RUNTIME;
+        }
+        return res;
     }
     // last arrival
     HcclResult res = HCCL_SUCCESS;
@@ -357,6 +377,7 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
     }
     if (res == HCCL_SUCCESS) {
         g->ctx = &g->pend;
+        g->pend.ranksWaitThemselves = g->cfg.blockingArrive != 0;   // the other ranks are all blocked in their calls
         res = IssueCollective(g, r);
     }
     if (res != HCCL_SUCCESS && res != HCCL_E_PARA) {

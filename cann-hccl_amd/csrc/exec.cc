@@ -833,9 +833,16 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         if (k == launcher || g->ctx->streams[k] == ls) {
             continue;
         }
+        if (k < g->ctx->recorded.size() && g->ctx->recorded[k]) {
+            // the rank put its own marker on its stream when it arrived (it is blocked in its call)
+            HIP_OK(hipStreamWaitEvent(ls, g->arriveEvents[k], 0));
+            others = true;
+            continue;
+        }
         bool seen = false;
         for (uint32_t q = 0; q < k; q++) {
-            seen = seen || (q != launcher && g->ctx->streams[q] == g->ctx->streams[k]);
+            seen = seen || (q != launcher && g->ctx->streams[q] == g->ctx->streams[k] &&
+                !(q < g->ctx->recorded.size() && g->ctx->recorded[q]));
         }
         if (!seen) {
             HIP_OK(hipEventRecord(g->arriveEvents[k], g->ctx->streams[k]));
@@ -859,9 +866,13 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
             HIP_OK(hipLaunchKernel(l.func, dim3(l.grid, 1, 1), dim3(kBlockThreads, 1, 1), args, 0, ls));
         }
     }
+    g->launchStreams[g->opSerial % 8] = ls;
+    g->doneRecorded[g->opSerial % 8] = false;
     if (others) {
         HIP_OK(hipEventRecord(g->doneEvent, ls));
-        for (uint32_t k = 0; k < g->p; k++) {
+        g->doneRecorded[g->opSerial % 8] = true;
+        // ranks blocked in their calls make their own streams wait when they wake up, each on its own thread
+        for (uint32_t k = 0; k < g->p && !g->ctx->ranksWaitThemselves; k++) {
             if (k != launcher && g->ctx->streams[k] != ls) {
                 HIP_OK(hipStreamWaitEvent(g->ctx->streams[k], g->doneEvent, 0));
             }

@@ -115,6 +115,8 @@ struct OpCtx {
     OpSig sig;
     std::vector<void *> send, recv;
     std::vector<hipStream_t> streams;
+    std::vector<uint8_t> recorded;    // per rank: the rank itself put its arrival marker on its stream (it is blocked in its call)
+    bool ranksWaitThemselves = false; // the blocked ranks order their streams after the launch when they wake
     std::vector<uint64_t> sendCounts, sdispls, recvCounts, rdispls;   // p x p (all-to-all-v)
     std::vector<uint64_t> vCounts, vDispls;                           // p (reduce-scatter-v / all-gather-v)
 };
@@ -154,6 +156,8 @@ struct Group {
     // How the most recent rendezvous ended, by serial number modulo the array size: a rank that blocked in
     // rendezvous n reads entry n even if the other ranks have moved on to n + 1 by the time it wakes.
     HcclResult issueResults[8] = {};
+    hipStream_t launchStreams[8] = {};   // same indexing: the stream the collective went to ...
+    bool doneRecorded[8] = {};           // ... and whether the done event was recorded after it for the other streams
     std::vector<uint8_t> here;
     OpCtx pend;                      // what the ranks of the current collective passed
     OpCtx *ctx = nullptr;            // the operation being issued (the rendezvous, or a matched send / receive)

@@ -982,6 +982,45 @@ def test_collectives_recorded_into_a_callers_graph(orc):
             g.close()
 
 
+def test_per_rank_threads_streams_stay_ordered_without_host_syncs(orc):
+    # every rank on its own thread and stream queues: a kernel that writes its send buffer, the all-reduce, a kernel
+    # that reads its receive buffer -- twenty times over without any host synchronisation.  The collective must
+    # come after every rank's producer and before every rank's consumer.
+    import threading
+    p, n, iters = 8, 1 << 16, 20
+    g = gh.Group(p, blocking_arrive=1, arrive_timeout_ms=20000)
+    try:
+        streams = [torch.cuda.Stream() for _ in range(p)]
+        sends = [torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(p)]
+        recvs = [torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(p)]
+        seen = [torch.zeros(iters, n, dtype=torch.float32, device="cuda") for _ in range(p)]
+        torch.cuda.synchronize()
+        codes = [[] for _ in range(p)]
+
+        def work(r):
+            with torch.cuda.stream(streams[r]):
+                for i in range(iters):
+                    sends[r].fill_(float(r + i))
+                    codes[r].append(H.lib().HcclAllReduce(sends[r].data_ptr(), recvs[r].data_ptr(), n, FP32, SUM, g.comms[r],
+                                                          streams[r].cuda_stream))
+                    seen[r][i].copy_(recvs[r])
+
+        ts = [threading.Thread(target=work, args=(r,)) for r in range(p)]
+        for t in ts:
+            t.start()
+        for t in ts:
+            t.join(100)
+        assert not any(t.is_alive() for t in ts)
+        torch.cuda.synchronize()
+        assert all(c == [0] * iters for c in codes), codes
+        for r in range(p):
+            got = seen[r].cpu().numpy()
+            for i in range(iters):
+                assert np.all(got[i] == float(sum(q + i for q in range(p)))), (r, i, got[i][:4])
+    finally:
+        g.close()
+
+
 def test_send_recv_and_batch():
     p, n = 4, 250007
     g = gh.Group(p)
