@@ -109,3 +109,39 @@ def test_rhd_allreduce_bf16_128mib_per_rank(p):
     orc.allreduce(ins, BF16, SUM, algo=orc.RHD, flags=orc.DIRECT | orc.ZERO_STAGING, threads=16, outs=outs)   # clobbers ins
     assert np.array_equal(results[1], outs[0])
     assert np.array_equal(outs[0], outs[p - 1])
+
+
+def test_buffers_larger_than_4_gib():
+    """Two ranks with 5 GiB each: byte offsets inside a buffer go beyond 32 bits.  Integer sum, checked on the GPU
+    against torch's own addition, fused and step by step, plus the all-gather of the same buffers' first GiB."""
+    from closed_forms import INT32
+    p, n = 2, (5 << 30) // 4
+    sends = [torch.arange(n, dtype=torch.int32, device="cuda") * (3 + 4 * r) + r for r in range(p)]
+    want = sends[0] + sends[1]
+    torch.cuda.synchronize()
+    for fuse in (1, 0):
+        g = gh.Group(p, fuse=fuse)
+        try:
+            recvs = [torch.zeros(n, dtype=torch.int32, device="cuda") for _ in range(p)]
+            torch.cuda.synchronize()
+            print("5 GiB per rank all-reduce fuse", fuse, flush=True)
+            H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, INT32, SUM, g.stream_ptr)
+            g.stream.synchronize()
+            for r in range(p):
+                assert torch.equal(recvs[r], want), (fuse, r)
+            del recvs
+        finally:
+            g.close()
+    del want
+    g = gh.Group(p)
+    try:
+        m = (3 << 30) // 4                      # 3 GiB in per rank: the second block of the output starts beyond 2^31 bytes
+        outs = [torch.zeros(m * p, dtype=torch.int32, device="cuda") for _ in range(p)]
+        torch.cuda.synchronize()
+        H.all_gather(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in outs], m, INT32, g.stream_ptr)
+        g.stream.synchronize()
+        for r in range(p):
+            for j in range(p):
+                assert torch.equal(outs[r][j * m:(j + 1) * m], sends[j][:m]), (r, j)
+    finally:
+        g.close()
