@@ -1540,6 +1540,7 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         rq.algo = Algo(uint32_t(algo) & 0xffu);
         rq.servers = std::max(1u, (uint32_t(algo) >> 8) & 0xffu);
         rq.meshAtomic = ((uint32_t(algo) >> 16) & 1u) != 0;
+        rq.level0Rings = (uint32_t(algo) >> 17) & 7u;
     } else {
         rq.algo = Algo(algo);
     }

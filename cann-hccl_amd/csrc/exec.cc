@@ -567,13 +567,15 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
             g->ctx->sig.op != HCCL_REDUCE_PROD;
     }
-    if (rq.coll == COLL_REDUCESCATTER && !g->ctx->sig.variable && g->cfg.servers > 1 && g->p % g->cfg.servers == 0 &&
-        g->cfg.level0Rings == 0) {
-        // two levels (coll_reduce_scatter_mesh_executor.cc:128-247): ring or halving-doubling between the
-        // groups first, then the mesh inside a group, uncut under the conditions of :216-218
+    if (rq.coll == COLL_REDUCESCATTER && !g->ctx->sig.variable && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
+        // two levels (coll_reduce_scatter_mesh_executor.cc:128-247, coll_reduce_scatter_ring_executor.cc:132-340):
+        // ring or halving-doubling between the groups first, then inside a group the mesh (uncut under the
+        // conditions of :216-218) or the ring(s)
         rq.servers = g->cfg.servers;
         rq.algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_RHD;
-        rq.meshAtomic = !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 && g->ctx->sig.op != HCCL_REDUCE_PROD;
+        rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
+        rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
+            g->ctx->sig.op != HCCL_REDUCE_PROD;
     }
     if (rq.coll == COLL_REDUCE && g->cfg.servers > 1 && g->p % g->cfg.servers == 0 && g->cfg.level0Rings == 0) {
         // two levels (coll_reduce_mesh_executor.cc:75-194): mesh inside the groups (uncut under the conditions

@@ -397,8 +397,11 @@ void RhdReduceScatterChunk(VProgram &vp, uint32_t p, const std::vector<Slice> &i
 //            blocks for the ranks of group s (:141-196)
 //   level 0  mesh reduce-scatter inside every group over those D blocks, in place (:198-238)
 //   then the rank's own block goes to the output (:240-243)
-void TwoLevelReduceScatterChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, const std::vector<uint64_t> &blockOff,
-    uint64_t bytes, uint64_t outOff, uint64_t align, bool meshAtomic)
+// With rings inside a group (CollReduceScatterRingExecutor::KernelRun, coll_reduce_scatter_ring_executor.cc:132-340;
+// slices coll_reduce_scatter_executor.cc:250-287) level 0 is the ring schedule over the same D blocks, one ring in
+// rank order or the four rings of the 8-device topology, each on its part of every block.
+void TwoLevelReduceScatterChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, uint32_t level0Rings,
+    const std::vector<uint64_t> &blockOff, uint64_t bytes, uint64_t outOff, uint64_t align, bool meshAtomic)
 {
     const uint32_t D = p / servers;
     size_t l1 = 0;
@@ -427,7 +430,20 @@ void TwoLevelReduceScatterChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t 
             sl[d] = Slice{blockOff[s * D + d], bytes};
         }
         vp.phaseBase = l1;
-        l0 = l1 + MeshReduceScatterPhases(vp, 0, D, 0, sl, align, meshAtomic);
+        if (level0Rings == 0) {
+            l0 = l1 + MeshReduceScatterPhases(vp, 0, D, 0, sl, align, meshAtomic);
+            continue;
+        }
+        std::vector<Slice> cut = RingSlicePlan(bytes, level0Rings, align);   // every block has the same size
+        for (uint32_t k = 0; k < level0Rings; k++) {
+            std::vector<Slice> part(D);
+            for (uint32_t i = 0; i < D; i++) {
+                uint32_t dev = level0Rings > 1 ? kRingOrders8[k][i] : i;
+                vp.rankMap[i] = s * D + dev;
+                part[i] = Slice{blockOff[s * D + dev] + cut[k].off, cut[k].size};
+            }
+            l0 = l1 + RingReduceScatterPhases(vp, 0, D, 0, part, BUF_SEND, 0, part);
+        }
     }
     vp.rankMap.clear();
     vp.phaseBase = 0;
@@ -822,8 +838,8 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                 for (uint32_t i = 0; i < p; i++) {
                     blockOff[i] = in[i].off;
                 }
-                TwoLevelReduceScatterChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, blockOff, bytes, done,
-                    rq.align, rq.meshAtomic);
+                TwoLevelReduceScatterChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, rq.level0Rings, blockOff,
+                    bytes, done, rq.align, rq.meshAtomic);
             } else if (rq.algo == ALGO_RING) {
                 RingReduceScatterPhases(*vp, 0, p, 0, in, BUF_RECV, 0, out);
             } else if (rq.algo == ALGO_RHD) {

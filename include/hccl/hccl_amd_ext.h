@@ -22,8 +22,8 @@ extern "C" {
  *   "align"         slice alignment in bytes (default 128)
  *   "servers"       number of rank groups for all-reduce, reduce-scatter and reduce: with n > 1 the p ranks form n groups of p / n
  *                   consecutive ranks and the two-level schedules run (mesh inside a group, "algo" ring or rhd between)
- *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce: the mesh schedule
- *                                (default), one ring in rank order, or -- for groups of 8 ranks, also with one group --
+ *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter: the mesh schedule
+ *                                (default), one ring in rank order, or -- for groups of 8 ranks, for the all-reduce also with one group --
  *                                the four rings of the 8-device ring topology, each on a quarter of every slice
  *   "step_stores"   "auto" | "nt" | "ordinary"   store kind of the step-by-step kernels (non-temporal, or write-back
  *                                so that the next phase finds the data in the memory-side cache); "auto" decides per collective
@@ -63,7 +63,7 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
  * groups of its two-level schedule in bits 20..27 and bit 28 for the mesh level without the piece cut; for the all-reduce (coll 0) bits 8..15 of algo
  * carry the number of rank groups of the two-level schedule (0 or 1: one level), bit 16 asks for its mesh level
  * without the piece cut and bits 17..19 give the rings inside a group (0: mesh, 1, or 4); the reduce-scatter (coll 1)
- * takes bits 8..16 the same way.  inPlaceMask bit r:
+ * takes bits 8..19 the same way.  inPlaceMask bit r:
  * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64
  * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); for the variable-count
  * reduce-scatter / all-gather, tables points to 2*p uint64 (block counts, block displacements); else NULL.

@@ -209,14 +209,15 @@ def reducescatter(ins, dt, op, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEF
 
 
 def reducescatter_two_level(ins, dt, op, servers, level1=RING, atomic=False, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN,
-                            flags=0, threads=1):
-    """`servers` groups of consecutive ranks: `level1` (RING or RHD) between the groups first, then the mesh inside
-    a group (piece cut, or uncut when `atomic`)."""
+                            flags=0, threads=1, level0="mesh"):
+    """`servers` groups of consecutive ranks: `level1` (RING or RHD) between the groups first, then inside a group
+    `level0`: "mesh" (piece cut, or uncut when `atomic`), "ring" or "ring4"."""
     p = len(ins)
     assert ins[0].size % p == 0
     n = ins[0].size // p
     outs = [np.empty(n, dtype=ins[0].dtype) for _ in range(p)]
-    rc = lib().orc_reducescatter_two_level(level1, 1 if atomic else 0, servers, p, _ptrs(ins), _ptrs(outs), n, dt, op,
+    mode = {"mesh": 1 if atomic else 0, "ring": 2, "ring4": 3}[level0]
+    rc = lib().orc_reducescatter_two_level(level1, mode, servers, p, _ptrs(ins), _ptrs(outs), n, dt, op,
                                            ccl_bytes, align, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle two-level reducescatter failed rc=%d" % rc)

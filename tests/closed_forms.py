@@ -302,7 +302,7 @@ def two_level_ring_allreduce(dt, op, ins, unit, ccl_bytes, align, servers, level
     return [out.copy() for _ in range(p)]
 
 
-def two_level_reducescatter(dt, op, ins, unit, ccl_bytes, align, servers, level1, atomic):
+def two_level_reducescatter(dt, op, ins, unit, ccl_bytes, align, servers, level1, atomic, rings=0):
     """Groups of D = p / servers consecutive ranks.  Block j = s * D + d of every input is first reduced over the
     ranks at one position d' of all groups (level1 "ring": the ring chain for ring slice s; "rhd": the halving
     tree of the block rank that owns slice s), giving one partial per position; the partials are then reduced
@@ -332,6 +332,14 @@ def two_level_reducescatter(dt, op, ins, unit, ccl_bytes, align, servers, level1
                     partial.append(rhd_tree(dt, op, xs, q, block, part1))
             if D == 1:
                 out[base:base + cur] = partial[0]
+            elif rings:
+                # ring(s) inside the group: part k of the block goes round ring k, whose order decides the chain
+                orders = EIGHT_DEVICE_RINGS if rings == 4 else (tuple(range(D)),)
+                for k, (poff, psize) in enumerate(slice_plan(cur * unit, len(orders), align)):
+                    a, b = poff // unit, (poff + psize) // unit
+                    if b > a:
+                        order = orders[k]
+                        out[base + a:base + b] = ring_chain(dt, op, [partial[order[i]][a:b] for i in range(D)], order.index(d))
             elif atomic:
                 out[base:base + cur] = mesh_atomic_chain(dt, op, partial, d)
             else:

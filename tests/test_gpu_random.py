@@ -190,12 +190,14 @@ def test_random_reducescatter_and_reduce_on_rank_groups(orc, seed):
         unit = H.DTYPE_SIZE[dt]
         pad = int(rng.choice([0, 0, unit, 16]))
         atomic = det == 0 and dt != INT64 and op != PROD
-        print("random grouped seed", seed, "case", case, "p", p, "servers", servers, "level1", level1, "deterministic", det, "type", dt,
-              "op", op, "n", n, "fuse", fuse, "root", root, "pad", pad, flush=True)
+        level0 = str(rng.choice(["mesh", "mesh", "ring", "ring4"] if p // servers == 8 else ["mesh", "mesh", "ring"]))
+        print("random grouped seed", seed, "case", case, "p", p, "servers", servers, level0, "level1", level1, "deterministic", det,
+              "type", dt, "op", op, "n", n, "fuse", fuse, "root", root, "pad", pad, flush=True)
         g = gh.Group(p, algo=NAMES[level1], deterministic=det, fuse=fuse, servers=servers)
         try:
             ins = [cf.random_input(dt, n * p, rng) for _ in range(p)]
-            want = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, atomic=atomic)
+            g.set(level0=level0)
+            want = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, atomic=atomic, level0=level0)
             sends = [gh.to_dev(x, pad) for x in ins]
             recvs = [gh.empty_dev(n * unit, pad if r % 2 else 0) for r in range(p)]
             torch.cuda.synchronize()
@@ -204,6 +206,7 @@ def test_random_reducescatter_and_reduce_on_rank_groups(orc, seed):
             for r in range(p):
                 assert gh.same(dt, gh.to_host(recvs[r], dt), want[r]), (seed, case, "reduce-scatter", r)
                 assert np.array_equal(gh.to_host(sends[r], dt), ins[r]), (seed, case, "send buffer changed", r)
+            g.set(level0="mesh")            # the rooted reduce is two-level with the mesh inside a group only
             want_root = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, atomic=atomic)
             outs = [gh.empty_dev(n * p * unit, 0 if r % 2 else pad, fill=0x33) for r in range(p)]
             torch.cuda.synchronize()

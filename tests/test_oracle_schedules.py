@@ -420,3 +420,20 @@ def test_two_level_reduce_to_root_matches_closed_form(orc, level1, atomic):
     a = orc.reduce_to_root_two_level(ins, FP32, SUM, 3, 1, level1=level1, atomic=atomic)
     b = orc.reduce_to_root(ins, FP32, SUM, 3, algo=MESH_ATOMIC if atomic else MESH)
     assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("level0", ["ring", "ring4"])
+def test_two_level_reducescatter_with_rings_inside_a_server_matches_closed_form(orc, level1, level0):
+    rings = 4 if level0 == "ring4" else 1
+    shapes = ((2, 8), (3, 8), (1, 8)) if rings == 4 else ((2, 4), (4, 2), (3, 4), (5, 3), (1, 6))
+    for servers, D in shapes:
+        p = servers * D
+        for dt, op, n, ccl in ((FP32, SUM, 211, 200 << 20), (FP32, SUM, 500, 4 * p * 128), (BF16, SUM, 301, 200 << 20),
+                               (INT32, MAX, 70, 200 << 20)):
+            ins = _inputs(dt, p, n * p, 47 * p + n)
+            got = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, level0=level0, ccl_bytes=ccl)
+            want = cf.two_level_reducescatter(dt, op, ins, orc.dtype_size(dt), ccl, 128, servers,
+                                              "ring" if level1 == RING else "rhd", False, rings=rings)
+            for r in range(p):
+                assert _eq(dt, got[r], want[r]), (servers, D, level1, level0, dt, ccl, r)

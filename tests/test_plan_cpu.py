@@ -447,3 +447,24 @@ def test_two_level_reduce_plan_matches_checker(orc, level1, shape):
                         assert np.array_equal(sends[r], ins[r].view(np.uint8))
                         if r != root:
                             assert np.all(recvs[r] == 0x77)              # only the root's output is written
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("level0", ["ring", "ring4"])
+def test_two_level_reducescatter_with_rings_inside_a_group_matches_checker(orc, level1, level0):
+    rings = 4 if level0 == "ring4" else 1
+    shapes = ((2, 8), (3, 8)) if rings == 4 else ((2, 4), (4, 2), (3, 4), (5, 3))
+    for servers, D in shapes:
+        p = servers * D
+        for dt, op, n, ccl in ((FP32, SUM, 211, 200 << 20), (FP32, SUM, 500, 4 * p * 128), (BF16, PROD, 77, 200 << 20)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n * p, 800 + p + n)
+            want = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, level0=level0, ccl_bytes=ccl)
+            plan = H.describe_plan(H.COLL_REDUCESCATTER, level1 | (servers << 8) | (rings << 17), p, n, dt, ccl_bytes=ccl)
+            assert plan["fusedOk"]
+            for fused in (False, True):
+                sends = _bytes(ins)
+                recvs = [np.full(n * unit, 0x5A, np.uint8) for _ in range(p)]
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+                for r in range(p):
+                    assert _same(dt, recvs[r], want[r]), (servers, D, level1, level0, dt, ccl, fused, r)

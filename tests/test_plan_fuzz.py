@@ -23,7 +23,7 @@ def _case(rng):
     if coll in (H.COLL_ALLREDUCE, H.COLL_REDUCESCATTER, H.COLL_REDUCE) and rng.random() < 0.4:
         servers = int(rng.choice([s for s in range(1, p + 1) if p % s == 0]))
         algo = int(rng.choice([RING, RHD]))
-        if coll == H.COLL_ALLREDUCE and rng.random() < 0.4:
+        if coll in (H.COLL_ALLREDUCE, H.COLL_REDUCESCATTER) and rng.random() < 0.4 and (coll == H.COLL_ALLREDUCE or servers > 1):
             rings = 4 if p // servers == 8 and rng.random() < 0.6 else 1
     mask = 0
     if coll == H.COLL_ALLREDUCE and rng.random() < 0.5:
@@ -42,7 +42,7 @@ def test_random_plans_compute_the_plain_result(seed):
         if coll == H.COLL_ALLREDUCE:
             word = algo | (servers << 8) | (rings << 17) if (servers > 1 or rings) else algo
         elif coll == H.COLL_REDUCESCATTER:
-            word = algo | (servers << 8) if servers > 1 else algo
+            word = algo | (servers << 8) | (rings << 17) if servers > 1 else algo
         elif coll == H.COLL_ALLGATHER:
             word = algo
         elif coll == H.COLL_REDUCE and servers > 1:
