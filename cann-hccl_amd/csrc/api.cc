@@ -1522,12 +1522,14 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
     rq.coll = CollKind(coll);
     if (coll >= COLL_BROADCAST) {
         // rooted collectives: low 16 bits = root rank, bits 16..19 = schedule (0 ring, 1 mesh, 2 rhd, 4 mesh uncut);
-        // reduce only: bits 20..27 = number of rank groups of the two-level schedule, bit 28 = its mesh level uncut
+        // reduce only: bits 20..27 = number of rank groups of the two-level schedule, bit 28 = its mesh level uncut,
+        // bit 29 / bit 30 = one ring / four rings inside a group instead of the mesh
         rq.root = uint32_t(algo) & 0xffffu;
         rq.algo = Algo((uint32_t(algo) >> 16) & 0xfu);
         if (coll == COLL_REDUCE) {
             rq.servers = std::max(1u, (uint32_t(algo) >> 20) & 0xffu);
             rq.meshAtomic = ((uint32_t(algo) >> 28) & 1u) != 0;
+            rq.level0Rings = ((uint32_t(algo) >> 29) & 1u) ? 1u : (((uint32_t(algo) >> 30) & 1u) ? 4u : 0u);   // bit 29 one ring, bit 30 four
         }
     } else if (coll == COLL_ALLREDUCE) {
         // all-reduce: low 8 bits = schedule, bits 8..15 = number of rank groups ("servers") of a two-level schedule

@@ -577,12 +577,15 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
             g->ctx->sig.op != HCCL_REDUCE_PROD;
     }
-    if (rq.coll == COLL_REDUCE && g->cfg.servers > 1 && g->p % g->cfg.servers == 0 && g->cfg.level0Rings == 0) {
-        // two levels (coll_reduce_mesh_executor.cc:75-194): mesh inside the groups (uncut under the conditions
-        // of :93-97), then ring or halving-doubling towards the root's group (:133-139)
+    if (rq.coll == COLL_REDUCE && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
+        // two levels (coll_reduce_mesh_executor.cc:75-194, coll_reduce_ring_plus_hd_executor.cc:75-168): inside the
+        // groups the mesh (uncut under the conditions of :93-97) or the ring(s), then ring or halving-doubling
+        // towards the root's group (:133-139)
         rq.servers = g->cfg.servers;
         rq.algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_RHD;
-        rq.meshAtomic = !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 && g->ctx->sig.op != HCCL_REDUCE_PROD;
+        rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
+        rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
+            g->ctx->sig.op != HCCL_REDUCE_PROD;
     }
     if (g->ctx->sig.variable) {
         rq.vCounts = g->ctx->vCounts;

@@ -538,8 +538,11 @@ size_t RhdReducePhases(VProgram &vp, uint32_t n, uint32_t root, uint64_t off, ui
 // in the root's group, ring or recursive halving-doubling (:109-160), and the root gathers the
 // slices inside its group (:164-187).  The level-1 results are written straight to the root's
 // output, which is where the gather would carry them.
-void TwoLevelReduceChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, uint32_t root, uint64_t base, uint64_t bytes,
-    uint64_t align, bool meshAtomic)
+// With rings inside a group (CollReduceRingPlusHdExecutor::KernelRun, coll_reduce_ring_plus_hd_executor.cc:75-168)
+// level 0 is the ring reduce-scatter of the two-level all-reduce, one ring or the four rings of the
+// 8-device topology on the parts of every slice; the rest is the same.
+void TwoLevelReduceChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, uint32_t level0Rings, uint32_t root,
+    uint64_t base, uint64_t bytes, uint64_t align, bool meshAtomic)
 {
     const uint32_t D = p / servers;
     const uint32_t rootServer = root / D;
@@ -547,11 +550,24 @@ void TwoLevelReduceChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers
     const size_t l1 = D > 1 ? D - 1 : 0;
     for (uint32_t s = 0; s < servers && D > 1; s++) {
         vp.rankMap.resize(D);
-        for (uint32_t d = 0; d < D; d++) {
-            vp.rankMap[d] = s * D + d;
-        }
         vp.phaseBase = 0;
-        MeshReduceScatterPhases(vp, 0, D, base, sl, align, meshAtomic);
+        if (level0Rings == 0) {
+            for (uint32_t d = 0; d < D; d++) {
+                vp.rankMap[d] = s * D + d;
+            }
+            MeshReduceScatterPhases(vp, 0, D, base, sl, align, meshAtomic);
+            continue;
+        }
+        for (uint32_t k = 0; k < level0Rings; k++) {
+            std::vector<Slice> part(D);
+            for (uint32_t i = 0; i < D; i++) {
+                uint32_t dev = level0Rings > 1 ? kRingOrders8[k][i] : i;
+                vp.rankMap[i] = s * D + dev;
+                std::vector<Slice> cut = RingSlicePlan(sl[dev].size, level0Rings, align);
+                part[i] = Slice{sl[dev].off + cut[k].off, cut[k].size};
+            }
+            RingReduceScatterPhases(vp, 0, D, base, part, BUF_SEND, base, part);
+        }
     }
     for (uint32_t d = 0; d < D; d++) {
         // local ranks 0 .. servers-1 are the groups' ranks at position d; one more entry names the root
@@ -699,8 +715,8 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                     EmitCopy(*vp, ph, data(rankOf[b] ^ 1u), data(rankOf[b]), bytes);
                 }
             } else if (rq.coll == COLL_REDUCE && rq.servers > 1 && p > 1) {
-                TwoLevelReduceChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, R, done, bytes, rq.align,
-                    rq.meshAtomic);
+                TwoLevelReduceChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, rq.level0Rings, R, done, bytes,
+                    rq.align, rq.meshAtomic);
             } else if (rq.coll == COLL_REDUCE && rq.algo == ALGO_MESH && p > 1) {
                 // mesh reduce (coll_reduce_mesh_executor.cc:75-194): mesh reduce-scatter over the ring
                 // slice plan, then the root gathers slice r from rank r (gather_mesh.cc:60-170)

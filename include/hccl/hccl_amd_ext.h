@@ -22,7 +22,7 @@ extern "C" {
  *   "align"         slice alignment in bytes (default 128)
  *   "servers"       number of rank groups for all-reduce, reduce-scatter and reduce: with n > 1 the p ranks form n groups of p / n
  *                   consecutive ranks and the two-level schedules run (mesh inside a group, "algo" ring or rhd between)
- *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter: the mesh schedule
+ *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter / reduce: the mesh schedule
  *                                (default), one ring in rank order, or -- for groups of 8 ranks, for the all-reduce also with one group --
  *                                the four rings of the 8-device ring topology, each on a quarter of every slice
  *   "step_stores"   "auto" | "nt" | "ordinary"   store kind of the step-by-step kernels (non-temporal, or write-back
@@ -60,7 +60,8 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
  * fused items, byte counts) into out[0..cap).  coll / algo as in HcclAmdOpInfo; for the rooted
  * collectives (coll 4 broadcast, 5 reduce, 6 scatter) the algo argument carries the root rank in its low 16 bits and the
  * schedule in bits 16..19 (0 ring, 1 mesh, 2 rhd, 4 mesh without the piece cut), for the reduce also the number of rank
- * groups of its two-level schedule in bits 20..27 and bit 28 for the mesh level without the piece cut; for the all-reduce (coll 0) bits 8..15 of algo
+ * groups of its two-level schedule in bits 20..27, bit 28 for the mesh level without the piece cut and bit 29 / bit 30 for
+ * one ring / four rings inside a group; for the all-reduce (coll 0) bits 8..15 of algo
  * carry the number of rank groups of the two-level schedule (0 or 1: one level), bit 16 asks for its mesh level
  * without the piece cut and bits 17..19 give the rings inside a group (0: mesh, 1, or 4); the reduce-scatter (coll 1)
  * takes bits 8..19 the same way.  inPlaceMask bit r:

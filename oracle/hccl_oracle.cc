@@ -2148,16 +2148,20 @@ int orc_reduce_to_root_mesh(uint32_t p, void **in, void *outRoot, uint64_t count
 
 // Two-level reduce, CollReduceMeshExecutor::KernelRun with several servers
 // (EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194): `servers` groups of D = p / servers consecutive ranks.
-// Mesh reduce-scatter inside every group over the ring slice plan for D (piece cut, or uncut when `atomic`); the
+// Reduce-scatter inside every group over the ring slice plan for D (level0 0 / 1: mesh with the piece cut / uncut;
+// 2 / 3: one ring / the four rings of the 8-device topology, EXE/coll_reduce/coll_reduce_ring_plus_hd_executor.cc:75-168); the
 // ranks at position d of all groups reduce slice d to the one in the root's group (level1 = ALGO_RING or ALGO_RHD,
 // input range to output range; a copy when there is one group); GatherMesh to the root inside its group.
-int orc_reduce_to_root_two_level(int level1, int atomic, uint32_t servers, uint32_t p, void **in, void *outRoot, uint64_t count,
+int orc_reduce_to_root_two_level(int level1, int level0, uint32_t servers, uint32_t p, void **in, void *outRoot, uint64_t count,
     int dt, int op, uint32_t root, uint64_t cclBytes, uint64_t align, int flags, int threads)
 {
     uint64_t unit = DtSize(dt);
-    if (unit == 0 || p == 0 || root >= p || servers == 0 || p % servers != 0 || (level1 != ALGO_RING && level1 != ALGO_RHD)) {
+    if (unit == 0 || p == 0 || root >= p || servers == 0 || p % servers != 0 || (level1 != ALGO_RING && level1 != ALGO_RHD) ||
+        level0 < 0 || level0 > 3 || (level0 == 3 && p / servers != 8)) {
         return -20;
     }
+    const bool atomic = level0 == 1;
+    const uint32_t ringCount = level0 == 3 ? 4u : 1u;
     uint64_t maxPer = cclBytes / unit;
     if (maxPer == 0) {
         return -21;
@@ -2196,6 +2200,32 @@ int orc_reduce_to_root_two_level(int level1, int atomic, uint32_t servers, uint3
             for (uint32_t d = 0; d < D; d++) {
                 m.buf[B_IN][d] = all.buf[B_IN][s * D + d];
                 m.buf[B_OUT][d] = all.buf[B_OUT][s * D + d];
+            }
+            if (level0 >= 2) {
+                // CollReduceRingPlusHdExecutor::KernelRun (EXE/coll_reduce/coll_reduce_ring_plus_hd_executor.cc:75-105):
+                // the ring reduce-scatter of the two-level all-reduce, one sub-machine per ring
+                std::vector<std::vector<Slice>> segs = MultiSegSlices(sl, ringCount, align);
+                for (uint32_t k = 0; k < ringCount; k++) {
+                    Machine ring = machine(D);
+                    std::vector<Slice> ringSl(D);
+                    for (uint32_t i = 0; i < D; i++) {
+                        uint32_t dev = ringCount > 1 ? kEightDeviceRings[k][i] : i;
+                        ring.buf[B_IN][i] = m.buf[B_IN][dev];
+                        ring.buf[B_OUT][i] = m.buf[B_OUT][dev];
+                        ringSl[i] = segs[dev][k];
+                    }
+                    for (uint32_t i = 0; i < D; i++) {
+                        Proc pr;
+                        pr.rank = i;
+                        ProgReduceScatterRing(pr.prog, i, D, B_IN, B_IN, ringSl, ringSl);
+                        ring.procs.push_back(std::move(pr));
+                    }
+                    int rc = ring.Run();
+                    if (rc != 0) {
+                        return rc;
+                    }
+                }
+                continue;
             }
             if (atomic) {
                 for (uint32_t d = 0; d < D; d++) {

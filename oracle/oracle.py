@@ -285,11 +285,12 @@ def reduce_to_root(ins, dt, op, root, ccl_bytes=DEFAULT_CCL_BYTES, flags=0, thre
 
 
 def reduce_to_root_two_level(ins, dt, op, root, servers, level1=RING, atomic=False, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN,
-                             flags=0, threads=1):
+                             flags=0, threads=1, level0="mesh"):
     """`servers` groups of consecutive ranks: mesh reduce-scatter inside a group (piece cut, or uncut when `atomic`),
     `level1` (RING or RHD) reduce of every slice towards the root's group, gather to the root inside its group."""
     out = np.empty_like(ins[0])
-    rc = lib().orc_reduce_to_root_two_level(level1, 1 if atomic else 0, servers, len(ins), _ptrs(ins), out.ctypes.data, ins[0].size,
+    mode = {"mesh": 1 if atomic else 0, "ring": 2, "ring4": 3}[level0]
+    rc = lib().orc_reduce_to_root_two_level(level1, mode, servers, len(ins), _ptrs(ins), out.ctypes.data, ins[0].size,
                                             dt, op, root, ccl_bytes, align, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle two-level reduce failed rc=%d" % rc)

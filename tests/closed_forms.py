@@ -353,7 +353,7 @@ def two_level_reducescatter(dt, op, ins, unit, ccl_bytes, align, servers, level1
     return outs
 
 
-def two_level_reduce_to_root(dt, op, ins, unit, ccl_bytes, align, servers, level1, atomic, root):
+def two_level_reduce_to_root(dt, op, ins, unit, ccl_bytes, align, servers, level1, atomic, root, rings=0):
     """Groups of D = p / servers consecutive ranks: the mesh chain inside every group for slice d (per piece when the
     slice is cut), then the groups' partial results of that slice reduced towards the root's group: level1 "ring" is
     the ring chain ending at that group, "rhd" the halving-doubling reduce tree."""
@@ -375,6 +375,15 @@ def two_level_reduce_to_root(dt, op, ins, unit, ccl_bytes, align, servers, level
                 xs = [x[lo:hi] for x in ins[s * D:(s + 1) * D]]
                 if D == 1:
                     partial.append(xs[0].copy())
+                elif rings:
+                    orders = EIGHT_DEVICE_RINGS if rings == 4 else (tuple(range(D)),)
+                    acc = np.empty_like(xs[0])
+                    for k, (poff, psize) in enumerate(slice_plan(size, len(orders), align)):
+                        a, b = poff // unit, (poff + psize) // unit
+                        if b > a:
+                            order = orders[k]
+                            acc[a:b] = ring_chain(dt, op, [xs[order[i]][a:b] for i in range(D)], order.index(d))
+                    partial.append(acc)
                 elif atomic:
                     partial.append(mesh_atomic_chain(dt, op, xs, d))
                 else:

@@ -206,8 +206,7 @@ def test_random_reducescatter_and_reduce_on_rank_groups(orc, seed):
             for r in range(p):
                 assert gh.same(dt, gh.to_host(recvs[r], dt), want[r]), (seed, case, "reduce-scatter", r)
                 assert np.array_equal(gh.to_host(sends[r], dt), ins[r]), (seed, case, "send buffer changed", r)
-            g.set(level0="mesh")            # the rooted reduce is two-level with the mesh inside a group only
-            want_root = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, atomic=atomic)
+            want_root = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, atomic=atomic, level0=level0)
             outs = [gh.empty_dev(n * p * unit, 0 if r % 2 else pad, fill=0x33) for r in range(p)]
             torch.cuda.synchronize()
             H.reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in outs], n * p, dt, op, root, g.stream_ptr)

@@ -437,3 +437,19 @@ def test_two_level_reducescatter_with_rings_inside_a_server_matches_closed_form(
                                               "ring" if level1 == RING else "rhd", False, rings=rings)
             for r in range(p):
                 assert _eq(dt, got[r], want[r]), (servers, D, level1, level0, dt, ccl, r)
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("level0", ["ring", "ring4"])
+def test_two_level_reduce_to_root_with_rings_inside_a_server_matches_closed_form(orc, level1, level0):
+    rings = 4 if level0 == "ring4" else 1
+    shapes = ((2, 8), (3, 8), (1, 8)) if rings == 4 else ((2, 4), (4, 2), (3, 4), (5, 3))
+    for servers, D in shapes:
+        p = servers * D
+        for dt, op, n, ccl in ((FP32, SUM, 2003, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, SUM, 1501, 200 << 20)):
+            ins = _inputs(dt, p, n, 53 * p + n)
+            for root in sorted({0, p - 1, (D + 1) % p}):
+                got = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, level0=level0, ccl_bytes=ccl)
+                want = cf.two_level_reduce_to_root(dt, op, ins, orc.dtype_size(dt), ccl, 128, servers,
+                                                   "ring" if level1 == RING else "rhd", False, root, rings=rings)
+                assert _eq(dt, got, want), (servers, D, level1, level0, dt, ccl, root)

@@ -468,3 +468,28 @@ def test_two_level_reducescatter_with_rings_inside_a_group_matches_checker(orc, 
                 (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
                 for r in range(p):
                     assert _same(dt, recvs[r], want[r]), (servers, D, level1, level0, dt, ccl, fused, r)
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("level0", ["ring", "ring4"])
+def test_two_level_reduce_with_rings_inside_a_group_matches_checker(orc, level1, level0):
+    rings = 4 if level0 == "ring4" else 1
+    shapes = ((2, 8), (3, 8)) if rings == 4 else ((2, 4), (4, 2), (3, 4), (5, 3))
+    for servers, D in shapes:
+        p = servers * D
+        for dt, op, n, ccl in ((FP32, SUM, 2003, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, PROD, 777, 200 << 20)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n, 900 + p + n)
+            for root in sorted({0, p - 1, (D + 1) % p}):
+                want = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, level0=level0, ccl_bytes=ccl)
+                word = root | (level1 << 16) | (servers << 20) | ((1 << 29) if rings == 1 else (1 << 30))
+                plan = H.describe_plan(H.COLL_REDUCE, word, p, n, dt, ccl_bytes=ccl)
+                assert plan["fusedOk"]
+                for fused in (False, True):
+                    sends = _bytes(ins)
+                    recvs = [np.full(n * unit, 0x77, np.uint8) for _ in range(p)]
+                    (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+                    assert _same(dt, recvs[root], want), (servers, D, level1, level0, dt, ccl, root, fused)
+                    for r in range(p):
+                        if r != root:
+                            assert np.all(recvs[r] == 0x77)
