@@ -549,6 +549,26 @@ def test_order_sensitive_known_answers_on_the_gpu():
                 g.close()
 
 
+def test_order_sensitive_known_answers_two_level_on_the_gpu():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_fp32.json")) as f:
+        kat = json.load(f)
+    xs = [np.array(v, np.float32) for v in kat["inputs"]]
+    want = kat["expected_two_level_2x2"]
+    for level1 in (RING, RHD):
+        for level0 in ("mesh", "ring"):
+            for fuse in (1, 0):
+                g = gh.Group(4, algo=ALGO_NAME[level1], servers=2, level0=level0, fuse=fuse, align=kat["align"])
+                try:
+                    outs, _ = gh.all_reduce(g, xs, FP32, SUM)
+                    assert all(float(o[0]) == want["allreduce_element0"] for o in outs), (level1, level0, fuse)
+                    rs, _ = gh.reduce_scatter(g, xs, FP32, SUM)
+                    assert float(rs[0][0]) == want["reducescatter_rank0"], (level1, level0, fuse)
+                finally:
+                    g.close()
+
+
 def test_broadcast_and_reduce_mesh_and_rhd_schedules(orc):
     n = 70001
     for p in (3, 8, 6):

@@ -453,3 +453,21 @@ def test_two_level_reduce_to_root_with_rings_inside_a_server_matches_closed_form
                 want = cf.two_level_reduce_to_root(dt, op, ins, orc.dtype_size(dt), ccl, 128, servers,
                                                    "ring" if level1 == RING else "rhd", False, root, rings=rings)
                 assert _eq(dt, got, want), (servers, D, level1, level0, dt, ccl, root)
+
+
+def test_order_sensitive_known_answers_two_level(orc):
+    # the same hand-derived input on two groups of two ranks: a fifth sum for the all-reduce, and the reduce-scatter's
+    # groups-first order
+    kat = _order_kat()
+    xs = [np.array(v, np.float32) for v in kat["inputs"]]
+    want = kat["expected_two_level_2x2"]
+    for level1 in (RING, RHD):
+        for level0, atomic in (("mesh", False), ("mesh", True), ("ring", False)):
+            got = orc.allreduce_two_level([x.copy() for x in xs], FP32, SUM, 2, level1=level1, atomic=atomic, align=kat["align"],
+                                          level0=level0)
+            assert all(float(g[0]) == want["allreduce_element0"] for g in got), (level1, level0, atomic)
+            rs = orc.reducescatter_two_level([x.copy() for x in xs], FP32, SUM, 2, level1=level1, atomic=atomic, align=kat["align"],
+                                             level0=level0)
+            assert float(rs[0][0]) == want["reducescatter_rank0"], (level1, level0, atomic)
+    closed = cf.two_level_allreduce(FP32, SUM, xs, 4, 200 << 20, kat["align"], 2, cf.ring_allreduce, False)
+    assert float(closed[0][0]) == want["allreduce_element0"]
