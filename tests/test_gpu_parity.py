@@ -569,6 +569,33 @@ def test_order_sensitive_known_answers_two_level_on_the_gpu():
                     g.close()
 
 
+def test_four_ring_known_answers_on_the_gpu():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_four_rings_fp32.json")) as f:
+        kat = json.load(f)
+    p, n = kat["ranks"], kat["elements"]
+    xs = []
+    for row in kat["inputs_first4"]:
+        x = np.zeros(n, np.float32)
+        x[:4] = row
+        xs.append(x)
+    for level0 in ("ring4", "ring"):
+        want = np.zeros(n, np.float32)
+        want[:4] = kat["expected_first4"][level0]
+        # one group and one ring is the plain ring schedule, whatever the upper level would be
+        for level1 in ((RING, RHD) if level0 == "ring4" else (RING,)):
+            for fuse in (1, 0):
+                g = gh.Group(p, algo=ALGO_NAME[level1], servers=1, level0=level0, fuse=fuse, align=kat["align"])
+                try:
+                    print("four-ring KAT", level0, level1, "fuse", fuse, flush=True)
+                    outs, _ = gh.all_reduce(g, xs, FP32, SUM)
+                    for r in range(p):
+                        assert np.array_equal(outs[r], want), (level0, level1, fuse, r, outs[r][:4])
+                finally:
+                    g.close()
+
+
 def test_broadcast_and_reduce_mesh_and_rhd_schedules(orc):
     n = 70001
     for p in (3, 8, 6):

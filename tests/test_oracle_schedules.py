@@ -471,3 +471,30 @@ def test_order_sensitive_known_answers_two_level(orc):
             assert float(rs[0][0]) == want["reducescatter_rank0"], (level1, level0, atomic)
     closed = cf.two_level_allreduce(FP32, SUM, xs, 4, 200 << 20, kat["align"], 2, cf.ring_allreduce, False)
     assert float(closed[0][0]) == want["allreduce_element0"]
+
+
+def _four_ring_kat():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_four_rings_fp32.json")) as f:
+        kat = json.load(f)
+    xs = []
+    for row in kat["inputs_first4"]:
+        x = np.zeros(kat["elements"], np.float32)
+        x[:4] = row
+        xs.append(x)
+    return kat, xs
+
+
+def test_order_sensitive_known_answers_four_rings(orc):
+    # hand-derived: each of the first four elements travels its own ring, and only that ring's order loses the 1
+    kat, xs = _four_ring_kat()
+    assert [list(o) for o in cf.EIGHT_DEVICE_RINGS] == kat["ring_orders"]
+    for level0 in ("ring4", "ring"):
+        want = np.zeros(kat["elements"], np.float32)
+        want[:4] = kat["expected_first4"][level0]
+        for level1 in (RING, RHD):
+            got = orc.allreduce_two_level([x.copy() for x in xs], FP32, SUM, 1, level1=level1, align=kat["align"], level0=level0)
+            assert all(np.array_equal(g, want) for g in got), (level0, level1, got[0][:4])
+    closed = cf.two_level_ring_allreduce(FP32, SUM, xs, 4, 200 << 20, kat["align"], 1, cf.ring_allreduce, 4)
+    assert np.array_equal(closed[0][:4], np.array(kat["expected_first4"]["ring4"], np.float32))

@@ -284,6 +284,32 @@ def test_order_sensitive_known_answers_through_the_planner():
                 assert float(recvs[r].view(np.float32)[0]) == kat["expected_element0"][name], (name, fused, r)
 
 
+def test_four_ring_known_answers_through_the_planner():
+    # hand-derived sums of tests/golden/order_sensitive_four_rings_fp32.json: each of the first four elements takes
+    # its own ring of the 8-device topology, and a single ring gives different bits
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_four_rings_fp32.json")) as f:
+        kat = json.load(f)
+    p, n = kat["ranks"], kat["elements"]
+    xs = []
+    for row in kat["inputs_first4"]:
+        x = np.zeros(n, np.float32)
+        x[:4] = row
+        xs.append(x)
+    for name, rings in (("ring4", 4), ("ring", 1)):
+        want = np.zeros(n, np.float32)
+        want[:4] = kat["expected_first4"][name]
+        for level1 in (RING, RHD):
+            plan = H.describe_plan(H.COLL_ALLREDUCE, level1 | (1 << 8) | (rings << 17), p, n, FP32, align=kat["align"])
+            for fused in (False, True):
+                sends = _bytes(xs)
+                recvs = [np.full(n * 4, 0xA5, np.uint8) for _ in range(p)]
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, FP32, SUM)
+                for r in range(p):
+                    assert np.array_equal(recvs[r].view(np.float32), want), (name, level1, fused, r)
+
+
 @pytest.mark.parametrize("p", [2, 3, 4, 5, 6, 7, 8, 12, 13, 24])
 def test_reduce_rhd_plan_matches_checker_and_tree(orc, p):
     n = 1003
