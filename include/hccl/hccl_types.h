@@ -17,8 +17,10 @@ extern "C" {
 typedef void *HcclComm;
 
 /* ---- element types and operators (reference :58-87) ------------------------------------------ */
-/* Sizes in bytes, in enumerator order: 1 2 4 2 4 8 8 1 2 4 8 2 16 1 1 1.  The three 8-bit float
- * formats and INT128 are accepted for data movement only. */
+/* Sizes in bytes, in enumerator order: 1 2 4 2 4 8 8 1 2 4 8 2 16 1 1 1.  INT128 is accepted for data
+ * movement only.  The three 8-bit float formats are named here and refused by every collective with
+ * HCCL_E_NOT_SUPPORT, as by the reference (its accepted set:
+ * src/domain/collective_communication/framework/common/src/param_check.cc:22-36). */
 typedef enum {
     HCCL_DATA_TYPE_INT8 = 0,    HCCL_DATA_TYPE_INT16 = 1,   HCCL_DATA_TYPE_INT32 = 2,    HCCL_DATA_TYPE_FP16 = 3,
     HCCL_DATA_TYPE_FP32 = 4,    HCCL_DATA_TYPE_INT64 = 5,   HCCL_DATA_TYPE_UINT64 = 6,   HCCL_DATA_TYPE_UINT8 = 7,
