@@ -234,6 +234,17 @@ def run_suite(pkg, torch, steps, warmup, only="", settings=()):
                 report("broadcast %s p=8 256MiB root 3" % ralgo, comms,
                        lambda: pkg.broadcast(comms, rp, n, FP32, 3, stream.cuda_stream))
         pkg.comm_destroy(comms)
+    # in place (send buffer == receive buffer on every rank).  max rather than sum: replays feed on their own
+    # output, which a sum would drive to infinity; after the first call the buffers hold full-entropy data
+    comms = pkg.comm_init_all(p)
+    for r in range(p):
+        recvs[r].copy_(sends[r])
+    torch.cuda.synchronize()
+    report("all-reduce ring p=8 fp32 max 256MiB/rank in place", comms,
+           lambda: pkg.all_reduce(comms, rp, rp, n, FP32, 2, stream.cuda_stream))
+    report("all-reduce ring p=8 fp32 max 256MiB/rank out of place", comms,
+           lambda: pkg.all_reduce(comms, sp, rp, n, FP32, 2, stream.cuda_stream))
+    pkg.comm_destroy(comms)
     for servers, level0, level1 in ((2, "mesh", "ring"), (2, "mesh", "rhd"), (4, "mesh", "rhd"), (2, "ring", "rhd"), (1, "ring4", "rhd")):
         comms = pkg.comm_init_all(p)
         pkg.set_param(comms[0], "servers", servers)
