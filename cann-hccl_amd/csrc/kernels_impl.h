@@ -540,10 +540,20 @@ __device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *con
                     }
                 } else {
                     const bool accLeft = OrderMatters<T, OP>::value && ((d.accLeftMask >> (j + jj)) & 1ull);
+                    // the flag is the same for the whole wave: a branch, not both results and a select per element
+                    if (accLeft) {
 #pragma unroll
-                    for (uint32_t u = 0; u < kChainVec; u++) {
-                        if (live[u]) {
-                            acc[u] = accLeft ? Combine16<T, OP>(acc[u], v[jj][u]) : Combine16<T, OP>(v[jj][u], acc[u]);
+                        for (uint32_t u = 0; u < kChainVec; u++) {
+                            if (live[u]) {
+                                acc[u] = Combine16<T, OP>(acc[u], v[jj][u]);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (uint32_t u = 0; u < kChainVec; u++) {
+                            if (live[u]) {
+                                acc[u] = Combine16<T, OP>(v[jj][u], acc[u]);
+                            }
                         }
                     }
                 }
@@ -957,10 +967,19 @@ __device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *con
                     StackVal<U> under;
                     HCCL_STACK_GET(depth - 2, under)
                     const bool underLeft = !OrderMatters<T, OP>::value || ((op >> (8 + f)) & 1u);
+                    if (underLeft) {           // the same for the whole wave
 #pragma unroll
-                    for (uint32_t u = 0; u < U; u++) {
-                        if (live[u]) {
-                            top.x[u] = underLeft ? Combine16<T, OP>(under.x[u], top.x[u]) : Combine16<T, OP>(top.x[u], under.x[u]);
+                        for (uint32_t u = 0; u < U; u++) {
+                            if (live[u]) {
+                                top.x[u] = Combine16<T, OP>(under.x[u], top.x[u]);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (uint32_t u = 0; u < U; u++) {
+                            if (live[u]) {
+                                top.x[u] = Combine16<T, OP>(top.x[u], under.x[u]);
+                            }
                         }
                     }
                     depth--;
