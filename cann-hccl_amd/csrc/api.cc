@@ -106,6 +106,8 @@ void ApplyEnv(GroupConfig *cfg)
             cfg->algo = ALGO_RHD;
         } else if (s.find("ring") != std::string::npos) {
             cfg->algo = ALGO_RING;
+        } else if (s.find("pairwise") != std::string::npos) {
+            cfg->algo = ALGO_PAIRWISE;
         }
     }
     if (const char *e = std::getenv("HCCL_DETERMINISTIC")) {
@@ -1390,6 +1392,8 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
             cfg.algo = ALGO_MESH;
         } else if (v == "rhd") {
             cfg.algo = ALGO_RHD;
+        } else if (v == "pairwise") {
+            cfg.algo = ALGO_PAIRWISE;   // all-to-all family: the flat schedule also over several servers; others: ring
         } else if (v == "auto") {
             cfg.algo = -1;
         } else {
@@ -1543,6 +1547,10 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         rq.servers = std::max(1u, (uint32_t(algo) >> 8) & 0xffu);
         rq.meshAtomic = ((uint32_t(algo) >> 16) & 1u) != 0;
         rq.level0Rings = (uint32_t(algo) >> 17) & 7u;
+    } else if (coll == COLL_ALLTOALLV) {
+        // all-to-all-v: bits 8..15 = number of servers of the staged schedule (0 or 1 = flat pairwise)
+        rq.algo = ALGO_PAIRWISE;
+        rq.servers = std::max(1u, (uint32_t(algo) >> 8) & 0xffu);
     } else {
         rq.algo = Algo(algo);
     }

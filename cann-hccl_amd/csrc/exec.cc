@@ -484,7 +484,7 @@ std::string CacheKey(const Group *g, int algo)
     uint64_t head[10] = {uint64_t(g->ctx->sig.coll), uint64_t(algo), uint64_t(g->ctx->sig.dtype), uint64_t(g->ctx->sig.op), g->ctx->sig.count,
         uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1) | (uint64_t(g->ctx->sig.root) << 8) | (uint64_t(g->ctx->sig.peer) << 20), g->cfg.cclBytes, g->cfg.align,
         uint64_t(g->cfg.blocksPerCu) | (uint64_t(uint32_t(g->cfg.stepStores + 1)) << 32) | (uint64_t(g->cfg.servers) << 40) |
-            (uint64_t(g->cfg.deterministic) << 56) | (uint64_t(g->cfg.level0Rings) << 57) |
+            (uint64_t(g->cfg.algo == ALGO_PAIRWISE ? 1 : 0) << 48) | (uint64_t(g->cfg.deterministic) << 56) | (uint64_t(g->cfg.level0Rings) << 57) |
             (uint64_t(uint32_t(g->cfg.fusedStores + 1)) << 60) | (uint64_t(g->cfg.stepSweep) << 62), g->p};
     put(head, sizeof(head));
     put(g->ctx->send.data(), g->ctx->send.size() * sizeof(void *));
@@ -553,8 +553,11 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
     rq.cclBytes = g->cfg.cclBytes;
     rq.align = g->cfg.align;
     rq.alias.assign(g->p, 0);
+    // only an all-reduce and a broadcast run in place as they are; any other collective whose send buffer is its
+    // receive buffer is staged below
+    const bool inPlaceKind = rq.coll == COLL_ALLREDUCE || rq.coll == COLL_BROADCAST;
     for (uint32_t r = 0; r < g->p; r++) {
-        rq.alias[r] = (g->ctx->send[r] == g->ctx->recv[r]) ? 1 : 0;
+        rq.alias[r] = (inPlaceKind && g->ctx->send[r] == g->ctx->recv[r]) ? 1 : 0;
     }
     const bool fourRings = g->cfg.level0Rings == 4 && g->cfg.servers >= 1 && g->p % g->cfg.servers == 0 && g->p / g->cfg.servers == 8;
     if (rq.coll == COLL_ALLREDUCE && ((g->cfg.servers > 1 && g->p % g->cfg.servers == 0) || fourRings)) {
@@ -592,6 +595,11 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         rq.vDispls = g->ctx->vDispls;
     }
     if (rq.coll == COLL_ALLTOALLV) {
+        // Several servers: the staged schedule, unless the flat pairwise one is asked for by name
+        // (alltoall_operator.cc:225-250).
+        if (g->cfg.servers > 1 && g->p % g->cfg.servers == 0 && g->cfg.algo != ALGO_PAIRWISE) {
+            rq.servers = g->cfg.servers;
+        }
         rq.sendCounts = g->ctx->sendCounts;
         rq.sdispls = g->ctx->sdispls;
         rq.recvCounts = g->ctx->recvCounts;

@@ -37,6 +37,9 @@ Ref MkRef(uint32_t rank, uint8_t buf, uint64_t off)
 struct VProgram {
     std::vector<Phase> phases;
     std::vector<uint64_t> inBytes, outBytes;
+    // Library-owned workspace a schedule addresses as input-buffer offsets [inBytes[r], inBytes[r] + workBytes[r])
+    // (empty = none): it is only read after it was written, so it lives in scratch.
+    std::vector<uint64_t> workBytes;
     // While a schedule is laid out for a sub-communicator: its ranks (local index -> rank of the whole
     // group; empty = identity) and the phase its own phase 0 stands for.
     std::vector<uint32_t> rankMap;
@@ -601,6 +604,48 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             rq.recvCounts.size() != size_t(p) * p || rq.rdispls.size() != size_t(p) * p) {
             *err = "all-to-all-v tables must be p x p";
             return 1;
+        }
+        if (rq.servers > 1) {
+            // Staged (coll_all_to_all_v_staged_executor.cc:378-470, zero-copy mode): inside a server of m ranks,
+            // rank (c, l) collects from its m neighbours everything addressed to the ranks with local index l,
+            // laid out by destination, then by source (coll_all_to_all_executor.cc:156-196, :235-265); then the
+            // ranks with the same local index exchange those runs pairwise between the servers, each block going
+            // to its place in the destination's receive buffer (:300-352; alltoallv_staged_pairwise.cc:65-147).
+            if (p % rq.servers != 0) {
+                *err = "staged all-to-all-v: the servers must hold the same number of ranks";
+                return 1;
+            }
+            const uint32_t S = rq.servers, m = p / S;
+            auto len = [&](uint32_t src, uint32_t dst) { return rq.sendCounts[size_t(src) * p + dst] * u; };
+            for (uint32_t r = 0; r < p; r++) {
+                for (uint32_t n = 0; n < p; n++) {
+                    uint64_t cnt = rq.sendCounts[size_t(r) * p + n];
+                    if (cnt) {
+                        vp->inBytes[r] = std::max(vp->inBytes[r], (rq.sdispls[size_t(r) * p + n] + cnt) * u);
+                        vp->outBytes[n] = std::max(vp->outBytes[n], (rq.rdispls[size_t(n) * p + r] + cnt) * u);
+                    }
+                }
+            }
+            vp->workBytes.assign(p, 0);
+            for (uint32_t r = 0; r < p; r++) {
+                const uint32_t c = r / m, l = r % m;
+                const uint64_t work = (vp->inBytes[r] + 255) & ~uint64_t(255);
+                uint64_t at = work;
+                for (uint32_t j = l; j < p; j += m) {
+                    for (uint32_t k = 0; k < m; k++) {
+                        const uint32_t src = c * m + k;
+                        const uint64_t n = len(src, j);
+                        // stage one: own blocks first (LocalCopy), the neighbours' all at once (alltoallv_staged_mesh.cc:51-130)
+                        EmitCopy(*vp, k == l ? 0 : 1, MkRef(r, BUF_SEND, at), MkRef(src, BUF_SEND, rq.sdispls[size_t(src) * p + j] * u), n);
+                        // stage two: step i hands the run for server c + i to the rank of that server with local index l
+                        const uint32_t step = (j / m + S - c) % S;
+                        EmitCopy(*vp, 2 + step, MkRef(j, BUF_RECV, rq.rdispls[size_t(j) * p + src] * u), MkRef(r, BUF_SEND, at), n);
+                        at += n;
+                    }
+                }
+                vp->workBytes[r] = at - vp->inBytes[r];
+            }
+            return 0;
         }
         // phase i: rank r's block for rank (r+i) goes straight into that rank's receive buffer
         for (uint32_t i = 0; i < p; i++) {
@@ -1676,7 +1721,7 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
     std::string want = OutputSignature(ref, p, alias);
 
     // lowering candidates: partials in the receive buffer (no scratch), else in scratch, else staged
-    bool fits = true;
+    bool fits = vp.workBytes.empty();
     for (uint32_t r = 0; r < p; r++) {
         fits = fits && vp.inBytes[r] <= vp.outBytes[r];
     }
@@ -1729,7 +1774,7 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
         plan->scratchBytes = 0;
         if (usesScratch) {
             for (uint32_t r = 0; r < p; r++) {
-                plan->scratchBytes = std::max(plan->scratchBytes, vp.inBytes[r]);
+                plan->scratchBytes = std::max(plan->scratchBytes, vp.inBytes[r] + (vp.workBytes.empty() ? 0 : vp.workBytes[r]));
             }
         }
         low = std::move(s);

@@ -12,7 +12,8 @@ extern "C" {
 #endif
 
 /* Settings of the communicator's whole group.  Keys and values:
- *   "algo"          "ring" | "mesh" | "rhd" | "auto"
+ *   "algo"          "ring" | "mesh" | "rhd" | "pairwise" | "auto"   ("pairwise" only matters to the all-to-all family,
+ *                                see "servers"; the other collectives then run their ring schedules)
  *   "deterministic" "0" | "1"    as HCCL_DETERMINISTIC; with "0" (the default) the mesh reduce phases of
  *                                all-reduce / reduce-scatter run without the piece cut (not for int64, not for products)
  *   "fuse"          "0" | "1"    run the single-pass fused form when the schedule has one
@@ -21,7 +22,9 @@ extern "C" {
  *   "buffsize_bytes" the same in bytes (tests of the chunk loop on small inputs)
  *   "align"         slice alignment in bytes (default 128)
  *   "servers"       number of rank groups for all-reduce, reduce-scatter and reduce: with n > 1 the p ranks form n groups of p / n
- *                   consecutive ranks and the two-level schedules run (mesh inside a group, "algo" ring or rhd between)
+ *                   consecutive ranks and the two-level schedules run (mesh inside a group, "algo" ring or rhd between);
+ *                   the all-to-all family then runs the staged schedule (gather inside a group into a workspace, pairwise
+ *                   between the groups) unless "algo" is "pairwise"
  *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter / reduce: the mesh schedule
  *                                (default), one ring in rank order, or -- for groups of 8 ranks, for the all-reduce also with one group --
  *                                the four rings of the 8-device ring topology, each on a quarter of every slice

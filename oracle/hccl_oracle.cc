@@ -27,6 +27,8 @@
 //                    TPL/temp_reduce_scatter/reduce_scatter_halving_doubling.cc:67-238,
 //                    TPL/temp_all_gather/all_gather_halving_doubling.cc:43-196
 //   pairwise         TPL/temp_alltoallv/alltoallv_pairwise.cc:75-282, ALG/impl/operator/alltoall_operator.cc:49-72
+//   staged a2av      TPL/temp_alltoallv/alltoallv_staged_{mesh,pairwise}.cc, ALG/impl/coll_executor/coll_all_to_all/
+//                    coll_all_to_all_v_staged_executor.cc:276-470, coll_all_to_all_executor.cc:156-335 (zero-copy mode)
 //   rooted           TPL/temp_broadcast/broadcast_ring.cc:24-160, TPL/temp_reduce/reduce_ring.cc:29-154,
 //                    TPL/temp_scatter/scatter_mesh.cc:46-160, TPL/temp_gather/gather_mesh.cc:60-170,
 //                    EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213, EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194,
@@ -2460,6 +2462,122 @@ int orc_alltoallv(uint32_t p, void **send, const uint64_t *sendCounts, const uin
         m.procs.push_back(std::move(pr));
     }
     return m.Run();
+}
+
+// Staged all-to-all-v over `servers` servers of m = p / servers ranks (zero-copy mode), same tables as
+// orc_alltoallv.  Stage one, inside a server (ALG/impl/coll_executor/coll_all_to_all/coll_all_to_all_v_staged_executor.cc:
+// 378-440; address tables coll_all_to_all_executor.cc:156-335; template TPL/temp_alltoallv/alltoallv_staged_mesh.cc:51-130):
+// rank (c, l) gathers into a workspace, from each rank k of its server, the blocks addressed to the ranks with local
+// index l, ordered by destination and then by source.  Stage two, between the servers (:300-352, :441-456; template
+// alltoallv_staged_pairwise.cc:65-147): the ranks with local index l exchange their runs pairwise, every block
+// landing at its displacement in the destination's receive buffer.  Returns 0, 1 for asymmetric tables, 2 when the
+// servers are not of one size.
+int orc_alltoallv_staged(uint32_t p, uint32_t servers, void **send, const uint64_t *sendCounts, const uint64_t *sdispls,
+    void **recv, const uint64_t *recvCounts, const uint64_t *rdispls, int dt, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || servers == 0) {
+        return -20;
+    }
+    if (p % servers != 0) {
+        return 2;
+    }
+    for (uint32_t i = 0; i < p; i++) {
+        for (uint32_t j = 0; j < p; j++) {
+            if (sendCounts[i * p + j] != recvCounts[j * p + i]) {
+                return 1;
+            }
+        }
+    }
+    const uint32_t m = p / servers;
+    auto len = [&](uint32_t src, uint32_t dst) { return sendCounts[size_t(src) * p + dst] * unit; };
+    // workspace offset of the block (destination j, source local rank k) at rank (c, l), j = l mod m:
+    // everything before it in (destination, source) order (coll_all_to_all_executor.cc:171-187)
+    auto workOff = [&](uint32_t c, uint32_t j, uint32_t k) {
+        uint64_t off = 0;
+        for (uint32_t jj = j % m; jj <= j; jj += m) {
+            for (uint32_t kk = 0; kk < m; kk++) {
+                if (jj == j && kk == k) {
+                    return off;
+                }
+                off += len(c * m + kk, jj);
+            }
+        }
+        return off;
+    };
+    std::vector<std::vector<uint8_t>> work(p);
+    for (uint32_t r = 0; r < p; r++) {
+        uint64_t total = 0;
+        for (uint32_t j = r % m; j < p; j += m) {
+            for (uint32_t k = 0; k < m; k++) {
+                total += len(r / m * m + k, j);
+            }
+        }
+        work[r].assign(total + 1, 0);
+    }
+    Pool pool(threads);
+    Machine mc;
+    mc.p = static_cast<int>(p);
+    mc.dt = dt;
+    mc.direct = (flags & 1) != 0;
+    mc.pool = &pool;
+    mc.buf[B_IN].resize(p);
+    mc.buf[B_OUT].resize(p);
+    // stage one: send buffer -> workspace
+    for (uint32_t r = 0; r < p; r++) {
+        mc.buf[B_IN][r] = static_cast<uint8_t *>(send[r]);
+        mc.buf[B_OUT][r] = work[r].data();
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        const uint32_t c = r / m, l = r % m;
+        Proc pr;
+        pr.rank = static_cast<int>(r);
+        for (uint32_t j = l; j < p; j += m) {   // LocalCopy (alltoallv_staged_base.cc:36-56)
+            pr.prog.push_back(MkLocalCopy(B_OUT, workOff(c, j, l), B_IN, sdispls[size_t(r) * p + j] * unit, len(r, j)));
+        }
+        for (uint32_t i = 1; i < m; i++) {      // one stream per neighbour (alltoallv_staged_mesh.cc:96-130)
+            const uint32_t dl = (l + i) % m, dest = c * m + dl;
+            for (uint32_t j = dl; j < p; j += m) {
+                pr.prog.push_back(MkSend(static_cast<int>(dest), static_cast<int>(i), B_IN, sdispls[size_t(r) * p + j] * unit, len(r, j)));
+            }
+        }
+        for (uint32_t i = 1; i < m; i++) {
+            const uint32_t sl = (l + m - i) % m, src = c * m + sl;
+            for (uint32_t j = l; j < p; j += m) {
+                pr.prog.push_back(MkRecvCopy(static_cast<int>(src), static_cast<int>(i), B_OUT, workOff(c, j, sl), len(src, j)));
+            }
+        }
+        mc.procs.push_back(std::move(pr));
+    }
+    int rc = mc.Run();
+    if (rc != 0) {
+        return rc;
+    }
+    // stage two: workspace -> receive buffers
+    for (uint32_t r = 0; r < p; r++) {
+        mc.buf[B_IN][r] = work[r].data();
+        mc.buf[B_OUT][r] = static_cast<uint8_t *>(recv[r]);
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        const uint32_t c = r / m, l = r % m;
+        Proc pr;
+        pr.rank = static_cast<int>(r);
+        for (uint32_t k = 0; k < m; k++) {      // LocalCopy: the run addressed to this rank itself
+            pr.prog.push_back(MkLocalCopy(B_OUT, rdispls[size_t(r) * p + c * m + k] * unit, B_IN, workOff(c, r, k), len(c * m + k, r)));
+        }
+        for (uint32_t i = 1; i < servers; i++) {
+            const uint32_t nc = (c + i) % servers, pc = (c + servers - i) % servers;
+            const uint32_t next = nc * m + l, prev = pc * m + l;
+            for (uint32_t k = 0; k < m; k++) {
+                pr.prog.push_back(MkSend(static_cast<int>(next), 0, B_IN, workOff(c, next, k), len(c * m + k, next)));
+            }
+            for (uint32_t k = 0; k < m; k++) {
+                pr.prog.push_back(MkRecvCopy(static_cast<int>(prev), 0, B_OUT, rdispls[size_t(r) * p + pc * m + k] * unit, len(pc * m + k, r)));
+            }
+        }
+        mc.procs.push_back(std::move(pr));
+    }
+    return mc.Run();
 }
 
 // ---- synthetic data ------------------------------------------------------------------------------

@@ -75,6 +75,8 @@ def lib():
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
         L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
         L.orc_alltoallv.argtypes = [u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, u64, i32, i32]
+        L.orc_alltoallv_staged.argtypes = [u32, u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, i32, i32]
+        L.orc_alltoallv_staged.restype = i32
         L.orc_fill_uniform_f32.argtypes = [vp, u64, u64, u32, i32]
         _lib = L
     return _lib
@@ -319,6 +321,22 @@ def alltoallv(sends, send_counts, sdispls, recvs, recv_counts, rdispls, dt, scra
                              rc_.ctypes.data_as(pu64), rd.ctypes.data_as(pu64), dt, scratch_bytes, flags, threads)
     if rc not in (0, 1):
         raise RuntimeError("oracle alltoallv failed rc=%d" % rc)
+    return rc
+
+
+def alltoallv_staged(sends, send_counts, sdispls, recvs, recv_counts, rdispls, dt, servers, flags=0, threads=1):
+    """The staged schedule over `servers` servers of equal size; arguments as alltoallv.  Returns 0, 1 (asymmetric
+    tables) or 2 (servers of different sizes)."""
+    p = len(sends)
+    sc = np.ascontiguousarray(send_counts, dtype=np.uint64)
+    sd = np.ascontiguousarray(sdispls, dtype=np.uint64)
+    rc_ = np.ascontiguousarray(recv_counts, dtype=np.uint64)
+    rd = np.ascontiguousarray(rdispls, dtype=np.uint64)
+    pu64 = ctypes.POINTER(ctypes.c_uint64)
+    rc = lib().orc_alltoallv_staged(p, servers, _ptrs(sends), sc.ctypes.data_as(pu64), sd.ctypes.data_as(pu64), _ptrs(recvs),
+                                    rc_.ctypes.data_as(pu64), rd.ctypes.data_as(pu64), dt, flags, threads)
+    if rc not in (0, 1, 2):
+        raise RuntimeError("oracle staged alltoallv failed rc=%d" % rc)
     return rc
 
 

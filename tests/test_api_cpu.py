@@ -235,7 +235,7 @@ def test_amd_params(comms):
     assert L.HcclAmdSetParam(comms[0], b"buffsize_mib", b"0") == H.HCCL_E_PARA
     assert L.HcclAmdSetParam(None, b"algo", b"ring") == H.HCCL_E_PTR
     # every documented key takes its documented values and nothing else
-    good = {b"algo": [b"ring", b"mesh", b"rhd", b"auto"], b"deterministic": [b"0", b"1"], b"fuse": [b"0", b"1"],
+    good = {b"algo": [b"ring", b"mesh", b"rhd", b"pairwise", b"auto"], b"deterministic": [b"0", b"1"], b"fuse": [b"0", b"1"],
             b"graph": [b"0", b"1"], b"buffsize_mib": [b"1", b"200"], b"buffsize_bytes": [b"4096"], b"align": [b"4", b"128"],
             b"level0": [b"mesh", b"ring", b"ring4"], b"step_stores": [b"auto", b"nt", b"ordinary"],
             b"fused_stores": [b"nt", b"ordinary"], b"step_sweep": [b"forward", b"alternate"], b"cache_entries": [b"1", b"1024"], b"blocks_per_cu": [b"0", b"2"],

@@ -291,6 +291,59 @@ def test_alltoallv_16_ranks_lognormal(orc):
             g.close()
 
 
+def test_staged_alltoallv_over_servers(orc):
+    # several servers: gather inside a server into the workspace, pairwise between the servers; the same bytes as the
+    # flat schedule, fused (no workspace) and step by step (through it)
+    for p, servers in ((4, 2), (8, 2), (8, 4), (6, 3), (16, 4), (12, 12)):
+        cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 60 + p + servers, max_count=5000)
+        sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+        want = [np.full(n, -1, np.int32) for n in rl]
+        assert orc.alltoallv_staged(sends, cnt, sdis, want, rcnt, rdis, INT32, servers) == 0
+        moved = 4 * int(cnt.sum())
+        for fuse in (1, 0):
+            g = gh.Group(p, fuse=fuse, servers=servers)
+            try:
+                print("staged alltoallv p", p, "servers", servers, "fuse", fuse, flush=True)
+                outs = gh.all_to_all_v(g, sends, cnt, sdis, rl, rcnt, rdis, INT32)
+                assert all(np.array_equal(outs[r], want[r]) for r in range(p)), (p, servers, fuse)
+                info = g.info()
+                assert info["fused"] == fuse
+                if fuse:
+                    assert info["bytesRead"] == moved and info["bytesWritten"] == moved and info["scratchBytes"] == 0
+                else:
+                    assert info["bytesRead"] == 2 * moved and info["bytesWritten"] == 2 * moved and info["scratchBytes"] > 0
+                    assert info["launches"] <= 2 + servers
+                # asked for by name, the flat pairwise schedule runs instead
+                H.set_param(g.comms[0], "algo", "pairwise")
+                outs = gh.all_to_all_v(g, sends, cnt, sdis, rl, rcnt, rdis, INT32)
+                assert all(np.array_equal(outs[r], want[r]) for r in range(p)), (p, servers, fuse, "flat")
+                info = g.info()
+                assert info["bytesRead"] == moved and info["scratchBytes"] == 0
+            finally:
+                g.close()
+
+
+def test_staged_uniform_alltoall_over_servers():
+    p, servers, n = 8, 2, 3001
+    rng = np.random.default_rng(77)
+    ins = [rng.integers(-1 << 30, 1 << 30, n * p).astype(np.int32) for _ in range(p)]
+    for fuse in (1, 0):
+        g = gh.Group(p, fuse=fuse, servers=servers)
+        try:
+            sends = [gh.to_dev(x) for x in ins]
+            recvs = [gh.to_dev(np.full(n * p, -1, np.int32)) for _ in range(p)]
+            torch.cuda.synchronize()
+            H.all_to_all(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, INT32, g.stream_ptr)
+            g.stream.synchronize()
+            assert (g.info()["scratchBytes"] > 0) == (fuse == 0)
+            for j in range(p):
+                got = gh.to_host(recvs[j], INT32)
+                for i in range(p):
+                    assert np.array_equal(got[i * n:(i + 1) * n], ins[i][j * n:(j + 1) * n]), (fuse, i, j)
+        finally:
+            g.close()
+
+
 def test_alltoallv_asymmetric_tables_fail(orc):
     p = 4
     g = gh.Group(p)

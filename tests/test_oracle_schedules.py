@@ -284,6 +284,44 @@ def test_alltoallv_is_the_permutation(orc):
                 assert np.array_equal(recvs[j], want), (p, scratch, j)
 
 
+def _a2av_definition(p, cnt, sdis, rdis, sends, rl):
+    """What an all-to-all-v is: rank j's receive buffer holds, at rdispls[j][i], the block rank i addressed to j."""
+    out = []
+    for j in range(p):
+        want = np.full(rl[j], -1, np.int32)
+        for i in range(p):
+            c = int(cnt[i, j])
+            want[int(rdis[j, i]):int(rdis[j, i]) + c] = sends[i][int(sdis[i, j]):int(sdis[i, j]) + c]
+        out.append(want)
+    return out
+
+
+def test_staged_alltoallv_is_the_permutation(orc):
+    # the staged route (gather inside a server, pairwise between servers) delivers exactly the definition
+    for p, servers in ((4, 2), (8, 2), (8, 4), (6, 3), (6, 2), (16, 2), (16, 4), (12, 12), (5, 1), (9, 3)):
+        cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 7 * p + servers)
+        sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+        keep = [x.copy() for x in sends]
+        for flags in (0, orc.DIRECT):
+            recvs = [np.full(n, -1, np.int32) for n in rl]
+            assert orc.alltoallv_staged(sends, cnt, sdis, recvs, rcnt, rdis, INT32, servers, flags=flags) == 0
+            want = _a2av_definition(p, cnt, sdis, rdis, sends, rl)
+            for j in range(p):
+                assert np.array_equal(recvs[j], want[j]), (p, servers, flags, j)
+        assert all(np.array_equal(a, b) for a, b in zip(sends, keep))
+
+
+def test_staged_alltoallv_rejects_bad_requests(orc):
+    p = 6
+    cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 3)
+    sends = [np.zeros(n + 8, np.int32) for n in sl]
+    recvs = [np.zeros(n + 8, np.int32) for n in rl]
+    assert orc.alltoallv_staged(sends, cnt, sdis, recvs, rcnt, rdis, INT32, 4) == 2       # 6 ranks do not fill 4 servers
+    bad = rcnt.copy()
+    bad[2, 1] += 1
+    assert orc.alltoallv_staged(sends, cnt, sdis, recvs, bad, rdis, INT32, 2) == 1
+
+
 def test_alltoallv_rejects_asymmetric_tables(orc):
     p = 4
     cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 1)

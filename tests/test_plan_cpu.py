@@ -117,6 +117,34 @@ def test_alltoallv_plan_matches_checker(orc, p):
             assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, fused, r)
 
 
+@pytest.mark.parametrize("p,servers", [(4, 2), (8, 2), (8, 4), (6, 3), (16, 4), (12, 12), (9, 3)])
+def test_staged_alltoallv_plan_matches_checker(orc, p, servers):
+    cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 40 + p + servers)
+    sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+    want = [np.full(n, -1, np.int32) for n in rl]
+    assert orc.alltoallv_staged(sends, cnt, sdis, want, rcnt, rdis, INT32, servers) == 0
+    plan = H.describe_plan(H.COLL_ALLTOALLV, H.ALGO_PAIRWISE | (servers << 8), p, 0, INT32, tables=(cnt, sdis, rcnt, rdis))
+    flat = H.describe_plan(H.COLL_ALLTOALLV, H.ALGO_PAIRWISE, p, 0, INT32, tables=(cnt, sdis, rcnt, rdis))
+    m = p // servers
+    # stage one: own blocks, then the neighbours' (none when a server holds one rank); stage two: one phase per server
+    assert len(plan["phases"]) <= 2 + servers
+    # the workspace holds, per rank, what its server addresses to the ranks with its local index
+    work = max(sum(int(cnt[r // m * m + k, j]) for j in range(r % m, p, m) for k in range(m)) for r in range(p)) * 4
+    assert work <= plan["scratchBytes"] <= work + max(sl) * 4 + 256
+    moved = 4 * int(cnt.sum())
+    assert sum(s["n"] for ph in plan["phases"] for s in ph) == 2 * moved      # every block moves twice step by step ...
+    assert sum(it["n"] for it in plan["fused"]) == moved                      # ... and once when fused
+    assert sum(it["n"] for it in flat["fused"]) == moved
+    for fused in (False, True):
+        recvs = [np.full(n, -1, np.int32).view(np.uint8).copy() for n in rl]
+        (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, _bytes(sends), recvs, INT32, 0)
+        for r in range(p):
+            assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, servers, fused, r)
+    uneven = next(s for s in range(2, p + 2) if p % s)         # a server count that does not divide the ranks
+    with pytest.raises(H.HcclError):
+        H.describe_plan(H.COLL_ALLTOALLV, H.ALGO_PAIRWISE | (uneven << 8), p, 0, INT32, tables=(cnt, sdis, rcnt, rdis))
+
+
 def test_plan_rejects_bad_requests():
     with pytest.raises(H.HcclError):
         H.describe_plan(H.COLL_ALLREDUCE, RING, 0, 10, FP32)
