@@ -194,6 +194,10 @@ def run_suite(pkg, torch, steps, warmup, only="", settings=()):
     report("all-to-all-v pairwise p=16 int32 lognormal (%.0f MB)" % (4 * cnt.sum() / 1e6), comms,
            lambda: pkg.all_to_all_v(comms, sp, None, None, rp, None, None, pkg.HCCL_DATA_TYPE_INT32, stream.cuda_stream,
                                     tables=tables))
+    pkg.set_param(comms[0], "servers", 2)
+    report("all-to-all-v staged 2x8 p=16 int32 lognormal (%.0f MB)" % (4 * cnt.sum() / 1e6), comms,
+           lambda: pkg.all_to_all_v(comms, sp, None, None, rp, None, None, pkg.HCCL_DATA_TYPE_INT32, stream.cuda_stream,
+                                    tables=tables))
     del sends, recvs
     pkg.comm_destroy(comms)
 
