@@ -888,6 +888,23 @@ def test_allreduce_on_a_rank_table_communicator(orc, tmp_path):
             stream.synchronize()
             for r in range(p):
                 assert np.array_equal(gh.to_host(recvs[r], FP32), want[r]), (algo, r)
+        # its all-to-all-v takes the staged route by itself (step by step here, so that the workspace is in play)
+        H.set_param(comms[0], "algo", "auto")
+        H.set_param(comms[0], "fuse", 0)
+        cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 91, max_count=3000)
+        ins = [(np.arange(m, dtype=np.int32) + (r << 20)) for r, m in enumerate(sl)]
+        want = [np.full(m, -1, np.int32) for m in rl]
+        assert orc.alltoallv_staged(ins, cnt, sdis, want, rcnt, rdis, INT32, servers) == 0
+        sends = [gh.to_dev(x) for x in ins]
+        recvs = [gh.to_dev(np.full(m, -1, np.int32)) for m in rl]
+        torch.cuda.synchronize()
+        H.all_to_all_v(comms, [t.data_ptr() for t in sends], cnt, sdis, [t.data_ptr() for t in recvs], rcnt, rdis, INT32,
+                       stream.cuda_stream)
+        stream.synchronize()
+        info = H.last_op_info(comms[0])
+        assert info["scratchBytes"] > 0 and info["launches"] <= 2 + servers
+        for r in range(p):
+            assert np.array_equal(gh.to_host(recvs[r], INT32), want[r]), ("staged all-to-all-v", r)
     finally:
         torch.cuda.synchronize()
         H.comm_destroy(comms)

@@ -217,3 +217,52 @@ def test_random_reducescatter_and_reduce_on_rank_groups(orc, seed):
                     assert bool((outs[r] == 0x33).all()), (seed, case, "a rank other than the root was written", r)
         finally:
             g.close()
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_alltoallv_flat_and_staged(orc, seed):
+    """All-to-all-v with random tables: element sizes 1, 2, 4 and 8 bytes (displacements then fall on every byte
+    alignment), counts from zero to tens of thousands, over one server or several, fused and step by step,
+    against the checker's staged or flat schedule; bytes outside the addressed blocks must stay as they were."""
+    from closed_forms import INT8, INT16, INT32
+    rng = np.random.default_rng(5200 + seed)
+    carriers = {INT8: np.int8, INT16: np.int16, INT32: np.int32, INT64: np.int64}
+    for case in range(8):
+        p = int(rng.choice([2, 3, 4, 6, 8, 12, 16]))
+        servers = int(rng.choice([s for s in range(1, p + 1) if p % s == 0]))
+        dt = int(rng.choice(list(carriers)))
+        fuse = int(rng.integers(0, 2))
+        big = int(rng.choice([50, 3000, 40000]))
+        cnt = rng.integers(0, big, (p, p)).astype(np.uint64)
+        cnt[rng.random((p, p)) < 0.2] = 0
+        sdis, rdis = np.zeros((p, p), np.uint64), np.zeros((p, p), np.uint64)
+        sl, rl = [], []
+        for r in range(p):
+            pos = 0
+            for j in rng.permutation(p):
+                pos += int(rng.integers(0, 37))
+                sdis[r, j] = pos
+                pos += int(cnt[r, j])
+            sl.append(pos + 7)
+            pos = 0
+            for i in rng.permutation(p):
+                pos += int(rng.integers(0, 37))
+                rdis[r, i] = pos
+                pos += int(cnt[i, r])
+            rl.append(pos + 7)
+        info = np.iinfo(carriers[dt])
+        ins = [rng.integers(info.min, info.max, n, dtype=carriers[dt]) for n in sl]
+        want = [np.full(n, 0x5A, carriers[dt]) for n in rl]
+        if servers > 1:
+            assert orc.alltoallv_staged(ins, cnt, sdis, want, cnt.T.copy(), rdis, dt, servers) == 0
+        else:
+            assert orc.alltoallv(ins, cnt, sdis, want, cnt.T.copy(), rdis, dt) == 0
+        print("random all-to-all-v seed", seed, "case", case, "p", p, "servers", servers, "dt", dt, "fuse", fuse, "max", big, flush=True)
+        g = gh.Group(p, fuse=fuse, servers=servers)
+        try:
+            outs = gh.all_to_all_v(g, ins, cnt, sdis, rl, cnt.T.copy(), rdis, dt, fill=0x5A)
+            for r in range(p):
+                assert np.array_equal(outs[r], want[r]), (seed, case, r)
+            assert g.info()["fused"] == fuse
+        finally:
+            g.close()
