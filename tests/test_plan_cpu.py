@@ -547,3 +547,48 @@ def test_two_level_reduce_with_rings_inside_a_group_matches_checker(orc, level1,
                     for r in range(p):
                         if r != root:
                             assert np.all(recvs[r] == 0x77)
+
+
+def _gold():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "slice_plans.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("case", _gold()["ring"])
+def test_planner_ring_slices_match_the_hand_derived_vectors(case):
+    # the product's own slice plan, read off its ring all-reduce: the all-gather's first phase copies each rank's
+    # reduced slice to its neighbour, so its steps name every non-empty slice once, by offset and size
+    total, p, align = case["total"], case["p"], case["align"]
+    if p == 1:
+        return
+    plan = H.describe_plan(H.COLL_ALLREDUCE, RING, p, total, H.HCCL_DATA_TYPE_INT8, align=align)
+    want = sorted((o, s) for o, s in zip(case["off"], case["size"]) if s)
+    seen = set()
+    for ph in plan["phases"]:
+        for s in ph:
+            seen.add((s["dst"][2], s["n"]))
+    assert set(want) <= seen, (want, sorted(seen))
+    # every step is one slice, whole: nothing in the plan cuts a slice differently
+    assert all(x in set(want) for x in seen), (want, sorted(seen))
+
+
+@pytest.mark.parametrize("case", [c for c in _gold()["chunks"] if c["kind"] == 0])
+def test_planner_chunk_plan_matches_the_hand_derived_vectors(case):
+    # all-reduce chunk loop: a chunk's steps stay inside [chunk start, chunk end) of the buffers, and the chunk
+    # boundaries are the hand-derived ones
+    p, unit = case["p"], case["unit"]
+    dt = {4: FP32, 8: INT64}[unit]
+    if case["count"] > (1 << 22):
+        return                                        # the big vector is covered by the checker's test; keep this one quick
+    plan = H.describe_plan(H.COLL_ALLREDUCE, RING, p, case["count"], dt, ccl_bytes=case["ccl"], align=case["align"])
+    bounds = [0]
+    for c in case["counts"]:
+        bounds.append(bounds[-1] + c * unit)
+    for ph in plan["phases"]:
+        for s in ph:
+            lo, hi = s["dst"][2], s["dst"][2] + s["n"]
+            assert any(b0 <= lo and hi <= b1 for b0, b1 in zip(bounds, bounds[1:])), (lo, hi, bounds)
+    starts = {s["dst"][2] for ph in plan["phases"] for s in ph}
+    assert set(bounds[:-1]) <= starts
