@@ -592,3 +592,23 @@ def test_planner_chunk_plan_matches_the_hand_derived_vectors(case):
             assert any(b0 <= lo and hi <= b1 for b0, b1 in zip(bounds, bounds[1:])), (lo, hi, bounds)
     starts = {s["dst"][2] for ph in plan["phases"] for s in ph}
     assert set(bounds[:-1]) <= starts
+
+
+@pytest.mark.parametrize("case", [c for c in _gold()["rhd_slices"] if c["total"] <= (1 << 22)])
+def test_planner_halving_doubling_slices_match_the_hand_derived_vectors(case):
+    # a halving-doubling all-reduce over a power-of-two block moves runs of 1, 2, 4, ... neighbouring slices:
+    # every step of the product's plan must be such a run of the hand-derived slices, and every slice moves alone once
+    block, total = case["block"], case["total"]
+    plan = H.describe_plan(H.COLL_ALLREDUCE, RHD, block, total, H.HCCL_DATA_TYPE_INT8, align=case["align"])
+    off, size = case["off"], case["size"]
+    runs = set()
+    w = 1
+    while w <= block:
+        for i in range(0, block, w):
+            n = sum(size[i:i + w])
+            if n:
+                runs.add((off[i], n))
+        w *= 2
+    seen = {(s["dst"][2], s["n"]) for ph in plan["phases"] for s in ph}
+    assert seen <= runs, (sorted(seen - runs), sorted(runs))
+    assert {(o, s) for o, s in zip(off, size) if s} <= seen
