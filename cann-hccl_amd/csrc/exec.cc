@@ -538,6 +538,18 @@ int CachedPlan(Group *g, const PlanRequest &rq, std::shared_ptr<const Plan> *out
     return 0;
 }
 
+// Schedule between the servers of a two-level collective: the one asked for, else the reference's default
+// (AlgConfigurator::GetDefaultAlgoLevel1V1, ALG/impl/alg_configurator.cc:226-241): halving-doubling for 8 servers
+// and more and for powers of two, ring otherwise.
+Algo Level1Algo(const Group *g)
+{
+    if (g->cfg.algo == ALGO_RING || g->cfg.algo == ALGO_RHD) {
+        return Algo(g->cfg.algo);
+    }
+    const uint32_t n = g->cfg.servers;
+    return (n >= 8 || (n > 1 && (n & (n - 1)) == 0)) ? ALGO_RHD : ALGO_RING;
+}
+
 HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
 {
     std::unique_ptr<Prepared> pp(new Prepared());
@@ -565,7 +577,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         // mesh, coll_all_reduce_mesh_executor.cc:108-112) or ring(s) when the group is set up as a ring
         // topology (coll_all_reduce_ring_executor.cc:95-135); ring or halving-doubling between the groups
         rq.servers = g->cfg.servers;
-        rq.algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_RHD;   // halving-doubling unless ring is asked for (:185-191)
+        rq.algo = Level1Algo(g);   // ring or halving-doubling (:185-191)
         rq.level0Rings = g->cfg.level0Rings == 4 ? (fourRings ? 4u : 1u) : g->cfg.level0Rings;
         rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
             g->ctx->sig.op != HCCL_REDUCE_PROD;
@@ -575,7 +587,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         // ring or halving-doubling between the groups first, then inside a group the mesh (uncut under the
         // conditions of :216-218) or the ring(s)
         rq.servers = g->cfg.servers;
-        rq.algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_RHD;
+        rq.algo = Level1Algo(g);
         rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
         rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
             g->ctx->sig.op != HCCL_REDUCE_PROD;
@@ -585,7 +597,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         // groups the mesh (uncut under the conditions of :93-97) or the ring(s), then ring or halving-doubling
         // towards the root's group (:133-139)
         rq.servers = g->cfg.servers;
-        rq.algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_RHD;
+        rq.algo = Level1Algo(g);
         rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
         rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
             g->ctx->sig.op != HCCL_REDUCE_PROD;

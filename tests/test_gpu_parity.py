@@ -910,6 +910,27 @@ def test_allreduce_on_a_rank_table_communicator(orc, tmp_path):
         H.comm_destroy(comms)
 
 
+def test_default_schedule_between_servers_follows_the_reference_rule(orc):
+    # no schedule asked for: halving-doubling between 2, 4 or 8 and more servers, ring between 3, 5, 6 or 7
+    # (order-sensitive fp32 data, so the two give different bits and the check can tell them apart)
+    n = 4099
+    for p, servers, level1 in ((6, 3, RING), (8, 4, RHD), (12, 6, RING), (16, 8, RHD), (10, 5, RING)):
+        ins = _ins(FP32, p, n, 300 + p)
+        ins[0][:] *= 1e7
+        ins[p - 1][:] *= -1e7
+        want = orc.allreduce_two_level(ins, FP32, SUM, servers, level1=level1, atomic=True)
+        other = orc.allreduce_two_level(ins, FP32, SUM, servers, level1=RING if level1 == RHD else RHD, atomic=True)
+        g = gh.Group(p, servers=servers)
+        try:
+            outs, _ = gh.all_reduce(g, ins, FP32, SUM)
+            for r in range(p):
+                assert np.array_equal(outs[r], want[r]), (p, servers, r)
+            if servers > 2:
+                assert not np.array_equal(want[0], other[0]), (p, servers, "the two schedules agree: weak case")
+        finally:
+            g.close()
+
+
 def test_fused_write_back_stores_give_the_same_bits(orc):
     p = 8
     g = _group(p, RING, fuse=1, fused_stores="ordinary")
