@@ -265,6 +265,11 @@ def run_suite(pkg, torch, steps, warmup, only="", settings=()):
     pkg.comm_destroy(comms)
     comms = pkg.comm_init_all(p)
     pkg.set_param(comms[0], "servers", 2)
+    report("all-gather two-level 2x4 mesh+rhd 32MiB/rank in", comms,
+           lambda: pkg.all_gather(comms, sp, rp, n // p, FP32, stream.cuda_stream))
+    pkg.comm_destroy(comms)
+    comms = pkg.comm_init_all(p)
+    pkg.set_param(comms[0], "servers", 2)
     report("reduce two-level 2x4 mesh+rhd fp32 sum 256MiB/rank root 3", comms,
            lambda: pkg.reduce(comms, sp, rp, n, FP32, 0, 3, stream.cuda_stream))
     pkg.comm_destroy(comms)

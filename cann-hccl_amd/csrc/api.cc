@@ -1541,8 +1541,8 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         rq.servers = std::max(1u, (uint32_t(algo) >> 8) & 0xffu);
         rq.meshAtomic = ((uint32_t(algo) >> 16) & 1u) != 0;   // bit 16: mesh level without the piece cut
         rq.level0Rings = (uint32_t(algo) >> 17) & 7u;         // bits 17..19: rings inside a group (0 = mesh, 1, 4)
-    } else if (coll == COLL_REDUCESCATTER) {
-        // reduce-scatter: the same fields (two-level with a mesh inside the groups only)
+    } else if (coll == COLL_REDUCESCATTER || coll == COLL_ALLGATHER) {
+        // reduce-scatter, all-gather: the same fields
         rq.algo = Algo(uint32_t(algo) & 0xffu);
         rq.servers = std::max(1u, (uint32_t(algo) >> 8) & 0xffu);
         rq.meshAtomic = ((uint32_t(algo) >> 16) & 1u) != 0;

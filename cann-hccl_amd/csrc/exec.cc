@@ -592,6 +592,13 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
             g->ctx->sig.op != HCCL_REDUCE_PROD;
     }
+    if (rq.coll == COLL_ALLGATHER && !g->ctx->sig.variable && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
+        // two levels (coll_all_gather_mesh_executor.cc:71-175, coll_all_gather_ring_executor.cc:81-200): inside a
+        // group first, mesh or ring(s), then ring or halving-doubling between the groups
+        rq.servers = g->cfg.servers;
+        rq.algo = Level1Algo(g);
+        rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
+    }
     if (rq.coll == COLL_REDUCE && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
         // two levels (coll_reduce_mesh_executor.cc:75-194, coll_reduce_ring_plus_hd_executor.cc:75-168): inside the
         // groups the mesh (uncut under the conditions of :93-97) or the ring(s), then ring or halving-doubling

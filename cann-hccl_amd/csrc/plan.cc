@@ -489,6 +489,61 @@ void RhdAllGatherChunk(VProgram &vp, size_t phase0, uint32_t p, const std::vecto
     }
 }
 
+// Two-level all-gather of one chunk (CollAllGatherMeshExecutor::KernelRun, coll_all_gather_mesh_executor.cc:71-175;
+// CollAllGatherRingExecutor::KernelRun, coll_all_gather_ring_executor.cc:81-200), after every rank copied its own
+// block in (phase 0): the all-gather inside every group of D = p / servers consecutive ranks over the group's D
+// blocks (mesh, one ring, or the four rings of the 8-device topology on quarters of every block), then the ranks
+// at position d of all groups exchange their groups' D blocks, ring or recursive halving-doubling.
+// sl[i] = where block i lies in every output buffer.
+void TwoLevelAllGatherChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers, uint32_t level0Rings,
+    const std::vector<Slice> &sl, uint64_t align)
+{
+    const uint32_t D = p / servers;
+    const size_t l0 = D > 1 ? (level0Rings == 0 ? 1 : D - 1) : 0;
+    for (uint32_t s = 0; s < servers && D > 1; s++) {
+        std::vector<Slice> own(sl.begin() + size_t(s) * D, sl.begin() + size_t(s + 1) * D);
+        vp.rankMap.resize(D);
+        vp.phaseBase = 1;
+        if (level0Rings == 0) {
+            for (uint32_t d = 0; d < D; d++) {
+                vp.rankMap[d] = s * D + d;
+            }
+            MeshAllGatherPhases(vp, 0, D, 0, own);
+            continue;
+        }
+        for (uint32_t k = 0; k < level0Rings; k++) {
+            std::vector<Slice> part(D);
+            for (uint32_t i = 0; i < D; i++) {
+                uint32_t dev = level0Rings > 1 ? kRingOrders8[k][i] : i;
+                vp.rankMap[i] = s * D + dev;
+                std::vector<Slice> cut = RingSlicePlan(own[dev].size, level0Rings, align);
+                part[i] = Slice{own[dev].off + cut[k].off, cut[k].size};
+            }
+            RingAllGatherPhases(vp, 0, D, 0, part);
+        }
+    }
+    for (uint32_t d = 0; d < D && servers > 1; d++) {
+        vp.rankMap.resize(servers);
+        for (uint32_t s = 0; s < servers; s++) {
+            vp.rankMap[s] = s * D + d;
+        }
+        vp.phaseBase = 1 + l0;
+        for (uint32_t k = 0; k < D; k++) {          // a group's blocks need not be neighbours in the caller's layout
+            std::vector<Slice> blk(servers);
+            for (uint32_t s = 0; s < servers; s++) {
+                blk[s] = sl[size_t(s) * D + k];
+            }
+            if (level1 == ALGO_RING) {
+                RingAllGatherPhases(vp, 0, servers, 0, blk);
+            } else {
+                RhdAllGatherChunk(vp, 0, servers, blk);
+            }
+        }
+    }
+    vp.rankMap.clear();
+    vp.phaseBase = 0;
+}
+
 // Ring reduce (reduce_ring.cc:29-154) among n ranks of `bytes` bytes at `off` in their input buffers:
 // the data walks root+1 -> ... -> root, every rank combining its own with what arrives; the last
 // combine writes `result` instead of the root's input.  Returns the phase after the last one used.
@@ -870,7 +925,10 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
     }
     // the two-level reduce-scatter sizes its chunks without rounding to the slice alignment
     // (CollReduceScatterMeshExecutor::CalcLoopMaxCount, coll_reduce_scatter_mesh_executor.cc:114-119)
-    const bool twoLevelScatter = rq.coll == COLL_REDUCESCATTER && rq.servers > 1;
+    // and so does the two-level all-gather with rings inside a group (CollAllGatherRingExecutor::CalcLoopMaxCount,
+    // coll_all_gather_ring_executor.cc:75-79; with the mesh the rounding stays, coll_all_gather_mesh_executor.cc:64-69)
+    const bool twoLevelScatter = (rq.coll == COLL_REDUCESCATTER && rq.servers > 1) ||
+        (rq.coll == COLL_ALLGATHER && rq.servers > 1 && rq.level0Rings > 0);
     std::vector<uint64_t> chunks = ChunkCounts(rq.coll, rq.count, rq.unit, p, rq.cclBytes, twoLevelScatter ? 1 : rq.align);
     if (rq.count > 0 && chunks.empty()) {
         *err = "CCL buffer too small for one element per rank";
@@ -919,7 +977,9 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             for (uint32_t r = 0; r < p; r++) {
                 EmitCopy(*vp, 0, MkRef(r, BUF_RECV, sl[r].off), MkRef(r, BUF_SEND, done), bytes);
             }
-            if (p > 1) {
+            if (p > 1 && rq.servers > 1) {
+                TwoLevelAllGatherChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, rq.level0Rings, sl, rq.align);
+            } else if (p > 1) {
                 if (rq.algo == ALGO_RING) {
                     RingAllGatherPhases(*vp, 1, p, 0, sl);
                 } else if (rq.algo == ALGO_RHD) {

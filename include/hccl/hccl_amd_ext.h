@@ -21,12 +21,12 @@ extern "C" {
  *   "buffsize_mib"  CCL buffer size that sets the chunk plan (default 200, as HCCL_BUFFSIZE);
  *   "buffsize_bytes" the same in bytes (tests of the chunk loop on small inputs)
  *   "align"         slice alignment in bytes (default 128)
- *   "servers"       number of rank groups for all-reduce, reduce-scatter and reduce: with n > 1 the p ranks form n groups of p / n
+ *   "servers"       number of rank groups for all-reduce, reduce-scatter, all-gather and reduce: with n > 1 the p ranks form n groups of p / n
  *                   consecutive ranks and the two-level schedules run (mesh inside a group, "algo" ring or rhd between;
  *                   with "auto": rhd for 2, 4, 8 or more groups, ring for 3, 5, 6, 7, the reference's default);
  *                   the all-to-all family then runs the staged schedule (gather inside a group into a workspace, pairwise
  *                   between the groups) unless "algo" is "pairwise"
- *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter / reduce: the mesh schedule
+ *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter / all-gather / reduce: the mesh schedule
  *                                (default), one ring in rank order, or -- for groups of 8 ranks, for the all-reduce also with one group --
  *                                the four rings of the 8-device ring topology, each on a quarter of every slice
  *   "step_stores"   "auto" | "nt" | "ordinary"   store kind of the step-by-step kernels (non-temporal, or write-back

@@ -1574,6 +1574,152 @@ int orc_allgather(int algo, uint32_t p, void **in, void **out, uint64_t sendCoun
     return 0;
 }
 
+// Two-level all-gather over `servers` groups of D = p / servers consecutive ranks
+// (CollAllGatherMeshExecutor::KernelRun, ALG/impl/coll_executor/coll_all_gather/coll_all_gather_mesh_executor.cc:71-175;
+// CollAllGatherRingExecutor::KernelRun, coll_all_gather_ring_executor.cc:81-200): every rank puts its block at its
+// place in the output staging buffer, the group gathers its D blocks (level0: 0 mesh, 2 one ring, 3 the four rings of
+// the 8-device topology on the parts MultiSegSlices cuts), then the ranks at position d of all groups gather the
+// groups' runs of D blocks, ring or recursive halving-doubling.  Chunks of cclBytes / p (rounded down to the
+// alignment with the mesh, :64-69; not with the rings, coll_all_gather_ring_executor.cc:75-79) per rank.
+int orc_allgather_two_level(int level1, int level0, uint32_t servers, uint32_t p, void **in, void **out, uint64_t sendCount, int dt,
+    uint64_t cclBytes, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || servers == 0 || p % servers != 0 || (level1 != ALGO_RING && level1 != ALGO_RHD) ||
+        (level0 != 0 && level0 != 2 && level0 != 3) || (level0 == 3 && p / servers != 8)) {
+        return -20;
+    }
+    const uint32_t D = p / servers;
+    const uint32_t ringCount = level0 == 3 ? 4u : 1u;
+    uint64_t maxPer = MaxCountPerLoop(2, cclBytes, p, unit, level0 == 0 ? align : 1);
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    auto machine = [&](uint32_t n) {
+        Machine m;
+        m.p = static_cast<int>(n);
+        m.dt = dt;
+        m.op = 0;
+        m.direct = (flags & 1) != 0;
+        m.pool = &pool;
+        m.buf[B_IN].resize(n);
+        m.buf[B_OUT].resize(n);
+        return m;
+    };
+    Machine all = machine(p);
+    uint64_t stage = std::min<uint64_t>(sendCount, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage)), cclOut(p, std::vector<uint8_t>(stage * p));
+    for (uint32_t r = 0; r < p; r++) {
+        all.buf[B_IN][r] = cclIn[r].data();
+        all.buf[B_OUT][r] = cclOut[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = sendCount; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            all.Copy(all.buf[B_IN][r], static_cast<uint8_t *>(in[r]) + offset, bytes);
+            all.Copy(all.buf[B_OUT][r] + bytes * r, all.buf[B_IN][r], bytes);    // own block to its place
+        }
+        // inside every group, on the group's run of D blocks
+        std::vector<Slice> segs(D);
+        for (uint32_t d = 0; d < D; d++) {
+            segs[d] = Slice{bytes * d, bytes};
+        }
+        for (uint32_t s = 0; s < servers && D > 1; s++) {
+            const uint64_t base = bytes * D * s;
+            if (level0 == 0) {
+                Machine m = machine(D);
+                for (uint32_t d = 0; d < D; d++) {
+                    m.buf[B_IN][d] = all.buf[B_IN][s * D + d];
+                    m.buf[B_OUT][d] = all.buf[B_OUT][s * D + d] + base;
+                    Proc pr;
+                    pr.rank = d;
+                    ProgAllGatherMesh(pr.prog, d, D, B_OUT, segs);
+                    m.procs.push_back(std::move(pr));
+                }
+                int rc = m.Run();
+                if (rc != 0) {
+                    return rc;
+                }
+                continue;
+            }
+            std::vector<std::vector<Slice>> parts = MultiSegSlices(segs, ringCount, align);
+            for (uint32_t k = 0; k < ringCount; k++) {
+                Machine ring = machine(D);
+                std::vector<Slice> ringSl(D);
+                for (uint32_t i = 0; i < D; i++) {
+                    uint32_t dev = ringCount > 1 ? kEightDeviceRings[k][i] : i;
+                    ring.buf[B_IN][i] = all.buf[B_IN][s * D + dev];
+                    ring.buf[B_OUT][i] = all.buf[B_OUT][s * D + dev] + base;
+                    ringSl[i] = ringCount > 1 ? parts[dev][k] : segs[dev];
+                }
+                for (uint32_t i = 0; i < D; i++) {
+                    Proc pr;
+                    pr.rank = i;
+                    ProgAllGatherRing(pr.prog, i, D, B_OUT, B_OUT, ringSl, ringSl);
+                    ring.procs.push_back(std::move(pr));
+                }
+                int rc = ring.Run();
+                if (rc != 0) {
+                    return rc;
+                }
+            }
+        }
+        // between the groups: the ranks at position d, on runs of D blocks
+        const uint64_t run = bytes * D;
+        for (uint32_t d = 0; d < D && servers > 1; d++) {
+            Machine m = machine(servers);
+            std::vector<Slice> runs(servers);
+            for (uint32_t s = 0; s < servers; s++) {
+                m.buf[B_IN][s] = all.buf[B_IN][s * D + d];
+                m.buf[B_OUT][s] = all.buf[B_OUT][s * D + d];
+                runs[s] = Slice{run * s, run};
+            }
+            for (uint32_t s = 0; s < servers; s++) {
+                Proc pr;
+                pr.rank = s;
+                if (level1 == ALGO_RING) {
+                    ProgAllGatherRing(pr.prog, s, servers, B_OUT, B_OUT, runs, runs);
+                } else {
+                    // AllGatherRecursiveHalvingDoubling::RunAsync, all_gather_recursive_hd.cc:26-238, data already in place
+                    uint32_t block, part1;
+                    std::vector<uint32_t> rankOf;
+                    std::vector<Slice> bsl;
+                    RhdBlockLayout(servers, run, &block, &part1, &rankOf, &bsl);
+                    if (s < part1 && (s % 2) == 1) {
+                        pr.prog.push_back(MkSend(static_cast<int>(s - 1), 1, B_OUT, run * s, run));
+                        pr.prog.push_back(MkRecvCopy(static_cast<int>(s - 1), 1, B_OUT, 0, run * servers));
+                    } else {
+                        if (s < part1) {
+                            pr.prog.push_back(MkRecvCopy(static_cast<int>(s + 1), 1, B_OUT, run * (s + 1), run));
+                        }
+                        uint32_t q = (s < part1) ? s / 2 : s - part1 / 2;
+                        ProgAllGatherHd(pr.prog, q, block, rankOf, B_OUT, bsl);
+                        if (s < part1) {
+                            pr.prog.push_back(MkSend(static_cast<int>(s + 1), 1, B_OUT, 0, run * servers));
+                        }
+                    }
+                }
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            for (uint32_t i = 0; i < p; i++) {
+                all.Copy(static_cast<uint8_t *>(out[r]) + sendCount * unit * i + offset, all.buf[B_OUT][r] + bytes * i, bytes);
+            }
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
 // Variable-count reduce-scatter: every rank's `in` holds the blocks {displs[i], counts[i]} (elements);
 // rank r receives the reduction of block r.  The templates run over these explicit slices
 // (reduce_scatter_ring.cc:179-297 takes any slice list; mesh and halving-doubling likewise).

@@ -60,6 +60,8 @@ def lib():
         L.orc_allreduce.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64, i32, i32, pu64]
         L.orc_reducescatter.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64, i32, i32]
         L.orc_allgather.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, u64, u64, i32, i32]
+        L.orc_allgather_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, u64, u64, i32, i32]
+        L.orc_allgather_two_level.restype = i32
         L.orc_reducescatter_v.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), pu64, pu64, i32, i32, u64, i32, i32]
         L.orc_allgather_v.argtypes = [i32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), pu64, pu64, i32, i32, i32]
         L.orc_broadcast.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
@@ -233,6 +235,20 @@ def allgather(ins, dt, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALI
     rc = lib().orc_allgather(algo, p, _ptrs(ins), _ptrs(outs), n, dt, ccl_bytes, align, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle allgather failed rc=%d" % rc)
+    return outs
+
+
+def allgather_two_level(ins, dt, servers, level1=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1,
+                        level0="mesh"):
+    """`servers` groups of consecutive ranks: the all-gather inside a group first (`level0`: "mesh", "ring" or
+    "ring4"), then `level1` (RING or RHD) between the groups."""
+    p = len(ins)
+    n = ins[0].size
+    outs = [np.empty(n * p, dtype=ins[0].dtype) for _ in range(p)]
+    mode = {"mesh": 0, "ring": 2, "ring4": 3}[level0]
+    rc = lib().orc_allgather_two_level(level1, mode, servers, p, _ptrs(ins), _ptrs(outs), n, dt, ccl_bytes, align, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle two-level allgather failed rc=%d" % rc)
     return outs
 
 

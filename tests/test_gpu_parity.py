@@ -910,6 +910,38 @@ def test_allreduce_on_a_rank_table_communicator(orc, tmp_path):
         H.comm_destroy(comms)
 
 
+def test_two_level_allgather_over_servers(orc):
+    # the group gathers first (mesh, ring or the four rings), then the ranks at the same position of the groups
+    # exchange the groups' blocks; fused the result is written in one pass, step by step in 1 + inside + between launches
+    for servers, D, level0 in ((2, 4, "mesh"), (4, 2, "ring"), (3, 4, "mesh"), (2, 8, "ring4"), (3, 8, "ring"), (5, 3, "mesh")):
+        p = servers * D
+        for level1 in (RING, RHD):
+            for dt, n, ccl in ((INT32, 70001, None), (BF16, 4099, None), (INT8, 100003, 64 << 10)):
+                ins = _ins(dt, p, n, 520 + p + n)
+                want = orc.allgather_two_level(ins, dt, servers, level1=level1, level0=level0,
+                                               **({"ccl_bytes": ccl} if ccl else {}))
+                for fuse in (1, 0):
+                    g = gh.Group(p, algo=ALGO_NAME[level1], servers=servers, level0=level0, fuse=fuse,
+                                 **({"buffsize_bytes": ccl} if ccl else {}))
+                    try:
+                        print("two-level all-gather", servers, D, level0, level1, dt, n, ccl, "fuse", fuse, flush=True)
+                        sends = [gh.to_dev(x) for x in ins]
+                        recvs = [gh.empty_dev(n * H.DTYPE_SIZE[dt] * p) for _ in range(p)]
+                        torch.cuda.synchronize()
+                        H.all_gather(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, g.stream_ptr)
+                        g.stream.synchronize()
+                        info = g.info()
+                        assert info["fused"] == fuse
+                        if not fuse and not ccl:
+                            inside = 1 if level0 == "mesh" else D - 1
+                            assert info["launches"] <= 1 + inside + (servers - 1 if level1 == RING else 4)
+                            assert info["launches"] < p - 1 or level0 != "mesh"      # fewer than the flat ring's
+                        for r in range(p):
+                            assert np.array_equal(gh.to_host(recvs[r], dt), want[r]), (servers, D, level0, level1, dt, fuse, r)
+                    finally:
+                        g.close()
+
+
 def test_default_schedule_between_servers_follows_the_reference_rule(orc):
     # no schedule asked for: halving-doubling between 2, 4 or 8 and more servers, ring between 3, 5, 6 or 7
     # (order-sensitive fp32 data, so the two give different bits and the check can tell them apart)

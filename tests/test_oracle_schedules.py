@@ -536,3 +536,17 @@ def test_order_sensitive_known_answers_four_rings(orc):
             assert all(np.array_equal(g, want) for g in got), (level0, level1, got[0][:4])
     closed = cf.two_level_ring_allreduce(FP32, SUM, xs, 4, 200 << 20, kat["align"], 1, cf.ring_allreduce, 4)
     assert np.array_equal(closed[0][:4], np.array(kat["expected_first4"]["ring4"], np.float32))
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("level0", ["mesh", "ring", "ring4"])
+def test_two_level_allgather_is_the_concatenation(orc, level1, level0):
+    shapes = ((1, 8), (2, 8), (3, 8)) if level0 == "ring4" else ((2, 4), (4, 2), (3, 4), (5, 3), (6, 1), (1, 5))
+    for servers, D in shapes:
+        p = servers * D
+        for dt, n, ccl in ((INT32, 1003, 200 << 20), (INT32, 777, 4096), (BF16, 301, 200 << 20), (INT8, 5000, 8192)):
+            ins = _inputs(dt, p, n, 31 * p + n)
+            got = orc.allgather_two_level(ins, dt, servers, level1=level1, level0=level0, ccl_bytes=ccl)
+            want = np.concatenate(ins)
+            for r in range(p):
+                assert np.array_equal(got[r], want), (servers, D, level1, level0, dt, ccl, r)

@@ -612,3 +612,47 @@ def test_planner_halving_doubling_slices_match_the_hand_derived_vectors(case):
     seen = {(s["dst"][2], s["n"]) for ph in plan["phases"] for s in ph}
     assert seen <= runs, (sorted(seen - runs), sorted(runs))
     assert {(o, s) for o, s in zip(off, size) if s} <= seen
+
+
+@pytest.mark.parametrize("level1", [RING, RHD])
+@pytest.mark.parametrize("level0", ["mesh", "ring", "ring4"])
+def test_two_level_allgather_plan_matches_checker(orc, level1, level0):
+    rings = {"mesh": 0, "ring": 1, "ring4": 4}[level0]
+    shapes = ((2, 8), (3, 8)) if rings == 4 else ((2, 4), (4, 2), (3, 4), (5, 3), (6, 1))
+    for servers, D in shapes:
+        p = servers * D
+        for dt, n, ccl in ((INT32, 1003, 200 << 20), (INT32, 777, 4096), (BF16, 301, 200 << 20)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n, 410 + p + n)
+            want = orc.allgather_two_level(ins, dt, servers, level1=level1, level0=level0, ccl_bytes=ccl)
+            plan = H.describe_plan(H.COLL_ALLGATHER, level1 | (servers << 8) | (rings << 17), p, n, dt, ccl_bytes=ccl)
+            if ccl >= n * unit * p:
+                # one chunk: the own copy, the group's phase(s), then the schedule between the groups
+                inside = 0 if D == 1 else (1 if rings == 0 else D - 1)
+                between = servers - 1 if level1 == RING else len(H.describe_plan(H.COLL_ALLGATHER, RHD, servers, 8, dt)["phases"]) - 1
+                # (an upper bound: the planner moves a step to the earliest phase its operands allow)
+                assert len(plan["phases"]) <= 1 + inside + between, (servers, D, level1, level0, len(plan["phases"]))
+            # the route, which the result cannot show: a block only moves inside a group or between two ranks
+            # at the same position of their groups, and every rank takes (servers - 1) * D blocks from other groups
+            crossing = [0] * p
+            for ph in plan["phases"]:
+                for st in ph:
+                    a, d = st["a"][0], st["dst"][0]
+                    assert a // D == d // D or a % D == d % D, (servers, D, level1, level0, a, d)
+                    if a // D != d // D:
+                        crossing[d] += st["n"]
+            if level1 == RING or servers & (servers - 1) == 0:
+                assert crossing == [(servers - 1) * D * n * unit] * p, (servers, D, level1, level0)
+            else:
+                # halving-doubling over a server count that is no power of two: the odd rank of a folded pair is
+                # handed the whole result, its own group's blocks included (all_gather_recursive_hd.cc:215-236)
+                assert all((servers - 1) * D * n * unit <= c <= p * n * unit for c in crossing), (servers, D, level0)
+            for fused in (False, True):
+                sends = _bytes(ins)
+                recvs = [np.full(n * unit * p, 0x5A, np.uint8) for _ in range(p)]
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, 0)
+                for r in range(p):
+                    assert np.array_equal(recvs[r].view(cf.CARRIER[dt]), want[r]), (servers, D, level1, level0, dt, ccl, fused, r)
+                    assert np.array_equal(sends[r], ins[r].view(np.uint8))
+            # fused, every rank's output is written once and every input read p times or less
+            assert sum(it["n"] * len(it["dst"]) for it in plan["fused"]) == p * p * n * unit

@@ -20,10 +20,10 @@ def _case(rng):
     ccl = int(rng.choice([200 << 20, 200 << 20, 4 * p * align, 4096, 4 * int(rng.integers(p, 40 * p))]))
     algo = int(rng.choice([RING, MESH, RHD, MESH_ATOMIC]))
     servers, rings = 1, 0
-    if coll in (H.COLL_ALLREDUCE, H.COLL_REDUCESCATTER, H.COLL_REDUCE) and rng.random() < 0.4:
+    if coll in (H.COLL_ALLREDUCE, H.COLL_REDUCESCATTER, H.COLL_REDUCE, H.COLL_ALLGATHER) and rng.random() < 0.4:
         servers = int(rng.choice([s for s in range(1, p + 1) if p % s == 0]))
         algo = int(rng.choice([RING, RHD]))
-        if coll in (H.COLL_ALLREDUCE, H.COLL_REDUCESCATTER) and rng.random() < 0.4 and (coll == H.COLL_ALLREDUCE or servers > 1):
+        if coll in (H.COLL_ALLREDUCE, H.COLL_REDUCESCATTER, H.COLL_ALLGATHER) and rng.random() < 0.4 and (coll == H.COLL_ALLREDUCE or servers > 1):
             rings = 4 if p // servers == 8 and rng.random() < 0.6 else 1
     mask = 0
     if coll == H.COLL_ALLREDUCE and rng.random() < 0.5:
@@ -44,7 +44,7 @@ def test_random_plans_compute_the_plain_result(seed):
         elif coll == H.COLL_REDUCESCATTER:
             word = algo | (servers << 8) | (rings << 17) if servers > 1 else algo
         elif coll == H.COLL_ALLGATHER:
-            word = algo
+            word = algo | (servers << 8) | (rings << 17) if servers > 1 else algo
         elif coll == H.COLL_REDUCE and servers > 1:
             word = root | (algo << 16) | (servers << 20)
         else:
@@ -59,7 +59,7 @@ def test_random_plans_compute_the_plain_result(seed):
         except Exception as e:   # noqa: BLE001
             # the only request the planner may turn down here: a buffer that holds no element per rank
             # under the executor's chunk rule (rounded down to the alignment, except in the two-level reduce-scatter)
-            if coll == H.COLL_REDUCESCATTER and servers > 1:
+            if (coll == H.COLL_REDUCESCATTER and servers > 1) or (coll == H.COLL_ALLGATHER and servers > 1 and rings):
                 per = ccl // (p * 4)
             elif coll in (H.COLL_REDUCESCATTER, H.COLL_ALLGATHER):
                 per = ccl // p // align * align // 4
