@@ -21,7 +21,8 @@
 //                    streams fixed to stream order: for floating point the reference itself has no single answer)
 //   two levels       EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240 (several servers),
 //                    EXE/coll_reduce_scatter/coll_reduce_scatter_mesh_executor.cc:114-119,128-247,
-//                    EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194 (several servers)
+//                    EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194 (several servers),
+//                    EXE/coll_all_gather/coll_all_gather_mesh_executor.cc:64-175, coll_all_gather_ring_executor.cc:75-200
 //   halving-doubling TPL/temp_all_reduce/all_reduce_recursive_hd.cc:33-302,
 //                    TPL/temp_reduce_scatter/reduce_scatter_recursive_hd.cc:33-254, TPL/temp_all_gather/all_gather_recursive_hd.cc:26-238,
 //                    TPL/temp_reduce_scatter/reduce_scatter_halving_doubling.cc:67-238,
