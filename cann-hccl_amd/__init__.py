@@ -129,6 +129,16 @@ def lib():
     if _lib is not None:
         return _lib
     if not os.path.exists(LIB_PATH):
+        # nothing built yet (a fresh checkout): build once, in tree; a built library is never rebuilt from here
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("cann_hccl_amd_build", os.path.join(os.path.dirname(__file__), "build.py"))
+        builder = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(builder)
+        try:
+            builder.build()
+        except Exception as e:   # noqa: BLE001
+            raise RuntimeError("libhccl.so is not built and building it failed (needs hipcc): %s" % e)
+    if not os.path.exists(LIB_PATH):
         raise RuntimeError("libhccl.so is not built: run `python cann-hccl_amd/build.py` (needs hipcc)")
     # Streams and device pointers handed to the library must belong to the HIP runtime the library
     # itself uses.  PyTorch ships its own libamdhip64 (same soname): when it is loaded first the
