@@ -79,7 +79,7 @@ def test_rhd_allreduce_bf16_128mib_per_rank(p):
     orc.build()
     n = 64 << 20                                     # bf16 elements per rank
     rng = np.random.default_rng(99 + p)
-    # bf16 bit patterns with exponents around 1.0 (no Inf / NaN), every rank a different rotation of one block
+    # bf16 bit patterns with exponents near 1.0 (no Inf / NaN), every rank a different rotation of one block
     base = (rng.integers(0, 2, n, dtype=np.uint16) << 15) | (rng.integers(118, 132, n, dtype=np.uint16) << 7) | \
         rng.integers(0, 128, n, dtype=np.uint16)
     ins = [np.roll(base, 1237 * r + 1) ^ np.uint16(r & 0x7f) for r in range(p)]
