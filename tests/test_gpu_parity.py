@@ -942,6 +942,57 @@ def test_two_level_allgather_over_servers(orc):
                         g.close()
 
 
+def test_overlapping_send_and_receive_buffers_are_staged(orc):
+    # a receive buffer that lies inside a send buffer (the in-place forms of reduce-scatter and all-gather, and an
+    # all-to-all whose output lands in its neighbour's input): the library copies the inputs aside first, so the
+    # results are those of the untouched inputs
+    p, n = 8, 5003
+    rng = np.random.default_rng(808)
+    for servers in (1, 2):
+        for fuse in (1, 0):
+            g = gh.Group(p, fuse=fuse, servers=servers)
+            try:
+                print("overlapping buffers servers", servers, "fuse", fuse, flush=True)
+                # reduce-scatter: rank r receives into block r of its own send buffer
+                ins = [rng.integers(-1000, 1000, n * p).astype(np.int32) for _ in range(p)]
+                total = np.sum(np.stack(ins).astype(np.int64), axis=0).astype(np.int32)
+                bufs = [torch.from_numpy(x).cuda() for x in ins]
+                torch.cuda.synchronize()
+                H.reduce_scatter(g.comms, [t.data_ptr() for t in bufs], [bufs[r][r * n:].data_ptr() for r in range(p)], n, INT32, SUM,
+                                 g.stream_ptr)
+                g.stream.synchronize()
+                assert g.info()["fused"] == 0 and g.info()["scratchBytes"] >= n * p * 4      # staged: never the fused form
+                for r in range(p):
+                    got = bufs[r].cpu().numpy()
+                    assert np.array_equal(got[r * n:(r + 1) * n], total[r * n:(r + 1) * n]), ("reduce-scatter", servers, fuse, r)
+                # all-gather: rank r sends block r of its own receive buffer
+                blocks = [rng.integers(-1000, 1000, n).astype(np.int32) for _ in range(p)]
+                outs = [torch.zeros(n * p, dtype=torch.int32, device="cuda") for _ in range(p)]
+                for r in range(p):
+                    outs[r][r * n:(r + 1) * n] = torch.from_numpy(blocks[r]).cuda()
+                torch.cuda.synchronize()
+                H.all_gather(g.comms, [outs[r][r * n:].data_ptr() for r in range(p)], [t.data_ptr() for t in outs], n, INT32, g.stream_ptr)
+                g.stream.synchronize()
+                for r in range(p):
+                    assert np.array_equal(outs[r].cpu().numpy(), np.concatenate(blocks)), ("all-gather", servers, fuse, r)
+                # all-to-all: rank r's receive buffer is rank r+1's send buffer
+                m = n // p
+                arena = torch.from_numpy(rng.integers(-1000, 1000, (p + 1) * m * p).astype(np.int32)).cuda()
+                before = arena.cpu().numpy().copy()
+                sends = [arena[(r + 1) * m * p:(r + 2) * m * p] for r in range(p)]
+                recvs = [arena[r * m * p:(r + 1) * m * p] for r in range(p)]
+                torch.cuda.synchronize()
+                H.all_to_all(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], m, INT32, g.stream_ptr)
+                g.stream.synchronize()
+                after = arena.cpu().numpy()
+                for j in range(p):
+                    for i in range(p):
+                        src = before[(i + 1) * m * p + j * m:(i + 1) * m * p + (j + 1) * m]
+                        assert np.array_equal(after[j * m * p + i * m:j * m * p + (i + 1) * m], src), ("all-to-all", servers, fuse, i, j)
+            finally:
+                g.close()
+
+
 def test_default_schedule_between_servers_follows_the_reference_rule(orc):
     # no schedule asked for: halving-doubling between 2, 4 or 8 and more servers, ring between 3, 5, 6 or 7
     # (order-sensitive fp32 data, so the two give different bits and the check can tell them apart)
