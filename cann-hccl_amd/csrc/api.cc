@@ -1530,6 +1530,9 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         // bit 29 / bit 30 = one ring / four rings inside a group instead of the mesh
         rq.root = uint32_t(algo) & 0xffffu;
         rq.algo = Algo((uint32_t(algo) >> 16) & 0xfu);
+        if (coll == COLL_SCATTER) {
+            rq.algo = ((uint32_t(algo) >> 20) & 1u) ? ALGO_RING : ALGO_MESH;   // scatter: bit 20 = the ring schedule
+        }
         if (coll == COLL_REDUCE) {
             rq.servers = std::max(1u, (uint32_t(algo) >> 20) & 0xffu);
             rq.meshAtomic = ((uint32_t(algo) >> 28) & 1u) != 0;

@@ -804,8 +804,10 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         algo = (algo == ALGO_MESH || algo == ALGO_RHD) ? algo : ALGO_RING;   // ring, mesh or halving-doubling reduce
     } else if (g->ctx->sig.coll == COLL_BROADCAST) {
         algo = (algo == ALGO_MESH || algo == ALGO_RHD) ? algo : ALGO_RING;   // ring, mesh or halving-doubling broadcast
+    } else if (g->ctx->sig.coll == COLL_SCATTER) {
+        algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_MESH;   // mesh scatter unless the ring is asked for
     } else if (g->ctx->sig.coll >= COLL_SCATTER) {
-        algo = ALGO_RING;   // one schedule each: mesh scatter, direct send / receive
+        algo = ALGO_RING;   // direct send / receive
     } else if (algo == ALGO_PAIRWISE) {
         algo = ALGO_RING;
     }

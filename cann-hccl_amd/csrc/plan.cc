@@ -735,6 +735,31 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
         }
         const uint32_t R = rq.root;
         uint64_t total = rq.count * u;
+        if (rq.coll == COLL_SCATTER && rq.algo == ALGO_RING && p > 1) {
+            // ring scatter (scatter_ring.cc:22-135,142-218): the root sends the blocks to its right neighbour one
+            // per step, the one with the longest way first (:38-52); every rank keeps the last block it receives
+            // and passes the others on (:77-118).  Blocks in transit lie in the rank's workspace (the reference's
+            // output staging buffer), at the block's own offset.
+            vp->workBytes.assign(p, 0);
+            vp->inBytes[R] = total * p;
+            EmitCopy(*vp, 0, MkRef(R, BUF_RECV, 0), MkRef(R, BUF_SEND, uint64_t(R) * total), total);
+            vp->outBytes[R] = total;
+            for (uint32_t j = 1; j < p; j++) {            // j = hops from the root to the block's owner
+                const uint32_t dest = (R + j) % p;
+                for (uint32_t h = 1; h <= j; h++) {
+                    const uint32_t from = (R + h - 1) % p, to = (R + h) % p;
+                    // (a rank in transit is never the root: its input buffer is empty and all of it is workspace)
+                    const Ref src = MkRef(from, BUF_SEND, uint64_t(dest) * total);
+                    const Ref dst = h == j ? MkRef(dest, BUF_RECV, 0) : MkRef(to, BUF_SEND, uint64_t(dest) * total);
+                    EmitCopy(*vp, size_t(p - j + h - 2), dst, src, total);
+                    if (h != j) {
+                        vp->workBytes[to] = std::max(vp->workBytes[to], uint64_t(dest + 1) * total);
+                    }
+                }
+                vp->outBytes[dest] = total;
+            }
+            return 0;
+        }
         if (rq.coll == COLL_SCATTER) {
             // mesh scatter (scatter_mesh.cc:46-160): the root hands rank i block i, all at once
             for (uint32_t r = 0; r < p; r++) {

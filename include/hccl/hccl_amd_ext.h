@@ -13,7 +13,8 @@ extern "C" {
 
 /* Settings of the communicator's whole group.  Keys and values:
  *   "algo"          "ring" | "mesh" | "rhd" | "pairwise" | "auto"   ("pairwise" only matters to the all-to-all family,
- *                                see "servers"; the other collectives then run their ring schedules)
+ *                                see "servers"; the other collectives then run their ring schedules; the scatter runs
+ *                                the mesh schedule unless "ring" is set)
  *   "deterministic" "0" | "1"    as HCCL_DETERMINISTIC; with "0" (the default) the mesh reduce phases of
  *                                all-reduce / reduce-scatter run without the piece cut (not for int64, not for products)
  *   "fuse"          "0" | "1"    run the single-pass fused form when the schedule has one
@@ -65,10 +66,12 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
  * collectives (coll 4 broadcast, 5 reduce, 6 scatter) the algo argument carries the root rank in its low 16 bits and the
  * schedule in bits 16..19 (0 ring, 1 mesh, 2 rhd, 4 mesh without the piece cut), for the reduce also the number of rank
  * groups of its two-level schedule in bits 20..27, bit 28 for the mesh level without the piece cut and bit 29 / bit 30 for
- * one ring / four rings inside a group; for the all-reduce (coll 0) bits 8..15 of algo
+ * one ring / four rings inside a group, for the scatter bit 20 for the ring schedule instead of the mesh;
+ * for the all-reduce (coll 0) bits 8..15 of algo
  * carry the number of rank groups of the two-level schedule (0 or 1: one level), bit 16 asks for its mesh level
  * without the piece cut and bits 17..19 give the rings inside a group (0: mesh, 1, or 4); the reduce-scatter (coll 1)
- * takes bits 8..19 the same way.  inPlaceMask bit r:
+ * and the all-gather (coll 2) take bits 8..19 the same way; for the all-to-all-v (coll 3) bits 8..15 give the number
+ * of servers of the staged schedule.  inPlaceMask bit r:
  * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64
  * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); for the variable-count
  * reduce-scatter / all-gather, tables points to 2*p uint64 (block counts, block displacements); else NULL.

@@ -2547,6 +2547,64 @@ int orc_scatter(uint32_t p, const void *inRoot, void **out, uint64_t count, int 
     return m.Run();
 }
 
+// Ring scatter (TPL/temp_scatter/scatter_ring.cc:22-135,142-218): the root sends the blocks to its right neighbour
+// one after the other, the block of the rank before it first (:38-52); a rank in between receives the blocks of all
+// ranks from the one before the root down to itself, passes each on before taking the next and keeps the last, its
+// own (:77-118); the rank before the root only receives (:55-71).  Blocks travel through an output staging buffer
+// of p blocks per rank, each at its own offset.
+int orc_scatter_ring(uint32_t p, const void *inRoot, void **out, uint64_t count, int dt, uint32_t root, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t bytes = count * unit;
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    std::vector<std::vector<uint8_t>> stage(p, std::vector<uint8_t>(bytes * p + 1));
+    m.buf[B_IN].assign(p, nullptr);
+    m.buf[B_OUT].resize(p);
+    m.buf[B_IN][root] = static_cast<uint8_t *>(const_cast<void *>(inRoot));
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_OUT][r] = stage[r].data();
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        const int left = static_cast<int>((r + p - 1) % p), right = static_cast<int>((r + 1) % p);
+        if (p == 1 || r == root) {
+            pr.prog.push_back(MkLocalCopy(B_OUT, bytes * r, B_IN, bytes * r, bytes));
+            for (uint32_t i = 1; i < p; i++) {
+                uint32_t owner = (r + p - i) % p;
+                pr.prog.push_back(MkSend(right, 0, B_IN, bytes * owner, bytes));
+            }
+        } else {
+            const uint32_t rounds = (root + p - r) % p;          // blocks this rank receives, its own last
+            for (uint32_t i = 1; i <= rounds; i++) {
+                uint32_t owner = (r + rounds - i) % p;
+                if (i != 1) {
+                    uint32_t previous = (r + rounds - i + 1) % p;
+                    pr.prog.push_back(MkSend(right, 0, B_OUT, bytes * previous, bytes));
+                }
+                pr.prog.push_back(MkRecvCopy(left, 0, B_OUT, bytes * owner, bytes));
+            }
+        }
+        m.procs.push_back(std::move(pr));
+    }
+    int rc = m.Run();
+    if (rc != 0) {
+        return rc;
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        m.Copy(static_cast<uint8_t *>(out[r]), stage[r].data() + bytes * r, bytes);
+    }
+    return 0;
+}
+
 // PairWise all-to-all-v.  counts / displs are p x p row-major tables in elements: row r is what
 // rank r passed to HcclAlltoAllV.  Returns 1 if the send / receive tables are not symmetric
 // (alltoall_operator.cc:49-72), 0 on success.

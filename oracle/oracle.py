@@ -76,6 +76,8 @@ def lib():
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
         L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
+        L.orc_scatter_ring.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
+        L.orc_scatter_ring.restype = i32
         L.orc_alltoallv.argtypes = [u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, u64, i32, i32]
         L.orc_alltoallv_staged.argtypes = [u32, u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, i32, i32]
         L.orc_alltoallv_staged.restype = i32
@@ -315,10 +317,12 @@ def reduce_to_root_two_level(ins, dt, op, root, servers, level1=RING, atomic=Fal
     return out
 
 
-def scatter(src, p, dt, root, flags=0, threads=1):
+def scatter(src, p, dt, root, flags=0, threads=1, algo=MESH):
+    """algo: MESH (the root hands every rank its block directly) or RING (the blocks travel round the ring)."""
     n = src.size // p
     outs = [np.empty(n, dtype=src.dtype) for _ in range(p)]
-    rc = lib().orc_scatter(p, src.ctypes.data, _ptrs(outs), n, dt, root, flags, threads)
+    fn = lib().orc_scatter_ring if algo == RING else lib().orc_scatter
+    rc = fn(p, src.ctypes.data, _ptrs(outs), n, dt, root, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle scatter failed rc=%d" % rc)
     return outs

@@ -581,6 +581,36 @@ def test_broadcast_reduce_scatter_rooted(orc):
                 g.close()
 
 
+def test_ring_scatter(orc):
+    # the ring schedule for the scatter: step by step the blocks rest in the ranks' workspace on their way round
+    n = 30011
+    for p in (2, 3, 8, 13):
+        for fuse in (1, 0):
+            g = gh.Group(p, algo="ring", fuse=fuse)
+            try:
+                for root in sorted({0, p - 1, p // 2}):
+                    print("ring scatter p", p, "fuse", fuse, "root", root, flush=True)
+                    src = (np.arange(n * p, dtype=np.int64) * 2654435761 % (1 << 31)).astype(np.int32)
+                    want = orc.scatter(src, p, INT32, root, algo=RING)
+                    sends = [gh.to_dev(src) if r == root else None for r in range(p)]
+                    recvs = [gh.empty_dev(n * 4) for _ in range(p)]
+                    torch.cuda.synchronize()
+                    H.scatter(g.comms, [t.data_ptr() if t is not None else None for t in sends], [t.data_ptr() for t in recvs],
+                              n, INT32, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    info = g.info()
+                    assert info["fused"] == fuse
+                    if fuse:
+                        assert info["bytesWritten"] == n * 4 * p and info["scratchBytes"] == 0
+                    else:
+                        assert info["launches"] == p - 1 and info["bytesWritten"] == n * 4 * (1 + p * (p - 1) // 2)
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(recvs[r], INT32), want[r]), ("ring scatter", p, fuse, root, r)
+                    assert np.array_equal(gh.to_host(sends[root], INT32), src)
+            finally:
+                g.close()
+
+
 def test_order_sensitive_known_answers_on_the_gpu():
     # hand-derived fp32 sums that differ between ring, the two mesh variants and halving-doubling
     import json

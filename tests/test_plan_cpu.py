@@ -656,3 +656,31 @@ def test_two_level_allgather_plan_matches_checker(orc, level1, level0):
                     assert np.array_equal(sends[r], ins[r].view(np.uint8))
             # fused, every rank's output is written once and every input read p times or less
             assert sum(it["n"] * len(it["dst"]) for it in plan["fused"]) == p * p * n * unit
+
+
+@pytest.mark.parametrize("p", [1, 2, 3, 5, 8, 13])
+def test_ring_scatter_plan_matches_checker(orc, p):
+    # the blocks travel round the ring, the farthest first; step by step they rest in the ranks' workspace on the way
+    n = 257
+    rng = np.random.default_rng(90 + p)
+    for root in sorted({0, p - 1, p // 2}):
+        src = rng.integers(0, 1 << 30, n * p).astype(np.int32)
+        want = orc.scatter(src, p, INT32, root, algo=RING)
+        for r in range(p):
+            assert np.array_equal(want[r], src[r * n:(r + 1) * n]), (p, root, r)          # the definition
+        plan = H.describe_plan(H.COLL_SCATTER, root | (1 << 20), p, n, INT32)
+        if p > 1:
+            assert len(plan["phases"]) == p - 1                                          # one block leaves the root per step
+            hops = sum(1 for ph in plan["phases"] for s in ph) - 1                       # minus the root's own copy
+            assert hops == p * (p - 1) // 2                                              # block of distance j takes j hops
+            for ph in plan["phases"]:
+                for s in ph:
+                    a, d = s["a"][0], s["dst"][0]
+                    assert d == a or d == (a + 1) % p, (p, root, a, d)                    # only to the right neighbour
+        assert sum(it["n"] for it in plan["fused"]) == n * 4 * p                         # fused: every block moves once
+        for fused in (False, True):
+            sends = [src.view(np.uint8).copy() if r == root else np.zeros(0, np.uint8) for r in range(p)]
+            recvs = [np.zeros(n * 4, np.uint8) for _ in range(p)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, INT32, 0)
+            for r in range(p):
+                assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, root, fused, r)
