@@ -648,6 +648,45 @@ void TwoLevelReduceChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t servers
     vp.phaseBase = 0;
 }
 
+// Recursive halving-doubling broadcast (bcast_recursive_halvingdoubling.cc:21-290) among n ranks, data(i) naming
+// rank i's copy of the chunk: a binomial tree over the block, whole chunk per hop, widest distance first (:162-203);
+// the block holds the root and, of every rank pair of part one, the rank with the root's parity (:120-160);
+// afterwards that rank hands the chunk to its neighbour (:205-262).  Returns the phase after the last one used.
+template <typename F> size_t RhdBroadcastPhases(VProgram &vp, size_t ph, uint32_t n, uint32_t root, F data, uint64_t bytes)
+{
+    uint32_t block, part1;
+    HalvingDoublingShape(n, &block, &part1);
+    const uint32_t par = (root < part1 && (root % 2) == 1) ? 1u : 0u;
+    std::vector<uint32_t> rankOf(block);
+    for (uint32_t b = 0; b < block; b++) {
+        rankOf[b] = b < part1 / 2 ? 2 * b + par : b + part1 / 2;
+    }
+    const uint32_t rootQ = root < part1 ? root / 2 : root - part1 / 2;
+    uint32_t rounds = 0;
+    while ((1u << rounds) < block) {
+        rounds++;
+    }
+    std::vector<uint8_t> has(block, 0);
+    has[rootQ] = 1;
+    for (uint32_t i = 0; i < rounds; i++, ph++) {
+        const uint32_t mask = 1u << (rounds - i - 1);
+        std::vector<uint32_t> got;
+        for (uint32_t q = 0; q < block; q++) {
+            if (has[q] && (q & (mask - 1)) == (rootQ & (mask - 1)) && !has[q ^ mask]) {
+                EmitCopy(vp, ph, data(rankOf[q ^ mask]), data(rankOf[q]), bytes);
+                got.push_back(q ^ mask);
+            }
+        }
+        for (uint32_t q : got) {
+            has[q] = 1;
+        }
+    }
+    for (uint32_t b = 0; b < part1 / 2; b++) {
+        EmitCopy(vp, ph, data(rankOf[b] ^ 1u), data(rankOf[b]), bytes);
+    }
+    return part1 > 0 ? ph + 1 : ph;
+}
+
 int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
 {
     uint32_t p = rq.p;
@@ -803,42 +842,8 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                     }
                 }
             } else if (rq.coll == COLL_BROADCAST && rq.algo == ALGO_RHD && p > 1) {
-                // recursive halving-doubling broadcast (bcast_recursive_halvingdoubling.cc:21-290): a binomial
-                // tree over the block, whole chunk per hop, widest distance first (:162-203); the block holds
-                // the root and, of every rank pair of part one, the rank with the root's parity (:120-160);
-                // afterwards that rank hands the chunk to its neighbour (:205-262)
-                uint32_t block, part1;
-                HalvingDoublingShape(p, &block, &part1);
-                const uint32_t par = (R < part1 && (R % 2) == 1) ? 1u : 0u;
-                std::vector<uint32_t> rankOf(block);
-                for (uint32_t b = 0; b < block; b++) {
-                    rankOf[b] = b < part1 / 2 ? 2 * b + par : b + part1 / 2;
-                }
-                const uint32_t rootQ = R < part1 ? R / 2 : R - part1 / 2;
                 auto data = [&](uint32_t r) { return r == R ? MkRef(R, BUF_SEND, done) : MkRef(r, BUF_RECV, done); };
-                uint32_t rounds = 0;
-                while ((1u << rounds) < block) {
-                    rounds++;
-                }
-                std::vector<uint8_t> has(block, 0);
-                has[rootQ] = 1;
-                size_t ph = 0;
-                for (uint32_t i = 0; i < rounds; i++, ph++) {
-                    const uint32_t mask = 1u << (rounds - i - 1);
-                    std::vector<uint32_t> got;
-                    for (uint32_t q = 0; q < block; q++) {
-                        if (has[q] && (q & (mask - 1)) == (rootQ & (mask - 1)) && !has[q ^ mask]) {
-                            EmitCopy(*vp, ph, data(rankOf[q ^ mask]), data(rankOf[q]), bytes);
-                            got.push_back(q ^ mask);
-                        }
-                    }
-                    for (uint32_t q : got) {
-                        has[q] = 1;
-                    }
-                }
-                for (uint32_t b = 0; b < part1 / 2; b++) {
-                    EmitCopy(*vp, ph, data(rankOf[b] ^ 1u), data(rankOf[b]), bytes);
-                }
+                RhdBroadcastPhases(*vp, 0, p, R, data, bytes);
             } else if (rq.coll == COLL_REDUCE && rq.servers > 1 && p > 1) {
                 TwoLevelReduceChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, rq.level0Rings, R, done, bytes,
                     rq.align, rq.meshAtomic);
