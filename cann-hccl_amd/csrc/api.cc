@@ -1533,6 +1533,9 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         if (coll == COLL_SCATTER) {
             rq.algo = ((uint32_t(algo) >> 20) & 1u) ? ALGO_RING : ALGO_MESH;   // scatter: bit 20 = the ring schedule
         }
+        if (coll == COLL_BROADCAST) {
+            rq.servers = std::max(1u, (uint32_t(algo) >> 20) & 0xffu);   // broadcast: bits 20..27 = rank groups (two levels)
+        }
         if (coll == COLL_REDUCE) {
             rq.servers = std::max(1u, (uint32_t(algo) >> 20) & 0xffu);
             rq.meshAtomic = ((uint32_t(algo) >> 28) & 1u) != 0;

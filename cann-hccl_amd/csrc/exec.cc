@@ -484,7 +484,7 @@ std::string CacheKey(const Group *g, int algo)
     uint64_t head[10] = {uint64_t(g->ctx->sig.coll), uint64_t(algo), uint64_t(g->ctx->sig.dtype), uint64_t(g->ctx->sig.op), g->ctx->sig.count,
         uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1) | (uint64_t(g->ctx->sig.root) << 8) | (uint64_t(g->ctx->sig.peer) << 20), g->cfg.cclBytes, g->cfg.align,
         uint64_t(g->cfg.blocksPerCu) | (uint64_t(uint32_t(g->cfg.stepStores + 1)) << 32) | (uint64_t(g->cfg.servers) << 40) |
-            (uint64_t(g->cfg.algo == ALGO_PAIRWISE ? 1 : 0) << 48) | (uint64_t(g->cfg.deterministic) << 56) | (uint64_t(g->cfg.level0Rings) << 57) |
+            (uint64_t(uint32_t(g->cfg.algo + 1) & 0xfu) << 48) | (uint64_t(g->cfg.deterministic) << 56) | (uint64_t(g->cfg.level0Rings) << 57) |
             (uint64_t(uint32_t(g->cfg.fusedStores + 1)) << 60) | (uint64_t(g->cfg.stepSweep) << 62), g->p};
     put(head, sizeof(head));
     put(g->ctx->send.data(), g->ctx->send.size() * sizeof(void *));
@@ -598,6 +598,12 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         rq.servers = g->cfg.servers;
         rq.algo = Level1Algo(g);
         rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
+    }
+    if (rq.coll == COLL_BROADCAST && g->cfg.servers > 1 && g->p % g->cfg.servers == 0 && g->cfg.algo != ALGO_RING &&
+        g->cfg.level0Rings == 0) {
+        // two levels (coll_broadcast_mesh_executor.cc:59-213): scatter in the root's group, halving-doubling between
+        // the groups, mesh all-gather in every group; the flat ring when the ring is asked for by name
+        rq.servers = g->cfg.servers;
     }
     if (rq.coll == COLL_REDUCE && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
         // two levels (coll_reduce_mesh_executor.cc:75-194, coll_reduce_ring_plus_hd_executor.cc:75-168): inside the

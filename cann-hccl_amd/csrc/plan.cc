@@ -816,7 +816,42 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
         uint64_t done = 0;
         for (uint64_t left = rq.count; left > 0;) {
             uint64_t cur = std::min(left, per), bytes = cur * u;
-            if (rq.coll == COLL_BROADCAST && rq.algo == ALGO_MESH) {
+            if (rq.coll == COLL_BROADCAST && rq.servers > 1 && p > 1) {
+                // Two levels (coll_broadcast_mesh_executor.cc:59-213 with several servers): the root scatters slice d
+                // to position d of its own group (scatter_mesh.cc), the ranks at position d of all groups pass it on by
+                // recursive halving-doubling from the root's group, and every group gathers the slices (mesh).
+                // The root keeps its data where it is.
+                const uint32_t S = rq.servers, D = p / S, rootGroup = R / D;
+                uint64_t avg = bytes / D + ((cur % D) > 0 ? 1 : 0);
+                uint64_t slice = RoundUpTo(avg, rq.align);
+                std::vector<Slice> sl(D);
+                uint64_t residue = bytes;
+                for (uint32_t i = 0; i < D; i++) {
+                    sl[i].size = std::min(slice, residue);
+                    sl[i].off = sl[i].size == 0 ? 0 : uint64_t(i) * slice;
+                    residue -= sl[i].size;
+                }
+                auto at = [&](uint32_t r, uint32_t d) {
+                    return r == R ? MkRef(R, BUF_SEND, done + sl[d].off) : MkRef(r, BUF_RECV, done + sl[d].off);
+                };
+                for (uint32_t d = 0; d < D; d++) {
+                    const uint32_t holder = rootGroup * D + d;
+                    if (holder != R) {
+                        EmitCopy(*vp, 0, at(holder, d), at(R, d), sl[d].size);
+                    }
+                }
+                size_t gather = 1;
+                for (uint32_t d = 0; d < D; d++) {
+                    auto data = [&](uint32_t g) { return at(g * D + d, d); };
+                    gather = std::max(gather, RhdBroadcastPhases(*vp, 1, S, rootGroup, data, sl[d].size));
+                }
+                for (uint32_t r = 0; r < p; r++) {
+                    for (uint32_t k = 1; k < D && r != R; k++) {
+                        const uint32_t d = (r % D + k) % D, from = r / D * D + d;
+                        EmitCopy(*vp, gather, at(r, d), at(from, d), sl[d].size);
+                    }
+                }
+            } else if (rq.coll == COLL_BROADCAST && rq.algo == ALGO_MESH) {
                 // mesh broadcast (coll_broadcast_mesh_executor.cc:59-213): the root scatters slice i to
                 // rank i (scatter_mesh.cc), then a mesh all-gather; slices from GetRankSliceSize
                 // (coll_broadcast_executor.cc:275-306).  The root keeps its data where it is.

@@ -1023,6 +1023,46 @@ def test_overlapping_send_and_receive_buffers_are_staged(orc):
                 g.close()
 
 
+def test_two_level_broadcast_and_schedule_switch_on_the_same_buffers(orc):
+    # broadcast over several groups: scatter in the root's group, halving-doubling between the groups, all-gather in
+    # every group.  Then the schedule setting changes while the buffers stay: the prepared collective of the old
+    # setting must not be reused (two-level all-reduce with the default schedule between the groups, then ring)
+    n = 70001
+    for servers, D in ((2, 4), (3, 4), (4, 2)):
+        p = servers * D
+        for fuse in (1, 0):
+            g = gh.Group(p, servers=servers, fuse=fuse)
+            try:
+                print("two-level broadcast", servers, D, "fuse", fuse, flush=True)
+                for root in (0, p - 1, D + 1):
+                    bufs_np = _ins(INT32, p, n, 640 + p + root)
+                    bufs = [gh.to_dev(x) for x in bufs_np]
+                    torch.cuda.synchronize()
+                    H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, INT32, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    info = g.info()
+                    if not fuse:
+                        assert info["launches"] >= 3                         # scatter, between the groups, gather
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(bufs[r], INT32), bufs_np[root]), (servers, D, fuse, root, r)
+                ins = _ins(FP32, p, n, 650 + p)
+                ins[0][:] *= 1e7
+                ins[p - 1][:] *= -1e7
+                sends = [gh.to_dev(x) for x in ins]
+                recvs = [gh.empty_dev(n * 4) for _ in range(p)]
+                torch.cuda.synchronize()
+                default = RHD if servers & (servers - 1) == 0 else RING
+                for setting, level1 in (("auto", default), ("ring", RING), ("rhd", RHD), ("auto", default)):
+                    H.set_param(g.comms[0], "algo", setting)
+                    want = orc.allreduce_two_level(ins, FP32, SUM, servers, level1=level1, atomic=True)
+                    H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, g.stream_ptr)
+                    g.stream.synchronize()
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(recvs[r], FP32), want[r]), (servers, D, fuse, setting, r)
+            finally:
+                g.close()
+
+
 def test_default_schedule_between_servers_follows_the_reference_rule(orc):
     # no schedule asked for: halving-doubling between 2, 4 or 8 and more servers, ring between 3, 5, 6 or 7
     # (order-sensitive fp32 data, so the two give different bits and the check can tell them apart)

@@ -684,3 +684,31 @@ def test_ring_scatter_plan_matches_checker(orc, p):
             (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, INT32, 0)
             for r in range(p):
                 assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, root, fused, r)
+
+
+@pytest.mark.parametrize("servers,D", [(2, 4), (4, 2), (3, 4), (5, 3), (6, 1), (2, 8)])
+def test_two_level_broadcast_plan(servers, D):
+    # scatter inside the root's group, halving-doubling between the groups, all-gather inside every group:
+    # every rank ends with the root's data, and a block only moves inside a group or between equal positions
+    p = servers * D
+    n = 1003
+    rng = np.random.default_rng(600 + p)
+    for root in sorted({0, p - 1, (D + 1) % p}):
+        for ccl in (200 << 20, 1024):
+            bufs = [rng.integers(0, 1 << 30, n).astype(np.int32) for _ in range(p)]
+            plan = H.describe_plan(H.COLL_BROADCAST, root | (MESH << 16) | (servers << 20), p, n, INT32, ccl_bytes=ccl,
+                                   in_place_mask=(1 << p) - 1)
+            for ph in plan["phases"]:
+                for st in ph:
+                    a, d = st["a"][0], st["dst"][0]
+                    assert a // D == d // D or a % D == d % D, (servers, D, root, a, d)
+                    assert d != root                                             # the root's data stays where it is
+            if ccl >= n * 4 and D > 1 and servers > 1:
+                flat = H.describe_plan(H.COLL_BROADCAST, root | (MESH << 16), p, n, INT32, in_place_mask=(1 << p) - 1)
+                assert len(plan["phases"]) > len(flat["phases"])                 # two more stages than scatter + gather
+            for fused in (False, True):
+                sends = _bytes(bufs)
+                recvs = [s for s in sends]                                       # one buffer per rank
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, INT32, 0, in_place=True)
+                for r in range(p):
+                    assert np.array_equal(recvs[r].view(np.int32), bufs[root]), (servers, D, root, ccl, fused, r)
