@@ -11,7 +11,7 @@ default, the fused single pass that reads every rank's input once and writes eve
 (2 * p * S bytes, same bits, about half the time), is timed in the same run and reported under
 `config.fused_single_pass` and `roofline_fused`.
 
-    python bench.py [--steps K] [--warmup W] [--size-mib M] [--sweep] [--suite] [--latency] [--probe] [--no-cpu]
+    python bench.py [--steps K] [--warmup W] [--size-mib M] [--sweep] [--suite] [--no-cpu]
 """
 import argparse
 import json
@@ -302,32 +302,12 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 1 GiB int32 copy (one-rank all-reduce, out of place) three times, so that a "
                          "counter profile of this command holds a copy of known size to scale FETCH_SIZE / WRITE_SIZE by")
-    ap.add_argument("--probe", action="store_true",
-                    help="run the stand-alone memory-bandwidth probe (cann-hccl_amd/lib/hbm_probe: plain kernels, n streams "
-                         "read : m written) and exit; its rates bound what the collectives can reach for the same mix")
-    ap.add_argument("--latency", action="store_true",
-                    help="run the compiled small-message timing (cann-hccl_amd/lib/call_latency: issue cost, back-to-back device "
-                         "time and call-to-completion time of 8 KiB ... 4 MiB all-reduces through the C ABI) and exit")
     ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
                     help="library setting for the run (see HcclAmdSetParam), e.g. --set blocks_per_cu=4")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is built and measured on one GPU (the ranks of the communicator are "
                  "simulated inside it); --gpus %d is not supported" % args.gpus)
-
-    if args.latency:
-        import subprocess
-        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cann-hccl_amd", "lib", "call_latency")
-        if not os.path.exists(exe):
-            sys.exit("bench.py: %s is not built (python cann-hccl_amd/build.py)" % exe)
-        rc = subprocess.run([exe, "1"]).returncode
-        sys.exit(rc or subprocess.run([exe, "0"]).returncode)
-    if args.probe:
-        import subprocess
-        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cann-hccl_amd", "lib", "hbm_probe")
-        if not os.path.exists(exe):
-            sys.exit("bench.py: %s is not built (python cann-hccl_amd/build.py)" % exe)
-        sys.exit(subprocess.run([exe, str(int(args.size_mib))]).returncode)
 
     import numpy as np
     import torch

@@ -17,8 +17,6 @@ OBJ = os.path.join(HERE, "build")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libhccl.so")
 ABI_CALLER = os.path.join(LIBDIR, "abi_caller")
-PROBE = os.path.join(LIBDIR, "hbm_probe")
-CALL_LATENCY = os.path.join(LIBDIR, "call_latency")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
@@ -70,26 +68,7 @@ def build(force=False, jobs=None):
     if force or tasks or _newer(LIB, objs):
         _run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs + ["-lpthread"])
     build_abi_caller(force)
-    build_probe(force)
-    build_call_latency(force)
     return LIB
-
-
-def build_probe(force=False):
-    """The stand-alone memory-bandwidth probe (csrc/hbm_probe.hip -> lib/hbm_probe)."""
-    src = os.path.join(CSRC, "hbm_probe.hip")
-    if force or _newer(PROBE, [src]):
-        _run([HIPCC, "-O3", "-std=c++17", "-Wno-unused-command-line-argument"] + DEVICE + [src, "-o", PROBE])
-    return PROBE
-
-
-def build_call_latency(force=False):
-    """Small-message timing of a compiled caller (csrc/call_latency.cc -> lib/call_latency)."""
-    src = os.path.join(CSRC, "call_latency.cc")
-    if force or _newer(CALL_LATENCY, [src, LIB]):
-        _run([HIPCC, "-O2", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-Wno-unused-command-line-argument", "-Wno-unused-result",
-              "-I", os.path.join(ROOT, "include"), src, "-L", LIBDIR, "-lhccl", "-Wl,-rpath,$ORIGIN", "-o", CALL_LATENCY])
-    return CALL_LATENCY
 
 
 def build_abi_caller(force=False, include_dirs=None, out=None):
