@@ -38,7 +38,7 @@ EXPORTS = [
     "HcclCommInitClusterInfoConfig", "HcclCreateSubCommConfig", "HcclGetRootInfo", "HcclCommInitRootInfo",
     "HcclCommInitRootInfoConfig", "HcclBroadcast", "HcclScatter", "HcclSend", "HcclRecv", "HcclReduce",
     "HcclBatchSendRecv", "HcclCommSetMemoryRange", "HcclCommUnsetMemoryRange", "HcclCommActivateCommMemory",
-    "HcclCommDeactivateCommMemory", "HcclAmdSetParam", "HcclAmdGetLastOpInfo", "HcclAmdDescribePlan",
+    "HcclCommDeactivateCommMemory", "HcclAmdSetParam", "HcclAmdGetLastOpInfo", "HcclAmdDescribePlan", "HcclAmdReduceScatterNoAlloc",
 ]
 
 
@@ -157,6 +157,7 @@ def lib():
     L.HcclGetCommName.argtypes = [vp, ctypes.c_char_p]
     L.HcclAllReduce.argtypes = [vp, vp, u64, i32, i32, vp, vp]
     L.HcclReduceScatter.argtypes = [vp, vp, u64, i32, i32, vp, vp]
+    L.HcclAmdReduceScatterNoAlloc.argtypes = [vp, vp, u64, i32, i32, vp, vp]
     L.HcclAllGather.argtypes = [vp, vp, u64, i32, vp, vp]
     L.HcclAlltoAllV.argtypes = [vp, vp, vp, i32, vp, vp, vp, i32, vp, vp]
     L.HcclAlltoAll.argtypes = [vp, u64, i32, vp, u64, i32, vp, vp]
@@ -235,6 +236,12 @@ def all_reduce(comms, sends, recvs, count, dtype, op, stream):
 def reduce_scatter(comms, sends, recvs, recv_count, dtype, op, stream):
     for c, s, r in zip(comms, sends, recvs):
         _check("HcclReduceScatter", lib().HcclReduceScatter(s, r, recv_count, dtype, op, c, stream))
+
+
+def reduce_scatter_no_alloc(comms, sends, recvs, recv_count, dtype, op, stream):
+    """HcclAmdReduceScatterNoAlloc on every rank: the reduce-scatter out of the fixed device workspace."""
+    for c, s, r in zip(comms, sends, recvs):
+        _check("HcclAmdReduceScatterNoAlloc", lib().HcclAmdReduceScatterNoAlloc(s, r, recv_count, dtype, op, c, stream))
 
 
 def all_gather(comms, sends, recvs, send_count, dtype, stream):

@@ -24,6 +24,7 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-I", os.path.join(
 # gfx950 only; packed fp32 instructions are switched off for device code
 DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 DTYPES = list(range(12)) + [255]
+DEVICE_SOURCES = ["noalloc.hip"]
 HOST_SOURCES = ["plan.cc", "ranktable.cc", "exec.cc", "api.cc", "kernels_table.cc"]
 
 
@@ -55,6 +56,12 @@ def build(force=False, jobs=None):
         src = os.path.join(CSRC, "kernels_dt.hip")
         if force or _newer(obj, [src] + headers):
             tasks.append([HIPCC] + COMMON + DEVICE + ["-DHCCL_DT=%d" % dt, "-c", src, "-o", obj])
+    for name in DEVICE_SOURCES:
+        obj = os.path.join(OBJ, name.replace(".hip", ".o"))
+        objs.append(obj)
+        src = os.path.join(CSRC, name)
+        if force or _newer(obj, [src] + headers):
+            tasks.append([HIPCC] + COMMON + DEVICE + ["-c", src, "-o", obj])
     for name in HOST_SOURCES:
         obj = os.path.join(OBJ, name.replace(".cc", ".o"))
         objs.append(obj)

@@ -476,6 +476,10 @@ HcclResult HcclCommInitAll(uint32_t ndev, int32_t *devices, HcclComm *comms)
         g->comms[r] = std::move(c);
     }
     g->liveComms = ndev;
+    // Device set-up (events, the fixed workspace's address, kernel code objects) happens here when a GPU
+    // is present, so that no collective call is the first to touch the device; without a GPU the group
+    // is still created and its collectives fail with HCCL_E_RUNTIME.
+    (void)EnsureDevice(g, true);
     std::lock_guard<std::mutex> reg(g_registryMutex);
     g_groups.insert(g);
     return HCCL_SUCCESS;
@@ -732,6 +736,46 @@ HcclResult HcclReduceScatter(void *sendBuf, void *recvBuf, uint64_t recvCount, H
     sig.dtype = dataType;
     sig.recvType = dataType;
     sig.op = op;
+    return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr);
+}
+
+// No counterpart in the reference.  HcclReduceScatter for callers that cannot allocate device memory
+// (code under HIP graph capture, tight serving loops, harnesses that forbid it): same arguments and
+// checks; descriptor tables and the step-by-step schedule's partial results live in a fixed device
+// workspace instead of library allocations, nothing is cached, no graph is instantiated.
+HcclResult HcclAmdReduceScatterNoAlloc(void *sendBuf, void *recvBuf, uint64_t recvCount, HcclDataType dataType,
+    HcclReduceOp op, HcclComm comm, aclrtStream stream)
+{
+    if (recvCount == 0) {
+        HCCL_LOG_WARN("HcclAmdReduceScatterNoAlloc: recvCount is 0, nothing to do");
+        return HCCL_SUCCESS;
+    }
+    CHK_PTR(comm);
+    CHK_PTR(sendBuf);
+    CHK_PTR(recvBuf);
+    Comm *c = AsComm(comm);
+    if (c == nullptr) {
+        return HCCL_E_PARA;
+    }
+    InUse guard(c);
+    HcclResult r = CheckOpParam("HcclAmdReduceScatterNoAlloc", recvCount, dataType, stream);
+    if (r == HCCL_SUCCESS) {
+        r = CheckReduce("HcclAmdReduceScatterNoAlloc", dataType, op);
+    }
+    if (r != HCCL_SUCCESS) {
+        return r;
+    }
+    if ((reinterpret_cast<uintptr_t>(sendBuf) | reinterpret_cast<uintptr_t>(recvBuf)) % ElemSize(dataType) != 0) {
+        HCCL_LOG_ERROR("HcclAmdReduceScatterNoAlloc: buffers must be aligned to the element size");
+        return HCCL_E_PARA;
+    }
+    OpSig sig;
+    sig.coll = COLL_REDUCESCATTER;
+    sig.count = recvCount;
+    sig.dtype = dataType;
+    sig.recvType = dataType;
+    sig.op = op;
+    sig.noAlloc = 1;
     return Arrive(c, sig, sendBuf, recvBuf, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, nullptr);
 }
 

@@ -6,6 +6,7 @@
 #include <sstream>
 
 #include "log.h"
+#include "noalloc.h"
 #include "runtime.h"
 
 namespace hcclamd {
@@ -51,6 +52,21 @@ HcclResult EnsureDevice(Group *g, bool quiet)
     }
     HIP_OK(hipEventCreateWithFlags(&g->doneEvent, hipEventDisableTiming));
     g->scratch.assign(g->p, nullptr);
+    // Set-up for the entry point that allocates nothing: the address of the fixed workspace on this
+    // device (g->device is the current device), and every kernel's code object loaded now, so that no
+    // later launch is the first use of its module.
+    HIP_OK(NoAllocWorkspace(g->device, &g->noAllocBase));
+    for (int dt = 0; dt <= 11; dt++) {
+        const void *f = LookupKernel(dt, 0, KK_STEP);
+        hipFuncAttributes attr;
+        if (f != nullptr) {
+            HIP_OK(hipFuncGetAttributes(&attr, f));
+        }
+    }
+    {
+        hipFuncAttributes attr;
+        HIP_OK(hipFuncGetAttributes(&attr, LookupCopyKernel(KK_STEP)));
+    }
     g->deviceReady = true;
     return HCCL_SUCCESS;
 }
@@ -81,6 +97,7 @@ HcclResult EnsureScratch(Group *g, uint64_t bytes)
 
 struct Builder {
     Group *g;
+    std::vector<void *> scratch;  // per rank: the group's own allocations, or shares of the fixed workspace
     std::vector<uint8_t> host;   // image of the device allocation
 
     size_t Reserve(size_t bytes)
@@ -95,7 +112,7 @@ struct Builder {
         switch (r.buf) {
             case BUF_SEND: base = static_cast<char *>(g->ctx->send[r.rank]); break;
             case BUF_RECV: base = static_cast<char *>(g->ctx->recv[r.rank]); break;
-            default: base = static_cast<char *>(g->scratch[r.rank]); break;
+            default: base = static_cast<char *>(scratch[r.rank]); break;
         }
         return base + r.off;
     }
@@ -206,10 +223,21 @@ bool PreferOrdinaryStores(const Plan &plan, const std::vector<void *> &send, con
     return maxWritten <= kMemorySideCacheBytes && 2 * readBack >= written;
 }
 
-HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int op)
+// With noAlloc the tables go to the fixed workspace through launches on `stream`, and the schedule's
+// scratch is the workspace's data part cut into equal shares, one per rank.
+HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int op, bool noAlloc, hipStream_t stream)
 {
     Builder b;
     b.g = g;
+    if (noAlloc) {
+        const size_t share = (kNoAllocDataBytes / g->p) & ~size_t(255);
+        char *data = static_cast<char *>(g->noAllocBase) + kNoAllocTableBytes;
+        for (uint32_t r = 0; r < g->p; r++) {
+            b.scratch.push_back(data + size_t(r) * share);
+        }
+    } else {
+        b.scratch = g->scratch;
+    }
     std::vector<PendingLaunch> pending;
     // Launch width.  Streaming kernels on this part run best with few, fat workgroups as long as a
     // lane keeps enough memory operations in flight: 1 workgroup per CU when an item touches 8 or
@@ -411,12 +439,23 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
     if (pending.empty()) {
         return HCCL_SUCCESS;   // nothing to move (e.g. one rank, in place)
     }
-    pp->devTables = g->arena.Alloc(b.host.size());
-    if (pp->devTables == nullptr) {
-        HCCL_LOG_ERROR("no device memory for %zu bytes of descriptor tables", b.host.size());
-        return HCCL_E_MEMORY;
+    if (noAlloc) {
+        b.host.resize((b.host.size() + 255) & ~size_t(255));
+        if (b.host.size() > kNoAllocTableBytes) {
+            HCCL_LOG_ERROR("%s without allocation: the descriptor tables need %zu bytes, the fixed workspace holds %zu",
+                CollName(g->ctx->sig.coll), b.host.size(), kNoAllocTableBytes);
+            return HCCL_E_PARA;
+        }
+        pp->devTables = g->noAllocBase;
+        HIP_OK(NoAllocUpload(pp->devTables, b.host.data(), b.host.size(), stream));
+    } else {
+        pp->devTables = g->arena.Alloc(b.host.size());
+        if (pp->devTables == nullptr) {
+            HCCL_LOG_ERROR("no device memory for %zu bytes of descriptor tables", b.host.size());
+            return HCCL_E_MEMORY;
+        }
+        HIP_OK(hipMemcpy(pp->devTables, b.host.data(), b.host.size(), hipMemcpyHostToDevice));
     }
-    HIP_OK(hipMemcpy(pp->devTables, b.host.data(), b.host.size(), hipMemcpyHostToDevice));
     char *base = static_cast<char *>(pp->devTables);
     for (PendingLaunch &pl : pending) {
         pl.rec.table = base + pl.tableAt;
@@ -550,7 +589,7 @@ Algo Level1Algo(const Group *g)
     return (n >= 8 || (n > 1 && (n & (n - 1)) == 0)) ? ALGO_RHD : ALGO_RING;
 }
 
-HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
+HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAlloc, hipStream_t stream)
 {
     std::unique_ptr<Prepared> pp(new Prepared());
     const bool reduceColl = g->ctx->sig.coll == COLL_ALLREDUCE || g->ctx->sig.coll == COLL_REDUCESCATTER || g->ctx->sig.coll == COLL_REDUCE;
@@ -672,18 +711,28 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out)
         }
     }
     if (!pp->fused && pp->plan->scratchBytes > 0) {
-        HcclResult r = EnsureScratch(g, pp->plan->scratchBytes);
-        if (r != HCCL_SUCCESS) {
-            return r;
+        if (noAlloc) {
+            const size_t share = (kNoAllocDataBytes / g->p) & ~size_t(255);
+            if (pp->plan->scratchBytes > share) {
+                HCCL_LOG_ERROR("%s without allocation: the step-by-step schedule keeps %llu bytes of partial results per rank, "
+                    "the fixed workspace has %zu per rank for %u ranks", CollName(g->ctx->sig.coll),
+                    (unsigned long long)pp->plan->scratchBytes, share, g->p);
+                return HCCL_E_PARA;
+            }
+        } else {
+            HcclResult r = EnsureScratch(g, pp->plan->scratchBytes);
+            if (r != HCCL_SUCCESS) {
+                return r;
+            }
         }
     }
     pp->scratchGen = g->scratchGen;
-    HcclResult r = BuildTables(g, pp.get(), reduceColl, g->ctx->sig.dtype, g->ctx->sig.op);
+    HcclResult r = BuildTables(g, pp.get(), reduceColl, g->ctx->sig.dtype, g->ctx->sig.op, noAlloc, stream);
     if (r != HCCL_SUCCESS) {
         return r;
     }
-    // one kernel is cheaper to launch directly than through a graph
-    if (g->cfg.graph && pp->launches.size() > 1) {
+    // one kernel is cheaper to launch directly than through a graph; instantiating a graph allocates
+    if (!noAlloc && g->cfg.graph && pp->launches.size() > 1) {
         r = BuildGraph(pp.get());
         if (r != HCCL_SUCCESS) {
             return r;
@@ -825,11 +874,27 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         (g->ctx->sig.coll == COLL_ALLREDUCE || g->ctx->sig.coll == COLL_REDUCESCATTER || g->ctx->sig.coll == COLL_REDUCE)) {
         algo = ALGO_MESH_ATOMIC;
     }
-    std::string key = CacheKey(g, algo);
     Prepared *pp = nullptr;
-    auto it = g->cache.find(key);
+    std::unique_ptr<Prepared> uncached;   // the collective of a call that allocates nothing: built, launched, dropped
     bool hit = false;
-    if (it != g->cache.end() && it->second->scratchGen == g->scratchGen) {
+    if (g->ctx->sig.noAlloc) {
+        // Tables and partial results live in the fixed workspace, which the next such call overwrites:
+        // nothing is kept, and the table upload is queued on the launcher's stream ahead of the kernels.
+        if (g->noAllocBase == nullptr) {
+            HCCL_LOG_ERROR("%s without allocation: the fixed workspace was not set up", CollName(g->ctx->sig.coll));
+            return HCCL_E_INTERNAL;
+        }
+        r = Prepare(g, algo, &uncached, true, g->ctx->streams[launcher]);
+        if (r != HCCL_SUCCESS) {
+            return r;
+        }
+        pp = uncached.get();
+    }
+    std::string key = pp ? std::string() : CacheKey(g, algo);
+    auto it = pp ? g->cache.end() : g->cache.find(key);
+    if (pp != nullptr) {
+        // issued below
+    } else if (it != g->cache.end() && it->second->scratchGen == g->scratchGen) {
         pp = it->second.get();
         hit = true;
     } else {
@@ -855,7 +920,7 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
             g->arena.Reset();
         }
         std::unique_ptr<Prepared> fresh;
-        r = Prepare(g, algo, &fresh);
+        r = Prepare(g, algo, &fresh, false, nullptr);
         if (r != HCCL_SUCCESS) {
             return r;
         }

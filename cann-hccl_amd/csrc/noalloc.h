@@ -1,0 +1,22 @@
+// Workspace of the entry point that allocates nothing (see noalloc.hip).
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace hcclamd {
+
+constexpr size_t kNoAllocTableBytes = size_t(256) << 10;   // descriptor tables of one collective
+constexpr size_t kNoAllocDataBytes = size_t(32) << 20;     // partial results, shared by all ranks of the group
+constexpr size_t kNoAllocUploadBytes = 3072;               // table bytes per upload launch (kernel-argument space)
+
+// Address of the workspace on `device`, which must be the current device.  The first call per device
+// looks the symbol up; later calls return the kept pointer.
+hipError_t NoAllocWorkspace(int device, void **base);
+
+// Queues on `stream` the launches that write hostBytes[0, bytes) to dst (inside the workspace, 16-byte
+// aligned; the copy is rounded up to a multiple of 16 bytes).  The host bytes are consumed before the call returns.
+hipError_t NoAllocUpload(void *dst, const void *hostBytes, size_t bytes, hipStream_t stream);
+
+}  // namespace hcclamd

@@ -103,10 +103,11 @@ struct OpSig {
     int variable = 0;                // 1: reduce-scatter-v / all-gather-v (block tables instead of a count)
     uint32_t peer = 0;               // send / receive: destination rank (root = source rank)
     uint32_t root = 0;               // broadcast / reduce / scatter
+    int noAlloc = 0;                 // 1: issued out of the fixed device workspace, nothing allocated, nothing cached
     bool operator==(const OpSig &o) const
     {
         return coll == o.coll && count == o.count && dtype == o.dtype && recvType == o.recvType && op == o.op &&
-            variable == o.variable && root == o.root && peer == o.peer;
+            variable == o.variable && root == o.root && peer == o.peer && noAlloc == o.noAlloc;
     }
 };
 
@@ -171,6 +172,7 @@ struct Group {
     hipEvent_t doneEvent = nullptr;
     std::vector<void *> scratch;
     void *barrierMem = nullptr;       // 2 x p small buffers for HcclBarrier's all-reduce
+    void *noAllocBase = nullptr;      // this device's copy of the fixed workspace (noalloc.hip), looked up at set-up
     uint64_t scratchBytes = 0;
     uint64_t scratchGen = 0;
     std::unordered_map<std::string, std::unique_ptr<Prepared>> cache;   // keyed by request, settings and buffer addresses

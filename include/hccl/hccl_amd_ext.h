@@ -81,6 +81,24 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
 extern HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint64_t count, HcclDataType dataType,
     uint64_t cclBytes, uint64_t align, uint64_t inPlaceMask, const uint64_t *tables, char *out, size_t cap, size_t *needed);
 
+/* HcclReduceScatter that allocates nothing.  No counterpart in the reference: it is for callers that cannot
+ * allocate device memory while they run -- code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it.  Arguments, checks and result are HcclReduceScatter's (every rank of the group calls it; the
+ * last call issues the work on its stream).  Descriptor tables, and with "fuse" = "0" the schedule's partial
+ * results, live in a fixed workspace that every GPU holds from library load to process end:
+ * HCCL_AMD_NOALLOC_TABLE_BYTES of tables and HCCL_AMD_NOALLOC_DATA_BYTES of partial results (shared
+ * equally by the ranks: nRanks * recvCount * sizeof(type) partial bytes per rank must fit its share).
+ * Larger requests fail with HCCL_E_PARA and a message.  Nothing is cached and no graph is built, so a call
+ * costs a plan lookup and one small upload launch per 3 KiB of tables on top of the kernels.  All calls on a
+ * GPU share that GPU's workspace, whichever group they come from: a call must not be issued while an earlier one may
+ * still be running on another stream (calls of one group whose ranks keep their streams are ordered by the
+ * library; anything else is the caller's to order).  Nothing in the workspace has to start at zero: tables
+ * are rewritten by every call and partial results are written before they are read. */
+#define HCCL_AMD_NOALLOC_TABLE_BYTES (256u << 10)
+#define HCCL_AMD_NOALLOC_DATA_BYTES (32u << 20)
+extern HcclResult HcclAmdReduceScatterNoAlloc(void *sendBuf, void *recvBuf, uint64_t recvCount, HcclDataType dataType,
+    HcclReduceOp op, HcclComm comm, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
