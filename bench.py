@@ -4,12 +4,13 @@ Default workload: ring all-reduce, sum, fp32, 8 simulated ranks x 256 MiB per ra
 (BASELINE.json configs[1] at its largest size).  A "step" is one complete collective (one call per
 rank).  Prints one JSON line.
 
-The headline (`value`, `ms_per_step`, `roofline`) is the schedule run step by step: one kernel launch per
-phase of copy / reduce steps, replayed from a HIP graph, moving 5 * (p - 1) * S bytes per collective
-(3 * S per reduce-scatter phase, 2 * S per all-gather phase) -- the bytes the metric counts.  The library's
-default, the fused single pass that reads every rank's input once and writes every rank's output once
-(2 * p * S bytes, same bits, about half the time), is timed in the same run and reported under
-`config.fused_single_pass` and `roofline_fused`.
+The headline (`value`, `ms_per_step`, `roofline`) is the library's default mode: the fused single pass (one
+launch of ChainKernel<float, sum>) that reads every rank's input once, combines in the ring schedule's order and
+writes every rank's output once -- 2 * p * S algorithmic bytes per collective, bit for bit the schedule's result.
+The schedule run step by step (library setting fuse=0: one launch per phase of copy / reduce steps, replayed from a
+HIP graph, 5 * (p - 1) * S bytes, 1.9 times slower per collective) is timed in the same run and reported under
+`config.step_by_step` and `roofline_steps`; part of what its phases read comes out of the 256 MB memory-side cache,
+so its rate is not a DRAM rate.
 
     python bench.py [--steps K] [--warmup W] [--size-mib M] [--sweep] [--suite] [--no-cpu]
 """
@@ -25,14 +26,22 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 METRIC = "achieved HBM GB/s & % of peak, 8-rank fp32 ring AllReduce 256MiB/rank"
 
-# HBM traffic of the fused all-reduce kernel at the default workload, from rocprofv3 --pmc
-# (FETCH_SIZE, WRITE_SIZE), scaled by the same counters over a plain copy of known size.
-# Valid for the default workload only (8 ranks x 256 MiB); the figures and the commands are in
-# profiles/ChainKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt.
-MEASURED_TRAFFIC_BYTES = 4295386000
-# The same for the 14 launches of the step-by-step mode together (traffic between L2 and the fabric per
-# collective); profiles/StepKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt.
-MEASURED_STEP_TRAFFIC_BYTES = 9395366000
+PROFILE_FUSED = os.path.join(ROOT, "profiles", "ChainKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt")
+PROFILE_STEPS = os.path.join(ROOT, "profiles", "StepKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt")
+
+
+def profiled_traffic(path):
+    """Bytes per launch between L2 and the fabric that the committed rocprofv3 --pmc summary of the default workload
+    reports (its line `traffic_bytes_per_launch = N`: FETCH_SIZE and WRITE_SIZE scaled by a plain copy of known
+    size in the same runs).  None when the summary is absent or has no such line."""
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.strip().startswith("traffic_bytes_per_launch"):
+                    return int(line.split("=", 1)[1].split()[0].replace("_", ""))
+    except (OSError, ValueError, IndexError):
+        pass
+    return None
 
 
 def run_mode(pkg, torch, comms, stream, sends, recvs, n, fuse, steps, warmup):
@@ -357,12 +366,13 @@ def main():
     cpu = None
     bit_exact = None
     if not args.no_cpu:
-        best = None
+        best, touched = None, 0
         outs = [np.empty(n, np.float32) for _ in range(p)]
         for _ in range(3):
             work = [x.copy() for x in ins]
             t0 = time.perf_counter()
-            oracle.allreduce(work, oracle.FP32, oracle.SUM, flags=oracle.DIRECT | oracle.ZERO_STAGING, threads=threads, outs=outs)
+            _, touched = oracle.allreduce(work, oracle.FP32, oracle.SUM, flags=oracle.DIRECT | oracle.ZERO_STAGING,
+                                          threads=threads, outs=outs, return_touched=True)
             dt = time.perf_counter() - t0
             best = dt if best is None else min(best, dt)
         bit_exact = bool(np.array_equal(outs[0], fused_out) and np.array_equal(outs[0], step_out))
@@ -370,11 +380,15 @@ def main():
         t0 = time.perf_counter()
         oracle.allreduce(work, oracle.FP32, oracle.SUM, flags=oracle.DIRECT | oracle.ZERO_STAGING, threads=1, outs=outs)
         single = time.perf_counter() - t0
-        cpu = {"value": round(s_actual / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-               "sample": "full workload (%d ranks x %.0f MiB fp32, out of place), checker in direct zero-staging "
-                         "mode, best of 3, %.3f s; bytes = those of the step-by-step schedule" % (p, args.size_mib, best),
-               "single_thread_value": round(s_actual / single / 1e9, 3), "single_thread_s": round(single, 3),
-               "cpu_model": cpu_model()}
+        # same byte basis as `value`: every input read once, every output written once (2 * p * S) per collective
+        cpu = {"value": round(actual / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+               "sample": "the full workload once per timing (%d ranks x %.0f MiB fp32, out of place), the checker's ring "
+                         "schedule in direct zero-staging mode on %d threads, best of 3 = %.3f s; value = 2*p*S bytes "
+                         "(the headline's basis) / that time; the checker itself read and wrote %d bytes per "
+                         "collective" % (p, args.size_mib, threads, best, touched),
+               "bytes_touched_GBps": round(touched / best / 1e9, 3),
+               "single_thread_value": round(actual / single / 1e9, 3), "single_thread_s": round(single, 3),
+               "host_cpus_visible": os.cpu_count(), "cpu_model": cpu_model()}
 
     if args.calibrate:
         one = pkg.comm_init_all(1)
@@ -421,21 +435,19 @@ def main():
                                 (5 * p - 3) * size / (cpu_us * 1e-6) / 1e9, note))
             size *= 2
 
-    headline = p == 8 and args.size_mib == 256.0 and not args.set
+    headline = p == 8 and args.size_mib == 256.0 and not args.set and info["algo"] == 0
     sched_name = {0: "ring", 1: "mesh", 2: "halving-doubling", 4: "mesh"}.get(info["algo"], "?")
     launches = max(1, s_info["launches"])
-    # The headline is the schedule as it stands: its copy / reduce steps, one kernel launch per phase, replayed
-    # from a HIP graph; the metric counts the bytes those steps move.  The library's default -- one fused pass that
-    # reads every input once and writes every output once, same bits -- moves 2.2 times fewer bytes and is
-    # reported next to it.
+    fused_kernel = "TreeKernel" if info["algo"] == 2 else "ChainKernel"
+    # The headline is what a caller of HcclAllReduce gets with the library's defaults (fuse=1): one fused launch.
     line = {
         "metric": METRIC,
-        "value": round(s_actual / (s_wall_ms * 1e-3) / 1e9, 2),
+        "value": round(actual / (wall_ms * 1e-3) / 1e9, 2),
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(s_wall_ms, 4),
+        "ms_per_step": round(wall_ms, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -443,45 +455,53 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "%s all-reduce sum fp32, %d simulated ranks x %.0f MiB per rank, out of place, one GPU%s"
-                        % (sched_name, p, args.size_mib, " (BASELINE.json configs[1] at its largest size)"
-                           if (p == 8 and args.size_mib == 256.0 and info["algo"] == 0) else ""),
-            "issue": "step by step: the schedule's %d phases of copy / reduce steps, one kernel launch each, replayed "
-                     "from a HIP graph (library setting fuse=0)" % s_info["launches"],
-            "launches_per_step": s_info["launches"],
-            "graph": s_info["graph"],
-            "bytes_per_step": s_actual,
-            "pct_of_hbm_peak": round(100.0 * s_achieved / HBM_PEAK_GBPS, 2),
-            "ms_per_step_device": round(s_dev_ms, 4),
+                        % (sched_name, p, args.size_mib, " (BASELINE.json configs[1] at its largest size)" if headline else ""),
+            "issue": "library default (fuse=1): one %s launch per collective reads every rank's input once, combines in "
+                     "the %s schedule's order and writes every rank's output; same bits as the schedule run step by step"
+                     % (fused_kernel, sched_name),
+            "default_mode": "fused single pass",
+            "launches_per_step": info["launches"],
+            "graph": info["graph"],
+            "bytes_per_step": actual,
+            "pct_of_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBPS, 2),
+            "ms_per_step_device": round(dev_ms, 4),
+            "launch_ms_median": round(med_ms, 4),
+            "launch_ms_min": round(min_ms, 4),
+            "schedule_bytes_per_second_GBps": round(s_actual / (dev_ms * 1e-3) / 1e9, 1),
             "bit_exact_vs_host_reference": bit_exact,
             "all_ranks_identical": bool(same_all),
-            "fused_single_pass": {
-                "note": "library default (fuse=1): one kernel reads every rank's input once, combines in the schedule's "
-                        "order and writes every rank's output; same bits as the step-by-step result",
-                "launches_per_step": info["launches"],
-                "ms_per_step": round(wall_ms, 4),
-                "bytes_per_step_actual": actual,
-                "hbm_GBps": round(achieved, 1),
-                "pct_of_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBPS, 2),
-                "schedule_bytes_per_second_GBps": round(s_actual / (dev_ms * 1e-3) / 1e9, 1),
-                "launch_ms_median": round(med_ms, 4),
-                "launch_ms_min": round(min_ms, 4),
+            "step_by_step": {
+                "note": "library setting fuse=0: the schedule's %d phases of copy / reduce steps, one StepKernel launch "
+                        "each, replayed from a HIP graph; same bits; not the default (%.2fx the time per collective)"
+                        % (s_info["launches"], s_dev_ms / dev_ms),
+                "launches_per_step": s_info["launches"],
+                "graph": s_info["graph"],
+                "ms_per_step": round(s_wall_ms, 4),
+                "ms_per_step_device": round(s_dev_ms, 4),
+                "bytes_per_step": s_actual,
             },
         },
         "roofline": {
-            "bound": "hbm", "achieved": round(s_achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(s_achieved / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_STEP_TRAFFIC_BYTES // 14 if headline else None,
-            "kernel": "StepKernel<float, sum>: %d launches per collective (one per phase), %.1f MB per launch on average, "
-                      "average launch %.1f us = %.4f ms per graph replay / %d, gaps between the graph's nodes included, "
-                      "over %d replays" % (s_info["launches"], s_actual / launches / 1e6, s_dev_ms * 1e3 / launches, s_dev_ms,
-                                           launches, args.steps),
-        },
-        "roofline_fused": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES if headline else None,
-            "kernel": "%s<float, sum> (fused %s all-reduce), bytes actually moved %d, avg launch %.4f ms over %d launches"
-                      % ("TreeKernel" if info["algo"] == 2 else "ChainKernel", sched_name, actual, dev_ms, args.steps),
+            "traffic": profiled_traffic(PROFILE_FUSED) if headline else None,
+            "traffic_source": "profiles/" + os.path.basename(PROFILE_FUSED) + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)"
+                              if headline else None,
+            "kernel": "%s<float, sum> (fused %s all-reduce, the library default): %d algorithmic bytes per launch "
+                      "(%d x %.0f MiB read + the same written), average launch %.4f ms over %d launches, HIP events on "
+                      "the launching stream" % (fused_kernel, sched_name, actual, p, args.size_mib, dev_ms, args.steps),
+        },
+        "roofline_steps": {
+            "bound": "hbm", "achieved": round(s_achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(s_achieved / HBM_PEAK_GBPS, 4),
+            "traffic": profiled_traffic(PROFILE_STEPS) if headline else None,
+            "kernel": "StepKernel<float, sum>, library setting fuse=0: %d launches per collective (one per phase), %.1f MB "
+                      "per launch on average, average launch %.1f us = %.4f ms per graph replay / %d, gaps between the "
+                      "graph's nodes included, over %d replays.  Includes memory-side-cache hits: from the second phase "
+                      "on, part of what a phase reads was written by the phase before and comes out of the 256 MB "
+                      "memory-side cache, so this is a rate between L2 and the fabric, not a DRAM rate (the one phase "
+                      "with cold inputs runs about 16 %% slower, see profiles/)"
+                      % (s_info["launches"], s_actual / launches / 1e6, s_dev_ms * 1e3 / launches, s_dev_ms, launches, args.steps),
         },
         "cpu_baseline": cpu,
     }
