@@ -122,7 +122,7 @@ def run_suite(pkg, torch, steps, warmup, only="", settings=()):
     out.write("%-46s %-6s %9s %10s %9s %8s\n" % ("configuration", "mode", "launches", "time_us", "GB/s", "%peak"))
 
     def report(name, comms, call):
-        if only and only not in name:
+        if only and not any(part in name for part in only.split(",")):
             return
         for kv in settings:
             k, v = kv.split("=", 1)
@@ -306,7 +306,7 @@ def main():
     ap.add_argument("--ranks", type=int, default=8)
     ap.add_argument("--sweep", action="store_true", help="also time 8 KiB .. 256 MiB per rank (x2), table on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--suite-filter", default="", help="with --suite: only configurations whose name contains this")
+    ap.add_argument("--suite-filter", default="", help="with --suite: only configurations whose name contains this (several alternatives separated by commas)")
     ap.add_argument("--suite", action="store_true", help="time the other BASELINE.json configurations (table on stderr) and exit")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 1 GiB int32 copy (one-rank all-reduce, out of place) three times, so that a "

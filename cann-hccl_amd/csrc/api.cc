@@ -1474,7 +1474,9 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         }
         cfg.cacheEntries = uint32_t(n);
     } else if (k == "fused_stores") {
-        if (v == "nt") {
+        if (v == "auto") {
+            cfg.fusedStores = -1;
+        } else if (v == "nt") {
             cfg.fusedStores = 0;
         } else if (v == "ordinary") {
             cfg.fusedStores = 1;

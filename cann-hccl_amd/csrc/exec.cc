@@ -257,6 +257,14 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
         }
         double streams = bytes > 0 ? streamBytes / bytes : 2.0;   // loads + stores per lane and vector
         fusedPerCu = streams >= 8.0 ? 1u : (streams >= 3.0 ? 2u : 4u);
+        // Plain copies (one source, one destination) go through the copy kernel, which really gets the
+        // occupancy it is launched with; with non-temporal stores more workgroups only widen the range
+        // of addresses written at a time, which this memory system likes less (measured, 8 ranks:
+        // uniform all-to-all of 32 MiB per pair 752 us at 1 or 2 per CU, 835 us at 4, 850 us at 8;
+        // 16-rank all-to-all-v, 106 MB of ragged segments: 55.6 / 40.5 / 42.5 / 41.3 us at 1 / 2 / 4 / 8).
+        if (!reduceColl && streams < 3.0) {
+            fusedPerCu = 2u;
+        }
         // few tiles per workgroup: a second workgroup per CU evens out the tail (measured: 16-rank
         // ring all-reduce of 32 MiB per rank 241 us at 1 per CU, 220 us at 2)
         if (fusedPerCu == 1 && bytes / kTileBytes < 32.0 * g->numCu) {
@@ -353,7 +361,19 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
         // write-back stores.  Measured, 8-rank fp32 all-reduce replayed on the same buffers: write-back is
         // 5 % and 12 % faster at 16 and 32 MiB per rank (the output then stays in the 256 MB memory-side
         // cache), 20 % slower at 4 MiB and 7 % slower from 64 MiB per rank up.
-        const bool fusedOrdinary = g->cfg.fusedStores == 1;
+        // Pure data movement with one source and many destinations (all-gather, broadcast) is 4 - 5 % faster with
+        // write-back stores once the output is far larger than the memory-side cache (8 ranks: all-gather to
+        // 256 MiB per rank 473 us against 501 us, broadcast of 256 MiB 425 us against 447 us); one-to-one copies
+        // are not (uniform all-to-all 773 us against 752 us).
+        bool fusedOrdinary = g->cfg.fusedStores == 1;
+        if (g->cfg.fusedStores < 0 && !reduceColl) {
+            double written = 0, read = 0;
+            for (const FusedItem &it : pp->plan->fused) {
+                written += double(it.dst.size()) * double(it.bytes);
+                read += double(it.bytes);
+            }
+            fusedOrdinary = written >= 4.0 * read && written >= 2.0 * double(kMemorySideCacheBytes);
+        }
         // one launch per kernel kind present
         for (int kind : {int(KK_CHAIN), int(KK_TREE), int(KK_STACK)}) {
             std::vector<FusedDesc> descs;

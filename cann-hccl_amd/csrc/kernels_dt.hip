@@ -51,10 +51,10 @@ using DT = uint8_t;
 #define HCCL_CAT(a, b) HCCL_CAT2(a, b)
 
 #if HCCL_DT == 255
-// pure data movement: only the copy paths of the step and chain kernels are reachable
+// pure data movement: the step kernel's copy path and the copy kernel
 extern const void *const HCCL_CAT(kKernels_, HCCL_DT_NAME)[2] = {
     reinterpret_cast<const void *>(&StepKernel<DT, ROP_SUM>),
-    reinterpret_cast<const void *>(&ChainKernel<DT, ROP_SUM>),
+    reinterpret_cast<const void *>(&CopyKernel<0>),
 };
 #else
 #define HCCL_ROW(OP)                                                     \

@@ -634,6 +634,87 @@ __global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__
     }
 }
 
+// ---- pure data movement: one source, m destinations ------------------------------------------------------
+// The chain kernel's copy path with nothing else in the kernel: about 40 registers instead of 170+, so eight
+// workgroups fit on a CU where the chain kernel fits two.  A copy keeps only 4 loads per lane in flight, and its
+// rate comes from how many waves do that at once (measured, 1 GiB copy: 5.1 TB/s through the chain kernel,
+// 6.3 TB/s for a plain copy kernel at full occupancy).
+template <uint32_t MODE, bool FULL, bool ORDINARY = false>
+__device__ __forceinline__ void CopyVecPass(const void *s, void *const *__restrict__ dst, uint32_t ndst, uint64_t off,
+    uint32_t vecBase, uint32_t nvec)
+{
+    uint64_t pos[kChainVec];
+    bool live[kChainVec];
+    V4 v[kChainVec];
+#pragma unroll
+    for (uint32_t u = 0; u < kChainVec; u++) {
+        const uint32_t i = vecBase + u * kBlockThreads + threadIdx.x;
+        live[u] = FULL || i < nvec;
+        pos[u] = off + uint64_t(i) * 16;
+        if (live[u]) {
+            v[u] = Load16<MODE>(s, pos[u]);
+        }
+    }
+    for (uint32_t k = 0; k < ndst; k++) {
+        void *o = dst[k];
+#pragma unroll
+        for (uint32_t u = 0; u < kChainVec; u++) {
+            if (live[u]) {
+                StoreAny16<MODE, ORDINARY>(o, pos[u], v[u]);
+            }
+        }
+    }
+}
+
+// Same arguments and tables as the chain kernel; every item has exactly one source.  (A template only so that the
+// definition may sit in this header; Variant is unused.)
+template <int Variant>
+__global__ void __launch_bounds__(kBlockThreads) CopyKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
+    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool)
+{
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const FusedDesc d = items[FindDesc(items, nitems, tile)];
+        const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
+        const uint64_t left = d.bytes - off;
+        const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
+        const void *s = srcPool[d.srcBase];
+        void *const *dst = dstPool + d.dstBase;
+        if (d.mode == ACC_ELEM) {
+            for (uint32_t i = threadIdx.x; i < n; i += kBlockThreads) {
+                const uint8_t b = LoadElem<uint8_t>(s, off + i);
+                for (uint32_t k = 0; k < d.ndst; k++) {
+                    StoreElem<uint8_t>(dst[k], off + i, b);
+                }
+            }
+        } else {
+            const uint32_t nvec = n >> 4;
+            constexpr uint32_t kPass = kChainVec * kBlockThreads;
+            uint32_t base = 0;
+            if (d.mode == ACC_VEC16) {
+                if (d.flags & kFusedOrdinaryStores) {
+                    for (; base + kPass <= nvec; base += kPass) {
+                        CopyVecPass<ACC_VEC16, true, true>(s, dst, d.ndst, off, base, nvec);
+                    }
+                } else {
+                    for (; base + kPass <= nvec; base += kPass) {
+                        CopyVecPass<ACC_VEC16, true>(s, dst, d.ndst, off, base, nvec);
+                    }
+                }
+                if (base < nvec) {
+                    CopyVecPass<ACC_VEC16, false>(s, dst, d.ndst, off, base, nvec);
+                }
+            } else {
+                for (; base + kPass <= nvec; base += kPass) {
+                    CopyVecPass<ACC_VEC16_ANY, true>(s, dst, d.ndst, off, base, nvec);
+                }
+                if (base < nvec) {
+                    CopyVecPass<ACC_VEC16_ANY, false>(s, dst, d.ndst, off, base, nvec);
+                }
+            }
+        }
+    }
+}
+
 // ---- fused perfect tree (halving-doubling): leaves pairwise bottom-up ----------------------------------
 // v[i] = v[i] (+) v[i+w] for w = 1, 2, 4, ... is evaluated group by group: the first three levels
 // inside groups of 8 consecutive leaves (8 loads per vector in flight, one result kept per group), the

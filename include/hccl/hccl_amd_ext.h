@@ -35,8 +35,10 @@ extern "C" {
  *                                so that the next phase finds the data in the memory-side cache); "auto" decides per collective
  *   "step_sweep"    "alternate" | "forward"   step-by-step kernels: every other launch walks its data backwards (default),
  *                                or all walk forwards
- *   "fused_stores"  "nt" | "ordinary"   store kind of the fused chain kernel: non-temporal (default), or write-back, which
- *                                keeps a result of up to 256 MB in the memory-side cache for whoever reads it next
+ *   "fused_stores"  "auto" | "nt" | "ordinary"   store kind of the fused kernels: non-temporal, or write-back, which
+ *                                keeps a result of up to 256 MB in the memory-side cache for whoever reads it next; "auto"
+ *                                (default): non-temporal, except write-back for pure data movement from one source to four
+ *                                or more destinations with more than 512 MB of output (all-gather, broadcast)
  *   "cache_entries" how many prepared collectives (distinct sizes, buffers, settings) the group keeps (default 1024);
  *                   when full, the library waits for the device once and starts over
  *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
