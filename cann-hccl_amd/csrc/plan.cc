@@ -1810,6 +1810,11 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
         *err = "bad plan request";
         return 1;
     }
+    if (request.align % request.unit != 0) {
+        // a slice boundary inside an element would make the kernels combine across element boundaries
+        *err = "bad plan request: the slice alignment must be a multiple of the element size";
+        return 1;
+    }
     if ((request.level0Rings != 0 && request.level0Rings != 1 && request.level0Rings != 4) ||
         (request.level0Rings == 4 && request.p / request.servers != 8)) {
         *err = "level 0 runs as a mesh, one ring, or the four rings of a group of 8 ranks";

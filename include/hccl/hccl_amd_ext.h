@@ -21,7 +21,7 @@ extern "C" {
  *   "graph"         "0" | "1"    issue through a HIP graph
  *   "buffsize_mib"  CCL buffer size that sets the chunk plan (default 200, as HCCL_BUFFSIZE);
  *   "buffsize_bytes" the same in bytes (tests of the chunk loop on small inputs)
- *   "align"         slice alignment in bytes (default 128)
+ *   "align"         slice alignment in bytes (default 128); a collective whose element size does not divide it fails with HCCL_E_PARA
  *   "servers"       number of rank groups for all-reduce, reduce-scatter, all-gather and reduce: with n > 1 the p ranks form n groups of p / n
  *                   consecutive ranks and the two-level schedules run (mesh inside a group, "algo" ring or rhd between;
  *                   with "auto": rhd for 2, 4, 8 or more groups, ring for 3, 5, 6, 7, the reference's default);

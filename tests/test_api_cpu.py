@@ -238,12 +238,12 @@ def test_amd_params(comms):
     good = {b"algo": [b"ring", b"mesh", b"rhd", b"pairwise", b"auto"], b"deterministic": [b"0", b"1"], b"fuse": [b"0", b"1"],
             b"graph": [b"0", b"1"], b"buffsize_mib": [b"1", b"200"], b"buffsize_bytes": [b"4096"], b"align": [b"4", b"128"],
             b"level0": [b"mesh", b"ring", b"ring4"], b"step_stores": [b"auto", b"nt", b"ordinary"],
-            b"fused_stores": [b"nt", b"ordinary"], b"step_sweep": [b"forward", b"alternate"], b"cache_entries": [b"1", b"1024"], b"blocks_per_cu": [b"0", b"2"],
+            b"fused_stores": [b"auto", b"nt", b"ordinary"], b"step_sweep": [b"forward", b"alternate"], b"cache_entries": [b"1", b"1024"], b"blocks_per_cu": [b"0", b"2"],
             b"blocking_arrive": [b"0", b"1"], b"arrive_timeout_ms": [b"1000"]}
     for key, values in good.items():
         for v in values:
             assert L.HcclAmdSetParam(comms[0], key, v) == 0, (key, v)
-    bad = {b"level0": b"star", b"step_stores": b"maybe", b"fused_stores": b"auto", b"cache_entries": b"0", b"align": b"0",
+    bad = {b"level0": b"star", b"step_stores": b"maybe", b"fused_stores": b"maybe", b"cache_entries": b"0", b"align": b"0",
            b"servers": b"0"}
     for key, v in bad.items():
         assert L.HcclAmdSetParam(comms[0], key, v) == H.HCCL_E_PARA, (key, v)

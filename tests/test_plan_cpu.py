@@ -152,6 +152,14 @@ def test_plan_rejects_bad_requests():
         H.describe_plan(H.COLL_REDUCESCATTER, H.ALGO_PAIRWISE, 4, 10, FP32)   # pairwise is an all-to-all schedule
     with pytest.raises(H.HcclError):
         H.describe_plan(H.COLL_ALLGATHER, RING, 8, 10, FP32, ccl_bytes=64)   # buffer below one aligned slice per rank
+    # a slice alignment that the element size does not divide would cut slices inside elements
+    for dt, align in ((FP32, 1), (FP32, 2), (FP32, 6), (H.HCCL_DATA_TYPE_FP64, 4), (H.HCCL_DATA_TYPE_FP64, 12)):
+        for coll in (H.COLL_ALLREDUCE, H.COLL_REDUCESCATTER, H.COLL_ALLGATHER):
+            with pytest.raises(H.HcclError) as e:
+                H.describe_plan(coll, RING, 3, 1000, dt, align=align)
+            assert e.value.code == H.HCCL_E_PARA
+    H.describe_plan(H.COLL_ALLREDUCE, RING, 3, 1000, FP32, align=4)
+    H.describe_plan(H.COLL_ALLREDUCE, RING, 3, 1000, H.HCCL_DATA_TYPE_INT8, align=1)
 
 
 def _v_case(p, seed):
