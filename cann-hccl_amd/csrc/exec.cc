@@ -52,6 +52,15 @@ HcclResult EnsureDevice(Group *g, bool quiet)
     }
     HIP_OK(hipEventCreateWithFlags(&g->doneEvent, hipEventDisableTiming));
     g->scratch.assign(g->p, nullptr);
+    g->arena.allocFn = [](size_t bytes) -> void * {
+        void *mem = nullptr;
+        if (hipMalloc(&mem, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        return mem;
+    };
+    g->arena.freeFn = [](void *mem) { (void)hipFree(mem); };
     // Set-up for the entry point that allocates nothing: the address of the fixed workspace on this
     // device (g->device is the current device), and every kernel's code object loaded now, so that no
     // later launch is the first use of its module.
@@ -78,12 +87,23 @@ HcclResult EnsureScratch(Group *g, uint64_t bytes)
     if (bytes <= g->scratchBytes) {
         return HCCL_SUCCESS;
     }
-    // A cached collective may still be running out of the old scratch.
-    HIP_OK(hipDeviceSynchronize());
-    for (uint32_t r = 0; r < g->p; r++) {
-        if (g->scratch[r]) {
-            HIP_OK(hipFree(g->scratch[r]));
-            g->scratch[r] = nullptr;
+    if (g->pinnedScratchUsers > 0) {
+        // a caller's graph replays collectives that point at these buffers: they stay until the group goes
+        for (uint32_t r = 0; r < g->p; r++) {
+            if (g->scratch[r]) {
+                g->retiredScratch.push_back(g->scratch[r]);
+                g->scratch[r] = nullptr;
+            }
+        }
+        g->pinnedScratchUsers = 0;
+    } else {
+        // A cached collective may still be running out of the old scratch.
+        HIP_OK(hipDeviceSynchronize());
+        for (uint32_t r = 0; r < g->p; r++) {
+            if (g->scratch[r]) {
+                HIP_OK(hipFree(g->scratch[r]));
+                g->scratch[r] = nullptr;
+            }
         }
     }
     g->scratchBytes = 0;
@@ -153,6 +173,8 @@ template <typename F> void SplitByAlignment(const std::vector<uintptr_t> &addrs,
         emit(head + body, tail, uint32_t(ACC_ELEM));
     }
 }
+
+constexpr size_t kAsyncUploadBytes = 4 * kNoAllocUploadBytes;   // tables up to this size are uploaded by launches
 
 uint32_t TilesOf(uint64_t bytes) { return uint32_t((bytes + kTileBytes - 1) / kTileBytes); }
 
@@ -467,14 +489,27 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
             return HCCL_E_PARA;
         }
         pp->devTables = g->noAllocBase;
-        HIP_OK(NoAllocUpload(pp->devTables, b.host.data(), b.host.size(), stream));
+        HIP_OK(UploadThroughKernelArgs(pp->devTables, b.host.data(), b.host.size(), stream));
     } else {
-        pp->devTables = g->arena.Alloc(b.host.size());
+        b.host.resize((b.host.size() + 255) & ~size_t(255));
+        pp->devTables = g->arena.Alloc(b.host.size(), &pp->tableChunk);
         if (pp->devTables == nullptr) {
             HCCL_LOG_ERROR("no device memory for %zu bytes of descriptor tables", b.host.size());
             return HCCL_E_MEMORY;
         }
-        HIP_OK(hipMemcpy(pp->devTables, b.host.data(), b.host.size(), hipMemcpyHostToDevice));
+        if (b.host.size() <= kAsyncUploadBytes && stream != nullptr) {
+            // small tables ride on a few upload launches in front of the collective instead of a copy that
+            // waits for the device (measured, fused 8-rank all-reduce with fresh buffers every call: 42 us
+            // of host time per call with the copy)
+            HIP_OK(hipEventCreateWithFlags(&pp->uploaded, hipEventDisableTiming));
+            HIP_OK(UploadThroughKernelArgs(pp->devTables, b.host.data(), b.host.size(), stream));
+            HIP_OK(hipEventRecord(pp->uploaded, stream));
+            pp->uploadStream = stream;
+            pp->uploadComplete = false;
+            pp->hostTables.swap(b.host);
+        } else {
+            HIP_OK(hipMemcpy(pp->devTables, b.host.data(), b.host.size(), hipMemcpyHostToDevice));
+        }
     }
     char *base = static_cast<char *>(pp->devTables);
     for (PendingLaunch &pl : pending) {
@@ -751,18 +786,13 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAl
     if (r != HCCL_SUCCESS) {
         return r;
     }
-    // one kernel is cheaper to launch directly than through a graph; instantiating a graph allocates
-    if (!noAlloc && g->cfg.graph && pp->launches.size() > 1) {
-        r = BuildGraph(pp.get());
-        if (r != HCCL_SUCCESS) {
-            return r;
-        }
-    }
+    // The graph of a plan with several launches is built when the collective comes back a second time
+    // (IssueCollective): a caller that brings fresh buffers every time pays for tables, not for a graph.
     OpInfo &info = pp->info;
     info.coll = g->ctx->sig.coll;
     info.algo = algo;
     info.fused = pp->fused ? 1 : 0;
-    info.graph = pp->exec ? 1 : 0;
+    info.graph = 0;
     info.launches = uint32_t(pp->launches.size());
     info.bytesRead = pp->fused ? pp->plan->fusedRead : pp->plan->stepRead;
     info.bytesWritten = pp->fused ? pp->plan->fusedWritten : pp->plan->stepWritten;
@@ -777,6 +807,9 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAl
 
 Prepared::~Prepared()
 {
+    if (uploaded) {
+        (void)hipEventDestroy(uploaded);
+    }
     if (exec) {
         (void)hipGraphExecDestroy(exec);
     }
@@ -785,52 +818,19 @@ Prepared::~Prepared()
     }
 }
 
-void *TableArena::Alloc(size_t bytes)
-{
-    bytes = (bytes + 255) & ~size_t(255);
-    if (chunks.empty() || chunks.back().size - chunks.back().used < bytes) {
-        Chunk c;
-        c.size = std::max<size_t>(bytes, size_t(4) << 20);
-        void *mem = nullptr;
-        if (hipMalloc(&mem, c.size) != hipSuccess) {
-            (void)hipGetLastError();
-            return nullptr;
-        }
-        c.base = static_cast<char *>(mem);
-        chunks.push_back(c);
-    }
-    Chunk &c = chunks.back();
-    void *out = c.base + c.used;
-    c.used += bytes;
-    return out;
-}
-
-void TableArena::Reset()
-{
-    while (chunks.size() > 1) {
-        (void)hipFree(chunks.back().base);
-        chunks.pop_back();
-    }
-    if (!chunks.empty()) {
-        chunks[0].used = 0;
-    }
-}
-
-void TableArena::FreeAll()
-{
-    for (Chunk &c : chunks) {
-        (void)hipFree(c.base);
-    }
-    chunks.clear();
-}
-
 Group::~Group()
 {
     if (deviceReady) {
         (void)hipDeviceSynchronize();
     }
     cache.clear();
-    arena.FreeAll();
+    pinnedStale.clear();
+    if (arena.freeFn != nullptr) {
+        arena.FreeAll();
+    }
+    for (void *s : retiredScratch) {
+        (void)hipFree(s);
+    }
     for (hipEvent_t e : arriveEvents) {
         if (e) {
             (void)hipEventDestroy(e);
@@ -928,31 +928,82 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
             return HCCL_E_NOT_SUPPORT;
         }
         if (it != g->cache.end()) {
-            HIP_OK(hipDeviceSynchronize());   // stale entry (the scratch buffers moved); its tables stay in the arena
+            // stale entry (the scratch buffers moved); its tables stay in the arena
+            if (it->second->pinned) {
+                g->pinnedStale.push_back(std::move(it->second));   // a caller's graph still replays it out of the retired buffers
+            } else {
+                HIP_OK(hipDeviceSynchronize());
+            }
             g->cache.erase(it);
         }
         if (g->cache.size() >= g->cfg.cacheEntries) {
             // Full: wait once for whatever is still in flight and start over.  Dropping one entry at a
             // time would put a device-wide wait on every call of a caller with more buffers than entries
             // (measured with 200 buffer sets against 64 entries: 42 us per small all-reduce instead of 7.5).
+            // Collectives recorded into a caller's graph stay, tables and all (the arena keeps their chunks).
             HIP_OK(hipDeviceSynchronize());
-            g->cache.clear();
+            for (auto e = g->cache.begin(); e != g->cache.end();) {
+                e = e->second->pinned ? std::next(e) : g->cache.erase(e);
+            }
             g->arena.Reset();
         }
         std::unique_ptr<Prepared> fresh;
-        r = Prepare(g, algo, &fresh, false, nullptr);
+        r = Prepare(g, algo, &fresh, false, g->ctx->streams[launcher]);
         if (r != HCCL_SUCCESS) {
             return r;
         }
         pp = fresh.get();
         g->cache[key] = std::move(fresh);
     }
+    hipStream_t ls = g->ctx->streams[launcher];
+    // A caller may be capturing this stream into a graph of its own.  A graph launched into a
+    // capturing stream is not recorded there (the caller's graph came out empty and replays did
+    // nothing), so the kernels are then launched one by one and become nodes of the caller's graph.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    HIP_OK(hipStreamIsCapturing(ls, &capture));
+    const bool capturing = capture != hipStreamCaptureStatusNone;
+    if (!pp->uploadComplete) {
+        // The tables were written by launches on the stream of the call that prepared them, and nothing says yet
+        // that those have run.  Outside a capture: ask, and order this stream behind them if need be.  Under
+        // capture events of work outside the capture may not be touched and the caller's graph may be replayed
+        // on any stream later, so the same upload launches are recorded in front of the collective's kernels:
+        // every replay rewrites the same bytes.
+        if (capturing) {
+            HIP_OK(UploadThroughKernelArgs(pp->devTables, pp->hostTables.data(), pp->hostTables.size(), ls));
+        } else if (hipEventQuery(pp->uploaded) == hipSuccess) {
+            pp->uploadComplete = true;
+            std::vector<uint8_t>().swap(pp->hostTables);
+        } else {
+            (void)hipGetLastError();
+            if (ls != pp->uploadStream) {
+                HIP_OK(hipStreamWaitEvent(ls, pp->uploaded, 0));
+            }
+        }
+    }
+    if (capturing && !pp->pinned && !g->ctx->sig.noAlloc) {
+        // The caller's graph keeps pointers to this collective's tables and, step by step, to the group's
+        // scratch buffers: from now on neither is freed or handed out again while the group lives.
+        pp->pinned = true;
+        g->arena.Pin(pp->tableChunk);
+        if (pp->info.scratchBytes > 0) {
+            g->pinnedScratchUsers++;
+        }
+    }
+    if (!capturing && !g->ctx->sig.noAlloc && g->cfg.graph && pp->launches.size() > 1 && pp->exec == nullptr && pp->uses >= 1) {
+        // second use of the same collective on the same buffers: from now on it is replayed from a graph
+        r = BuildGraph(pp);
+        if (r != HCCL_SUCCESS) {
+            return r;
+        }
+    }
+    pp->uses++;
+    const bool viaGraph = pp->exec != nullptr && !capturing;
     g->lastInfo = pp->info;
     g->lastInfo.cacheHit = hit ? 1 : 0;
+    g->lastInfo.graph = viaGraph ? 1 : 0;
 
     // Order the launch after everything queued so far on the other ranks' streams, and order those
     // streams after the collective.  Ranks that share the launcher's stream need nothing.
-    hipStream_t ls = g->ctx->streams[launcher];
     bool others = false;
     for (uint32_t k = 0; k < g->p; k++) {
         if (k == launcher || g->ctx->streams[k] == ls) {
@@ -975,14 +1026,7 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         }
         others = true;
     }
-    // A caller may be capturing this stream into a graph of its own.  A graph launched into a
-    // capturing stream is not recorded there (the caller's graph came out empty and replays did
-    // nothing), so the kernels are then launched one by one and become nodes of the caller's graph.
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (pp->exec) {
-        HIP_OK(hipStreamIsCapturing(ls, &capture));
-    }
-    if (pp->exec && capture == hipStreamCaptureStatusNone) {
+    if (viaGraph) {
         HIP_OK(hipGraphLaunch(pp->exec, ls));
     } else {
         for (LaunchRec &l : pp->launches) {

@@ -15,8 +15,9 @@ constexpr size_t kNoAllocUploadBytes = 3072;               // table bytes per up
 // looks the symbol up; later calls return the kept pointer.
 hipError_t NoAllocWorkspace(int device, void **base);
 
-// Queues on `stream` the launches that write hostBytes[0, bytes) to dst (inside the workspace, 16-byte
-// aligned; the copy is rounded up to a multiple of 16 bytes).  The host bytes are consumed before the call returns.
-hipError_t NoAllocUpload(void *dst, const void *hostBytes, size_t bytes, hipStream_t stream);
+// Queues on `stream` the launches that write hostBytes[0, bytes) to dst (device memory, 16-byte aligned; the
+// copy is rounded up to a multiple of 16 bytes).  The host bytes are consumed before the call returns.
+// Also used for the small tables of ordinary collectives: unlike a host-to-device copy it never waits.
+hipError_t UploadThroughKernelArgs(void *dst, const void *hostBytes, size_t bytes, hipStream_t stream);
 
 }  // namespace hcclamd

@@ -67,7 +67,7 @@ hipError_t NoAllocWorkspace(int device, void **base)
     return hipSuccess;
 }
 
-hipError_t NoAllocUpload(void *dst, const void *hostBytes, size_t bytes, hipStream_t stream)
+hipError_t UploadThroughKernelArgs(void *dst, const void *hostBytes, size_t bytes, hipStream_t stream)
 {
     const unsigned char *from = static_cast<const unsigned char *>(hostBytes);
     unsigned char *to = static_cast<unsigned char *>(dst);

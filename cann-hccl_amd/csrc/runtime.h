@@ -19,6 +19,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include "arena.h"
 #include "hccl/hccl_types.h"
 #include "kernels.h"
 #include "plan.h"
@@ -70,28 +71,25 @@ struct OpInfo {
     uint64_t scratchBytes = 0;
 };
 
-// Device memory for the descriptor tables of the prepared collectives: carved out of a few large
-// allocations, handed back all at once (hipFree waits for the whole device, so it is kept off the
-// path of a caller that cycles through many buffers).
-struct TableArena {
-    struct Chunk {
-        char *base = nullptr;
-        size_t size = 0, used = 0;
-    };
-    std::vector<Chunk> chunks;
-    void *Alloc(size_t bytes);       // nullptr when the device is out of memory
-    void Reset();                    // every block handed out becomes invalid; the first chunk is kept
-    void FreeAll();
-};
-
 struct Prepared {
     std::shared_ptr<const Plan> plan;   // shared with the group's plan cache (plans do not depend on addresses)
     bool fused = false;
     void *devTables = nullptr;        // inside the group's table arena
+    uint32_t tableChunk = 0;          // the arena chunk they came from
     std::vector<LaunchRec> launches;
-    hipGraph_t graph = nullptr;
+    hipGraph_t graph = nullptr;       // built on the second use: a caller that always comes with fresh buffers never pays for it
     hipGraphExec_t exec = nullptr;
     uint64_t scratchGen = 0;
+    uint32_t uses = 0;                // times issued
+    // Small tables are written by upload launches on the stream of the call that prepared them; until those are
+    // known to have finished, a call on another stream orders itself behind them.
+    hipEvent_t uploaded = nullptr;
+    hipStream_t uploadStream = nullptr;
+    bool uploadComplete = true;
+    std::vector<uint8_t> hostTables;  // kept until the upload is known to have finished (a capture records it again)
+    // Recorded into a caller's HIP graph at least once: that graph's kernel nodes point at the tables (and, for a
+    // step-by-step schedule, at the group's scratch buffers), so neither may be freed or reused while the group lives.
+    bool pinned = false;
     OpInfo info;
     ~Prepared();
 };
@@ -171,6 +169,9 @@ struct Group {
     std::vector<hipEvent_t> arriveEvents;
     hipEvent_t doneEvent = nullptr;
     std::vector<void *> scratch;
+    std::vector<void *> retiredScratch;   // scratch buffers a pinned collective still points at; freed with the group
+    uint32_t pinnedScratchUsers = 0;      // pinned collectives that use the current scratch buffers
+    std::vector<std::unique_ptr<Prepared>> pinnedStale;   // pinned collectives that left the cache
     void *barrierMem = nullptr;       // 2 x p small buffers for HcclBarrier's all-reduce
     void *noAllocBase = nullptr;      // this device's copy of the fixed workspace (noalloc.hip), looked up at set-up
     uint64_t scratchBytes = 0;

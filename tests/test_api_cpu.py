@@ -386,6 +386,24 @@ def test_caller_compiles_against_the_reference_header_and_links(tmp_path):
     assert os.path.exists(theirs)
 
 
+def test_table_arena_keeps_blocks_of_collectives_recorded_into_a_callers_graph(tmp_path):
+    """The bookkeeping behind the lifetime rule for captured collectives, on the host: a pinned block's chunk
+    survives Reset() untouched, unpinned chunks are reused or freed, nothing leaks (tests/c_abi/arena_check.cc
+    against cann-hccl_amd/csrc/arena.h with malloc / free as the allocator)."""
+    import os
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        pytest.skip("no host C++ compiler")
+    exe = str(tmp_path / "arena_check")
+    subprocess.run([cxx, "-std=c++17", "-Wall", "-Werror", "-I", os.path.join(root, "cann-hccl_amd", "csrc"),
+                    os.path.join(root, "tests", "c_abi", "arena_check.cc"), "-o", exe], check=True)
+    out = subprocess.run([exe], stdout=subprocess.PIPE, text=True)
+    assert out.returncode == 0 and out.stdout.strip() == "OK", out.stdout
+
+
 def _rank_table(path, servers, per_server, **edits):
     import json
     table = {"server_count": str(servers), "status": "completed", "version": "1.0", "server_list": []}

@@ -143,7 +143,8 @@ def test_graph_replay_and_cache(orc):
             H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, g.stream_ptr)
             g.stream.synchronize()
             info = g.info()
-            assert info["graph"] == 1 and info["launches"] == 2 * (p - 1)
+            # the graph is built when the collective comes back on the same buffers: the first call launches directly
+            assert info["graph"] == (1 if rep else 0) and info["launches"] == 2 * (p - 1)
             assert info["cacheHit"] == (1 if rep else 0)
             for r in range(p):
                 assert np.array_equal(gh.to_host(recvs[r], FP32), want[r]), (rep, r)
@@ -1269,6 +1270,120 @@ def test_collectives_recorded_into_a_callers_graph(orc):
                 finally:
                     graph2.capture_end()
             assert codes[:-1] == [0] * (p - 1) and codes[-1] == H.HCCL_E_NOT_SUPPORT
+        finally:
+            g.close()
+
+
+def test_two_hundred_buffer_sets(orc):
+    # A caller that comes with other buffers every time: every call is a miss of the prepared-collective cache (the
+    # plan itself is shared), tables travel with the call, no graph is built until a buffer set comes back, and a
+    # cache smaller than the number of sets wraps several times.  Every result is checked.
+    p, n, nsets = 8, 3001, 200
+    rng = np.random.default_rng(9)
+    base = [rng.standard_normal(n).astype(np.float32) for _ in range(p)]
+    want = orc.allreduce(base, FP32, SUM)
+    for fuse in (1, 0):
+        g = gh.Group(p, fuse=fuse, cache_entries=64)
+        try:
+            sends = [[torch.from_numpy(base[r] * np.float32(k + 1)).cuda() for r in range(p)] for k in range(nsets)]
+            recvs = [[torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(p)] for _ in range(nsets)]
+            torch.cuda.synchronize()
+            for sweep in range(2):
+                for k in range(nsets):
+                    H.all_reduce(g.comms, [t.data_ptr() for t in sends[k]], [t.data_ptr() for t in recvs[k]], n, FP32, SUM,
+                                 g.stream_ptr)
+                    info = g.info()
+                    assert info["cacheHit"] == 0 and info["graph"] == 0, (fuse, sweep, k)   # 200 sets through 64 entries
+                g.stream.synchronize()
+                for k in (0, 1, 63, 64, 65, 127, 128, 199):
+                    # scaling every input by a power of two or a small integer keeps the sums' rounding: compare with
+                    # the checker on the scaled inputs
+                    scaled = orc.allreduce([x * np.float32(k + 1) for x in base], FP32, SUM)
+                    for r in range(p):
+                        assert np.array_equal(recvs[k][r].cpu().numpy(), scaled[r]), (fuse, sweep, k, r)
+                for row in recvs:
+                    for t in row:
+                        t.zero_()
+                torch.cuda.synchronize()
+            # the same set three times in a row: a hit from the second call, a graph (step by step only) from then on
+            for rep in range(3):
+                H.all_reduce(g.comms, [t.data_ptr() for t in sends[5]], [t.data_ptr() for t in recvs[5]], n, FP32, SUM, g.stream_ptr)
+                info = g.info()
+                assert info["cacheHit"] == (1 if rep else 0)
+                assert info["graph"] == (1 if (rep and not fuse) else 0)
+            g.stream.synchronize()
+            scaled = orc.allreduce([x * np.float32(6) for x in base], FP32, SUM)
+            assert all(np.array_equal(recvs[5][r].cpu().numpy(), scaled[r]) for r in range(p))
+        finally:
+            g.close()
+    del want
+
+
+def test_captured_collectives_survive_cache_wrap_and_scratch_growth(orc):
+    # A caller's graph holds kernel nodes that point at a collective's tables and, step by step, at the group's scratch
+    # buffers.  Later library activity -- a wrap of the prepared-collective cache, a larger scratch request -- must
+    # not free or reuse either: every replay still gives the eager result.
+    p, n = 8, 50021
+    for fuse in (1, 0):
+        g = gh.Group(p, fuse=fuse, cache_entries=4)
+        try:
+            rng = np.random.default_rng(70 + fuse)
+            ins = [rng.standard_normal(n * p).astype(np.float32) for _ in range(p)]
+            sends = [torch.from_numpy(x).cuda() for x in ins]
+            recvs = [torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(p)]
+            torch.cuda.synchronize()
+            want = orc.reducescatter(ins, FP32, SUM)
+
+            def rs():
+                H.reduce_scatter(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, g.stream_ptr)
+
+            rs()                                     # prepared outside the capture
+            g.stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(g.stream):
+                graph.capture_begin()
+                try:
+                    rs()
+                finally:
+                    graph.capture_end()
+
+            def replay_and_check(what):
+                for t in recvs:
+                    t.zero_()
+                torch.cuda.synchronize()
+                graph.replay()
+                torch.cuda.synchronize()
+                for r in range(p):
+                    assert np.array_equal(recvs[r].cpu().numpy(), want[r]), (fuse, what, r)
+
+            replay_and_check("fresh")
+            # wrap the cache several times over with other buffers and sizes
+            others = [torch.ones(4096, dtype=torch.float32, device="cuda") for _ in range(2 * p)]
+            for k in range(14):
+                m = 64 + 16 * k
+                H.all_reduce(g.comms, [t.data_ptr() for t in others[:p]], [t.data_ptr() for t in others[p:]], m, FP32, SUM,
+                             g.stream_ptr)
+            g.stream.synchronize()
+            replay_and_check("after cache wraps")
+            # a step-by-step reduce-scatter three times the size asks for larger scratch buffers
+            big_s = [torch.ones(3 * n * p, dtype=torch.float32, device="cuda") for _ in range(p)]
+            big_r = [torch.zeros(3 * n, dtype=torch.float32, device="cuda") for _ in range(p)]
+            torch.cuda.synchronize()
+            H.reduce_scatter(g.comms, [t.data_ptr() for t in big_s], [t.data_ptr() for t in big_r], 3 * n, FP32, SUM, g.stream_ptr)
+            g.stream.synchronize()
+            assert all(float(t[0]) == p for t in big_r)
+            for k in range(6):
+                H.all_reduce(g.comms, [t.data_ptr() for t in others[:p]], [t.data_ptr() for t in others[p:]], 1000 + k, FP32, SUM,
+                             g.stream_ptr)
+            g.stream.synchronize()
+            replay_and_check("after scratch growth")
+            # and the eager path still works on the same buffers
+            for t in recvs:
+                t.zero_()
+            rs()
+            g.stream.synchronize()
+            for r in range(p):
+                assert np.array_equal(recvs[r].cpu().numpy(), want[r]), (fuse, "eager", r)
         finally:
             g.close()
 
