@@ -145,3 +145,110 @@ def test_buffers_larger_than_4_gib():
                 assert torch.equal(outs[r][j * m:(j + 1) * m], sends[j][:m]), (r, j)
     finally:
         g.close()
+
+
+def _device_inputs(dt, p, n, seed):
+    """Inputs of BASELINE.json's reduce-scatter configuration, made on the device: fp16 / bf16 ~ N(0, 1), int8 / int32
+    uniform over the full range, int64 uniform in [-2^40, 2^40).  Returns device tensors and their host copies as
+    carrier arrays."""
+    from closed_forms import BF16, CARRIER, FP16, INT8, INT32, INT64
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    dev = []
+    for _ in range(p):
+        if dt in (FP16, BF16):
+            t = torch.randn(n, dtype=torch.float32, device="cuda", generator=gen).to(torch.float16 if dt == FP16 else torch.bfloat16)
+        elif dt == INT64:
+            t = torch.randint(-(1 << 40), 1 << 40, (n,), dtype=torch.int64, device="cuda", generator=gen)
+        elif dt == INT32:
+            t = torch.randint(-(1 << 31), 1 << 31, (n,), dtype=torch.int64, device="cuda", generator=gen).to(torch.int32)
+        else:
+            assert dt == INT8
+            t = torch.randint(-128, 128, (n,), dtype=torch.int16, device="cuda", generator=gen).to(torch.int8)
+        dev.append(t)
+    torch.cuda.synchronize()
+    host = [t.view(torch.int16).cpu().numpy().view(CARRIER[dt]) if dt in (FP16, BF16) else t.cpu().numpy() for t in dev]
+    return dev, host
+
+
+def test_reducescatter_64mib_per_rank_every_op_and_type():
+    """BASELINE.json configs[2] in full: ring reduce-scatter over 8 ranks, 64 MiB per rank, {sum, prod, max, min} x
+    {fp16, bf16, int8, int32, int64}, fused and step by step, against the checker at full size.  Integers bit-exact;
+    fp16 / bf16 within 1 ulp (they come out bit-equal: both sides accumulate in fp32 and round once per stored step)."""
+    from closed_forms import BF16, CARRIER, FP16, INT8, INT32, INT64, MAX, MIN, PROD
+    from oracle import oracle as orc
+    from test_gpu_parity import _ulp_close
+    orc.build()
+    p = 8
+    bit_equal_16 = 0
+    for dt in (FP16, BF16, INT8, INT32, INT64):
+        unit = H.DTYPE_SIZE[dt]
+        n = (64 << 20) // unit // p                          # elements each rank receives
+        sends, ins = _device_inputs(dt, p, n * p, 4242 + dt)
+        for op in (SUM, PROD, MAX, MIN):
+            print("reduce-scatter 64 MiB per rank: type", dt, "op", op, flush=True)
+            want = orc.reducescatter(ins, dt, op, flags=orc.DIRECT, threads=16)
+            for fuse in (1, 0):
+                g = gh.Group(p, fuse=fuse)
+                try:
+                    recvs = [gh.empty_dev(n * unit) for _ in range(p)]
+                    torch.cuda.synchronize()
+                    H.reduce_scatter(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, op, g.stream_ptr)
+                    g.stream.synchronize()
+                    assert g.info()["fused"] == fuse
+                    for r in range(p):
+                        got = gh.to_host(recvs[r], dt)
+                        if dt in (FP16, BF16):
+                            assert _ulp_close(dt, got, want[r]), (dt, op, fuse, r)       # the bar: within 1 ulp
+                            bit_equal_16 += int(gh.same(dt, got, want[r]))
+                        else:
+                            assert np.array_equal(got, want[r]), (dt, op, fuse, r)
+                    del recvs
+                finally:
+                    g.close()
+        # the inputs are still what they were
+        assert np.array_equal(sends[p - 1].view(torch.int16).cpu().numpy().view(CARRIER[dt]) if dt in (FP16, BF16)
+                              else sends[p - 1].cpu().numpy(), ins[p - 1])
+        del sends, ins
+    assert bit_equal_16 == 2 * 4 * 2 * p                      # and in fact every 16-bit float result was bit-equal
+
+
+def test_ring_allreduce_size_sweep_8kib_to_256mib():
+    """BASELINE.json configs[1]: ring all-reduce, sum, fp32, 8 ranks, every size of the sweep (8 KiB ... 256 MiB per
+    rank, doubling), fused and step by step, bit for bit against the checker; inputs uniform in [-1, 1) from a seed."""
+    from oracle import oracle as orc
+    orc.build()
+    p, nmax = 8, 64 << 20
+    ins = [orc.fill_uniform_f32(nmax, 77, r, threads=16) for r in range(p)]
+    sends = [torch.from_numpy(x).cuda() for x in ins]
+    recvs = [torch.empty(nmax, dtype=torch.float32, device="cuda") for _ in range(p)]
+    torch.cuda.synchronize()
+    groups = {fuse: gh.Group(p, fuse=fuse) for fuse in (1, 0)}
+    try:
+        size = 8 << 10
+        sizes = []
+        while size <= (256 << 20):
+            sizes.append(size)
+            size *= 2
+        assert len(sizes) == 16
+        for size in sizes:
+            n = size // 4
+            work = [x[:n].copy() for x in ins]
+            outs = [np.empty(n, np.float32) for _ in range(p)]
+            orc.allreduce(work, FP32, SUM, flags=orc.DIRECT | orc.ZERO_STAGING, threads=16, outs=outs)
+            for fuse in (1, 0):
+                g = groups[fuse]
+                print("all-reduce sweep: bytes per rank", size, "fuse", fuse, flush=True)
+                for t in recvs:
+                    t[:n].zero_()
+                torch.cuda.synchronize()
+                H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, g.stream_ptr)
+                g.stream.synchronize()
+                assert g.info()["fused"] == fuse
+                for r in (0, 3, p - 1):
+                    assert np.array_equal(recvs[r][:n].cpu().numpy(), outs[r]), (size, fuse, r)
+                for r in range(1, p):
+                    assert torch.equal(recvs[0][:n], recvs[r][:n]), (size, fuse, r)
+    finally:
+        for g in groups.values():
+            g.close()
