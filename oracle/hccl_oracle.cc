@@ -32,7 +32,8 @@
 //                    coll_all_to_all_v_staged_executor.cc:276-470, coll_all_to_all_executor.cc:156-335 (zero-copy mode)
 //   rooted           TPL/temp_broadcast/broadcast_ring.cc:24-160, TPL/temp_reduce/reduce_ring.cc:29-154,
 //                    TPL/temp_scatter/scatter_mesh.cc:46-160, TPL/temp_gather/gather_mesh.cc:60-170,
-//                    EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213, EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194,
+//                    EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213 (one server and several: scatter, halving-doubling
+//                    between the servers, all-gather), EXE/coll_reduce/coll_reduce_mesh_executor.cc:75-194,
 //                    TPL/temp_reduce/reduce_recursive_hd.cc:31-316, TPL/temp_broadcast/bcast_recursive_halvingdoubling.cc:21-290
 //
 // Method: every template is restated as the per-rank program it issues (send / receive-and-reduce /
@@ -1974,29 +1975,13 @@ int orc_broadcast_mesh(uint32_t p, void **buf, uint64_t count, int dt, uint32_t 
     return 0;
 }
 
-// Recursive halving-doubling broadcast, BcastRecursiveHalvingDoubling::RunAsync
-// (TPL/temp_broadcast/bcast_recursive_halvingdoubling.cc:21-290): BroadcastInBlock (:162-203) and the hand-over
-// inside the rank pairs of part one (:205-262); block membership from GetRankIndexInBlock (:138-160).
-int orc_broadcast_rhd(uint32_t p, void **buf, uint64_t count, int dt, uint32_t root, uint64_t cclBytes, uint64_t align,
-    int flags, int threads)
+// Per-rank programs of BcastRecursiveHalvingDoubling::RunAsync
+// (TPL/temp_broadcast/bcast_recursive_halvingdoubling.cc:21-290) on the machine's buffers: the `bytes` bytes at
+// offset `off` of the root's buffer reach every rank.  BroadcastInBlock (:162-203) and the hand-over inside the rank
+// pairs of part one (:205-262); block membership from GetRankIndexInBlock (:138-160).
+void AddBroadcastRhdProcs(Machine &m, uint32_t root, uint64_t off, uint64_t bytes)
 {
-    (void)align;
-    uint64_t unit = DtSize(dt);
-    if (unit == 0 || p == 0 || root >= p) {
-        return -20;
-    }
-    uint64_t maxPer = cclBytes / unit;
-    if (maxPer == 0) {
-        return -21;
-    }
-    Pool pool(threads);
-    Machine m;
-    m.p = static_cast<int>(p);
-    m.dt = dt;
-    m.direct = (flags & 1) != 0;
-    m.pool = &pool;
-    m.buf[B_IN].resize(p);
-    m.buf[B_OUT].resize(p);
+    const uint32_t p = static_cast<uint32_t>(m.p);
     uint32_t block, part1;
     RhdParams(p, &block, &part1);
     const bool rootEven = (root < part1 && (root % 2) == 0) || root >= part1;
@@ -2019,6 +2004,60 @@ int orc_broadcast_rhd(uint32_t p, void **buf, uint64_t count, int dt, uint32_t r
     while ((1u << rounds) < block) {
         rounds++;
     }
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        int q = inBlock(r);
+        if (q >= 0) {
+            const uint32_t rq = static_cast<uint32_t>(q), rootQ = static_cast<uint32_t>(inBlock(root));
+            bool hasData = r == root;
+            for (uint32_t i = 0; i < rounds; i++) {
+                const uint32_t mask = 1u << (rounds - i - 1);
+                const uint32_t peer = real(rq ^ mask);
+                if ((rq & (mask - 1)) == (rootQ & (mask - 1)) && r != root && !hasData) {
+                    pr.prog.push_back(MkRecvCopy(static_cast<int>(peer), 0, B_IN, off, bytes));
+                    hasData = true;
+                    continue;
+                }
+                if (hasData) {
+                    pr.prog.push_back(MkSend(static_cast<int>(peer), 0, B_IN, off, bytes));
+                }
+            }
+        }
+        if (r < part1) {
+            const uint32_t pairPeer = (r % 2) == 0 ? r + 1 : r - 1;
+            const bool sends = ((r % 2) == 0) == rootEven;   // EvenNumberRankProcess / OddNumberRankProcess
+            if (sends) {
+                pr.prog.push_back(MkSend(static_cast<int>(pairPeer), 1, B_IN, off, bytes));
+            } else {
+                pr.prog.push_back(MkRecvCopy(static_cast<int>(pairPeer), 1, B_IN, off, bytes));
+            }
+        }
+        m.procs.push_back(std::move(pr));
+    }
+}
+
+// Recursive halving-doubling broadcast with the executor's chunk loop.
+int orc_broadcast_rhd(uint32_t p, void **buf, uint64_t count, int dt, uint32_t root, uint64_t cclBytes, uint64_t align,
+    int flags, int threads)
+{
+    (void)align;
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
     uint64_t offset = 0;
     for (uint64_t left = count; left > 0 && p > 1;) {
         uint64_t cur = left > maxPer ? maxPer : left;
@@ -2027,43 +2066,131 @@ int orc_broadcast_rhd(uint32_t p, void **buf, uint64_t count, int dt, uint32_t r
             m.buf[B_IN][r] = static_cast<uint8_t *>(buf[r]) + offset;
             m.buf[B_OUT][r] = static_cast<uint8_t *>(buf[r]) + offset;
         }
-        for (uint32_t r = 0; r < p; r++) {
-            Proc pr;
-            pr.rank = r;
-            int q = inBlock(r);
-            if (q >= 0) {
-                const uint32_t rq = static_cast<uint32_t>(q), rootQ = static_cast<uint32_t>(inBlock(root));
-                bool hasData = r == root;
-                for (uint32_t i = 0; i < rounds; i++) {
-                    const uint32_t mask = 1u << (rounds - i - 1);
-                    const uint32_t peer = real(rq ^ mask);
-                    if ((rq & (mask - 1)) == (rootQ & (mask - 1)) && r != root && !hasData) {
-                        pr.prog.push_back(MkRecvCopy(static_cast<int>(peer), 0, B_IN, 0, bytes));
-                        hasData = true;
-                        continue;
-                    }
-                    if (hasData) {
-                        pr.prog.push_back(MkSend(static_cast<int>(peer), 0, B_IN, 0, bytes));
-                    }
-                }
-            }
-            if (r < part1) {
-                const uint32_t pairPeer = (r % 2) == 0 ? r + 1 : r - 1;
-                const bool sends = ((r % 2) == 0) == rootEven;   // EvenNumberRankProcess / OddNumberRankProcess
-                if (sends) {
-                    pr.prog.push_back(MkSend(static_cast<int>(pairPeer), 1, B_IN, 0, bytes));
-                } else {
-                    pr.prog.push_back(MkRecvCopy(static_cast<int>(pairPeer), 1, B_IN, 0, bytes));
-                }
-            }
-            m.procs.push_back(std::move(pr));
-        }
+        AddBroadcastRhdProcs(m, root, 0, bytes);
         int rc = m.Run();
         if (rc != 0) {
             return rc;
         }
         offset += bytes;
         left -= cur;
+    }
+    return 0;
+}
+
+// Two-level broadcast, CollBroadcastMeshExecutor::KernelRun with several servers
+// (EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213) under the chunk loop of
+// CollBroadcastExecutor::RunLoop (coll_broadcast_executor.cc:83-121); `servers` groups of D = p / servers consecutive
+// ranks.  Per chunk: slices over the D ranks of a group (GetRankSliceSize, coll_broadcast_executor.cc:275-306);
+// stage 0 (:131-147) only in the root's group: the root scatters slice d to the rank at position d
+// (TPL/temp_scatter/scatter_mesh.cc:46-160); stage 1 (:148-186): the ranks at position d of all groups broadcast
+// slice d from the root's group by recursive halving-doubling (the default level-1 choice of :113-117; count =
+// the slice's size, base offset = the slice's offset); stage 2 (:189-207): mesh all-gather of the slices inside
+// every group (TPL/temp_all_gather/all_gather_mesh.cc:91-145).
+// `touched` (optional) receives the bytes read + written by all ranks (2 x the bytes received).
+int orc_broadcast_two_level(uint32_t servers, uint32_t p, void **buf, uint64_t count, int dt, uint32_t root,
+    uint64_t cclBytes, uint64_t align, int flags, int threads, uint64_t *touched)
+{
+    uint64_t moved = 0;
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p || servers == 0 || p % servers != 0) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    const uint32_t D = p / servers, rootGroup = root / D, rootLocal = root % D;
+    Pool pool(threads);
+    auto machine = [&](uint32_t n) {
+        Machine m;
+        m.p = static_cast<int>(n);
+        m.dt = dt;
+        m.direct = (flags & 1) != 0;
+        m.pool = &pool;
+        m.buf[B_IN].resize(n);
+        m.buf[B_OUT].resize(n);
+        return m;
+    };
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0 && p > 1;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        uint64_t avg = bytes / D + ((cur % D) > 0 ? 1 : 0);
+        uint64_t per = RoundUp(avg, align);
+        std::vector<Slice> sl(D);
+        uint64_t residue = bytes;
+        for (uint32_t i = 0; i < D; i++) {
+            sl[i].size = per < residue ? per : residue;
+            sl[i].off = sl[i].size == 0 ? 0 : i * per;
+            residue -= sl[i].size;
+        }
+        auto at = [&](uint32_t g, uint32_t d) { return static_cast<uint8_t *>(buf[g * D + d]) + offset; };
+        if (D > 1) {                                   // stage 0: scatter inside the root's group
+            Machine m = machine(D);
+            for (uint32_t d = 0; d < D; d++) {
+                m.buf[B_IN][d] = m.buf[B_OUT][d] = at(rootGroup, d);
+            }
+            for (uint32_t d = 0; d < D; d++) {
+                Proc pr;
+                pr.rank = d;
+                if (d == rootLocal) {
+                    for (uint32_t to = 0; to < D; to++) {
+                        if (to != rootLocal) {
+                            pr.prog.push_back(MkSend(static_cast<int>(to), 0, B_IN, sl[to].off, sl[to].size));
+                        }
+                    }
+                } else {
+                    pr.prog.push_back(MkRecvCopy(static_cast<int>(rootLocal), 0, B_OUT, sl[d].off, sl[d].size));
+                }
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+            moved += m.bytesTouched;
+        }
+        if (servers > 1) {                             // stage 1: slice d between the groups
+            for (uint32_t d = 0; d < D; d++) {
+                if (sl[d].size == 0) {
+                    continue;
+                }
+                Machine m = machine(servers);
+                for (uint32_t g = 0; g < servers; g++) {
+                    m.buf[B_IN][g] = m.buf[B_OUT][g] = at(g, d);
+                }
+                AddBroadcastRhdProcs(m, rootGroup, sl[d].off, sl[d].size);
+                int rc = m.Run();
+                if (rc != 0) {
+                    return rc;
+                }
+                moved += m.bytesTouched;
+            }
+        }
+        if (D > 1) {                                   // stage 2: all-gather inside every group
+            for (uint32_t g = 0; g < servers; g++) {
+                Machine m = machine(D);
+                for (uint32_t d = 0; d < D; d++) {
+                    m.buf[B_IN][d] = m.buf[B_OUT][d] = at(g, d);
+                }
+                for (uint32_t d = 0; d < D; d++) {
+                    Proc pr;
+                    pr.rank = d;
+                    ProgAllGatherMesh(pr.prog, d, D, B_OUT, sl);
+                    m.procs.push_back(std::move(pr));
+                }
+                int rc = m.Run();
+                if (rc != 0) {
+                    return rc;
+                }
+                moved += m.bytesTouched;
+            }
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    if (touched != nullptr) {
+        *touched = moved;
     }
     return 0;
 }

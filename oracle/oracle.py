@@ -74,6 +74,7 @@ def lib():
         L.orc_reduce_to_root_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_rhd.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
+        L.orc_broadcast_two_level.argtypes = [u32, u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32, ctypes.POINTER(u64)]
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
         L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
         L.orc_scatter_ring.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
@@ -286,6 +287,18 @@ def broadcast(bufs, dt, root, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, 
     if rc != 0:
         raise RuntimeError("oracle broadcast failed rc=%d" % rc)
     return bufs
+
+
+def broadcast_two_level(bufs, dt, root, servers, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1,
+                        return_touched=False):
+    """`servers` groups of consecutive ranks: scatter in the root's group, halving-doubling broadcast of slice d among
+    the ranks at position d, mesh all-gather in every group.  bufs are written in place."""
+    touched = ctypes.c_uint64(0)
+    rc = lib().orc_broadcast_two_level(servers, len(bufs), _ptrs(bufs), bufs[0].size, dt, root, ccl_bytes, align, flags, threads,
+                                       ctypes.byref(touched))
+    if rc != 0:
+        raise RuntimeError("oracle two-level broadcast failed rc=%d" % rc)
+    return (bufs, touched.value) if return_touched else bufs
 
 
 def reduce_to_root(ins, dt, op, root, ccl_bytes=DEFAULT_CCL_BYTES, flags=0, threads=1, algo=RING, align=DEFAULT_ALIGN):

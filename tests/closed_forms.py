@@ -74,6 +74,19 @@ def slice_plan(total, n, align):
     return out
 
 
+def broadcast_slices(count, unit, n, align):
+    """Slices of the mesh broadcast's scatter / all-gather (CollBroadcastExecutor::GetRankSliceSize,
+    coll_broadcast_executor.cc:275-306): ceil-ish share of the bytes rounded up to `align`, the rest to the last."""
+    share = (count * unit) // n + (1 if count % n else 0)
+    per = -(-share // align) * align
+    out, residue = [], count * unit
+    for i in range(n):
+        size = min(per, residue)
+        out.append((i * per if size else 0, size))
+        residue -= size
+    return out
+
+
 def ring_chain(dt, op, xs, s):
     """Ring reduce-scatter result for slice s: x[s] (+) (x[s-1] (+) (... (x[s+2] (+) x[s+1])))."""
     p = len(xs)

@@ -1044,8 +1044,14 @@ def test_two_level_broadcast_and_schedule_switch_on_the_same_buffers(orc):
                     info = g.info()
                     if not fuse:
                         assert info["launches"] >= 3                         # scatter, between the groups, gather
+                    want, touched = orc.broadcast_two_level([x.copy() for x in bufs_np], INT32, root, servers, return_touched=True)
                     for r in range(p):
-                        assert np.array_equal(gh.to_host(bufs[r], INT32), bufs_np[root]), (servers, D, fuse, root, r)
+                        assert np.array_equal(gh.to_host(bufs[r], INT32), want[r]), (servers, D, fuse, root, r)
+                    if not fuse:
+                        # what the launches wrote = what the checker's ranks received, less the slices the all-gather
+                        # of the root's group hands back to the root
+                        back = n * 4 - cf.broadcast_slices(n, 4, D, 128)[root % D][1]
+                        assert info["bytesWritten"] == touched // 2 - back, (servers, D, root)
                 ins = _ins(FP32, p, n, 650 + p)
                 ins[0][:] *= 1e7
                 ins[p - 1][:] *= -1e7

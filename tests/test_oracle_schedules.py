@@ -550,3 +550,110 @@ def test_two_level_allgather_is_the_concatenation(orc, level1, level0):
             want = np.concatenate(ins)
             for r in range(p):
                 assert np.array_equal(got[r], want), (servers, D, level1, level0, dt, ccl, r)
+
+
+def _v_blocks(p, seed, scale=400):
+    """Block table of a variable-count collective: some empty blocks, shuffled order, gaps between the blocks."""
+    rng = np.random.default_rng(seed)
+    counts = rng.integers(0, scale, p)
+    counts[rng.random(p) < 0.2] = 0
+    displs, pos = np.zeros(p, np.int64), 0
+    for i in rng.permutation(p):
+        pos += int(rng.integers(0, 9))
+        displs[i] = pos
+        pos += int(counts[i])
+    return counts, displs, pos + 3
+
+
+@pytest.mark.parametrize("algo", [RING, MESH, MESH_ATOMIC])
+def test_reducescatter_v_matches_chain(orc, algo):
+    # the variable-count reduce-scatter runs the same templates over the caller's block table: block r comes out as
+    # the ring chain / the mesh chains of its pieces, evaluated here with numpy on the block's elements alone
+    for dt in (FP32, BF16, INT8, INT64):
+        unit = orc.dtype_size(dt)
+        for p in (1, 2, 3, 6, 8):
+            for op in (SUM, MAX) if dt != FP32 else OPS:
+                counts, displs, extent = _v_blocks(p, 31 * p + dt + op)
+                ins = _inputs(dt, p, extent, 7 * p + op)
+                got = orc.reducescatter_v(ins, counts, displs, dt, op, algo=algo)
+                for r in range(p):
+                    lo, n = int(displs[r]), int(counts[r])
+                    xs = [x[lo:lo + n] for x in ins]
+                    if p == 1:
+                        want = xs[0]
+                    elif algo == RING:
+                        want = cf.ring_chain(dt, op, xs, r)
+                    elif algo == MESH_ATOMIC:
+                        want = cf.mesh_atomic_chain(dt, op, xs, r)
+                    else:
+                        want = np.empty_like(xs[0])
+                        nstream = p - 1 if p > 2 else 1
+                        for t, (po, ps) in enumerate(cf.slice_plan(n * unit, nstream, 128) if n else []):
+                            a, b = po // unit, (po + ps) // unit
+                            if b > a:
+                                want[a:b] = cf.mesh_chain(dt, op, [x[a:b] for x in xs], r, t)
+                    assert got[r].size == n and _eq(dt, got[r], want), (algo, dt, p, op, r)
+
+
+def test_reducescatter_v_order_sensitive_known_answer(orc):
+    # fp32 sums where the association decides the bits: 2^24 absorbs a 1 added to it directly.  Three ranks, the
+    # three blocks in shuffled places; block r of rank j holds v[(j - r) % 3] with v = (2^24, 1, 1), so that the
+    # ring (x_r + (x_{r-1} + x_{r+1})) gives 2^24 + 2 and the uncut mesh ((x_r + x_{r+1}) + x_{r+2}) gives 2^24
+    big = np.float32(16777216.0)
+    counts, displs = [5, 5, 5], [11, 0, 22]
+    v = [big, np.float32(1.0), np.float32(1.0)]
+    ins = []
+    for j in range(3):
+        x = np.zeros(30, np.float32)
+        for r in range(3):
+            x[displs[r]:displs[r] + 5] = v[(j - r) % 3]
+        ins.append(x)
+    ring = orc.reducescatter_v(ins, counts, displs, FP32, SUM, algo=RING)
+    atomic = orc.reducescatter_v(ins, counts, displs, FP32, SUM, algo=MESH_ATOMIC)
+    for r in range(3):
+        assert np.all(ring[r] == np.float32(16777218.0)), r
+        assert np.all(atomic[r] == big), r
+
+
+@pytest.mark.parametrize("algo", [RING, MESH])
+def test_allgather_v_is_the_permutation(orc, algo):
+    for dt in (INT8, FP16, INT32, INT64):
+        for p in (1, 2, 3, 6, 8, 13):
+            counts, displs, extent = _v_blocks(p, 5 * p + dt)
+            ins = [_inputs(dt, 1, int(counts[r]), 100 * p + r)[0] for r in range(p)]
+            fill = 0x5A
+            got = orc.allgather_v(ins, counts, displs, extent, dt, algo=algo, fill=fill)
+            want = np.full(extent, fill, dtype=ins[0].dtype)
+            for r in range(p):
+                want[int(displs[r]):int(displs[r]) + int(counts[r])] = ins[r]
+            for r in range(p):
+                assert np.array_equal(got[r], want), (algo, dt, p, r)       # blocks in place, gaps untouched
+
+
+@pytest.mark.parametrize("shape", [(2, 4), (4, 2), (3, 2), (3, 4), (1, 4), (8, 1), (5, 3)])
+def test_two_level_broadcast_delivers_and_moves_the_closed_form_bytes(orc, shape):
+    # Definition: every rank ends with the root's bytes.  Structure: the bytes received over all ranks are those of
+    # scatter (root's group) + one halving-doubling broadcast per slice between the groups + one mesh all-gather per
+    # group -- a flat broadcast, or a level 1 that moved the whole buffer, would count differently.
+    servers, D = shape
+    p = servers * D
+    for dt, n in ((INT32, 1), (INT32, 1000), (INT8, 100003), (INT64, 5000)):
+        unit = orc.dtype_size(dt)
+        for root in sorted({0, p - 1, p // 2, D - 1, min(D, p - 1)}):
+            for ccl in (200 << 20, 8192):
+                bufs = _inputs(dt, p, n, root + n)
+                src = bufs[root].copy()
+                bufs, touched = orc.broadcast_two_level(bufs, dt, root, servers, ccl_bytes=ccl, return_touched=True)
+                assert all(np.array_equal(b, src) for b in bufs), (shape, dt, n, root, ccl)
+                received, left = 0, n
+                max_per = ccl // unit
+                while left > 0 and p > 1:
+                    cur = min(left, max_per)
+                    sl = cf.broadcast_slices(cur, unit, D, 128)
+                    total = cur * unit
+                    if D > 1:
+                        received += total - sl[root % D][1]                   # scatter in the root's group
+                        received += servers * (D - 1) * total                 # all-gather in every group
+                    received += (servers - 1) * total                        # slice d reaches position d of every other group
+                    left -= cur
+                assert touched == 2 * received, (shape, dt, n, root, ccl)

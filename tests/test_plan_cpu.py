@@ -695,7 +695,7 @@ def test_ring_scatter_plan_matches_checker(orc, p):
 
 
 @pytest.mark.parametrize("servers,D", [(2, 4), (4, 2), (3, 4), (5, 3), (6, 1), (2, 8)])
-def test_two_level_broadcast_plan(servers, D):
+def test_two_level_broadcast_plan(orc, servers, D):
     # scatter inside the root's group, halving-doubling between the groups, all-gather inside every group:
     # every rank ends with the root's data, and a block only moves inside a group or between equal positions
     p = servers * D
@@ -714,6 +714,18 @@ def test_two_level_broadcast_plan(servers, D):
             if ccl >= n * 4 and D > 1 and servers > 1:
                 flat = H.describe_plan(H.COLL_BROADCAST, root | (MESH << 16), p, n, INT32, in_place_mask=(1 << p) - 1)
                 assert len(plan["phases"]) > len(flat["phases"])                 # two more stages than scatter + gather
+            # The checker's executor for the same schedule receives the same bytes, plus the slices that the all-gather
+            # of the root's group hands back to the root, which holds them already: the plan leaves the root alone.
+            out, touched = orc.broadcast_two_level([b.copy() for b in bufs], INT32, root, servers, ccl_bytes=ccl,
+                                                   return_touched=True)
+            assert all(np.array_equal(b, bufs[root]) for b in out)
+            back_to_root, left = 0, n
+            while left > 0 and D > 1:
+                cur = min(left, ccl // 4)
+                back_to_root += cur * 4 - cf.broadcast_slices(cur, 4, D, 128)[root % D][1]
+                left -= cur
+            assert plan["stepWritten"] == touched // 2 - back_to_root, (servers, D, root, ccl)
+            assert plan["stepRead"] == plan["stepWritten"]
             for fused in (False, True):
                 sends = _bytes(bufs)
                 recvs = [s for s in sends]                                       # one buffer per rank
