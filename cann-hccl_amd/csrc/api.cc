@@ -1473,6 +1473,32 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
             return HCCL_E_PARA;
         }
         cfg.cacheEntries = uint32_t(n);
+    } else if (k == "nic_ranks") {
+        // the ranks of an 8-rank ring that own a network port: "all", or a comma-separated list of 1, 2 or 4 ranks
+        uint32_t mask = 0;
+        if (v != "all" && !v.empty()) {
+            if (c->group->p != 8) {
+                return HCCL_E_PARA;
+            }
+            std::stringstream in(v);
+            std::string item;
+            while (std::getline(in, item, ',')) {
+                char *end = nullptr;
+                long r = std::strtol(item.c_str(), &end, 10);
+                if (item.empty() || *end != 0 || r < 0 || r > 7 || ((mask >> r) & 1u)) {
+                    return HCCL_E_PARA;
+                }
+                mask |= 1u << r;
+            }
+            const int ports = __builtin_popcount(mask);
+            if (ports != 1 && ports != 2 && ports != 4 && ports != 8) {
+                return HCCL_E_PARA;
+            }
+            if (ports == 8) {
+                mask = 0;
+            }
+        }
+        cfg.nicMask = mask;
     } else if (k == "fused_stores") {
         if (v == "auto") {
             cfg.fusedStores = -1;
@@ -1593,6 +1619,7 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         rq.servers = std::max(1u, (uint32_t(algo) >> 8) & 0xffu);
         rq.meshAtomic = ((uint32_t(algo) >> 16) & 1u) != 0;   // bit 16: mesh level without the piece cut
         rq.level0Rings = (uint32_t(algo) >> 17) & 7u;         // bits 17..19: rings inside a group (0 = mesh, 1, 4)
+        rq.nicMask = (uint32_t(algo) >> 20) & 0xffu;          // bits 20..27: ranks with a network port (8-rank ring)
     } else if (coll == COLL_REDUCESCATTER || coll == COLL_ALLGATHER) {
         // reduce-scatter, all-gather: the same fields
         rq.algo = Algo(uint32_t(algo) & 0xffu);

@@ -575,7 +575,7 @@ std::string CacheKey(const Group *g, int algo)
         put(g->ctx->vDispls.data(), g->ctx->vDispls.size() * 8);
         key.push_back('v');
     }
-    uint64_t head[10] = {uint64_t(g->ctx->sig.coll), uint64_t(algo), uint64_t(g->ctx->sig.dtype), uint64_t(g->ctx->sig.op), g->ctx->sig.count,
+    uint64_t head[11] = {uint64_t(g->cfg.nicMask), uint64_t(g->ctx->sig.coll), uint64_t(algo), uint64_t(g->ctx->sig.dtype), uint64_t(g->ctx->sig.op), g->ctx->sig.count,
         uint64_t(g->cfg.fuse) | (uint64_t(g->cfg.graph) << 1) | (uint64_t(g->ctx->sig.root) << 8) | (uint64_t(g->ctx->sig.peer) << 20), g->cfg.cclBytes, g->cfg.align,
         uint64_t(g->cfg.blocksPerCu) | (uint64_t(uint32_t(g->cfg.stepStores + 1)) << 32) | (uint64_t(g->cfg.servers) << 40) |
             (uint64_t(uint32_t(g->cfg.algo + 1) & 0xfu) << 48) | (uint64_t(g->cfg.deterministic) << 56) | (uint64_t(g->cfg.level0Rings) << 57) |
@@ -604,7 +604,7 @@ int CachedPlan(Group *g, const PlanRequest &rq, std::shared_ptr<const Plan> *out
         put(&n, sizeof(n));
         put(v.data(), v.size() * sizeof(uint64_t));
     };
-    uint64_t head[10] = {uint64_t(rq.coll), uint64_t(rq.algo), rq.p, rq.count, rq.root, rq.peer, rq.unit, rq.cclBytes, rq.align,
+    uint64_t head[11] = {uint64_t(rq.nicMask), uint64_t(rq.coll), uint64_t(rq.algo), rq.p, rq.count, rq.root, rq.peer, rq.unit, rq.cclBytes, rq.align,
         uint64_t(rq.meshAtomic) | (uint64_t(rq.stageInput) << 1) | (uint64_t(rq.servers) << 8) | (uint64_t(rq.level0Rings) << 40)};
     put(head, sizeof(head));
     put(rq.alias.data(), rq.alias.size());
@@ -675,6 +675,11 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAl
         rq.level0Rings = g->cfg.level0Rings == 4 ? (fourRings ? 4u : 1u) : g->cfg.level0Rings;
         rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
             g->ctx->sig.op != HCCL_REDUCE_PROD;
+    }
+    if (rq.coll == COLL_ALLREDUCE && rq.servers <= 1 && rq.level0Rings == 0 && rq.algo == ALGO_RING && g->p == 8) {
+        // an 8-rank ring some of whose ranks have no network port: the port-pruned reduce-scatter
+        // (reduce_scatter_ring.cc:160-168)
+        rq.nicMask = g->cfg.nicMask;
     }
     if (rq.coll == COLL_REDUCESCATTER && !g->ctx->sig.variable && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
         // two levels (coll_reduce_scatter_mesh_executor.cc:128-247, coll_reduce_scatter_ring_executor.cc:132-340):

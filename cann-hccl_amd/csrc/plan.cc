@@ -114,6 +114,59 @@ size_t RingAllGatherPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t bas
     return phase0 + (p - 1);
 }
 
+// The ring reduce-scatter and all-gather with the slices' chains ending at other ranks than "slice i at rank i":
+// slice i is reduced along owner[i] + 1 -> owner[i] + 2 -> ... -> owner[i] and later leaves from owner[i].
+// This is the data flow of the port-pruned reduce-scatter of an 8-rank ring (ReduceScatterRing::RunReduceScatterChunk,
+// reduce_scatter_ring.cc:299-477 with the send lists of ReduceScatterSlicesPrep, :458-477): with n ranks that own a
+// network port the 8 slices form n chunks of 8 / n, chunk j belongs to the j-th port rank, and every rank sends, in
+// the order of the ring distance to the port rank behind it, the chunks of the port ranks other than itself.  Hop h
+// of a slice's chain is phase h - 1 here, as in the plain ring; a rank combines its own copy (left operand) with
+// what its left neighbour sends.
+size_t OwnedRingReduceScatterPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t base, const std::vector<Slice> &sl,
+    const std::vector<uint32_t> &owner)
+{
+    for (uint32_t k = 0; k + 1 < p; k++) {
+        for (uint32_t i = 0; i < sl.size(); i++) {
+            uint32_t r = (owner[i] + 2 + k) % p, left = (owner[i] + 1 + k) % p;
+            Ref own = MkRef(r, BUF_SEND, base + sl[i].off);
+            EmitReduce(vp, phase0 + k, own, own, MkRef(left, BUF_SEND, base + sl[i].off), sl[i].size);
+        }
+    }
+    return phase0 + (p - 1);
+}
+
+size_t OwnedRingAllGatherPhases(VProgram &vp, size_t phase0, uint32_t p, uint64_t base, const std::vector<Slice> &sl,
+    const std::vector<uint32_t> &owner)
+{
+    for (uint32_t k = 0; k + 1 < p; k++) {
+        for (uint32_t i = 0; i < sl.size(); i++) {
+            uint32_t r = (owner[i] + 1 + k) % p, left = (owner[i] + k) % p;
+            EmitCopy(vp, phase0 + k, MkRef(r, BUF_RECV, base + sl[i].off), MkRef(left, BUF_RECV, base + sl[i].off), sl[i].size);
+        }
+    }
+    return phase0 + (p - 1);
+}
+
+// Port ranks of a mask in ascending order (the executor sorts its list, coll_comm_executor.cc:1768), and for every
+// slice of an 8-rank ring the rank its chain ends at.  Empty: no pruning.
+std::vector<uint32_t> PrunedRingOwners(uint32_t p, uint32_t nicMask)
+{
+    std::vector<uint32_t> nic, owner;
+    for (uint32_t r = 0; r < 8; r++) {
+        if ((nicMask >> r) & 1u) {
+            nic.push_back(r);
+        }
+    }
+    if (p != 8 || nic.empty() || nic.size() == 8) {
+        return owner;
+    }
+    const uint32_t chunk = 8 / uint32_t(nic.size());
+    for (uint32_t i = 0; i < 8; i++) {
+        owner.push_back(nic[i / chunk]);
+    }
+    return owner;
+}
+
 // Deterministic mesh reduce-scatter: every rank slice is cut into (p-1) pieces, piece t follows the
 // peer order rotated by t, so that in each round the pieces of one rank read p-1 different peers.
 // Atomic variant (reduce_scatter_mesh_atomic.cc:82-141): no piece cut; stream j of rank r pulls the
@@ -177,10 +230,24 @@ size_t HalvingSteps(VProgram &vp, size_t ph, uint32_t block, const std::vector<u
     return ph;
 }
 
-void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t bytes, uint64_t align, bool meshAtomic)
+void AllReduceChunk(VProgram &vp, Algo algo, uint32_t p, uint64_t base, uint64_t bytes, uint64_t align, bool meshAtomic,
+    uint32_t nicMask = 0)
 {
     if (p == 1) {
         EmitCopy(vp, 0, MkRef(0, BUF_RECV, base), MkRef(0, BUF_SEND, base), bytes);
+        return;
+    }
+    const std::vector<uint32_t> owner = algo == ALGO_RING ? PrunedRingOwners(p, nicMask) : std::vector<uint32_t>();
+    if (!owner.empty()) {
+        // Port-pruned ring: reduce-scatter on the input buffer with every chunk's chains ending at its port rank;
+        // the all-gather hands the finished slices round the ring from there (the reference tree holds no
+        // port-pruned form of the all-gather template; this one only moves bytes).
+        std::vector<Slice> sl = RingSlicePlan(bytes, p, align);
+        size_t ph = OwnedRingReduceScatterPhases(vp, 0, p, base, sl, owner);
+        for (uint32_t i = 0; i < p; i++) {
+            EmitCopy(vp, ph, MkRef(owner[i], BUF_RECV, base + sl[i].off), MkRef(owner[i], BUF_SEND, base + sl[i].off), sl[i].size);
+        }
+        OwnedRingAllGatherPhases(vp, ph + 1, p, base, sl, owner);
         return;
     }
     if (algo == ALGO_RING || algo == ALGO_MESH) {
@@ -1007,7 +1074,7 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             TwoLevelAllReduceChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, rq.level0Rings, done, bytes,
                 rq.align, rq.meshAtomic);
         } else if (rq.coll == COLL_ALLREDUCE) {
-            AllReduceChunk(*vp, rq.algo, p, done, bytes, rq.align, rq.meshAtomic);
+            AllReduceChunk(*vp, rq.algo, p, done, bytes, rq.align, rq.meshAtomic, rq.nicMask);
         } else if (rq.coll == COLL_REDUCESCATTER) {
             // input slice i of this chunk sits at i * total + done in the caller's layout
             std::vector<Slice> in(p), out(p);
@@ -1809,6 +1876,13 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
     if (request.p == 0 || request.unit == 0 || request.align == 0 || request.servers == 0 || request.p % request.servers != 0) {
         *err = "bad plan request";
         return 1;
+    }
+    if (request.nicMask != 0) {
+        const int ports = __builtin_popcount(request.nicMask & 0xffu);
+        if (request.p != 8 || (request.nicMask >> 8) != 0 || (ports != 1 && ports != 2 && ports != 4 && ports != 8)) {
+            *err = "bad plan request: network ports are given for a ring of 8 ranks, 1, 2, 4 or 8 of them";
+            return 1;
+        }
     }
     if (request.align % request.unit != 0) {
         // a slice boundary inside an element would make the kernels combine across element boundaries

@@ -91,6 +91,10 @@ struct PlanRequest {
                                    // (mesh inside a group, `algo` ring or halving-doubling between the groups)
     uint32_t level0Rings = 0;      // two-level all-reduce: 0 = mesh inside a group, 1 = one ring, 4 = the four rings of
                                    // the 8-device ring topology (groups of 8 ranks only), each on a quarter of every slice
+    uint32_t nicMask = 0;          // one-level ring all-reduce over 8 ranks: bit r set = rank r has a network port.  With 1, 2
+                                   // or 4 ports the reduce-scatter runs the port-pruned form (reduce_scatter_ring.cc:160-168,
+                                   // 299-477): the slices of chunk j all end their ring chain at the j-th port rank.  0 or all
+                                   // 8 bits: the plain ring
     bool meshAtomic = false;       // mesh reduce phases without the piece cut (the reference's non-deterministic variant)
     bool stageInput = false;       // copy the send buffers to scratch first (used when buffers overlap)
     // all-to-all-v only: p x p tables in elements, row r = what rank r passed

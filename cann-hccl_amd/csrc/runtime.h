@@ -38,6 +38,7 @@ struct GroupConfig {
     bool deterministic = false;
     uint32_t servers = 1;            // all-reduce: > 1 = two-level schedule over `servers` groups of consecutive ranks
     uint32_t level0Rings = 0;        // two-level all-reduce inside a group: 0 = mesh, 1 = one ring, 4 = four rings (groups of 8)
+    uint32_t nicMask = 0;            // 8-rank ring all-reduce: bit r = rank r has a network port (0: all have one)
     int stepStores = -1;             // step kernel stores: -1 chosen per launch, 0 non-temporal, 1 ordinary
     int fusedStores = -1;            // fused kernels' stores: 0 non-temporal, 1 ordinary, -1 chosen per collective (reductions: non-temporal)
     int stepSweep = 1;               // step kernel: 0 every phase walks its steps forwards, 1 every other phase backwards

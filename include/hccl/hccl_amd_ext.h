@@ -31,6 +31,11 @@ extern "C" {
  *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter / all-gather / reduce: the mesh schedule
  *                                (default), one ring in rank order, or -- for groups of 8 ranks, for the all-reduce also with one group --
  *                                the four rings of the 8-device ring topology, each on a quarter of every slice
+ *   "nic_ranks"     "all" | list of 1, 2 or 4 ranks, e.g. "0,4"   groups of 8 ranks only: the ranks that own a network port.
+ *                                With fewer than 8 the one-level ring all-reduce runs the port-pruned reduce-scatter of the
+ *                                reference (the 8 slices form as many chunks as there are ports; all slices of chunk j end
+ *                                their ring chain at the j-th listed rank, in ascending rank order), which changes the
+ *                                floating-point association of the slices whose chain ends elsewhere
  *   "step_stores"   "auto" | "nt" | "ordinary"   store kind of the step-by-step kernels (non-temporal, or write-back
  *                                so that the next phase finds the data in the memory-side cache); "auto" decides per collective
  *   "step_sweep"    "alternate" | "forward"   step-by-step kernels: every other launch walks its data backwards (default),
@@ -73,7 +78,8 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
  * bit 20 for the ring schedule instead of the mesh;
  * for the all-reduce (coll 0) bits 8..15 of algo
  * carry the number of rank groups of the two-level schedule (0 or 1: one level), bit 16 asks for its mesh level
- * without the piece cut and bits 17..19 give the rings inside a group (0: mesh, 1, or 4); the reduce-scatter (coll 1)
+ * without the piece cut, bits 17..19 give the rings inside a group (0: mesh, 1, or 4) and bits 20..27 the ranks of an
+ * 8-rank ring that own a network port (bit 20 + r for rank r; 0: all of them); the reduce-scatter (coll 1)
  * and the all-gather (coll 2) take bits 8..19 the same way; for the all-to-all-v (coll 3) bits 8..15 give the number
  * of servers of the staged schedule.  inPlaceMask bit r:
  * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64

@@ -11,7 +11,8 @@
 //   chunk loops      EXE/coll_all_reduce/coll_all_reduce_executor.cc:86-93,155-272,
 //                    EXE/coll_reduce_scatter/coll_reduce_scatter_executor.cc:83-90,118-245,
 //                    EXE/coll_all_gather/coll_all_gather_executor.cc:79-87,109-193
-//   ring             TPL/temp_reduce_scatter/reduce_scatter_ring.cc:89-297, TPL/temp_all_gather/all_gather_ring.cc:51-171,
+//   ring             TPL/temp_reduce_scatter/reduce_scatter_ring.cc:89-297 and, for an 8-rank ring with fewer network ports
+//                    than ranks, :160-168,299-477 (the port-pruned form); TPL/temp_all_gather/all_gather_ring.cc:51-171,
 //                    TPL/temp_all_reduce/all_reduce_ring.cc:32-53,143-191
 //   mesh             TPL/temp_reduce_scatter/reduce_scatter_mesh.cc:57-203, TPL/temp_all_gather/all_gather_mesh.cc:91-253,
 //                    EXE/coll_all_reduce/coll_all_reduce_mesh_executor.cc:95-240, EXE/coll_comm_executor.cc:1458-1574,
@@ -751,6 +752,120 @@ int RunAllReduceRing(Machine &m, uint64_t bytes, uint64_t align)
     return m.Run();
 }
 
+// Send lists of the port-pruned ring reduce-scatter, ReduceScatterRing::ReduceScatterSlicesPrep
+// (TPL/temp_reduce_scatter/reduce_scatter_ring.cc:458-477): rank r sends, for the ranks at ring distance 1, 2, ...
+// behind it that own a network port, the chunkSize slices of that port (chunk j = slices j * chunkSize ...).
+std::vector<std::vector<uint32_t>> PrunedRingSendLists(uint32_t p, const std::vector<uint32_t> &nic)
+{
+    const uint32_t chunk = 8 / static_cast<uint32_t>(nic.size());   // HCCL_NIC_MAX_NUM / nicSize
+    std::vector<std::vector<uint32_t>> lists;
+    for (uint32_t r = 0; r < p; r++) {
+        std::vector<uint32_t> one;
+        for (uint32_t dis = 1; dis < p; dis++) {
+            uint32_t at = (r + p - dis) % p;
+            auto it = std::find(nic.begin(), nic.end(), at);
+            if (it != nic.end()) {
+                uint32_t j = static_cast<uint32_t>(it - nic.begin());
+                for (uint32_t c = 0; c < chunk; c++) {
+                    one.push_back(chunk * j + c);
+                }
+            }
+        }
+        lists.push_back(one);
+    }
+    return lists;
+}
+
+// Per-rank program of ReduceScatterRing::RunReduceScatterChunk (reduce_scatter_ring.cc:299-333) with its parts
+// HeadReduceScatterChunk (:335-370), MidReduceScatterChunk (:372-411) and TailReduceScatterChunk (:413-442), taken
+// when 8 ranks share fewer than 8 network ports (:160-168).  A receive combines into the input buffer
+// (RunDestRducer, :76-87: destination = the rank's own input slice); empty slices are neither sent nor received.
+void ProgReduceScatterRingChunk(std::vector<Action> &pg, uint32_t r, uint32_t p, const std::vector<uint32_t> &nic,
+    const std::vector<std::vector<uint32_t>> &lists, int inB, const std::vector<Slice> &sl)
+{
+    const uint32_t left = (r + p - 1) % p, right = (r + 1) % p;
+    const std::vector<uint32_t> &mine = lists[r], &prev = lists[left];
+    const uint32_t chunk = 8 / static_cast<uint32_t>(nic.size());
+    auto inPrev = [&](uint32_t s) { return std::find(prev.begin(), prev.end(), s) != prev.end(); };
+    auto send = [&](uint32_t s) {
+        if (sl[s].size > 0) {
+            pg.push_back(MkSend(static_cast<int>(right), 0, inB, sl[s].off, sl[s].size));
+        }
+    };
+    auto recv = [&](uint32_t s) {
+        if (sl[s].size > 0) {
+            pg.push_back(MkRecvReduce(static_cast<int>(left), 0, inB, sl[s].off, inB, sl[s].off, sl[s].size));
+        }
+    };
+    auto mid = [&](uint32_t idx) {
+        const uint32_t rx = mine[idx + 1], tx = mine[idx];
+        send(tx);                       // both branches of :384-408 send; only one of them receives
+        if (inPrev(rx)) {
+            recv(rx);
+        }
+    };
+    const uint32_t len = static_cast<uint32_t>(mine.size());
+    if (len >= chunk && len >= 2) {
+        if (inPrev(mine[0])) {          // head, :345-356
+            recv(mine[0]);
+        }
+        if (inPrev(mine[1])) {          // :357-367
+            mid(0);
+        } else {
+            send(mine[0]);
+        }
+        for (uint32_t idx = 1; idx + 1 < len; idx++) {
+            mid(idx);
+        }
+    }
+    if (len > 0) {
+        send(mine[len - 1]);            // tail, :433-440
+    }
+    auto it = std::find(nic.begin(), nic.end(), r);
+    if (it != nic.end()) {              // a port rank ends the chains of its own chunk, :316-331
+        const uint32_t j = static_cast<uint32_t>(it - nic.begin());
+        for (uint32_t c = 0; c < chunk; c++) {
+            recv(j * chunk + c);
+        }
+    }
+}
+
+// All-reduce over an 8-rank ring whose network ports are fewer than its ranks: the port-pruned reduce-scatter on
+// the input buffer, then the finished slices go round the ring from the port ranks.  The reference tree has no
+// port-pruned all-gather template; this one is the reduce-scatter's mirror image and only moves bytes.
+int RunAllReduceRingPruned(Machine &m, uint64_t bytes, uint64_t align, const std::vector<uint32_t> &nic)
+{
+    const uint32_t p = static_cast<uint32_t>(m.p);
+    std::vector<Slice> sl = RingSlices(bytes, p, align);
+    std::vector<std::vector<uint32_t>> lists = PrunedRingSendLists(p, nic);
+    const uint32_t chunk = 8 / static_cast<uint32_t>(nic.size());
+    for (uint32_t r = 0; r < p; r++) {
+        Proc pr;
+        pr.rank = r;
+        ProgReduceScatterRingChunk(pr.prog, r, p, nic, lists, B_IN, sl);
+        const uint32_t left = (r + p - 1) % p, right = (r + 1) % p;
+        for (uint32_t i = 0; i < p; i++) {
+            if (nic[i / chunk] == r) {
+                pr.prog.push_back(MkLocalCopy(B_OUT, sl[i].off, B_IN, sl[i].off, sl[i].size));
+            }
+        }
+        for (uint32_t k = 0; k + 1 < p; k++) {
+            for (uint32_t i = 0; i < p; i++) {
+                if ((nic[i / chunk] + k) % p == r) {          // holds slice i after k hops
+                    pr.prog.push_back(MkSend(static_cast<int>(right), 1, B_OUT, sl[i].off, sl[i].size));
+                }
+            }
+            for (uint32_t i = 0; i < p; i++) {
+                if ((nic[i / chunk] + k) % p == left) {
+                    pr.prog.push_back(MkRecvCopy(static_cast<int>(left), 1, B_OUT, sl[i].off, sl[i].size));
+                }
+            }
+        }
+        m.procs.push_back(std::move(pr));
+    }
+    return m.Run();
+}
+
 // CollAllReduceMeshExecutor::KernelRun, deterministic branch (coll_all_reduce_mesh_executor.cc:95-240).
 int RunAllReduceMesh(Machine &m, uint64_t bytes, uint64_t align, bool atomic)
 {
@@ -1015,6 +1130,67 @@ int orc_allreduce(int algo, uint32_t p, void **in, void **out, uint64_t count, i
     }
     if (touched) {
         *touched = m.bytesTouched;
+    }
+    return 0;
+}
+
+// Ring all-reduce over 8 ranks of which only nic[0..nnic) (ascending, 1, 2 or 4 of them) own a network port: the
+// executor's chunk loop around RunAllReduceRingPruned.  Flags as for orc_allreduce.
+int orc_allreduce_ring_pruned(uint32_t p, void **in, void **out, uint64_t count, int dt, int op, const uint32_t *nic,
+    uint32_t nnic, uint64_t cclBytes, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p != 8 || cclBytes < unit || (nnic != 1 && nnic != 2 && nnic != 4)) {
+        return -20;
+    }
+    std::vector<uint32_t> ports(nic, nic + nnic);
+    for (uint32_t i = 0; i < nnic; i++) {
+        if (ports[i] >= p || (i > 0 && ports[i] <= ports[i - 1])) {
+            return -20;
+        }
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.op = op;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    bool zero = (flags & 2) != 0;
+    uint64_t maxPer = MaxCountPerLoop(0, cclBytes, p, unit, align);
+    uint64_t stage = std::min<uint64_t>(count, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn, cclOut;
+    if (!zero) {
+        cclIn.assign(p, std::vector<uint8_t>(stage));
+        cclOut.assign(p, std::vector<uint8_t>(stage));
+    }
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            if (zero) {
+                m.buf[B_IN][r] = static_cast<uint8_t *>(in[r]) + offset;
+                m.buf[B_OUT][r] = static_cast<uint8_t *>(out[r]) + offset;
+            } else {
+                m.buf[B_IN][r] = cclIn[r].data();
+                m.buf[B_OUT][r] = cclOut[r].data();
+                m.Copy(m.buf[B_IN][r], static_cast<uint8_t *>(in[r]) + offset, bytes);
+            }
+        }
+        int rc = RunAllReduceRingPruned(m, bytes, align, ports);
+        if (rc != 0) {
+            return rc;
+        }
+        if (!zero) {
+            for (uint32_t r = 0; r < p; r++) {
+                m.Copy(static_cast<uint8_t *>(out[r]) + offset, m.buf[B_OUT][r], bytes);
+            }
+        }
+        offset += bytes;
+        left -= cur;
     }
     return 0;
 }

@@ -74,6 +74,8 @@ def lib():
         L.orc_reduce_to_root_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_rhd.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
+        L.orc_allreduce_ring_pruned.argtypes = [u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, ctypes.POINTER(u32), u32,
+                                                u64, u64, i32, i32]
         L.orc_broadcast_two_level.argtypes = [u32, u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32, ctypes.POINTER(u64)]
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
         L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
@@ -188,6 +190,18 @@ def allreduce(ins, dt, op, algo=RING, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT
     if rc != 0:
         raise RuntimeError("oracle allreduce failed rc=%d" % rc)
     return (outs, touched.value) if return_touched else outs
+
+
+def allreduce_ring_pruned(ins, dt, op, nic_ranks, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1):
+    """Ring all-reduce over 8 ranks of which only nic_ranks (1, 2 or 4, ascending) own a network port."""
+    assert len(ins) == 8
+    outs = [np.empty_like(x) for x in ins]
+    nic = (ctypes.c_uint32 * len(nic_ranks))(*[int(x) for x in nic_ranks])
+    rc = lib().orc_allreduce_ring_pruned(8, _ptrs(ins), _ptrs(outs), ins[0].size, dt, op, nic, len(nic_ranks), ccl_bytes, align,
+                                         flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle port-pruned ring allreduce failed rc=%d" % rc)
+    return outs
 
 
 def allreduce_two_level(ins, dt, op, servers, level1=RING, atomic=False, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0,

@@ -243,6 +243,15 @@ def test_amd_params(comms):
     for key, values in good.items():
         for v in values:
             assert L.HcclAmdSetParam(comms[0], key, v) == 0, (key, v)
+    # network ports are named for groups of 8 ranks only (this group has 4)
+    assert L.HcclAmdSetParam(comms[0], b"nic_ranks", b"all") == 0
+    assert L.HcclAmdSetParam(comms[0], b"nic_ranks", b"0,2") == H.HCCL_E_PARA
+    eight = H.comm_init_all(8)
+    for v in (b"0", b"0,4", b"7,3", b"0,2,4,6", b"0,1,2,3,4,5,6,7", b"all", b""):
+        assert L.HcclAmdSetParam(eight[0], b"nic_ranks", v) == 0, v
+    for v in (b"0,1,2", b"8", b"0,0", b"x", b"0,,1", b"-1", b"0,1,2,3,4"):
+        assert L.HcclAmdSetParam(eight[0], b"nic_ranks", v) == H.HCCL_E_PARA, v
+    H.comm_destroy(eight)
     bad = {b"level0": b"star", b"step_stores": b"maybe", b"fused_stores": b"maybe", b"cache_entries": b"0", b"align": b"0",
            b"servers": b"0"}
     for key, v in bad.items():

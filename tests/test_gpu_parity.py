@@ -1280,6 +1280,50 @@ def test_collectives_recorded_into_a_callers_graph(orc):
             g.close()
 
 
+def test_ring_allreduce_with_fewer_network_ports_than_ranks(orc):
+    # 8-rank ring, group setting nic_ranks: the port-pruned reduce-scatter (reduce_scatter_ring.cc:160-168, 299-477).
+    # Fused and step by step against the checker, order-sensitive fp32 data (so that a plain ring would be caught),
+    # the hand-derived known answer, and back to the plain ring on the same buffers.
+    import json
+    import os
+    p = 8
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_ring_pruned_fp32.json")) as f:
+        kat = json.load(f)
+    for fuse in (1, 0):
+        g = gh.Group(p, fuse=fuse)
+        try:
+            for nic in ([0, 4], [3], [1, 2, 3, 7], [0, 2, 4, 6]):
+                g.set(nic_ranks=",".join(str(r) for r in nic))
+                for dt, op, n in ((FP32, SUM, 100003), (BF16, SUM, 40001), (INT32, MAX, 777), (FP32, SUM, 1 << 20)):
+                    ins = _ins(dt, p, n, 900 + n + len(nic))
+                    if dt == FP32:
+                        ins[0][:] *= 1e7
+                        ins[5][:] *= -1e7
+                    print("pruned ring all-reduce fuse", fuse, "ports", nic, "type", dt, "n", n, flush=True)
+                    want = orc.allreduce_ring_pruned([x.copy() for x in ins], dt, op, nic)
+                    outs, keep = gh.all_reduce(g, ins, dt, op)
+                    assert g.info()["fused"] == fuse
+                    for r in range(p):
+                        assert gh.same(dt, outs[r], want[r]), (fuse, nic, dt, n, r)
+                        assert np.array_equal(keep[r], ins[r])
+                    if dt == FP32 and n == 100003:
+                        plain = orc.allreduce(ins, dt, op)
+                        assert not np.array_equal(plain[0], want[0])        # the data does tell the two schedules apart
+            n = kat["elements"]
+            xs = [np.full(n, v, np.float32) for v in kat["inputs_per_rank"]]
+            for case in kat["cases"]:
+                g.set(nic_ranks=",".join(str(r) for r in case["nic_ranks"]))
+                outs, _ = gh.all_reduce(g, xs, FP32, SUM)
+                want = np.repeat(np.array(case["slice_values"], np.float32), n // 8)
+                assert all(np.array_equal(outs[r], want) for r in range(p)), (fuse, case["nic_ranks"])
+            g.set(nic_ranks="all")
+            outs, _ = gh.all_reduce(g, xs, FP32, SUM)
+            want = np.repeat(np.array(kat["plain_ring"]["slice_values"], np.float32), n // 8)
+            assert all(np.array_equal(outs[r], want) for r in range(p)), fuse
+        finally:
+            g.close()
+
+
 def test_two_hundred_buffer_sets(orc):
     # A caller that comes with other buffers every time: every call is a miss of the prepared-collective cache (the
     # plan itself is shared), tables travel with the call, no graph is built until a buffer set comes back, and a

@@ -732,3 +732,57 @@ def test_two_level_broadcast_plan(orc, servers, D):
                 (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, INT32, 0, in_place=True)
                 for r in range(p):
                     assert np.array_equal(recvs[r].view(np.int32), bufs[root]), (servers, D, root, ccl, fused, r)
+
+
+PRUNED_PORTS = ([0], [5], [0, 4], [2, 3], [1, 6], [0, 2, 4, 6], [1, 2, 3, 7], [4, 5, 6, 7])
+
+
+def _nic_bits(nic):
+    return sum(1 << (20 + r) for r in nic)
+
+
+def test_ring_pruned_allreduce_plan_matches_checker(orc):
+    # 8-rank ring with fewer network ports than ranks (reduce_scatter_ring.cc:160-168, 299-477): the plan, step by
+    # step and fused, against the checker's restatement of the template, out of place and in place
+    p = 8
+    for nic in PRUNED_PORTS:
+        for dt, op, n, ccl in ((FP32, SUM, 1000, 200 << 20), (FP32, SUM, 5000, 4096), (BF16, PROD, 777, 200 << 20), (INT8, MAX, 333, 200 << 20)):
+            unit = H.DTYPE_SIZE[dt]
+            ins = _ins(dt, p, n, len(nic) * 11 + op)
+            want = orc.allreduce_ring_pruned([x.copy() for x in ins], dt, op, nic, ccl_bytes=ccl)
+            for mask in (0, (1 << p) - 1):
+                plan = H.describe_plan(H.COLL_ALLREDUCE, RING | _nic_bits(nic), p, n, dt, ccl_bytes=ccl, in_place_mask=mask)
+                assert plan["scratchBytes"] == 0 and plan["fusedOk"]
+                assert len(plan["phases"]) == 14 or ccl < n * unit           # 7 reduce hops, 7 copy hops, as the plain ring
+                for fused in (False, True):
+                    sends = _bytes(ins)
+                    recvs = _bytes(ins) if mask else [np.full(n * unit, 0xA5, np.uint8) for _ in range(p)]
+                    (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op, in_place=bool(mask))
+                    for r in range(p):
+                        assert _same(dt, recvs[r], want[r]), (nic, dt, op, ccl, mask, fused, r)
+    # all eight ports, or none named: the plain ring
+    plain = H.describe_plan(H.COLL_ALLREDUCE, RING, p, 1000, FP32)
+    assert H.describe_plan(H.COLL_ALLREDUCE, RING | _nic_bits(range(8)), p, 1000, FP32) == plain
+    # 3 ports do not divide 8 slices; ports on a ring that is not 8 ranks make no sense
+    for bad_p, nic in ((8, [0, 1, 2]), (8, [0, 1, 2, 3, 4]), (6, [0, 3]), (16, [0, 4])):
+        with pytest.raises(H.HcclError):
+            H.describe_plan(H.COLL_ALLREDUCE, RING | _nic_bits(nic), bad_p, 1000, FP32)
+
+
+def test_ring_pruned_known_answers_through_the_planner():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_ring_pruned_fp32.json")) as f:
+        kat = json.load(f)
+    n = kat["elements"]
+    xs = [np.full(n, v, np.float32) for v in kat["inputs_per_rank"]]
+    per = n // 8
+    for case in kat["cases"] + [dict(kat["plain_ring"], nic_ranks=[])]:
+        want = np.repeat(np.array(case["slice_values"], np.float32), per)
+        plan = H.describe_plan(H.COLL_ALLREDUCE, RING | _nic_bits(case["nic_ranks"]), 8, n, FP32)
+        for fused in (False, True):
+            sends = _bytes(xs)
+            recvs = [np.full(n * 4, 0xA5, np.uint8) for _ in range(8)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, FP32, SUM)
+            for r in range(8):
+                assert np.array_equal(recvs[r].view(np.float32), want), (case["nic_ranks"], fused, r)
