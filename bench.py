@@ -210,6 +210,37 @@ def run_suite(pkg, torch, steps, warmup, only="", settings=()):
     del sends, recvs
     pkg.comm_destroy(comms)
 
+    # the same with segments below a KiB: counts lognormal(ln 64, 1) elements, ragged displacements
+    for p in (16, 64):
+        rng = np.random.default_rng(2025 + p)
+        cnt = np.clip(np.rint(np.exp(np.log(64.0) + rng.standard_normal((p, p)))), 0, 4 << 20).astype(np.uint64)
+        sdis, rdis = np.zeros((p, p), np.uint64), np.zeros((p, p), np.uint64)
+        sl, rl = [], []
+        for r in range(p):
+            pos = 0
+            for j in rng.permutation(p):
+                pos += int(rng.integers(0, 16))
+                sdis[r, j] = pos
+                pos += int(cnt[r, j])
+            sl.append(pos)
+            pos = 0
+            for i in rng.permutation(p):
+                pos += int(rng.integers(0, 16))
+                rdis[r, i] = pos
+                pos += int(cnt[i, r])
+            rl.append(pos)
+        comms = pkg.comm_init_all(p)
+        sends = [rand(max(x, 1), torch.int32) for x in sl]
+        recvs = [torch.empty(max(x, 1), dtype=torch.int32, device="cuda") for x in rl]
+        sp, rp = [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs]
+        torch.cuda.synchronize()
+        tables = pkg.a2av_tables(cnt, sdis, cnt.T.copy(), rdis)
+        report("all-to-all-v pairwise p=%d int32 small segments (%.0f KB)" % (p, 4 * cnt.sum() / 1e3), comms,
+               lambda: pkg.all_to_all_v(comms, sp, None, None, rp, None, None, pkg.HCCL_DATA_TYPE_INT32, stream.cuda_stream,
+                                        tables=tables))
+        del sends, recvs
+        pkg.comm_destroy(comms)
+
     # halving-doubling all-reduce, bf16, 128 MiB per rank, 32 and 24 ranks
     for p in (32, 24):
         comms = pkg.comm_init_all(p)

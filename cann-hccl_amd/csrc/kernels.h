@@ -59,7 +59,17 @@ constexpr uint32_t kFusedOrdinaryStores = 1u;  // whole passes of the chain kern
 constexpr uint32_t kStepOrdinaryStores = 1u;   // write-back stores instead of non-temporal ones in the fast loop
 constexpr uint32_t kStepReverse = 2u;          // the fast loop walks every step from its last tile to its first
 
-enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_STACK = 3, KK_COUNT = 4 };
+// Small-segment gather (pure data movement, one source and one destination per segment, any byte alignment of
+// either): one wave moves one segment through its share of the workgroup's LDS.
+struct SegDesc {
+    const void *src;
+    void *dst;
+    uint64_t bytes;     // <= kGatherMaxBytes
+    uint64_t pad;
+};
+constexpr uint32_t kGatherMaxBytes = 8192;
+
+enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_STACK = 3, KK_COUNT = 4, KK_GATHER = 4 };
 
 // Kernel entry for (data type, reduce op, kind); nullptr if the combination is not built.
 // Signatures:
@@ -70,7 +80,9 @@ enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_STACK = 3, KK
 //                       const void *const *srcPool, void *const *dstPool)
 const void *LookupKernel(int hcclDataType, int hcclReduceOp, KernelKind kind);
 
-// Byte-wise variants for pure data movement (all-gather, all-to-all-v): KK_STEP and KK_CHAIN only.
+//   KK_GATHER          (const SegDesc *segs, uint32_t nsegs, uint32_t unused, const void *unused, void *unused)
+//                      copy kernel table only
+// Byte-wise variants for pure data movement (all-gather, all-to-all-v): KK_STEP, KK_CHAIN and KK_GATHER.
 const void *LookupCopyKernel(KernelKind kind);
 
 }  // namespace hcclamd

@@ -52,9 +52,10 @@ using DT = uint8_t;
 
 #if HCCL_DT == 255
 // pure data movement: the step kernel's copy path and the copy kernel
-extern const void *const HCCL_CAT(kKernels_, HCCL_DT_NAME)[2] = {
+extern const void *const HCCL_CAT(kKernels_, HCCL_DT_NAME)[3] = {
     reinterpret_cast<const void *>(&StepKernel<DT, ROP_SUM>),
     reinterpret_cast<const void *>(&CopyKernel<0>),
+    reinterpret_cast<const void *>(&GatherKernel<0>),
 };
 #else
 #define HCCL_ROW(OP)                                                     \

@@ -715,6 +715,68 @@ __global__ void __launch_bounds__(kBlockThreads) CopyKernel(const FusedDesc *__r
     }
 }
 
+// ---- small-segment gather: LDS staging ---------------------------------------------------------------------
+// An all-to-all-v of many short segments (a few hundred bytes each, at any byte offset in the send and receive
+// buffers) is all overhead in the tile kernels: a descriptor search per tile, a head / body / tail split per
+// segment, unaligned accesses.  Here a wave takes a whole segment: it reads the aligned 16-byte granules that cover
+// the source bytes into its share of LDS (coalesced, aligned loads; the bytes in front of and behind the segment that
+// come along lie in the same granules as valid bytes), then every lane picks the 16 bytes of one aligned granule of
+// the destination out of LDS at whatever offset they sit and stores them aligned; the two ragged ends go byte by
+// byte.  Segments are dealt to waves round robin, no search.
+// Stands where the reference's AIV kernel stages small all-to-all-v slices through its unified buffer
+// (ALG/base/alg_aiv_template/aiv_all_to_all_v_910b.h:39-222); nothing of it is reused.
+constexpr uint32_t kGatherLdsPerWave = kGatherMaxBytes + 32;
+typedef V4 __attribute__((address_space(3))) LdsV4;
+typedef V4U __attribute__((address_space(3))) LdsV4U;
+
+template <int Variant>
+__global__ void __launch_bounds__(kBlockThreads) GatherKernel(const SegDesc *__restrict__ segs, uint32_t nsegs, uint32_t,
+    const void *const *__restrict__, void *const *__restrict__)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[(kBlockThreads / 64) * kGatherLdsPerWave];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint8_t *mine = lds + wave * kGatherLdsPerWave;
+    const uint32_t wavesPerBlock = kBlockThreads / 64;
+    for (uint32_t i = blockIdx.x * wavesPerBlock + wave; i < nsegs; i += gridDim.x * wavesPerBlock) {
+        const SegDesc d = segs[i];
+        const uint32_t n = uint32_t(d.bytes);
+        if (n == 0) {
+            continue;
+        }
+        const uintptr_t s = reinterpret_cast<uintptr_t>(d.src), t = reinterpret_cast<uintptr_t>(d.dst);
+        const uintptr_t s0 = s & ~uintptr_t(15);
+        const uint32_t delta = uint32_t(s - s0);                       // where the segment starts inside LDS
+        const uint32_t nin = (delta + n + 15u) >> 4;                   // granules to read
+        for (uint32_t v = lane; v < nin; v += 64) {
+            const V4 x = __builtin_nontemporal_load((const GlobalV4 *)(s0 + uintptr_t(v) * 16));
+            *(LdsV4 *)(mine + v * 16) = x;
+        }
+        // LDS operations of one wave complete in order; the compiler must keep that order too
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uintptr_t t0 = (t + 15) & ~uintptr_t(15);               // first aligned granule inside the destination
+        const uint32_t head = uint32_t(t0 - t) < n ? uint32_t(t0 - t) : n;
+        const uint32_t body = (n - head) >> 4;                         // whole granules
+        const uint32_t tail = n - head - body * 16;
+        for (uint32_t v = lane; v < body; v += 64) {
+            const LdsV4U *from = (const LdsV4U *)(mine + delta + head + v * 16);
+            const V4U x = *from;
+            __builtin_nontemporal_store(V4{x.x, x.y, x.z, x.w}, (GlobalV4 *)(t0 + uintptr_t(v) * 16));
+        }
+        if (lane < head) {
+            StoreElem<uint8_t>(d.dst, lane, mine[delta + lane]);
+        }
+        if (lane < tail) {
+            const uint32_t at = head + body * 16 + lane;
+            StoreElem<uint8_t>(d.dst, at, mine[delta + at]);
+        }
+        // the next segment's loads into LDS must not overtake this segment's reads
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 // ---- fused perfect tree (halving-doubling): leaves pairwise bottom-up ----------------------------------
 // v[i] = v[i] (+) v[i+w] for w = 1, 2, 4, ... is evaluated group by group: the first three levels
 // inside groups of 8 consecutive leaves (8 loads per vector in flight, one result kept per group), the

@@ -255,6 +255,51 @@ def test_alltoallv_small_ragged(orc):
                 g.close()
 
 
+def test_alltoallv_sub_kib_segments_go_through_the_gather_kernel(orc):
+    # many short segments at every byte alignment: int8 payload (so displacements are byte offsets), counts lognormal
+    # around 64 elements, and int32 / int64 for the element-aligned case; segments up to and just beyond the gather
+    # kernel's limit of 8 KiB; the bytes around every segment must stay untouched
+    for p, dt, scale in ((16, INT8, 64), (64, INT8, 200), (16, INT32, 64), (33, INT64, 30), (16, INT8, 6000)):
+        unit = H.DTYPE_SIZE[dt]
+        rng = np.random.default_rng(7000 + p + dt)
+        cnt = np.clip(np.rint(np.exp(np.log(float(scale)) + rng.standard_normal((p, p)))), 0, 20000).astype(np.uint64)
+        cnt[rng.random((p, p)) < 0.1] = 0
+        if scale >= 6000:
+            cnt[0, 1], cnt[2, 3], cnt[4, 4] = 8192, 8193, 8191          # at, above and below the limit (bytes, int8)
+        sdis, rdis = np.zeros((p, p), np.uint64), np.zeros((p, p), np.uint64)
+        sl, rl = [], []
+        for r in range(p):
+            pos = int(rng.integers(0, 16))
+            for j in rng.permutation(p):
+                pos += int(rng.integers(0, 23))
+                sdis[r, j] = pos
+                pos += int(cnt[r, j])
+            sl.append(pos + 19)
+            pos = int(rng.integers(0, 16))
+            for i in rng.permutation(p):
+                pos += int(rng.integers(0, 23))
+                rdis[r, i] = pos
+                pos += int(cnt[i, r])
+            rl.append(pos + 19)
+        sends = [cf.random_input(dt, n, rng) for n in sl]
+        fill = np.array([-1], np.int64).astype(cf.CARRIER[dt])[0]
+        want = [np.full(n, fill, cf.CARRIER[dt]) for n in rl]
+        assert orc.alltoallv(sends, cnt, sdis, want, cnt.T.copy(), rdis, dt) == 0
+        for fuse in (1, 0):
+            g = gh.Group(p, fuse=fuse)
+            try:
+                print("alltoallv short segments p", p, "type", dt, "scale", scale, "fuse", fuse, flush=True)
+                outs = gh.all_to_all_v(g, sends, cnt, sdis, rl, cnt.T.copy(), rdis, dt)
+                for r in range(p):
+                    assert np.array_equal(outs[r], want[r]), (p, dt, scale, fuse, r)
+                info = g.info()
+                if fuse:
+                    assert info["fused"] == 1 and info["launches"] == 1      # pieces of up to 64 KiB ride along
+                assert unit == H.DTYPE_SIZE[dt]
+            finally:
+                g.close()
+
+
 def test_alltoallv_16_ranks_lognormal(orc):
     # 16 ranks, per-pair counts lognormal(ln 64K, 1) clamped to [0, 4M] int32 elements, shuffled displacements with gaps
     p = 16
