@@ -317,9 +317,25 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
     g->pend.recv[r] = recv;
     g->pend.streams[r] = stream;
     g->pend.recorded[r] = 0;
-    if (g->cfg.blockingArrive && g->deviceReady && g->arrived + 1 < g->p) {
-        // This rank is going to wait inside its call: it marks its stream now, on its own thread, so that
-        // the rank that issues the collective only has to make its stream wait for the markers.
+    // A rank marks its stream when it arrives, so that the rank that issues the collective orders it behind exactly
+    // what this stream held at the time of the call: always when the rank is going to wait inside its call (it is on
+    // its own thread), otherwise when the ranks are on different streams (ranks that share one stream need no
+    // marker, and the common single-stream caller pays nothing).  Not under capture: the marker would become part of
+    // the caller's graph for no use.
+    bool mark = g->deviceReady && g->arrived + 1 < g->p && g->cfg.blockingArrive;
+    if (!mark && g->deviceReady && g->arrived + 1 < g->p && g->arrived > 0) {
+        for (uint32_t q = 0; q < g->p && !mark; q++) {
+            mark = g->here[q] && q != r && g->pend.streams[q] != stream;
+        }
+        if (mark) {
+            hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) {
+                (void)hipGetLastError();
+                mark = false;
+            }
+        }
+    }
+    if (mark) {
         if (hipEventRecord(g->arriveEvents[r], stream) == hipSuccess) {
             g->pend.recorded[r] = 1;
         } else {
@@ -419,6 +435,9 @@ HcclResult PointToPoint(Comm *c, bool isSend, void *buf, uint64_t count, HcclDat
     queue.pop_front();
     if (match.count != count || match.dtype != int(dataType)) {
         HCCL_LOG_ERROR("send / receive between rank %u and rank %u disagree on count or type", src, dst);
+        // the call that came first has returned already: its caller learns of the failure through
+        // HcclGetCommAsyncError
+        g->asyncError = HCCL_E_PARA;
         return HCCL_E_PARA;
     }
     OpCtx ctx;
@@ -433,10 +452,32 @@ HcclResult PointToPoint(Comm *c, bool isSend, void *buf, uint64_t count, HcclDat
     ctx.streams.assign(g->p, stream);
     ctx.send[src] = isSend ? buf : match.buf;
     ctx.recv[dst] = isSend ? match.buf : buf;
-    ctx.streams[other] = match.stream;
+    const bool toSelf = other == c->rank;
+    if (!toSelf) {
+        ctx.streams[other] = match.stream;
+    }
+    HcclResult res = HCCL_SUCCESS;
+    if (toSelf && match.stream != stream) {
+        // A rank sending to itself on two streams: the copy runs on this call's stream, after what the earlier
+        // call's stream holds so far, and that stream goes on after the copy.
+        res = EnsureDevice(g, false);
+        if (res == HCCL_SUCCESS && (hipEventRecord(g->arriveEvents[c->rank], match.stream) != hipSuccess ||
+            hipStreamWaitEvent(stream, g->arriveEvents[c->rank], 0) != hipSuccess)) {
+            (void)hipGetLastError();
+            res = HCCL_E_RUNTIME;
+        }
+    }
     g->ctx = &ctx;
-    HcclResult res = IssueCollective(g, c->rank);
+    if (res == HCCL_SUCCESS) {
+        res = IssueCollective(g, c->rank);
+    }
     g->ctx = &g->pend;
+    if (res == HCCL_SUCCESS && toSelf && match.stream != stream) {
+        if (hipEventRecord(g->doneEvent, stream) != hipSuccess || hipStreamWaitEvent(match.stream, g->doneEvent, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            res = HCCL_E_RUNTIME;
+        }
+    }
     if (res != HCCL_SUCCESS && res != HCCL_E_PARA) {
         g->asyncError = res;
     }

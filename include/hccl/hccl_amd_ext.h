@@ -47,7 +47,13 @@ extern "C" {
  *   "cache_entries" how many prepared collectives (distinct sizes, buffers, settings) the group keeps (default 1024);
  *                   when full, the library waits for the device once and starts over
  *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
- *   "blocking_arrive" "0" | "1"  a rank's call waits inside the library until the group is complete
+ *   "blocking_arrive" "0" | "1"  a rank's call waits inside the library until the group is complete.  With "0" (default)
+ *                                a call returns at once and the last rank's call issues the collective; what a rank's
+ *                                stream held when the rank called runs before the collective, but work queued on that
+ *                                stream between the rank's call and the last rank's call is NOT ordered after the
+ *                                collective (it may read a receive buffer that is not written yet): a caller that drives
+ *                                all ranks from one thread queues such work after the last rank's call, or uses one thread
+ *                                per rank with "1", which gives every rank the reference's per-stream semantics
  *   "arrive_timeout_ms"          limit of that wait (HCCL_E_TIMEOUT)
  * Unknown key or bad value: HCCL_E_PARA. */
 extern HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value);

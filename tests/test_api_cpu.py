@@ -281,8 +281,12 @@ def test_send_recv_checks_and_matching(comms):
     assert L.HcclRecv(None, 4, FP32, 1, comms[0], STREAM) == H.HCCL_E_PTR
     assert L.HcclBatchSendRecv(None, 1, comms[0], STREAM) == H.HCCL_E_PTR
     # a send waits for its receive; a receive that disagrees on the count is refused
+    err = ctypes.c_int32(-1)
+    assert L.HcclGetCommAsyncError(comms[0], ctypes.byref(err)) == 0 and err.value == H.HCCL_SUCCESS
     assert L.HcclSend(BUF_A, 4, FP32, 1, comms[0], STREAM) == H.HCCL_SUCCESS
     assert L.HcclRecv(BUF_B, 8, FP32, 0, comms[1], STREAM) == H.HCCL_E_PARA
+    # the send returned success before its receive turned up: the sender learns of the failure here
+    assert L.HcclGetCommAsyncError(comms[0], ctypes.byref(err)) == 0 and err.value == H.HCCL_E_PARA
 
 
 def test_rooted_entry_checks(comms):

@@ -1554,6 +1554,19 @@ def test_send_recv_and_batch():
         torch.cuda.synchronize()
         for r in range(p):
             assert np.array_equal(gh.to_host(dst[r], INT32), data[(r + 1) % p]), r
+        # a rank sending to itself, the send on one stream and the receive on another: the copy comes after what the
+        # first stream held (the fill of the source) and before what the first stream does next (its overwrite)
+        big = torch.zeros(8 << 20, dtype=torch.int32, device="cuda")
+        out = torch.zeros_like(big)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(streams[0]):
+            big.fill_(41)
+            H.send(g.comms[2], big.data_ptr(), big.numel(), INT32, 2, streams[0].cuda_stream)
+        H.recv(g.comms[2], out.data_ptr(), big.numel(), INT32, 2, streams[1].cuda_stream)
+        with torch.cuda.stream(streams[0]):
+            big.fill_(7)
+        torch.cuda.synchronize()
+        assert bool((out == 41).all()) and bool((big == 7).all())
     finally:
         g.close()
 
