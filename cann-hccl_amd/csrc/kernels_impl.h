@@ -223,6 +223,26 @@ template <int OP> __device__ __forceinline__ uint32_t PkBf16(uint32_t a, uint32_
     }
 }
 
+// fp16, two elements per word: widen both to fp32, combine, round to nearest even (the hardware conversions);
+// max / min compare the halves as they are (the conversion to fp32 is exact and keeps the order) and keep the chosen
+// operand's bits.
+typedef _Float16 H2 __attribute__((ext_vector_type(2)));
+template <int OP> __device__ __forceinline__ uint32_t PkF16(uint32_t a, uint32_t b)
+{
+    const H2 x = BitCast<H2>(a), y = BitCast<H2>(b);
+    if (OP == ROP_SUM || OP == ROP_PROD) {
+        const F2 fx = __builtin_convertvector(x, F2), fy = __builtin_convertvector(y, F2);
+        F2 r;
+        r.x = (OP == ROP_SUM) ? fx.x + fy.x : fx.x * fy.x;
+        r.y = (OP == ROP_SUM) ? fx.y + fy.y : fx.y * fy.y;
+        return BitCast<uint32_t>(__builtin_convertvector(r, H2));
+    } else {
+        const bool pickLo = (OP == ROP_MAX) ? (y.x > x.x) : (y.x < x.x);
+        const bool pickHi = (OP == ROP_MAX) ? (y.y > x.y) : (y.y < x.y);
+        return ((pickHi ? b : a) & 0xffff0000u) | ((pickLo ? b : a) & 0x0000ffffu);
+    }
+}
+
 #define HCCL_WORDWISE_COMBINER(TYPE, EXPR)                                  \
     template <int OP> struct Combiner<TYPE, OP> {                           \
         static __device__ __forceinline__ V4 Apply(V4 a, V4 b)              \
@@ -240,11 +260,13 @@ template <int OP> __device__ __forceinline__ uint32_t PkBf16(uint32_t a, uint32_
 #define HCCL_EXPR_I8(x, y) Pk8<true, OP>(x, y)
 #define HCCL_EXPR_U8(x, y) Pk8<false, OP>(x, y)
 #define HCCL_EXPR_BF16(x, y) PkBf16<OP>(x, y)
+#define HCCL_EXPR_F16(x, y) PkF16<OP>(x, y)
 HCCL_WORDWISE_COMBINER(int16_t, HCCL_EXPR_I16)
 HCCL_WORDWISE_COMBINER(uint16_t, HCCL_EXPR_U16)
 HCCL_WORDWISE_COMBINER(int8_t, HCCL_EXPR_I8)
 HCCL_WORDWISE_COMBINER(uint8_t, HCCL_EXPR_U8)
 HCCL_WORDWISE_COMBINER(Bf16Bits, HCCL_EXPR_BF16)
+HCCL_WORDWISE_COMBINER(HalfBits, HCCL_EXPR_F16)
 
 template <typename T, int OP> __device__ __forceinline__ V4 Combine16(V4 a, V4 b) { return Combiner<T, OP>::Apply(a, b); }
 
