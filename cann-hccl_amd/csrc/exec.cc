@@ -755,6 +755,11 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAl
         // the groups, mesh all-gather in every group; the flat ring when the ring is asked for by name
         rq.servers = g->cfg.servers;
     }
+    if (rq.coll == COLL_SCATTER && g->cfg.servers > 1 && g->p % g->cfg.servers == 0 && rq.algo != ALGO_RING) {
+        // two levels (coll_scatter_mesh_executor.cc:40-110): ring scatter of the groups' runs between the sub-roots,
+        // mesh scatter inside every group; the flat ring when the ring is asked for by name
+        rq.servers = g->cfg.servers;
+    }
     if (rq.coll == COLL_REDUCE && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
         // two levels (coll_reduce_mesh_executor.cc:75-194, coll_reduce_ring_plus_hd_executor.cc:75-168): inside the
         // groups the mesh (uncut under the conditions of :93-97) or the ring(s), then ring or halving-doubling

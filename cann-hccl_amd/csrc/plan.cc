@@ -866,6 +866,33 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             }
             return 0;
         }
+        if (rq.coll == COLL_SCATTER && rq.servers > 1) {
+            // Two levels (coll_scatter_mesh_executor.cc:40-110): S groups of D consecutive ranks.  The rank at the
+            // root's position in a group is the group's sub-root (topo_matcher.cc:341-370).  Level 1
+            // (coll_scatter_executor.cc:198-241, the ring choice): a group's run of D blocks travels round the ring of
+            // sub-roots from the root, the farthest group's first, each run at its own offset of the sub-roots'
+            // workspace.  Level 0 (scatter_mesh.cc:46-160): every sub-root hands the ranks of its group their blocks.
+            // The reference lands a block in the receiver's staging buffer and copies it out (:103-106); here the
+            // hand-over writes the receive buffer itself.
+            const uint32_t S = rq.servers, D = p / S, rootGroup = R / D, rootLocal = R % D;
+            const uint64_t run = total * D;
+            vp->workBytes.assign(p, 0);
+            vp->inBytes[R] = total * p;
+            for (uint32_t j = 1; j < S; j++) {            // j = hops from the root's group to the run's group
+                const uint32_t dest = (rootGroup + j) % S;
+                for (uint32_t h = 1; h <= j; h++) {
+                    const uint32_t from = ((rootGroup + h - 1) % S) * D + rootLocal, to = ((rootGroup + h) % S) * D + rootLocal;
+                    EmitCopy(*vp, size_t(S - j + h - 2), MkRef(to, BUF_SEND, uint64_t(dest) * run),
+                        MkRef(from, BUF_SEND, uint64_t(dest) * run), run);
+                    vp->workBytes[to] = std::max(vp->workBytes[to], uint64_t(dest + 1) * run);
+                }
+            }
+            for (uint32_t r = 0; r < p; r++) {
+                EmitCopy(*vp, size_t(S - 1), MkRef(r, BUF_RECV, 0), MkRef(r / D * D + rootLocal, BUF_SEND, uint64_t(r) * total), total);
+                vp->outBytes[r] = total;
+            }
+            return 0;
+        }
         if (rq.coll == COLL_SCATTER) {
             // mesh scatter (scatter_mesh.cc:46-160): the root hands rank i block i, all at once
             for (uint32_t r = 0; r < p; r++) {

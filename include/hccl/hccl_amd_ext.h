@@ -26,6 +26,8 @@ extern "C" {
  *                   consecutive ranks and the two-level schedules run (mesh inside a group, "algo" ring or rhd between;
  *                   with "auto": rhd for 2, 4, 8 or more groups, ring for 3, 5, 6, 7, the reference's default);
  *                   the broadcast then runs scatter / halving-doubling between the groups / all-gather unless "algo" is "ring";
+ *                   the scatter then sends a group's blocks round the ring of the ranks at the root's position and hands them out
+ *                   inside the group, unless "algo" is "ring";
  *                   the all-to-all family then runs the staged schedule (gather inside a group into a workspace, pairwise
  *                   between the groups) unless "algo" is "pairwise"
  *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter / all-gather / reduce: the mesh schedule
@@ -81,7 +83,7 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
  * schedule in bits 16..19 (0 ring, 1 mesh, 2 rhd, 4 mesh without the piece cut), for the reduce also the number of rank
  * groups of its two-level schedule in bits 20..27, bit 28 for the mesh level without the piece cut and bit 29 / bit 30 for
  * one ring / four rings inside a group, for the broadcast the number of rank groups in bits 20..27, for the scatter
- * bit 20 for the ring schedule instead of the mesh;
+ * bit 20 for the ring schedule instead of the mesh and the number of rank groups of the two-level mesh schedule in bits 21..28;
  * for the all-reduce (coll 0) bits 8..15 of algo
  * carry the number of rank groups of the two-level schedule (0 or 1: one level), bit 16 asks for its mesh level
  * without the piece cut, bits 17..19 give the rings inside a group (0: mesh, 1, or 4) and bits 20..27 the ranks of an

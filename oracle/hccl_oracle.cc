@@ -2908,6 +2908,130 @@ int orc_scatter_ring(uint32_t p, const void *inRoot, void **out, uint64_t count,
     return 0;
 }
 
+// Two-level scatter, CollScatterMeshExecutor::KernelRun with several servers
+// (EXE/coll_scatter/coll_scatter_mesh_executor.cc:40-110) under the chunk loop of CollScatterExecutor::RunLoop /
+// RunLoopInner (coll_scatter_executor.cc:54-175); `servers` groups of D = p / servers consecutive ranks.
+// Per chunk of `cur` elements the root packs the p blocks' parts into its staging buffer (:137-145, source stride =
+// the whole block, destination stride = the chunk).  Step 1 (KernelRunLevel1, :198-241, the ring choice of :226-229):
+// the ranks at the root's position in every group -- each its group's sub-root (topo_matcher.cc:341-370) -- run
+// the ring scatter from the root over `servers` runs of D blocks, in place in their staging buffers.  Step 2
+// (:72-101): mesh scatter inside every group from the sub-root over the group's run (scatter_mesh.cc:46-160, base
+// offset = the run's), again in place in the staging buffers; then every rank copies its block out (:103-106).
+// `touched` (optional) receives the bytes read + written by all ranks.
+int orc_scatter_two_level(uint32_t servers, uint32_t p, const void *inRoot, void **out, uint64_t count, int dt,
+    uint32_t root, uint64_t cclBytes, uint64_t align, int flags, int threads, uint64_t *touched)
+{
+    const uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p || servers == 0 || p % servers != 0 || align == 0) {
+        return -20;
+    }
+    const uint64_t maxPer = cclBytes / p / align * align / unit;
+    if (maxPer == 0 && count > 0) {
+        return -21;
+    }
+    const uint32_t D = p / servers, rootGroup = root / D, rootLocal = root % D;
+    const uint64_t total = count * unit;
+    uint64_t moved = 0;
+    Pool pool(threads);
+    auto machine = [&](uint32_t n) {
+        Machine m;
+        m.p = static_cast<int>(n);
+        m.dt = dt;
+        m.direct = (flags & 1) != 0;
+        m.pool = &pool;
+        m.buf[B_IN].resize(n);
+        m.buf[B_OUT].resize(n);
+        return m;
+    };
+    std::vector<std::vector<uint8_t>> stage(p);
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0;) {
+        const uint64_t cur = left * unit * p > cclBytes ? maxPer : left;
+        const uint64_t cb = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            stage[r].assign(cb * p + 1, 0);
+        }
+        {
+            Machine m = machine(1);
+            for (uint32_t i = 0; i < p; i++) {
+                m.Copy(stage[root].data() + cb * i, static_cast<const uint8_t *>(inRoot) + total * i + offset, cb);
+                moved += 2 * cb;
+            }
+        }
+        if (servers > 1) {                             // step 1: runs of D blocks round the ring of sub-roots
+            const uint64_t run = cb * D;
+            Machine m = machine(servers);
+            for (uint32_t g = 0; g < servers; g++) {
+                m.buf[B_IN][g] = m.buf[B_OUT][g] = stage[g * D + rootLocal].data();
+            }
+            for (uint32_t g = 0; g < servers; g++) {
+                Proc pr;
+                pr.rank = g;
+                const int lft = static_cast<int>((g + servers - 1) % servers), rgt = static_cast<int>((g + 1) % servers);
+                if (g == rootGroup) {
+                    for (uint32_t i = 1; i < servers; i++) {
+                        const uint32_t owner = (g + servers - i) % servers;
+                        pr.prog.push_back(MkSend(rgt, 0, B_IN, run * owner, run));
+                    }
+                } else {
+                    const uint32_t rounds = (rootGroup + servers - g) % servers;
+                    for (uint32_t i = 1; i <= rounds; i++) {
+                        const uint32_t owner = (g + rounds - i) % servers;
+                        if (i != 1) {
+                            pr.prog.push_back(MkSend(rgt, 0, B_OUT, run * ((g + rounds - i + 1) % servers), run));
+                        }
+                        pr.prog.push_back(MkRecvCopy(lft, 0, B_OUT, run * owner, run));
+                    }
+                }
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+            moved += m.bytesTouched;
+        }
+        for (uint32_t g = 0; g < servers && D > 1; g++) {      // step 2: inside every group, from the sub-root
+            Machine m = machine(D);
+            for (uint32_t d = 0; d < D; d++) {
+                m.buf[B_IN][d] = m.buf[B_OUT][d] = stage[g * D + d].data() + cb * D * g;
+            }
+            for (uint32_t d = 0; d < D; d++) {
+                Proc pr;
+                pr.rank = d;
+                if (d == rootLocal) {
+                    for (uint32_t to = 0; to < D; to++) {
+                        if (to != rootLocal) {
+                            pr.prog.push_back(MkSend(static_cast<int>(to), 0, B_IN, cb * to, cb));
+                        }
+                    }
+                } else {
+                    pr.prog.push_back(MkRecvCopy(static_cast<int>(rootLocal), 0, B_OUT, cb * d, cb));
+                }
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+            moved += m.bytesTouched;
+        }
+        {
+            Machine m = machine(1);
+            for (uint32_t r = 0; r < p; r++) {
+                m.Copy(static_cast<uint8_t *>(out[r]) + offset, stage[r].data() + cb * r, cb);
+                moved += 2 * cb;
+            }
+        }
+        offset += cb;
+        left -= cur;
+    }
+    if (touched != nullptr) {
+        *touched = moved;
+    }
+    return 0;
+}
+
 // PairWise all-to-all-v.  counts / displs are p x p row-major tables in elements: row r is what
 // rank r passed to HcclAlltoAllV.  Returns 1 if the send / receive tables are not symmetric
 // (alltoall_operator.cc:49-72), 0 on success.

@@ -657,6 +657,41 @@ def test_ring_scatter(orc):
                 g.close()
 
 
+def test_two_level_scatter(orc):
+    # scatter over several groups: a group's run of blocks goes round the ring of the ranks at the root's position,
+    # then each of those hands the ranks of its group their blocks; step by step the runs rest in the workspace
+    n = 30011
+    for servers, D in ((2, 4), (3, 4), (4, 2), (5, 1)):
+        p = servers * D
+        for fuse in (1, 0):
+            g = gh.Group(p, servers=servers, fuse=fuse)
+            try:
+                for root in sorted({0, p - 1, (D + 1) % p}):
+                    print("two-level scatter", servers, D, "fuse", fuse, "root", root, flush=True)
+                    src = (np.arange(n * p, dtype=np.int64) * 2654435761 % (1 << 31)).astype(np.int32)
+                    want, touched = orc.scatter_two_level(src, p, INT32, root, servers, return_touched=True)
+                    sends = [gh.to_dev(src) if r == root else None for r in range(p)]
+                    recvs = [gh.empty_dev(n * 4) for _ in range(p)]
+                    torch.cuda.synchronize()
+                    H.scatter(g.comms, [t.data_ptr() if t is not None else None for t in sends], [t.data_ptr() for t in recvs],
+                              n, INT32, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    info = g.info()
+                    assert info["fused"] == fuse
+                    if fuse:
+                        assert info["bytesWritten"] == n * 4 * p and info["scratchBytes"] == 0
+                    else:
+                        # what the launches wrote = what the checker's ranks moved, less the root's packing and the
+                        # stop in the receivers' staging buffers (p - servers blocks), which the hand-over skips
+                        assert info["launches"] == servers
+                        assert info["bytesWritten"] == touched // 2 - (2 * p - servers) * n * 4
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(recvs[r], INT32), want[r]), ("two-level scatter", servers, D, fuse, root, r)
+                    assert np.array_equal(gh.to_host(sends[root], INT32), src)
+            finally:
+                g.close()
+
+
 def test_order_sensitive_known_answers_on_the_gpu():
     # hand-derived fp32 sums that differ between ring, the two mesh variants and halving-doubling
     import json

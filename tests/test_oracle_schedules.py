@@ -659,6 +659,35 @@ def test_two_level_broadcast_delivers_and_moves_the_closed_form_bytes(orc, shape
                 assert touched == 2 * received, (shape, dt, n, root, ccl)
 
 
+@pytest.mark.parametrize("shape", [(2, 4), (4, 2), (3, 2), (3, 4), (1, 4), (8, 1), (5, 3)])
+def test_two_level_scatter_delivers_and_moves_the_closed_form_bytes(orc, shape):
+    # Definition: rank r ends with block r of the root.  Structure: the root packs every block, a group's run of D
+    # blocks makes as many hops round the ring of sub-roots as its group is away from the root's, every group's
+    # sub-root hands out D - 1 blocks, every rank copies its block out -- a flat scatter, or a level 1 that went
+    # point to point, would count differently.
+    servers, D = shape
+    p = servers * D
+    for dt, n in ((INT32, 1), (INT32, 1000), (INT8, 10003), (INT64, 500)):
+        unit = orc.dtype_size(dt)
+        for root in sorted({0, p - 1, p // 2, D - 1, min(D, p - 1)}):
+            for ccl in (200 << 20, 8192):
+                src = _inputs(dt, 1, n * p, root + n)[0]
+                outs, touched = orc.scatter_two_level(src, p, dt, root, servers, ccl_bytes=ccl, return_touched=True)
+                for r in range(p):
+                    assert np.array_equal(outs[r], src[r * n:(r + 1) * n]), (shape, dt, n, root, ccl, r)
+                max_per = ccl // p // 128 * 128 // unit
+                moved, left = 0, n
+                while left > 0:
+                    cur = max_per if left * unit * p > ccl else left
+                    block = cur * unit
+                    moved += p * block                                                  # packed by the root
+                    moved += (servers * (servers - 1) // 2) * D * block                 # hops round the ring of sub-roots
+                    moved += servers * (D - 1) * block                                  # handed out inside the groups
+                    moved += p * block                                                  # copied out
+                    left -= cur
+                assert touched == 2 * moved, (shape, dt, n, root, ccl)
+
+
 PRUNED_PORTS = ([0], [5], [0, 4], [2, 3], [1, 6], [0, 2, 4, 6], [1, 2, 3, 7], [4, 5, 6, 7])
 
 

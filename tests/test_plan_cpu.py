@@ -734,6 +734,46 @@ def test_two_level_broadcast_plan(orc, servers, D):
                     assert np.array_equal(recvs[r].view(np.int32), bufs[root]), (servers, D, root, ccl, fused, r)
 
 
+@pytest.mark.parametrize("servers,D", [(2, 4), (4, 2), (3, 4), (5, 3), (6, 1), (2, 8), (1, 4)])
+def test_two_level_scatter_plan(orc, servers, D):
+    # a group's run of blocks travels round the ring of the ranks at the root's position, then every such rank hands
+    # the ranks of its group their blocks
+    p = servers * D
+    n = 1003
+    rng = np.random.default_rng(640 + p)
+    for root in sorted({0, p - 1, (D + 1) % p}):
+        src = rng.integers(0, 1 << 30, n * p).astype(np.int32)
+        plan = H.describe_plan(H.COLL_SCATTER, root | (servers << 21), p, n, INT32)
+        if servers > 1:
+            assert len(plan["phases"]) == servers                        # servers - 1 ring steps, one hand-over
+            for ph in plan["phases"][:-1]:
+                for st in ph:
+                    a, d = st["a"][0], st["dst"][0]
+                    assert a % D == d % D == root % D and d // D == (a // D + 1) % servers, (servers, D, root, a, d)
+                    assert st["n"] == n * 4 * D
+            hops = sum(1 for ph in plan["phases"][:-1] for st in ph)
+            assert hops == servers * (servers - 1) // 2                   # the run of the group j away makes j hops
+        for st in plan["phases"][-1]:
+            a, d = st["a"][0], st["dst"][0]
+            assert a == d // D * D + root % D and st["n"] == n * 4, (servers, D, root, a, d)
+        # The checker's executor for the same schedule moves the same bytes, plus what the reference's staging costs
+        # and the plan leaves out: the root packing its p blocks, and the p - servers blocks that land in a
+        # receiver's staging buffer before they are copied out (the plan's hand-over writes the receive buffer).
+        for ccl in (200 << 20, 4096 * p):
+            want, touched = orc.scatter_two_level(src, p, INT32, root, servers, ccl_bytes=ccl, return_touched=True)
+            for r in range(p):
+                assert np.array_equal(want[r], src[r * n:(r + 1) * n])
+            assert plan["stepWritten"] == touched // 2 - (2 * p - servers) * n * 4, (servers, D, root, ccl)
+        assert plan["stepRead"] == plan["stepWritten"]
+        for fused in (False, True):
+            sends = [src.view(np.uint8).copy() if r == root else np.zeros(0, np.uint8) for r in range(p)]
+            recvs = [np.zeros(n * 4, np.uint8) for _ in range(p)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, INT32, 0)
+            for r in range(p):
+                assert np.array_equal(recvs[r].view(np.int32), src[r * n:(r + 1) * n]), (servers, D, root, fused, r)
+        assert sum(it["n"] for it in plan["fused"]) == n * 4 * p          # fused: every block moves once
+
+
 PRUNED_PORTS = ([0], [5], [0, 4], [2, 3], [1, 6], [0, 2, 4, 6], [1, 2, 3, 7], [4, 5, 6, 7])
 
 
