@@ -808,18 +808,39 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             }
             return 0;
         }
-        // phase i: rank r's block for rank (r+i) goes straight into that rank's receive buffer
+        // Step i: rank r's block for rank (r+i) goes straight into that rank's receive buffer.  A block larger than
+        // the CCL buffer travels in pieces of the buffer's size, one after the other (the BCopy form,
+        // alltoallv_pairwise.cc:112-189, which the reference takes when a rank's send or receive extent exceeds the
+        // buffer, alltoall_operator.cc:122-145; in its ZCopy form every block fits, so the one rule covers both).
+        // The reference stages each piece through the buffer on both sides; here the piece goes direct.
+        if (rq.cclBytes == 0) {
+            *err = "CCL buffer too small";
+            return 1;
+        }
+        size_t phase = 0;
         for (uint32_t i = 0; i < p; i++) {
+            uint64_t pieces = 1;
+            for (uint32_t r = 0; r < p && i > 0; r++) {
+                const uint64_t bytes = rq.sendCounts[size_t(r) * p + (r + i) % p] * u;
+                pieces = std::max(pieces, (bytes + rq.cclBytes - 1) / rq.cclBytes);
+            }
             for (uint32_t r = 0; r < p; r++) {
                 uint32_t n = (r + i) % p;
                 uint64_t cnt = rq.sendCounts[size_t(r) * p + n];
                 uint64_t so = rq.sdispls[size_t(r) * p + n] * u, ro = rq.rdispls[size_t(n) * p + r] * u;
-                EmitCopy(*vp, i, MkRef(n, BUF_RECV, ro), MkRef(r, BUF_SEND, so), cnt * u);
+                if (i == 0) {
+                    EmitCopy(*vp, phase, MkRef(n, BUF_RECV, ro), MkRef(r, BUF_SEND, so), cnt * u);   // LocalCopy (:95-108)
+                }
+                for (uint64_t t = 0, off = 0; i > 0 && off < cnt * u; t++, off += rq.cclBytes) {
+                    EmitCopy(*vp, phase + t, MkRef(n, BUF_RECV, ro + off), MkRef(r, BUF_SEND, so + off),
+                        std::min(rq.cclBytes, cnt * u - off));
+                }
                 if (cnt) {
                     vp->inBytes[r] = std::max(vp->inBytes[r], so + cnt * u);
                     vp->outBytes[n] = std::max(vp->outBytes[n], ro + cnt * u);
                 }
             }
+            phase += pieces;
         }
         return 0;
     }

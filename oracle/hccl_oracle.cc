@@ -3096,6 +3096,59 @@ int orc_alltoallv(uint32_t p, void **send, const uint64_t *sendCounts, const uin
     return m.Run();
 }
 
+// Rounds of the BCopy form per step: the loop of AlltoAllVPairWise::RunBCopyAlltoAll (alltoallv_pairwise.cc:112-171)
+// with CalcSendRecvCounts (:173-189) restated literally for every rank.  rounds[i] (i = 1 .. p-1; rounds[0] = 1, the
+// local copy) = the SendRecv calls of the rank that makes the most in step i; maxPiece = the largest piece any call
+// moves; pieceBytes = the sum over all ranks and calls of the bytes sent.  Returns 0, or -20 on bad arguments.
+int orc_alltoallv_rounds(uint32_t p, const uint64_t *sendCounts, const uint64_t *recvCounts, int dt, uint64_t scratchBytes,
+    uint64_t *rounds, uint64_t *maxPiece, uint64_t *pieceBytes)
+{
+    const uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || scratchBytes == 0) {
+        return -20;
+    }
+    auto curBytes = [&](uint64_t times, uint64_t cur, uint64_t total) -> uint64_t {
+        if (times == 0) {
+            return 0;
+        } else if (times == 1 && cur == times - 1) {
+            return total;
+        } else if (times > 1 && total % scratchBytes == 0 && cur < times) {
+            return scratchBytes;
+        } else if (times > 1 && total % scratchBytes != 0 && cur < times - 1) {
+            return scratchBytes;
+        } else if (times > 1 && total % scratchBytes != 0 && cur == times - 1) {
+            return total % scratchBytes;
+        }
+        return 0;
+    };
+    *maxPiece = 0;
+    *pieceBytes = 0;
+    rounds[0] = 1;
+    for (uint32_t i = 1; i < p; i++) {
+        rounds[i] = 0;
+        for (uint32_t r = 0; r < p; r++) {
+            const uint32_t prev = (r + p - i) % p, next = (r + i) % p;
+            const uint64_t sendBytes = sendCounts[r * p + next] * unit, recvBytes = recvCounts[r * p + prev] * unit;
+            const uint64_t sendTimes = sendBytes / scratchBytes + (sendBytes % scratchBytes == 0 ? 0 : 1);
+            const uint64_t recvTimes = recvBytes / scratchBytes + (recvBytes % scratchBytes == 0 ? 0 : 1);
+            uint64_t curSend = 0, curRecv = 0, calls = 0;
+            while (sendTimes != 0 || recvTimes != 0) {
+                const uint64_t s = curBytes(sendTimes, curSend, sendBytes), v = curBytes(recvTimes, curRecv, recvBytes);
+                calls++;
+                *maxPiece = std::max(*maxPiece, std::max(s, v));
+                *pieceBytes += s;
+                curSend = s != 0 ? curSend + 1 : curSend;
+                curRecv = v != 0 ? curRecv + 1 : curRecv;
+                if (curSend == sendTimes && curRecv == recvTimes) {
+                    break;
+                }
+            }
+            rounds[i] = std::max(rounds[i], calls);
+        }
+    }
+    return 0;
+}
+
 // Staged all-to-all-v over `servers` servers of m = p / servers ranks (zero-copy mode), same tables as
 // orc_alltoallv.  Stage one, inside a server (ALG/impl/coll_executor/coll_all_to_all/coll_all_to_all_v_staged_executor.cc:
 // 378-440; address tables coll_all_to_all_executor.cc:156-335; template TPL/temp_alltoallv/alltoallv_staged_mesh.cc:51-130):

@@ -86,6 +86,8 @@ def lib():
         L.orc_alltoallv.argtypes = [u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, u64, i32, i32]
         L.orc_alltoallv_staged.argtypes = [u32, u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, i32, i32]
         L.orc_alltoallv_staged.restype = i32
+        L.orc_alltoallv_rounds.argtypes = [u32, pu64, pu64, i32, u64, pu64, pu64, pu64]
+        L.orc_alltoallv_rounds.restype = i32
         L.orc_fill_uniform_f32.argtypes = [vp, u64, u64, u32, i32]
         _lib = L
     return _lib
@@ -385,6 +387,20 @@ def alltoallv(sends, send_counts, sdispls, recvs, recv_counts, rdispls, dt, scra
     if rc not in (0, 1):
         raise RuntimeError("oracle alltoallv failed rc=%d" % rc)
     return rc
+
+
+def alltoallv_rounds(send_counts, recv_counts, dt, scratch_bytes):
+    """The BCopy form's transfer loop, per step: (rounds per step as a list, largest piece, bytes sent over all ranks)."""
+    p = send_counts.shape[0]
+    sc = np.ascontiguousarray(send_counts, dtype=np.uint64)
+    rc = np.ascontiguousarray(recv_counts, dtype=np.uint64)
+    rounds, biggest, total = _u64arr(p), ctypes.c_uint64(0), ctypes.c_uint64(0)
+    pu64 = ctypes.POINTER(ctypes.c_uint64)
+    rc_ = lib().orc_alltoallv_rounds(p, sc.ctypes.data_as(pu64), rc.ctypes.data_as(pu64), dt, scratch_bytes, rounds,
+                                     ctypes.byref(biggest), ctypes.byref(total))
+    if rc_ != 0:
+        raise RuntimeError("oracle all-to-all-v rounds failed rc=%d" % rc_)
+    return list(rounds), biggest.value, total.value
 
 
 def alltoallv_staged(sends, send_counts, sdispls, recvs, recv_counts, rdispls, dt, servers, flags=0, threads=1):

@@ -255,6 +255,30 @@ def test_alltoallv_small_ragged(orc):
                 g.close()
 
 
+def test_alltoallv_blocks_larger_than_the_buffer_go_in_pieces(orc):
+    # the reference's piecewise (BCopy) form: with a small CCL buffer a big block takes several transfers; step by step
+    # that is one launch per piece of the slowest rank, as many as the checker's restatement of the transfer loop counts
+    for p in (3, 8):
+        cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 140 + p, max_count=20000)
+        sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+        for ccl in (16384, 1 << 20):
+            want = [np.full(n, -1, np.int32) for n in rl]
+            assert orc.alltoallv(sends, cnt, sdis, want, rcnt, rdis, INT32, scratch_bytes=ccl) == 0
+            rounds, _, total = orc.alltoallv_rounds(cnt, rcnt, INT32, ccl)
+            for fuse in (0, 1):
+                g = gh.Group(p, fuse=fuse, buffsize_bytes=ccl)
+                try:
+                    print("alltoallv in pieces p", p, "buffer", ccl, "fuse", fuse, flush=True)
+                    outs = gh.all_to_all_v(g, sends, cnt, sdis, rl, rcnt, rdis, INT32)
+                    info = g.info()
+                    assert all(np.array_equal(outs[r], want[r]) for r in range(p)), (p, ccl, fuse)
+                    if not fuse:
+                        assert info["launches"] == sum(max(1, x) for x in rounds), (p, ccl, rounds)
+                    assert info["bytesWritten"] == total + 4 * int(np.trace(cnt))
+                finally:
+                    g.close()
+
+
 def test_alltoallv_sub_kib_segments_go_through_the_gather_kernel(orc):
     # many short segments at every byte alignment: int8 payload (so displacements are byte offsets), counts lognormal
     # around 64 elements, and int32 / int64 for the element-aligned case; segments up to and just beyond the gather

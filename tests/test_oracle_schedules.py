@@ -284,6 +284,28 @@ def test_alltoallv_is_the_permutation(orc):
                 assert np.array_equal(recvs[j], want), (p, scratch, j)
 
 
+def test_alltoallv_rounds_of_the_piecewise_form(orc):
+    # Hand-worked: 3 ranks, int32, a 400-byte buffer.  Step 1: rank 0 sends 1000 B (3 pieces: 400, 400, 200), rank 1
+    # 800 B (2 pieces of 400), rank 2 nothing -> the slowest rank makes 3 calls (rank 1 receives 1000 B in 3 and sends
+    # in 2).  Step 2: 0 -> 2 400 B (1 piece), 1 -> 0 4 B, 2 -> 1 1204 B (4 pieces: 3 x 400 + 4) -> 4 calls.
+    cnt = np.array([[5, 250, 100], [1, 7, 200], [0, 301, 9]], np.uint64)
+    rounds, biggest, total = orc.alltoallv_rounds(cnt, cnt.T.copy(), INT32, 400)
+    assert rounds == [1, 3, 4] and biggest == 400 and total == 4 * (250 + 200 + 0 + 100 + 1 + 301)
+    # with a buffer that holds every block each step is one call; an empty step makes none
+    assert orc.alltoallv_rounds(cnt, cnt.T.copy(), INT32, 1 << 20)[0] == [1, 1, 1]
+    only_diag = np.diag([3, 4, 5]).astype(np.uint64)
+    assert orc.alltoallv_rounds(only_diag, only_diag.T.copy(), INT32, 400)[0] == [1, 0, 0]
+    # any table: the slowest rank of step i needs ceil(largest block of the step / buffer) calls
+    for p in (2, 5, 8):
+        cnt, _, rcnt, _, _, _ = _a2av_case(p, 900 + p, max_count=3000)
+        for scratch in (64, 1000, 4096):
+            rounds, biggest, total = orc.alltoallv_rounds(cnt, rcnt, INT32, scratch)
+            for i in range(1, p):
+                big = max(int(cnt[r, (r + i) % p]) * 4 for r in range(p))
+                assert rounds[i] == -(-big // scratch), (p, scratch, i)
+            assert total == 4 * (int(cnt.sum()) - int(np.trace(cnt))) and biggest <= scratch
+
+
 def _a2av_definition(p, cnt, sdis, rdis, sends, rl):
     """What an all-to-all-v is: rank j's receive buffer holds, at rdispls[j][i], the block rank i addressed to j."""
     out = []

@@ -117,6 +117,38 @@ def test_alltoallv_plan_matches_checker(orc, p):
             assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, fused, r)
 
 
+@pytest.mark.parametrize("p", [2, 3, 8])
+def test_alltoallv_plan_moves_big_blocks_in_pieces_of_the_buffer(orc, p):
+    # a block larger than the CCL buffer goes in pieces, one phase each: as many phases per step as the checker's
+    # restatement of the reference's transfer loop makes calls, no piece larger than the buffer
+    cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 70 + p, max_count=3000)
+    cnt[cnt == 0] = 1                       # every step moves something (an empty step has no phase to count)
+    sdis = np.concatenate([np.zeros((p, 1), np.uint64), np.cumsum(cnt, axis=1)[:, :-1]], axis=1).astype(np.uint64)
+    rcnt = cnt.T.copy()
+    rdis = np.concatenate([np.zeros((p, 1), np.uint64), np.cumsum(rcnt, axis=1)[:, :-1]], axis=1).astype(np.uint64)
+    sl, rl = [int(x) for x in cnt.sum(axis=1)], [int(x) for x in rcnt.sum(axis=1)]
+    sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+    for ccl in (512, 4096, 1 << 20):
+        want = [np.full(n, -1, np.int32) for n in rl]
+        assert orc.alltoallv(sends, cnt, sdis, want, rcnt, rdis, INT32, scratch_bytes=ccl) == 0
+        rounds, biggest, total = orc.alltoallv_rounds(cnt, rcnt, INT32, ccl)
+        plan = H.describe_plan(H.COLL_ALLTOALLV, H.ALGO_PAIRWISE, p, 0, INT32, ccl_bytes=ccl, tables=(cnt, sdis, rcnt, rdis))
+        assert len(plan["phases"]) == sum(rounds), (p, ccl, rounds)
+        assert max(st["n"] for ph in plan["phases"] for st in ph) == max(biggest, 4 * int(np.diag(cnt).max()))
+        assert sum(st["n"] for ph in plan["phases"][1:] for st in ph) == total
+        at = 1
+        for i in range(1, p):                                        # step i: ranks r -> r + i, piece t in phase t of the step
+            for t in range(rounds[i]):
+                for st in plan["phases"][at + t]:
+                    assert st["dst"][0] == (st["a"][0] + i) % p and st["n"] <= ccl
+            at += rounds[i]
+        for fused in (False, True):
+            recvs = [np.full(n, -1, np.int32).view(np.uint8).copy() for n in rl]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, _bytes(sends), recvs, INT32, 0)
+            for r in range(p):
+                assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, ccl, fused, r)
+
+
 @pytest.mark.parametrize("p,servers", [(4, 2), (8, 2), (8, 4), (6, 3), (16, 4), (12, 12), (9, 3)])
 def test_staged_alltoallv_plan_matches_checker(orc, p, servers):
     cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 40 + p + servers)
