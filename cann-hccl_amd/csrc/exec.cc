@@ -51,6 +51,7 @@ HcclResult EnsureDevice(Group *g, bool quiet)
         HIP_OK(hipEventCreateWithFlags(&g->arriveEvents[r], hipEventDisableTiming));
     }
     HIP_OK(hipEventCreateWithFlags(&g->doneEvent, hipEventDisableTiming));
+    HIP_OK(hipStreamCreateWithFlags(&g->copyStream, hipStreamNonBlocking));
     g->scratch.assign(g->p, nullptr);
     g->arena.allocFn = [](size_t bytes) -> void * {
         void *mem = nullptr;
@@ -87,25 +88,18 @@ HcclResult EnsureScratch(Group *g, uint64_t bytes)
     if (bytes <= g->scratchBytes) {
         return HCCL_SUCCESS;
     }
-    if (g->pinnedScratchUsers > 0) {
-        // a caller's graph replays collectives that point at these buffers: they stay until the group goes
-        for (uint32_t r = 0; r < g->p; r++) {
-            if (g->scratch[r]) {
-                g->retiredScratch.push_back(g->scratch[r]);
-                g->scratch[r] = nullptr;
-            }
-        }
-        g->pinnedScratchUsers = 0;
-    } else {
-        // A cached collective may still be running out of the old scratch.
-        HIP_OK(hipDeviceSynchronize());
-        for (uint32_t r = 0; r < g->p; r++) {
-            if (g->scratch[r]) {
-                HIP_OK(hipFree(g->scratch[r]));
-                g->scratch[r] = nullptr;
-            }
+    // Collectives issued earlier may still be running out of the old buffers, and a caller's graph may replay
+    // some: the buffers are set aside, not freed (freeing waits for the whole device).  Those a graph points at
+    // stay until the group goes; the others are freed at the next point where the device is known to be idle.
+    // Growing by at least a factor of two keeps what is set aside below the size in use.
+    for (uint32_t r = 0; r < g->p; r++) {
+        if (g->scratch[r]) {
+            (g->pinnedScratchUsers > 0 ? g->retiredScratch : g->idleScratch).push_back(g->scratch[r]);
+            g->scratch[r] = nullptr;
         }
     }
+    g->pinnedScratchUsers = 0;
+    bytes = std::max(bytes, 2 * g->scratchBytes);
     g->scratchBytes = 0;
     g->scratchGen++;
     for (uint32_t r = 0; r < g->p; r++) {
@@ -113,6 +107,16 @@ HcclResult EnsureScratch(Group *g, uint64_t bytes)
     }
     g->scratchBytes = bytes;
     return HCCL_SUCCESS;
+}
+
+// With the device idle: frees what earlier calls set aside.
+void ReleaseIdle(Group *g)
+{
+    g->stale.clear();
+    for (void *s : g->idleScratch) {
+        (void)hipFree(s);
+    }
+    g->idleScratch.clear();
 }
 
 struct Builder {
@@ -559,7 +563,10 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
             pp->uploadComplete = false;
             pp->hostTables.swap(b.host);
         } else {
-            HIP_OK(hipMemcpy(pp->devTables, b.host.data(), b.host.size(), hipMemcpyHostToDevice));
+            // over a stream of the library's own, which no caller captures (a plain copy goes through the null
+            // stream, which a caller's capture of a blocking stream would not tolerate)
+            HIP_OK(hipMemcpyAsync(pp->devTables, b.host.data(), b.host.size(), hipMemcpyHostToDevice, g->copyStream));
+            HIP_OK(hipStreamSynchronize(g->copyStream));
         }
     }
     char *base = static_cast<char *>(pp->devTables);
@@ -886,6 +893,13 @@ Group::~Group()
     }
     cache.clear();
     pinnedStale.clear();
+    stale.clear();
+    for (void *s : idleScratch) {
+        (void)hipFree(s);
+    }
+    if (copyStream) {
+        (void)hipStreamDestroy(copyStream);
+    }
     if (arena.freeFn != nullptr) {
         arena.FreeAll();
     }
@@ -975,41 +989,49 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     auto it = pp ? g->cache.end() : g->cache.find(key);
     if (pp != nullptr) {
         // issued below
-    } else if (it != g->cache.end() && it->second->scratchGen == g->scratchGen) {
+    } else if (it != g->cache.end() && (it->second->scratchGen == g->scratchGen || it->second->info.scratchBytes == 0)) {
+        // (an entry that points into scratch buffers the group has since outgrown is stale)
         pp = it->second.get();
         hit = true;
     } else {
-        // Preparing a collective allocates and fills its device tables, which a stream under capture
-        // does not allow: a caller that records collectives into a graph runs each of them once before.
+        // A caller may be recording this stream into a graph of its own and come with a collective for the first
+        // time.  Preparing it allocates device memory and copies its tables, which must happen now and not as part
+        // of that graph: the thread's capture mode is relaxed for the duration (a capture in the default mode
+        // refuses such calls), and the tables go over a stream of the library's own (Prepare without a stream).
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         HIP_OK(hipStreamIsCapturing(g->ctx->streams[launcher], &capture));
-        if (capture != hipStreamCaptureStatusNone) {
-            HCCL_LOG_ERROR("%s: first use of this collective (sizes, buffers, settings) while its stream is being captured; "
-                "run it once before the capture", CollName(g->ctx->sig.coll));
-            return HCCL_E_NOT_SUPPORT;
-        }
+        const bool underCapture = capture != hipStreamCaptureStatusNone;
         if (it != g->cache.end()) {
-            // stale entry (the scratch buffers moved); its tables stay in the arena
-            if (it->second->pinned) {
-                g->pinnedStale.push_back(std::move(it->second));   // a caller's graph still replays it out of the retired buffers
-            } else {
-                HIP_OK(hipDeviceSynchronize());
-            }
+            // stale entry (the scratch buffers moved); earlier launches may still be running out of its tables and
+            // a caller's graph may replay it out of the retired buffers, so it is set aside
+            (it->second->pinned ? g->pinnedStale : g->stale).push_back(std::move(it->second));
             g->cache.erase(it);
         }
-        if (g->cache.size() >= g->cfg.cacheEntries) {
+        if (g->cache.size() >= g->cfg.cacheEntries && !underCapture) {
             // Full: wait once for whatever is still in flight and start over.  Dropping one entry at a
             // time would put a device-wide wait on every call of a caller with more buffers than entries
             // (measured with 200 buffer sets against 64 entries: 42 us per small all-reduce instead of 7.5).
             // Collectives recorded into a caller's graph stay, tables and all (the arena keeps their chunks).
+            // (Under capture the device may not be waited for: the cache runs over until the next call outside.)
             HIP_OK(hipDeviceSynchronize());
             for (auto e = g->cache.begin(); e != g->cache.end();) {
                 e = e->second->pinned ? std::next(e) : g->cache.erase(e);
             }
+            ReleaseIdle(g);
             g->arena.Reset();
         }
         std::unique_ptr<Prepared> fresh;
-        r = Prepare(g, algo, &fresh, false, g->ctx->streams[launcher]);
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        if (underCapture) {
+            HIP_OK(hipThreadExchangeStreamCaptureMode(&mode));
+        }
+        r = Prepare(g, algo, &fresh, false, underCapture ? nullptr : g->ctx->streams[launcher]);
+        if (underCapture) {
+            hipError_t back = hipThreadExchangeStreamCaptureMode(&mode);
+            if (r == HCCL_SUCCESS) {
+                HIP_OK(back);
+            }
+        }
         if (r != HCCL_SUCCESS) {
             return r;
         }

@@ -173,6 +173,9 @@ struct Group {
     std::vector<void *> retiredScratch;   // scratch buffers a pinned collective still points at; freed with the group
     uint32_t pinnedScratchUsers = 0;      // pinned collectives that use the current scratch buffers
     std::vector<std::unique_ptr<Prepared>> pinnedStale;   // pinned collectives that left the cache
+    std::vector<void *> idleScratch;      // outgrown scratch buffers that work in flight may still use; freed when the device is next known idle
+    std::vector<std::unique_ptr<Prepared>> stale;         // collectives that left the cache while work in flight may still use them; same
+    hipStream_t copyStream = nullptr;     // the library's own stream for table copies (non-blocking, never captured)
     void *barrierMem = nullptr;       // 2 x p small buffers for HcclBarrier's all-reduce
     void *noAllocBase = nullptr;      // this device's copy of the fixed workspace (noalloc.hip), looked up at set-up
     uint64_t scratchBytes = 0;

@@ -1330,7 +1330,7 @@ def test_two_groups_on_two_host_threads(orc):
 
 
 def test_collectives_recorded_into_a_callers_graph(orc):
-    # a caller captures its stream (collectives it has run once before, so nothing needs preparing) and replays
+    # a caller captures its stream (first collectives it has run once before, then ones the library has not seen) and replays
     # the graph with other work of its own in between; every replay must give the eager result
     p, n = 8, 100003
     for fuse in (1, 0):
@@ -1347,7 +1347,7 @@ def test_collectives_recorded_into_a_callers_graph(orc):
                 H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, FP32, SUM, g.stream_ptr)
                 H.all_gather(g.comms, [t.data_ptr() for t in recvs], [t.data_ptr() for t in gath], n, FP32, g.stream_ptr)
 
-            both()                                   # first use prepares the tables (not allowed under capture)
+            both()                                   # first use prepares the tables
             g.stream.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.stream(g.stream):
@@ -1370,16 +1370,47 @@ def test_collectives_recorded_into_a_callers_graph(orc):
                 for r in range(p):
                     assert np.array_equal(recvs[r].cpu().numpy(), want[r]), (fuse, replay, r)
                     assert np.array_equal(gath[r].cpu().numpy(), np.concatenate(want)), (fuse, replay, r)
-            # a collective the library has not seen yet cannot be prepared while the stream is being captured
+            # collectives the library has not seen yet (another count; a reduce-scatter, which step by step also
+            # needs the group's scratch buffers allocated) are prepared while the stream is being captured: tables
+            # and buffers are set up at once, outside the caller's graph, and the kernels become its nodes
+            m = (n - 7) // p * p
+            parts = [torch.zeros(m // p, dtype=torch.float32, device="cuda") for _ in range(p)]
+            torch.cuda.synchronize()
             graph2 = torch.cuda.CUDAGraph()
             with torch.cuda.stream(g.stream):
                 graph2.capture_begin()
                 try:
-                    codes = [H.lib().HcclAllReduce(sends[r].data_ptr(), recvs[r].data_ptr(), n - 7, FP32, SUM, g.comms[r], g.stream_ptr)
-                             for r in range(p)]
+                    H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n - 7, FP32, SUM, g.stream_ptr)
+                    first = g.info()
+                    H.reduce_scatter(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in parts], m // p, FP32, SUM,
+                                     g.stream_ptr)
                 finally:
                     graph2.capture_end()
-            assert codes[:-1] == [0] * (p - 1) and codes[-1] == H.HCCL_E_NOT_SUPPORT
+            assert first["cacheHit"] == 0 and first["graph"] == 0
+            for replay in range(3):
+                for t in sends:
+                    t.mul_(0.75)
+                torch.cuda.synchronize()
+                host = [t.cpu().numpy() for t in sends]
+                want = orc.allreduce([x[:n - 7] for x in host], FP32, SUM)
+                want_rs = orc.reducescatter([x[:m] for x in host], FP32, SUM)
+                for t in recvs + parts:
+                    t.zero_()
+                torch.cuda.synchronize()
+                graph2.replay()
+                torch.cuda.synchronize()
+                for r in range(p):
+                    assert np.array_equal(recvs[r].cpu().numpy()[:n - 7], want[r]), (fuse, replay, r)
+                    assert not recvs[r].cpu().numpy()[n - 7:].any()
+                    assert np.array_equal(parts[r].cpu().numpy(), want_rs[r]), (fuse, replay, r)
+            # and the same collective outside the capture finds what the capture prepared
+            for t in recvs:
+                t.zero_()
+            H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n - 7, FP32, SUM, g.stream_ptr)
+            g.stream.synchronize()
+            assert g.info()["cacheHit"] == 1
+            for r in range(p):
+                assert np.array_equal(recvs[r].cpu().numpy()[:n - 7], want[r]), (fuse, "eager", r)
         finally:
             g.close()
 
