@@ -157,9 +157,12 @@ HcclResult LoadCommConfig(const HcclCommConfig *user, GroupConfig *cfg, std::str
 {
     HcclCommConfig local;
     std::memset(&local, 0, sizeof(local));   // bytes the caller's (older, smaller) struct does not have stay zero
-    size_t size = *reinterpret_cast<const size_t *>(user);
+    size_t size = 0;
+    std::memcpy(&size, user, sizeof(size));   // the struct is only 4-byte aligned: its leading fields are read by copy
     std::memcpy(&local, user, std::min(size, sizeof(local)));
-    const ConfigHeader *h = reinterpret_cast<const ConfigHeader *>(&local);
+    ConfigHeader header;
+    std::memcpy(&header, &local, sizeof(header));
+    const ConfigHeader *h = &header;
     if (h->magicWord != HCCL_COMM_CONFIG_MAGIC_WORD) {
         HCCL_LOG_ERROR("comm config: bad magic word 0x%x; initialise the struct with HcclCommConfigInit()", h->magicWord);
         return HCCL_E_PARA;
@@ -671,10 +674,14 @@ const char *HcclGetErrorString(HcclResult code)
         "timeout", "open file fail", "tcp connect fail", "roce connect fail", "tcp transfer fail", "roce transfer fail",
         "call runtime api fail", "call driver api fail", "call profiling api fail", "call cce api fail",
         "call network api fail", "try again", "error cqe", "communicator suspending"};
-    if (int(code) < int(HCCL_SUCCESS) || int(code) >= int(HCCL_E_RESERVED)) {
+    // a caller may hand over any number; it is read as one, not as the enumeration it may not belong to
+    int32_t value = 0;
+    static_assert(sizeof(value) == sizeof(code), "HcclResult is a 32-bit enumeration");
+    std::memcpy(&value, &code, sizeof(value));
+    if (value < int32_t(HCCL_SUCCESS) || value >= int32_t(HCCL_E_RESERVED)) {
         return "unknow error";
     }
-    return names[int(code)];
+    return names[value];
 }
 
 // op_base.cc:3567-3571.
