@@ -923,6 +923,18 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             vp->inBytes[R] = total * p;
             return 0;
         }
+        if (rq.coll == COLL_BROADCAST && rq.algo == ALGO_STAR) {
+            // star broadcast (broadcast_star.cc:47-99): the root sends every other rank the whole buffer, in one go
+            // (its one caller, broadcast_operator_for_hetero.cc:91-113, runs it without a chunk loop)
+            for (uint32_t r = 0; r < p; r++) {
+                if (r != R) {
+                    EmitCopy(*vp, 0, MkRef(r, BUF_RECV, 0), MkRef(R, BUF_SEND, 0), total);
+                }
+                vp->inBytes[r] = (r == R) ? total : 0;
+                vp->outBytes[r] = (r == R) ? 0 : total;
+            }
+            return 0;
+        }
         uint64_t per = (rq.coll == COLL_BROADCAST || rq.coll == COLL_REDUCE) ? rq.cclBytes / u : 0;
         if (per == 0) {
             *err = "CCL buffer too small";

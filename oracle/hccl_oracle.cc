@@ -2078,6 +2078,49 @@ int orc_broadcast(uint32_t p, void **buf, uint64_t count, int dt, uint32_t root,
     return 0;
 }
 
+// Star broadcast (TPL/temp_broadcast/broadcast_star.cc:47-99, run by ALG/impl/legacy/operator/
+// broadcast_operator_for_hetero.cc:91-113 over the whole buffer, no chunk loop): the root sends every other rank all
+// of it (RunSendBroadcast :137-165), every other rank receives it from the root (RunRecvBroadcast :101-135).
+// `touched` (optional) receives the bytes read + written by all ranks.
+int orc_broadcast_star(uint32_t p, void **buf, uint64_t count, int dt, uint32_t root, int flags, int threads, uint64_t *touched)
+{
+    const uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    const uint64_t bytes = count * unit;
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    for (uint32_t r = 0; r < p; r++) {
+        m.buf[B_IN][r] = m.buf[B_OUT][r] = static_cast<uint8_t *>(buf[r]);
+    }
+    for (uint32_t r = 0; r < p && p > 1; r++) {
+        Proc pr;
+        pr.rank = r;
+        if (r == root) {
+            for (uint32_t d = 0; d < p; d++) {
+                if (d != root && bytes > 0) {
+                    pr.prog.push_back(MkSend(static_cast<int>(d), 0, B_IN, 0, bytes));
+                }
+            }
+        } else if (bytes > 0) {
+            pr.prog.push_back(MkRecvCopy(static_cast<int>(root), 0, B_OUT, 0, bytes));
+        }
+        m.procs.push_back(std::move(pr));
+    }
+    int rc = p > 1 ? m.Run() : 0;
+    if (touched != nullptr) {
+        *touched = m.bytesTouched;
+    }
+    return rc;
+}
+
 // Mesh broadcast, CollBroadcastMeshExecutor::KernelRun (EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213)
 // on one server: the root scatters slice i to rank i (TPL/temp_scatter/scatter_mesh.cc:46-160), then a mesh
 // all-gather; slices from GetRankSliceSize (EXE/coll_broadcast/coll_broadcast_executor.cc:275-306).

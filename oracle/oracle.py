@@ -29,9 +29,13 @@ NP_CARRIER = {
 
 def build(force=False):
     """Compile the checker with g++ (a few seconds)."""
+    import fcntl
     src = os.path.join(_HERE, "hccl_oracle.cc")
-    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
-        subprocess.check_call(["make", "-C", _HERE, "-B", "libhccl_oracle.so"], stdout=subprocess.DEVNULL)
+    # one builder at a time (test workers start together): the others wait and then find the library up to date
+    with open(os.path.join(_HERE, ".build.lock"), "w") as lock:
+        fcntl.flock(lock, fcntl.LOCK_EX)
+        if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+            subprocess.check_call(["make", "-C", _HERE, "-B", "libhccl_oracle.so"], stdout=subprocess.DEVNULL)
     return _LIB_PATH
 
 
@@ -74,6 +78,8 @@ def lib():
         L.orc_reduce_to_root_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_rhd.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
+        L.orc_broadcast_star.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, i32, i32, ctypes.POINTER(u64)]
+        L.orc_broadcast_star.restype = i32
         L.orc_allreduce_ring_pruned.argtypes = [u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, ctypes.POINTER(u32), u32,
                                                 u64, u64, i32, i32]
         L.orc_broadcast_two_level.argtypes = [u32, u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32, ctypes.POINTER(u64)]
@@ -305,6 +311,15 @@ def broadcast(bufs, dt, root, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, 
     if rc != 0:
         raise RuntimeError("oracle broadcast failed rc=%d" % rc)
     return bufs
+
+
+def broadcast_star(bufs, dt, root, flags=0, threads=1, return_touched=False):
+    """The root hands every rank the whole buffer, all at once.  bufs are written in place."""
+    touched = ctypes.c_uint64(0)
+    rc = lib().orc_broadcast_star(len(bufs), _ptrs(bufs), bufs[0].size, dt, root, flags, threads, ctypes.byref(touched))
+    if rc != 0:
+        raise RuntimeError("oracle star broadcast failed rc=%d" % rc)
+    return (bufs, touched.value) if return_touched else bufs
 
 
 def broadcast_two_level(bufs, dt, root, servers, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1,

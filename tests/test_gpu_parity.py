@@ -819,6 +819,36 @@ def test_broadcast_and_reduce_mesh_and_rhd_schedules(orc):
                     g.close()
 
 
+def test_star_broadcast(orc):
+    # the root hands every rank the whole buffer: step by step one launch of p - 1 transfers, also over several servers
+    n = 70001
+    for p, servers in ((2, 1), (5, 1), (8, 1), (8, 2)):
+        for fuse in (1, 0):
+            g = gh.Group(p, algo="star", fuse=fuse, servers=servers, buffsize_bytes=4096)
+            try:
+                for root in sorted({0, p - 1, p // 2}):
+                    print("star broadcast p", p, "servers", servers, "fuse", fuse, "root", root, flush=True)
+                    bufs_np = _ins(INT32, p, n, 195 + p + root)
+                    want, touched = orc.broadcast_star([x.copy() for x in bufs_np], INT32, root, return_touched=True)
+                    bufs = [gh.to_dev(x) for x in bufs_np]
+                    torch.cuda.synchronize()
+                    H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, INT32, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    info = g.info()
+                    assert info["algo"] == 5 and info["launches"] == 1 and info["bytesWritten"] == touched // 2
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(bufs[r], INT32), want[r]), ("star", p, fuse, root, r)
+                # the setting only concerns the broadcast: an all-reduce of the same group runs its ring
+                ins = _ins(FP32, p, 4099, 196 + p)
+                outs, _ = gh.all_reduce(g, ins, FP32, SUM)
+                want = orc.allreduce(ins, FP32, SUM, ccl_bytes=4096) if servers == 1 else None
+                if want is not None:
+                    for r in range(p):
+                        assert np.array_equal(outs[r], want[r]), ("ring under star", p, fuse, r)
+            finally:
+                g.close()
+
+
 def test_allreduce_at_the_rank_limit(orc):
     # 64 ranks is the most a group holds: ring / uncut mesh = chains of 64 sources (the fused kernel's limit),
     # halving-doubling at 48 ranks = 32 leaves of which 16 are folded pairs, at 64 ranks = 32 leaves of two

@@ -652,6 +652,20 @@ def test_allgather_v_is_the_permutation(orc, algo):
                 assert np.array_equal(got[r], want), (algo, dt, p, r)       # blocks in place, gaps untouched
 
 
+def test_star_broadcast_delivers_and_every_byte_comes_from_the_root(orc):
+    # Definition: every rank ends with the root's bytes.  Structure: p - 1 transfers of the whole buffer and nothing
+    # else (a ring or a tree would move the same bytes; what tells the star apart is checked on the plan: every
+    # transfer starts at the root).
+    for p in (1, 2, 5, 8):
+        for dt, n in ((INT32, 1), (INT8, 100003), (INT64, 5000)):
+            for root in sorted({0, p - 1, p // 2}):
+                bufs = _inputs(dt, p, n, root + n)
+                src = bufs[root].copy()
+                bufs, touched = orc.broadcast_star(bufs, dt, root, return_touched=True)
+                assert all(np.array_equal(b, src) for b in bufs), (p, dt, n, root)
+                assert touched == 2 * (p - 1) * n * orc.dtype_size(dt)
+
+
 @pytest.mark.parametrize("shape", [(2, 4), (4, 2), (3, 2), (3, 4), (1, 4), (8, 1), (5, 3)])
 def test_two_level_broadcast_delivers_and_moves_the_closed_form_bytes(orc, shape):
     # Definition: every rank ends with the root's bytes.  Structure: the bytes received over all ranks are those of

@@ -726,6 +726,25 @@ def test_ring_scatter_plan_matches_checker(orc, p):
                 assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, root, fused, r)
 
 
+@pytest.mark.parametrize("p", [1, 2, 5, 8])
+def test_star_broadcast_plan(orc, p):
+    # one phase, every transfer from the root, the whole buffer each; same bytes as the checker's star
+    n = 1003
+    for root in sorted({0, p - 1, p // 2}):
+        bufs = _ins(INT32, p, n, 170 + p)
+        want, touched = orc.broadcast_star([b.copy() for b in bufs], INT32, root, return_touched=True)
+        plan = H.describe_plan(H.COLL_BROADCAST, root | (5 << 16), p, n, INT32, ccl_bytes=1024, in_place_mask=(1 << p) - 1)
+        if p > 1:
+            assert len(plan["phases"]) == 1 and len(plan["phases"][0]) == p - 1
+            assert all(st["a"][0] == root and st["n"] == n * 4 for st in plan["phases"][0])
+        assert plan["stepWritten"] == touched // 2
+        for fused in (False, True):
+            mem = _bytes(bufs)
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, mem, mem, INT32, 0, in_place=True)
+            for r in range(p):
+                assert np.array_equal(mem[r].view(np.int32), want[r]), (p, root, fused, r)
+
+
 @pytest.mark.parametrize("servers,D", [(2, 4), (4, 2), (3, 4), (5, 3), (6, 1), (2, 8)])
 def test_two_level_broadcast_plan(orc, servers, D):
     # scatter inside the root's group, halving-doubling between the groups, all-gather inside every group:
