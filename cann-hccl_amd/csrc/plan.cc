@@ -787,20 +787,55 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                     }
                 }
             }
+            // Between the servers a run larger than the CCL buffer goes in batches of the buffer's size: the blocks of
+            // a run are packed into a batch in order and the block that does not fit is cut where the batch is full
+            // (alltoallv_staged_pairwise.cc:143-244, the BCopy form; a run that fits is one batch, as in the ZCopy
+            // form).  Batch t of a step's slowest pair is phase t of that step.  The reference stages a batch
+            // through the buffer on both sides; here every part of a block goes direct.
+            if (rq.cclBytes == 0) {
+                *err = "CCL buffer too small";
+                return 1;
+            }
+            std::vector<uint64_t> batches(S, 1), firstPhase(S, 2);
+            for (uint32_t r = 0; r < p; r++) {
+                for (uint32_t j = r % m; j < p; j += m) {
+                    const uint32_t step = (j / m + S - r / m) % S;
+                    uint64_t run = 0;
+                    for (uint32_t k = 0; k < m; k++) {
+                        run += len(r / m * m + k, j);
+                    }
+                    if (step > 0) {
+                        batches[step] = std::max(batches[step], (run + rq.cclBytes - 1) / rq.cclBytes);
+                    }
+                }
+            }
+            for (uint32_t st = 1; st < S; st++) {
+                firstPhase[st] = firstPhase[st - 1] + batches[st - 1];
+            }
             vp->workBytes.assign(p, 0);
             for (uint32_t r = 0; r < p; r++) {
                 const uint32_t c = r / m, l = r % m;
                 const uint64_t work = (vp->inBytes[r] + 255) & ~uint64_t(255);
                 uint64_t at = work;
                 for (uint32_t j = l; j < p; j += m) {
+                    const uint32_t step = (j / m + S - c) % S;
+                    uint64_t sent = 0;      // bytes of this run handed over so far
                     for (uint32_t k = 0; k < m; k++) {
                         const uint32_t src = c * m + k;
                         const uint64_t n = len(src, j);
                         // stage one: own blocks first (LocalCopy), the neighbours' all at once (alltoallv_staged_mesh.cc:51-130)
                         EmitCopy(*vp, k == l ? 0 : 1, MkRef(r, BUF_SEND, at), MkRef(src, BUF_SEND, rq.sdispls[size_t(src) * p + j] * u), n);
                         // stage two: step i hands the run for server c + i to the rank of that server with local index l
-                        const uint32_t step = (j / m + S - c) % S;
-                        EmitCopy(*vp, 2 + step, MkRef(j, BUF_RECV, rq.rdispls[size_t(j) * p + src] * u), MkRef(r, BUF_SEND, at), n);
+                        const uint64_t to = rq.rdispls[size_t(j) * p + src] * u;
+                        if (step == 0) {
+                            EmitCopy(*vp, firstPhase[0], MkRef(j, BUF_RECV, to), MkRef(r, BUF_SEND, at), n);
+                        }
+                        for (uint64_t off = 0; step > 0 && off < n;) {
+                            const uint64_t room = rq.cclBytes - sent % rq.cclBytes, part = std::min(room, n - off);
+                            EmitCopy(*vp, firstPhase[step] + sent / rq.cclBytes, MkRef(j, BUF_RECV, to + off), MkRef(r, BUF_SEND, at + off), part);
+                            off += part;
+                            sent += part;
+                        }
                         at += n;
                     }
                 }

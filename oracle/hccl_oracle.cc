@@ -3192,6 +3192,102 @@ int orc_alltoallv_rounds(uint32_t p, const uint64_t *sendCounts, const uint64_t 
     return 0;
 }
 
+// Batches of the staged schedule's second stage in its buffer-copy form: CalcSendRecvTimes and LoadPolicies of
+// AlltoAllVStagedPairwise (alltoallv_staged_pairwise.cc:185-244) restated literally for the send side of every rank
+// (c, l) and step i: the run for server c + i is the list of blocks (source k = 0 .. m-1 of the own server, addressed
+// to rank (c + i, l)); blocks are packed into a batch of `scratchBytes` in order, a block that does not fit is cut
+// where the batch is full (SplitSendRecvAddrInfo :317-330), an empty block is skipped.  rounds[i] (i = 1 ..
+// servers-1; rounds[0] = 1, the local copies) = the batches of the pair with the most in step i; entries = the list
+// entries of all batches of all ranks that carry bytes (blocks and parts of blocks; when the rest of a cut block fills
+// a batch exactly, the reference closes that batch only at the next block, with an entry of no bytes in front, :226-236:
+// restated, not counted); maxBatch = the bytes of the fullest batch.
+// Returns 0, -20 on bad arguments, -22 if a batch count disagrees with CalcSendRecvTimes (CheckPolicies :246-265).
+int orc_alltoallv_staged_rounds(uint32_t p, uint32_t servers, const uint64_t *sendCounts, int dt, uint64_t scratchBytes,
+    uint64_t *rounds, uint64_t *entries, uint64_t *maxBatch)
+{
+    const uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || servers == 0 || p % servers != 0 || scratchBytes == 0) {
+        return -20;
+    }
+    const uint32_t m = p / servers;
+    *entries = 0;
+    *maxBatch = 0;
+    rounds[0] = 1;
+    for (uint32_t i = 1; i < servers; i++) {
+        rounds[i] = 0;
+        for (uint32_t r = 0; r < p; r++) {
+            const uint32_t c = r / m, l = r % m, dest = ((c + i) % servers) * m + l;
+            std::vector<uint64_t> blocks;
+            uint64_t sendBytes = 0;
+            for (uint32_t k = 0; k < m; k++) {
+                blocks.push_back(sendCounts[size_t(c * m + k) * p + dest] * unit);
+                sendBytes += blocks.back();
+            }
+            const uint64_t sendTimes = sendBytes / scratchBytes + (sendBytes % scratchBytes == 0 ? 0 : 1);
+            std::vector<std::vector<uint64_t>> policies(sendTimes);
+            std::vector<uint64_t> temp;
+            uint64_t curTime = 0, room = scratchBytes;
+            for (uint64_t block : blocks) {
+                if (block == 0) {
+                    continue;
+                }
+                if (block <= room) {
+                    temp.push_back(block);
+                    room -= block;
+                    if (room == 0) {
+                        room = scratchBytes;
+                        if (curTime >= sendTimes) {
+                            return -22;
+                        }
+                        policies[curTime++] = temp;
+                        temp.clear();
+                    }
+                } else {
+                    uint64_t rest = block;
+                    while (rest > room) {
+                        temp.push_back(room);
+                        rest -= room;
+                        room = scratchBytes;
+                        if (curTime >= sendTimes) {
+                            return -22;
+                        }
+                        policies[curTime++] = temp;
+                        temp.clear();
+                    }
+                    if (rest != 0) {
+                        temp.push_back(rest);
+                        room -= rest;
+                    }
+                }
+            }
+            if (room != scratchBytes) {
+                if (curTime >= sendTimes) {
+                    return -22;
+                }
+                policies[curTime++] = temp;
+            }
+            if (curTime != sendTimes) {
+                return -22;
+            }
+            for (const std::vector<uint64_t> &batch : policies) {
+                uint64_t sum = 0;
+                for (uint64_t part : batch) {
+                    sum += part;
+                }
+                if (sum > scratchBytes) {
+                    return -22;
+                }
+                *maxBatch = std::max(*maxBatch, sum);
+                for (uint64_t part : batch) {
+                    *entries += part > 0 ? 1 : 0;
+                }
+            }
+            rounds[i] = std::max(rounds[i], sendTimes);
+        }
+    }
+    return 0;
+}
+
 // Staged all-to-all-v over `servers` servers of m = p / servers ranks (zero-copy mode), same tables as
 // orc_alltoallv.  Stage one, inside a server (ALG/impl/coll_executor/coll_all_to_all/coll_all_to_all_v_staged_executor.cc:
 // 378-440; address tables coll_all_to_all_executor.cc:156-335; template TPL/temp_alltoallv/alltoallv_staged_mesh.cc:51-130):

@@ -94,6 +94,8 @@ def lib():
         L.orc_alltoallv_staged.restype = i32
         L.orc_alltoallv_rounds.argtypes = [u32, pu64, pu64, i32, u64, pu64, pu64, pu64]
         L.orc_alltoallv_rounds.restype = i32
+        L.orc_alltoallv_staged_rounds.argtypes = [u32, u32, pu64, i32, u64, pu64, pu64, pu64]
+        L.orc_alltoallv_staged_rounds.restype = i32
         L.orc_fill_uniform_f32.argtypes = [vp, u64, u64, u32, i32]
         _lib = L
     return _lib
@@ -416,6 +418,19 @@ def alltoallv_rounds(send_counts, recv_counts, dt, scratch_bytes):
     if rc_ != 0:
         raise RuntimeError("oracle all-to-all-v rounds failed rc=%d" % rc_)
     return list(rounds), biggest.value, total.value
+
+
+def alltoallv_staged_rounds(send_counts, servers, dt, scratch_bytes):
+    """Second stage of the staged schedule in its buffer-copy form: (batches per step as a list of `servers` entries,
+    list entries over all batches and ranks, bytes of the fullest batch)."""
+    p = send_counts.shape[0]
+    sc = np.ascontiguousarray(send_counts, dtype=np.uint64)
+    rounds, entries, biggest = _u64arr(servers), ctypes.c_uint64(0), ctypes.c_uint64(0)
+    rc_ = lib().orc_alltoallv_staged_rounds(p, servers, sc.ctypes.data_as(ctypes.POINTER(ctypes.c_uint64)), dt, scratch_bytes,
+                                            rounds, ctypes.byref(entries), ctypes.byref(biggest))
+    if rc_ != 0:
+        raise RuntimeError("oracle staged all-to-all-v rounds failed rc=%d" % rc_)
+    return list(rounds), entries.value, biggest.value
 
 
 def alltoallv_staged(sends, send_counts, sdispls, recvs, recv_counts, rdispls, dt, servers, flags=0, threads=1):

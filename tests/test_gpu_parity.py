@@ -393,6 +393,31 @@ def test_staged_alltoallv_over_servers(orc):
                 g.close()
 
 
+def test_staged_alltoallv_batches_runs_larger_than_the_buffer(orc):
+    # several servers and a small CCL buffer: between the servers a run goes in batches of the buffer's size, step by
+    # step one launch per batch of the slowest pair (the checker's restatement of the reference's packing counts them)
+    for p, servers in ((8, 2), (12, 3)):
+        cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 160 + p, max_count=6000)
+        sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+        want = [np.full(n, -1, np.int32) for n in rl]
+        assert orc.alltoallv_staged(sends, cnt, sdis, want, rcnt, rdis, INT32, servers) == 0
+        for ccl in (8192, 1 << 20):
+            rounds, _, _ = orc.alltoallv_staged_rounds(cnt, servers, INT32, ccl)
+            for fuse in (0, 1):
+                g = gh.Group(p, fuse=fuse, servers=servers, buffsize_bytes=ccl)
+                try:
+                    print("staged alltoallv in batches p", p, "servers", servers, "buffer", ccl, "fuse", fuse, flush=True)
+                    outs = gh.all_to_all_v(g, sends, cnt, sdis, rl, rcnt, rdis, INT32)
+                    info = g.info()
+                    assert all(np.array_equal(outs[r], want[r]) for r in range(p)), (p, servers, ccl, fuse)
+                    if not fuse:
+                        assert info["launches"] == 2 + sum(max(1, x) for x in rounds), (p, servers, ccl, rounds)
+                    else:
+                        assert info["bytesWritten"] == 4 * int(cnt.sum())
+                finally:
+                    g.close()
+
+
 def test_staged_uniform_alltoall_over_servers():
     p, servers, n = 8, 2, 3001
     rng = np.random.default_rng(77)

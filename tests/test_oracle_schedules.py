@@ -306,6 +306,35 @@ def test_alltoallv_rounds_of_the_piecewise_form(orc):
             assert total == 4 * (int(cnt.sum()) - int(np.trace(cnt))) and biggest <= scratch
 
 
+def test_staged_alltoallv_batches_of_the_buffer_copy_form(orc):
+    # Hand-worked: 2 servers of 2 ranks, int8, a 10-byte buffer.  Rank 0 hands rank 2 the blocks of its server's two
+    # ranks, 7 and 8 bytes: batches [7, 3] and [5] (the second block is cut where the first batch is full) = 2 batches,
+    # 3 list entries.  Rank 1 hands rank 3 one block of 25 bytes and an empty one: [10] [10] [5] = 3 batches, 3 entries.
+    cnt = np.zeros((4, 4), np.uint64)
+    cnt[0, 2], cnt[1, 2], cnt[0, 3] = 7, 8, 25
+    assert orc.alltoallv_staged_rounds(cnt, 2, INT8, 10) == ([1, 3], 6, 10)
+    assert orc.alltoallv_staged_rounds(cnt, 2, INT8, 100) == ([1, 1], 3, 25)      # everything fits: one batch per run
+    # any table: a pair's batches = ceil(run / buffer), and every full batch adds one cut unless it ends on a block's end
+    for p, servers in ((8, 2), (12, 3), (8, 4)):
+        m = p // servers
+        cnt = _a2av_case(p, 950 + p, max_count=900)[0]
+        for scratch in (256, 4096):
+            rounds, entries, biggest = orc.alltoallv_staged_rounds(cnt, servers, INT32, scratch)
+            want_entries = 0
+            for i in range(1, servers):
+                most = 0
+                for r in range(p):
+                    c, l = divmod(r, m)
+                    dest = (c + i) % servers * m + l
+                    blocks = [int(cnt[c * m + k, dest]) * 4 for k in range(m)]
+                    most = max(most, -(-sum(blocks) // scratch))
+                    ends = set(np.cumsum(blocks).tolist())
+                    cuts = [x for x in range(scratch, sum(blocks), scratch) if x not in ends]
+                    want_entries += sum(1 for b in blocks if b) + len(cuts)
+                assert rounds[i] == most, (p, servers, scratch, i)
+            assert entries == want_entries and biggest <= scratch
+
+
 def _a2av_definition(p, cnt, sdis, rdis, sends, rl):
     """What an all-to-all-v is: rank j's receive buffer holds, at rdispls[j][i], the block rank i addressed to j."""
     out = []

@@ -177,6 +177,44 @@ def test_staged_alltoallv_plan_matches_checker(orc, p, servers):
         H.describe_plan(H.COLL_ALLTOALLV, H.ALGO_PAIRWISE | (uneven << 8), p, 0, INT32, tables=(cnt, sdis, rcnt, rdis))
 
 
+@pytest.mark.parametrize("p,servers", [(8, 2), (12, 3), (8, 4)])
+def test_staged_alltoallv_plan_batches_runs_larger_than_the_buffer(orc, p, servers):
+    # between the servers a run larger than the CCL buffer goes in batches, one phase each, a block cut where a batch
+    # is full: as many phases and as many transfers as the checker's restatement of the reference's packing counts
+    m = p // servers
+    cnt = _a2av_case(p, 75 + p + servers, max_count=900)[0]
+    cnt[cnt == 0] = 3
+    rcnt = cnt.T.copy()
+    sdis = np.concatenate([np.zeros((p, 1), np.uint64), np.cumsum(cnt, axis=1)[:, :-1]], axis=1).astype(np.uint64)
+    rdis = np.concatenate([np.zeros((p, 1), np.uint64), np.cumsum(rcnt, axis=1)[:, :-1]], axis=1).astype(np.uint64)
+    sl, rl = [int(x) for x in cnt.sum(axis=1)], [int(x) for x in rcnt.sum(axis=1)]
+    sends = [(np.arange(n, dtype=np.int32) + (r << 20)) for r, n in enumerate(sl)]
+    want = [np.full(n, -1, np.int32) for n in rl]
+    assert orc.alltoallv_staged(sends, cnt, sdis, want, rcnt, rdis, INT32, servers) == 0
+    for ccl in (1024, 4096, 1 << 20):
+        rounds, entries, biggest = orc.alltoallv_staged_rounds(cnt, servers, INT32, ccl)
+        plan = H.describe_plan(H.COLL_ALLTOALLV, H.ALGO_PAIRWISE | (servers << 8), p, 0, INT32, ccl_bytes=ccl,
+                               tables=(cnt, sdis, rcnt, rdis))
+        assert len(plan["phases"]) == 2 + sum(rounds), (p, servers, ccl, rounds)
+        between = [st for ph in plan["phases"][3:] for st in ph]              # after stage one and the local runs
+        assert len(between) == entries, (p, servers, ccl)
+        at = 3
+        for i in range(1, servers):
+            for t in range(rounds[i]):
+                per_pair = {}
+                for st in plan["phases"][at + t]:
+                    a, d = st["a"][0], st["dst"][0]
+                    assert d % m == a % m and d // m == (a // m + i) % servers
+                    per_pair[(a, d)] = per_pair.get((a, d), 0) + st["n"]
+                assert max(per_pair.values()) <= ccl                         # a batch fits the buffer
+            at += rounds[i]
+        for fused in (False, True):
+            recvs = [np.full(n, -1, np.int32).view(np.uint8).copy() for n in rl]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, _bytes(sends), recvs, INT32, 0)
+            for r in range(p):
+                assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, servers, ccl, fused, r)
+
+
 def test_plan_rejects_bad_requests():
     with pytest.raises(H.HcclError):
         H.describe_plan(H.COLL_ALLREDUCE, RING, 0, 10, FP32)
