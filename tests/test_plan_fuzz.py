@@ -1,6 +1,8 @@
 """Seeded random walk over the planner's parameter space on the CPU: collective, schedule, rank count, size,
 buffer size, alignment, which ranks run in place, rank groups.  Integer sums, so the expected result needs no
 schedule: it is the plain numpy sum / concatenation / copy.  Both forms of every plan are interpreted."""
+import os
+
 import numpy as np
 import pytest
 
@@ -8,6 +10,8 @@ import plan_interp
 from closed_forms import INT32, SUM
 from hccl_loader import load
 
+# other random cases without touching the file: HCCL_AMD_TEST_SEED_SHIFT=1000 python -m pytest ...
+SEED_SHIFT = int(os.environ.get("HCCL_AMD_TEST_SEED_SHIFT", "0"))
 H = load()
 RING, MESH, RHD, MESH_ATOMIC = 0, 1, 2, 4
 
@@ -33,7 +37,7 @@ def _case(rng):
 
 @pytest.mark.parametrize("seed", range(8))
 def test_random_plans_compute_the_plain_result(seed):
-    rng = np.random.default_rng(7000 + seed)
+    rng = np.random.default_rng(7000 + SEED_SHIFT + seed)
     done = 0
     while done < 40:
         coll, p, n, align, ccl, algo, servers, rings, mask, root = _case(rng)
@@ -103,7 +107,7 @@ def test_random_alltoallv_plans_deliver_every_block(seed):
     """All-to-all-v with random counts (many of them zero), displacements in shuffled order with gaps, element
     sizes 1 to 8, flat and staged over every server count that divides the ranks: each block arrives where the
     receiver's table says, nothing else in the receive buffers changes, the send buffers stay as they were."""
-    rng = np.random.default_rng(9100 + seed)
+    rng = np.random.default_rng(9100 + SEED_SHIFT + seed)
     from closed_forms import INT8, INT16, INT64
     unit_of = {INT8: 1, INT16: 2, INT32: 4, INT64: 8}
     for case in range(25):
