@@ -261,12 +261,53 @@ def test_random_alltoallv_flat_and_staged(orc, seed):
             assert orc.alltoallv_staged(ins, cnt, sdis, want, cnt.T.copy(), rdis, dt, servers) == 0
         else:
             assert orc.alltoallv(ins, cnt, sdis, want, cnt.T.copy(), rdis, dt) == 0
-        print("random all-to-all-v seed", seed, "case", case, "p", p, "servers", servers, "dt", dt, "fuse", fuse, "max", big, flush=True)
-        g = gh.Group(p, fuse=fuse, servers=servers)
+        ccl = int(rng.choice([200 << 20, 1 << 16, 4096]))          # small buffers: blocks and runs travel in pieces
+        print("random all-to-all-v seed", seed, "case", case, "p", p, "servers", servers, "dt", dt, "fuse", fuse, "max", big,
+              "buffer", ccl, flush=True)
+        g = gh.Group(p, fuse=fuse, servers=servers, buffsize_bytes=ccl)
         try:
             outs = gh.all_to_all_v(g, ins, cnt, sdis, rl, cnt.T.copy(), rdis, dt, fill=0x5A)
             for r in range(p):
                 assert np.array_equal(outs[r], want[r]), (seed, case, r)
             assert g.info()["fused"] == fuse
+        finally:
+            g.close()
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_scatter_and_broadcast_over_rank_groups(orc, seed):
+    """Scatter and broadcast with random roots, rank groups and schedule settings (auto, ring, star): whatever the route,
+    rank r ends with the root's block r / with the root's buffer, the root's input stays as it was."""
+    rng = np.random.default_rng(5300 + SEED_SHIFT + seed)
+    for case in range(8):
+        p = int(rng.choice([2, 3, 4, 6, 8, 12, 16]))
+        servers = int(rng.choice([s for s in range(1, p + 1) if p % s == 0]))
+        setting = str(rng.choice(["auto", "ring", "star", "mesh", "rhd"]))
+        dt = int(rng.choice(ALL_TYPES))
+        n = _size(rng) // 4 + 1
+        fuse = int(rng.integers(0, 2))
+        root = int(rng.integers(0, p))
+        ccl = int(rng.choice([200 << 20, 1 << 16]))
+        print("random scatter / broadcast seed", seed, "case", case, "p", p, "servers", servers, "algo", setting, "type", dt,
+              "n", n, "fuse", fuse, "root", root, "buffer", ccl, flush=True)
+        g = gh.Group(p, algo=setting, fuse=fuse, servers=servers, buffsize_bytes=ccl)
+        try:
+            src = cf.random_input(dt, n * p, rng)
+            sends = [gh.to_dev(src) if r == root else None for r in range(p)]
+            recvs = [gh.empty_dev(n * H.DTYPE_SIZE[dt], fill=0x33) for _ in range(p)]
+            torch.cuda.synchronize()
+            H.scatter(g.comms, [t.data_ptr() if t is not None else None for t in sends], [t.data_ptr() for t in recvs],
+                      n, dt, root, g.stream_ptr)
+            g.stream.synchronize()
+            for r in range(p):
+                assert np.array_equal(gh.to_host(recvs[r], dt), src[r * n:(r + 1) * n]), (seed, case, "scatter", r)
+            assert np.array_equal(gh.to_host(sends[root], dt), src)
+            ins = [cf.random_input(dt, n, rng) for _ in range(p)]
+            bufs = [gh.to_dev(x) for x in ins]
+            torch.cuda.synchronize()
+            H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, dt, root, g.stream_ptr)
+            g.stream.synchronize()
+            for r in range(p):
+                assert np.array_equal(gh.to_host(bufs[r], dt), ins[root]), (seed, case, "broadcast", r)
         finally:
             g.close()
