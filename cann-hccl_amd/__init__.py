@@ -319,9 +319,24 @@ def barrier(comms, stream):
         _check("HcclBarrier", lib().HcclBarrier(c, stream))
 
 
+class _A2avTables(list):
+    """Rows of four host uint64 tables, as addresses; keeps the arrays they point into alive."""
+
+
 def a2av_tables(send_counts, sdispls, recv_counts, rdispls):
-    """Per rank, the four host uint64[p] arrays HcclAlltoAllV takes (build once, reuse across calls)."""
+    """Per rank, the four host uint64[p] arrays HcclAlltoAllV takes (build once, reuse across calls).  Sequences of
+    sequences or p x p numpy arrays (the latter cost no per-element conversion)."""
     p = len(send_counts)
+    try:
+        import numpy as np
+    except ImportError:
+        np = None
+    if np is not None and all(isinstance(t, np.ndarray) for t in (send_counts, sdispls, recv_counts, rdispls)):
+        keep = [np.ascontiguousarray(t, dtype=np.uint64) for t in (send_counts, sdispls, recv_counts, rdispls)]
+        base = [t.ctypes.data for t in keep]
+        out = _A2avTables([b + r * p * 8 for b in base] for r in range(p))
+        out.keep = keep
+        return out
     return [[(ctypes.c_uint64 * p)(*[int(x) for x in t[r]]) for t in (send_counts, sdispls, recv_counts, rdispls)]
             for r in range(p)]
 

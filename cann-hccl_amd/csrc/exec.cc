@@ -30,6 +30,10 @@ uint32_t DtypeSize(int dt)
 
 }  // namespace
 
+// Descriptor tables too large to ride in kernel arguments pass through a ring of pinned host buffers of this size.
+constexpr size_t kStageSlotBytes = size_t(128) << 10;
+constexpr uint32_t kStageSlots = 8;
+
 HcclResult EnsureDevice(Group *g, bool quiet)
 {
     if (g->deviceReady) {
@@ -52,6 +56,11 @@ HcclResult EnsureDevice(Group *g, bool quiet)
     }
     HIP_OK(hipEventCreateWithFlags(&g->doneEvent, hipEventDisableTiming));
     HIP_OK(hipStreamCreateWithFlags(&g->copyStream, hipStreamNonBlocking));
+    g->stageSlots.resize(kStageSlots);
+    for (StageSlot &slot : g->stageSlots) {
+        HIP_OK(hipHostMalloc(&slot.host, kStageSlotBytes, hipHostMallocDefault));
+        HIP_OK(hipEventCreateWithFlags(&slot.done, hipEventDisableTiming));
+    }
     g->scratch.assign(g->p, nullptr);
     g->arena.allocFn = [](size_t bytes) -> void * {
         void *mem = nullptr;
@@ -419,6 +428,7 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
         auto shortSegment = [&](const FusedItem &it) { return gather && movable(it, 8 * uint64_t(kGatherMaxBytes)); };
         if (gather) {
             std::vector<SegDesc> segs;
+            segs.reserve(pp->plan->fused.size());
             for (const FusedItem &it : pp->plan->fused) {
                 if (!shortSegment(it)) {
                     continue;
@@ -458,13 +468,16 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
             std::vector<uint32_t> opPool;      // stack items: one word per source-pool entry
             std::vector<void *> dstPool;
             uint32_t tiles = 0;
+            std::vector<char *> srcs, dsts;        // reused from item to item: an all-to-all-v has thousands
+            std::vector<uintptr_t> addrs;
             for (const FusedItem &it : pp->plan->fused) {
                 int want = it.kind == FK_TREE ? int(KK_TREE) : (it.kind == FK_STACK ? int(KK_STACK) : int(KK_CHAIN));
                 if (want != kind || shortSegment(it)) {
                     continue;
                 }
-                std::vector<char *> srcs, dsts;
-                std::vector<uintptr_t> addrs;
+                srcs.clear();
+                dsts.clear();
+                addrs.clear();
                 for (const Ref &d : it.dst) {
                     dsts.push_back(b.Ptr(d));
                     addrs.push_back(reinterpret_cast<uintptr_t>(dsts.back()));
@@ -562,6 +575,23 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
             pp->uploadStream = stream;
             pp->uploadComplete = false;
             pp->hostTables.swap(b.host);
+        } else if (b.host.size() <= kStageSlotBytes && stream != nullptr && !g->stageSlots.empty()) {
+            // medium tables (an all-to-all-v between 16 ranks: 40 KiB) go through a ring of pinned host buffers as an
+            // asynchronous copy on the caller's stream: the call does not wait for it.  A slot comes round again
+            // after as many collectives as the ring has slots; its previous copy has normally long finished.
+            StageSlot &slot = g->stageSlots[g->stageNext++ % g->stageSlots.size()];
+            if (slot.used) {
+                HIP_OK(hipEventSynchronize(slot.done));
+            }
+            std::memcpy(slot.host, b.host.data(), b.host.size());
+            HIP_OK(hipMemcpyAsync(pp->devTables, slot.host, b.host.size(), hipMemcpyHostToDevice, stream));
+            HIP_OK(hipEventRecord(slot.done, stream));
+            slot.used = true;
+            HIP_OK(hipEventCreateWithFlags(&pp->uploaded, hipEventDisableTiming));
+            HIP_OK(hipEventRecord(pp->uploaded, stream));
+            pp->uploadStream = stream;
+            pp->uploadComplete = false;
+            pp->hostTables.swap(b.host);
         } else {
             // over a stream of the library's own, which no caller captures (a plain copy goes through the null
             // stream, which a caller's capture of a blocking stream would not tolerate)
@@ -655,6 +685,18 @@ std::string CacheKey(const Group *g, int algo)
 // comes back with other buffers gets the plan from here and pays for the pointer tables only.
 int CachedPlan(Group *g, const PlanRequest &rq, std::shared_ptr<const Plan> *out, std::string *err)
 {
+    if (rq.coll == COLL_ALLTOALLV) {
+        // Its plan depends on four p x p tables, which callers like an expert-parallel layer change on every call:
+        // a key over the tables and a kept copy of the plan (megabytes at 64 ranks) would cost more than planning,
+        // which for this collective is a direct pass over the tables.  A call that does repeat finds the prepared
+        // collective in the group's cache before it gets here.
+        std::shared_ptr<Plan> fresh = std::make_shared<Plan>();
+        int rc = BuildPlan(rq, fresh.get(), err);
+        if (rc == 0) {
+            *out = fresh;
+        }
+        return rc;
+    }
     std::string key;
     auto put = [&](const void *p, size_t n) { key.append(static_cast<const char *>(p), n); };
     auto putVec = [&](const std::vector<uint64_t> &v) {
@@ -899,6 +941,14 @@ Group::~Group()
     }
     if (copyStream) {
         (void)hipStreamDestroy(copyStream);
+    }
+    for (StageSlot &slot : stageSlots) {
+        if (slot.done) {
+            (void)hipEventDestroy(slot.done);
+        }
+        if (slot.host) {
+            (void)hipHostFree(slot.host);
+        }
     }
     if (arena.freeFn != nullptr) {
         arena.FreeAll();

@@ -66,15 +66,69 @@ enum FusedKind : uint8_t {
 constexpr uint32_t kStackDepth = 8;
 constexpr uint32_t kStackMaxSrc = 64;
 
+// A vector whose first N elements live inside the object.  An all-to-all-v between 64 ranks is 4096 items of one
+// source and one destination each, planned anew whenever its tables change: with ordinary vectors the allocations of
+// those items were most of the planning time.
+template <typename T, uint32_t N> class SmallVec {
+public:
+    uint32_t size() const { return n_; }
+    bool empty() const { return n_ == 0; }
+    T *data() { return n_ <= N ? inl_ : heap_.data(); }
+    const T *data() const { return n_ <= N ? inl_ : heap_.data(); }
+    T *begin() { return data(); }
+    T *end() { return data() + n_; }
+    const T *begin() const { return data(); }
+    const T *end() const { return data() + n_; }
+    T &operator[](size_t i) { return data()[i]; }
+    const T &operator[](size_t i) const { return data()[i]; }
+    T &back() { return data()[n_ - 1]; }
+    void clear()
+    {
+        n_ = 0;
+        heap_.clear();
+    }
+    void push_back(const T &v)
+    {
+        if (n_ < N) {
+            inl_[n_++] = v;
+            return;
+        }
+        if (n_ == N) {
+            heap_.assign(inl_, inl_ + N);
+        }
+        heap_.push_back(v);
+        n_++;
+    }
+    template <typename It> void assign(It first, It last)
+    {
+        clear();
+        for (; first != last; ++first) {
+            push_back(*first);
+        }
+    }
+    void assign(size_t count, const T &v)
+    {
+        clear();
+        for (size_t i = 0; i < count; i++) {
+            push_back(v);
+        }
+    }
+
+private:
+    T inl_[N] = {};
+    uint32_t n_ = 0;
+    std::vector<T> heap_;
+};
+
 struct FusedItem {
     FusedKind kind = FK_COPY;
     uint64_t bytes = 0;
-    std::vector<Ref> src;
-    std::vector<uint8_t> srcValid;   // FK_TREE: second source of a leaf may be absent
-    std::vector<uint8_t> accLeft;    // FK_CHAIN: one flag per src (index 0 unused)
-    std::vector<uint16_t> ops;       // FK_STACK: one word per src
+    SmallVec<Ref, 2> src;
+    SmallVec<uint8_t, 4> srcValid;   // FK_TREE: second source of a leaf may be absent
+    SmallVec<uint8_t, 4> accLeft;    // FK_CHAIN: one flag per src (index 0 unused)
+    SmallVec<uint16_t, 2> ops;       // FK_STACK: one word per src
     uint32_t nleaf = 0;              // FK_TREE: leaves; FK_STACK: stack depth the program needs
-    std::vector<Ref> dst;
+    SmallVec<Ref, 2> dst;
 };
 
 struct PlanRequest {

@@ -130,6 +130,13 @@ struct P2PPending {
     hipStream_t stream = nullptr;
 };
 
+// A pinned host buffer that descriptor tables pass through on their way to the device.
+struct StageSlot {
+    void *host = nullptr;
+    hipEvent_t done = nullptr;      // recorded behind the slot's latest copy
+    bool used = false;
+};
+
 struct Group;
 
 struct Comm {
@@ -176,6 +183,8 @@ struct Group {
     std::vector<void *> idleScratch;      // outgrown scratch buffers that work in flight may still use; freed when the device is next known idle
     std::vector<std::unique_ptr<Prepared>> stale;         // collectives that left the cache while work in flight may still use them; same
     hipStream_t copyStream = nullptr;     // the library's own stream for table copies (non-blocking, never captured)
+    std::vector<StageSlot> stageSlots;    // ring of pinned buffers for tables too large to ride in kernel arguments
+    uint32_t stageNext = 0;
     void *barrierMem = nullptr;       // 2 x p small buffers for HcclBarrier's all-reduce
     void *noAllocBase = nullptr;      // this device's copy of the fixed workspace (noalloc.hip), looked up at set-up
     uint64_t scratchBytes = 0;

@@ -215,6 +215,65 @@ def test_staged_alltoallv_plan_batches_runs_larger_than_the_buffer(orc, p, serve
                 assert np.array_equal(recvs[r].view(np.int32), want[r]), (p, servers, ccl, fused, r)
 
 
+def _copy_items(plan):
+    """The fused copy items of a plan as (destination rank, offset, source rank, offset, bytes), neighbours joined."""
+    rows = sorted((d[0], d[2], it["src"][0][0], it["src"][0][2], it["n"]) for it in plan["fused"] for d in it["dst"])
+    out = []
+    for row in rows:
+        if out and out[-1][0] == row[0] and out[-1][2] == row[2] and out[-1][1] + out[-1][4] == row[1] and \
+                out[-1][3] + out[-1][4] == row[3]:
+            out[-1] = out[-1][:4] + (out[-1][4] + row[4],)
+        else:
+            out.append(row)
+    return out
+
+
+def test_block_moving_plans_take_the_short_cut_and_agree_with_the_general_path(orc):
+    # all-to-all-v, scatter and send / receive are planned by a direct pass over their blocks; with
+    # HCCL_AMD_PLAN_VERIFY=1 (read once per process, hence the child process) every request goes through the general
+    # planner with its symbolic verification: same phases, same bytes, the same blocks in the fused form
+    import json
+    import os
+    import subprocess
+    import sys
+    p = 6
+    cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 77, max_count=2000)
+    requests = [
+        dict(coll=H.COLL_ALLTOALLV, algo=H.ALGO_PAIRWISE, p=p, count=0, ccl_bytes=200 << 20, tables=True),
+        dict(coll=H.COLL_ALLTOALLV, algo=H.ALGO_PAIRWISE, p=p, count=0, ccl_bytes=1024, tables=True),
+        dict(coll=H.COLL_SCATTER, algo=2, p=p, count=1003, ccl_bytes=200 << 20, tables=False),
+        dict(coll=H.COLL_SCATTER, algo=2 | (3 << 21), p=p, count=1003, ccl_bytes=200 << 20, tables=False),
+    ]
+
+    def plans():
+        out = []
+        for rq in requests:
+            plan = H.describe_plan(rq["coll"], rq["algo"], rq["p"], rq["count"], INT32, ccl_bytes=rq["ccl_bytes"],
+                                   tables=(cnt, sdis, rcnt, rdis) if rq["tables"] else None)
+            steps = [sorted((st["dst"][0], st["dst"][2], st["a"][0], st["a"][2], st["n"]) for st in ph) for ph in plan["phases"]]
+            out.append(dict(steps=steps, items=_copy_items(plan), bytes=[plan[k] for k in ("stepRead", "stepWritten", "fusedRead",
+                                                                                         "fusedWritten", "scratchBytes")],
+                            fusedOk=plan["fusedOk"]))
+        return out
+
+    if os.environ.get("HCCL_AMD_PLAN_CHILD") == "1":
+        return plans()
+    here = plans()
+    code = ("import json, sys; sys.path.insert(0, %r); import test_plan_cpu as t; from oracle import oracle; "
+            "print('PLANS' + json.dumps(t.test_block_moving_plans_take_the_short_cut_and_agree_with_the_general_path(oracle)))"
+            % os.path.dirname(__file__))
+    env = dict(os.environ, HCCL_AMD_PLAN_VERIFY="1", HCCL_AMD_PLAN_CHILD="1")
+    env["PYTHONPATH"] = os.pathsep.join([os.path.dirname(os.path.dirname(__file__)), env.get("PYTHONPATH", "")])
+    res = subprocess.run([sys.executable, "-c", code], env=env, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr[-2000:]
+    there = json.loads(res.stdout[res.stdout.index("PLANS") + 5:])
+    for i, (a, b) in enumerate(zip(here, there)):
+        assert a["fusedOk"] and b["fusedOk"]
+        assert a["bytes"] == b["bytes"], (i, a["bytes"], b["bytes"])
+        assert [[list(x) for x in ph] for ph in a["steps"]] == b["steps"], i
+        assert [list(x) for x in a["items"]] == b["items"], i
+
+
 def test_plan_rejects_bad_requests():
     with pytest.raises(H.HcclError):
         H.describe_plan(H.COLL_ALLREDUCE, RING, 0, 10, FP32)
