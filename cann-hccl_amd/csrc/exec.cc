@@ -719,13 +719,47 @@ int CachedPlan(Group *g, const PlanRequest &rq, std::shared_ptr<const Plan> *out
         *out = it->second;
         return 0;
     }
-    std::shared_ptr<Plan> fresh = std::make_shared<Plan>();
-    int rc = BuildPlan(rq, fresh.get(), err);
-    if (rc != 0) {
-        return rc;
-    }
     if (g->planCache.size() >= 128) {
         g->planCache.clear();   // plans in use stay alive through the prepared collectives that hold them
+    }
+    // A new count of a request seen before: its plan is an earlier one's scaled, whenever the schedule is (counts that
+    // cut into whole slices).  Templates are kept per request-without-count, a few each.
+    std::string shape = key;
+    const uint64_t noCount = 0;
+    shape.replace(4 * sizeof(uint64_t), sizeof(uint64_t), reinterpret_cast<const char *>(&noCount), sizeof(uint64_t));   // head[4] = count
+    std::vector<TemplateSlot> &templates = g->planTemplates[shape];
+    std::shared_ptr<Plan> fresh = std::make_shared<Plan>();
+    for (TemplateSlot &t : templates) {
+        if (PlanFromTemplate(rq, *t.tmpl, fresh.get())) {
+            t.hits++;
+            g->planCache[key] = fresh;
+            *out = fresh;
+            return 0;
+        }
+    }
+    std::shared_ptr<PlanTemplate> made = std::make_shared<PlanTemplate>();
+    int rc = BuildPlanTemplate(rq, made.get(), err);
+    if (rc != 0) {
+        if (templates.empty()) {
+            g->planTemplates.erase(shape);
+        }
+        return rc;
+    }
+    *fresh = made->plan;
+    if (made->count != 0) {
+        if (g->planTemplates.size() > 64) {
+            g->planTemplates.clear();            // (invalidates `templates`)
+            g->planTemplates[shape].push_back(TemplateSlot{made, 0});
+        } else if (templates.size() < 4) {
+            templates.push_back(TemplateSlot{made, 0});
+        } else {
+            // the one that served least goes (a count with a ragged last slice serves no other count)
+            size_t worst = 0;
+            for (size_t i = 1; i < templates.size(); i++) {
+                worst = templates[i].hits < templates[worst].hits ? i : worst;
+            }
+            templates[worst] = TemplateSlot{made, 0};
+        }
     }
     g->planCache[key] = fresh;
     *out = fresh;

@@ -2261,6 +2261,124 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
     return 0;
 }
 
+namespace {
+
+bool Templatable(const PlanRequest &rq)
+{
+    return rq.count > 0 && rq.coll != COLL_ALLTOALLV && rq.vCounts.empty();
+}
+
+// The schedule as two flat lists: its shape and its numbers.
+void Fingerprint(const VProgram &vp, std::vector<uint64_t> *numbers, std::vector<uint32_t> *structure)
+{
+    numbers->clear();
+    structure->clear();
+    for (const std::vector<uint64_t> *v : {&vp.inBytes, &vp.outBytes, &vp.workBytes}) {
+        structure->push_back(uint32_t(v->size()));
+        numbers->insert(numbers->end(), v->begin(), v->end());
+    }
+    for (const Phase &ph : vp.phases) {
+        structure->push_back(uint32_t(ph.steps.size()));
+        for (const Step &st : ph.steps) {
+            structure->push_back(st.dst.rank << 8 | uint32_t(st.dst.buf) << 1 | (st.reduce ? 1u : 0u));
+            structure->push_back(st.a.rank << 8 | uint32_t(st.a.buf));
+            structure->push_back(st.reduce ? (st.b.rank << 8 | uint32_t(st.b.buf)) : 0u);
+            numbers->push_back(st.dst.off);
+            numbers->push_back(st.a.off);
+            numbers->push_back(st.reduce ? st.b.off : 0);
+            numbers->push_back(st.bytes);
+        }
+    }
+}
+
+PlanRequest Normalised(const PlanRequest &request)
+{
+    PlanRequest rq = request;
+    if (rq.algo == ALGO_MESH_ATOMIC) {
+        rq.algo = ALGO_MESH;
+        rq.meshAtomic = true;
+    }
+    return rq;
+}
+
+}  // namespace
+
+int BuildPlanTemplate(const PlanRequest &request, PlanTemplate *tmpl, std::string *err)
+{
+    tmpl->count = 0;
+    int rc = BuildPlan(request, &tmpl->plan, err);
+    if (rc != 0 || !Templatable(request)) {
+        return rc;
+    }
+    VProgram vp;
+    std::string ignored;
+    if (BuildVirtual(Normalised(request), &vp, &ignored) == 0) {
+        Fingerprint(vp, &tmpl->numbers, &tmpl->structure);
+        tmpl->count = request.count;
+    }
+    return 0;
+}
+
+bool PlanFromTemplate(const PlanRequest &request, const PlanTemplate &tmpl, Plan *plan)
+{
+    if (tmpl.count == 0 || !Templatable(request)) {
+        return false;
+    }
+    VProgram vp;
+    std::string ignored;
+    if (BuildVirtual(Normalised(request), &vp, &ignored) != 0) {
+        return false;
+    }
+    std::vector<uint64_t> numbers;
+    std::vector<uint32_t> structure;
+    Fingerprint(vp, &numbers, &structure);
+    if (structure != tmpl.structure || numbers.size() != tmpl.numbers.size()) {
+        return false;
+    }
+    typedef unsigned __int128 Wide;
+    const Wide c1 = request.count, c0 = tmpl.count;
+    for (size_t i = 0; i < numbers.size(); i++) {
+        if (Wide(numbers[i]) * c0 != Wide(tmpl.numbers[i]) * c1) {
+            return false;
+        }
+    }
+    // every number of the plan is a sum or difference of schedule numbers, so it scales with them (and comes out whole)
+    bool whole = true;
+    auto scale = [&](uint64_t &x) {
+        const Wide y = Wide(x) * c1;
+        whole = whole && y % c0 == 0;
+        x = uint64_t(y / c0);
+    };
+    *plan = tmpl.plan;
+    for (Phase &ph : plan->phases) {
+        for (Step &st : ph.steps) {
+            scale(st.dst.off);
+            scale(st.a.off);
+            scale(st.b.off);
+            scale(st.bytes);
+        }
+    }
+    for (FusedItem &it : plan->fused) {
+        scale(it.bytes);
+        for (Ref &r : it.src) {
+            scale(r.off);
+        }
+        for (Ref &r : it.dst) {
+            scale(r.off);
+        }
+    }
+    for (uint64_t &x : plan->sendBytes) {
+        scale(x);
+    }
+    for (uint64_t &x : plan->recvBytes) {
+        scale(x);
+    }
+    for (uint64_t *x : {&plan->scratchBytes, &plan->stepRead, &plan->stepWritten, &plan->fusedRead, &plan->fusedWritten}) {
+        scale(*x);
+    }
+    return whole;
+}
+
 std::string DescribePlan(const Plan &plan)
 {
     std::ostringstream os;

@@ -130,6 +130,12 @@ struct P2PPending {
     hipStream_t stream = nullptr;
 };
 
+// A plan kept as a template for other counts of the same request, and how often it served as one.
+struct TemplateSlot {
+    std::shared_ptr<const PlanTemplate> tmpl;
+    uint32_t hits = 0;
+};
+
 // A pinned host buffer that descriptor tables pass through on their way to the device.
 struct StageSlot {
     void *host = nullptr;
@@ -192,6 +198,7 @@ struct Group {
     std::unordered_map<std::string, std::unique_ptr<Prepared>> cache;   // keyed by request, settings and buffer addresses
     TableArena arena;
     std::unordered_map<std::string, std::shared_ptr<const Plan>> planCache;   // keyed by the plan request
+    std::unordered_map<std::string, std::vector<TemplateSlot>> planTemplates;   // keyed by the request without its count
     OpInfo lastInfo;
 
     ~Group();

@@ -417,6 +417,28 @@ def test_table_arena_keeps_blocks_of_collectives_recorded_into_a_callers_graph(t
     assert out.returncode == 0 and out.stdout.strip() == "OK", out.stdout
 
 
+def test_plans_derived_from_a_template_of_another_count_are_the_planners_own(tmp_path):
+    """A caller whose sizes change from call to call gets its plans by scaling an earlier plan of the same request
+    whenever the schedule scales (counts that cut into whole slices).  tests/c_abi/plan_template_check.cc holds every
+    derived plan against the plan made from scratch (21 schedules x 2 element sizes x in place or not x 10 x 10
+    counts), on the host, against cann-hccl_amd/csrc/plan.cc alone."""
+    import os
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        pytest.skip("no host C++ compiler")
+    exe = str(tmp_path / "plan_template_check")
+    subprocess.run([cxx, "-O2", "-std=c++17", "-Wall", "-Werror", "-I", os.path.join(root, "cann-hccl_amd", "csrc"),
+                    "-I", os.path.join(root, "include"), os.path.join(root, "tests", "c_abi", "plan_template_check.cc"),
+                    os.path.join(root, "cann-hccl_amd", "csrc", "plan.cc"), "-o", exe], check=True)
+    out = subprocess.run([exe], stdout=subprocess.PIPE, text=True)
+    assert out.returncode == 0 and out.stdout.startswith("OK"), out.stdout
+    derived = int(out.stdout.split()[3])
+    assert derived > 1000, out.stdout
+
+
 def _rank_table(path, servers, per_server, **edits):
     import json
     table = {"server_count": str(servers), "status": "completed", "version": "1.0", "server_list": []}

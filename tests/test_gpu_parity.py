@@ -1514,6 +1514,37 @@ def test_ring_allreduce_with_fewer_network_ports_than_ranks(orc):
             g.close()
 
 
+def test_sizes_that_change_from_call_to_call(orc):
+    # a new count on every call: the plan of a count that cuts into whole slices is an earlier plan scaled, a ragged
+    # count is planned from scratch; either way the result is the checker's
+    p = 8
+    for algo, dt in ((RING, FP32), (MESH_ATOMIC, BF16), (RHD, FP32)):
+        for fuse in (1, 0):
+            g = _group(p, algo, fuse=fuse)
+            try:
+                top = 64 * 1024 + 7
+                ins_all = _ins(dt, p, top, 720 + algo)
+                sends = [gh.to_dev(x) for x in ins_all]
+                recvs = [gh.empty_dev(top * H.DTYPE_SIZE[dt]) for _ in range(p)]
+                torch.cuda.synchronize()
+                for n in (8192, 16384, 8192 * 3, 8192 * 5, 1000, 8192 * 7, 12345, 8192 * 2, 64 * 1024, top):
+                    print("changing sizes", algo, "fuse", fuse, "n", n, flush=True)
+                    ins = [x[:n] for x in ins_all]
+                    want = orc.allreduce(ins, dt, SUM, algo=algo)
+                    H.all_reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, SUM, g.stream_ptr)
+                    g.stream.synchronize()
+                    for r in range(p):
+                        got = gh.to_host(recvs[r], dt)[:n]
+                        assert gh.same(dt, got, want[r]), (algo, fuse, n, r)
+                    want_rs = orc.reducescatter([x[:n // p * p] for x in ins_all], dt, SUM, algo=algo)
+                    H.reduce_scatter(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n // p, dt, SUM, g.stream_ptr)
+                    g.stream.synchronize()
+                    for r in range(p):
+                        assert gh.same(dt, gh.to_host(recvs[r], dt)[:n // p], want_rs[r]), (algo, fuse, n, "reduce-scatter", r)
+            finally:
+                g.close()
+
+
 def test_two_hundred_buffer_sets(orc):
     # A caller that comes with other buffers every time: every call is a miss of the prepared-collective cache (the
     # plan itself is shared), tables travel with the call, no graph is built until a buffer set comes back, and a
