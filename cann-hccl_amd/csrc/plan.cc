@@ -1656,21 +1656,25 @@ std::vector<OutRange> Outputs(const Sym &sym, uint32_t p)
     return v;
 }
 
-// Text that identifies the final receive-buffer contents independently of how ranges were split.
+// Numbers that identify the final receive-buffer contents independently of how ranges were split.
 // Ranges of an in-place rank that still hold their original bytes (never written) are left out: the
 // same memory seen as "send buffer" is not an output.
-std::string OutputSignature(const Sym &sym, uint32_t p, const std::vector<uint8_t> &alias)
+std::vector<uint64_t> OutputSignature(const Sym &sym, const std::vector<OutRange> &outs, const std::vector<uint8_t> &alias)
 {
-    std::string sig;
-    for (const OutRange &o : Outputs(sym, p)) {
+    std::vector<uint64_t> sig;
+    sig.reserve(outs.size() * 5);
+    for (const OutRange &o : outs) {
         const ENode &n = sym.nodes[o.expr];
         bool untouched = !n.red && n.leaf.rank == o.rank && n.leaf.buf == BUF_SEND && n.leaf.off + o.delta == o.start &&
             o.rank < alias.size() && alias[o.rank];
         if (untouched) {
             continue;
         }
-        sig += "r" + std::to_string(o.rank) + "@" + std::to_string(o.start) + "+" + std::to_string(o.len) + "=" +
-            std::to_string(o.shape) + ":" + std::to_string(o.rel) + ";";
+        sig.push_back(o.rank);
+        sig.push_back(o.start);
+        sig.push_back(o.len);
+        sig.push_back(uint64_t(o.shape));
+        sig.push_back(uint64_t(o.rel));
     }
     return sig;
 }
@@ -1828,9 +1832,8 @@ bool AsStack(const Sym &sym, int e, uint64_t delta, FusedItem *item)
     return true;
 }
 
-bool BuildFused(const Sym &sym, const PlanRequest &rq, std::vector<FusedItem> *items)
+bool BuildFused(const Sym &sym, const std::vector<OutRange> &outs, const PlanRequest &rq, std::vector<FusedItem> *items)
 {
-    std::vector<OutRange> outs = Outputs(sym, rq.p);
     std::map<std::tuple<uint64_t, int, int64_t>, size_t> index;   // (length, shape, leftmost source offset)
     for (const OutRange &o : outs) {
         auto key = std::make_tuple(o.len, o.shape, o.abs);
@@ -2145,7 +2148,8 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
         *err = "virtual program: " + ref.err;
         return 2;
     }
-    std::string want = OutputSignature(ref, p, alias);
+    const std::vector<OutRange> refOuts = Outputs(ref, p);   // shared by the comparison below and by the fused form
+    const std::vector<uint64_t> want = OutputSignature(ref, refOuts, alias);
 
     // lowering candidates: partials in the receive buffer (no scratch), else in scratch, else staged
     bool fits = vp.workBytes.empty();
@@ -2187,7 +2191,7 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
             why = s.err;
             continue;
         }
-        if (OutputSignature(s, p, alias) != want) {
+        if (OutputSignature(s, Outputs(s, p), alias) != want) {
             why = "lowered program computes different outputs";
             continue;
         }
@@ -2223,7 +2227,7 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
 
     // fused form, derived from the virtual program's expressions (leaves are send-buffer ranges)
     plan->fused.clear();
-    plan->fusedOk = BuildFused(ref, rq, &plan->fused);
+    plan->fusedOk = BuildFused(ref, refOuts, rq, &plan->fused);
     plan->fusedRead = plan->fusedWritten = 0;
     if (plan->fusedOk) {
         for (FusedItem &it : plan->fused) {
