@@ -831,6 +831,9 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                     for (uint32_t k = 0; k < m; k++) {
                         const uint32_t src = c * m + k;
                         const uint64_t n = len(src, j);
+                        if (n) {
+                            vp->blocks.push_back(VProgram::Block{rq.rdispls[size_t(j) * p + src] * u, rq.sdispls[size_t(src) * p + j] * u, n, j, src});
+                        }
                         // stage one: own blocks first (LocalCopy), the neighbours' all at once (alltoallv_staged_mesh.cc:51-130)
                         EmitCopy(*vp, k == l ? 0 : 1, MkRef(r, BUF_SEND, at), MkRef(src, BUF_SEND, rq.sdispls[size_t(src) * p + j] * u), n);
                         // stage two: step i hands the run for server c + i to the rank of that server with local index l
@@ -2002,7 +2005,10 @@ bool DirectCopyPlan(VProgram &vp, const PlanRequest &rq, const std::vector<uint8
         const char *e = std::getenv("HCCL_AMD_PLAN_VERIFY");
         return e != nullptr && e[0] != '\0' && e[0] != '0';
     }();
-    if (verifyAll || rq.stageInput || !vp.workBytes.empty() ||
+    // A schedule with a workspace qualifies when it lists its whole blocks itself (the staged all-to-all-v: blocks rest
+    // in the gathering rank's workspace between the two stages).
+    const bool viaWorkspace = !vp.workBytes.empty();
+    if (verifyAll || rq.stageInput || (viaWorkspace && vp.blocks.empty()) ||
         (rq.coll != COLL_ALLTOALLV && rq.coll != COLL_SCATTER && rq.coll != COLL_SENDRECV)) {
         return false;
     }
@@ -2012,16 +2018,25 @@ bool DirectCopyPlan(VProgram &vp, const PlanRequest &rq, const std::vector<uint8
         }
     }
     typedef VProgram::Block Block;
-    uint64_t moved = 0;
+    uint64_t stepped = 0;
+    auto inWorkspace = [&](const Ref &r) { return viaWorkspace && r.buf == BUF_SEND && r.off >= vp.inBytes[r.rank]; };
     for (const Phase &ph : vp.phases) {
         for (const Step &st : ph.steps) {
-            if (st.reduce || st.a.buf != BUF_SEND || st.dst.buf != BUF_RECV || st.a.rank >= rq.p || st.dst.rank >= rq.p) {
+            if (st.reduce || st.a.buf != BUF_SEND || st.a.rank >= rq.p || st.dst.rank >= rq.p ||
+                !(st.dst.buf == BUF_RECV || inWorkspace(st.dst))) {
                 return false;
             }
-            moved += st.bytes;
+            stepped += st.bytes;
         }
     }
     std::vector<Block> &blocks = vp.blocks;
+    bool grouped = true;
+    for (size_t i = 1; i < blocks.size() && grouped; i++) {
+        grouped = blocks[i - 1].dstRank <= blocks[i].dstRank;
+    }
+    if (!grouped) {
+        std::stable_sort(blocks.begin(), blocks.end(), [](const Block &x, const Block &y) { return x.dstRank < y.dstRank; });
+    }
     if (blocks.empty()) {
         // no list of whole blocks: the steps are the blocks, those that continue one another joined
         for (const Phase &ph : vp.phases) {
@@ -2069,15 +2084,35 @@ bool DirectCopyPlan(VProgram &vp, const PlanRequest &rq, const std::vector<uint8
         }
         i = j;
     }
+    uint64_t moved = 0;
+    for (const Block &b : blocks) {
+        moved += b.bytes;
+    }
     plan->phases.clear();
     plan->phases.reserve(vp.phases.size());
-    for (Phase &vph : vp.phases) {
-        if (!vph.steps.empty()) {
-            plan->phases.push_back(std::move(vph));
-        }
-    }
     plan->scratchBytes = 0;
-    plan->stepRead = plan->stepWritten = plan->fusedRead = plan->fusedWritten = moved;
+    for (Phase &vph : vp.phases) {
+        if (vph.steps.empty()) {
+            continue;
+        }
+        if (viaWorkspace) {
+            // the workspace lies in the library's scratch buffer behind the rank's input, as the general lowering puts it
+            for (Step &st : vph.steps) {
+                if (inWorkspace(st.a)) {
+                    st.a.buf = BUF_SCRATCH;
+                }
+                if (st.dst.buf == BUF_SEND) {
+                    st.dst.buf = BUF_SCRATCH;
+                }
+            }
+        }
+        plan->phases.push_back(std::move(vph));
+    }
+    for (uint32_t r = 0; viaWorkspace && r < rq.p; r++) {
+        plan->scratchBytes = std::max(plan->scratchBytes, vp.inBytes[r] + vp.workBytes[r]);
+    }
+    plan->stepRead = plan->stepWritten = stepped;
+    plan->fusedRead = plan->fusedWritten = moved;
     // fused: a block that the schedule moved in pieces is one item again
     plan->fused.clear();
     plan->fused.reserve(blocks.size());

@@ -241,6 +241,8 @@ def test_block_moving_plans_take_the_short_cut_and_agree_with_the_general_path(o
     requests = [
         dict(coll=H.COLL_ALLTOALLV, algo=H.ALGO_PAIRWISE, p=p, count=0, ccl_bytes=200 << 20, tables=True),
         dict(coll=H.COLL_ALLTOALLV, algo=H.ALGO_PAIRWISE, p=p, count=0, ccl_bytes=1024, tables=True),
+        dict(coll=H.COLL_ALLTOALLV, algo=H.ALGO_PAIRWISE | (2 << 8), p=p, count=0, ccl_bytes=200 << 20, tables=True),   # staged, 2 x 3
+        dict(coll=H.COLL_ALLTOALLV, algo=H.ALGO_PAIRWISE | (3 << 8), p=p, count=0, ccl_bytes=2048, tables=True),       # staged in batches
         dict(coll=H.COLL_SCATTER, algo=2, p=p, count=1003, ccl_bytes=200 << 20, tables=False),
         dict(coll=H.COLL_SCATTER, algo=2 | (3 << 21), p=p, count=1003, ccl_bytes=200 << 20, tables=False),
     ]
