@@ -1451,17 +1451,24 @@ struct Sym {
     mutable std::vector<int> shapeOf;        // per node, -1 = not computed yet
     mutable std::vector<int64_t> baseOf;     // offset of the node's leftmost leaf at delta 0
     std::vector<ENode> nodes;
-    std::map<std::pair<uint32_t, uint8_t>, std::map<uint64_t, Region>> mem;
+    std::vector<std::map<uint64_t, Region>> mem;   // per (rank, buffer): index rank * 3 + buffer, grown on demand
     std::vector<uint8_t> alias;
     std::string err;
 
-    std::pair<uint32_t, uint8_t> Key(const Ref &r) const
+    size_t Key(const Ref &r) const
     {
         uint8_t b = r.buf;
         if (b == BUF_SEND && r.rank < alias.size() && alias[r.rank]) {
             b = BUF_RECV;
         }
-        return std::make_pair(r.rank, b);
+        return size_t(r.rank) * 3 + b;
+    }
+    std::map<uint64_t, Region> &Mem(size_t key)
+    {
+        if (mem.size() <= key) {
+            mem.resize(key + 1);
+        }
+        return mem[key];
     }
     void Init(uint32_t rank, uint64_t bytes)
     {
@@ -1474,14 +1481,14 @@ struct Sym {
         Region rg;
         rg.len = bytes;
         rg.expr = int(nodes.size()) - 1;
-        mem[Key(MkRef(rank, BUF_SEND, 0))][0] = rg;
+        Mem(Key(MkRef(rank, BUF_SEND, 0)))[0] = rg;
     }
     bool Read(const Ref &ref, uint64_t len, std::vector<Piece> *out)
     {
-        auto mit = mem.find(Key(ref));
+        const size_t key = Key(ref);
         uint64_t pos = ref.off, end = ref.off + len;
-        if (mit != mem.end()) {
-            auto &m = mit->second;
+        if (key < mem.size()) {
+            auto &m = mem[key];
             auto it = m.upper_bound(pos);
             if (it != m.begin()) {
                 --it;
@@ -1509,7 +1516,7 @@ struct Sym {
     }
     void Write(const Ref &ref, const std::vector<Piece> &pieces, uint64_t len)
     {
-        auto &m = mem[Key(ref)];
+        auto &m = Mem(Key(ref));
         uint64_t b = ref.off, e = ref.off + len;
         auto it = m.upper_bound(b);
         if (it != m.begin()) {
@@ -1550,13 +1557,17 @@ struct Sym {
     {
         for (const Phase &ph : phases) {
             std::vector<std::tuple<Ref, std::vector<Piece>, uint64_t>> writes;
+            writes.reserve(ph.steps.size());
+            std::vector<Piece> pa, pb, res;    // reused from step to step
             for (const Step &s : ph.steps) {
-                std::vector<Piece> pa, pb, res;
+                pa.clear();
+                pb.clear();
+                res.clear();
                 if (!Read(s.a, s.bytes, &pa)) {
                     return false;
                 }
                 if (!s.reduce) {
-                    res = pa;
+                    res.swap(pa);
                 } else {
                     if (!Read(s.b, s.bytes, &pb)) {
                         return false;
@@ -1583,7 +1594,7 @@ struct Sym {
                         }
                     }
                 }
-                writes.emplace_back(s.dst, std::move(res), s.bytes);
+                writes.emplace_back(s.dst, res, s.bytes);
             }
             for (auto &w : writes) {
                 Write(std::get<0>(w), std::get<1>(w), std::get<2>(w));
@@ -1633,11 +1644,11 @@ std::vector<OutRange> Outputs(const Sym &sym, uint32_t p)
 {
     std::vector<OutRange> v;
     for (uint32_t r = 0; r < p; r++) {
-        auto it = sym.mem.find(std::make_pair(r, uint8_t(BUF_RECV)));
-        if (it == sym.mem.end()) {
+        const size_t key = size_t(r) * 3 + BUF_RECV;
+        if (key >= sym.mem.size()) {
             continue;
         }
-        for (auto &kv : it->second) {
+        for (auto &kv : sym.mem[key]) {
             OutRange o;
             o.rank = r;
             o.start = kv.first;
@@ -1914,6 +1925,7 @@ bool PhaseIsHazardFree(const Phase &ph, const std::vector<uint8_t> &alias, std::
 {
     struct Acc { uint32_t rank; uint8_t buf; uint64_t off, len; size_t step; bool write; };
     std::vector<Acc> acc;
+    acc.reserve(ph.steps.size() * 3);
     auto phys = [&](const Ref &r) { return (r.buf == BUF_SEND && r.rank < alias.size() && alias[r.rank]) ? uint8_t(BUF_RECV) : r.buf; };
     for (size_t i = 0; i < ph.steps.size(); i++) {
         const Step &s = ph.steps[i];
