@@ -521,6 +521,9 @@ def main():
             "kernel": "%s<float, sum> (fused %s all-reduce, the library default): %d algorithmic bytes per launch "
                       "(%d x %.0f MiB read + the same written), average launch %.4f ms over %d launches, HIP events on "
                       "the launching stream" % (fused_kernel, sched_name, actual, p, args.size_mib, dev_ms, args.steps),
+            "shape_ceiling": "a plain kernel that only reads 8 streams and writes 8 (no tables, no arithmetic) reaches 5.4-5.7 TB/s "
+                             "on this part, read-only 7.0, write-only 6.5 (profiles/hbm_probe__plain_kernels_256MiB_streams.txt; "
+                             "write-path counters in profiles/ChainKernel__write_path_counters_8ranks_256MiB.txt)" if headline else None,
         },
         "roofline_steps": {
             "bound": "hbm", "achieved": round(s_achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
