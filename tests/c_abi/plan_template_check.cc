@@ -16,6 +16,7 @@ int main()
     struct Shape {
         int coll, algo;
         uint32_t p, servers, level0;
+        uint32_t nicMask = 0;
     };
     const std::vector<Shape> shapes = {
         {COLL_ALLREDUCE, ALGO_RING, 8, 1, 0}, {COLL_ALLREDUCE, ALGO_MESH, 4, 1, 0}, {COLL_ALLREDUCE, ALGO_MESH_ATOMIC, 8, 1, 0},
@@ -25,6 +26,8 @@ int main()
         {COLL_BROADCAST, ALGO_RING, 8, 1, 0}, {COLL_BROADCAST, ALGO_MESH, 8, 2, 0}, {COLL_BROADCAST, ALGO_RHD, 5, 1, 0},
         {COLL_REDUCE, ALGO_RING, 8, 1, 0}, {COLL_REDUCE, ALGO_MESH, 4, 1, 0}, {COLL_REDUCE, ALGO_RHD, 8, 2, 0},
         {COLL_SCATTER, ALGO_MESH, 8, 1, 0}, {COLL_SCATTER, ALGO_RING, 6, 1, 0}, {COLL_SCATTER, ALGO_MESH, 8, 2, 0},
+        {COLL_ALLREDUCE, ALGO_RING, 8, 1, 4}, {COLL_ALLREDUCE, ALGO_RHD, 16, 2, 4}, {COLL_ALLREDUCE, ALGO_RING, 8, 1, 0, 0x11},
+        {COLL_ALLREDUCE, ALGO_RING, 8, 1, 0, 0x04}, {COLL_BROADCAST, ALGO_STAR, 5, 1, 0}, {COLL_REDUCESCATTER, ALGO_RING, 16, 2, 4},
     };
     for (const Shape &sh : shapes) {
         for (uint32_t unit : {4u, 2u}) {
@@ -35,6 +38,7 @@ int main()
                 base.p = sh.p;
                 base.servers = sh.servers;
                 base.level0Rings = sh.level0;
+                base.nicMask = sh.nicMask;
                 base.unit = unit;
                 base.root = sh.p - 1;
                 base.cclBytes = 16 << 20;
@@ -87,7 +91,7 @@ int main()
                         }
                         // (collectives that cut the count into aligned slices; the per-rank-block ones scale at any count)
                         const bool slices = sh.coll == COLL_ALLREDUCE || (sh.coll == COLL_REDUCE && sh.algo != ALGO_RING) ||
-                            (sh.coll == COLL_BROADCAST && sh.algo != ALGO_RHD);
+                            (sh.coll == COLL_BROADCAST && sh.algo != ALGO_RHD && sh.algo != ALGO_STAR);
                         if (c0 == regular && c1 == regular + 1 && slices && ok) {
                             printf("a ragged count was derived from a whole one: coll %d algo %d p %u\n", sh.coll, sh.algo, sh.p);
                             return 1;

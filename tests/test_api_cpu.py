@@ -420,7 +420,7 @@ def test_table_arena_keeps_blocks_of_collectives_recorded_into_a_callers_graph(t
 def test_plans_derived_from_a_template_of_another_count_are_the_planners_own(tmp_path):
     """A caller whose sizes change from call to call gets its plans by scaling an earlier plan of the same request
     whenever the schedule scales (counts that cut into whole slices).  tests/c_abi/plan_template_check.cc holds every
-    derived plan against the plan made from scratch (21 schedules x 2 element sizes x in place or not x 10 x 10
+    derived plan against the plan made from scratch (27 schedules x 2 element sizes x in place or not x 10 x 10
     counts), on the host, against cann-hccl_amd/csrc/plan.cc alone."""
     import os
     import shutil
