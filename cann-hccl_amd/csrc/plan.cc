@@ -2319,29 +2319,6 @@ bool Templatable(const PlanRequest &rq)
     return rq.count > 0 && rq.coll != COLL_ALLTOALLV && rq.vCounts.empty();
 }
 
-// The schedule as two flat lists: its shape and its numbers.
-void Fingerprint(const VProgram &vp, std::vector<uint64_t> *numbers, std::vector<uint32_t> *structure)
-{
-    numbers->clear();
-    structure->clear();
-    for (const std::vector<uint64_t> *v : {&vp.inBytes, &vp.outBytes, &vp.workBytes}) {
-        structure->push_back(uint32_t(v->size()));
-        numbers->insert(numbers->end(), v->begin(), v->end());
-    }
-    for (const Phase &ph : vp.phases) {
-        structure->push_back(uint32_t(ph.steps.size()));
-        for (const Step &st : ph.steps) {
-            structure->push_back(st.dst.rank << 8 | uint32_t(st.dst.buf) << 1 | (st.reduce ? 1u : 0u));
-            structure->push_back(st.a.rank << 8 | uint32_t(st.a.buf));
-            structure->push_back(st.reduce ? (st.b.rank << 8 | uint32_t(st.b.buf)) : 0u);
-            numbers->push_back(st.dst.off);
-            numbers->push_back(st.a.off);
-            numbers->push_back(st.reduce ? st.b.off : 0);
-            numbers->push_back(st.bytes);
-        }
-    }
-}
-
 PlanRequest Normalised(const PlanRequest &request)
 {
     PlanRequest rq = request;
@@ -2351,6 +2328,8 @@ PlanRequest Normalised(const PlanRequest &request)
     }
     return rq;
 }
+
+bool SameOffsets(const Step &st) { return st.dst.off == st.a.off && (!st.reduce || st.b.off == st.a.off); }
 
 }  // namespace
 
@@ -2363,10 +2342,42 @@ int BuildPlanTemplate(const PlanRequest &request, PlanTemplate *tmpl, std::strin
     }
     VProgram vp;
     std::string ignored;
-    if (BuildVirtual(Normalised(request), &vp, &ignored) == 0) {
-        Fingerprint(vp, &tmpl->numbers, &tmpl->structure);
-        tmpl->count = request.count;
+    if (BuildVirtual(Normalised(request), &vp, &ignored) != 0) {
+        return 0;
     }
+    tmpl->schedule = std::move(vp.phases);
+    tmpl->inBytes = vp.inBytes;
+    tmpl->outBytes = vp.outBytes;
+    tmpl->workBytes = vp.workBytes;
+    tmpl->workspace = !vp.workBytes.empty();
+    // position by position: every step, of the schedule and of the plan, touches one offset in all its buffers, every
+    // fused item likewise, and every buffer in use is as long as the count
+    bool pw = !tmpl->workspace &&
+        (request.coll == COLL_ALLREDUCE || request.coll == COLL_BROADCAST || request.coll == COLL_REDUCE);
+    const uint64_t extent = request.count * request.unit;
+    for (const std::vector<uint64_t> *v : {&tmpl->inBytes, &tmpl->outBytes, &tmpl->plan.sendBytes, &tmpl->plan.recvBytes}) {
+        for (uint64_t x : *v) {
+            pw = pw && (x == 0 || x == extent);
+        }
+    }
+    pw = pw && (tmpl->plan.scratchBytes == 0 || tmpl->plan.scratchBytes == extent);
+    for (const std::vector<Phase> *phases : {&tmpl->schedule, &tmpl->plan.phases}) {
+        for (const Phase &ph : *phases) {
+            for (const Step &st : ph.steps) {
+                pw = pw && SameOffsets(st) && st.dst.off + st.bytes <= extent;
+            }
+        }
+    }
+    for (const FusedItem &it : tmpl->plan.fused) {
+        for (size_t k = 0; k < it.src.size(); k++) {
+            pw = pw && (!it.srcValid[k] || it.src[k].off == it.dst[0].off);
+        }
+        for (const Ref &d : it.dst) {
+            pw = pw && d.off == it.dst[0].off && d.off + it.bytes <= extent;
+        }
+    }
+    tmpl->positionWise = pw;
+    tmpl->count = request.count;
     return 0;
 }
 
@@ -2377,56 +2388,136 @@ bool PlanFromTemplate(const PlanRequest &request, const PlanTemplate &tmpl, Plan
     }
     VProgram vp;
     std::string ignored;
-    if (BuildVirtual(Normalised(request), &vp, &ignored) != 0) {
-        return false;
-    }
-    std::vector<uint64_t> numbers;
-    std::vector<uint32_t> structure;
-    Fingerprint(vp, &numbers, &structure);
-    if (structure != tmpl.structure || numbers.size() != tmpl.numbers.size()) {
+    if (BuildVirtual(Normalised(request), &vp, &ignored) != 0 || vp.workBytes.empty() == tmpl.workspace) {
         return false;
     }
     typedef unsigned __int128 Wide;
-    const Wide c1 = request.count, c0 = tmpl.count;
-    for (size_t i = 0; i < numbers.size(); i++) {
-        if (Wide(numbers[i]) * c0 != Wide(tmpl.numbers[i]) * c1) {
+    // The factor: the longest step of the new schedule over the longest of the template's (a whole slice on both
+    // sides whenever there is one; if the guess is wrong the comparison below fails and nothing is derived).
+    uint64_t num = 0, den = 0;
+    for (const Phase &ph : vp.phases) {
+        for (const Step &st : ph.steps) {
+            num = std::max(num, st.bytes);
+        }
+    }
+    for (const Phase &ph : tmpl.schedule) {
+        for (const Step &st : ph.steps) {
+            den = std::max(den, st.bytes);
+        }
+    }
+    if (num == 0 || den == 0) {
+        return false;
+    }
+    const bool cut = tmpl.positionWise;
+    const uint64_t extent = request.count * request.unit;
+    bool whole = true;
+    auto scaled = [&](uint64_t x) {
+        const Wide y = Wide(x) * num;
+        whole = whole && y % den == 0;
+        return uint64_t(y / den);
+    };
+    // length of a range that starts at (scaled) offset `at` and had (scaled) length `len`: cut off at the extent
+    auto kept = [&](uint64_t at, uint64_t len) { return !cut ? len : (at >= extent ? 0 : std::min(len, extent - at)); };
+    // 1. the new schedule is the template's, scaled and cut off
+    if (vp.inBytes.size() != tmpl.inBytes.size() || vp.outBytes.size() != tmpl.outBytes.size() ||
+        vp.phases.size() > tmpl.schedule.size()) {
+        return false;
+    }
+    for (size_t r = 0; r < vp.inBytes.size(); r++) {
+        if (vp.inBytes[r] != kept(0, scaled(tmpl.inBytes[r])) || vp.outBytes[r] != kept(0, scaled(tmpl.outBytes[r]))) {
             return false;
         }
     }
-    // every number of the plan is a sum or difference of schedule numbers, so it scales with them (and comes out whole)
-    bool whole = true;
-    auto scale = [&](uint64_t &x) {
-        const Wide y = Wide(x) * c1;
-        whole = whole && y % c0 == 0;
-        x = uint64_t(y / c0);
-    };
-    *plan = tmpl.plan;
-    for (Phase &ph : plan->phases) {
-        for (Step &st : ph.steps) {
-            scale(st.dst.off);
-            scale(st.a.off);
-            scale(st.b.off);
-            scale(st.bytes);
+    if (vp.workBytes.size() != tmpl.workBytes.size()) {
+        return false;
+    }
+    for (size_t r = 0; r < vp.workBytes.size(); r++) {
+        if (vp.workBytes[r] != scaled(tmpl.workBytes[r])) {
+            return false;
         }
     }
-    for (FusedItem &it : plan->fused) {
-        scale(it.bytes);
+    for (size_t i = 0; i < tmpl.schedule.size(); i++) {
+        static const Phase none;
+        const Phase &fresh = i < vp.phases.size() ? vp.phases[i] : none;
+        size_t at = 0;
+        for (const Step &t : tmpl.schedule[i].steps) {
+            const uint64_t dst = scaled(t.dst.off), a = scaled(t.a.off), b = t.reduce ? scaled(t.b.off) : 0;
+            const uint64_t bytes = kept(dst, scaled(t.bytes));
+            if (bytes == 0) {
+                continue;
+            }
+            if (at >= fresh.steps.size()) {
+                return false;
+            }
+            const Step &f = fresh.steps[at++];
+            if (f.reduce != t.reduce || f.bytes != bytes || f.dst.rank != t.dst.rank || f.dst.buf != t.dst.buf || f.dst.off != dst ||
+                f.a.rank != t.a.rank || f.a.buf != t.a.buf || f.a.off != a ||
+                (t.reduce && (f.b.rank != t.b.rank || f.b.buf != t.b.buf || f.b.off != b))) {
+                return false;
+            }
+        }
+        if (at != fresh.steps.size()) {
+            return false;
+        }
+    }
+    if (!whole) {
+        return false;
+    }
+    // 2. so its plan is the template's plan, scaled and cut off the same way (every number of the plan is a sum or
+    // difference of schedule numbers, so it scales with them and comes out whole)
+    plan->p = tmpl.plan.p;
+    plan->fusedOk = tmpl.plan.fusedOk;
+    plan->phases.clear();
+    plan->fused.clear();
+    plan->stepRead = plan->stepWritten = plan->fusedRead = plan->fusedWritten = 0;
+    for (const Phase &tph : tmpl.plan.phases) {
+        Phase ph;
+        ph.steps.reserve(tph.steps.size());
+        for (const Step &t : tph.steps) {
+            Step st = t;
+            st.dst.off = scaled(t.dst.off);
+            st.a.off = scaled(t.a.off);
+            st.b.off = scaled(t.b.off);
+            st.bytes = kept(st.dst.off, scaled(t.bytes));
+            if (st.bytes == 0) {
+                continue;
+            }
+            plan->stepRead += st.bytes * (st.reduce ? 2 : 1);
+            plan->stepWritten += st.bytes;
+            ph.steps.push_back(st);
+        }
+        if (!ph.steps.empty()) {
+            plan->phases.push_back(std::move(ph));
+        }
+    }
+    for (const FusedItem &t : tmpl.plan.fused) {
+        FusedItem it = t;
         for (Ref &r : it.src) {
-            scale(r.off);
+            r.off = scaled(r.off);
         }
         for (Ref &r : it.dst) {
-            scale(r.off);
+            r.off = scaled(r.off);
+        }
+        it.bytes = kept(it.dst.empty() ? 0 : it.dst[0].off, scaled(t.bytes));
+        if (it.bytes == 0) {
+            continue;
+        }
+        uint64_t nsrc = 0;
+        for (uint8_t v : it.srcValid) {
+            nsrc += v;
+        }
+        plan->fusedRead += nsrc * it.bytes;
+        plan->fusedWritten += uint64_t(it.dst.size()) * it.bytes;
+        plan->fused.push_back(std::move(it));
+    }
+    plan->sendBytes = tmpl.plan.sendBytes;
+    plan->recvBytes = tmpl.plan.recvBytes;
+    for (std::vector<uint64_t> *v : {&plan->sendBytes, &plan->recvBytes}) {
+        for (uint64_t &x : *v) {
+            x = kept(0, scaled(x));
         }
     }
-    for (uint64_t &x : plan->sendBytes) {
-        scale(x);
-    }
-    for (uint64_t &x : plan->recvBytes) {
-        scale(x);
-    }
-    for (uint64_t *x : {&plan->scratchBytes, &plan->stepRead, &plan->stepWritten, &plan->fusedRead, &plan->fusedWritten}) {
-        scale(*x);
-    }
+    plan->scratchBytes = kept(0, scaled(tmpl.plan.scratchBytes));
     return whole;
 }
 

@@ -176,23 +176,31 @@ int BuildPlan(const PlanRequest &req, Plan *plan, std::string *err);
 
 // A plan together with what is needed to derive from it the plan of the same request with another count.
 // Everything the planner does after laying out the schedule compares, adds and subtracts byte offsets and nothing
-// else, so when the schedule of a request is the template's with every offset and length multiplied by
-// count / template count (what happens whenever both counts cut into whole slices: multiples of ranks x alignment
-// inside one chunk), its plan is the template's plan multiplied the same way.  Laying out the schedule costs
-// microseconds; planning a ring all-reduce of 8 ranks from scratch costs a few hundred, a mesh of 32 ranks tens of
-// milliseconds -- which a caller whose sizes change from call to call would otherwise pay on every call.
+// else, so when the schedule of a request is the template's with every offset and length multiplied by one factor
+// (what happens whenever both counts cut into whole slices: multiples of ranks x alignment inside one chunk; for the
+// collectives with one block per rank at any count), its plan is the template's plan multiplied the same way.
+// A count with a ragged last slice is covered as well where the collective works position by position (all-reduce,
+// broadcast, reduce: every step reads and writes the same offset of every buffer it touches, so what happens below
+// an offset does not depend on what lies above it): its schedule then is a whole-slice schedule cut off at the
+// count's last byte, and so is its plan.  Either way the new count's schedule is laid out (microseconds) and held
+// against the scaled, cut-off template step by step before anything is derived; planning a ring all-reduce of 8
+// ranks from scratch costs about a hundred microseconds, a piece-cut mesh of 32 ranks tens of milliseconds --
+// which a caller whose sizes change from call to call would otherwise pay on every call.
 struct PlanTemplate {
-    uint64_t count = 0;
-    std::vector<uint64_t> numbers;      // every offset and length of the schedule, in order
-    std::vector<uint32_t> structure;    // steps per phase and, per step, what is combined from where to where
+    uint64_t count = 0;                       // 0: not usable as a template
+    std::vector<Phase> schedule;              // the schedule as laid out, before lowering
+    std::vector<uint64_t> inBytes, outBytes, workBytes;
+    bool workspace = false;                   // the schedule rests data in a workspace: exact multiples only
+    bool positionWise = false;                // may be cut off at a count's last byte
     Plan plan;
 };
 
 // BuildPlan that also fills `tmpl` (requests with a count: not all-to-all-v, not the variable-count collectives).
 int BuildPlanTemplate(const PlanRequest &req, PlanTemplate *tmpl, std::string *err);
 
-// The plan of `req`, if its schedule is the template's scaled by req.count / tmpl.count (`req` must differ from the
-// template's request in nothing but the count); false if it is not, and the caller plans from scratch.
+// The plan of `req` (which must differ from the template's request in nothing but the count), if its schedule is the
+// template's multiplied by one factor and, for a position-wise collective, cut off at the count's last byte; false if
+// it is not, and the caller plans from scratch.
 bool PlanFromTemplate(const PlanRequest &req, const PlanTemplate &tmpl, Plan *plan);
 
 // JSON rendering of a plan (phases, steps, fused items) for tests and debugging.

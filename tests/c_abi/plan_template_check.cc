@@ -1,7 +1,7 @@
 // Plans derived from a template of another count against plans made from scratch, on the host
 // (cann-hccl_amd/csrc/plan.cc alone, no GPU): wherever PlanFromTemplate says it can derive a plan, the derived plan
-// must be the planner's own, number for number; counts that cut into whole slices must be derivable, and a count
-// with a ragged last slice must be refused when the template's slices are whole.
+// must be the planner's own, number for number; counts that cut into whole slices must be derivable, and so must a
+// count with a ragged last slice from a whole-slice template of a ring or uncut-mesh all-reduce or a ring broadcast.
 #include <cstdio>
 #include <string>
 #include <vector>
@@ -12,7 +12,7 @@ using namespace hcclamd;
 
 int main()
 {
-    int derived = 0, refused = 0, cases = 0;
+    int derived = 0, refused = 0, cases = 0, ragged = 0;
     struct Shape {
         int coll, algo;
         uint32_t p, servers, level0;
@@ -89,13 +89,16 @@ int main()
                                 sh.algo, sh.p, sh.servers, (unsigned long long)c0, (unsigned long long)c1);
                             return 1;
                         }
-                        // (collectives that cut the count into aligned slices; the per-rank-block ones scale at any count)
-                        const bool slices = sh.coll == COLL_ALLREDUCE || (sh.coll == COLL_REDUCE && sh.algo != ALGO_RING) ||
-                            (sh.coll == COLL_BROADCAST && sh.algo != ALGO_RHD && sh.algo != ALGO_STAR);
-                        if (c0 == regular && c1 == regular + 1 && slices && ok) {
-                            printf("a ragged count was derived from a whole one: coll %d algo %d p %u\n", sh.coll, sh.algo, sh.p);
+                        // a ragged count is the whole-slice schedule cut off at its last byte wherever the collective
+                        // works position by position and does not cut slices any further: the ring and the uncut mesh
+                        const bool cutOff = (sh.coll == COLL_ALLREDUCE && sh.servers == 1 && sh.level0 == 0 && sh.nicMask == 0 &&
+                            (sh.algo == ALGO_RING || sh.algo == ALGO_MESH_ATOMIC)) || (sh.coll == COLL_BROADCAST && sh.algo == ALGO_RING);
+                        if (c0 == 3 * regular && (c1 == regular + 1 || c1 == 3 * regular + 5) && cutOff && !ok) {
+                            printf("a ragged count was not derived from a whole one: coll %d algo %d p %u, count %llu\n", sh.coll, sh.algo,
+                                sh.p, (unsigned long long)c1);
                             return 1;
                         }
+                        ragged += (ok && c1 % regular != 0 && c0 % regular == 0) ? 1 : 0;
                     }
                 }
             }
@@ -115,6 +118,6 @@ int main()
         printf("a variable-count request got a template\n");
         return 1;
     }
-    printf("OK %d cases, %d derived, %d refused\n", cases, derived, refused);
+    printf("OK %d cases, %d derived, %d refused, %d ragged counts derived from whole-slice templates\n", cases, derived, refused, ragged);
     return 0;
 }
