@@ -1171,6 +1171,14 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                 vp->inBytes[r] = sl[r].size;
                 vp->outBytes[r] = extent;
             }
+            // whole blocks for the planner's short cut: rank r's block lands at its displacement in every receive buffer
+            for (uint32_t q = 0; q < p; q++) {
+                for (uint32_t r = 0; r < p; r++) {
+                    if (sl[r].size) {
+                        vp->blocks.push_back(VProgram::Block{sl[r].off, 0, sl[r].size, q, r});
+                    }
+                }
+            }
         }
         return 0;
     }
@@ -2019,9 +2027,13 @@ bool DirectCopyPlan(VProgram &vp, const PlanRequest &rq, const std::vector<uint8
     }();
     // A schedule with a workspace qualifies when it lists its whole blocks itself (the staged all-to-all-v: blocks rest
     // in the gathering rank's workspace between the two stages).
+    // So does an all-gather that lists its blocks (the variable-count one): its steps pass blocks on from receive buffer
+    // to receive buffer, which needs no lowering either, and its fused form is one item per rank's block with every
+    // receive buffer as a destination.
     const bool viaWorkspace = !vp.workBytes.empty();
+    const bool gathers = rq.coll == COLL_ALLGATHER && !vp.blocks.empty() && !viaWorkspace;
     if (verifyAll || rq.stageInput || (viaWorkspace && vp.blocks.empty()) ||
-        (rq.coll != COLL_ALLTOALLV && rq.coll != COLL_SCATTER && rq.coll != COLL_SENDRECV)) {
+        (rq.coll != COLL_ALLTOALLV && rq.coll != COLL_SCATTER && rq.coll != COLL_SENDRECV && !gathers)) {
         return false;
     }
     for (uint8_t a : alias) {
@@ -2034,7 +2046,7 @@ bool DirectCopyPlan(VProgram &vp, const PlanRequest &rq, const std::vector<uint8
     auto inWorkspace = [&](const Ref &r) { return viaWorkspace && r.buf == BUF_SEND && r.off >= vp.inBytes[r.rank]; };
     for (const Phase &ph : vp.phases) {
         for (const Step &st : ph.steps) {
-            if (st.reduce || st.a.buf != BUF_SEND || st.a.rank >= rq.p || st.dst.rank >= rq.p ||
+            if (st.reduce || !(st.a.buf == BUF_SEND || (gathers && st.a.buf == BUF_RECV)) || st.a.rank >= rq.p || st.dst.rank >= rq.p ||
                 !(st.dst.buf == BUF_RECV || inWorkspace(st.dst))) {
                 return false;
             }
@@ -2096,6 +2108,16 @@ bool DirectCopyPlan(VProgram &vp, const PlanRequest &rq, const std::vector<uint8
         }
         i = j;
     }
+    if (gathers) {
+        // every rank contributes one block, the same wherever it lands (checked before anything is handed over)
+        std::vector<uint64_t> size(rq.p, 0);
+        for (const Block &b : blocks) {
+            if (b.srcOff != 0 || (size[b.srcRank] != 0 && size[b.srcRank] != b.bytes)) {
+                return false;
+            }
+            size[b.srcRank] = b.bytes;
+        }
+    }
     uint64_t moved = 0;
     for (const Block &b : blocks) {
         moved += b.bytes;
@@ -2125,6 +2147,28 @@ bool DirectCopyPlan(VProgram &vp, const PlanRequest &rq, const std::vector<uint8
     }
     plan->stepRead = plan->stepWritten = stepped;
     plan->fusedRead = plan->fusedWritten = moved;
+    if (gathers) {
+        // one item per source block, read once, written to every rank that receives it (ranks in rising order)
+        std::vector<int> itemOf(rq.p, -1);
+        plan->fused.clear();
+        plan->fusedRead = 0;
+        for (const Block &b : blocks) {
+            if (itemOf[b.srcRank] < 0) {
+                itemOf[b.srcRank] = int(plan->fused.size());
+                plan->fused.emplace_back();
+                FusedItem &item = plan->fused.back();
+                item.kind = FK_COPY;
+                item.bytes = b.bytes;
+                item.src.push_back(MkRef(b.srcRank, BUF_SEND, 0));
+                item.srcValid.push_back(1);
+                plan->fusedRead += b.bytes;
+            }
+            FusedItem &item = plan->fused[size_t(itemOf[b.srcRank])];
+            item.dst.push_back(MkRef(b.dstRank, BUF_RECV, b.dstOff));
+        }
+        plan->fusedOk = true;
+        return true;
+    }
     // fused: a block that the schedule moved in pieces is one item again
     plan->fused.clear();
     plan->fused.reserve(blocks.size());

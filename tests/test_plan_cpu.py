@@ -247,11 +247,16 @@ def test_block_moving_plans_take_the_short_cut_and_agree_with_the_general_path(o
         dict(coll=H.COLL_SCATTER, algo=2 | (3 << 21), p=p, count=1003, ccl_bytes=200 << 20, tables=False),
     ]
 
+    vcounts = [5, 0, 301, 77, 1024, 3]
+    vdispls = [400, 0, 0, 2000, 410, 395]                      # not in rank order, with gaps
+    for algo in (RING, MESH, RHD):
+        requests.append(dict(coll=H.COLL_ALLGATHER, algo=algo, p=p, count=0, ccl_bytes=200 << 20, tables="v"))
+
     def plans():
         out = []
         for rq in requests:
-            plan = H.describe_plan(rq["coll"], rq["algo"], rq["p"], rq["count"], INT32, ccl_bytes=rq["ccl_bytes"],
-                                   tables=(cnt, sdis, rcnt, rdis) if rq["tables"] else None)
+            tables = (vcounts, vdispls) if rq["tables"] == "v" else ((cnt, sdis, rcnt, rdis) if rq["tables"] else None)
+            plan = H.describe_plan(rq["coll"], rq["algo"], rq["p"], rq["count"], INT32, ccl_bytes=rq["ccl_bytes"], tables=tables)
             steps = [sorted((st["dst"][0], st["dst"][2], st["a"][0], st["a"][2], st["n"]) for st in ph) for ph in plan["phases"]]
             out.append(dict(steps=steps, items=_copy_items(plan), bytes=[plan[k] for k in ("stepRead", "stepWritten", "fusedRead",
                                                                                          "fusedWritten", "scratchBytes")],
