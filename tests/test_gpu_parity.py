@@ -1541,6 +1541,20 @@ def test_sizes_that_change_from_call_to_call(orc):
                     g.stream.synchronize()
                     for r in range(p):
                         assert gh.same(dt, gh.to_host(recvs[r], dt)[:n // p], want_rs[r]), (algo, fuse, n, "reduce-scatter", r)
+                    # rooted collectives and an in-place all-reduce of the same changing counts
+                    root = n % p
+                    want_red = orc.reduce_to_root(ins, dt, SUM, root, algo=algo)
+                    H.reduce(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, SUM, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    assert gh.same(dt, gh.to_host(recvs[root], dt)[:n], want_red), (algo, fuse, n, "reduce")
+                    bufs = [gh.to_dev(x) for x in ins]
+                    torch.cuda.synchronize()
+                    H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, dt, root, g.stream_ptr)
+                    H.all_reduce(g.comms, [t.data_ptr() for t in bufs], [t.data_ptr() for t in bufs], n, dt, SUM, g.stream_ptr)
+                    g.stream.synchronize()
+                    want_in = orc.allreduce([ins[root].copy() for _ in range(p)], dt, SUM, algo=algo)
+                    for r in range(p):
+                        assert gh.same(dt, gh.to_host(bufs[r], dt), want_in[r]), (algo, fuse, n, "broadcast + in-place all-reduce", r)
             finally:
                 g.close()
 
