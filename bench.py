@@ -203,6 +203,38 @@ def run_suite(pkg, torch, steps, warmup, only="", settings=()):
     report("all-to-all-v pairwise p=16 int32 lognormal (%.0f MB)" % (4 * cnt.sum() / 1e6), comms,
            lambda: pkg.all_to_all_v(comms, sp, None, None, rp, None, None, pkg.HCCL_DATA_TYPE_INT32, stream.cuda_stream,
                                     tables=tables))
+    # the same exchange when the tables change on every call (an expert-parallel layer): nothing can be reused, so
+    # this is wall time per call, from the first rank's call to completion, one call at a time
+    name = "all-to-all-v pairwise p=16 lognormal, new tables every call"
+    if not only or any(part in name for part in only.split(",")):
+        import time
+        sets = []
+        for k in range(24):
+            rng_k = np.random.default_rng(3000 + k)
+            c = np.clip(np.rint(np.exp(np.log(65536.0) + rng_k.standard_normal((p, p)))), 0, 4 << 20).astype(np.uint64)
+            sd = np.concatenate([np.zeros((p, 1), np.uint64), np.cumsum(c, axis=1)[:, :-1]], axis=1).astype(np.uint64)
+            rc = c.T.copy()
+            rd = np.concatenate([np.zeros((p, 1), np.uint64), np.cumsum(rc, axis=1)[:, :-1]], axis=1).astype(np.uint64)
+            sets.append((pkg.a2av_tables(c, sd, rc, rd), int(max(c.sum(axis=1).max(), rc.sum(axis=1).max()))))
+        longest = max(n for _, n in sets)
+        sends2 = [torch.zeros(longest, dtype=torch.int32, device="cuda") for _ in range(p)]
+        recvs2 = [torch.zeros(longest, dtype=torch.int32, device="cuda") for _ in range(p)]
+        sp2, rp2 = [t.data_ptr() for t in sends2], [t.data_ptr() for t in recvs2]
+        for fuse in (1, 0):
+            pkg.set_param(comms[0], "fuse", fuse)
+            walls = []
+            for tabs, _ in sets:
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                pkg.all_to_all_v(comms, sp2, None, None, rp2, None, None, pkg.HCCL_DATA_TYPE_INT32, stream.cuda_stream, tables=tabs)
+                stream.synchronize()
+                walls.append(time.perf_counter() - t0)
+            if len(walls) > 4:
+                info = pkg.last_op_info(comms[0])
+                out.write("%-46s %-6s %9d %10.1f %9s %8s   (wall, median of %d calls, all cache misses: hit=%d)\n" % (
+                    name, "fused" if info["fused"] else "steps", info["launches"], 1e6 * float(np.median(walls[2:])), "-", "-",
+                    len(walls) - 2, info["cacheHit"]))
+        del sends2, recvs2
     pkg.set_param(comms[0], "servers", 2)
     report("all-to-all-v staged 2x8 p=16 int32 lognormal (%.0f MB)" % (4 * cnt.sum() / 1e6), comms,
            lambda: pkg.all_to_all_v(comms, sp, None, None, rp, None, None, pkg.HCCL_DATA_TYPE_INT32, stream.cuda_stream,
