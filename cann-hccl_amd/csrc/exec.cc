@@ -722,11 +722,18 @@ int CachedPlan(Group *g, const PlanRequest &rq, std::shared_ptr<const Plan> *out
     if (g->planCache.size() >= 128) {
         g->planCache.clear();   // plans in use stay alive through the prepared collectives that hold them
     }
-    // A new count of a request seen before: its plan is an earlier one's scaled, whenever the schedule is (counts that
-    // cut into whole slices).  Templates are kept per request-without-count, a few each.
-    std::string shape = key;
-    const uint64_t noCount = 0;
-    shape.replace(4 * sizeof(uint64_t), sizeof(uint64_t), reinterpret_cast<const char *>(&noCount), sizeof(uint64_t));   // head[4] = count
+    // A new count (or, for the variable-count reduce-scatter, a new table of blocks) of a request seen before: its plan
+    // is derived from a template of that request where the planner knows how.  Templates are kept per request without
+    // its count and tables, a few each.
+    std::string shape;
+    {
+        uint64_t head0[11];
+        std::memcpy(head0, head, sizeof(head));
+        head0[4] = 0;   // count
+        shape.append(reinterpret_cast<const char *>(head0), sizeof(head0));
+        shape.append(reinterpret_cast<const char *>(rq.alias.data()), rq.alias.size());
+        shape.push_back(rq.vCounts.empty() ? 'c' : 'v');
+    }
     std::vector<TemplateSlot> &templates = g->planTemplates[shape];
     std::shared_ptr<Plan> fresh = std::make_shared<Plan>();
     for (TemplateSlot &t : templates) {
@@ -738,15 +745,14 @@ int CachedPlan(Group *g, const PlanRequest &rq, std::shared_ptr<const Plan> *out
         }
     }
     std::shared_ptr<PlanTemplate> made = std::make_shared<PlanTemplate>();
-    int rc = BuildPlanTemplate(rq, made.get(), err);
+    int rc = BuildPlanTemplate(rq, made.get(), fresh.get(), err);
     if (rc != 0) {
         if (templates.empty()) {
             g->planTemplates.erase(shape);
         }
         return rc;
     }
-    *fresh = made->plan;
-    if (made->count != 0) {
+    if (made->count != 0 || made->blockTable) {
         if (g->planTemplates.size() > 64) {
             g->planTemplates.clear();            // (invalidates `templates`)
             g->planTemplates[shape].push_back(TemplateSlot{made, 0});

@@ -2377,7 +2377,9 @@ bool SameOffsets(const Step &st) { return st.dst.off == st.a.off && (!st.reduce 
 
 }  // namespace
 
-int BuildPlanTemplate(const PlanRequest &request, PlanTemplate *tmpl, std::string *err)
+namespace {
+
+int BuildCountTemplate(const PlanRequest &request, PlanTemplate *tmpl, std::string *err)
 {
     tmpl->count = 0;
     int rc = BuildPlan(request, &tmpl->plan, err);
@@ -2425,7 +2427,7 @@ int BuildPlanTemplate(const PlanRequest &request, PlanTemplate *tmpl, std::strin
     return 0;
 }
 
-bool PlanFromTemplate(const PlanRequest &request, const PlanTemplate &tmpl, Plan *plan)
+bool PlanFromCountTemplate(const PlanRequest &request, const PlanTemplate &tmpl, Plan *plan)
 {
     if (tmpl.count == 0 || !Templatable(request)) {
         return false;
@@ -2563,6 +2565,201 @@ bool PlanFromTemplate(const PlanRequest &request, const PlanTemplate &tmpl, Plan
     }
     plan->scratchBytes = kept(0, scaled(tmpl.plan.scratchBytes));
     return whole;
+}
+
+// ---- block-table templates (variable-count reduce-scatter) --------------------------------------------------------
+constexpr uint32_t kCanonicalShift = 4;       // canonical block s has 2^(s + 4) elements
+constexpr uint32_t kBlockTableMaxRanks = 32;
+
+bool BlockTableRequest(const PlanRequest &rq)
+{
+    if (rq.coll != COLL_REDUCESCATTER || rq.vCounts.size() != rq.p || rq.vDispls.size() != rq.p || rq.p < 2 ||
+        rq.p > kBlockTableMaxRanks || rq.servers > 1) {
+        return false;
+    }
+    if (rq.algo == ALGO_MESH && !rq.meshAtomic) {
+        return false;       // the piece cut splits blocks at aligned lengths: its numbers are not runs of blocks
+    }
+    for (uint8_t shared : rq.alias) {
+        if (shared) {
+            return false;   // in place, a block's length is held against offsets of the send buffer: an order the sizes decide
+        }
+    }
+    if (rq.stageInput) {
+        return false;
+    }
+    uint64_t at = 0;
+    for (uint32_t r = 0; r < rq.p; r++) {
+        if (rq.vCounts[r] == 0 || rq.vDispls[r] != at) {
+            return false;
+        }
+        at += rq.vCounts[r];
+    }
+    return true;
+}
+
+// A canonical number (bytes) as the run of blocks [first, last) it measures; false if it is not one.
+bool RunOf(uint64_t bytes, uint64_t unit, uint32_t p, uint32_t *first, uint32_t *last)
+{
+    const uint64_t scale = unit << kCanonicalShift;
+    if (bytes % scale != 0) {
+        return false;
+    }
+    const uint64_t m = bytes / scale;      // 2^last - 2^first
+    if (m == 0) {
+        *first = *last = 0;
+        return true;
+    }
+    const uint32_t a = uint32_t(__builtin_ctzll(m));
+    const uint64_t ones = (m >> a) + 1;    // 2^(last - first)
+    if ((ones & (ones - 1)) != 0) {
+        return false;
+    }
+    const uint32_t b = a + uint32_t(__builtin_ctzll(ones));
+    if (b > p) {
+        return false;
+    }
+    *first = a;
+    *last = b;
+    return true;
+}
+
+bool PlanFromBlockTemplate(const PlanRequest &request, const PlanTemplate &tmpl, Plan *plan)
+{
+    if (!tmpl.blockTable || !BlockTableRequest(request)) {
+        return false;
+    }
+    VProgram vp;
+    std::string ignored;
+    if (BuildVirtual(Normalised(request), &vp, &ignored) != 0 || !vp.workBytes.empty()) {
+        return false;
+    }
+    const uint32_t p = request.p;
+    std::vector<uint64_t> prefix(p + 1, 0);   // bytes in front of block s
+    for (uint32_t s = 0; s < p; s++) {
+        prefix[s + 1] = prefix[s] + request.vCounts[s] * request.unit;
+    }
+    bool ok = true;
+    auto measured = [&](uint64_t canonical) -> uint64_t {
+        uint32_t a = 0, b = 0;
+        if (!RunOf(canonical, request.unit, p, &a, &b)) {
+            ok = false;
+            return 0;
+        }
+        return prefix[b] - prefix[a];
+    };
+    // 1. the new schedule is the canonical one re-measured
+    if (vp.phases.size() != tmpl.schedule.size() || vp.inBytes.size() != tmpl.inBytes.size()) {
+        return false;
+    }
+    for (size_t r = 0; r < vp.inBytes.size(); r++) {
+        if (vp.inBytes[r] != measured(tmpl.inBytes[r]) || vp.outBytes[r] != measured(tmpl.outBytes[r])) {
+            return false;
+        }
+    }
+    for (size_t i = 0; i < vp.phases.size(); i++) {
+        if (vp.phases[i].steps.size() != tmpl.schedule[i].steps.size()) {
+            return false;
+        }
+        for (size_t j = 0; j < vp.phases[i].steps.size(); j++) {
+            const Step &f = vp.phases[i].steps[j], &t = tmpl.schedule[i].steps[j];
+            if (f.reduce != t.reduce || f.dst.rank != t.dst.rank || f.dst.buf != t.dst.buf || f.a.rank != t.a.rank ||
+                f.a.buf != t.a.buf || (t.reduce && (f.b.rank != t.b.rank || f.b.buf != t.b.buf)) ||
+                f.bytes != measured(t.bytes) || f.dst.off != measured(t.dst.off) || f.a.off != measured(t.a.off) ||
+                (t.reduce && f.b.off != measured(t.b.off))) {
+                return false;
+            }
+        }
+    }
+    if (!ok) {
+        return false;
+    }
+    // 2. so its plan is the canonical plan re-measured
+    *plan = tmpl.plan;
+    plan->stepRead = plan->stepWritten = plan->fusedRead = plan->fusedWritten = 0;
+    for (Phase &ph : plan->phases) {
+        for (Step &st : ph.steps) {
+            st.dst.off = measured(st.dst.off);
+            st.a.off = measured(st.a.off);
+            st.b.off = st.reduce ? measured(st.b.off) : 0;
+            st.bytes = measured(st.bytes);
+            plan->stepRead += st.bytes * (st.reduce ? 2 : 1);
+            plan->stepWritten += st.bytes;
+        }
+    }
+    for (FusedItem &it : plan->fused) {
+        it.bytes = measured(it.bytes);
+        uint64_t nsrc = 0;
+        for (size_t k = 0; k < it.src.size(); k++) {
+            if (it.srcValid[k]) {
+                it.src[k].off = measured(it.src[k].off);
+                nsrc++;
+            }
+        }
+        for (Ref &r : it.dst) {
+            r.off = measured(r.off);
+        }
+        plan->fusedRead += nsrc * it.bytes;
+        plan->fusedWritten += uint64_t(it.dst.size()) * it.bytes;
+    }
+    for (std::vector<uint64_t> *v : {&plan->sendBytes, &plan->recvBytes}) {
+        for (uint64_t &x : *v) {
+            x = measured(x);
+        }
+    }
+    plan->scratchBytes = measured(plan->scratchBytes);
+    return ok;
+}
+
+int BuildBlockTemplate(const PlanRequest &request, PlanTemplate *tmpl, std::string *err)
+{
+    PlanRequest canonical = request;
+    uint64_t at = 0;
+    for (uint32_t s = 0; s < request.p; s++) {
+        canonical.vCounts[s] = uint64_t(1) << (s + kCanonicalShift);
+        canonical.vDispls[s] = at;
+        at += canonical.vCounts[s];
+    }
+    int rc = BuildPlan(canonical, &tmpl->plan, err);
+    if (rc != 0) {
+        return rc;
+    }
+    VProgram vp;
+    std::string ignored;
+    if (BuildVirtual(Normalised(canonical), &vp, &ignored) != 0 || !vp.workBytes.empty()) {
+        return 0;
+    }
+    tmpl->schedule = std::move(vp.phases);
+    tmpl->inBytes = vp.inBytes;
+    tmpl->outBytes = vp.outBytes;
+    tmpl->blockTable = true;
+    return 0;
+}
+
+}  // namespace
+
+int BuildPlanTemplate(const PlanRequest &request, PlanTemplate *tmpl, Plan *plan, std::string *err)
+{
+    tmpl->count = 0;
+    tmpl->blockTable = false;
+    if (BlockTableRequest(request)) {
+        int rc = BuildBlockTemplate(request, tmpl, err);
+        if (rc == 0 && tmpl->blockTable && PlanFromBlockTemplate(request, *tmpl, plan)) {
+            return 0;
+        }
+        tmpl->blockTable = false;      // not the canonical schedule re-measured: no template, plan the request itself
+        return BuildPlan(request, plan, err);
+    }
+    int rc = BuildCountTemplate(request, tmpl, err);
+    if (rc == 0) {
+        *plan = tmpl->plan;
+    }
+    return rc;
+}
+
+bool PlanFromTemplate(const PlanRequest &request, const PlanTemplate &tmpl, Plan *plan)
+{
+    return tmpl.blockTable ? PlanFromBlockTemplate(request, tmpl, plan) : PlanFromCountTemplate(request, tmpl, plan);
 }
 
 std::string DescribePlan(const Plan &plan)

@@ -186,8 +186,16 @@ int BuildPlan(const PlanRequest &req, Plan *plan, std::string *err);
 // against the scaled, cut-off template step by step before anything is derived; planning a ring all-reduce of 8
 // ranks from scratch costs about a hundred microseconds, a piece-cut mesh of 32 ranks tens of milliseconds --
 // which a caller whose sizes change from call to call would otherwise pay on every call.
+//
+// A reduce-scatter over a table of blocks (the variable-count one) whose blocks are all non-empty and lie one
+// behind the other in rank order has a template of another kind: the plan of the same request over blocks of
+// 16, 32, 64 ... elements.  Every offset and length of that schedule and of its plan is a run of consecutive blocks,
+// and with those sizes the run can be read off the number; the plan for other block sizes is the same plan with every
+// run measured in the new sizes (the order of all range ends, which is all the planner looks at, is the same for any
+// non-empty blocks laid out that way).  As above, the new schedule is held against the re-measured template first.
 struct PlanTemplate {
-    uint64_t count = 0;                       // 0: not usable as a template
+    uint64_t count = 0;                       // 0: not usable as a count template
+    bool blockTable = false;                  // the other kind: canonical block sizes, re-measured per request
     std::vector<Phase> schedule;              // the schedule as laid out, before lowering
     std::vector<uint64_t> inBytes, outBytes, workBytes;
     bool workspace = false;                   // the schedule rests data in a workspace: exact multiples only
@@ -195,8 +203,9 @@ struct PlanTemplate {
     Plan plan;
 };
 
-// BuildPlan that also fills `tmpl` (requests with a count: not all-to-all-v, not the variable-count collectives).
-int BuildPlanTemplate(const PlanRequest &req, PlanTemplate *tmpl, std::string *err);
+// BuildPlan that also fills `tmpl` where the request has a template of either kind (tmpl->count != 0 or tmpl->blockTable).
+// `plan` receives the plan of `req` itself.
+int BuildPlanTemplate(const PlanRequest &req, PlanTemplate *tmpl, Plan *plan, std::string *err);
 
 // The plan of `req` (which must differ from the template's request in nothing but the count), if its schedule is the
 // template's multiplied by one factor and, for a position-wise collective, cut off at the count's last byte; false if

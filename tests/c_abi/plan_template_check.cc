@@ -53,7 +53,8 @@ int main()
                     r0.count = c0;
                     PlanTemplate tmpl;
                     std::string err;
-                    if (BuildPlanTemplate(r0, &tmpl, &err) != 0) {
+                    Plan own;
+                    if (BuildPlanTemplate(r0, &tmpl, &own, &err) != 0) {
                         printf("template failed: coll %d algo %d p %u count %llu: %s\n", sh.coll, sh.algo, sh.p, (unsigned long long)c0, err.c_str());
                         return 1;
                     }
@@ -104,7 +105,7 @@ int main()
             }
         }
     }
-    // requests without a count have no template
+    // requests without a count have no count template
     PlanRequest v;
     v.coll = COLL_ALLGATHER;
     v.p = 4;
@@ -114,10 +115,104 @@ int main()
     PlanTemplate tv;
     std::string err;
     Plan out;
-    if (BuildPlanTemplate(v, &tv, &err) != 0 || tv.count != 0 || PlanFromTemplate(v, tv, &out)) {
-        printf("a variable-count request got a template\n");
+    if (BuildPlanTemplate(v, &tv, &out, &err) != 0 || tv.count != 0 || tv.blockTable || PlanFromTemplate(v, tv, &out)) {
+        printf("a variable-count all-gather got a template\n");
         return 1;
     }
-    printf("OK %d cases, %d derived, %d refused, %d ragged counts derived from whole-slice templates\n", cases, derived, refused, ragged);
+    // the variable-count reduce-scatter over non-empty blocks in rank order: one template per schedule serves every table
+    int tables = 0;
+    uint64_t seed = 12345;
+    auto next = [&] { seed = seed * 6364136223846793005ull + 1442695040888963407ull; return seed >> 33; };
+    for (int algo : {int(ALGO_RING), int(ALGO_MESH_ATOMIC), int(ALGO_RHD), int(ALGO_MESH)}) {
+        for (uint32_t p : {2u, 3u, 5u, 8u, 12u, 16u, 32u}) {
+            for (uint32_t unit : {4u, 2u}) {
+                PlanRequest base;
+                base.coll = COLL_REDUCESCATTER;
+                base.algo = Algo(algo);
+                base.p = p;
+                base.unit = unit;
+                base.alias.assign(p, 0);
+                PlanTemplate bt;
+                bool have = false;
+                for (int t = 0; t < 12; t++) {
+                    PlanRequest rq = base;
+                    rq.vCounts.resize(p);
+                    rq.vDispls.resize(p);
+                    uint64_t at = 0;
+                    for (uint32_t r = 0; r < p; r++) {
+                        rq.vCounts[r] = t == 0 ? 7 : (t == 1 ? 1 : 1 + next() % (t < 5 ? 50 : (t < 9 ? 100000 : (1u << 26))));   // equal, tiny, mixed
+                        rq.vDispls[r] = at;
+                        at += rq.vCounts[r];
+                    }
+                    Plan direct, fromTable;
+                    if (BuildPlan(rq, &direct, &err) != 0) {
+                        printf("plan failed: %s\n", err.c_str());
+                        return 1;
+                    }
+                    if (!have) {
+                        if (BuildPlanTemplate(rq, &bt, &fromTable, &err) != 0) {
+                            printf("block template failed: %s\n", err.c_str());
+                            return 1;
+                        }
+                        have = true;
+                        if (DescribePlan(fromTable) != DescribePlan(direct)) {
+                            printf("plan returned with the block template differs: algo %d p %u\n", algo, p);
+                            return 1;
+                        }
+                        if (bt.blockTable != (algo != int(ALGO_MESH))) {
+                            printf("block template %s: algo %d p %u\n", bt.blockTable ? "made for a schedule that cuts blocks" : "missing", algo, p);
+                            return 1;
+                        }
+                        continue;
+                    }
+                    if (!bt.blockTable) {
+                        continue;       // the piece-cut mesh cuts blocks: no template
+                    }
+                    if (!PlanFromTemplate(rq, bt, &fromTable)) {
+                        printf("block table not derived: algo %d p %u table %d\n", algo, p, t);
+                        return 1;
+                    }
+                    if (DescribePlan(fromTable) != DescribePlan(direct)) {
+                        printf("plan derived from the block template differs: algo %d p %u unit %u table %d\n", algo, p, unit, t);
+                        return 1;
+                    }
+                    tables++;
+                }
+                // a gap between blocks or an empty block: not this template's case
+                if (bt.blockTable) {
+                    PlanRequest gap = base;
+                    gap.vCounts.assign(p, 5);
+                    gap.vDispls.resize(p);
+                    for (uint32_t r = 0; r < p; r++) {
+                        gap.vDispls[r] = r * 6;
+                    }
+                    Plan none;
+                    if (PlanFromTemplate(gap, bt, &none)) {
+                        printf("a table with gaps was derived\n");
+                        return 1;
+                    }
+                    gap.vCounts[p - 1] = 0;
+                    if (PlanFromTemplate(gap, bt, &none)) {
+                        printf("a table with an empty block was derived\n");
+                        return 1;
+                    }
+                    PlanRequest inPlace = base;
+                    inPlace.vCounts.assign(p, 5);
+                    inPlace.vDispls.resize(p);
+                    for (uint32_t r = 0; r < p; r++) {
+                        inPlace.vDispls[r] = r * 5;
+                    }
+                    inPlace.alias.assign(p, 1);
+                    PlanTemplate ip;
+                    if (BuildPlanTemplate(inPlace, &ip, &none, &err) != 0 || ip.blockTable || PlanFromTemplate(inPlace, bt, &none)) {
+                        printf("an in-place table got a block template\n");
+                        return 1;
+                    }
+                }
+            }
+        }
+    }
+    printf("OK %d cases, %d derived, %d refused, %d ragged counts derived from whole-slice templates, %d block tables derived\n", cases, derived,
+        refused, ragged, tables);
     return 0;
 }

@@ -421,7 +421,10 @@ def test_plans_derived_from_a_template_of_another_count_are_the_planners_own(tmp
     """A caller whose sizes change from call to call gets its plans by scaling an earlier plan of the same request
     whenever the schedule scales (counts that cut into whole slices).  tests/c_abi/plan_template_check.cc holds every
     derived plan against the plan made from scratch (27 schedules x 2 element sizes x in place or not x 10 x 10
-    counts), on the host, against cann-hccl_amd/csrc/plan.cc alone."""
+    counts), on the host, against cann-hccl_amd/csrc/plan.cc alone.  The same program holds the plans of the
+    variable-count reduce-scatter that are derived from the plan over blocks of 16, 32, 64 ... elements against the
+    planner's own (ring, uncut mesh, halving-doubling; 2 to 32 ranks; tables of equal, tiny, mixed and large blocks),
+    and checks that the piece-cut mesh, tables with gaps or empty blocks and in-place calls get no such template."""
     import os
     import shutil
     import subprocess
@@ -437,6 +440,8 @@ def test_plans_derived_from_a_template_of_another_count_are_the_planners_own(tmp
     assert out.returncode == 0 and out.stdout.startswith("OK"), out.stdout
     derived = int(out.stdout.split()[3])
     assert derived > 1000, out.stdout
+    tables = int(out.stdout.split("templates,")[1].split()[0])
+    assert tables > 300, out.stdout
 
 
 def _rank_table(path, servers, per_server, **edits):
