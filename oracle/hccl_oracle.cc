@@ -1957,6 +1957,57 @@ int orc_reducescatter_v(int algo, uint32_t p, void **in, void **out, const uint6
                     m.procs.push_back(std::move(pr));
                 }
             }
+        } else if (algo == ALGO_RHD) {
+            // No counterpart in the reference, which runs the variable-count reduce-scatter on the mesh only: the order of
+            // ReduceScatterRecursiveHalvingDoubling (reduce_scatter_recursive_hd.cc:33-254) over the caller's table.  The
+            // blocks of a table need not lie one behind the other, so a step's range travels block by block.
+            uint32_t block, part1;
+            RhdParams(p, &block, &part1);
+            const uint32_t half = part1 / 2;
+            std::vector<uint32_t> rankOf(block);
+            std::vector<std::vector<uint32_t>> owned(block);
+            for (uint32_t b = 0; b < block; b++) {
+                rankOf[b] = b < half ? 2 * b : b + half;
+                owned[b] = b < half ? std::vector<uint32_t>{2 * b, 2 * b + 1} : std::vector<uint32_t>{b + half};
+            }
+            uint32_t steps = 0;
+            while ((1u << steps) < block) {
+                steps++;
+            }
+            for (uint32_t r = 0; r < p; r++) {
+                Proc pr;
+                pr.rank = r;
+                if (r < part1 && (r % 2) == 1) {
+                    pr.prog.push_back(MkSend(static_cast<int>(r - 1), 1, B_IN, 0, extent));
+                    pr.prog.push_back(MkRecvCopy(static_cast<int>(r - 1), 1, B_IN, sl[r].off, sl[r].size));
+                    m.procs.push_back(std::move(pr));
+                    continue;
+                }
+                if (r < part1) {
+                    pr.prog.push_back(MkRecvReduce(static_cast<int>(r + 1), 1, B_IN, 0, B_IN, 0, extent));
+                }
+                const uint32_t q = r < part1 ? r / 2 : r - half;
+                for (uint32_t step = 0; step < steps; step++) {
+                    const uint32_t mask = 1u << (steps - step - 1);
+                    const uint32_t peer = q ^ mask;
+                    const uint32_t txId = peer & ~(mask - 1), rxId = q & ~(mask - 1);
+                    for (uint32_t b = txId; b < txId + mask; b++) {
+                        for (uint32_t u : owned[b]) {
+                            pr.prog.push_back(MkSend(static_cast<int>(rankOf[peer]), 0, B_IN, sl[u].off, sl[u].size));
+                        }
+                    }
+                    for (uint32_t b = rxId; b < rxId + mask; b++) {
+                        for (uint32_t u : owned[b]) {
+                            pr.prog.push_back(MkRecvReduce(static_cast<int>(rankOf[peer]), 0, B_IN, sl[u].off, B_IN, sl[u].off,
+                                sl[u].size));
+                        }
+                    }
+                }
+                if (r < part1) {
+                    pr.prog.push_back(MkSend(static_cast<int>(r + 1), 1, B_IN, sl[r + 1].off, sl[r + 1].size));
+                }
+                m.procs.push_back(std::move(pr));
+            }
         } else {
             return -10;
         }

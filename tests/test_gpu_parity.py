@@ -512,7 +512,7 @@ def _v_case(p, seed, scale):
     return counts, displs, pos + 3
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, MESH_ATOMIC])
+@pytest.mark.parametrize("algo", [RING, MESH, MESH_ATOMIC, RHD])
 def test_reducescatter_v(orc, algo):
     for p in (1, 3, 8):
         for fuse in (1, 0):
@@ -542,9 +542,7 @@ def test_reducescatter_v_with_a_new_table_on_every_call(orc):
     # general path.  Every result is the checker's.
     p = 8
     rng = np.random.default_rng(77)
-    # (the checker has no halving-doubling over a table of blocks: that schedule runs on integers, whose sums do not
-    # depend on the order, against the checker's ring)
-    for algo, dt in ((RING, FP32), (MESH_ATOMIC, BF16), (RHD, INT32), (MESH, FP32)):
+    for algo, dt in ((RING, FP32), (MESH_ATOMIC, BF16), (RHD, FP32), (MESH, FP32)):
         for fuse in (1, 0):
             g = _group(p, algo, fuse=fuse)
             try:
@@ -563,7 +561,7 @@ def test_reducescatter_v_with_a_new_table_on_every_call(orc):
                     extent = int((displs + counts).max())
                     print("new table", ALGO_NAME[algo], "fuse", fuse, "call", call, counts.tolist(), flush=True)
                     want = orc.reducescatter_v([x[:extent] for x in ins_all], counts, displs, dt, SUM,
-                                               algo=RING if algo == RHD else _expected_algo(algo, dt, SUM))
+                                               algo=_expected_algo(algo, dt, SUM))
                     H.reduce_scatter_v(g.comms, [t.data_ptr() for t in sends], counts, displs, [t.data_ptr() for t in recvs],
                                        dt, SUM, g.stream_ptr)
                     g.stream.synchronize()

@@ -616,7 +616,7 @@ def _v_blocks(p, seed, scale=400):
     return counts, displs, pos + 3
 
 
-@pytest.mark.parametrize("algo", [RING, MESH, MESH_ATOMIC])
+@pytest.mark.parametrize("algo", [RING, MESH, MESH_ATOMIC, RHD])
 def test_reducescatter_v_matches_chain(orc, algo):
     # the variable-count reduce-scatter runs the same templates over the caller's block table: block r comes out as
     # the ring chain / the mesh chains of its pieces, evaluated here with numpy on the block's elements alone
@@ -636,6 +636,11 @@ def test_reducescatter_v_matches_chain(orc, algo):
                         want = cf.ring_chain(dt, op, xs, r)
                     elif algo == MESH_ATOMIC:
                         want = cf.mesh_atomic_chain(dt, op, xs, r)
+                    elif algo == RHD:
+                        # the halving tree of the block rank that ends up with block r (a folded pair's block rank has
+                        # both blocks of the pair)
+                        block, part1 = cf.rhd_params(p)
+                        want = cf.rhd_tree(dt, op, xs, r // 2 if r < part1 else r - part1 // 2, block, part1)
                     else:
                         want = np.empty_like(xs[0])
                         nstream = p - 1 if p > 2 else 1
