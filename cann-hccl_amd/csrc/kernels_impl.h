@@ -223,19 +223,19 @@ template <int OP> __device__ __forceinline__ uint32_t PkBf16(uint32_t a, uint32_
     }
 }
 
-// fp16, two elements per word: widen both to fp32, combine, round to nearest even (the hardware conversions);
-// max / min compare the halves as they are (the conversion to fp32 is exact and keeps the order) and keep the chosen
-// operand's bits.
+// fp16, two elements per word.  Sum and product use the packed half instructions (v_pk_add_f16 / v_pk_mul_f16), one
+// per word instead of four conversions, two operations and a conversion back.  The bits are those of "widen to fp32,
+// combine, round to nearest even": an fp32 has 24 significant bits, 2 x 11 + 2, and with that many the second rounding
+// of a sum never changes what a single rounding to 11 bits gives (the product of two halves is exact in fp32 to begin
+// with); denormal halves are kept by both forms.  Max / min compare the halves as they are (the conversion to fp32 is
+// exact and keeps the order) and keep the chosen operand's bits.
 typedef _Float16 H2 __attribute__((ext_vector_type(2)));
 template <int OP> __device__ __forceinline__ uint32_t PkF16(uint32_t a, uint32_t b)
 {
     const H2 x = BitCast<H2>(a), y = BitCast<H2>(b);
     if (OP == ROP_SUM || OP == ROP_PROD) {
-        const F2 fx = __builtin_convertvector(x, F2), fy = __builtin_convertvector(y, F2);
-        F2 r;
-        r.x = (OP == ROP_SUM) ? fx.x + fy.x : fx.x * fy.x;
-        r.y = (OP == ROP_SUM) ? fx.y + fy.y : fx.y * fy.y;
-        return BitCast<uint32_t>(__builtin_convertvector(r, H2));
+        const H2 r = (OP == ROP_SUM) ? x + y : x * y;
+        return BitCast<uint32_t>(r);
     } else {
         const bool pickLo = (OP == ROP_MAX) ? (y.x > x.x) : (y.x < x.x);
         const bool pickHi = (OP == ROP_MAX) ? (y.y > x.y) : (y.y < x.y);

@@ -668,6 +668,35 @@ def test_special_values_16bit(orc):
                 g.close()
 
 
+def test_fp16_sum_and_product_of_every_half_with_many_partners(orc):
+    # The kernels add and multiply halves with the packed half instructions, the checker widens to fp32, combines and
+    # rounds.  Both must be the correctly rounded result, which numpy gives independently of either: the sum and the
+    # product of two halves are exact in float64, and its conversion to float16 rounds once, to nearest even.  Every
+    # half bit pattern meets 512 partners: the specials (zeros, infinities, largest, smallest, denormals, ties) and
+    # random bit patterns.
+    rng = np.random.default_rng(16)
+    hf = np.array([0x0000, 0x8000, 0x7c00, 0xfc00, 0x7bff, 0xfbff, 0x0001, 0x8001, 0x03ff, 0x83ff, 0x0400, 0x8400, 0x3c00,
+                   0xbc00, 0x3c01, 0x3bff, 0x4000, 0x7800, 0x1400, 0x0002, 0x7e00, 0x3555], np.uint16)
+    partners = np.concatenate([hf, rng.integers(0, 1 << 16, 512 - hf.size).astype(np.uint16)])
+    a = np.repeat(np.arange(1 << 16, dtype=np.uint32).astype(np.uint16), partners.size)
+    b = np.tile(partners, 1 << 16)
+    fa, fb = a.view(np.float16).astype(np.float64), b.view(np.float16).astype(np.float64)
+    with np.errstate(all="ignore"):
+        exact = {SUM: (fa + fb).astype(np.float16).view(np.uint16), PROD: (fa * fb).astype(np.float16).view(np.uint16)}
+    for fuse in (1, 0):
+        g = gh.Group(2, fuse=fuse)
+        try:
+            for op in (SUM, PROD):
+                print("every half", "fuse", fuse, "op", op, flush=True)
+                want = orc.allreduce([a, b], FP16, op, threads=16)
+                outs, _ = gh.all_reduce(g, [a, b], FP16, op)
+                for r in range(2):
+                    assert gh.same(FP16, outs[r], want[r]), (fuse, op, r, "checker")
+                    assert gh.same(FP16, outs[r], exact[op]), (fuse, op, r, "correctly rounded")
+        finally:
+            g.close()
+
+
 def test_broadcast_reduce_scatter_rooted(orc):
     for p in (1, 3, 8):
         for fuse in (1, 0):
