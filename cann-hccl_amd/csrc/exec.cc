@@ -283,17 +283,27 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
     const uint32_t stepGrid = std::max(1u, g->numCu * (g->cfg.blocksPerCu ? g->cfg.blocksPerCu : 2u));
     uint32_t fusedPerCu = g->cfg.blocksPerCu;
     if (fusedPerCu == 0) {
-        double streamBytes = 0, bytes = 0;
+        double streamBytes = 0, storeBytes = 0, bytes = 0;
         for (const FusedItem &it : pp->plan->fused) {
             uint32_t nsrc = 0;
             for (uint8_t v : it.srcValid) {
                 nsrc += v;
             }
             streamBytes += double(nsrc + it.dst.size()) * double(it.bytes);
+            storeBytes += double(it.dst.size()) * double(it.bytes);
             bytes += double(it.bytes);
         }
         double streams = bytes > 0 ? streamBytes / bytes : 2.0;   // loads + stores per lane and vector
         fusedPerCu = streams >= 8.0 ? 1u : (streams >= 3.0 ? 2u : 4u);
+        // That holds for shapes that write as much as they read or more, and for everything much larger than the
+        // memory-side cache.  Many sources into one destination (reduce-scatter, reduce) of 8- and 16-bit elements,
+        // where a combine costs several instructions, run better wide up to about a gigabyte in all (measured, bf16
+        // sum: 8 ranks x 64 MiB 104 us at 1 per CU, 99 at 8; 16 ranks x 64 MiB 196 / 189; 8 ranks x 256 MiB 415 / 421,
+        // so not there; fp32 within a percent either way at every size).
+        if (fusedPerCu == 1 && reduceColl && DtypeSize(dtype) <= 2 && storeBytes * 5.0 <= streamBytes &&
+            streamBytes <= 1.25 * 1024.0 * 1024.0 * 1024.0) {
+            fusedPerCu = 8;
+        }
         // Plain copies (one source, one destination) go through the copy kernel, which really gets the
         // occupancy it is launched with; with non-temporal stores more workgroups only widen the range
         // of addresses written at a time, which this memory system likes less (measured, 8 ranks:
