@@ -311,3 +311,88 @@ def test_random_scatter_and_broadcast_over_rank_groups(orc, seed):
                 assert np.array_equal(gh.to_host(bufs[r], dt), ins[root]), (seed, case, "broadcast", r)
         finally:
             g.close()
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_sequence_of_calls_on_one_group(orc, seed):
+    # What a training or serving loop does to one communicator: collectives of every kind with sizes and tables that
+    # change from call to call, repeats of earlier calls, the issue mode switched in between.  The library answers
+    # from its caches where it can (prepared collectives, plans, plans derived from earlier plans) and grows its
+    # scratch memory on the way; every result is the checker's.
+    rng = np.random.default_rng(5400 + SEED_SHIFT + seed)
+    p = int(rng.choice([4, 8, 16]))
+    algo = int(rng.choice([RING, MESH_ATOMIC, RHD]))
+    dt = int(rng.choice([cf.FP32, cf.BF16, cf.INT32, cf.FP16]))
+    op = 0
+    unit = H.DTYPE_SIZE[dt]
+    top = 48 * 1024
+    pool = [cf.random_input(dt, top * p, rng) for _ in range(p)]          # every call reads a prefix of these
+    sends = [gh.to_dev(x) for x in pool]
+    recvs = [gh.empty_dev(top * p * unit) for _ in range(p)]
+    ptr = lambda ts: [t.data_ptr() for t in ts]
+    g = gh.Group(p, algo=NAMES[algo], deterministic=0 if algo == MESH_ATOMIC else 1, cache_entries=16)
+    seen = []
+    try:
+        torch.cuda.synchronize()
+        for call in range(60):
+            if call % 7 == 3:
+                g.set(fuse=int(rng.integers(0, 2)))
+            kind = str(rng.choice(["ar", "ar", "rs", "rsv", "ag", "agv", "red", "bc"]))
+            if seen and rng.random() < 0.25:
+                kind, n, counts = seen[int(rng.integers(0, len(seen)))]      # an earlier call again
+            else:
+                n = int(rng.choice([int(rng.integers(1, 64)), int(rng.integers(1, 6)) * p * 32 * 16, int(rng.integers(64, top))]))
+                counts = rng.integers(1, top // 2, p) if rng.random() < 0.8 else rng.integers(0, 50, p)
+                seen.append((kind, n, counts))
+            displs = np.concatenate(([0], np.cumsum(counts)[:-1])).astype(np.int64)
+            print("sequence seed", seed, "call", call, kind, "p", p, "algo", algo, "type", dt, "n", n, flush=True)
+            if kind == "ar":
+                ins = [x[:n] for x in pool]
+                want = orc.allreduce(ins, dt, op, algo=algo)
+                H.all_reduce(g.comms, ptr(sends), ptr(recvs), n, dt, op, g.stream_ptr)
+                g.stream.synchronize()
+                got = [gh.to_host(recvs[r], dt)[:n] for r in range(p)]
+            elif kind == "rs":
+                m = max(1, n // p)
+                want = orc.reducescatter([x[:m * p] for x in pool], dt, op, algo=algo)
+                H.reduce_scatter(g.comms, ptr(sends), ptr(recvs), m, dt, op, g.stream_ptr)
+                g.stream.synchronize()
+                got = [gh.to_host(recvs[r], dt)[:m] for r in range(p)]
+            elif kind == "rsv":
+                extent = int(counts.sum())
+                want = orc.reducescatter_v([x[:extent] for x in pool], counts, displs, dt, op, algo=algo)
+                H.reduce_scatter_v(g.comms, ptr(sends), counts, displs, ptr(recvs), dt, op, g.stream_ptr)
+                g.stream.synchronize()
+                got = [gh.to_host(recvs[r], dt)[:int(counts[r])] for r in range(p)]
+            elif kind == "ag":
+                m = max(1, n // p)
+                want = [np.concatenate([x[:m] for x in pool])] * p
+                H.all_gather(g.comms, ptr(sends), ptr(recvs), m, dt, g.stream_ptr)
+                g.stream.synchronize()
+                got = [gh.to_host(recvs[r], dt)[:m * p] for r in range(p)]
+            elif kind == "agv":
+                want = [np.concatenate([pool[r][:int(counts[r])] for r in range(p)])] * p
+                H.all_gather_v(g.comms, ptr(sends), ptr(recvs), counts, displs, dt, g.stream_ptr)
+                g.stream.synchronize()
+                got = [gh.to_host(recvs[r], dt)[:int(counts.sum())] for r in range(p)]
+            elif kind == "red":
+                root = n % p
+                want = [orc.reduce_to_root([x[:n] for x in pool], dt, op, root, algo=algo)]
+                H.reduce(g.comms, ptr(sends), ptr(recvs), n, dt, op, root, g.stream_ptr)
+                g.stream.synchronize()
+                got = [gh.to_host(recvs[root], dt)[:n]]
+            else:
+                root = n % p
+                for r in range(p):
+                    recvs[r][:n * unit].copy_(sends[r][:n * unit])
+                torch.cuda.synchronize()
+                want = [pool[root][:n]] * p
+                H.broadcast(g.comms, ptr(recvs), n, dt, root, g.stream_ptr)
+                g.stream.synchronize()
+                got = [gh.to_host(recvs[r], dt)[:n] for r in range(p)]
+            for r in range(len(want)):
+                assert gh.same(dt, got[r], want[r]), (seed, call, kind, r)
+        for r in range(p):
+            assert np.array_equal(gh.to_host(sends[r], dt), pool[r]), ("send buffer changed", r)
+    finally:
+        g.close()
