@@ -551,6 +551,15 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
             pl.rec.func = func;
             pl.rec.nitems = uint32_t(descs.size());
             pl.rec.ntiles = tiles;
+            // equal slices (the usual collective): the kernels find a tile's item without searching the table
+            pl.rec.tilesPerItem = TilesOf(descs[0].bytes);
+            for (size_t i = 0; i < descs.size(); i++) {
+                const uint32_t t = TilesOf(descs[i].bytes);
+                if (i + 1 < descs.size() ? t != pl.rec.tilesPerItem : t > pl.rec.tilesPerItem) {
+                    pl.rec.tilesPerItem = 0;
+                    break;
+                }
+            }
             pl.rec.grid = std::min(tiles, kind == int(KK_TREE) ? treeGrid : fusedGrid);
             pl.rec.fusedArgs = true;
             pending.push_back(pl);
@@ -629,6 +638,7 @@ void KernelArgs(LaunchRec &l, void **args)
         args[2] = &l.ntiles;
         args[3] = &l.srcPool;
         args[4] = &l.dstPool;
+        args[5] = &l.tilesPerItem;
     } else {
         args[2] = &l.nwhole;
         args[3] = &l.ntiles;
@@ -641,7 +651,7 @@ HcclResult BuildGraph(Prepared *pp)
     HIP_OK(hipGraphCreate(&pp->graph, 0));
     hipGraphNode_t prev = nullptr;
     for (LaunchRec &l : pp->launches) {
-        void *args[5];
+        void *args[6];
         KernelArgs(l, args);
         hipKernelNodeParams kp = {};
         kp.func = const_cast<void *>(l.func);
@@ -1217,7 +1227,7 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         HIP_OK(hipGraphLaunch(pp->exec, ls));
     } else {
         for (LaunchRec &l : pp->launches) {
-            void *args[5];
+            void *args[6];
             KernelArgs(l, args);
             HIP_OK(hipLaunchKernel(l.func, dim3(l.grid, 1, 1), dim3(kBlockThreads, 1, 1), args, 0, ls));
         }

@@ -353,6 +353,18 @@ template <typename D> __device__ __forceinline__ uint32_t FindDesc(const D *tabl
     return lo;
 }
 
+// Item of a tile in a fused launch.  When every item of the launch covers `tilesPerItem` tiles (the last one at most
+// as many; 0 = they differ), the index follows from the tile number and the table search, a chain of dependent loads
+// that is most of a small collective's time, is not needed.
+template <typename D> __device__ __forceinline__ uint32_t ItemOfTile(const D *table, uint32_t n, uint32_t tile, uint32_t tilesPerItem)
+{
+    if (tilesPerItem != 0) {
+        const uint32_t i = tile / tilesPerItem;
+        return i < n ? i : n - 1;
+    }
+    return FindDesc(table, n, tile);
+}
+
 constexpr uint32_t kVecPerLane = kTileBytes / (kBlockThreads * 16);   // 4
 
 // ---- one phase of copy / reduce steps -----------------------------------------------------------------
@@ -614,10 +626,10 @@ __device__ __forceinline__ void ChainElem(const FusedDesc &d, const void *const 
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
-    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool)
+    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem)
 {
     for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const FusedDesc d = items[FindDesc(items, nitems, tile)];
+        const FusedDesc d = items[ItemOfTile(items, nitems, tile, tilesPerItem)];
         const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
         const uint64_t left = d.bytes - off;
         const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
@@ -692,10 +704,10 @@ __device__ __forceinline__ void CopyVecPass(const void *s, void *const *__restri
 // definition may sit in this header; Variant is unused.)
 template <int Variant>
 __global__ void __launch_bounds__(kBlockThreads) CopyKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
-    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool)
+    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem)
 {
     for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const FusedDesc d = items[FindDesc(items, nitems, tile)];
+        const FusedDesc d = items[ItemOfTile(items, nitems, tile, tilesPerItem)];
         const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
         const uint64_t left = d.bytes - off;
         const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
@@ -753,7 +765,7 @@ typedef V4U __attribute__((address_space(3))) LdsV4U;
 
 template <int Variant>
 __global__ void __launch_bounds__(kBlockThreads) GatherKernel(const SegDesc *__restrict__ segs, uint32_t nsegs, uint32_t,
-    const void *const *__restrict__, void *const *__restrict__)
+    const void *const *__restrict__, void *const *__restrict__, uint32_t)
 {
     __shared__ __attribute__((aligned(16))) uint8_t lds[(kBlockThreads / 64) * kGatherLdsPerWave];
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -997,10 +1009,10 @@ __device__ __forceinline__ void TreeElem(const FusedDesc &d, const void *const *
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) TreeKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
-    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool)
+    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem)
 {
     for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const FusedDesc d = items[FindDesc(items, nitems, tile)];
+        const FusedDesc d = items[ItemOfTile(items, nitems, tile, tilesPerItem)];
         const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
         const uint64_t left = d.bytes - off;
         const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
@@ -1199,11 +1211,11 @@ __device__ __forceinline__ void StackElem(const FusedDesc &d, const void *const 
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) StackKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
-    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool)
+    uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem)
 {
     const uint32_t *opPool = reinterpret_cast<const uint32_t *>(items + nitems);
     for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const FusedDesc d = items[FindDesc(items, nitems, tile)];
+        const FusedDesc d = items[ItemOfTile(items, nitems, tile, tilesPerItem)];
         const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
         const uint64_t left = d.bytes - off;
         const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;

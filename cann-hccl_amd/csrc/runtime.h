@@ -53,7 +53,7 @@ struct LaunchRec {
     const void *func = nullptr;
     uint32_t grid = 0;
     // kernel arguments: step kernels take (table, nitems, nwhole, ntiles, flags), fused kernels
-    // (table, nitems, ntiles, srcPool, dstPool)
+    // (table, nitems, ntiles, srcPool, dstPool, tilesPerItem)
     const void *table = nullptr;
     uint32_t nitems = 0;
     uint32_t ntiles = 0;
@@ -61,6 +61,7 @@ struct LaunchRec {
     uint32_t flags = 0;
     const void *srcPool = nullptr;
     const void *dstPool = nullptr;
+    uint32_t tilesPerItem = 0;    // fused: every item covers this many tiles (the last at most as many); 0 = they differ
     bool fusedArgs = false;
 };
 
