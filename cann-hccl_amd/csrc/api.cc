@@ -1616,6 +1616,12 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
             return HCCL_E_PARA;
         }
         cfg.blocksPerCu = uint32_t(n);
+    } else if (k == "launch_cap_mib") {
+        long n = v == "auto" ? -1 : std::atol(value);
+        if (n < -1 || n > (1 << 20)) {
+            return HCCL_E_PARA;
+        }
+        cfg.launchCapMiB = int32_t(n);
     } else if (k == "blocking_arrive") {
         cfg.blockingArrive = v != "0";
     } else if (k == "arrive_timeout_ms") {

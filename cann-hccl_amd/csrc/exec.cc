@@ -471,19 +471,77 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                 pending.push_back(pl);
             }
         }
-        // one launch per kernel kind present
+        // one launch per kernel kind present, or several when a launch cap is set: the items in their order, cut where
+        // the bytes a launch moves (read and written) reach the cap
+        // A long launch slows down as it goes when its items move from buffer to buffer (all-to-all, scatter, reduce-
+        // scatter: workgroups drift apart and with them the regions of memory in use at one time), and launch boundaries
+        // bring them together again.  Measured, 8 ranks: all-to-all of 32 / 64 MiB per pair 774 / 1614 us in one launch,
+        // 688 / 1382 us cut at 512 MiB; reduce-scatter to 32 / 64 MiB per rank 408 / 825 us against 393 / 787 us.
+        // Collectives that sweep the same buffers from end to end (all-reduce, reduce, broadcast, all-gather) gain
+        // nothing or lose (all-reduce of 256 MiB per rank 756 us in one launch, 769 us cut at 512 MiB).
+        uint64_t capBytes = g->cfg.launchCapMiB > 0 ? uint64_t(g->cfg.launchCapMiB) << 20 : 0;
+        if (g->cfg.launchCapMiB < 0) {
+            const int coll = g->ctx->sig.coll;
+            // (the two-level reduce-scatter, whose items read their blocks group by group, loses 2 - 4 % and is left whole)
+            const bool hops = coll == COLL_ALLTOALLV || coll == COLL_SCATTER || coll == COLL_SENDRECV ||
+                (coll == COLL_REDUCESCATTER && g->cfg.servers <= 1);
+            capBytes = hops ? uint64_t(512) << 20 : 0;
+        }
         for (int kind : {int(KK_CHAIN), int(KK_TREE), int(KK_STACK)}) {
             std::vector<FusedDesc> descs;
             std::vector<const void *> srcPool;
             std::vector<uint32_t> opPool;      // stack items: one word per source-pool entry
             std::vector<void *> dstPool;
             uint32_t tiles = 0;
+            uint64_t traffic = 0;
             std::vector<char *> srcs, dsts;        // reused from item to item: an all-to-all-v has thousands
             std::vector<uintptr_t> addrs;
+            const void *func = reduceColl ? LookupKernel(dtype, op, KernelKind(kind)) : LookupCopyKernel(KernelKind(kind));
+            auto flush = [&]() {
+                if (descs.empty()) {
+                    return;
+                }
+                PendingLaunch pl;
+                // the op words of the stack kernel sit right behind its item table
+                pl.tableAt = b.Reserve(descs.size() * sizeof(FusedDesc) + opPool.size() * sizeof(uint32_t));
+                std::memcpy(b.host.data() + pl.tableAt, descs.data(), descs.size() * sizeof(FusedDesc));
+                if (!opPool.empty()) {
+                    std::memcpy(b.host.data() + pl.tableAt + descs.size() * sizeof(FusedDesc), opPool.data(),
+                        opPool.size() * sizeof(uint32_t));
+                }
+                pl.srcAt = b.Reserve(srcPool.size() * sizeof(void *));
+                std::memcpy(b.host.data() + pl.srcAt, srcPool.data(), srcPool.size() * sizeof(void *));
+                pl.dstAt = b.Reserve(dstPool.size() * sizeof(void *));
+                std::memcpy(b.host.data() + pl.dstAt, dstPool.data(), dstPool.size() * sizeof(void *));
+                pl.rec.func = func;
+                pl.rec.nitems = uint32_t(descs.size());
+                pl.rec.ntiles = tiles;
+                // equal slices (the usual collective): the kernels find a tile's item without searching the table
+                pl.rec.tilesPerItem = TilesOf(descs[0].bytes);
+                for (size_t i = 0; i < descs.size(); i++) {
+                    const uint32_t t = TilesOf(descs[i].bytes);
+                    if (i + 1 < descs.size() ? t != pl.rec.tilesPerItem : t > pl.rec.tilesPerItem) {
+                        pl.rec.tilesPerItem = 0;
+                        break;
+                    }
+                }
+                pl.rec.grid = std::min(tiles, kind == int(KK_TREE) ? treeGrid : fusedGrid);
+                pl.rec.fusedArgs = true;
+                pending.push_back(pl);
+                descs.clear();
+                srcPool.clear();
+                opPool.clear();
+                dstPool.clear();
+                tiles = 0;
+                traffic = 0;
+            };
             for (const FusedItem &it : pp->plan->fused) {
                 int want = it.kind == FK_TREE ? int(KK_TREE) : (it.kind == FK_STACK ? int(KK_STACK) : int(KK_CHAIN));
                 if (want != kind || shortSegment(it)) {
                     continue;
+                }
+                if (func == nullptr) {
+                    return HCCL_E_NOT_SUPPORT;
                 }
                 srcs.clear();
                 dsts.clear();
@@ -492,77 +550,56 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                     dsts.push_back(b.Ptr(d));
                     addrs.push_back(reinterpret_cast<uintptr_t>(dsts.back()));
                 }
+                uint32_t streams = uint32_t(dsts.size());
                 for (size_t k = 0; k < it.src.size(); k++) {
                     char *s = it.srcValid[k] ? b.Ptr(it.src[k]) : nullptr;
                     srcs.push_back(s);
                     if (s) {
                         addrs.push_back(reinterpret_cast<uintptr_t>(s));
+                        streams++;
                     }
                 }
                 uint64_t mask = 0;
                 for (size_t k = 0; k < it.accLeft.size() && k < 64; k++) {
                     mask |= uint64_t(it.accLeft[k] ? 1 : 0) << k;
                 }
-                SplitByAlignment(addrs, it.bytes, [&](uint64_t off, uint64_t n, uint32_t mode) {
-                    FusedDesc d;
-                    std::memset(&d, 0, sizeof(d));
-                    d.bytes = n;
-                    d.accLeftMask = mask;
-                    d.tile0 = tiles;
-                    d.mode = mode;
-                    d.nsrc = uint32_t(srcs.size());
-                    d.ndst = uint32_t(dsts.size());
-                    d.srcBase = uint32_t(srcPool.size());
-                    d.dstBase = uint32_t(dstPool.size());
-                    d.nleaf = it.nleaf;
-                    d.flags = fusedOrdinary ? kFusedOrdinaryStores : 0u;
-                    for (size_t k = 0; k < srcs.size(); k++) {
-                        srcPool.push_back(srcs[k] ? srcs[k] + off : nullptr);
-                        if (kind == int(KK_STACK)) {
-                            opPool.push_back(k < it.ops.size() ? it.ops[k] : 0u);
+                // an item that alone exceeds the cap goes in pieces of whole tiles
+                const uint64_t piece = capBytes == 0 ? ~uint64_t(0)
+                                                     : std::max<uint64_t>(kTileBytes, capBytes / streams / kTileBytes * kTileBytes);
+                SplitByAlignment(addrs, it.bytes, [&](uint64_t off0, uint64_t n0, uint32_t mode) {
+                    for (uint64_t at = 0; at < n0; at += piece) {
+                        const uint64_t off = off0 + at, n = std::min(piece, n0 - at);
+                        FusedDesc d;
+                        std::memset(&d, 0, sizeof(d));
+                        d.bytes = n;
+                        d.accLeftMask = mask;
+                        d.tile0 = tiles;
+                        d.mode = mode;
+                        d.nsrc = uint32_t(srcs.size());
+                        d.ndst = uint32_t(dsts.size());
+                        d.srcBase = uint32_t(srcPool.size());
+                        d.dstBase = uint32_t(dstPool.size());
+                        d.nleaf = it.nleaf;
+                        d.flags = fusedOrdinary ? kFusedOrdinaryStores : 0u;
+                        for (size_t k = 0; k < srcs.size(); k++) {
+                            srcPool.push_back(srcs[k] ? srcs[k] + off : nullptr);
+                            if (kind == int(KK_STACK)) {
+                                opPool.push_back(k < it.ops.size() ? it.ops[k] : 0u);
+                            }
+                        }
+                        for (char *t : dsts) {
+                            dstPool.push_back(t + off);
+                        }
+                        tiles += TilesOf(n);
+                        traffic += n * streams;
+                        descs.push_back(d);
+                        if (capBytes != 0 && traffic >= capBytes) {
+                            flush();
                         }
                     }
-                    for (char *t : dsts) {
-                        dstPool.push_back(t + off);
-                    }
-                    tiles += TilesOf(n);
-                    descs.push_back(d);
                 });
             }
-            if (descs.empty()) {
-                continue;
-            }
-            const void *func = reduceColl ? LookupKernel(dtype, op, KernelKind(kind)) : LookupCopyKernel(KernelKind(kind));
-            if (func == nullptr) {
-                return HCCL_E_NOT_SUPPORT;
-            }
-            PendingLaunch pl;
-            // the op words of the stack kernel sit right behind its item table
-            pl.tableAt = b.Reserve(descs.size() * sizeof(FusedDesc) + opPool.size() * sizeof(uint32_t));
-            std::memcpy(b.host.data() + pl.tableAt, descs.data(), descs.size() * sizeof(FusedDesc));
-            if (!opPool.empty()) {
-                std::memcpy(b.host.data() + pl.tableAt + descs.size() * sizeof(FusedDesc), opPool.data(),
-                    opPool.size() * sizeof(uint32_t));
-            }
-            pl.srcAt = b.Reserve(srcPool.size() * sizeof(void *));
-            std::memcpy(b.host.data() + pl.srcAt, srcPool.data(), srcPool.size() * sizeof(void *));
-            pl.dstAt = b.Reserve(dstPool.size() * sizeof(void *));
-            std::memcpy(b.host.data() + pl.dstAt, dstPool.data(), dstPool.size() * sizeof(void *));
-            pl.rec.func = func;
-            pl.rec.nitems = uint32_t(descs.size());
-            pl.rec.ntiles = tiles;
-            // equal slices (the usual collective): the kernels find a tile's item without searching the table
-            pl.rec.tilesPerItem = TilesOf(descs[0].bytes);
-            for (size_t i = 0; i < descs.size(); i++) {
-                const uint32_t t = TilesOf(descs[i].bytes);
-                if (i + 1 < descs.size() ? t != pl.rec.tilesPerItem : t > pl.rec.tilesPerItem) {
-                    pl.rec.tilesPerItem = 0;
-                    break;
-                }
-            }
-            pl.rec.grid = std::min(tiles, kind == int(KK_TREE) ? treeGrid : fusedGrid);
-            pl.rec.fusedArgs = true;
-            pending.push_back(pl);
+            flush();
         }
     }
     if (pending.empty()) {
@@ -689,6 +726,7 @@ std::string CacheKey(const Group *g, int algo)
             (uint64_t(uint32_t(g->cfg.algo + 1) & 0xfu) << 48) | (uint64_t(g->cfg.deterministic) << 56) | (uint64_t(g->cfg.level0Rings) << 57) |
             (uint64_t(uint32_t(g->cfg.fusedStores + 1)) << 60) | (uint64_t(g->cfg.stepSweep) << 62), g->p};
     put(head, sizeof(head));
+    put(&g->cfg.launchCapMiB, sizeof(g->cfg.launchCapMiB));
     put(g->ctx->send.data(), g->ctx->send.size() * sizeof(void *));
     put(g->ctx->recv.data(), g->ctx->recv.size() * sizeof(void *));
     if (g->ctx->sig.coll == COLL_ALLTOALLV) {

@@ -706,12 +706,29 @@ template <int Variant>
 __global__ void __launch_bounds__(kBlockThreads) CopyKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem)
 {
-    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const FusedDesc d = items[ItemOfTile(items, nitems, tile, tilesPerItem)];
+    uint32_t tile = blockIdx.x;
+    if (tile >= ntiles) {
+        return;
+    }
+    // The item of a tile costs a chain of dependent loads (table, item, pointer).  A workgroup that stays inside one
+    // item from one tile to the next keeps what it has; when the next tile lies in another item, that item is looked
+    // up before the current tile's data is loaded, so that the chain completes behind those loads.
+    FusedDesc d = items[ItemOfTile(items, nitems, tile, tilesPerItem)];
+    const void *s = srcPool[d.srcBase];
+    uint32_t dEnd = d.tile0 + uint32_t((d.bytes + kTileBytes - 1) / kTileBytes);
+    for (;;) {
+        const uint32_t next = tile + gridDim.x;
+        FusedDesc dn = d;
+        const void *sn = s;
+        uint32_t dnEnd = dEnd;
+        if (next < ntiles && next >= dEnd) {
+            dn = items[ItemOfTile(items, nitems, next, tilesPerItem)];
+            sn = srcPool[dn.srcBase];
+            dnEnd = dn.tile0 + uint32_t((dn.bytes + kTileBytes - 1) / kTileBytes);
+        }
         const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
         const uint64_t left = d.bytes - off;
         const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
-        const void *s = srcPool[d.srcBase];
         void *const *dst = dstPool + d.dstBase;
         if (d.mode == ACC_ELEM) {
             for (uint32_t i = threadIdx.x; i < n; i += kBlockThreads) {
@@ -746,6 +763,13 @@ __global__ void __launch_bounds__(kBlockThreads) CopyKernel(const FusedDesc *__r
                 }
             }
         }
+        if (next >= ntiles) {
+            break;
+        }
+        tile = next;
+        d = dn;
+        s = sn;
+        dEnd = dnEnd;
     }
 }
 

@@ -44,6 +44,8 @@ struct GroupConfig {
     int stepSweep = 1;               // step kernel: 0 every phase walks its steps forwards, 1 every other phase backwards
     uint32_t cacheEntries = 1024;    // prepared collectives kept (distinct sizes / buffers / settings)
     uint32_t blocksPerCu = 0;             // workgroups per CU; 0 = per-kernel default
+    int32_t launchCapMiB = -1;            // fused issue: cut the work into launches that move about this much; 0 = one launch per
+                                          // kernel kind, -1 = the library decides per collective
     bool blockingArrive = false;          // ranks wait inside the call until the collective is issued
     uint32_t arriveTimeoutMs = 1800 * 1000;
 };

@@ -50,6 +50,10 @@ extern "C" {
  *   "cache_entries" how many prepared collectives (distinct sizes, buffers, settings) the group keeps (default 1024);
  *                   when full, the library waits for the device once and starts over
  *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
+ *   "launch_cap_mib" fused issue: the items go out in several launches, cut where a launch has moved about this many
+ *                                MiB (read and written); "0": one launch per kernel kind; "auto" (default): 512 for the
+ *                                collectives whose items hop from buffer to buffer (all-to-all family, scatter, send /
+ *                                receive, one-level reduce-scatter), whole for the others
  *   "blocking_arrive" "0" | "1"  a rank's call waits inside the library until the group is complete.  With "0" (default)
  *                                a call returns at once and the last rank's call issues the collective; what a rank's
  *                                stream held when the rank called runs before the collective, but work queued on that

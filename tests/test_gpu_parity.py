@@ -439,6 +439,55 @@ def test_staged_uniform_alltoall_over_servers():
             g.close()
 
 
+def test_fused_work_cut_into_several_launches(orc):
+    # `launch_cap_mib` cuts the fused items into launches of about that much traffic, items larger than the cap into
+    # pieces of whole tiles.  With a cap of 1 MiB every kind of fused kernel (chain, tree, stack, copy) goes out in many
+    # launches, misaligned buffers and ragged ends included; the results stay the checker's.
+    n = 300000 + 77
+    for p, algo, servers in ((8, RING, 1), (8, RHD, 1), (6, RHD, 1), (8, MESH, 1), (8, RHD, 2)):
+        g = _group(p, algo, fuse=1, launch_cap_mib=1, **({"servers": servers} if servers > 1 else {}))
+        try:
+            for dt, op, pad in ((FP32, SUM, 0), (BF16, SUM, 2), (INT32, MAX, 16)):
+                print("launch cap", ALGO_NAME[algo], "p", p, "servers", servers, "type", dt, flush=True)
+                ins = _ins(dt, p, n, 400 + p + dt)
+                if servers > 1:
+                    want = orc.allreduce_two_level(ins, dt, op, servers, level1=RHD)
+                else:
+                    want = orc.allreduce(ins, dt, op, algo=algo)
+                outs, _ = gh.all_reduce(g, ins, dt, op, pad=pad)
+                info = g.info()
+                assert info["fused"] == 1 and info["launches"] > 4, info
+                for r in range(p):
+                    assert gh.same(dt, outs[r], want[r]), (p, algo, servers, dt, "all-reduce", r)
+                if servers == 1:
+                    m = n // p
+                    ins_rs = [x[:m * p] for x in ins]
+                    want = orc.reducescatter(ins_rs, dt, op, algo=algo)
+                    outs, _ = gh.reduce_scatter(g, ins_rs, dt, op, pad=pad)
+                    assert g.info()["launches"] >= 2
+                    for r in range(p):
+                        assert gh.same(dt, outs[r], want[r]), (p, algo, dt, "reduce-scatter", r)
+                    outs = gh.all_gather(g, [x[:m] for x in ins], dt, pad=pad)
+                    whole = np.concatenate([x[:m] for x in ins])
+                    for r in range(p):
+                        assert np.array_equal(outs[r], whole), (p, algo, dt, "all-gather", r)
+        finally:
+            g.close()
+    # all-to-all-v: blocks of up to 1.2 MiB, so that single blocks are cut as well
+    p = 8
+    cnt, sdis, rcnt, rdis, sl, rl = _a2av_case(p, 77, max_count=300000)
+    sends = [(np.arange(k, dtype=np.int32) + (r << 24)) for r, k in enumerate(sl)]
+    want = [np.full(k, -1, np.int32) for k in rl]
+    assert orc.alltoallv(sends, cnt, sdis, want, rcnt, rdis, INT32) == 0
+    g = gh.Group(p, fuse=1, launch_cap_mib=1)
+    try:
+        outs = gh.all_to_all_v(g, sends, cnt, sdis, rl, rcnt, rdis, INT32)
+        assert g.info()["launches"] > 4
+        assert all(np.array_equal(outs[r], want[r]) for r in range(p))
+    finally:
+        g.close()
+
+
 def test_alltoallv_asymmetric_tables_fail(orc):
     p = 4
     g = gh.Group(p)
