@@ -628,8 +628,22 @@ template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem)
 {
-    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const FusedDesc d = items[ItemOfTile(items, nitems, tile, tilesPerItem)];
+    uint32_t tile = blockIdx.x;
+    if (tile >= ntiles) {
+        return;
+    }
+    // a workgroup keeps its item while its tiles stay inside it; the next item is looked up ahead of the current
+    // tile's loads (see the copy kernel)
+    FusedDesc d = items[ItemOfTile(items, nitems, tile, tilesPerItem)];
+    uint32_t dEnd = d.tile0 + uint32_t((d.bytes + kTileBytes - 1) / kTileBytes);
+    for (;;) {
+        const uint32_t next = tile + gridDim.x;
+        FusedDesc dn = d;
+        uint32_t dnEnd = dEnd;
+        if (next < ntiles && next >= dEnd) {
+            dn = items[ItemOfTile(items, nitems, next, tilesPerItem)];
+            dnEnd = dn.tile0 + uint32_t((dn.bytes + kTileBytes - 1) / kTileBytes);
+        }
         const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
         const uint64_t left = d.bytes - off;
         const uint32_t n = left < kTileBytes ? uint32_t(left) : kTileBytes;
@@ -665,6 +679,12 @@ __global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__
                 }
             }
         }
+        if (next >= ntiles) {
+            break;
+        }
+        tile = next;
+        d = dn;
+        dEnd = dnEnd;
     }
 }
 
