@@ -276,6 +276,20 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
         b.scratch = g->scratch;
     }
     std::vector<PendingLaunch> pending;
+    // A long launch slows down as it goes when its items move from buffer to buffer (all-to-all, scatter, reduce-
+    // scatter: workgroups drift apart and with them the regions of memory in use at one time), and launch boundaries
+    // bring them together again.  Measured, 8 ranks: all-to-all of 32 / 64 MiB per pair 774 / 1614 us in one launch,
+    // 688 / 1382 us cut at 512 MiB; reduce-scatter to 32 / 64 MiB per rank 408 / 825 us against 393 / 787 us.
+    // Collectives that sweep the same buffers from end to end (all-reduce, reduce, broadcast, all-gather) gain
+    // nothing or lose (all-reduce of 256 MiB per rank 756 us in one launch, 769 us cut at 512 MiB).
+    uint64_t capBytes = g->cfg.launchCapMiB > 0 ? uint64_t(g->cfg.launchCapMiB) << 20 : 0;
+    if (g->cfg.launchCapMiB < 0) {
+        const int coll = g->ctx->sig.coll;
+        // (the two-level reduce-scatter, whose items read their blocks group by group, loses 2 - 4 % and is left whole)
+        const bool hops = coll == COLL_ALLTOALLV || coll == COLL_SCATTER || coll == COLL_SENDRECV ||
+            (coll == COLL_REDUCESCATTER && g->cfg.servers <= 1);
+        capBytes = hops ? uint64_t(512) << 20 : 0;
+    }
     // Launch width.  Streaming kernels on this part run best with few, fat workgroups as long as a
     // lane keeps enough memory operations in flight: 1 workgroup per CU when an item touches 8 or
     // more streams (sources + destinations), more when it touches fewer (measured on MI355X: 8 -> 8
@@ -298,10 +312,12 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
         // That holds for shapes that write as much as they read or more, and for everything much larger than the
         // memory-side cache.  Many sources into one destination (reduce-scatter, reduce) of 8- and 16-bit elements,
         // where a combine costs several instructions, run better wide up to about a gigabyte in all (measured, bf16
-        // sum: 8 ranks x 64 MiB 104 us at 1 per CU, 99 at 8; 16 ranks x 64 MiB 196 / 189; 8 ranks x 256 MiB 415 / 421,
-        // so not there; fp32 within a percent either way at every size).
+        // sum: 8 ranks x 64 MiB 104 us at 1 per CU, 99 at 8; 16 ranks x 64 MiB 196 / 189; a reduce of 8 x 256 MiB in one
+        // launch 416 / 423, so not there, but a reduce-scatter of that size, which goes out in launches of 512 MiB, 413 /
+        // 396; fp32 within a percent either way at every size).
+        const double launchBytes = capBytes != 0 ? std::min(streamBytes, double(capBytes)) : streamBytes;
         if (fusedPerCu == 1 && reduceColl && DtypeSize(dtype) <= 2 && storeBytes * 5.0 <= streamBytes &&
-            streamBytes <= 1.25 * 1024.0 * 1024.0 * 1024.0) {
+            launchBytes <= 1.25 * 1024.0 * 1024.0 * 1024.0) {
             fusedPerCu = 8;
         }
         // Plain copies (one source, one destination) go through the copy kernel, which really gets the
@@ -471,22 +487,8 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                 pending.push_back(pl);
             }
         }
-        // one launch per kernel kind present, or several when a launch cap is set: the items in their order, cut where
-        // the bytes a launch moves (read and written) reach the cap
-        // A long launch slows down as it goes when its items move from buffer to buffer (all-to-all, scatter, reduce-
-        // scatter: workgroups drift apart and with them the regions of memory in use at one time), and launch boundaries
-        // bring them together again.  Measured, 8 ranks: all-to-all of 32 / 64 MiB per pair 774 / 1614 us in one launch,
-        // 688 / 1382 us cut at 512 MiB; reduce-scatter to 32 / 64 MiB per rank 408 / 825 us against 393 / 787 us.
-        // Collectives that sweep the same buffers from end to end (all-reduce, reduce, broadcast, all-gather) gain
-        // nothing or lose (all-reduce of 256 MiB per rank 756 us in one launch, 769 us cut at 512 MiB).
-        uint64_t capBytes = g->cfg.launchCapMiB > 0 ? uint64_t(g->cfg.launchCapMiB) << 20 : 0;
-        if (g->cfg.launchCapMiB < 0) {
-            const int coll = g->ctx->sig.coll;
-            // (the two-level reduce-scatter, whose items read their blocks group by group, loses 2 - 4 % and is left whole)
-            const bool hops = coll == COLL_ALLTOALLV || coll == COLL_SCATTER || coll == COLL_SENDRECV ||
-                (coll == COLL_REDUCESCATTER && g->cfg.servers <= 1);
-            capBytes = hops ? uint64_t(512) << 20 : 0;
-        }
+        // one launch per kernel kind present, or several under a launch cap: the items in their order, cut where the
+        // bytes a launch moves (read and written) reach the cap
         for (int kind : {int(KK_CHAIN), int(KK_TREE), int(KK_STACK)}) {
             std::vector<FusedDesc> descs;
             std::vector<const void *> srcPool;
