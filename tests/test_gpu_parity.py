@@ -484,6 +484,23 @@ def test_fused_work_cut_into_several_launches(orc):
         outs = gh.all_to_all_v(g, sends, cnt, sdis, rl, rcnt, rdis, INT32)
         assert g.info()["launches"] > 4
         assert all(np.array_equal(outs[r], want[r]) for r in range(p))
+        # the same all-reduce three times on the same buffers: from the second call on the many launches are a graph
+        n = 3 << 20
+        ins = _ins(FP32, p, n, 4242)
+        want_ar = orc.allreduce(ins, FP32, SUM)
+        dev_in = [gh.to_dev(x) for x in ins]
+        dev_out = [gh.empty_dev(n * 4) for _ in range(p)]
+        torch.cuda.synchronize()
+        for rep in range(3):
+            for t in dev_out:
+                t.fill_(0x5A)
+            torch.cuda.synchronize()
+            H.all_reduce(g.comms, [t.data_ptr() for t in dev_in], [t.data_ptr() for t in dev_out], n, FP32, SUM, g.stream_ptr)
+            g.stream.synchronize()
+            info = g.info()
+            assert info["fused"] == 1 and info["launches"] >= 12 and info["graph"] == (1 if rep else 0), (rep, info)
+            for r in range(p):
+                assert gh.same(FP32, gh.to_host(dev_out[r], FP32), want_ar[r]), (rep, r)
     finally:
         g.close()
 
