@@ -127,6 +127,10 @@ void ApplyEnv(GroupConfig *cfg)
             cfg->blocksPerCu = uint32_t(v);
         }
     }
+    if (const char *e = std::getenv("HCCL_AMD_TEAM")) {
+        const std::string v(e);
+        cfg->team = v == "1" ? 1 : (v == "0" ? 0 : -1);
+    }
     if (const char *e = std::getenv("HCCL_AMD_BLOCKING_ARRIVE")) {
         cfg->blockingArrive = std::atoi(e) != 0;
     }
@@ -1573,6 +1577,14 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
             cfg.fusedStores = 0;
         } else if (v == "ordinary") {
             cfg.fusedStores = 1;
+        } else {
+            return HCCL_E_PARA;
+        }
+    } else if (k == "team") {
+        if (v == "auto") {
+            cfg.team = -1;
+        } else if (v == "0" || v == "1") {
+            cfg.team = v == "1" ? 1 : 0;
         } else {
             return HCCL_E_PARA;
         }

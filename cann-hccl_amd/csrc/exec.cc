@@ -86,6 +86,18 @@ HcclResult EnsureDevice(Group *g, bool quiet)
         hipFuncAttributes attr;
         HIP_OK(hipFuncGetAttributes(&attr, LookupCopyKernel(KK_STEP)));
     }
+    // the team kernels park their results in more LDS than a kernel gets without asking
+    for (int dt = 0; dt <= 11; dt++) {
+        for (int op = 0; op <= 3; op++) {
+            for (KernelKind kind : {KK_TEAM_CHAIN, KK_TEAM_TREE, KK_TEAM_STACK}) {
+                const void *f = LookupKernel(dt, op, kind);
+                if (f != nullptr) {
+                    HIP_OK(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, int(kTeamDynamicLds)));
+                }
+            }
+        }
+    }
+    HIP_OK(hipFuncSetAttribute(LookupCopyKernel(KK_TEAM_CHAIN), hipFuncAttributeMaxDynamicSharedMemorySize, int(kTeamDynamicLds)));
     g->deviceReady = true;
     return HCCL_SUCCESS;
 }
@@ -188,13 +200,14 @@ template <typename F> void SplitByAlignment(const std::vector<uintptr_t> &addrs,
 }
 
 constexpr size_t kGraphMinLaunches = 12;   // fewer launches go out one by one
+constexpr uint32_t kTeamMinRounds = 4;     // the team kernels are chosen for launches of at least this many rounds
 constexpr size_t kAsyncUploadBytes = 4 * kNoAllocUploadBytes;   // tables up to this size are uploaded by launches
 
 uint32_t TilesOf(uint64_t bytes) { return uint32_t((bytes + kTileBytes - 1) / kTileBytes); }
 
 struct PendingLaunch {
     LaunchRec rec;
-    size_t tableAt = 0, srcAt = 0, dstAt = 0;
+    size_t tableAt = 0, srcAt = 0, dstAt = 0, ctrAt = 0;
     bool gather = false;     // no pointer pools
 };
 
@@ -529,6 +542,35 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                 }
                 pl.rec.grid = std::min(tiles, kind == int(KK_TREE) ? treeGrid : fusedGrid);
                 pl.rec.fusedArgs = true;
+                // Team form (kernels_team.h): pays when every workgroup has much to read or to write per tile and the
+                // launch runs for many rounds.  Measured on MI355X with streams of 256 MiB (sources : destinations,
+                // plain / team, TB/s): 8 : 8 5.3 / 5.9, 1 : 8 4.9 / 5.9, 1 : 7 4.9 / 5.8, 4 : 4 5.4 / 5.7, 8 : 1
+                // 5.8 / 6.0; 2 : 2 5.5 / 5.3, 2 : 1 5.8 / 4.9, 1 : 1 5.8 / 4.2 (a round is then too short for its barrier).
+                const KernelKind teamKind = kind == int(KK_TREE) ? KK_TEAM_TREE : (kind == int(KK_STACK) ? KK_TEAM_STACK : KK_TEAM_CHAIN);
+                const void *teamFunc = reduceColl ? LookupKernel(dtype, op, teamKind) : LookupCopyKernel(teamKind);
+                const bool teamFits = teamFunc != nullptr && g->numCu >= kTeamXcds && g->numCu % kTeamXcds == 0 && g->cfg.blocksPerCu == 0;
+                bool team = teamFits && g->cfg.team == 1;
+                if (teamFits && g->cfg.team < 0) {
+                    double storeStreams = 0, allStreams = 0, bytes = 0;
+                    for (const FusedDesc &d : descs) {
+                        uint32_t nsrc = 0;
+                        for (uint32_t k = 0; k < d.nsrc; k++) {
+                            nsrc += srcPool[d.srcBase + k] != nullptr ? 1u : 0u;
+                        }
+                        storeStreams += double(d.ndst) * double(d.bytes);
+                        allStreams += double(d.ndst + nsrc) * double(d.bytes);
+                        bytes += double(d.bytes);
+                    }
+                    team = bytes > 0 && storeStreams >= 4.0 * bytes && allStreams >= 8.0 * bytes &&
+                        tiles >= kTeamMinRounds * kTeamTiles * g->numCu;
+                }
+                if (team) {
+                    pl.rec.func = teamFunc;
+                    pl.rec.team = true;
+                    pl.rec.grid = g->numCu;
+                    pl.rec.dynamicLds = kTeamDynamicLds;
+                    pl.ctrAt = b.Reserve(kTeamCtrBytes);     // zero in the image, and zero again after every launch
+                }
                 pending.push_back(pl);
                 descs.clear();
                 srcPool.clear();
@@ -664,6 +706,9 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
             pl.rec.srcPool = base + pl.srcAt;
             pl.rec.dstPool = base + pl.dstAt;
         }
+        if (pl.rec.team) {
+            pl.rec.teamCtr = base + pl.ctrAt;
+        }
         pp->launches.push_back(pl.rec);
     }
     return HCCL_SUCCESS;
@@ -678,6 +723,7 @@ void KernelArgs(LaunchRec &l, void **args)
         args[3] = &l.srcPool;
         args[4] = &l.dstPool;
         args[5] = &l.tilesPerItem;
+        args[6] = &l.teamCtr;      // read by the team kernels only
     } else {
         args[2] = &l.nwhole;
         args[3] = &l.ntiles;
@@ -690,13 +736,13 @@ HcclResult BuildGraph(Prepared *pp)
     HIP_OK(hipGraphCreate(&pp->graph, 0));
     hipGraphNode_t prev = nullptr;
     for (LaunchRec &l : pp->launches) {
-        void *args[6];
+        void *args[7];
         KernelArgs(l, args);
         hipKernelNodeParams kp = {};
         kp.func = const_cast<void *>(l.func);
         kp.gridDim = dim3(l.grid, 1, 1);
         kp.blockDim = dim3(kBlockThreads, 1, 1);
-        kp.sharedMemBytes = 0;
+        kp.sharedMemBytes = l.dynamicLds;
         kp.kernelParams = args;
         kp.extra = nullptr;
         hipGraphNode_t node = nullptr;
@@ -729,6 +775,7 @@ std::string CacheKey(const Group *g, int algo)
             (uint64_t(uint32_t(g->cfg.fusedStores + 1)) << 60) | (uint64_t(g->cfg.stepSweep) << 62), g->p};
     put(head, sizeof(head));
     put(&g->cfg.launchCapMiB, sizeof(g->cfg.launchCapMiB));
+    put(&g->cfg.team, sizeof(g->cfg.team));
     put(g->ctx->send.data(), g->ctx->send.size() * sizeof(void *));
     put(g->ctx->recv.data(), g->ctx->recv.size() * sizeof(void *));
     if (g->ctx->sig.coll == COLL_ALLTOALLV) {
@@ -1267,9 +1314,9 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         HIP_OK(hipGraphLaunch(pp->exec, ls));
     } else {
         for (LaunchRec &l : pp->launches) {
-            void *args[6];
+            void *args[7];
             KernelArgs(l, args);
-            HIP_OK(hipLaunchKernel(l.func, dim3(l.grid, 1, 1), dim3(kBlockThreads, 1, 1), args, 0, ls));
+            HIP_OK(hipLaunchKernel(l.func, dim3(l.grid, 1, 1), dim3(kBlockThreads, 1, 1), args, l.dynamicLds, ls));
         }
     }
     g->launchStreams[g->opSerial % 8] = ls;

@@ -69,7 +69,22 @@ struct SegDesc {
 };
 constexpr uint32_t kGatherMaxBytes = 8192;
 
-enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_STACK = 3, KK_COUNT = 4, KK_GATHER = 4 };
+enum KernelKind : int {
+    KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_STACK = 3,
+    KK_TEAM_CHAIN = 4, KK_TEAM_TREE = 5, KK_TEAM_STACK = 6,   // team forms of the fused kernels, see below
+    KK_COUNT = 7,
+    KK_GATHER = 7                                              // copy kernel table only
+};
+
+// Team form of a fused kernel: the workgroups of one XCD read their tiles together, park the results in LDS, and write
+// them together (kernels_team.h).  Launched with a multiple of kTeamXcds workgroups (one per CU) and kTeamLdsBytes of
+// dynamic LDS; takes one more argument, the team counters: kTeamXcds * kTeamCtrStride zero-initialised uint32 in
+// device memory that belong to this launch alone (the kernel leaves them zero again).
+constexpr uint32_t kTeamTiles = 8;        // tiles a workgroup parks per round
+constexpr uint32_t kTeamXcds = 8;
+constexpr uint32_t kTeamCtrStride = 16;   // uint32 per XCD (64 bytes: arrivals, finished workgroups, gave-up flag)
+constexpr uint32_t kTeamCtrBytes = kTeamXcds * kTeamCtrStride * 4;
+constexpr uint32_t kTeamDynamicLds = kTeamTiles * kTileBytes;
 
 // Kernel entry for (data type, reduce op, kind); nullptr if the combination is not built.
 // Signatures:
@@ -77,12 +92,13 @@ enum KernelKind : int { KK_STEP = 0, KK_CHAIN = 1, KK_TREE = 2, KK_STACK = 3, KK
 //                      steps whose tiles are all whole and ACC_VEC16 come first: tiles [0, nwhole)
 //   KK_CHAIN / KK_TREE / KK_STACK
 //                      (const FusedDesc *items, uint32_t nitems, uint32_t ntiles,
-//                       const void *const *srcPool, void *const *dstPool)
+//                       const void *const *srcPool, void *const *dstPool, uint32_t tilesPerItem)
+//   KK_TEAM_*          the same and (uint32_t *teamCtr)
 const void *LookupKernel(int hcclDataType, int hcclReduceOp, KernelKind kind);
 
 //   KK_GATHER          (const SegDesc *segs, uint32_t nsegs, uint32_t unused, const void *unused, void *unused)
 //                      copy kernel table only
-// Byte-wise variants for pure data movement (all-gather, all-to-all-v): KK_STEP, KK_CHAIN and KK_GATHER.
+// Byte-wise variants for pure data movement (all-gather, all-to-all-v): KK_STEP, KK_CHAIN, KK_TEAM_CHAIN and KK_GATHER.
 const void *LookupCopyKernel(KernelKind kind);
 
 }  // namespace hcclamd

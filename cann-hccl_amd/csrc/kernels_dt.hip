@@ -1,6 +1,6 @@
 // Instantiates the kernels for one HcclDataType (selected with -DHCCL_DT=<enum value>), so that the
 // twelve element types build in parallel, plus the byte-wise copy variants (-DHCCL_DT=255).
-#include "kernels_impl.h"
+#include "kernels_team.h"
 
 namespace hcclamd {
 
@@ -52,10 +52,11 @@ using DT = uint8_t;
 
 #if HCCL_DT == 255
 // pure data movement: the step kernel's copy path and the copy kernel
-extern const void *const HCCL_CAT(kKernels_, HCCL_DT_NAME)[3] = {
+extern const void *const HCCL_CAT(kKernels_, HCCL_DT_NAME)[4] = {
     reinterpret_cast<const void *>(&StepKernel<DT, ROP_SUM>),
     reinterpret_cast<const void *>(&CopyKernel<0>),
     reinterpret_cast<const void *>(&GatherKernel<0>),
+    reinterpret_cast<const void *>(&TeamCopyKernel<0>),
 };
 #else
 #define HCCL_ROW(OP)                                                     \
@@ -64,6 +65,9 @@ extern const void *const HCCL_CAT(kKernels_, HCCL_DT_NAME)[3] = {
         reinterpret_cast<const void *>(&ChainKernel<DT, OP>),            \
         reinterpret_cast<const void *>(&TreeKernel<DT, OP>),             \
         reinterpret_cast<const void *>(&StackKernel<DT, OP>),            \
+        reinterpret_cast<const void *>(&TeamChainKernel<DT, OP>),        \
+        reinterpret_cast<const void *>(&TeamTreeKernel<DT, OP>),         \
+        reinterpret_cast<const void *>(&TeamStackKernel<DT, OP>),        \
     }
 extern const void *const HCCL_CAT(kKernels_, HCCL_DT_NAME)[4][KK_COUNT] = {
     HCCL_ROW(ROP_SUM), HCCL_ROW(ROP_PROD), HCCL_ROW(ROP_MAX), HCCL_ROW(ROP_MIN),

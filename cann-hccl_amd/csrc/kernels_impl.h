@@ -283,6 +283,10 @@ typedef uint32_t V4U __attribute__((ext_vector_type(4), aligned(1)));
 typedef V4 HCCL_GLOBAL GlobalV4;
 typedef V4U HCCL_GLOBAL GlobalV4U;
 
+// 16 bytes in LDS (the gather kernel's staging area; the tiles a team kernel holds between its read and write phases)
+typedef V4 __attribute__((address_space(3))) LdsV4;
+typedef V4U __attribute__((address_space(3))) LdsV4U;
+
 template <uint32_t MODE> __device__ __forceinline__ V4 Load16(const void *base, uint64_t byteOff)
 {
     const char *p = static_cast<const char *>(base) + byteOff;
@@ -535,9 +539,11 @@ template <uint32_t MODE, bool ORDINARY = false> __device__ __forceinline__ void 
 
 // One pass over kChainVec * 256 vectors starting at vector vecBase of the tile.
 // FULL: every lane has all its vectors inside the tile (no per-lane guards).
-template <typename T, int OP, uint32_t MODE, bool FULL, bool ORDINARY = false>
+// PARK: the results are not stored to the destinations but left in LDS, vector i of the tile at park[i] (the team
+// kernels write them out later); dst is not used then.
+template <typename T, int OP, uint32_t MODE, bool FULL, bool ORDINARY = false, bool PARK = false>
 __device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *const *__restrict__ src,
-    void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec)
+    void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec, LdsV4 *park = nullptr)
 {
     const uint32_t tid = threadIdx.x;
     uint64_t pos[kChainVec];
@@ -593,6 +599,15 @@ __device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *con
                 }
             }
         }
+    }
+    if (PARK) {
+#pragma unroll
+        for (uint32_t u = 0; u < kChainVec; u++) {
+            if (live[u]) {
+                park[vecBase + u * kBlockThreads + tid] = acc[u];
+            }
+        }
+        return;
     }
     const uint32_t ndst = d.ndst;
     for (uint32_t k = 0; k < ndst; k++) {
@@ -693,9 +708,9 @@ __global__ void __launch_bounds__(kBlockThreads) ChainKernel(const FusedDesc *__
 // workgroups fit on a CU where the chain kernel fits two.  A copy keeps only 4 loads per lane in flight, and its
 // rate comes from how many waves do that at once (measured, 1 GiB copy: 5.1 TB/s through the chain kernel,
 // 6.3 TB/s for a plain copy kernel at full occupancy).
-template <uint32_t MODE, bool FULL, bool ORDINARY = false>
+template <uint32_t MODE, bool FULL, bool ORDINARY = false, bool PARK = false>
 __device__ __forceinline__ void CopyVecPass(const void *s, void *const *__restrict__ dst, uint32_t ndst, uint64_t off,
-    uint32_t vecBase, uint32_t nvec)
+    uint32_t vecBase, uint32_t nvec, LdsV4 *park = nullptr)
 {
     uint64_t pos[kChainVec];
     bool live[kChainVec];
@@ -708,6 +723,15 @@ __device__ __forceinline__ void CopyVecPass(const void *s, void *const *__restri
         if (live[u]) {
             v[u] = Load16<MODE>(s, pos[u]);
         }
+    }
+    if (PARK) {
+#pragma unroll
+        for (uint32_t u = 0; u < kChainVec; u++) {
+            if (live[u]) {
+                park[vecBase + u * kBlockThreads + threadIdx.x] = v[u];
+            }
+        }
+        return;
     }
     for (uint32_t k = 0; k < ndst; k++) {
         void *o = dst[k];
@@ -804,8 +828,6 @@ __global__ void __launch_bounds__(kBlockThreads) CopyKernel(const FusedDesc *__r
 // Stands where the reference's AIV kernel stages small all-to-all-v slices through its unified buffer
 // (ALG/base/alg_aiv_template/aiv_all_to_all_v_910b.h:39-222); nothing of it is reused.
 constexpr uint32_t kGatherLdsPerWave = kGatherMaxBytes + 32;
-typedef V4 __attribute__((address_space(3))) LdsV4;
-typedef V4U __attribute__((address_space(3))) LdsV4U;
 
 template <int Variant>
 __global__ void __launch_bounds__(kBlockThreads) GatherKernel(const SegDesc *__restrict__ segs, uint32_t nsegs, uint32_t,
@@ -968,9 +990,9 @@ __device__ __forceinline__ void TreeValue(const FusedDesc &d, const void *const 
 }
 
 // One pass over kTreeVec * 256 vectors starting at vector vecBase of the tile.
-template <typename T, int OP, uint32_t MODE, bool FULL, uint32_t G>
+template <typename T, int OP, uint32_t MODE, bool FULL, uint32_t G, bool PARK = false>
 __device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *const *__restrict__ src,
-    void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec)
+    void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec, LdsV4 *park = nullptr)
 {
     uint64_t pos[kTreeVec];
     bool live[kTreeVec];
@@ -982,6 +1004,15 @@ __device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *cons
     }
     V4 r[kTreeVec];
     TreeValue<T, OP, MODE, FULL, G>(d, src, pos, live, r);
+    if (PARK) {
+#pragma unroll
+        for (uint32_t u = 0; u < kTreeVec; u++) {
+            if (live[u]) {
+                park[vecBase + u * kBlockThreads + threadIdx.x] = r[u];
+            }
+        }
+        return;
+    }
     const uint32_t ndst = d.ndst;
     for (uint32_t k = 0; k < ndst; k++) {
         void *o = dst[k];
@@ -995,23 +1026,39 @@ __device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *cons
 }
 
 // All vector passes of one tile.
-template <typename T, int OP, uint32_t G>
+template <typename T, int OP, uint32_t G, bool PARK = false>
 __device__ __forceinline__ void TreeTileVec(const FusedDesc &d, const void *const *__restrict__ src,
-    void *const *__restrict__ dst, uint64_t off, uint32_t nvec)
+    void *const *__restrict__ dst, uint64_t off, uint32_t nvec, LdsV4 *park = nullptr)
 {
     constexpr uint32_t kPass = kTreeVec * kBlockThreads;
     uint32_t base = 0;
     if (d.mode == ACC_VEC16) {
         for (; base + kPass <= nvec; base += kPass) {
-            TreeVecPass<T, OP, ACC_VEC16, true, G>(d, src, dst, off, base, nvec);
+            TreeVecPass<T, OP, ACC_VEC16, true, G, PARK>(d, src, dst, off, base, nvec, park);
         }
         if (base < nvec) {
-            TreeVecPass<T, OP, ACC_VEC16, false, G>(d, src, dst, off, base, nvec);
+            TreeVecPass<T, OP, ACC_VEC16, false, G, PARK>(d, src, dst, off, base, nvec, park);
         }
     } else {
         for (; base < nvec; base += kPass) {
-            TreeVecPass<T, OP, ACC_VEC16_ANY, false, G>(d, src, dst, off, base, nvec);
+            TreeVecPass<T, OP, ACC_VEC16_ANY, false, G, PARK>(d, src, dst, off, base, nvec, park);
         }
+    }
+}
+
+// All vector passes of one tile, whatever the number of leaves.
+template <typename T, int OP, bool PARK = false>
+__device__ __forceinline__ void TreeTile(const FusedDesc &d, const void *const *__restrict__ src,
+    void *const *__restrict__ dst, uint64_t off, uint32_t nvec, LdsV4 *park = nullptr)
+{
+    if (d.nleaf >= kTreeGroup) {
+        TreeTileVec<T, OP, kTreeGroup, PARK>(d, src, dst, off, nvec, park);
+    } else if (d.nleaf == 4) {
+        TreeTileVec<T, OP, 4, PARK>(d, src, dst, off, nvec, park);
+    } else if (d.nleaf == 2) {
+        TreeTileVec<T, OP, 2, PARK>(d, src, dst, off, nvec, park);
+    } else {
+        TreeTileVec<T, OP, 1, PARK>(d, src, dst, off, nvec, park);
     }
 }
 
@@ -1065,16 +1112,7 @@ __global__ void __launch_bounds__(kBlockThreads) TreeKernel(const FusedDesc *__r
         if (d.mode == ACC_ELEM) {
             TreeElem<T, OP>(d, src, dst, off, n);
         } else {
-            const uint32_t nvec = n >> 4;
-            if (d.nleaf >= kTreeGroup) {
-                TreeTileVec<T, OP, kTreeGroup>(d, src, dst, off, nvec);
-            } else if (d.nleaf == 4) {
-                TreeTileVec<T, OP, 4>(d, src, dst, off, nvec);
-            } else if (d.nleaf == 2) {
-                TreeTileVec<T, OP, 2>(d, src, dst, off, nvec);
-            } else {
-                TreeTileVec<T, OP, 1>(d, src, dst, off, nvec);
-            }
+            TreeTile<T, OP>(d, src, dst, off, n >> 4);
         }
     }
 }
@@ -1138,9 +1176,10 @@ template <uint32_t U> struct StackVal {
         }                                 \
     }
 
-template <typename T, int OP, uint32_t MODE, bool FULL, bool DEEP>
+template <typename T, int OP, uint32_t MODE, bool FULL, bool DEEP, bool PARK = false>
 __device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *const *__restrict__ src,
-    const uint32_t *__restrict__ ops, void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec)
+    const uint32_t *__restrict__ ops, void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec,
+    LdsV4 *park = nullptr)
 {
     constexpr uint32_t U = DEEP ? kStackVecDeep : kStackVecShallow;
     uint64_t pos[U];
@@ -1208,6 +1247,15 @@ __device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *con
             }
         }
     }
+    if (PARK) {
+#pragma unroll
+        for (uint32_t u = 0; u < U; u++) {
+            if (live[u]) {
+                park[vecBase + u * kBlockThreads + threadIdx.x] = top.x[u];
+            }
+        }
+        return;
+    }
     const uint32_t ndst = d.ndst;
     for (uint32_t k = 0; k < ndst; k++) {
         void *o = dst[k];
@@ -1253,6 +1301,33 @@ __device__ __forceinline__ void StackElem(const FusedDesc &d, const void *const 
     }
 }
 
+// All vector passes of one tile.
+template <typename T, int OP, bool PARK = false>
+__device__ __forceinline__ void StackTile(const FusedDesc &d, const void *const *__restrict__ src,
+    const uint32_t *__restrict__ ops, void *const *__restrict__ dst, uint64_t off, uint32_t nvec, LdsV4 *park = nullptr)
+{
+    constexpr uint32_t kPassShallow = kStackVecShallow * kBlockThreads, kPassDeep = kStackVecDeep * kBlockThreads;
+    uint32_t base = 0;
+    if (d.mode == ACC_VEC16) {
+        // d.nleaf: the stack depth the item needs
+        if (d.nleaf <= kStackShallowDepth) {
+            for (; base + kPassShallow <= nvec; base += kPassShallow) {
+                StackVecPass<T, OP, ACC_VEC16, true, false, PARK>(d, src, ops, dst, off, base, nvec, park);
+            }
+        }
+        for (; base + kPassDeep <= nvec; base += kPassDeep) {
+            StackVecPass<T, OP, ACC_VEC16, true, true, PARK>(d, src, ops, dst, off, base, nvec, park);
+        }
+        if (base < nvec) {
+            StackVecPass<T, OP, ACC_VEC16, false, true, PARK>(d, src, ops, dst, off, base, nvec, park);
+        }
+    } else {
+        for (; base < nvec; base += kPassDeep) {
+            StackVecPass<T, OP, ACC_VEC16_ANY, false, true, PARK>(d, src, ops, dst, off, base, nvec, park);
+        }
+    }
+}
+
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) StackKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem)
@@ -1269,27 +1344,7 @@ __global__ void __launch_bounds__(kBlockThreads) StackKernel(const FusedDesc *__
         if (d.mode == ACC_ELEM) {
             StackElem<T, OP>(d, src, ops, dst, off, n);
         } else {
-            const uint32_t nvec = n >> 4;
-            constexpr uint32_t kPassShallow = kStackVecShallow * kBlockThreads, kPassDeep = kStackVecDeep * kBlockThreads;
-            uint32_t base = 0;
-            if (d.mode == ACC_VEC16) {
-                // d.nleaf: the stack depth the item needs
-                if (d.nleaf <= kStackShallowDepth) {
-                    for (; base + kPassShallow <= nvec; base += kPassShallow) {
-                        StackVecPass<T, OP, ACC_VEC16, true, false>(d, src, ops, dst, off, base, nvec);
-                    }
-                }
-                for (; base + kPassDeep <= nvec; base += kPassDeep) {
-                    StackVecPass<T, OP, ACC_VEC16, true, true>(d, src, ops, dst, off, base, nvec);
-                }
-                if (base < nvec) {
-                    StackVecPass<T, OP, ACC_VEC16, false, true>(d, src, ops, dst, off, base, nvec);
-                }
-            } else {
-                for (; base < nvec; base += kPassDeep) {
-                    StackVecPass<T, OP, ACC_VEC16_ANY, false, true>(d, src, ops, dst, off, base, nvec);
-                }
-            }
+            StackTile<T, OP>(d, src, ops, dst, off, n >> 4);
         }
     }
 }

@@ -6,7 +6,7 @@ namespace hcclamd {
 #define HCCL_DECL(name) extern const void *const kKernels_##name[4][KK_COUNT];
 HCCL_DECL(int8) HCCL_DECL(int16) HCCL_DECL(int32) HCCL_DECL(fp16) HCCL_DECL(fp32) HCCL_DECL(int64)
 HCCL_DECL(uint64) HCCL_DECL(uint8) HCCL_DECL(uint16) HCCL_DECL(uint32) HCCL_DECL(fp64) HCCL_DECL(bf16)
-extern const void *const kKernels_bytes[3];
+extern const void *const kKernels_bytes[4];
 
 const void *LookupKernel(int dt, int op, KernelKind kind)
 {
@@ -40,6 +40,9 @@ const void *LookupCopyKernel(KernelKind kind)
     }
     if (kind == KK_GATHER) {
         return kKernels_bytes[2];
+    }
+    if (kind == KK_TEAM_CHAIN) {
+        return kKernels_bytes[3];
     }
     return nullptr;
 }

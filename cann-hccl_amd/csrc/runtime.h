@@ -46,6 +46,8 @@ struct GroupConfig {
     uint32_t blocksPerCu = 0;             // workgroups per CU; 0 = per-kernel default
     int32_t launchCapMiB = -1;            // fused issue: cut the work into launches that move about this much; 0 = one launch per
                                           // kernel kind, -1 = the library decides per collective
+    int team = -1;                        // team form of the fused kernels (an XCD's workgroups read together, then write together):
+                                          // 1 wherever it can run, 0 never, -1 for large launches whose items touch many streams
     bool blockingArrive = false;          // ranks wait inside the call until the collective is issued
     uint32_t arriveTimeoutMs = 1800 * 1000;
 };
@@ -54,8 +56,9 @@ struct GroupConfig {
 struct LaunchRec {
     const void *func = nullptr;
     uint32_t grid = 0;
+    uint32_t dynamicLds = 0;      // bytes of dynamic LDS the launch asks for (team kernels)
     // kernel arguments: step kernels take (table, nitems, nwhole, ntiles, flags), fused kernels
-    // (table, nitems, ntiles, srcPool, dstPool, tilesPerItem)
+    // (table, nitems, ntiles, srcPool, dstPool, tilesPerItem), their team forms one more: (..., teamCtr)
     const void *table = nullptr;
     uint32_t nitems = 0;
     uint32_t ntiles = 0;
@@ -64,7 +67,9 @@ struct LaunchRec {
     const void *srcPool = nullptr;
     const void *dstPool = nullptr;
     uint32_t tilesPerItem = 0;    // fused: every item covers this many tiles (the last at most as many); 0 = they differ
+    void *teamCtr = nullptr;      // team kernels: this launch's barrier counters inside the prepared tables (zero between launches)
     bool fusedArgs = false;
+    bool team = false;
 };
 
 struct OpInfo {

@@ -47,6 +47,11 @@ extern "C" {
  *                                keeps a result of up to 256 MB in the memory-side cache for whoever reads it next; "auto"
  *                                (default): non-temporal, except write-back for pure data movement from one source to four
  *                                or more destinations with more than 512 MB of output (all-gather, broadcast)
+ *   "team"          "auto" | "0" | "1"   team form of the fused kernels: the workgroups of one XCD read their tiles together,
+ *                                hold the results in LDS and write them together, which this memory system serves faster
+ *                                than reads and writes interleaved; "auto" (default): for launches of at least four rounds
+ *                                whose items write four or more destinations and touch eight or more buffers (all-reduce,
+ *                                all-gather, broadcast); "1": wherever the device allows it; "0": never
  *   "cache_entries" how many prepared collectives (distinct sizes, buffers, settings) the group keeps (default 1024);
  *                   when full, the library waits for the device once and starts over
  *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
