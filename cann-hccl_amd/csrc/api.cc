@@ -1580,6 +1580,12 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         } else {
             return HCCL_E_PARA;
         }
+    } else if (k == "team_tiles") {
+        long n = std::atol(value);
+        if (n < 0 || n > long(kTeamTiles)) {
+            return HCCL_E_PARA;
+        }
+        cfg.teamTiles = uint32_t(n);
     } else if (k == "team") {
         if (v == "auto") {
             cfg.team = -1;

@@ -550,8 +550,8 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                 const void *teamFunc = reduceColl ? LookupKernel(dtype, op, teamKind) : LookupCopyKernel(teamKind);
                 const bool teamFits = teamFunc != nullptr && g->numCu >= kTeamXcds && g->numCu % kTeamXcds == 0 && g->cfg.blocksPerCu == 0;
                 bool team = teamFits && g->cfg.team == 1;
-                if (teamFits && g->cfg.team < 0) {
-                    double storeStreams = 0, allStreams = 0, bytes = 0;
+                double storeStreams = 0, allStreams = 0, bytes = 0;
+                if (teamFits && g->cfg.team != 0) {
                     for (const FusedDesc &d : descs) {
                         uint32_t nsrc = 0;
                         for (uint32_t k = 0; k < d.nsrc; k++) {
@@ -561,8 +561,17 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                         allStreams += double(d.ndst + nsrc) * double(d.bytes);
                         bytes += double(d.bytes);
                     }
-                    team = bytes > 0 && storeStreams >= 4.0 * bytes && allStreams >= 8.0 * bytes &&
-                        tiles >= kTeamMinRounds * kTeamTiles * g->numCu;
+                    // A round should keep a workgroup busy for a mebibyte or two per phase (8 tiles of 8 streams): fewer
+                    // tiles per round when a tile has many more sources or destinations than that (measured, 32-rank
+                    // bf16 all-reduce of 128 MiB per rank: 1650 / 1607 / 1623 us with 2 / 4 / 8 tiles; 8 ranks x 256 MiB
+                    // fp32: 892 / 788 / 743 us).
+                    const double widest = bytes > 0 ? std::max(storeStreams, allStreams - storeStreams) / bytes : 1.0;
+                    pl.rec.roundTiles = g->cfg.teamTiles != 0 ? std::min(g->cfg.teamTiles, kTeamTiles)
+                                                              : std::max(1u, std::min(kTeamTiles, uint32_t(128.0 / std::max(1.0, widest))));
+                    if (g->cfg.team < 0) {
+                        team = bytes > 0 && storeStreams >= 4.0 * bytes && allStreams >= 8.0 * bytes &&
+                            tiles >= kTeamMinRounds * pl.rec.roundTiles * g->numCu;
+                    }
                 }
                 if (team) {
                     pl.rec.func = teamFunc;
@@ -723,7 +732,8 @@ void KernelArgs(LaunchRec &l, void **args)
         args[3] = &l.srcPool;
         args[4] = &l.dstPool;
         args[5] = &l.tilesPerItem;
-        args[6] = &l.teamCtr;      // read by the team kernels only
+        args[6] = &l.teamCtr;      // these two are read by the team kernels only
+        args[7] = &l.roundTiles;
     } else {
         args[2] = &l.nwhole;
         args[3] = &l.ntiles;
@@ -736,7 +746,7 @@ HcclResult BuildGraph(Prepared *pp)
     HIP_OK(hipGraphCreate(&pp->graph, 0));
     hipGraphNode_t prev = nullptr;
     for (LaunchRec &l : pp->launches) {
-        void *args[7];
+        void *args[8];
         KernelArgs(l, args);
         hipKernelNodeParams kp = {};
         kp.func = const_cast<void *>(l.func);
@@ -776,6 +786,7 @@ std::string CacheKey(const Group *g, int algo)
     put(head, sizeof(head));
     put(&g->cfg.launchCapMiB, sizeof(g->cfg.launchCapMiB));
     put(&g->cfg.team, sizeof(g->cfg.team));
+    put(&g->cfg.teamTiles, sizeof(g->cfg.teamTiles));
     put(g->ctx->send.data(), g->ctx->send.size() * sizeof(void *));
     put(g->ctx->recv.data(), g->ctx->recv.size() * sizeof(void *));
     if (g->ctx->sig.coll == COLL_ALLTOALLV) {
@@ -1314,7 +1325,7 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         HIP_OK(hipGraphLaunch(pp->exec, ls));
     } else {
         for (LaunchRec &l : pp->launches) {
-            void *args[7];
+            void *args[8];
             KernelArgs(l, args);
             HIP_OK(hipLaunchKernel(l.func, dim3(l.grid, 1, 1), dim3(kBlockThreads, 1, 1), args, l.dynamicLds, ls));
         }

@@ -80,7 +80,7 @@ enum KernelKind : int {
 // them together (kernels_team.h).  Launched with a multiple of kTeamXcds workgroups (one per CU) and kTeamLdsBytes of
 // dynamic LDS; takes one more argument, the team counters: kTeamXcds * kTeamCtrStride zero-initialised uint32 in
 // device memory that belong to this launch alone (the kernel leaves them zero again).
-constexpr uint32_t kTeamTiles = 8;        // tiles a workgroup parks per round
+constexpr uint32_t kTeamTiles = 8;        // tiles a workgroup can park per round
 constexpr uint32_t kTeamXcds = 8;
 constexpr uint32_t kTeamCtrStride = 16;   // uint32 per XCD (64 bytes: arrivals, finished workgroups, gave-up flag)
 constexpr uint32_t kTeamCtrBytes = kTeamXcds * kTeamCtrStride * 4;
@@ -93,7 +93,8 @@ constexpr uint32_t kTeamDynamicLds = kTeamTiles * kTileBytes;
 //   KK_CHAIN / KK_TREE / KK_STACK
 //                      (const FusedDesc *items, uint32_t nitems, uint32_t ntiles,
 //                       const void *const *srcPool, void *const *dstPool, uint32_t tilesPerItem)
-//   KK_TEAM_*          the same and (uint32_t *teamCtr)
+//   KK_TEAM_*          the same and (uint32_t *teamCtr, uint32_t roundTiles): roundTiles <= kTeamTiles tiles per workgroup
+//                      and round
 const void *LookupKernel(int hcclDataType, int hcclReduceOp, KernelKind kind);
 
 //   KK_GATHER          (const SegDesc *segs, uint32_t nsegs, uint32_t unused, const void *unused, void *unused)

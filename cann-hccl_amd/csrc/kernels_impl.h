@@ -886,12 +886,14 @@ __global__ void __launch_bounds__(kBlockThreads) GatherKernel(const SegDesc *__r
 constexpr uint32_t kTreeGroup = 8;
 constexpr uint32_t kTreeMaxGroups = 4;   // up to 32 leaves
 
-constexpr uint32_t kTreeVec = 2;         // vectors per lane per pass
+constexpr uint32_t kTreeVecPlain = 2;    // vectors per lane per pass
+constexpr uint32_t kTreeVecTeam = 4;     // in the team kernels, which run one workgroup per CU: twice the loads in flight
 
 // Evaluates the tree for kTreeVec vectors of one lane (positions pos[u], skipped where !live[u]).
+// kTreeVec is kTreeVecPlain, or kTreeVecTeam when the results are parked (PARK).
 // G = leaves per group: 8 when the tree has 8 or more leaves, else the leaf count itself (1, 2, 4),
 // so that no group is ever partial and the loads of a group are issued back to back.
-template <typename T, int OP, uint32_t MODE, bool FULL, uint32_t G>
+template <typename T, int OP, uint32_t MODE, bool FULL, uint32_t G, uint32_t kTreeVec>
 __device__ __forceinline__ void TreeValue(const FusedDesc &d, const void *const *__restrict__ src,
     const uint64_t (&pos)[kTreeVec], const bool (&live)[kTreeVec], V4 (&x)[kTreeVec])
 {
@@ -994,6 +996,7 @@ template <typename T, int OP, uint32_t MODE, bool FULL, uint32_t G, bool PARK = 
 __device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *const *__restrict__ src,
     void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec, LdsV4 *park = nullptr)
 {
+    constexpr uint32_t kTreeVec = PARK ? kTreeVecTeam : kTreeVecPlain;
     uint64_t pos[kTreeVec];
     bool live[kTreeVec];
 #pragma unroll
@@ -1003,7 +1006,7 @@ __device__ __forceinline__ void TreeVecPass(const FusedDesc &d, const void *cons
         pos[u] = off + uint64_t(i) * 16;
     }
     V4 r[kTreeVec];
-    TreeValue<T, OP, MODE, FULL, G>(d, src, pos, live, r);
+    TreeValue<T, OP, MODE, FULL, G, kTreeVec>(d, src, pos, live, r);
     if (PARK) {
 #pragma unroll
         for (uint32_t u = 0; u < kTreeVec; u++) {
@@ -1030,7 +1033,7 @@ template <typename T, int OP, uint32_t G, bool PARK = false>
 __device__ __forceinline__ void TreeTileVec(const FusedDesc &d, const void *const *__restrict__ src,
     void *const *__restrict__ dst, uint64_t off, uint32_t nvec, LdsV4 *park = nullptr)
 {
-    constexpr uint32_t kPass = kTreeVec * kBlockThreads;
+    constexpr uint32_t kPass = (PARK ? kTreeVecTeam : kTreeVecPlain) * kBlockThreads;
     uint32_t base = 0;
     if (d.mode == ACC_VEC16) {
         for (; base + kPass <= nvec; base += kPass) {

@@ -90,7 +90,7 @@ __device__ __forceinline__ void TeamDrain(const LdsV4 *park, void *o, uint64_t o
 template <typename Eval>
 __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, uint32_t nitems, uint32_t ntiles,
     const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr, const void *extra)
+    uint32_t *__restrict__ teamCtr, uint32_t roundTiles, const void *extra)
 {
     extern __shared__ V4 teamLds[];
     __shared__ uint32_t heldItem[kTeamTiles];
@@ -104,9 +104,10 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
     uint32_t target = 0;
     uint32_t done = 0;                            // tiles of earlier rounds
     while (done < ntiles) {
-        // tiles per workgroup this round: kTeamTiles, fewer in the last round so that it spreads over all workgroups
+        // tiles per workgroup this round: roundTiles (at most kTeamTiles), fewer in the last round so that it spreads
+        // over all workgroups
         const uint32_t left = ntiles - done;
-        const uint32_t per = left >= grid * kTeamTiles ? kTeamTiles : (left + grid - 1) / grid;
+        const uint32_t per = left >= grid * roundTiles ? roundTiles : (left + grid - 1) / grid;
         const uint32_t first = done + (xcd * teamSize + inTeam) * per;
         const uint32_t n = first < ntiles ? (ntiles - first < per ? ntiles - first : per) : 0;
         uint32_t maxDst = 0;
@@ -173,7 +174,7 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
         }
         // the next round's results must not land in LDS before this round's have been read
         __syncthreads();
-        done += left >= grid * kTeamTiles ? grid * kTeamTiles : left;
+        done += left >= grid * roundTiles ? grid * roundTiles : left;
     }
     TeamLeave(ctr, teamSize);
 }
@@ -275,38 +276,39 @@ template <typename T, int OP> struct TeamStackEval {
     }
 };
 
-// Same tables and arguments as the plain fused kernels, plus the team counters.  Launched with one workgroup per CU
+// Same tables and arguments as the plain fused kernels, plus the team counters and the number of tiles a workgroup
+// takes per round (1 .. kTeamTiles).  Launched with one workgroup per CU
 // (a multiple of kTeamXcds workgroups) and kTeamDynamicLds bytes of dynamic LDS.
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) TeamChainKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr)
+    uint32_t *__restrict__ teamCtr, uint32_t roundTiles)
 {
-    TeamBody<TeamChainEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, nullptr);
+    TeamBody<TeamChainEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, roundTiles, nullptr);
 }
 
 template <int Variant>
 __global__ void __launch_bounds__(kBlockThreads) TeamCopyKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr)
+    uint32_t *__restrict__ teamCtr, uint32_t roundTiles)
 {
-    TeamBody<TeamCopyEval>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, nullptr);
+    TeamBody<TeamCopyEval>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, roundTiles, nullptr);
 }
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) TeamTreeKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr)
+    uint32_t *__restrict__ teamCtr, uint32_t roundTiles)
 {
-    TeamBody<TeamTreeEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, nullptr);
+    TeamBody<TeamTreeEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, roundTiles, nullptr);
 }
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) TeamStackKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr)
+    uint32_t *__restrict__ teamCtr, uint32_t roundTiles)
 {
-    TeamBody<TeamStackEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, items + nitems);
+    TeamBody<TeamStackEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, roundTiles, items + nitems);
 }
 
 }  // namespace hcclamd

@@ -46,6 +46,7 @@ struct GroupConfig {
     uint32_t blocksPerCu = 0;             // workgroups per CU; 0 = per-kernel default
     int32_t launchCapMiB = -1;            // fused issue: cut the work into launches that move about this much; 0 = one launch per
                                           // kernel kind, -1 = the library decides per collective
+    uint32_t teamTiles = 0;               // team kernels: tiles per workgroup and round, 0 = chosen per launch
     int team = -1;                        // team form of the fused kernels (an XCD's workgroups read together, then write together):
                                           // 1 wherever it can run, 0 never, -1 for large launches whose items touch many streams
     bool blockingArrive = false;          // ranks wait inside the call until the collective is issued
@@ -58,7 +59,7 @@ struct LaunchRec {
     uint32_t grid = 0;
     uint32_t dynamicLds = 0;      // bytes of dynamic LDS the launch asks for (team kernels)
     // kernel arguments: step kernels take (table, nitems, nwhole, ntiles, flags), fused kernels
-    // (table, nitems, ntiles, srcPool, dstPool, tilesPerItem), their team forms one more: (..., teamCtr)
+    // (table, nitems, ntiles, srcPool, dstPool, tilesPerItem), their team forms two more: (..., teamCtr, roundTiles)
     const void *table = nullptr;
     uint32_t nitems = 0;
     uint32_t ntiles = 0;
@@ -68,6 +69,7 @@ struct LaunchRec {
     const void *dstPool = nullptr;
     uint32_t tilesPerItem = 0;    // fused: every item covers this many tiles (the last at most as many); 0 = they differ
     void *teamCtr = nullptr;      // team kernels: this launch's barrier counters inside the prepared tables (zero between launches)
+    uint32_t roundTiles = 0;      // team kernels: tiles per workgroup and round
     bool fusedArgs = false;
     bool team = false;
 };

@@ -52,6 +52,8 @@ extern "C" {
  *                                than reads and writes interleaved; "auto" (default): for launches of at least four rounds
  *                                whose items write four or more destinations and touch eight or more buffers (all-reduce,
  *                                all-gather, broadcast); "1": wherever the device allows it; "0": never
+ *   "team_tiles"    tiles of 16 KiB a workgroup of a team kernel takes per round, 1 ... 8 ("0", default: 8, fewer when an
+ *                                item has more than 8 sources or destinations)
  *   "cache_entries" how many prepared collectives (distinct sizes, buffers, settings) the group keeps (default 1024);
  *                   when full, the library waits for the device once and starts over
  *   "blocks_per_cu" launch width in workgroups per compute unit ("0": chosen per collective)
