@@ -578,7 +578,27 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                     pl.rec.team = true;
                     pl.rec.grid = g->numCu;
                     pl.rec.dynamicLds = kTeamDynamicLds;
-                    pl.ctrAt = b.Reserve(kTeamCtrBytes);     // zero in the image, and zero again after every launch
+                    // The regions the teams draw: roundTiles tiles per workgroup at first; over the last quarter of the
+                    // tiles the size is halved whenever fewer than 16 regions of the current size are left, so that
+                    // the XCDs finish together (measured, 8 x 256 MiB fp32 all-reduce: 727 us with 64 equal regions
+                    // dealt out in order, 714 us with the shrinking tail drawn from the counter).
+                    const uint32_t perX = g->numCu / kTeamXcds;
+                    std::vector<TeamRegion> regions;
+                    for (uint32_t at = 0, per = pl.rec.roundTiles; at < tiles;) {
+                        const uint32_t left = tiles - at;
+                        if (uint64_t(at) * 4 >= uint64_t(tiles) * 3) {
+                            while (per > 1 && uint64_t(per) * perX * 16 > left) {
+                                per /= 2;
+                            }
+                        }
+                        regions.push_back(TeamRegion{at, per});
+                        at += uint32_t(std::min<uint64_t>(left, uint64_t(per) * perX));
+                    }
+                    const uint32_t n = uint32_t(regions.size());
+                    pl.ctrAt = b.Reserve(size_t(TeamBlockWords(n)) * 4);     // zero in the image, and zero again after every launch
+                    uint32_t *block = reinterpret_cast<uint32_t *>(b.host.data() + pl.ctrAt);
+                    block[kTeamRegionCount] = n;
+                    std::memcpy(block + kTeamHeaderWords, regions.data(), regions.size() * sizeof(TeamRegion));
                 }
                 pending.push_back(pl);
                 descs.clear();
@@ -732,8 +752,7 @@ void KernelArgs(LaunchRec &l, void **args)
         args[3] = &l.srcPool;
         args[4] = &l.dstPool;
         args[5] = &l.tilesPerItem;
-        args[6] = &l.teamCtr;      // these two are read by the team kernels only
-        args[7] = &l.roundTiles;
+        args[6] = &l.teamCtr;      // read by the team kernels only
     } else {
         args[2] = &l.nwhole;
         args[3] = &l.ntiles;
@@ -746,7 +765,7 @@ HcclResult BuildGraph(Prepared *pp)
     HIP_OK(hipGraphCreate(&pp->graph, 0));
     hipGraphNode_t prev = nullptr;
     for (LaunchRec &l : pp->launches) {
-        void *args[8];
+        void *args[7];
         KernelArgs(l, args);
         hipKernelNodeParams kp = {};
         kp.func = const_cast<void *>(l.func);
@@ -1325,7 +1344,7 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
         HIP_OK(hipGraphLaunch(pp->exec, ls));
     } else {
         for (LaunchRec &l : pp->launches) {
-            void *args[8];
+            void *args[7];
             KernelArgs(l, args);
             HIP_OK(hipLaunchKernel(l.func, dim3(l.grid, 1, 1), dim3(kBlockThreads, 1, 1), args, l.dynamicLds, ls));
         }

@@ -77,14 +77,28 @@ enum KernelKind : int {
 };
 
 // Team form of a fused kernel: the workgroups of one XCD read their tiles together, park the results in LDS, and write
-// them together (kernels_team.h).  Launched with a multiple of kTeamXcds workgroups (one per CU) and kTeamLdsBytes of
-// dynamic LDS; takes one more argument, the team counters: kTeamXcds * kTeamCtrStride zero-initialised uint32 in
-// device memory that belong to this launch alone (the kernel leaves them zero again).
+// them together (kernels_team.h).  Launched with a multiple of kTeamXcds workgroups (one per CU) and kTeamDynamicLds
+// bytes of dynamic LDS; takes one more argument, the launch's team block in device memory, which belongs to this launch
+// alone.  Layout, in uint32 words:
+//   [x * kTeamCtrStride + kTeamArrive / kTeamGaveUp]   x < kTeamXcds: barrier arrivals of team x; set once a wait ran out
+//   [kTeamTicket]       regions handed out beyond the first kTeamXcds
+//   [kTeamFinished]     workgroups that have finished
+//   [kTeamRegionCount]  number of regions n (written by the host, never changed)
+//   [kTeamHeaderWords ...]            n x TeamRegion (written by the host, never changed)
+//   [kTeamHeaderWords + 2 n ...]      kTeamXcds x (n + 1) slots: the region of team x's round r + 1, plus 2; 1 = being drawn
+// Everything but the count and the table starts out zero, and the kernel leaves it zero again.
 constexpr uint32_t kTeamTiles = 8;        // tiles a workgroup can park per round
 constexpr uint32_t kTeamXcds = 8;
-constexpr uint32_t kTeamCtrStride = 16;   // uint32 per XCD (64 bytes: arrivals, finished workgroups, gave-up flag)
-constexpr uint32_t kTeamCtrBytes = kTeamXcds * kTeamCtrStride * 4;
+constexpr uint32_t kTeamCtrStride = 16;   // words per XCD (64 bytes)
+constexpr uint32_t kTeamArrive = 0, kTeamGaveUp = 1;
+constexpr uint32_t kTeamTicket = kTeamXcds * kTeamCtrStride, kTeamFinished = kTeamTicket + 1, kTeamRegionCount = kTeamTicket + 2;
+constexpr uint32_t kTeamHeaderWords = kTeamTicket + 4;
 constexpr uint32_t kTeamDynamicLds = kTeamTiles * kTileBytes;
+struct TeamRegion {
+    uint32_t first;   // first tile
+    uint32_t per;     // tiles per workgroup, 1 ... kTeamTiles: workgroup i of the team takes [first + i * per, first + (i + 1) * per)
+};
+inline uint32_t TeamBlockWords(uint32_t nregions) { return kTeamHeaderWords + 2u * nregions + kTeamXcds * (nregions + 1u); }
 
 // Kernel entry for (data type, reduce op, kind); nullptr if the combination is not built.
 // Signatures:
@@ -93,8 +107,7 @@ constexpr uint32_t kTeamDynamicLds = kTeamTiles * kTileBytes;
 //   KK_CHAIN / KK_TREE / KK_STACK
 //                      (const FusedDesc *items, uint32_t nitems, uint32_t ntiles,
 //                       const void *const *srcPool, void *const *dstPool, uint32_t tilesPerItem)
-//   KK_TEAM_*          the same and (uint32_t *teamCtr, uint32_t roundTiles): roundTiles <= kTeamTiles tiles per workgroup
-//                      and round
+//   KK_TEAM_*          the same and (uint32_t *teamBlock)
 const void *LookupKernel(int hcclDataType, int hcclReduceOp, KernelKind kind);
 
 //   KK_GATHER          (const SegDesc *segs, uint32_t nsegs, uint32_t unused, const void *unused, void *unused)

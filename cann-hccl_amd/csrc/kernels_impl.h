@@ -541,7 +541,9 @@ template <uint32_t MODE, bool ORDINARY = false> __device__ __forceinline__ void 
 // FULL: every lane has all its vectors inside the tile (no per-lane guards).
 // PARK: the results are not stored to the destinations but left in LDS, vector i of the tile at park[i] (the team
 // kernels write them out later); dst is not used then.
-template <typename T, int OP, uint32_t MODE, bool FULL, bool ORDINARY = false, bool PARK = false>
+// ONE_BATCH: the item has at most kChainSrcBatch sources (the caller has checked), so `src` is only ever indexed with
+// constants: a caller that keeps the pointers in a local array then keeps them in registers from tile to tile.
+template <typename T, int OP, uint32_t MODE, bool FULL, bool ORDINARY = false, bool PARK = false, bool ONE_BATCH = false>
 __device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *const *__restrict__ src,
     void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec, LdsV4 *park = nullptr)
 {
@@ -556,7 +558,8 @@ __device__ __forceinline__ void ChainVecPass(const FusedDesc &d, const void *con
     }
     V4 acc[kChainVec];
     const uint32_t nsrc = d.nsrc;
-    for (uint32_t j = 0; j < nsrc; j += kChainSrcBatch) {
+    const uint32_t batched = ONE_BATCH ? 1u : nsrc;
+    for (uint32_t j = 0; j < batched; j += kChainSrcBatch) {
         V4 v[kChainSrcBatch][kChainVec];
 #pragma unroll
         for (uint32_t jj = 0; jj < kChainSrcBatch; jj++) {

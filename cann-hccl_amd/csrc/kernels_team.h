@@ -14,8 +14,8 @@
 // not resident all at once, only the speed changes: nothing passes between workgroups through the barrier, it only
 // aligns them in time, every wait is bounded, and after one wait that ran out a team stops waiting for that launch.
 //
-// The barrier counters live in device memory that starts out zero; the last workgroup of a team to finish puts them
-// back to zero, so a launch (or a replay of a HIP graph) finds them as the first one did.
+// The counters live in device memory that starts out zero; the last workgroup of a launch to finish puts them back to
+// zero, so the next launch (or a replay of a HIP graph) finds them as the first one did.
 #pragma once
 #include "kernels_impl.h"
 
@@ -24,23 +24,63 @@ namespace hcclamd {
 constexpr uint32_t kTeamVecPerTile = kTileBytes / 16;
 constexpr uint64_t kTeamWaitTicks = 20000;                       // 200 us of the 100 MHz clock
 
+// All atomics here are relaxed and at agent scope: they are carried out in memory, beyond the XCDs' separate L2 caches,
+// and order nothing else (no data is handed from workgroup to workgroup).
 __device__ __forceinline__ uint32_t TeamLoad(const uint32_t *p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void TeamStore(uint32_t *p, uint32_t v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t TeamAdd(uint32_t *p, uint32_t v)
+{
+    return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
-// c[0] arrivals, c[1] workgroups that have finished, c[2] set once a wait ran out.  Atomics at agent scope are carried
-// out in memory, beyond the XCDs' separate L2 caches; relaxed, because no data is handed over.
-__device__ __forceinline__ void TeamBarrier(uint32_t *c, uint32_t target)
+// The team's region for its next round.  Every workgroup of the team asks on its own; whoever comes first to the
+// round's slot claims it (0 -> 1), draws the next region from the launch's ticket counter and leaves the answer
+// (region + 2) in the slot.  The others wait for that answer: the claimer is running and needs nobody to get there,
+// so the wait ends whether or not the rest of the grid is resident.  `seen` is what an earlier look at the slot showed.
+__device__ __forceinline__ uint32_t TeamNextRegion(uint32_t *slot, uint32_t *ticket, uint32_t seen)
+{
+    uint32_t v = seen;
+    for (;;) {
+        if (v >= 2u) {
+            return v - 2u;
+        }
+        if (v == 0u) {
+            // (also reached when the slot was put back to zero under a waiting workgroup: two launches of one prepared
+            // collective running at the same time share this block; each region is then still worked on at least once)
+            uint32_t expected = 0u;
+            if (__hip_atomic_compare_exchange_strong(slot, &expected, 1u, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+                v = TeamAdd(ticket, 1u) + kTeamXcds + 2u;      // regions 0 .. kTeamXcds - 1 are the first round's
+                TeamStore(slot, v);
+            } else {
+                v = expected;
+            }
+            continue;
+        }
+        __builtin_amdgcn_s_sleep(2);
+        v = TeamLoad(slot);
+    }
+}
+
+// Arrival at the team's barrier, then (thread 0) the question for the next region while the others arrive, then the
+// wait: bounded, and given up for the rest of the launch once it has run out.
+__device__ __forceinline__ uint32_t TeamBarrier(uint32_t *c, uint32_t target, uint32_t *slot, uint32_t *ticket, uint32_t seen,
+    uint32_t *nextShared)
 {
     __syncthreads();
     if (threadIdx.x == 0) {
-        __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (TeamLoad(c + 2) == 0u) {
+        TeamAdd(c + kTeamArrive, 1u);
+        *nextShared = TeamNextRegion(slot, ticket, seen);
+        if (TeamLoad(c + kTeamGaveUp) == 0u) {
             const uint64_t t0 = wall_clock64();
-            while (TeamLoad(c) < target) {
+            while (TeamLoad(c + kTeamArrive) < target) {
                 if (wall_clock64() - t0 > kTeamWaitTicks) {
-                    __hip_atomic_store(c + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    TeamStore(c + kTeamGaveUp, 1u);
                     break;
                 }
                 __builtin_amdgcn_s_sleep(2);
@@ -48,17 +88,30 @@ __device__ __forceinline__ void TeamBarrier(uint32_t *c, uint32_t target)
         }
     }
     __syncthreads();
+    return *nextShared;
 }
 
-__device__ __forceinline__ void TeamLeave(uint32_t *c, uint32_t teamSize)
+// The last workgroup of the launch to finish puts every counter and slot back to zero.
+__device__ __forceinline__ void TeamLeave(uint32_t *teamCtr, uint32_t nregions)
 {
+    __shared__ uint32_t last;
     __syncthreads();
     if (threadIdx.x == 0) {
-        const uint32_t before = __hip_atomic_fetch_add(c + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (before + 1 == teamSize) {      // everybody else is past every barrier
-            __hip_atomic_store(c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(c + 2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(c + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last = TeamAdd(teamCtr + kTeamFinished, 1u) + 1u == gridDim.x ? 1u : 0u;
+    }
+    __syncthreads();
+    if (last) {       // everybody else is past every barrier and every slot
+        uint32_t *slots = teamCtr + kTeamHeaderWords + 2u * nregions;
+        for (uint32_t i = threadIdx.x; i < kTeamXcds * (nregions + 1u); i += kBlockThreads) {
+            TeamStore(slots + i, 0u);
+        }
+        if (threadIdx.x < kTeamXcds) {
+            TeamStore(teamCtr + threadIdx.x * kTeamCtrStride + kTeamArrive, 0u);
+            TeamStore(teamCtr + threadIdx.x * kTeamCtrStride + kTeamGaveUp, 0u);
+        }
+        if (threadIdx.x == 0) {
+            TeamStore(teamCtr + kTeamTicket, 0u);
+            TeamStore(teamCtr + kTeamFinished, 0u);
         }
     }
 }
@@ -85,41 +138,54 @@ __device__ __forceinline__ void TeamDrain(const LdsV4 *park, void *o, uint64_t o
     }
 }
 
-// Eval::Vec(d, srcPool, extra, off, nvec, park) leaves the vectors of one tile in LDS; Eval::Elem(d, srcPool, extra,
-// dstPool, off, n) handles an element-wise piece (a few bytes of head or tail) there and then.
+// Eval: SetItem(d, srcPool) is called when the tiles move on to another item, Vec(d, srcPool, extra, off, nvec, park)
+// leaves the vectors of one tile in LDS, the static Elem(d, srcPool, extra, dstPool, off, n) handles an element-wise
+// piece (a few bytes of head or tail) there and then.
+//
+// The tile space is cut into regions (first tile, tiles per workgroup), a table the host wrote behind the counters:
+// workgroup i of a team takes tiles [first + i * per, first + (i + 1) * per) of the team's region.  Team x starts
+// with region x; the later ones are drawn from a counter as the teams get there, and the last regions are smaller,
+// so that the XCDs, which do not all move data at the same rate, finish together.
 template <typename Eval>
 __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, uint32_t nitems, uint32_t ntiles,
     const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr, uint32_t roundTiles, const void *extra)
+    uint32_t *__restrict__ teamCtr, const void *extra)
 {
     extern __shared__ V4 teamLds[];
     __shared__ uint32_t heldItem[kTeamTiles];
     __shared__ uint32_t heldTile[kTeamTiles];
     __shared__ uint32_t heldVec[kTeamTiles];      // vectors parked; 0 = nothing (no tile, or an element-wise piece)
+    __shared__ uint32_t nextShared;
     LdsV4 *park = (LdsV4 *)teamLds;
 
-    const uint32_t grid = gridDim.x;
-    const uint32_t xcd = blockIdx.x % kTeamXcds, inTeam = blockIdx.x / kTeamXcds, teamSize = grid / kTeamXcds;
+    const uint32_t xcd = blockIdx.x % kTeamXcds, inTeam = blockIdx.x / kTeamXcds, teamSize = gridDim.x / kTeamXcds;
+    const uint32_t nregions = teamCtr[kTeamRegionCount];
+    const TeamRegion *regions = reinterpret_cast<const TeamRegion *>(teamCtr + kTeamHeaderWords);
+    uint32_t *slots = teamCtr + kTeamHeaderWords + 2u * nregions + xcd * (nregions + 1u);
     uint32_t *ctr = teamCtr + xcd * kTeamCtrStride;
     uint32_t target = 0;
-    uint32_t done = 0;                            // tiles of earlier rounds
-    while (done < ntiles) {
-        // tiles per workgroup this round: roundTiles (at most kTeamTiles), fewer in the last round so that it spreads
-        // over all workgroups
-        const uint32_t left = ntiles - done;
-        const uint32_t per = left >= grid * roundTiles ? roundTiles : (left + grid - 1) / grid;
-        const uint32_t first = done + (xcd * teamSize + inTeam) * per;
-        const uint32_t n = first < ntiles ? (ntiles - first < per ? ntiles - first : per) : 0;
+    uint32_t region = xcd;
+    for (uint32_t round = 0; region < nregions; round++) {
+        const TeamRegion reg = regions[region];
+        const uint32_t first = reg.first + inTeam * reg.per;
+        const uint32_t n = first < ntiles ? (ntiles - first < reg.per ? ntiles - first : reg.per) : 0;
+        // an early look at the slot of the next round: a workgroup that is behind finds the answer there already
+        uint32_t seen = 0;
+        if (threadIdx.x == 0) {
+            seen = TeamLoad(slots + round);
+        }
         uint32_t maxDst = 0;
         uint32_t idx = 0;
         FusedDesc d;
         uint32_t dEnd = 0;
+        Eval eval;
         for (uint32_t q = 0; q < n; q++) {
             const uint32_t tile = first + q;
             if (q == 0 || tile >= dEnd) {
                 idx = ItemOfTile(items, nitems, tile, tilesPerItem);
                 d = items[idx];
                 dEnd = d.tile0 + uint32_t((d.bytes + kTileBytes - 1) / kTileBytes);
+                eval.SetItem(d, srcPool);
             }
             const uint64_t off = uint64_t(tile - d.tile0) * kTileBytes;
             const uint64_t rest = d.bytes - off;
@@ -129,7 +195,7 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
                 Eval::Elem(d, srcPool, extra, dstPool, off, bytes);
             } else {
                 nvec = bytes >> 4;
-                Eval::Vec(d, srcPool, extra, off, nvec, park + q * kTeamVecPerTile);
+                eval.Vec(d, srcPool, extra, off, nvec, park + q * kTeamVecPerTile);
                 maxDst = d.ndst > maxDst ? d.ndst : maxDst;
             }
             if (threadIdx.x == 0) {
@@ -139,7 +205,7 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
             }
         }
         target += teamSize;
-        TeamBarrier(ctr, target);
+        region = TeamBarrier(ctr, target, slots + round, teamCtr + kTeamTicket, seen, &nextShared);
         // Every lane reads back the vectors it parked itself.  A workgroup's tiles mostly belong to one item, so its
         // descriptor and the destination pointer are kept from tile to tile.
         for (uint32_t k = 0; k < maxDst; k++) {
@@ -174,32 +240,51 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
         }
         // the next round's results must not land in LDS before this round's have been read
         __syncthreads();
-        done += left >= grid * roundTiles ? grid * roundTiles : left;
     }
-    TeamLeave(ctr, teamSize);
+    TeamLeave(teamCtr, nregions);
 }
 
 // ---- what a tile's value is, per kernel family --------------------------------------------------------------------
 template <typename T, int OP> struct TeamChainEval {
-    static __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__ srcPool, const void *,
-        uint64_t off, uint32_t nvec, LdsV4 *park)
+    // Up to kChainSrcBatch source pointers are kept in registers from tile to tile: fetched per tile they are a chain
+    // of dependent loads in front of the tile's data, with nothing else on the CU to hide it.
+    const void *sp[kChainSrcBatch];
+    bool few;
+    __device__ __forceinline__ void SetItem(const FusedDesc &d, const void *const *__restrict__ srcPool)
     {
-        const void *const *src = srcPool + d.srcBase;
+        few = d.nsrc <= kChainSrcBatch;
+#pragma unroll
+        for (uint32_t j = 0; j < kChainSrcBatch; j++) {
+            sp[j] = j < d.nsrc ? srcPool[d.srcBase + j] : nullptr;
+        }
+    }
+    template <uint32_t MODE, bool ONE>
+    __device__ __forceinline__ void Passes(const FusedDesc &d, const void *const *__restrict__ src, uint64_t off, uint32_t nvec,
+        LdsV4 *park) const
+    {
         constexpr uint32_t kPass = kChainVec * kBlockThreads;
         uint32_t base = 0;
-        if (d.mode == ACC_VEC16) {
-            for (; base + kPass <= nvec; base += kPass) {
-                ChainVecPass<T, OP, ACC_VEC16, true, false, true>(d, src, nullptr, off, base, nvec, park);
-            }
-            if (base < nvec) {
-                ChainVecPass<T, OP, ACC_VEC16, false, false, true>(d, src, nullptr, off, base, nvec, park);
+        for (; base + kPass <= nvec; base += kPass) {
+            ChainVecPass<T, OP, MODE, true, false, true, ONE>(d, src, nullptr, off, base, nvec, park);
+        }
+        if (base < nvec) {
+            ChainVecPass<T, OP, MODE, false, false, true, ONE>(d, src, nullptr, off, base, nvec, park);
+        }
+    }
+    __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__ srcPool, const void *,
+        uint64_t off, uint32_t nvec, LdsV4 *park) const
+    {
+        if (few) {
+            if (d.mode == ACC_VEC16) {
+                Passes<ACC_VEC16, true>(d, sp, off, nvec, park);
+            } else {
+                Passes<ACC_VEC16_ANY, true>(d, sp, off, nvec, park);
             }
         } else {
-            for (; base + kPass <= nvec; base += kPass) {
-                ChainVecPass<T, OP, ACC_VEC16_ANY, true, false, true>(d, src, nullptr, off, base, nvec, park);
-            }
-            if (base < nvec) {
-                ChainVecPass<T, OP, ACC_VEC16_ANY, false, false, true>(d, src, nullptr, off, base, nvec, park);
+            if (d.mode == ACC_VEC16) {
+                Passes<ACC_VEC16, false>(d, srcPool + d.srcBase, off, nvec, park);
+            } else {
+                Passes<ACC_VEC16_ANY, false>(d, srcPool + d.srcBase, off, nvec, park);
             }
         }
     }
@@ -211,10 +296,11 @@ template <typename T, int OP> struct TeamChainEval {
 };
 
 struct TeamCopyEval {
-    static __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__ srcPool, const void *,
-        uint64_t off, uint32_t nvec, LdsV4 *park)
+    const void *s;
+    __device__ __forceinline__ void SetItem(const FusedDesc &d, const void *const *__restrict__ srcPool) { s = srcPool[d.srcBase]; }
+    __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__, const void *, uint64_t off,
+        uint32_t nvec, LdsV4 *park) const
     {
-        const void *s = srcPool[d.srcBase];
         constexpr uint32_t kPass = kChainVec * kBlockThreads;
         uint32_t base = 0;
         if (d.mode == ACC_VEC16) {
@@ -248,8 +334,9 @@ struct TeamCopyEval {
 };
 
 template <typename T, int OP> struct TeamTreeEval {
-    static __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__ srcPool, const void *,
-        uint64_t off, uint32_t nvec, LdsV4 *park)
+    __device__ __forceinline__ void SetItem(const FusedDesc &, const void *const *__restrict__) {}
+    __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__ srcPool, const void *,
+        uint64_t off, uint32_t nvec, LdsV4 *park) const
     {
         TreeTile<T, OP, true>(d, srcPool + d.srcBase, nullptr, off, nvec, park);
     }
@@ -262,8 +349,9 @@ template <typename T, int OP> struct TeamTreeEval {
 
 // extra = the launch's op words (they follow the item table)
 template <typename T, int OP> struct TeamStackEval {
-    static __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__ srcPool, const void *extra,
-        uint64_t off, uint32_t nvec, LdsV4 *park)
+    __device__ __forceinline__ void SetItem(const FusedDesc &, const void *const *__restrict__) {}
+    __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__ srcPool, const void *extra,
+        uint64_t off, uint32_t nvec, LdsV4 *park) const
     {
         const uint32_t *ops = static_cast<const uint32_t *>(extra) + d.srcBase;
         StackTile<T, OP, true>(d, srcPool + d.srcBase, ops, nullptr, off, nvec, park);
@@ -276,39 +364,39 @@ template <typename T, int OP> struct TeamStackEval {
     }
 };
 
-// Same tables and arguments as the plain fused kernels, plus the team counters and the number of tiles a workgroup
-// takes per round (1 .. kTeamTiles).  Launched with one workgroup per CU
+// Same tables and arguments as the plain fused kernels, plus the team block (counters, region table, slots; layout in
+// kernels.h).  Launched with one workgroup per CU
 // (a multiple of kTeamXcds workgroups) and kTeamDynamicLds bytes of dynamic LDS.
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) TeamChainKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr, uint32_t roundTiles)
+    uint32_t *__restrict__ teamCtr)
 {
-    TeamBody<TeamChainEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, roundTiles, nullptr);
+    TeamBody<TeamChainEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, nullptr);
 }
 
 template <int Variant>
 __global__ void __launch_bounds__(kBlockThreads) TeamCopyKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr, uint32_t roundTiles)
+    uint32_t *__restrict__ teamCtr)
 {
-    TeamBody<TeamCopyEval>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, roundTiles, nullptr);
+    TeamBody<TeamCopyEval>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, nullptr);
 }
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) TeamTreeKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr, uint32_t roundTiles)
+    uint32_t *__restrict__ teamCtr)
 {
-    TeamBody<TeamTreeEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, roundTiles, nullptr);
+    TeamBody<TeamTreeEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, nullptr);
 }
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlockThreads) TeamStackKernel(const FusedDesc *__restrict__ items, uint32_t nitems,
     uint32_t ntiles, const void *const *__restrict__ srcPool, void *const *__restrict__ dstPool, uint32_t tilesPerItem,
-    uint32_t *__restrict__ teamCtr, uint32_t roundTiles)
+    uint32_t *__restrict__ teamCtr)
 {
-    TeamBody<TeamStackEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, roundTiles, items + nitems);
+    TeamBody<TeamStackEval<T, OP>>(items, nitems, ntiles, srcPool, dstPool, tilesPerItem, teamCtr, items + nitems);
 }
 
 }  // namespace hcclamd

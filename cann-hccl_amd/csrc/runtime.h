@@ -59,7 +59,7 @@ struct LaunchRec {
     uint32_t grid = 0;
     uint32_t dynamicLds = 0;      // bytes of dynamic LDS the launch asks for (team kernels)
     // kernel arguments: step kernels take (table, nitems, nwhole, ntiles, flags), fused kernels
-    // (table, nitems, ntiles, srcPool, dstPool, tilesPerItem), their team forms two more: (..., teamCtr, roundTiles)
+    // (table, nitems, ntiles, srcPool, dstPool, tilesPerItem), their team forms one more: (..., teamCtr)
     const void *table = nullptr;
     uint32_t nitems = 0;
     uint32_t ntiles = 0;
@@ -68,8 +68,8 @@ struct LaunchRec {
     const void *srcPool = nullptr;
     const void *dstPool = nullptr;
     uint32_t tilesPerItem = 0;    // fused: every item covers this many tiles (the last at most as many); 0 = they differ
-    void *teamCtr = nullptr;      // team kernels: this launch's barrier counters inside the prepared tables (zero between launches)
-    uint32_t roundTiles = 0;      // team kernels: tiles per workgroup and round
+    void *teamCtr = nullptr;      // team kernels: this launch's team block inside the prepared tables (counters, regions, slots)
+    uint32_t roundTiles = 0;      // team kernels: tiles per workgroup in a full-size region
     bool fusedArgs = false;
     bool team = false;
 };
