@@ -46,7 +46,7 @@ class HcclAmdOpInfo(ctypes.Structure):
     _fields_ = [("coll", ctypes.c_int32), ("algo", ctypes.c_int32), ("fused", ctypes.c_int32), ("graph", ctypes.c_int32),
                 ("cacheHit", ctypes.c_int32), ("launches", ctypes.c_uint32), ("bytesRead", ctypes.c_uint64),
                 ("bytesWritten", ctypes.c_uint64), ("schedRead", ctypes.c_uint64), ("schedWritten", ctypes.c_uint64),
-                ("scratchBytes", ctypes.c_uint64)]
+                ("scratchBytes", ctypes.c_uint64), ("teamLaunches", ctypes.c_uint32), ("reserved", ctypes.c_uint32)]
 
 
 class HcclCommConfig(ctypes.Structure):

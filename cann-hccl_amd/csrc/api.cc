@@ -1675,6 +1675,8 @@ HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info)
     info->schedRead = o.stepRead;
     info->schedWritten = o.stepWritten;
     info->scratchBytes = o.scratchBytes;
+    info->teamLaunches = o.teamLaunches;
+    info->reserved = 0;
     return HCCL_SUCCESS;
 }
 

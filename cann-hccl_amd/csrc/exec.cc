@@ -200,7 +200,7 @@ template <typename F> void SplitByAlignment(const std::vector<uintptr_t> &addrs,
 }
 
 constexpr size_t kGraphMinLaunches = 12;   // fewer launches go out one by one
-constexpr uint32_t kTeamMinRounds = 4;     // the team kernels are chosen for launches of at least this many rounds
+constexpr uint32_t kTeamMinRounds = 2;     // the team kernels are chosen for launches of at least this many full rounds
 constexpr size_t kAsyncUploadBytes = 4 * kNoAllocUploadBytes;   // tables up to this size are uploaded by launches
 
 uint32_t TilesOf(uint64_t bytes) { return uint32_t((bytes + kTileBytes - 1) / kTileBytes); }
@@ -578,13 +578,19 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                     pl.rec.team = true;
                     pl.rec.grid = g->numCu;
                     pl.rec.dynamicLds = kTeamDynamicLds;
-                    // The regions the teams draw: roundTiles tiles per workgroup at first; over the last quarter of the
-                    // tiles the size is halved whenever fewer than 16 regions of the current size are left, so that
-                    // the XCDs finish together (measured, 8 x 256 MiB fp32 all-reduce: 727 us with 64 equal regions
-                    // dealt out in order, 714 us with the shrinking tail drawn from the counter).
+                    // The regions the teams draw: roundTiles tiles per workgroup (fewer when that would leave an XCD
+                    // without a region); over the last quarter of the tiles the size is halved whenever fewer than 16
+                    // regions of the current size are left.  The XCDs do not all move data at the same rate, and with
+                    // regions that get smaller towards the end they finish together (measured, 8 x 256 MiB fp32
+                    // all-reduce: 727 us with 64 equal regions dealt out in order, 714 us with the shrinking tail
+                    // drawn from the counter; shrinking earlier costs more than it brings, small regions run slower).
                     const uint32_t perX = g->numCu / kTeamXcds;
                     std::vector<TeamRegion> regions;
-                    for (uint32_t at = 0, per = pl.rec.roundTiles; at < tiles;) {
+                    uint32_t per = pl.rec.roundTiles;
+                    while (per > 1 && uint64_t(per) * perX * kTeamXcds > tiles) {
+                        per /= 2;
+                    }
+                    for (uint32_t at = 0; at < tiles;) {
                         const uint32_t left = tiles - at;
                         if (uint64_t(at) * 4 >= uint64_t(tiles) * 3) {
                             while (per > 1 && uint64_t(per) * perX * 16 > left) {
@@ -1081,6 +1087,10 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAl
     info.fused = pp->fused ? 1 : 0;
     info.graph = 0;
     info.launches = uint32_t(pp->launches.size());
+    info.teamLaunches = 0;
+    for (const LaunchRec &l : pp->launches) {
+        info.teamLaunches += l.team ? 1u : 0u;
+    }
     info.bytesRead = pp->fused ? pp->plan->fusedRead : pp->plan->stepRead;
     info.bytesWritten = pp->fused ? pp->plan->fusedWritten : pp->plan->stepWritten;
     info.stepRead = pp->plan->stepRead;

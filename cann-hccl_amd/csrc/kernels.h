@@ -80,17 +80,19 @@ enum KernelKind : int {
 // them together (kernels_team.h).  Launched with a multiple of kTeamXcds workgroups (one per CU) and kTeamDynamicLds
 // bytes of dynamic LDS; takes one more argument, the launch's team block in device memory, which belongs to this launch
 // alone.  Layout, in uint32 words:
-//   [x * kTeamCtrStride + kTeamArrive / kTeamGaveUp]   x < kTeamXcds: barrier arrivals of team x; set once a wait ran out
+//   [x * kTeamCtrStride + kTeamArrive]   x < kTeamXcds: barrier arrivals of team x; kTeamGaveUpBit set once a wait ran out
+//   [x * kTeamCtrStride + kTeamLeft]     workgroups of team x that have finished
 //   [kTeamTicket]       regions handed out beyond the first kTeamXcds
-//   [kTeamFinished]     workgroups that have finished
+//   [kTeamFinished]     teams that have finished
 //   [kTeamRegionCount]  number of regions n (written by the host, never changed)
 //   [kTeamHeaderWords ...]            n x TeamRegion (written by the host, never changed)
 //   [kTeamHeaderWords + 2 n ...]      kTeamXcds x (n + 1) slots: the region of team x's round r + 1, plus 2; 1 = being drawn
 // Everything but the count and the table starts out zero, and the kernel leaves it zero again.
 constexpr uint32_t kTeamTiles = 8;        // tiles a workgroup can park per round
 constexpr uint32_t kTeamXcds = 8;
-constexpr uint32_t kTeamCtrStride = 16;   // words per XCD (64 bytes)
-constexpr uint32_t kTeamArrive = 0, kTeamGaveUp = 1;
+constexpr uint32_t kTeamCtrStride = 32;   // words per XCD (128 bytes, a memory line of its own)
+constexpr uint32_t kTeamArrive = 0, kTeamLeft = 1;
+constexpr uint32_t kTeamGaveUpBit = 0x80000000u;
 constexpr uint32_t kTeamTicket = kTeamXcds * kTeamCtrStride, kTeamFinished = kTeamTicket + 1, kTeamRegionCount = kTeamTicket + 2;
 constexpr uint32_t kTeamHeaderWords = kTeamTicket + 4;
 constexpr uint32_t kTeamDynamicLds = kTeamTiles * kTileBytes;

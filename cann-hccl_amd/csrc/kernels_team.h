@@ -68,22 +68,29 @@ __device__ __forceinline__ uint32_t TeamNextRegion(uint32_t *slot, uint32_t *tic
 }
 
 // Arrival at the team's barrier, then (thread 0) the question for the next region while the others arrive, then the
-// wait: bounded, and given up for the rest of the launch once it has run out.
+// wait: bounded, and given up for the rest of the launch once it has run out (kTeamGaveUpBit in the arrival word).
+// Every access here is a trip to memory and back, a few microseconds under load, and whatever the last workgroup to
+// arrive does here delays its whole team: it learns from its own arrival that nobody is missing, and it has
+// normally seen the next region already (`seen`: a look at the slot taken before its last tile).
 __device__ __forceinline__ uint32_t TeamBarrier(uint32_t *c, uint32_t target, uint32_t *slot, uint32_t *ticket, uint32_t seen,
     uint32_t *nextShared)
 {
     __syncthreads();
     if (threadIdx.x == 0) {
-        TeamAdd(c + kTeamArrive, 1u);
+        uint32_t v = TeamAdd(c + kTeamArrive, 1u) + 1u;
         *nextShared = TeamNextRegion(slot, ticket, seen);
-        if (TeamLoad(c + kTeamGaveUp) == 0u) {
+        if ((v & ~kTeamGaveUpBit) < target && (v & kTeamGaveUpBit) == 0u) {
             const uint64_t t0 = wall_clock64();
-            while (TeamLoad(c + kTeamArrive) < target) {
-                if (wall_clock64() - t0 > kTeamWaitTicks) {
-                    TeamStore(c + kTeamGaveUp, 1u);
+            for (;;) {
+                v = TeamLoad(c + kTeamArrive);
+                if ((v & ~kTeamGaveUpBit) >= target || (v & kTeamGaveUpBit) != 0u) {
                     break;
                 }
-                __builtin_amdgcn_s_sleep(2);
+                if (wall_clock64() - t0 > kTeamWaitTicks) {
+                    __hip_atomic_fetch_or(c + kTeamArrive, kTeamGaveUpBit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
             }
         }
     }
@@ -91,13 +98,18 @@ __device__ __forceinline__ uint32_t TeamBarrier(uint32_t *c, uint32_t target, ui
     return *nextShared;
 }
 
-// The last workgroup of the launch to finish puts every counter and slot back to zero.
-__device__ __forceinline__ void TeamLeave(uint32_t *teamCtr, uint32_t nregions)
+// The last workgroup of the launch to finish puts every counter and slot back to zero.  Counted in two levels (the last
+// of a team reports for the team): atomics on one address are carried out one after the other, a hundred nanoseconds
+// and more each, and a whole grid counting on one word is most of a small launch's time.
+__device__ __forceinline__ void TeamLeave(uint32_t *teamCtr, uint32_t *ctr, uint32_t teamSize, uint32_t nregions)
 {
     __shared__ uint32_t last;
     __syncthreads();
     if (threadIdx.x == 0) {
-        last = TeamAdd(teamCtr + kTeamFinished, 1u) + 1u == gridDim.x ? 1u : 0u;
+        last = 0u;
+        if (TeamAdd(ctr + kTeamLeft, 1u) + 1u == teamSize) {
+            last = TeamAdd(teamCtr + kTeamFinished, 1u) + 1u == kTeamXcds ? 1u : 0u;
+        }
     }
     __syncthreads();
     if (last) {       // everybody else is past every barrier and every slot
@@ -107,7 +119,7 @@ __device__ __forceinline__ void TeamLeave(uint32_t *teamCtr, uint32_t nregions)
         }
         if (threadIdx.x < kTeamXcds) {
             TeamStore(teamCtr + threadIdx.x * kTeamCtrStride + kTeamArrive, 0u);
-            TeamStore(teamCtr + threadIdx.x * kTeamCtrStride + kTeamGaveUp, 0u);
+            TeamStore(teamCtr + threadIdx.x * kTeamCtrStride + kTeamLeft, 0u);
         }
         if (threadIdx.x == 0) {
             TeamStore(teamCtr + kTeamTicket, 0u);
@@ -169,11 +181,7 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
         const TeamRegion reg = regions[region];
         const uint32_t first = reg.first + inTeam * reg.per;
         const uint32_t n = first < ntiles ? (ntiles - first < reg.per ? ntiles - first : reg.per) : 0;
-        // an early look at the slot of the next round: a workgroup that is behind finds the answer there already
         uint32_t seen = 0;
-        if (threadIdx.x == 0) {
-            seen = TeamLoad(slots + round);
-        }
         uint32_t maxDst = 0;
         uint32_t idx = 0;
         FusedDesc d;
@@ -181,6 +189,11 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
         Eval eval;
         for (uint32_t q = 0; q < n; q++) {
             const uint32_t tile = first + q;
+            if (q + 1 == n && threadIdx.x == 0) {
+                // a look at the slot of the next round, in flight together with the last tile's loads: a workgroup
+                // that is behind the others finds the answer there
+                seen = TeamLoad(slots + round);
+            }
             if (q == 0 || tile >= dEnd) {
                 idx = ItemOfTile(items, nitems, tile, tilesPerItem);
                 d = items[idx];
@@ -241,7 +254,7 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
         // the next round's results must not land in LDS before this round's have been read
         __syncthreads();
     }
-    TeamLeave(teamCtr, nregions);
+    TeamLeave(teamCtr, ctr, teamSize, nregions);
 }
 
 // ---- what a tile's value is, per kernel family --------------------------------------------------------------------

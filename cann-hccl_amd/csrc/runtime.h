@@ -77,6 +77,7 @@ struct LaunchRec {
 struct OpInfo {
     int coll = 0, algo = 0, fused = 0, graph = 0, cacheHit = 0;
     uint32_t launches = 0;
+    uint32_t teamLaunches = 0;
     uint64_t bytesRead = 0, bytesWritten = 0;     // what the issued kernels move in HBM, all ranks
     uint64_t stepRead = 0, stepWritten = 0;       // the step-by-step schedule's figure
     uint64_t scratchBytes = 0;

@@ -84,6 +84,8 @@ typedef struct HcclAmdOpInfoDef {
     uint64_t schedRead;      /* same for the step-by-step schedule (direct peer reads, no staging) */
     uint64_t schedWritten;
     uint64_t scratchBytes;   /* per-rank scratch in use */
+    uint32_t teamLaunches;   /* how many of the launches are team kernels (setting "team") */
+    uint32_t reserved;
 } HcclAmdOpInfo;
 
 /* What the most recent collective of this communicator's group issued. */
