@@ -5,8 +5,9 @@ Default workload: ring all-reduce, sum, fp32, 8 simulated ranks x 256 MiB per ra
 rank).  Prints one JSON line.
 
 The headline (`value`, `ms_per_step`, `roofline`) is the library's default mode: the fused single pass (one
-launch of ChainKernel<float, sum>) that reads every rank's input once, combines in the ring schedule's order and
-writes every rank's output once -- 2 * p * S algorithmic bytes per collective, bit for bit the schedule's result.
+launch of TeamChainKernel<float, sum>: the workgroups of an XCD read their tiles together, hold the results in LDS
+and write them together) that reads every rank's input once, combines in the ring schedule's order and writes
+every rank's output once -- 2 * p * S algorithmic bytes per collective, bit for bit the schedule's result.
 The schedule run step by step (library setting fuse=0: one launch per phase of copy / reduce steps, replayed from a
 HIP graph, 5 * (p - 1) * S bytes, 1.9 times slower per collective) is timed in the same run and reported under
 `config.step_by_step` and `roofline_steps`; part of what its phases read comes out of the 256 MB memory-side cache,
@@ -26,7 +27,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 METRIC = "achieved HBM GB/s & % of peak, 8-rank fp32 ring AllReduce 256MiB/rank"
 
-PROFILE_FUSED = os.path.join(ROOT, "profiles", "ChainKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt")
+PROFILE_FUSED = os.path.join(ROOT, "profiles", "TeamChainKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt")
 PROFILE_STEPS = os.path.join(ROOT, "profiles", "StepKernel_fp32_sum__ring_allreduce_8ranks_256MiB.txt")
 
 
@@ -501,7 +502,7 @@ def main():
     headline = p == 8 and args.size_mib == 256.0 and not args.set and info["algo"] == 0
     sched_name = {0: "ring", 1: "mesh", 2: "halving-doubling", 4: "mesh"}.get(info["algo"], "?")
     launches = max(1, s_info["launches"])
-    fused_kernel = "TreeKernel" if info["algo"] == 2 else "ChainKernel"
+    fused_kernel = ("Team" if info.get("teamLaunches") else "") + ("TreeKernel" if info["algo"] == 2 else "ChainKernel")
     # The headline is what a caller of HcclAllReduce gets with the library's defaults (fuse=1): one fused launch.
     line = {
         "metric": METRIC,
@@ -522,6 +523,7 @@ def main():
             "issue": "library default (fuse=1): one %s launch per collective reads every rank's input once, combines in "
                      "the %s schedule's order and writes every rank's output; same bits as the schedule run step by step"
                      % (fused_kernel, sched_name),
+            "team_kernel": bool(info.get("teamLaunches")),
             "default_mode": "fused single pass",
             "launches_per_step": info["launches"],
             "graph": info["graph"],
@@ -553,9 +555,6 @@ def main():
             "kernel": "%s<float, sum> (fused %s all-reduce, the library default): %d algorithmic bytes per launch "
                       "(%d x %.0f MiB read + the same written), average launch %.4f ms over %d launches, HIP events on "
                       "the launching stream" % (fused_kernel, sched_name, actual, p, args.size_mib, dev_ms, args.steps),
-            "shape_ceiling": "a plain kernel that only reads 8 streams and writes 8 (no tables, no arithmetic) reaches 5.4-5.7 TB/s "
-                             "on this part, read-only 7.0, write-only 6.5 (profiles/hbm_probe__plain_kernels_256MiB_streams.txt; "
-                             "write-path counters in profiles/ChainKernel__write_path_counters_8ranks_256MiB.txt)" if headline else None,
         },
         "roofline_steps": {
             "bound": "hbm", "achieved": round(s_achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
