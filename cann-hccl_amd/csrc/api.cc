@@ -265,6 +265,10 @@ HcclResult JoinFormingGroup(const std::string &key, uint32_t nRanks, uint32_t ra
     }
     if (complete) {
         g_forming.erase(key);
+        // Device set-up with the last rank's device current, as HcclCommInitAll does it: no collective call -- in
+        // particular not the one that promises to allocate nothing -- is then the first to touch the device.
+        // Without a GPU the group exists all the same and its collectives fail with HCCL_E_RUNTIME.
+        (void)EnsureDevice(g, true);
     }
     return HCCL_SUCCESS;
 }

@@ -1216,6 +1216,8 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
             HCCL_LOG_ERROR("%s without allocation: the fixed workspace was not set up", CollName(g->ctx->sig.coll));
             return HCCL_E_INTERNAL;
         }
+        // an earlier call's work may still be reading the workspace from another stream
+        HIP_OK(NoAllocBegin(g->device, g->ctx->streams[launcher]));
         r = Prepare(g, algo, &uncached, true, g->ctx->streams[launcher]);
         if (r != HCCL_SUCCESS) {
             return r;
@@ -1358,6 +1360,9 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
             KernelArgs(l, args);
             HIP_OK(hipLaunchKernel(l.func, dim3(l.grid, 1, 1), dim3(kBlockThreads, 1, 1), args, l.dynamicLds, ls));
         }
+    }
+    if (g->ctx->sig.noAlloc) {
+        HIP_OK(NoAllocEnd(g->device, ls));
     }
     g->launchStreams[g->opSerial % 8] = ls;
     g->doneRecorded[g->opSerial % 8] = false;

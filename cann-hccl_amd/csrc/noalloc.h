@@ -15,6 +15,13 @@ constexpr size_t kNoAllocUploadBytes = 3072;               // table bytes per up
 // looks the symbol up; later calls return the kept pointer.
 hipError_t NoAllocWorkspace(int device, void **base);
 
+// Calls on one GPU share that GPU's workspace.  NoAllocBegin, called before a call's first launch on `stream`, makes the
+// stream wait for the previous call's work when that went to another stream (an event created with the workspace: nothing
+// is allocated here); NoAllocEnd, after the call's last launch, marks the stream as the workspace's latest user.  Both
+// do nothing while `stream` is being captured: a graph's replays are the caller's to order.
+hipError_t NoAllocBegin(int device, hipStream_t stream);
+hipError_t NoAllocEnd(int device, hipStream_t stream);
+
 // Queues on `stream` the launches that write hostBytes[0, bytes) to dst (device memory, 16-byte aligned; the
 // copy is rounded up to a multiple of 16 bytes).  The host bytes are consumed before the call returns.
 // Also used for the small tables of ordinary collectives: unlike a host-to-device copy it never waits.

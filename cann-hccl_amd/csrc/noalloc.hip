@@ -23,6 +23,10 @@ static __device__ __align__(256) unsigned char scratch[kNoAllocTableBytes + kNoA
 constexpr int kMaxDevices = 64;
 std::mutex g_lock;
 void *g_scratchOnDevice[kMaxDevices] = {};
+// the workspace's latest user: an event recorded behind its work, and the stream that work went to
+hipEvent_t g_lastUse[kMaxDevices] = {};
+hipStream_t g_lastStream[kMaxDevices] = {};
+bool g_used[kMaxDevices] = {};
 
 // Table bytes travel as kernel arguments: no host-to-device copy, nothing to stage or allocate, and a
 // launch is ordered on the caller's stream like every other kernel of the collective.
@@ -61,10 +65,62 @@ hipError_t NoAllocWorkspace(int device, void **base)
         if (e != hipSuccess) {
             return e;
         }
+        e = hipEventCreateWithFlags(&g_lastUse[device], hipEventDisableTiming);
+        if (e != hipSuccess) {
+            return e;
+        }
         g_scratchOnDevice[device] = ptr;
     }
     *base = g_scratchOnDevice[device];
     return hipSuccess;
+}
+
+namespace {
+
+hipError_t Capturing(hipStream_t stream, bool *capturing)
+{
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    hipError_t e = hipStreamIsCapturing(stream, &status);
+    *capturing = status != hipStreamCaptureStatusNone;
+    return e;
+}
+
+}  // namespace
+
+hipError_t NoAllocBegin(int device, hipStream_t stream)
+{
+    if (device < 0 || device >= kMaxDevices) {
+        return hipErrorInvalidDevice;
+    }
+    bool capturing = false;
+    hipError_t e = Capturing(stream, &capturing);
+    if (e != hipSuccess || capturing) {
+        return e;
+    }
+    std::lock_guard<std::mutex> hold(g_lock);
+    if (g_used[device] && g_lastStream[device] != stream) {
+        return hipStreamWaitEvent(stream, g_lastUse[device], 0);
+    }
+    return hipSuccess;
+}
+
+hipError_t NoAllocEnd(int device, hipStream_t stream)
+{
+    if (device < 0 || device >= kMaxDevices) {
+        return hipErrorInvalidDevice;
+    }
+    bool capturing = false;
+    hipError_t e = Capturing(stream, &capturing);
+    if (e != hipSuccess || capturing) {
+        return e;
+    }
+    std::lock_guard<std::mutex> hold(g_lock);
+    e = hipEventRecord(g_lastUse[device], stream);
+    if (e == hipSuccess) {
+        g_lastStream[device] = stream;
+        g_used[device] = true;
+    }
+    return e;
 }
 
 hipError_t UploadThroughKernelArgs(void *dst, const void *hostBytes, size_t bytes, hipStream_t stream)

@@ -9,6 +9,7 @@
 #pragma once
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
 #include <condition_variable>
 #include <deque>
 #include <cstdint>
@@ -188,7 +189,7 @@ struct Group {
     std::map<std::pair<uint32_t, uint32_t>, std::deque<P2PPending>> p2p;
 
     // device resources
-    bool deviceReady = false;
+    std::atomic<bool> deviceReady{false};   // set last by EnsureDevice; a rank's early stream marker reads it without the group's lock
     int device = 0;
     uint32_t numCu = 256;
     std::vector<hipEvent_t> arriveEvents;

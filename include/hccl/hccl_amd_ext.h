@@ -120,10 +120,14 @@ extern HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRank
  * equally by the ranks: nRanks * recvCount * sizeof(type) partial bytes per rank must fit its share).
  * Larger requests fail with HCCL_E_PARA and a message.  Nothing is cached and no graph is built, so a call
  * costs a plan lookup and one small upload launch per 3 KiB of tables on top of the kernels.  All calls on a
- * GPU share that GPU's workspace, whichever group they come from: a call must not be issued while an earlier one may
- * still be running on another stream (calls of one group whose ranks keep their streams are ordered by the
- * library; anything else is the caller's to order).  Nothing in the workspace has to start at zero: tables
- * are rewritten by every call and partial results are written before they are read. */
+ * GPU share that GPU's workspace, whichever group they come from.  The library orders them: a call whose work goes to
+ * another stream than the previous call's is queued behind that work (an event created at set-up, nothing allocated),
+ * so calls from several groups or streams each get their own result, one after the other.  The exception is a call
+ * recorded under stream capture: no event is waited for or recorded there, and replays of the captured graph that may
+ * overlap other calls of this kind on another stream are the caller's to order.  The device is set up when a group is
+ * complete (HcclCommInitAll, or the last rank's HcclCommInitRootInfo / ...ClusterInfo / HcclCreateSubCommConfig), so
+ * this call may be a group's first collective.  Nothing in the workspace has to start at zero: tables are rewritten by
+ * every call and partial results are written before they are read. */
 #define HCCL_AMD_NOALLOC_TABLE_BYTES (256u << 10)
 #define HCCL_AMD_NOALLOC_DATA_BYTES (32u << 20)
 extern HcclResult HcclAmdReduceScatterNoAlloc(void *sendBuf, void *recvBuf, uint64_t recvCount, HcclDataType dataType,
