@@ -75,6 +75,7 @@ def build(force=False, jobs=None):
     if force or tasks or _newer(LIB, objs):
         _run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs + ["-lpthread"])
     build_abi_caller(force)
+    build_threads_latency(force)
     return LIB
 
 
@@ -91,6 +92,18 @@ def build_abi_caller(force=False, include_dirs=None, out=None):
             inc += ["-I", d]
         _run([HIPCC, "-O1", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-Wno-unused-command-line-argument"] + inc +
              [src, "-L", LIBDIR, "-lhccl", "-Wl,-rpath,$ORIGIN", "-o", out])
+    return out
+
+
+def build_threads_latency(force=False):
+    """Links the calling-model timing program (tests/c_abi/threads_latency.cc) against the library."""
+    src = os.path.join(ROOT, "tests", "c_abi", "threads_latency.cc")
+    out = os.path.join(LIBDIR, "threads_latency")
+    if not os.path.exists(src):
+        return None
+    if force or _newer(out, [src, LIB]):
+        _run([HIPCC, "-O2", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"),
+              src, "-L", LIBDIR, "-lhccl", "-lpthread", "-Wl,-rpath,$ORIGIN", "-o", out])
     return out
 
 

@@ -397,7 +397,7 @@ HcclResult Arrive(Comm *c, const OpSig &sig, void *send, void *recv, hipStream_t
         const HcclResult res = g->issueResults[serial % 8];
         // what follows on this rank's stream comes after the collective
         const bool wait = res == HCCL_SUCCESS && g->doneRecorded[serial % 8] && g->launchStreams[serial % 8] != stream;
-        hipEvent_t doneEvent = g->doneEvent;
+        hipEvent_t doneEvent = g->doneEvents[serial % 8];
         lock.unlock();
         if (wait && hipStreamWaitEvent(stream, doneEvent, 0) != hipSuccess) {
             (void)hipGetLastError();
@@ -501,7 +501,7 @@ HcclResult PointToPoint(Comm *c, bool isSend, void *buf, uint64_t count, HcclDat
     }
     g->ctx = &g->pend;
     if (res == HCCL_SUCCESS && toSelf && match.stream != stream) {
-        if (hipEventRecord(g->doneEvent, stream) != hipSuccess || hipStreamWaitEvent(match.stream, g->doneEvent, 0) != hipSuccess) {
+        if (hipEventRecord(g->p2pDoneEvent, stream) != hipSuccess || hipStreamWaitEvent(match.stream, g->p2pDoneEvent, 0) != hipSuccess) {
             (void)hipGetLastError();
             res = HCCL_E_RUNTIME;
         }

@@ -54,7 +54,10 @@ HcclResult EnsureDevice(Group *g, bool quiet)
     for (uint32_t r = 0; r < g->p; r++) {
         HIP_OK(hipEventCreateWithFlags(&g->arriveEvents[r], hipEventDisableTiming));
     }
-    HIP_OK(hipEventCreateWithFlags(&g->doneEvent, hipEventDisableTiming));
+    for (hipEvent_t &e : g->doneEvents) {
+        HIP_OK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    }
+    HIP_OK(hipEventCreateWithFlags(&g->p2pDoneEvent, hipEventDisableTiming));
     HIP_OK(hipStreamCreateWithFlags(&g->copyStream, hipStreamNonBlocking));
     g->stageSlots.resize(kStageSlots);
     for (StageSlot &slot : g->stageSlots) {
@@ -1148,8 +1151,13 @@ Group::~Group()
             (void)hipEventDestroy(e);
         }
     }
-    if (doneEvent) {
-        (void)hipEventDestroy(doneEvent);
+    for (hipEvent_t e : doneEvents) {
+        if (e) {
+            (void)hipEventDestroy(e);
+        }
+    }
+    if (p2pDoneEvent) {
+        (void)hipEventDestroy(p2pDoneEvent);
     }
     for (void *s : scratch) {
         if (s) {
@@ -1364,15 +1372,24 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     if (g->ctx->sig.noAlloc) {
         HIP_OK(NoAllocEnd(g->device, ls));
     }
-    g->launchStreams[g->opSerial % 8] = ls;
-    g->doneRecorded[g->opSerial % 8] = false;
+    // A rank blocked in its call picks up "its" collective's entry and event after it wakes, when later operations may
+    // already have been issued: every rendezvous has its own entry and event (by serial number modulo the ring's
+    // size), and a matched send / receive, which is not a rendezvous, has an event of its own.
+    const bool p2p = g->ctx->sig.coll == COLL_SENDRECV;
+    hipEvent_t done = p2p ? g->p2pDoneEvent : g->doneEvents[g->opSerial % 8];
+    if (!p2p) {
+        g->launchStreams[g->opSerial % 8] = ls;
+        g->doneRecorded[g->opSerial % 8] = false;
+    }
     if (others) {
-        HIP_OK(hipEventRecord(g->doneEvent, ls));
-        g->doneRecorded[g->opSerial % 8] = true;
+        HIP_OK(hipEventRecord(done, ls));
+        if (!p2p) {
+            g->doneRecorded[g->opSerial % 8] = true;
+        }
         // ranks blocked in their calls make their own streams wait when they wake up, each on its own thread
         for (uint32_t k = 0; k < g->p && !g->ctx->ranksWaitThemselves; k++) {
             if (k != launcher && g->ctx->streams[k] != ls) {
-                HIP_OK(hipStreamWaitEvent(g->ctx->streams[k], g->doneEvent, 0));
+                HIP_OK(hipStreamWaitEvent(g->ctx->streams[k], done, 0));
             }
         }
     }

@@ -182,7 +182,7 @@ struct Group {
     // rendezvous n reads entry n even if the other ranks have moved on to n + 1 by the time it wakes.
     HcclResult issueResults[8] = {};
     hipStream_t launchStreams[8] = {};   // same indexing: the stream the collective went to ...
-    bool doneRecorded[8] = {};           // ... and whether the done event was recorded after it for the other streams
+    bool doneRecorded[8] = {};           // ... and whether its done event was recorded after it for the other streams
     std::vector<uint8_t> here;
     OpCtx pend;                      // what the ranks of the current collective passed
     OpCtx *ctx = nullptr;            // the operation being issued (the rendezvous, or a matched send / receive)
@@ -193,7 +193,8 @@ struct Group {
     int device = 0;
     uint32_t numCu = 256;
     std::vector<hipEvent_t> arriveEvents;
-    hipEvent_t doneEvent = nullptr;
+    hipEvent_t doneEvents[8] = {};        // one per entry of the ring above: recorded behind that collective for the other ranks' streams
+    hipEvent_t p2pDoneEvent = nullptr;    // the same for a matched send / receive, which is no rendezvous and has no entry
     std::vector<void *> scratch;
     std::vector<void *> retiredScratch;   // scratch buffers a pinned collective still points at; freed with the group
     uint32_t pinnedScratchUsers = 0;      // pinned collectives that use the current scratch buffers

@@ -1440,6 +1440,26 @@ def test_compiled_caller_through_the_c_abi():
     assert r.returncode == 0 and "ABI_CALLER_OK" in r.stdout, r.stdout[-2000:]
 
 
+def test_host_cost_of_a_small_collective_per_calling_model():
+    # One thread and one stream per rank with blocking calls (the reference's calling model) against one thread driving
+    # all ranks on one stream: prints the microseconds per 8 KiB all-reduce.  The threaded model costs about 3p calls
+    # into the HIP runtime per collective, which the runtime serialises; the bounds only catch a regression by a
+    # factor (measured: 53 - 60 us at 8 ranks, 92 - 104 us at 16; one thread 3.7 / 6 us).
+    import os
+    import re
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "cann-hccl_amd", "lib", "threads_latency")
+    assert os.path.exists(exe), "run cann-hccl_amd/build.py first"
+    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+    print(r.stdout, flush=True)
+    assert r.returncode == 0, r.stdout[-2000:]
+    got = {(int(m.group(1)), "thread per rank" in m.group(2)): float(m.group(3))
+           for m in re.finditer(r"p=\s*(\d+) (.*?): ([0-9.]+) us per all-reduce", r.stdout)}
+    assert len(got) == 4, r.stdout
+    assert got[(8, True)] < 150 and got[(16, True)] < 300, got
+    assert got[(8, False)] < 20 and got[(16, False)] < 30, got
+
+
 def test_one_thread_per_rank_blocking_arrival(orc):
     # the reference's model: every rank on its own thread and stream; calls return once the collective is issued
     import threading
