@@ -444,6 +444,31 @@ def test_plans_derived_from_a_template_of_another_count_are_the_planners_own(tmp
     assert tables > 300, out.stdout
 
 
+def test_seeded_walk_over_requests_and_counts_derives_only_the_planners_own_plans(tmp_path):
+    """tests/c_abi/plan_template_walk.cc: random requests (collective, schedule, 2 .. 33 ranks, rank groups, rings inside a
+    group, ranks with a network port, ranks in place, element size, CCL buffer size) and for each a sequence of counts --
+    whole slices, ragged, tiny, several chunks -- or of block tables, with up to four templates kept per request as the
+    library keeps them: 20 000 derived plans per run, each compared with the plan made from scratch; tables with gaps or
+    empty blocks must not be derived.  HCCL_AMD_TEST_SEED_SHIFT moves the walk to other cases."""
+    import os
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        pytest.skip("no host C++ compiler")
+    exe = str(tmp_path / "plan_template_walk")
+    subprocess.run([cxx, "-O2", "-std=c++17", "-Wall", "-Werror", "-I", os.path.join(root, "cann-hccl_amd", "csrc"),
+                    "-I", os.path.join(root, "include"), os.path.join(root, "tests", "c_abi", "plan_template_walk.cc"),
+                    os.path.join(root, "cann-hccl_amd", "csrc", "plan.cc"), "-o", exe], check=True)
+    out = subprocess.run([exe, "20000"], stdout=subprocess.PIPE, text=True, timeout=300)
+    print(out.stdout)
+    assert out.returncode == 0 and out.stdout.startswith("OK"), out.stdout
+    words = out.stdout.replace("(", " ").split()
+    assert int(words[1]) >= 20000, out.stdout
+    assert int(words[3]) > 1000 and int(words[8]) > 100, out.stdout          # ragged counts, block templates
+
+
 def _rank_table(path, servers, per_server, **edits):
     import json
     table = {"server_count": str(servers), "status": "completed", "version": "1.0", "server_list": []}
