@@ -1513,6 +1513,8 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
             cfg.algo = ALGO_PAIRWISE;   // all-to-all family: the flat schedule also over several servers; others: ring
         } else if (v == "star") {
             cfg.algo = ALGO_STAR;       // broadcast: the root hands every rank the whole buffer; others: as "auto" would not, ring
+        } else if (v == "hd_blocks") {
+            cfg.algo = ALGO_HD_BLOCKS;  // broadcast: halving-doubling over blocks of power-of-two sizes; others: ring
         } else if (v == "auto") {
             cfg.algo = -1;
         } else {
@@ -1694,7 +1696,7 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
     PlanRequest rq;
     rq.coll = CollKind(coll);
     if (coll >= COLL_BROADCAST) {
-        // rooted collectives: low 16 bits = root rank, bits 16..19 = schedule (0 ring, 1 mesh, 2 rhd, 4 mesh uncut, 5 star);
+        // rooted collectives: low 16 bits = root rank, bits 16..19 = schedule (0 ring, 1 mesh, 2 rhd, 4 mesh uncut, 5 star, 6 hd over blocks);
         // reduce only: bits 20..27 = number of rank groups of the two-level schedule, bit 28 = its mesh level uncut,
         // bit 29 / bit 30 = one ring / four rings inside a group instead of the mesh
         rq.root = uint32_t(algo) & 0xffffu;

@@ -985,7 +985,7 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAl
         rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
     }
     if (rq.coll == COLL_BROADCAST && g->cfg.servers > 1 && g->p % g->cfg.servers == 0 && g->cfg.algo != ALGO_RING &&
-        g->cfg.algo != ALGO_STAR && g->cfg.level0Rings == 0) {
+        g->cfg.algo != ALGO_STAR && g->cfg.algo != ALGO_HD_BLOCKS && g->cfg.level0Rings == 0) {
         // two levels (coll_broadcast_mesh_executor.cc:59-213): scatter in the root's group, halving-doubling between
         // the groups, mesh all-gather in every group; the flat ring when the ring is asked for by name
         rq.servers = g->cfg.servers;
@@ -1198,12 +1198,12 @@ HcclResult IssueCollective(Group *g, uint32_t launcher)
     } else if (g->ctx->sig.coll == COLL_REDUCE) {
         algo = (algo == ALGO_MESH || algo == ALGO_RHD) ? algo : ALGO_RING;   // ring, mesh or halving-doubling reduce
     } else if (g->ctx->sig.coll == COLL_BROADCAST) {
-        algo = (algo == ALGO_MESH || algo == ALGO_RHD || algo == ALGO_STAR) ? algo : ALGO_RING;   // ring, mesh, halving-doubling or star broadcast
+        algo = (algo == ALGO_MESH || algo == ALGO_RHD || algo == ALGO_STAR || algo == ALGO_HD_BLOCKS) ? algo : ALGO_RING;   // ring, mesh, halving-doubling (either kind) or star
     } else if (g->ctx->sig.coll == COLL_SCATTER) {
         algo = (g->cfg.algo == ALGO_RING) ? ALGO_RING : ALGO_MESH;   // mesh scatter unless the ring is asked for
     } else if (g->ctx->sig.coll >= COLL_SCATTER) {
         algo = ALGO_RING;   // direct send / receive
-    } else if (algo == ALGO_PAIRWISE || algo == ALGO_STAR) {
+    } else if (algo == ALGO_PAIRWISE || algo == ALGO_STAR || algo == ALGO_HD_BLOCKS) {
         algo = ALGO_RING;
     }
     // coll_all_reduce_mesh_executor.cc:108-112, coll_reduce_scatter_mesh_executor.cc:227-229,

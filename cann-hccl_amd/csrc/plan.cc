@@ -762,6 +762,76 @@ template <typename F> size_t RhdBroadcastPhases(VProgram &vp, size_t ph, uint32_
     return part1 > 0 ? ph + 1 : ph;
 }
 
+// Binary-block halving-doubling broadcast (bcast_halvingdoubling.cc:26-398) among n ranks, whole chunk per hop.  The
+// ranks are cut into blocks whose sizes are the powers of two in n, the largest block at rank 0
+// (PrepareBlockParams :26-62).  The chunk spreads through the root's block as a binomial tree, widest distance first
+// (BcastInRootBlock :165-228), and then from block to block in both directions: into the next smaller block (the one at
+// the higher ranks) every (size ratio)-th rank sends to one rank; into the next larger block every rank sends to (size
+// ratio) consecutive ranks, one after the other (GatherBetweenBlocksRootBlock :231-281, ...HigherBlock :284-335,
+// ...LowerBlock :338-396).  A rank's transfers keep their program order: each takes the phase after the rank's last.
+template <typename F> void HdBlocksBroadcastPhases(VProgram &vp, uint32_t n, uint32_t root, F data, uint64_t bytes)
+{
+    struct Block {
+        uint32_t first, size;
+    };
+    std::vector<Block> blocks;      // from the largest (rank 0) to the smallest
+    for (uint32_t bit = 1u << 31, at = 0; bit != 0; bit >>= 1) {
+        if ((n & bit) != 0) {
+            blocks.push_back(Block{at, bit});
+            at += bit;
+        }
+    }
+    size_t home = 0;
+    while (root >= blocks[home].first + blocks[home].size) {
+        home++;
+    }
+    std::vector<size_t> free(n, 0);      // the first phase in which a rank holds the chunk and is not sending
+    auto hop = [&](uint32_t from, uint32_t to) {
+        EmitCopy(vp, free[from], data(to), data(from), bytes);
+        free[from]++;
+        free[to] = free[from];
+    };
+    const Block hb = blocks[home];
+    const uint32_t rootIn = root - hb.first;
+    std::vector<uint8_t> has(hb.size, 0);
+    has[rootIn] = 1;
+    for (uint32_t mask = hb.size >> 1; mask != 0; mask >>= 1) {
+        std::vector<uint32_t> senders;
+        for (uint32_t q = 0; q < hb.size; q++) {
+            if (has[q] && !has[q ^ mask]) {
+                senders.push_back(q);
+            }
+        }
+        for (uint32_t q : senders) {
+            hop(hb.first + q, hb.first + (q ^ mask));
+            has[q ^ mask] = 1;
+        }
+    }
+    auto intoSmaller = [&](size_t b) {
+        const Block from = blocks[b], to = blocks[b + 1];
+        const uint32_t ratio = from.size / to.size;
+        for (uint32_t q = 0; q < to.size; q++) {
+            hop(from.first + q * ratio, to.first + q);
+        }
+    };
+    auto intoLarger = [&](size_t b) {
+        const Block from = blocks[b], to = blocks[b - 1];
+        const uint32_t ratio = to.size / from.size;
+        for (uint32_t i = 0; i < ratio; i++) {
+            for (uint32_t q = 0; q < from.size; q++) {
+                hop(from.first + q, to.first + q * ratio + i);
+            }
+        }
+    };
+    // the root's block serves the smaller block first, then the larger one (:246-279)
+    for (size_t b = home; b + 1 < blocks.size(); b++) {
+        intoSmaller(b);
+    }
+    for (size_t b = home; b > 0; b--) {
+        intoLarger(b);
+    }
+}
+
 int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
 {
     uint32_t p = rq.p;
@@ -1065,6 +1135,9 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
             } else if (rq.coll == COLL_BROADCAST && rq.algo == ALGO_RHD && p > 1) {
                 auto data = [&](uint32_t r) { return r == R ? MkRef(R, BUF_SEND, done) : MkRef(r, BUF_RECV, done); };
                 RhdBroadcastPhases(*vp, 0, p, R, data, bytes);
+            } else if (rq.coll == COLL_BROADCAST && rq.algo == ALGO_HD_BLOCKS && p > 1) {
+                auto data = [&](uint32_t r) { return r == R ? MkRef(R, BUF_SEND, done) : MkRef(r, BUF_RECV, done); };
+                HdBlocksBroadcastPhases(*vp, p, R, data, bytes);
             } else if (rq.coll == COLL_REDUCE && rq.servers > 1 && p > 1) {
                 TwoLevelReduceChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, rq.level0Rings, R, done, bytes,
                     rq.align, rq.meshAtomic);

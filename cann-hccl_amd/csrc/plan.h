@@ -28,7 +28,8 @@ enum CollKind : int {
 // ALGO_MESH_ATOMIC: the mesh schedule whose reduce phases skip the piece cut (the reference's
 // non-deterministic variant, taken in stream order); BuildPlan turns it into ALGO_MESH + meshAtomic.
 // ALGO_STAR: broadcast only, the root hands every rank the whole buffer (broadcast_star.cc).
-enum Algo : int { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2, ALGO_PAIRWISE = 3, ALGO_MESH_ATOMIC = 4, ALGO_STAR = 5 };
+// ALGO_HD_BLOCKS: broadcast only, halving-doubling over blocks of power-of-two sizes (bcast_halvingdoubling.cc).
+enum Algo : int { ALGO_RING = 0, ALGO_MESH = 1, ALGO_RHD = 2, ALGO_PAIRWISE = 3, ALGO_MESH_ATOMIC = 4, ALGO_STAR = 5, ALGO_HD_BLOCKS = 6 };
 
 // Physical buffers of a rank: the caller's send and receive buffers and a library-owned scratch.
 enum Buf : uint8_t { BUF_SEND = 0, BUF_RECV = 1, BUF_SCRATCH = 2 };

@@ -12,10 +12,13 @@ extern "C" {
 #endif
 
 /* Settings of the communicator's whole group.  Keys and values:
- *   "algo"          "ring" | "mesh" | "rhd" | "pairwise" | "star" | "auto"   ("pairwise" only matters to the all-to-all family,
- *                                see "servers"; the other collectives then run their ring schedules; the scatter runs
- *                                the mesh schedule unless "ring" is set; "star" only matters to the broadcast: the root
- *                                hands every rank the whole buffer at once, also over several servers)
+ *   "algo"          "ring" | "mesh" | "rhd" | "pairwise" | "star" | "hd_blocks" | "auto"   ("pairwise" only matters to the
+ *                                all-to-all family, see "servers"; the other collectives then run their ring schedules;
+ *                                the scatter runs the mesh schedule unless "ring" is set; "star" and "hd_blocks" only
+ *                                matter to the broadcast, also over several servers: with "star" the root hands every
+ *                                rank the whole buffer at once, with "hd_blocks" the buffer spreads by halving-doubling
+ *                                over blocks of power-of-two sizes, a binomial tree inside the root's block and then
+ *                                from block to block)
  *   "deterministic" "0" | "1"    as HCCL_DETERMINISTIC; with "0" (the default) the mesh reduce phases of
  *                                all-reduce / reduce-scatter run without the piece cut (not for int64, not for products)
  *   "fuse"          "0" | "1"    run the single-pass fused form when the schedule has one
@@ -74,7 +77,7 @@ extern HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *va
 
 typedef struct HcclAmdOpInfoDef {
     int32_t coll;            /* 0 all-reduce, 1 reduce-scatter, 2 all-gather, 3 all-to-all-v, 4 broadcast, 5 reduce, 6 scatter */
-    int32_t algo;            /* 0 ring, 1 mesh, 2 rhd, 3 pairwise, 4 mesh without the piece cut, 5 star */
+    int32_t algo;            /* 0 ring, 1 mesh, 2 rhd, 3 pairwise, 4 mesh without the piece cut, 5 star, 6 hd over blocks */
     int32_t fused;           /* 1: issued as fused single-pass kernels */
     int32_t graph;           /* 1: issued as a HIP graph */
     int32_t cacheHit;        /* 1: an instantiated graph / table set was reused */
@@ -94,7 +97,7 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
 /* Plans a collective without a device and writes the plan as JSON (phases of copy / reduce steps,
  * fused items, byte counts) into out[0..cap).  coll / algo as in HcclAmdOpInfo; for the rooted
  * collectives (coll 4 broadcast, 5 reduce, 6 scatter) the algo argument carries the root rank in its low 16 bits and the
- * schedule in bits 16..19 (0 ring, 1 mesh, 2 rhd, 4 mesh without the piece cut, 5 star: broadcast only), for the reduce also the number of rank
+ * schedule in bits 16..19 (0 ring, 1 mesh, 2 rhd, 4 mesh without the piece cut, 5 star, 6 hd over blocks: broadcast only), for the reduce also the number of rank
  * groups of its two-level schedule in bits 20..27, bit 28 for the mesh level without the piece cut and bit 29 / bit 30 for
  * one ring / four rings inside a group, for the broadcast the number of rank groups in bits 20..27, for the scatter
  * bit 20 for the ring schedule instead of the mesh and the number of rank groups of the two-level mesh schedule in bits 21..28;

@@ -2347,6 +2347,177 @@ int orc_broadcast_rhd(uint32_t p, void **buf, uint64_t count, int dt, uint32_t r
     return 0;
 }
 
+// Binary-block halving-doubling broadcast (TPL/temp_broadcast/bcast_halvingdoubling.cc:26-398).  The ranks are cut into
+// blocks whose sizes are the powers of two in the rank count, the smallest block at the highest ranks
+// (PrepareBlockParams :26-62, PrepareRootBlockParam :64-90).  Inside the root's block the buffer spreads as a binomial
+// tree, widest distance first (BcastInRootBlock :165-228); then it goes from block to block: towards the smaller block
+// every `times`-th rank sends to one rank, towards the larger block every rank sends to `rounds` consecutive ranks, one
+// after the other (GatherBetweenBlocksRootBlock :231-281, ...HigherBlock :284-335, ...LowerBlock :338-396).  Every
+// transfer carries the whole buffer.
+namespace {
+
+struct HdBlocks {
+    uint32_t myOffset = 0, mySize = 0, lower = 0, higher = 0, rankIn = 0, steps = 0;
+};
+
+HdBlocks HdBlockOf(uint32_t rank, uint32_t n)
+{
+    HdBlocks b;
+    uint32_t offset = n, blockSize = 1, current = 0, pre = 0;
+    while (offset > 0) {
+        if ((n & blockSize) != 0) {
+            pre = current;
+            current = blockSize;
+            offset -= blockSize;
+            if (b.mySize != 0) {
+                b.higher = current;
+                break;
+            }
+            if (offset <= rank) {
+                b.myOffset = offset;
+                b.mySize = current;
+                b.lower = pre;
+            }
+        }
+        blockSize <<= 1;
+    }
+    while ((1u << b.steps) < b.mySize) {
+        b.steps++;
+    }
+    b.rankIn = b.mySize != 0 ? rank % b.mySize : 0;
+    return b;
+}
+
+// the program of one rank: (peer, isSend) in order
+std::vector<std::pair<uint32_t, bool>> HdBlocksProgram(uint32_t rank, uint32_t n, uint32_t root)
+{
+    std::vector<std::pair<uint32_t, bool>> ops;
+    const HdBlocks me = HdBlockOf(rank, n), rb = HdBlockOf(root, n);
+    auto toLower = [&] {            // :246-258, :372-393
+        if (me.lower != 0) {
+            const uint32_t times = me.mySize / me.lower;
+            if (me.rankIn % times == 0) {
+                ops.emplace_back(me.myOffset + me.mySize + me.rankIn / times, true);
+            }
+        }
+    };
+    auto toHigher = [&] {           // :261-279, :310-332
+        if (me.higher != 0) {
+            const uint32_t rounds = me.higher / me.mySize;
+            uint32_t dst = (me.myOffset - me.higher) + me.rankIn * rounds;
+            for (uint32_t i = 0; i < rounds; i++) {
+                ops.emplace_back(dst + i, true);
+            }
+        }
+    };
+    if (rank >= rb.myOffset + rb.mySize) {          // my block lies below the root's: from the larger block, on to the smaller
+        if (me.higher != 0) {
+            ops.emplace_back((me.myOffset - me.higher) + me.rankIn * (me.higher / me.mySize), false);
+        }
+        toLower();
+    } else if (rank < rb.myOffset) {                 // above: from the smaller block, on to the larger
+        if (me.lower != 0) {
+            ops.emplace_back(me.myOffset + me.mySize + me.rankIn / (me.mySize / me.lower), false);
+        }
+        toHigher();
+    } else {
+        if (me.mySize > 1) {
+            const uint32_t rootOff = root - rb.myOffset;
+            uint32_t mask = 1u << (me.steps - 1);
+            bool have = false;
+            for (uint32_t round = 1; round <= me.steps; round++, mask >>= 1) {
+                const uint32_t peer = rank ^ mask, low = (1u << (me.steps - round)) - 1;
+                if ((me.rankIn & low) == (rootOff & low) && rank != root && !have) {
+                    ops.emplace_back(peer, false);
+                    have = true;
+                    continue;
+                }
+                if (have || rank == root) {
+                    ops.emplace_back(peer, true);
+                }
+            }
+        }
+        toLower();
+        toHigher();
+    }
+    return ops;
+}
+
+}  // namespace
+
+// The transfers of the binary-block broadcast as (sender, receiver) pairs, rank by rank in program order (sends only):
+// what tests hold the route against.  Returns the number of pairs (at most cap are written).
+int orc_broadcast_hd_blocks_route(uint32_t p, uint32_t root, uint32_t *pairs, uint32_t cap)
+{
+    uint32_t n = 0;
+    for (uint32_t r = 0; r < p; r++) {
+        for (const auto &op : HdBlocksProgram(r, p, root)) {
+            if (op.second) {
+                if (n < cap) {
+                    pairs[2 * n] = r;
+                    pairs[2 * n + 1] = op.first;
+                }
+                n++;
+            }
+        }
+    }
+    return static_cast<int>(n);
+}
+
+// With a chunk loop over the CCL buffer like the other one-level broadcasts (coll_broadcast_executor.cc:83-121).
+// `touched` (optional) receives the bytes read + written by all ranks.
+int orc_broadcast_hd_blocks(uint32_t p, void **buf, uint64_t count, int dt, uint32_t root, uint64_t cclBytes, int flags,
+    int threads, uint64_t *touched)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    Machine m;
+    m.p = static_cast<int>(p);
+    m.dt = dt;
+    m.direct = (flags & 1) != 0;
+    m.pool = &pool;
+    m.buf[B_IN].resize(p);
+    m.buf[B_OUT].resize(p);
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0 && p > 1;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        for (uint32_t r = 0; r < p; r++) {
+            m.buf[B_IN][r] = static_cast<uint8_t *>(buf[r]) + offset;
+            m.buf[B_OUT][r] = static_cast<uint8_t *>(buf[r]) + offset;
+        }
+        for (uint32_t r = 0; r < p; r++) {
+            Proc pr;
+            pr.rank = r;
+            for (const auto &op : HdBlocksProgram(r, p, root)) {
+                if (op.second) {
+                    pr.prog.push_back(MkSend(static_cast<int>(op.first), 0, B_IN, 0, bytes));
+                } else {
+                    pr.prog.push_back(MkRecvCopy(static_cast<int>(op.first), 0, B_IN, 0, bytes));
+                }
+            }
+            m.procs.push_back(std::move(pr));
+        }
+        int rc = m.Run();
+        if (rc != 0) {
+            return rc;
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    if (touched != nullptr) {
+        *touched = m.bytesTouched;
+    }
+    return 0;
+}
+
 // Two-level broadcast, CollBroadcastMeshExecutor::KernelRun with several servers
 // (EXE/coll_broadcast/coll_broadcast_mesh_executor.cc:59-213) under the chunk loop of
 // CollBroadcastExecutor::RunLoop (coll_broadcast_executor.cc:83-121); `servers` groups of D = p / servers consecutive

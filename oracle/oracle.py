@@ -77,6 +77,8 @@ def lib():
                                                   i32, i32]
         L.orc_reduce_to_root_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_rhd.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
+        L.orc_broadcast_hd_blocks.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, i32, i32, ctypes.POINTER(u64)]
+        L.orc_broadcast_hd_blocks_route.argtypes = [u32, u32, ctypes.POINTER(u32), u32]
         L.orc_broadcast_mesh.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_star.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, i32, i32, ctypes.POINTER(u64)]
         L.orc_broadcast_star.restype = i32
@@ -322,6 +324,25 @@ def broadcast_star(bufs, dt, root, flags=0, threads=1, return_touched=False):
     if rc != 0:
         raise RuntimeError("oracle star broadcast failed rc=%d" % rc)
     return (bufs, touched.value) if return_touched else bufs
+
+
+def broadcast_hd_blocks(bufs, dt, root, ccl_bytes=DEFAULT_CCL_BYTES, flags=0, threads=1, return_touched=False):
+    """Binary-block halving-doubling broadcast (bcast_halvingdoubling.cc): blocks of power-of-two sizes, a binomial tree
+    inside the root's block, then block to block.  bufs are written in place."""
+    touched = ctypes.c_uint64(0)
+    rc = lib().orc_broadcast_hd_blocks(len(bufs), _ptrs(bufs), bufs[0].size, dt, root, ccl_bytes, flags, threads, ctypes.byref(touched))
+    if rc != 0:
+        raise RuntimeError("oracle binary-block broadcast failed rc=%d" % rc)
+    return (bufs, touched.value) if return_touched else bufs
+
+
+def broadcast_hd_blocks_route(p, root):
+    """[(sender, receiver), ...] of the binary-block broadcast, rank by rank in program order."""
+    cap = 4 * p + 4
+    pairs = (ctypes.c_uint32 * (2 * cap))()
+    n = lib().orc_broadcast_hd_blocks_route(p, root, pairs, cap)
+    assert 0 <= n <= cap
+    return [(pairs[2 * i], pairs[2 * i + 1]) for i in range(n)]
 
 
 def broadcast_two_level(bufs, dt, root, servers, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1,

@@ -60,6 +60,8 @@ int main(int argc, char **argv)
         base.algo = a < 3 ? ALGO_RING : a < 4 ? ALGO_MESH : a < 6 ? ALGO_MESH_ATOMIC : ALGO_RHD;
         if (base.coll == COLL_BROADCAST && Below(6) == 0) {
             base.algo = ALGO_STAR;
+        } else if (base.coll == COLL_BROADCAST && Below(5) == 0) {
+            base.algo = ALGO_HD_BLOCKS;
         }
         if (base.coll == COLL_SCATTER) {
             base.algo = Below(2) ? ALGO_MESH : ALGO_RING;

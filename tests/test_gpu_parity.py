@@ -1005,6 +1005,38 @@ def test_star_broadcast(orc):
                 g.close()
 
 
+def test_binary_block_broadcast(orc):
+    # halving-doubling over blocks of power-of-two sizes: step by step one launch per phase of the longest chain, fused
+    # one launch; rank counts with one, two and three blocks, every kind of root position
+    n = 70001
+    for p in (2, 6, 7, 8, 12, 13):
+        for fuse in (1, 0):
+            g = gh.Group(p, algo="hd_blocks", fuse=fuse, buffsize_bytes=1 << 17)
+            try:
+                for root in sorted({0, p - 1, p // 2}):
+                    print("binary-block broadcast p", p, "fuse", fuse, "root", root, flush=True)
+                    bufs_np = _ins(INT32, p, n, 197 + p + root)
+                    want, touched = orc.broadcast_hd_blocks([x.copy() for x in bufs_np], INT32, root, ccl_bytes=1 << 17,
+                                                            return_touched=True)
+                    bufs = [gh.to_dev(x) for x in bufs_np]
+                    torch.cuda.synchronize()
+                    H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, INT32, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    info = g.info()
+                    assert info["algo"] == 6 and info["fused"] == fuse, info
+                    if not fuse:
+                        assert info["bytesWritten"] == touched // 2
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(bufs[r], INT32), want[r]), ("hd blocks", p, fuse, root, r)
+                ins = _ins(FP32, p, 4099, 198 + p)          # the setting only concerns the broadcast
+                outs, _ = gh.all_reduce(g, ins, FP32, SUM)
+                want = orc.allreduce(ins, FP32, SUM, ccl_bytes=1 << 17)
+                for r in range(p):
+                    assert np.array_equal(outs[r], want[r]), ("ring under hd blocks", p, fuse, r)
+            finally:
+                g.close()
+
+
 def test_allreduce_at_the_rank_limit(orc):
     # 64 ranks is the most a group holds: ring / uncut mesh = chains of 64 sources (the fused kernel's limit),
     # halving-doubling at 48 ranks = 32 leaves of which 16 are folded pairs, at 64 ranks = 32 leaves of two

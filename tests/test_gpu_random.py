@@ -276,13 +276,13 @@ def test_random_alltoallv_flat_and_staged(orc, seed):
 
 @pytest.mark.parametrize("seed", range(3))
 def test_random_scatter_and_broadcast_over_rank_groups(orc, seed):
-    """Scatter and broadcast with random roots, rank groups and schedule settings (auto, ring, star): whatever the route,
+    """Scatter and broadcast with random roots, rank groups and schedule settings (auto, ring, star, ...): whatever the route,
     rank r ends with the root's block r / with the root's buffer, the root's input stays as it was."""
     rng = np.random.default_rng(5300 + SEED_SHIFT + seed)
     for case in range(8):
         p = int(rng.choice([2, 3, 4, 6, 8, 12, 16]))
         servers = int(rng.choice([s for s in range(1, p + 1) if p % s == 0]))
-        setting = str(rng.choice(["auto", "ring", "star", "mesh", "rhd"]))
+        setting = str(rng.choice(["auto", "ring", "star", "mesh", "rhd", "hd_blocks"]))
         dt = int(rng.choice(ALL_TYPES))
         n = _size(rng) // 4 + 1
         fuse = int(rng.integers(0, 2))

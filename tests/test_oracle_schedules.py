@@ -700,6 +700,51 @@ def test_star_broadcast_delivers_and_every_byte_comes_from_the_root(orc):
                 assert touched == 2 * (p - 1) * n * orc.dtype_size(dt)
 
 
+# Routes of the binary-block broadcast worked out by hand from bcast_halvingdoubling.cc (block parameters :26-62, the
+# binomial tree of the root's block :165-228, block to block :231-396), as (sender, receiver), senders in rank order,
+# each sender's transfers in the order it issues them.
+HD_BLOCK_ROUTES = {
+    (6, 5): [(4, 0), (4, 1), (5, 4), (5, 2), (5, 3)],                                         # blocks 4 + 2, root in the small one
+    (7, 0): [(0, 2), (0, 1), (0, 4), (2, 3), (2, 5), (4, 6)],                                 # blocks 4 + 2 + 1, downwards twice
+    (7, 4): [(4, 5), (4, 6), (4, 0), (4, 1), (5, 2), (5, 3)],                                 # the root's block serves both sides
+    (7, 6): [(4, 0), (4, 1), (5, 2), (5, 3), (6, 4), (6, 5)],                                 # upwards twice
+    (12, 3): [(0, 8), (1, 0), (2, 9), (3, 7), (3, 1), (3, 2), (4, 10), (5, 4), (6, 11), (7, 5), (7, 6)],
+    (8, 5): [(1, 3), (1, 0), (3, 2), (5, 1), (5, 7), (5, 4), (7, 6)],                         # a power of two: one block, a tree
+    (2, 1): [(1, 0)],
+    (3, 1): [(0, 2), (1, 0)],
+}
+
+
+def test_binary_block_broadcast_routes_and_bytes(orc):
+    # the hand-derived routes; the definition; every rank but the root receives exactly once (p - 1 transfers of the
+    # whole buffer, so 2 (p - 1) n bytes touched), also under a chunk loop
+    for (p, root), want in HD_BLOCK_ROUTES.items():
+        assert orc.broadcast_hd_blocks_route(p, root) == want, (p, root)
+    for p in list(range(1, 18)) + [24, 31, 33]:
+        for root in sorted({0, p - 1, p // 2, p // 3}):
+            route = orc.broadcast_hd_blocks_route(p, root)
+            assert sorted(d for _, d in route) == [r for r in range(p) if r != root], (p, root)
+            for dt, n, ccl in ((INT32, 1, 200 << 20), (INT8, 100003, 200 << 20), (INT64, 5000, 4096)):
+                bufs = _inputs(dt, p, n, root + n)
+                src = bufs[root].copy()
+                bufs, touched = orc.broadcast_hd_blocks(bufs, dt, root, ccl_bytes=ccl, return_touched=True)
+                assert all(np.array_equal(b, src) for b in bufs), (p, dt, n, root)
+                assert touched == 2 * (p - 1) * n * orc.dtype_size(dt), (p, dt, n, root)
+    # for a power of two it is the binomial tree of the recursive halving-doubling broadcast: same transfers
+    for p in (2, 4, 8, 16):
+        for root in range(p):
+            route = orc.broadcast_hd_blocks_route(p, root)
+            have = {root}
+            mask = p >> 1
+            tree = set()
+            while mask:
+                for q in sorted(have):
+                    tree.add((q, q ^ mask))
+                have |= {q ^ mask for q in have}
+                mask >>= 1
+            assert set(route) == tree, (p, root)
+
+
 @pytest.mark.parametrize("shape", [(2, 4), (4, 2), (3, 2), (3, 4), (1, 4), (8, 1), (5, 3)])
 def test_two_level_broadcast_delivers_and_moves_the_closed_form_bytes(orc, shape):
     # Definition: every rank ends with the root's bytes.  Structure: the bytes received over all ranks are those of

@@ -848,6 +848,38 @@ def test_star_broadcast_plan(orc, p):
                 assert np.array_equal(mem[r].view(np.int32), want[r]), (p, root, fused, r)
 
 
+def test_binary_block_broadcast_plan(orc):
+    # the plan's transfers are the hand-derived routes, a rank's transfers in consecutive phases from the one after it
+    # received; results and bytes as the checker's, step by step and fused, also under a chunk loop
+    from test_oracle_schedules import HD_BLOCK_ROUTES
+    n = 1003
+    for (p, root), want in HD_BLOCK_ROUTES.items():
+        plan = H.describe_plan(H.COLL_BROADCAST, root | (6 << 16), p, n, INT32, in_place_mask=(1 << p) - 1)
+        got = sorted((st["a"][0], k, st["dst"][0]) for k, ph in enumerate(plan["phases"]) for st in ph)
+        assert [(a, d) for a, _, d in got] == want, (p, root, got)
+        got_at = {d: k for _, k, d in got}
+        for a in range(p):
+            mine = [k for s, k, _ in got if s == a]
+            first = 0 if a == root else got_at[a] + 1
+            assert mine == list(range(first, first + len(mine))), (p, root, a, mine)
+        assert all(st["n"] == n * 4 for ph in plan["phases"] for st in ph)
+    phases = {(7, 4): 4, (7, 6): 4, (6, 5): 3, (12, 3): 4, (8, 5): 3}      # the longest chain of each worked example
+    for (p, root), k in phases.items():
+        assert len(H.describe_plan(H.COLL_BROADCAST, root | (6 << 16), p, n, INT32)["phases"]) == k, (p, root)
+    for p in (1, 2, 3, 5, 6, 7, 8, 11, 12, 13, 24, 33):
+        for root in sorted({0, p - 1, p // 2}):
+            for ccl in (200 << 20, 1024):
+                bufs = _ins(INT32, p, n, 180 + p)
+                want, touched = orc.broadcast_hd_blocks([b.copy() for b in bufs], INT32, root, ccl_bytes=ccl, return_touched=True)
+                plan = H.describe_plan(H.COLL_BROADCAST, root | (6 << 16), p, n, INT32, ccl_bytes=ccl, in_place_mask=(1 << p) - 1)
+                assert plan["stepWritten"] == touched // 2
+                for fused in (False, True):
+                    mem = _bytes(bufs)
+                    (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, mem, mem, INT32, 0, in_place=True)
+                    for r in range(p):
+                        assert np.array_equal(mem[r].view(np.int32), want[r]), (p, root, ccl, fused, r)
+
+
 @pytest.mark.parametrize("servers,D", [(2, 4), (4, 2), (3, 4), (5, 3), (6, 1), (2, 8)])
 def test_two_level_broadcast_plan(orc, servers, D):
     # scatter inside the root's group, halving-doubling between the groups, all-gather inside every group:
