@@ -1551,10 +1551,11 @@ HcclResult HcclAmdSetParam(HcclComm comm, const char *key, const char *value)
         }
         cfg.cacheEntries = uint32_t(n);
     } else if (k == "nic_ranks") {
-        // the ranks of an 8-rank ring that own a network port: "all", or a comma-separated list of 1, 2 or 4 ranks
+        // the ranks of an 8-rank ring (the devices of every server of 8) that own a network port: "all", or a
+        // comma-separated list of 1, 2 or 4 of them
         uint32_t mask = 0;
         if (v != "all" && !v.empty()) {
-            if (c->group->p != 8) {
+            if (c->group->p % 8 != 0) {
                 return HCCL_E_PARA;
             }
             std::stringstream in(v);
@@ -1726,6 +1727,9 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         rq.servers = std::max(1u, (uint32_t(algo) >> 8) & 0xffu);
         rq.meshAtomic = ((uint32_t(algo) >> 16) & 1u) != 0;
         rq.level0Rings = (uint32_t(algo) >> 17) & 7u;
+        if (coll == COLL_REDUCESCATTER) {
+            rq.nicMask = (uint32_t(algo) >> 20) & 0xffu;      // bits 20..27: devices of every server with a network port
+        }
     } else if (coll == COLL_ALLTOALLV) {
         // all-to-all-v: bits 8..15 = number of servers of the staged schedule (0 or 1 = flat pairwise)
         rq.algo = ALGO_PAIRWISE;

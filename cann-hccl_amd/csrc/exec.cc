@@ -976,6 +976,11 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAl
         rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
         rq.meshAtomic = rq.level0Rings == 0 && !g->cfg.deterministic && g->ctx->sig.dtype != HCCL_DATA_TYPE_INT64 &&
             g->ctx->sig.op != HCCL_REDUCE_PROD;
+        if (rq.level0Rings == 4 && rq.algo == ALGO_RING) {
+            // servers of 8 devices some of which have no network port (:150-170, 264-300); the branch only holds
+            // together with the ring between the servers, so the halving-doubling schedule ignores the ports
+            rq.nicMask = g->cfg.nicMask;
+        }
     }
     if (rq.coll == COLL_ALLGATHER && !g->ctx->sig.variable && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
         // two levels (coll_all_gather_mesh_executor.cc:71-175, coll_all_gather_ring_executor.cc:81-200): inside a

@@ -530,6 +530,111 @@ void TwoLevelReduceScatterChunk(VProgram &vp, Algo level1, uint32_t p, uint32_t 
     }
 }
 
+// Two-level ring reduce-scatter of one chunk when only some of a server's 8 devices have a network port: the isMultiNic
+// branch of CollReduceScatterRingExecutor::KernelRun (coll_reduce_scatter_ring_executor.cc:150-170, 264-300), ring
+// between the servers.  Block i of the input lies at blockOff[i]; the reference works on a staged copy in which the
+// blocks follow each other, so a range of that copy is taken block by block here.
+//   1. all-reduce of the whole input inside every server over the four rings (MultiRingAllReduce, coll_comm_executor.cc:
+//      44-170): the p blocks together are cut into 8 slices (PrepareSliceData) and every slice into one part per ring;
+//      the reference gathers on its scratch buffer and copies back (:160-168), here the parts go round on the input
+//   2. the devices with a port reduce-scatter the whole input among the same devices of all servers (:172-191)
+//   3. the port devices hand the blocks of their server's slice on, part k of a block along ring k
+//      (MultiRingMultiRootScatter, coll_comm_executor.cc:1312-1415; multi_root_scatter_ring.cc:299-345): with n ports
+//      a ring's 8 parts form n runs of 8 / n, run j leaves the ring position of the j-th port (positions ascending),
+//      and part i of the order rotated by the first port's position stops at position (i + that position) % 8
+//   4. the rank's own block goes to the output (:298-299)
+void PrunedTwoLevelReduceScatterChunk(VProgram &vp, uint32_t p, uint32_t servers, uint32_t nicMask,
+    const std::vector<uint64_t> &blockOff, uint64_t bytes, uint64_t outOff, uint64_t align)
+{
+    const uint32_t D = 8, rings = 4;
+    VProgram flat;       // step 1 on the staged layout: offsets count through the blocks
+    std::vector<Slice> sl = RingSlicePlan(bytes * p, D, align);
+    for (uint32_t s = 0; s < servers; s++) {
+        flat.rankMap.resize(D);
+        for (uint32_t k = 0; k < rings; k++) {
+            std::vector<Slice> part(D);
+            for (uint32_t i = 0; i < D; i++) {
+                const uint32_t dev = kRingOrders8[k][i];
+                flat.rankMap[i] = s * D + dev;
+                std::vector<Slice> cut = RingSlicePlan(sl[dev].size, rings, align);
+                part[i] = Slice{sl[dev].off + cut[k].off, cut[k].size};
+            }
+            RingReduceScatterPhases(flat, 0, D, 0, part, BUF_SEND, 0, part);
+            for (uint32_t h = 0; h + 1 < D; h++) {
+                for (uint32_t r = 0; r < D; r++) {
+                    const uint32_t i = Mod(int64_t(r) - 1 - h, D), left = Mod(int64_t(r) - 1, D);
+                    EmitCopy(flat, D - 1 + h, MkRef(r, BUF_SEND, part[i].off), MkRef(left, BUF_SEND, part[i].off), part[i].size);
+                }
+            }
+        }
+    }
+    for (size_t ph = 0; ph < flat.phases.size(); ph++) {
+        for (const Step &st : flat.phases[ph].steps) {
+            uint64_t at = st.a.off, left = st.bytes;
+            while (left > 0) {
+                const uint64_t block = at / bytes, within = at % bytes, n = std::min(left, bytes - within);
+                Step piece = st;
+                piece.dst.off = piece.a.off = blockOff[block] + within;
+                if (st.reduce) {
+                    piece.b.off = piece.a.off;
+                }
+                Emit(vp, ph, piece.reduce, piece.dst, piece.a, piece.b, n);
+                at += n;
+                left -= n;
+            }
+        }
+    }
+    const size_t l1 = flat.phases.size();
+    std::vector<uint32_t> nic;
+    for (uint32_t d = 0; d < D; d++) {
+        if ((nicMask >> d) & 1u) {
+            nic.push_back(d);
+        }
+    }
+    for (uint32_t d : nic) {
+        vp.rankMap.resize(servers);
+        for (uint32_t s = 0; s < servers; s++) {
+            vp.rankMap[s] = s * D + d;
+        }
+        vp.phaseBase = l1;
+        for (uint32_t k = 0; k < D && servers > 1; k++) {
+            std::vector<Slice> in(servers);
+            for (uint32_t s = 0; s < servers; s++) {
+                in[s] = Slice{blockOff[s * D + k], bytes};
+            }
+            RingReduceScatterPhases(vp, 0, servers, 0, in, BUF_SEND, 0, in);
+        }
+    }
+    vp.rankMap.clear();
+    vp.phaseBase = 0;
+    const size_t l2 = l1 + (servers - 1);
+    const uint32_t run = D / uint32_t(nic.size());
+    std::vector<Slice> cut = RingSlicePlan(bytes, rings, align);
+    size_t l3 = l2;
+    for (uint32_t s = 0; s < servers; s++) {
+        for (uint32_t k = 0; k < rings; k++) {
+            std::vector<uint32_t> portAt;       // ring positions of the port devices
+            for (uint32_t i = 0; i < D; i++) {
+                if ((nicMask >> kRingOrders8[k][i]) & 1u) {
+                    portAt.push_back(i);
+                }
+            }
+            for (uint32_t j = 0; j < D; j++) {
+                const uint32_t from = portAt[j / run], to = (j + portAt[0]) % D, hops = (to + D - from) % D;
+                const uint64_t off = blockOff[s * D + kRingOrders8[k][to]] + cut[k].off;
+                for (uint32_t h = 0; h < hops; h++) {
+                    EmitCopy(vp, l2 + h, MkRef(s * D + kRingOrders8[k][(from + h + 1) % D], BUF_SEND, off),
+                        MkRef(s * D + kRingOrders8[k][(from + h) % D], BUF_SEND, off), cut[k].size);
+                }
+                l3 = std::max(l3, l2 + hops);
+            }
+        }
+    }
+    for (uint32_t r = 0; r < p; r++) {
+        EmitCopy(vp, l3, MkRef(r, BUF_RECV, outOff), MkRef(r, BUF_SEND, blockOff[r]), bytes);
+    }
+}
+
 // Standalone recursive halving-doubling all-gather (all_gather_recursive_hd.cc:26-238) on the output
 // buffer; phase0 is the first phase after the ranks copied their own block in.
 void RhdAllGatherChunk(VProgram &vp, size_t phase0, uint32_t p, const std::vector<Slice> &sl)
@@ -1289,8 +1394,12 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                 for (uint32_t i = 0; i < p; i++) {
                     blockOff[i] = in[i].off;
                 }
-                TwoLevelReduceScatterChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, rq.level0Rings, blockOff,
-                    bytes, done, rq.align, rq.meshAtomic);
+                if (rq.nicMask != 0 && (rq.nicMask & 0xffu) != 0xffu) {
+                    PrunedTwoLevelReduceScatterChunk(*vp, p, rq.servers, rq.nicMask, blockOff, bytes, done, rq.align);
+                } else {
+                    TwoLevelReduceScatterChunk(*vp, rq.algo == ALGO_RING ? ALGO_RING : ALGO_RHD, p, rq.servers, rq.level0Rings,
+                        blockOff, bytes, done, rq.align, rq.meshAtomic);
+                }
             } else if (rq.algo == ALGO_RING) {
                 RingReduceScatterPhases(*vp, 0, p, 0, in, BUF_RECV, 0, out);
             } else if (rq.algo == ALGO_RHD) {
@@ -2266,8 +2375,11 @@ int BuildPlan(const PlanRequest &request, Plan *plan, std::string *err)
     }
     if (request.nicMask != 0) {
         const int ports = __builtin_popcount(request.nicMask & 0xffu);
-        if (request.p != 8 || (request.nicMask >> 8) != 0 || (ports != 1 && ports != 2 && ports != 4 && ports != 8)) {
-            *err = "bad plan request: network ports are given for a ring of 8 ranks, 1, 2, 4 or 8 of them";
+        const bool twoLevel = request.coll == COLL_REDUCESCATTER && request.servers > 1 && request.p == request.servers * 8 &&
+            request.level0Rings == 4 && request.algo == ALGO_RING && request.vCounts.empty();
+        if ((request.p != 8 && !twoLevel) || (request.nicMask >> 8) != 0 || (ports != 1 && ports != 2 && ports != 4 && ports != 8)) {
+            *err = "bad plan request: network ports are given for a ring of 8 ranks, or for a two-level reduce-scatter over "
+                   "servers of 8 ranks with four rings inside and the ring between them; 1, 2, 4 or 8 of them";
             return 1;
         }
     }

@@ -150,7 +150,10 @@ struct PlanRequest {
     uint32_t nicMask = 0;          // one-level ring all-reduce over 8 ranks: bit r set = rank r has a network port.  With 1, 2
                                    // or 4 ports the reduce-scatter runs the port-pruned form (reduce_scatter_ring.cc:160-168,
                                    // 299-477): the slices of chunk j all end their ring chain at the j-th port rank.  0 or all
-                                   // 8 bits: the plain ring
+                                   // 8 bits: the plain ring.  Two-level reduce-scatter over servers of 8 ranks (four rings
+                                   // inside, ring between): bit d = device d of every server has a port; with 1, 2 or 4 ports
+                                   // the servers all-reduce first, the port devices run the ring between the servers and
+                                   // scatter the result inside (coll_reduce_scatter_ring_executor.cc:150-170, 264-300)
     bool meshAtomic = false;       // mesh reduce phases without the piece cut (the reference's non-deterministic variant)
     bool stageInput = false;       // copy the send buffers to scratch first (used when buffers overlap)
     // all-to-all-v only: p x p tables in elements, row r = what rank r passed

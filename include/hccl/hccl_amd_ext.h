@@ -41,7 +41,12 @@ extern "C" {
  *                                With fewer than 8 the one-level ring all-reduce runs the port-pruned reduce-scatter of the
  *                                reference (the 8 slices form as many chunks as there are ports; all slices of chunk j end
  *                                their ring chain at the j-th listed rank, in ascending rank order), which changes the
- *                                floating-point association of the slices whose chain ends elsewhere
+ *                                floating-point association of the slices whose chain ends elsewhere.  With several
+ *                                groups of 8 ("servers" = ranks / 8, "level0" = "ring4", "algo" = "ring") the list names
+ *                                devices of every group, and the reduce-scatter runs the reference's branch for servers
+ *                                with fewer ports than devices: all-reduce inside every group, ring reduce-scatter
+ *                                between the groups on the listed devices only, then these hand the blocks on inside
+ *                                their group; sums are associated inside a group first, then between the groups
  *   "step_stores"   "auto" | "nt" | "ordinary"   store kind of the step-by-step kernels (non-temporal, or write-back
  *                                so that the next phase finds the data in the memory-side cache); "auto" decides per collective
  *   "step_sweep"    "alternate" | "forward"   step-by-step kernels: every other launch walks its data backwards (default),
@@ -105,7 +110,8 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
  * carry the number of rank groups of the two-level schedule (0 or 1: one level), bit 16 asks for its mesh level
  * without the piece cut, bits 17..19 give the rings inside a group (0: mesh, 1, or 4) and bits 20..27 the ranks of an
  * 8-rank ring that own a network port (bit 20 + r for rank r; 0: all of them); the reduce-scatter (coll 1)
- * and the all-gather (coll 2) take bits 8..19 the same way; for the all-to-all-v (coll 3) bits 8..15 give the number
+ * and the all-gather (coll 2) take bits 8..19 the same way, the reduce-scatter over rank groups of 8 with four rings inside
+ * and the ring between them also bits 20..27 (bit 20 + d: device d of every group has a port); for the all-to-all-v (coll 3) bits 8..15 give the number
  * of servers of the staged schedule.  inPlaceMask bit r:
  * rank r's send and receive buffer are the same.  For all-to-all-v, tables points to 4*p*p uint64
  * (sendCounts, sdispls, recvCounts, rdispls, each p x p row-major, row = rank); for the variable-count

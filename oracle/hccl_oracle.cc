@@ -1665,6 +1665,256 @@ int orc_reducescatter_two_level(int level1, int level0, uint32_t servers, uint32
     return 0;
 }
 
+// Send lists of the multi-root ring scatter, MultiRootScatterRing::MultiRootScatterSlicesPrep
+// (TPL/temp_scatter/multi_root_scatter_ring.cc:299-345): slice j leaves the ring position of port j / chunk and stops at
+// position (j + first port position) % 8; a position forwards the slices that pass through it, the farthest first.
+std::vector<std::vector<uint32_t>> MultiRootScatterLists(const std::vector<uint32_t> &nicPos)
+{
+    const uint32_t n = 8, chunk = n / static_cast<uint32_t>(nicPos.size());
+    struct Range {
+        uint32_t slice, start, end;
+    };
+    std::vector<Range> ranges;
+    for (uint32_t i = 0; i < nicPos.size(); i++) {
+        for (uint32_t c = 0; c < chunk; c++) {
+            Range g{i * chunk + c, nicPos[i], (i * chunk + c + nicPos[0]) % n};
+            if (g.end < g.start) {
+                g.end += n;
+            }
+            ranges.push_back(g);
+        }
+    }
+    std::vector<std::vector<uint32_t>> lists;
+    for (uint32_t pos = 0; pos < n; pos++) {
+        std::vector<std::pair<uint32_t, uint32_t>> mine;     // (hops still to go, slice)
+        for (size_t i = ranges.size(); i-- > 0;) {
+            const Range &g = ranges[i];
+            const uint32_t at = pos >= g.start ? pos : pos + n;
+            if (at < g.end) {
+                mine.emplace_back(g.end - at, g.slice);
+            }
+        }
+        std::sort(mine.begin(), mine.end(), [](const std::pair<uint32_t, uint32_t> &a, const std::pair<uint32_t, uint32_t> &b) {
+            return a.first > b.first;
+        });
+        std::vector<uint32_t> one;
+        for (const auto &e : mine) {
+            one.push_back(e.second);
+        }
+        lists.push_back(one);
+    }
+    return lists;
+}
+
+// Per-position program of MultiRootScatterRing::RunMultiRootScatterChunk (multi_root_scatter_ring.cc:100-140) with
+// HeadScatterChunk (:142-205), MidScatterChunk (:207-246) and TailScatterChunk (:248-297); the data lies in buffer b at
+// base + slice offset on both sides of a transfer.
+void ProgMultiRootScatter(std::vector<Action> &pg, uint32_t pos, const std::vector<uint32_t> &nicPos,
+    const std::vector<std::vector<uint32_t>> &lists, int b, uint64_t base, const std::vector<Slice> &sl)
+{
+    const uint32_t n = 8, left = (pos + n - 1) % n, right = (pos + 1) % n;
+    const std::vector<uint32_t> &mine = lists[pos], &prev = lists[left];
+    auto inPrev = [&](uint32_t s) { return std::find(prev.begin(), prev.end(), s) != prev.end(); };
+    auto send = [&](uint32_t s) { pg.push_back(MkSend(static_cast<int>(right), 0, b, base + sl[s].off, sl[s].size)); };
+    auto recv = [&](uint32_t s) { pg.push_back(MkRecvCopy(static_cast<int>(left), 0, b, base + sl[s].off, sl[s].size)); };
+    const uint32_t own = (pos + n - nicPos[0]) % n;          // the slice this position keeps
+    const uint32_t len = static_cast<uint32_t>(mine.size());
+    auto mid = [&](uint32_t idx) {
+        send(mine[idx]);
+        if (inPrev(mine[idx + 1])) {
+            recv(mine[idx + 1]);
+        }
+    };
+    if (len == 0) {
+        if (inPrev(own)) {
+            recv(own);
+        }
+        return;
+    }
+    // head
+    bool headDone = false;
+    if (inPrev(mine[0])) {
+        recv(mine[0]);
+    }
+    if (len >= 2) {
+        if (inPrev(mine[1])) {
+            mid(0);
+            headDone = true;
+        }
+    } else if (inPrev(mine[0])) {       // the only slice: head and tail at once
+        send(mine[0]);
+        recv(own);
+        headDone = true;
+    }
+    if (!headDone) {
+        send(mine[0]);
+    }
+    for (uint32_t idx = 1; idx + 1 < len; idx++) {
+        mid(idx);
+    }
+    if (len >= 2) {                     // tail
+        send(mine[len - 1]);
+        if (inPrev(own)) {
+            recv(own);
+        }
+    }
+}
+
+// Two-level ring reduce-scatter over servers of 8 devices of which only some have a network port: the isMultiNic
+// branch of CollReduceScatterRingExecutor::KernelRun (EXE/coll_reduce_scatter/coll_reduce_scatter_ring_executor.cc:
+// 150-170, 264-300) with the ring between the servers.  Per chunk of the loop:
+//   1. all-reduce of the whole staged input inside every server over the four rings of the 8-device topology
+//      (MultiRingAllReduce, EXE/coll_comm_executor.cc:44-170; slices PrepareSliceData over the whole input, then one
+//      part per ring), into the scratch buffer and back to the input buffer (:160-168)
+//   2. the devices with a port reduce-scatter the whole input among the same devices of all servers (:172-191);
+//      the others skip this step
+//   3. input buffer -> scratch (:288-291), then the port devices hand the blocks of the server's slice to the devices
+//      they belong to, part k of every block along ring k (MultiRingMultiRootScatter, EXE/coll_comm_executor.cc:
+//      1312-1415 with the slices of ReduceScatterRingSlicePrepare rotated by the first port's ring position, :264-273)
+//   4. the device's own block of the scratch buffer goes to the output (:298-299, :343-345)
+// nic: device numbers 0..7 with a port, ascending; 1, 2 or 4 of them.
+int orc_reducescatter_two_level_pruned(uint32_t servers, uint32_t p, void **in, void **out, uint64_t recvCount, int dt, int op,
+    const uint32_t *nic, uint32_t nNic, uint64_t cclBytes, uint64_t align, int flags, int threads)
+{
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || servers == 0 || p != servers * 8 || (nNic != 1 && nNic != 2 && nNic != 4)) {
+        return -20;
+    }
+    for (uint32_t i = 0; i < nNic; i++) {
+        if (nic[i] > 7 || (i > 0 && nic[i] <= nic[i - 1])) {
+            return -20;
+        }
+    }
+    const uint32_t D = 8, ringCount = 4;
+    uint64_t maxPer = cclBytes / (uint64_t(p) * unit);
+    if (maxPer == 0) {
+        return -21;
+    }
+    Pool pool(threads);
+    auto machine = [&](uint32_t n) {
+        Machine m;
+        m.p = static_cast<int>(n);
+        m.dt = dt;
+        m.op = op;
+        m.direct = (flags & 1) != 0;
+        m.pool = &pool;
+        m.buf[B_IN].resize(n);
+        m.buf[B_OUT].resize(n);
+        return m;
+    };
+    Machine all = machine(p);          // B_IN: the staged input, B_OUT: the scratch buffer of the same size
+    uint64_t stage = std::min<uint64_t>(recvCount, maxPer) * unit;
+    std::vector<std::vector<uint8_t>> cclIn(p, std::vector<uint8_t>(stage * p)), scratch(p, std::vector<uint8_t>(stage * p));
+    for (uint32_t r = 0; r < p; r++) {
+        all.buf[B_IN][r] = cclIn[r].data();
+        all.buf[B_OUT][r] = scratch[r].data();
+    }
+    uint64_t offset = 0;
+    for (uint64_t left = recvCount; left > 0;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit, whole = bytes * p;
+        for (uint32_t r = 0; r < p; r++) {
+            for (uint32_t i = 0; i < p; i++) {
+                all.Copy(all.buf[B_IN][r] + bytes * i, static_cast<uint8_t *>(in[r]) + recvCount * unit * i + offset, bytes);
+            }
+        }
+        // 1. all-reduce inside every server
+        std::vector<std::vector<Slice>> segs = MultiSegSlices(RingSlices(whole, D, align), ringCount, align);
+        for (uint32_t s = 0; s < servers; s++) {
+            for (uint32_t k = 0; k < ringCount; k++) {
+                Machine ring = machine(D);
+                std::vector<Slice> ringSl(D);
+                for (uint32_t i = 0; i < D; i++) {
+                    const uint32_t dev = kEightDeviceRings[k][i];
+                    ring.buf[B_IN][i] = all.buf[B_IN][s * D + dev];
+                    ring.buf[B_OUT][i] = all.buf[B_OUT][s * D + dev];
+                    ringSl[i] = segs[dev][k];
+                }
+                for (uint32_t i = 0; i < D; i++) {
+                    Proc pr;
+                    pr.rank = i;
+                    ProgReduceScatterRing(pr.prog, i, D, B_IN, B_IN, ringSl, ringSl);
+                    ProgAllGatherRing(pr.prog, i, D, B_IN, B_OUT, ringSl, ringSl);
+                    ring.procs.push_back(std::move(pr));
+                }
+                int rc = ring.Run();
+                if (rc != 0) {
+                    return rc;
+                }
+            }
+            for (uint32_t d = 0; d < D; d++) {
+                all.Copy(all.buf[B_IN][s * D + d], all.buf[B_OUT][s * D + d], whole);
+            }
+        }
+        // 2. between the servers, port devices only
+        const uint64_t serverSlice = bytes * D;
+        for (uint32_t i = 0; i < nNic && servers > 1; i++) {
+            Machine m = machine(servers);
+            std::vector<Slice> sl(servers);
+            for (uint32_t s = 0; s < servers; s++) {
+                m.buf[B_IN][s] = all.buf[B_IN][s * D + nic[i]];
+                m.buf[B_OUT][s] = all.buf[B_OUT][s * D + nic[i]];
+                sl[s] = Slice{serverSlice * s, serverSlice};
+            }
+            for (uint32_t s = 0; s < servers; s++) {
+                Proc pr;
+                pr.rank = s;
+                ProgReduceScatterRing(pr.prog, s, servers, B_IN, B_IN, sl, sl);
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+        }
+        // 3. scatter inside every server from the port devices
+        std::vector<Slice> blocks(D);
+        for (uint32_t d = 0; d < D; d++) {
+            blocks[d] = Slice{bytes * d, bytes};
+        }
+        std::vector<std::vector<Slice>> parts = MultiSegSlices(blocks, ringCount, align);
+        for (uint32_t s = 0; s < servers; s++) {
+            for (uint32_t d = 0; d < D; d++) {
+                all.Copy(all.buf[B_OUT][s * D + d], all.buf[B_IN][s * D + d], whole);
+            }
+            for (uint32_t k = 0; k < ringCount; k++) {
+                std::vector<uint32_t> nicPos;
+                for (uint32_t i = 0; i < D; i++) {
+                    if (std::find(nic, nic + nNic, kEightDeviceRings[k][i]) != nic + nNic) {
+                        nicPos.push_back(i);
+                    }
+                }
+                Machine ring = machine(D);
+                std::vector<Slice> ringSl(D);
+                for (uint32_t i = 0; i < D; i++) {
+                    const uint32_t dev = kEightDeviceRings[k][i];
+                    ring.buf[B_IN][i] = all.buf[B_IN][s * D + dev];
+                    ring.buf[B_OUT][i] = all.buf[B_OUT][s * D + dev];
+                    ringSl[i] = parts[kEightDeviceRings[k][(i + nicPos[0]) % D]][k];      // rotated by the first port
+                }
+                std::vector<std::vector<uint32_t>> lists = MultiRootScatterLists(nicPos);
+                for (uint32_t i = 0; i < D; i++) {
+                    Proc pr;
+                    pr.rank = i;
+                    ProgMultiRootScatter(pr.prog, i, nicPos, lists, B_OUT, serverSlice * s, ringSl);
+                    ring.procs.push_back(std::move(pr));
+                }
+                int rc = ring.Run();
+                if (rc != 0) {
+                    return rc;
+                }
+            }
+        }
+        // 4. the own block
+        for (uint32_t r = 0; r < p; r++) {
+            all.Copy(static_cast<uint8_t *>(out[r]) + offset, all.buf[B_OUT][r] + bytes * r, bytes);
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    return 0;
+}
+
 // in[r]: sendCount elements, out[r]: p * sendCount elements.
 int orc_allgather(int algo, uint32_t p, void **in, void **out, uint64_t sendCount, int dt,
     uint64_t cclBytes, uint64_t align, int flags, int threads)

@@ -75,6 +75,8 @@ def lib():
                                               i32, i32]
         L.orc_reducescatter_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, u64, u64,
                                                   i32, i32]
+        L.orc_reducescatter_two_level_pruned.argtypes = [u32, u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32,
+                                                         ctypes.POINTER(u32), u32, u64, u64, i32, i32]
         L.orc_reduce_to_root_two_level.argtypes = [i32, i32, u32, u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_rhd.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32]
         L.orc_broadcast_hd_blocks.argtypes = [u32, ctypes.POINTER(vp), u64, i32, u32, u64, i32, i32, ctypes.POINTER(u64)]
@@ -256,6 +258,22 @@ def reducescatter_two_level(ins, dt, op, servers, level1=RING, atomic=False, ccl
                                            ccl_bytes, align, flags, threads)
     if rc != 0:
         raise RuntimeError("oracle two-level reducescatter failed rc=%d" % rc)
+    return outs
+
+
+def reducescatter_two_level_pruned(ins, dt, op, servers, nic, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1):
+    """Two-level ring reduce-scatter over servers of 8 devices of which only the devices in `nic` have a network port
+    (the isMultiNic branch of coll_reduce_scatter_ring_executor.cc): all-reduce inside the servers, ring between the
+    servers on the port devices, scatter inside the servers."""
+    p = len(ins)
+    n = ins[0].size // p
+    outs = [np.empty(n, dtype=ins[0].dtype) for _ in range(p)]
+    nic = sorted(nic)
+    arr = (ctypes.c_uint32 * len(nic))(*nic)
+    rc = lib().orc_reducescatter_two_level_pruned(servers, p, _ptrs(ins), _ptrs(outs), n, dt, op, arr, len(nic),
+                                                  ccl_bytes, align, flags, threads)
+    if rc != 0:
+        raise RuntimeError("oracle port-pruned two-level reducescatter failed rc=%d" % rc)
     return outs
 
 

@@ -92,6 +92,10 @@ int main(int argc, char **argv)
             const uint32_t masks[] = {0x01, 0x80, 0x11, 0x22, 0x0f, 0x55, 0xaa, 0x04};
             base.nicMask = masks[Below(8)];
         }
+        if (base.coll == COLL_REDUCESCATTER && base.algo == ALGO_RING && base.servers > 1 && base.level0Rings == 4 && Below(2) == 0) {
+            const uint32_t masks[] = {0x01, 0x80, 0x11, 0x22, 0x0f, 0x55, 0xaa, 0x04};
+            base.nicMask = masks[Below(8)];       // servers whose devices do not all have a network port
+        }
         const uint32_t units[] = {1, 2, 4, 8};
         base.unit = units[Below(4)];
         const uint64_t ccls[] = {1ull << 20, 16ull << 20, 200ull << 20};

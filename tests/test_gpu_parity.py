@@ -1697,6 +1697,55 @@ def test_ring_allreduce_with_fewer_network_ports_than_ranks(orc):
             g.close()
 
 
+def test_two_level_reducescatter_with_fewer_network_ports_than_devices(orc):
+    # servers of 8 devices, four rings inside, ring between them, ports on some devices only: the executor's branch that
+    # all-reduces inside a server first (coll_reduce_scatter_ring_executor.cc:150-170, 264-300).  Fused and step by step
+    # against the checker on order-sensitive data, the hand-derived answers, and back to the ordinary branch.
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_two_level_pruned_fp32.json")) as f:
+        kat = json.load(f)
+    for servers in (2, 3):
+        p = 8 * servers
+        for fuse in (1, 0):
+            g = gh.Group(p, algo="ring", servers=servers, level0="ring4", fuse=fuse)
+            try:
+                for nic in ([0, 4], [3], [1, 2, 3, 7]):
+                    g.set(nic_ranks=",".join(str(r) for r in nic))
+                    for dt, op, n in ((FP32, SUM, 10007), (BF16, SUM, 4001), (INT32, MAX, 777), (FP32, SUM, 1 << 17)):
+                        ins = _ins(dt, p, n * p, 950 + n + len(nic))
+                        if dt == FP32:
+                            ins[0][:] *= 1e7
+                            ins[9][:] *= -1e7
+                        print("pruned two-level reduce-scatter servers", servers, "fuse", fuse, "ports", nic, "type", dt, "n", n, flush=True)
+                        want = orc.reducescatter_two_level_pruned([x.copy() for x in ins], dt, op, servers, nic)
+                        outs, keep = gh.reduce_scatter(g, ins, dt, op)
+                        assert g.info()["fused"] == fuse
+                        for r in range(p):
+                            assert gh.same(dt, outs[r], want[r]), (servers, fuse, nic, dt, n, r)
+                            assert np.array_equal(keep[r], ins[r])
+                        if dt == FP32 and n == 10007:
+                            plain = orc.reducescatter_two_level(ins, dt, op, servers, level1=RING, level0="ring4")
+                            assert any(not np.array_equal(a, b) for a, b in zip(plain, want))     # the data tells the branches apart
+                if servers == 2:
+                    n = kat["elements_per_block"]
+                    g.set(nic_ranks=",".join(str(r) for r in kat["nic_devices"]))
+                    for case in kat["cases"]:
+                        xs = [np.full(16 * n, v, np.float32) for v in case["inputs_per_rank"]]
+                        outs, _ = gh.reduce_scatter(g, xs, FP32, SUM)
+                        for b in range(16):
+                            want = (np.full(n, case["pruned_every_element"], np.float32) if "pruned_every_element" in case
+                                    else np.repeat(np.array(case["block_halves"][b], np.float32), n // 2))
+                            assert np.array_equal(outs[b], want), (fuse, case["name"], b)
+                    g.set(nic_ranks="all")
+                    case = kat["cases"][0]
+                    xs = [np.full(16 * n, v, np.float32) for v in case["inputs_per_rank"]]
+                    outs, _ = gh.reduce_scatter(g, xs, FP32, SUM)
+                    assert all(np.all(o == np.float32(case["ordinary_two_level_every_element"])) for o in outs), fuse
+            finally:
+                g.close()
+
+
 def test_sizes_that_change_from_call_to_call(orc):
     # a new count on every call: the plan of a count that cuts into whole slices is an earlier plan scaled, a ragged
     # count is planned from scratch; either way the result is the checker's

@@ -589,6 +589,43 @@ def test_order_sensitive_known_answers_four_rings(orc):
     assert np.array_equal(closed[0][:4], np.array(kat["expected_first4"]["ring4"], np.float32))
 
 
+def _two_level_pruned_kat():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "order_sensitive_two_level_pruned_fp32.json")) as f:
+        return json.load(f)
+
+
+def test_two_level_reducescatter_with_fewer_ports_than_devices(orc):
+    # Definition on integers for every choice of 1 and 2 port devices and some of 4, several servers, ragged counts
+    # and a chunk loop; then the hand-derived order-sensitive answers, which the ordinary two-level branch misses.
+    import itertools
+    rng = np.random.default_rng(4100)
+    ports = [list(c) for k in (1, 2) for c in itertools.combinations(range(8), k)] + [[0, 1, 2, 3], [1, 3, 4, 6], [0, 2, 5, 7]]
+    for servers, n, ccl in ((2, 37, 200 << 20), (3, 200, 1 << 16), (1, 64, 200 << 20)):
+        p = 8 * servers
+        for nic in ports:
+            ins = [rng.integers(-1000, 1000, n * p).astype(np.int32) for _ in range(p)]
+            outs = orc.reducescatter_two_level_pruned(ins, INT32, SUM, servers, nic, ccl_bytes=ccl)
+            total = np.sum(ins, axis=0, dtype=np.int64).astype(np.int32)
+            for r in range(p):
+                assert np.array_equal(outs[r], total[r * n:(r + 1) * n]), (servers, nic, r)
+    kat = _two_level_pruned_kat()
+    n, nic = kat["elements_per_block"], kat["nic_devices"]
+    for case in kat["cases"]:
+        xs = [np.full(16 * n, v, np.float32) for v in case["inputs_per_rank"]]
+        got = orc.reducescatter_two_level_pruned([x.copy() for x in xs], FP32, SUM, 2, nic)
+        plain = orc.reducescatter_two_level([x.copy() for x in xs], FP32, SUM, 2, level1=RING, level0="ring4")
+        if "pruned_every_element" in case:
+            assert all(np.all(g == np.float32(case["pruned_every_element"])) for g in got)
+            assert all(np.all(g == np.float32(case["ordinary_two_level_every_element"])) for g in plain)
+        else:
+            for b in range(16):
+                want = np.repeat(np.array(case["block_halves"][b], np.float32), n // 2)
+                assert np.array_equal(got[b], want), (b, got[b][0], got[b][-1])
+            assert any(not np.array_equal(g, q) for g, q in zip(got, plain))          # the ordinary branch slices block by block
+
+
 @pytest.mark.parametrize("level1", [RING, RHD])
 @pytest.mark.parametrize("level0", ["mesh", "ring", "ring4"])
 def test_two_level_allgather_is_the_concatenation(orc, level1, level0):

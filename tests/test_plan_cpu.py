@@ -995,6 +995,47 @@ def test_ring_pruned_allreduce_plan_matches_checker(orc):
             H.describe_plan(H.COLL_ALLREDUCE, RING | _nic_bits(nic), bad_p, 1000, FP32)
 
 
+def test_two_level_reducescatter_with_fewer_ports_than_devices_plan(orc):
+    # servers of 8 devices of which only some have a network port: the plan, step by step and fused if it fuses, against
+    # the checker's restatement of the executor's branch and against the hand-derived answers
+    from test_oracle_schedules import _two_level_pruned_kat
+    for servers in (2, 3):
+        p = 8 * servers
+        for nic in ([0], [5], [0, 4], [2, 3], [1, 6], [0, 2, 4, 6], [1, 2, 3, 7]):
+            for dt, op, n, ccl in ((FP32, SUM, 211, 200 << 20), (FP32, SUM, 500, 4 * p * 128), (BF16, PROD, 77, 200 << 20)):
+                unit = H.DTYPE_SIZE[dt]
+                ins = _ins(dt, p, n * p, 850 + p + n)
+                want = orc.reducescatter_two_level_pruned(ins, dt, op, servers, nic, ccl_bytes=ccl)
+                plan = H.describe_plan(H.COLL_REDUCESCATTER, RING | (servers << 8) | (4 << 17) | _nic_bits(nic), p, n, dt, ccl_bytes=ccl)
+                for fused in ((False, True) if plan["fusedOk"] else (False,)):
+                    sends = _bytes(ins)
+                    recvs = [np.full(n * unit, 0x5A, np.uint8) for _ in range(p)]
+                    (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, dt, op)
+                    for r in range(p):
+                        assert _same(dt, recvs[r], want[r]), (servers, nic, dt, ccl, fused, r)
+                        assert np.array_equal(sends[r], ins[r].view(np.uint8))
+    kat = _two_level_pruned_kat()
+    n = kat["elements_per_block"]
+    for case in kat["cases"]:
+        xs = [np.full(16 * n, v, np.float32) for v in case["inputs_per_rank"]]
+        plan = H.describe_plan(H.COLL_REDUCESCATTER, RING | (2 << 8) | (4 << 17) | _nic_bits(kat["nic_devices"]), 16, n, FP32)
+        for fused in ((False, True) if plan["fusedOk"] else (False,)):
+            sends = _bytes(xs)
+            recvs = [np.full(n * 4, 0x5A, np.uint8) for _ in range(16)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, FP32, SUM)
+            for b in range(16):
+                want = (np.full(n, case["pruned_every_element"], np.float32) if "pruned_every_element" in case
+                        else np.repeat(np.array(case["block_halves"][b], np.float32), n // 2))
+                assert np.array_equal(recvs[b].view(np.float32), want), (case["name"], fused, b)
+    # all ports: the ordinary branch; the halving-doubling schedule between the servers, one ring inside, or a variable-count
+    # table do not go with a port list
+    plain = H.describe_plan(H.COLL_REDUCESCATTER, RING | (2 << 8) | (4 << 17), 16, 100, FP32)
+    assert H.describe_plan(H.COLL_REDUCESCATTER, RING | (2 << 8) | (4 << 17) | _nic_bits(range(8)), 16, 100, FP32) == plain
+    for word in (RHD | (2 << 8) | (4 << 17), RING | (2 << 8) | (1 << 17), RING | (2 << 8)):
+        with pytest.raises(H.HcclError):
+            H.describe_plan(H.COLL_REDUCESCATTER, word | _nic_bits([0, 4]), 16, 100, FP32)
+
+
 def test_ring_pruned_known_answers_through_the_planner():
     import json
     import os
