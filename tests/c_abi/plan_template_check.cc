@@ -1,5 +1,5 @@
 // Plans derived from a template of another count against plans made from scratch, on the host
-// (cann-hccl_amd/csrc/plan.cc alone, no GPU): wherever PlanFromTemplate says it can derive a plan, the derived plan
+// (cann-hccl_amd/csrc/plan*.cc alone, no GPU): wherever PlanFromTemplate says it can derive a plan, the derived plan
 // must be the planner's own, number for number; counts that cut into whole slices must be derivable, and so must a
 // count with a ragged last slice from a whole-slice template of a ring or uncut-mesh all-reduce or a ring broadcast.
 #include <cstdio>

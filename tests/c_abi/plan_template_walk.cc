@@ -1,6 +1,6 @@
 // A seeded walk over plan requests and, for each request, over a sequence of counts (or block tables): every plan that
 // PlanFromTemplate derives from a template of an earlier count of the same request must be the planner's own plan for
-// that count, number for number.  Host only (cann-hccl_amd/csrc/plan.cc alone, no GPU).
+// that count, number for number.  Host only (cann-hccl_amd/csrc/plan*.cc alone, no GPU).
 //
 // The requests: collective, schedule, 2 .. 33 ranks, rank groups ("servers"), rings inside a group, ranks with a network
 // port, which ranks run in place, element size, CCL buffer size.  The counts: whole slices, ragged last slices, a few

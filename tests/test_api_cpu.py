@@ -421,7 +421,7 @@ def test_plans_derived_from_a_template_of_another_count_are_the_planners_own(tmp
     """A caller whose sizes change from call to call gets its plans by scaling an earlier plan of the same request
     whenever the schedule scales (counts that cut into whole slices).  tests/c_abi/plan_template_check.cc holds every
     derived plan against the plan made from scratch (27 schedules x 2 element sizes x in place or not x 10 x 10
-    counts), on the host, against cann-hccl_amd/csrc/plan.cc alone.  The same program holds the plans of the
+    counts), on the host, against the planner's sources (cann-hccl_amd/csrc/plan*.cc) alone.  The same program holds the plans of the
     variable-count reduce-scatter that are derived from the plan over blocks of 16, 32, 64 ... elements against the
     planner's own (ring, uncut mesh, halving-doubling; 2 to 32 ranks; tables of equal, tiny, mixed and large blocks),
     and checks that the piece-cut mesh, tables with gaps or empty blocks and in-place calls get no such template."""
@@ -435,13 +435,18 @@ def test_plans_derived_from_a_template_of_another_count_are_the_planners_own(tmp
     exe = str(tmp_path / "plan_template_check")
     subprocess.run([cxx, "-O2", "-std=c++17", "-Wall", "-Werror", "-I", os.path.join(root, "cann-hccl_amd", "csrc"),
                     "-I", os.path.join(root, "include"), os.path.join(root, "tests", "c_abi", "plan_template_check.cc"),
-                    os.path.join(root, "cann-hccl_amd", "csrc", "plan.cc"), "-o", exe], check=True)
+                    *_planner_sources(root), "-o", exe], check=True)
     out = subprocess.run([exe], stdout=subprocess.PIPE, text=True)
     assert out.returncode == 0 and out.stdout.startswith("OK"), out.stdout
     derived = int(out.stdout.split()[3])
     assert derived > 1000, out.stdout
     tables = int(out.stdout.split("templates,")[1].split()[0])
     assert tables > 300, out.stdout
+
+
+def _planner_sources(root):
+    return [os.path.join(root, "cann-hccl_amd", "csrc", f)
+            for f in ("plan.cc", "plan_schedules.cc", "plan_lower.cc", "plan_fuse.cc", "plan_template.cc")]
 
 
 def test_seeded_walk_over_requests_and_counts_derives_only_the_planners_own_plans(tmp_path):
@@ -460,7 +465,7 @@ def test_seeded_walk_over_requests_and_counts_derives_only_the_planners_own_plan
     exe = str(tmp_path / "plan_template_walk")
     subprocess.run([cxx, "-O2", "-std=c++17", "-Wall", "-Werror", "-I", os.path.join(root, "cann-hccl_amd", "csrc"),
                     "-I", os.path.join(root, "include"), os.path.join(root, "tests", "c_abi", "plan_template_walk.cc"),
-                    os.path.join(root, "cann-hccl_amd", "csrc", "plan.cc"), "-o", exe], check=True)
+                    *_planner_sources(root), "-o", exe], check=True)
     out = subprocess.run([exe, "20000"], stdout=subprocess.PIPE, text=True, timeout=300)
     print(out.stdout)
     assert out.returncode == 0 and out.stdout.startswith("OK"), out.stdout
