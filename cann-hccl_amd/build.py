@@ -25,7 +25,7 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-I", os.path.join(
 DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 DTYPES = list(range(12)) + [255]
 DEVICE_SOURCES = ["noalloc.hip"]
-HOST_SOURCES = ["plan.cc", "plan_schedules.cc", "plan_lower.cc", "plan_fuse.cc", "plan_template.cc", "ranktable.cc", "exec.cc", "api.cc", "kernels_table.cc"]
+HOST_SOURCES = ["plan.cc", "plan_schedules.cc", "plan_lower.cc", "plan_fuse.cc", "plan_template.cc", "ranktable.cc", "exec.cc", "api.cc", "api_rendezvous.cc", "api_comm.cc", "api_ext.cc", "kernels_table.cc"]
 
 
 def _newer(target, deps):
