@@ -50,14 +50,19 @@ HcclResult EnsureDevice(Group *g, bool quiet)
     hipDeviceProp_t prop;
     HIP_OK(hipGetDeviceProperties(&prop, g->device));
     g->numCu = prop.multiProcessorCount > 0 ? uint32_t(prop.multiProcessorCount) : 256u;
+    // Events that only order streams of this device against each other: no timestamps, and no system-scope fence when
+    // they complete (the kernels on either side release and acquire at device scope themselves; a caller that reads
+    // results on the host synchronises its own stream, which fences).  One thread per rank, 8 KiB all-reduce: 47 us
+    // per collective at 8 ranks against 55 us with the fence, 78 against 95 at 16.
+    constexpr unsigned kOrderOnly = hipEventDisableTiming | hipEventDisableSystemFence;
     g->arriveEvents.assign(g->p, nullptr);
     for (uint32_t r = 0; r < g->p; r++) {
-        HIP_OK(hipEventCreateWithFlags(&g->arriveEvents[r], hipEventDisableTiming));
+        HIP_OK(hipEventCreateWithFlags(&g->arriveEvents[r], kOrderOnly));
     }
     for (hipEvent_t &e : g->doneEvents) {
-        HIP_OK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        HIP_OK(hipEventCreateWithFlags(&e, kOrderOnly));
     }
-    HIP_OK(hipEventCreateWithFlags(&g->p2pDoneEvent, hipEventDisableTiming));
+    HIP_OK(hipEventCreateWithFlags(&g->p2pDoneEvent, kOrderOnly));
     HIP_OK(hipStreamCreateWithFlags(&g->copyStream, hipStreamNonBlocking));
     g->stageSlots.resize(kStageSlots);
     for (StageSlot &slot : g->stageSlots) {
