@@ -719,15 +719,16 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
             pp->uploadComplete = false;
             pp->hostTables.swap(b.host);
         } else if (b.host.size() <= kStageSlotBytes && stream != nullptr && !g->stageSlots.empty()) {
-            // medium tables (an all-to-all-v between 16 ranks: 40 KiB) go through a ring of pinned host buffers as an
-            // asynchronous copy on the caller's stream: the call does not wait for it.  A slot comes round again
-            // after as many collectives as the ring has slots; its previous copy has normally long finished.
+            // medium tables (an all-to-all-v between 16 ranks: 40 KiB) go through a ring of pinned host buffers, from
+            // where a launch on the caller's stream fetches them: the call does not wait for it, and the stream does
+            // not change engines as it would for a copy command.  A slot comes round again after as many collectives
+            // as the ring has slots; its previous fetch has normally long finished.
             StageSlot &slot = g->stageSlots[g->stageNext++ % g->stageSlots.size()];
             if (slot.used) {
                 HIP_OK(hipEventSynchronize(slot.done));
             }
             std::memcpy(slot.host, b.host.data(), b.host.size());
-            HIP_OK(hipMemcpyAsync(pp->devTables, slot.host, b.host.size(), hipMemcpyHostToDevice, stream));
+            HIP_OK(UploadFromPinned(pp->devTables, slot.host, b.host.size(), stream));
             HIP_OK(hipEventRecord(slot.done, stream));
             slot.used = true;
             HIP_OK(hipEventCreateWithFlags(&pp->uploaded, hipEventDisableTiming));

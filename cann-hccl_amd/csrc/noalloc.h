@@ -26,5 +26,7 @@ hipError_t NoAllocEnd(int device, hipStream_t stream);
 // copy is rounded up to a multiple of 16 bytes).  The host bytes are consumed before the call returns.
 // Also used for the small tables of ordinary collectives: unlike a host-to-device copy it never waits.
 hipError_t UploadThroughKernelArgs(void *dst, const void *hostBytes, size_t bytes, hipStream_t stream);
+// The same for bytes in pinned host memory (rounded up to 16): one launch that reads them from there.
+hipError_t UploadFromPinned(void *dst, const void *pinnedHost, size_t bytes, hipStream_t stream);
 
 }  // namespace hcclamd

@@ -43,7 +43,30 @@ __global__ void __launch_bounds__(256) UploadKernel(UploadPiece piece, unsigned 
     }
 }
 
+// Table bytes that lie in pinned host memory: the device fetches them itself, as a launch in the stream's order (a copy
+// command would hand the stream to a copy engine and back).
+__global__ void __launch_bounds__(256) FetchKernel(const unsigned char *__restrict__ pinned, unsigned char *__restrict__ dst,
+    uint32_t nwords)
+{
+    typedef Word4 __attribute__((address_space(1))) GlobalWord4;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nwords) {
+        ((GlobalWord4 *)dst)[i] = ((const GlobalWord4 *)pinned)[i];
+    }
+}
+
 }  // namespace
+
+hipError_t UploadFromPinned(void *dst, const void *pinnedHost, size_t bytes, hipStream_t stream)
+{
+    const uint32_t nwords = uint32_t((bytes + 15) / 16);
+    if (nwords == 0) {
+        return hipSuccess;
+    }
+    hipLaunchKernelGGL(FetchKernel, dim3((nwords + 255) / 256), dim3(256), 0, stream,
+        static_cast<const unsigned char *>(pinnedHost), static_cast<unsigned char *>(dst), nwords);
+    return hipGetLastError();
+}
 
 hipError_t NoAllocWorkspace(int device, void **base)
 {
