@@ -237,6 +237,7 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         }
         if (coll == COLL_BROADCAST) {
             rq.servers = std::max(1u, (uint32_t(algo) >> 20) & 0xffu);   // broadcast: bits 20..27 = rank groups (two levels)
+            rq.level0Rings = ((uint32_t(algo) >> 29) & 1u) ? 1u : (((uint32_t(algo) >> 30) & 1u) ? 4u : 0u);   // as for the reduce
         }
         if (coll == COLL_REDUCE) {
             rq.servers = std::max(1u, (uint32_t(algo) >> 20) & 0xffu);

@@ -995,6 +995,15 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAl
         rq.algo = Level1Algo(g);
         rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
     }
+    if (rq.coll == COLL_BROADCAST && g->cfg.level0Rings > 0 && g->p % g->cfg.servers == 0 && g->cfg.algo != ALGO_RING &&
+        g->cfg.algo != ALGO_STAR && g->cfg.algo != ALGO_HD_BLOCKS &&
+        (g->cfg.servers > 1 || (g->cfg.level0Rings == 4 && g->p == 8))) {
+        // the ring topologies' broadcast (coll_broadcast_ring_executor.cc:64-211): ring scatter in the root's group over
+        // one ring or the four rings of a group of 8, halving-doubling between the groups, ring all-gather in every
+        // group; also for a single group of 8 with its four rings
+        rq.servers = g->cfg.servers;
+        rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
+    }
     if (rq.coll == COLL_BROADCAST && g->cfg.servers > 1 && g->p % g->cfg.servers == 0 && g->cfg.algo != ALGO_RING &&
         g->cfg.algo != ALGO_STAR && g->cfg.algo != ALGO_HD_BLOCKS && g->cfg.level0Rings == 0) {
         // two levels (coll_broadcast_mesh_executor.cc:59-213): scatter in the root's group, halving-doubling between

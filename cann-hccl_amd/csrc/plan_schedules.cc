@@ -1133,7 +1133,60 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
         uint64_t done = 0;
         for (uint64_t left = rq.count; left > 0;) {
             uint64_t cur = std::min(left, per), bytes = cur * u;
-            if (rq.coll == COLL_BROADCAST && rq.servers > 1 && p > 1) {
+            if (rq.coll == COLL_BROADCAST && rq.level0Rings > 0 && p > 1) {
+                // The ring topologies' broadcast (coll_broadcast_ring_executor.cc:64-211): slices over the D ranks of a
+                // group, every slice cut into one part per ring.  Step 1, in the root's group only: ring k runs the
+                // ring scatter (scatter_ring.cc:22-135) from the root's position over part k of its members' slices --
+                // the part with the longest way leaves first, a member keeps the last part it receives and passes the
+                // others on.  Step 2: the ranks at position d of all groups pass slice d on by recursive
+                // halving-doubling from the root's group.  Step 3: ring all-gather of the parts in every group, ring
+                // by ring.  In place; the root keeps its data where it is, so what the all-gather would hand back to
+                // it is left out.
+                const uint32_t S = rq.servers, D = p / S, rootGroup = R / D, rings = rq.level0Rings;
+                std::vector<Slice> sl = RingSlicePlan(bytes, D, rq.align);
+                auto at = [&](uint32_t r, uint64_t off) {
+                    return r == R ? MkRef(R, BUF_SEND, done + off) : MkRef(r, BUF_RECV, done + off);
+                };
+                auto device = [&](uint32_t k, uint32_t i) { return rings > 1 ? kRingOrders8[k][i] : i; };
+                auto part = [&](uint32_t k, uint32_t i) {
+                    const Slice &whole = sl[device(k, i)];
+                    std::vector<Slice> cut = RingSlicePlan(whole.size, rings, rq.align);
+                    return Slice{whole.off + cut[k].off, cut[k].size};
+                };
+                const size_t l1 = D > 1 ? D - 1 : 0;
+                for (uint32_t k = 0; k < rings && D > 1; k++) {
+                    uint32_t rootPos = 0;
+                    for (uint32_t i = 0; i < D; i++) {
+                        rootPos = device(k, i) == R % D ? i : rootPos;
+                    }
+                    for (uint32_t j = 1; j < D; j++) {            // j = hops from the root to the part's owner
+                        const Slice pt = part(k, (rootPos + j) % D);
+                        for (uint32_t h = 1; h <= j; h++) {
+                            const uint32_t from = rootGroup * D + device(k, (rootPos + h - 1) % D);
+                            const uint32_t to = rootGroup * D + device(k, (rootPos + h) % D);
+                            EmitCopy(*vp, size_t(D - j + h - 2), at(to, pt.off), at(from, pt.off), pt.size);
+                        }
+                    }
+                }
+                size_t l2 = l1;
+                for (uint32_t d = 0; d < D && S > 1; d++) {
+                    auto data = [&](uint32_t g) { return at(g * D + d, sl[d].off); };
+                    l2 = std::max(l2, RhdBroadcastPhases(*vp, l1, S, rootGroup, data, sl[d].size));
+                }
+                for (uint32_t g = 0; g < S && D > 1; g++) {
+                    for (uint32_t k = 0; k < rings; k++) {
+                        for (uint32_t h = 0; h + 1 < D; h++) {
+                            for (uint32_t i = 0; i < D; i++) {
+                                const uint32_t to = g * D + device(k, i), from = g * D + device(k, Mod(int64_t(i) - 1, D));
+                                const Slice pt = part(k, Mod(int64_t(i) - 1 - h, D));
+                                if (to != R) {
+                                    EmitCopy(*vp, l2 + h, at(to, pt.off), at(from, pt.off), pt.size);
+                                }
+                            }
+                        }
+                    }
+                }
+            } else if (rq.coll == COLL_BROADCAST && rq.servers > 1 && p > 1) {
                 // Two levels (coll_broadcast_mesh_executor.cc:59-213 with several servers): the root scatters slice d
                 // to position d of its own group (scatter_mesh.cc), the ranks at position d of all groups pass it on by
                 // recursive halving-doubling from the root's group, and every group gathers the slices (mesh).

@@ -2886,6 +2886,135 @@ int orc_broadcast_two_level(uint32_t servers, uint32_t p, void **buf, uint64_t c
     return 0;
 }
 
+// Two-level broadcast of the ring topologies, CollBroadcastRingExecutor::KernelRun
+// (EXE/coll_broadcast/coll_broadcast_ring_executor.cc:64-211) under the chunk loop of CollBroadcastExecutor::RunLoop;
+// `servers` groups of D = p / servers consecutive ranks, `rings` = 1 (one ring in rank order) or 4 (the four rings of
+// the 8-device topology, D = 8).  Per chunk: slices over the D devices (PrepareSliceData, :80), every slice cut into one
+// part per ring (PrepareMultiRingSlice with all ports, :86-93).
+//   step 1 (:95-102, MultiRingScatter, EXE/coll_comm_executor.cc:1995-2130): only in the root's server, ring k runs the
+//          ring scatter (TPL/temp_scatter/scatter_ring.cc:22-135) from the root's position over part k of its members'
+//          slices, in place in the input buffer
+//   step 2 (:105-187): the devices at position d of all servers broadcast slice d from the root's server by recursive
+//          halving-doubling (segment and size from PrepareLevel1CommInfo, EXE/coll_comm_executor.cc:2176-2214)
+//   step 3 (:189-207, MultiRingAllGather): ring all-gather of the parts inside every server, ring by ring
+// `touched` (optional) receives the bytes read + written by all ranks.
+int orc_broadcast_two_level_ring(uint32_t servers, uint32_t rings, uint32_t p, void **buf, uint64_t count, int dt, uint32_t root,
+    uint64_t cclBytes, uint64_t align, int flags, int threads, uint64_t *touched)
+{
+    uint64_t moved = 0;
+    uint64_t unit = DtSize(dt);
+    if (unit == 0 || p == 0 || root >= p || servers == 0 || p % servers != 0 || (rings != 1 && rings != 4) ||
+        (rings == 4 && p / servers != 8)) {
+        return -20;
+    }
+    uint64_t maxPer = cclBytes / unit;
+    if (maxPer == 0) {
+        return -21;
+    }
+    const uint32_t D = p / servers, rootGroup = root / D, rootLocal = root % D;
+    Pool pool(threads);
+    auto machine = [&](uint32_t n) {
+        Machine m;
+        m.p = static_cast<int>(n);
+        m.dt = dt;
+        m.direct = (flags & 1) != 0;
+        m.pool = &pool;
+        m.buf[B_IN].resize(n);
+        m.buf[B_OUT].resize(n);
+        return m;
+    };
+    auto device = [&](uint32_t k, uint32_t i) { return rings > 1 ? kEightDeviceRings[k][i] : i; };
+    uint64_t offset = 0;
+    for (uint64_t left = count; left > 0 && p > 1;) {
+        uint64_t cur = left > maxPer ? maxPer : left;
+        uint64_t bytes = cur * unit;
+        std::vector<Slice> sl = RingSlices(bytes, D, align);
+        std::vector<std::vector<Slice>> segs = MultiSegSlices(sl, rings, align);
+        auto at = [&](uint32_t g, uint32_t d) { return static_cast<uint8_t *>(buf[g * D + d]) + offset; };
+        for (uint32_t k = 0; k < rings && D > 1; k++) {               // step 1
+            Machine m = machine(D);
+            std::vector<Slice> ringSl(D);
+            uint32_t rootPos = 0;
+            for (uint32_t i = 0; i < D; i++) {
+                m.buf[B_IN][i] = m.buf[B_OUT][i] = at(rootGroup, device(k, i));
+                ringSl[i] = segs[device(k, i)][k];
+                if (device(k, i) == rootLocal) {
+                    rootPos = i;
+                }
+            }
+            for (uint32_t r = 0; r < D; r++) {
+                Proc pr;
+                pr.rank = r;
+                const int lft = static_cast<int>((r + D - 1) % D), rgt = static_cast<int>((r + 1) % D);
+                if (r == rootPos) {
+                    for (uint32_t i = 1; i < D; i++) {
+                        const uint32_t owner = (r + D - i) % D;
+                        pr.prog.push_back(MkSend(rgt, 0, B_IN, ringSl[owner].off, ringSl[owner].size));
+                    }
+                } else {
+                    const uint32_t rounds = (rootPos + D - r) % D;     // parts this position receives, its own last
+                    for (uint32_t i = 1; i <= rounds; i++) {
+                        const uint32_t owner = (r + rounds - i) % D;
+                        if (i != 1) {
+                            const uint32_t previous = (r + rounds - i + 1) % D;
+                            pr.prog.push_back(MkSend(rgt, 0, B_OUT, ringSl[previous].off, ringSl[previous].size));
+                        }
+                        pr.prog.push_back(MkRecvCopy(lft, 0, B_OUT, ringSl[owner].off, ringSl[owner].size));
+                    }
+                }
+                m.procs.push_back(std::move(pr));
+            }
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+            moved += m.bytesTouched;
+        }
+        for (uint32_t d = 0; d < D && servers > 1; d++) {              // step 2
+            if (sl[d].size == 0) {
+                continue;
+            }
+            Machine m = machine(servers);
+            for (uint32_t g = 0; g < servers; g++) {
+                m.buf[B_IN][g] = m.buf[B_OUT][g] = at(g, d);
+            }
+            AddBroadcastRhdProcs(m, rootGroup, sl[d].off, sl[d].size);
+            int rc = m.Run();
+            if (rc != 0) {
+                return rc;
+            }
+            moved += m.bytesTouched;
+        }
+        for (uint32_t g = 0; g < servers && D > 1; g++) {              // step 3
+            for (uint32_t k = 0; k < rings; k++) {
+                Machine m = machine(D);
+                std::vector<Slice> ringSl(D);
+                for (uint32_t i = 0; i < D; i++) {
+                    m.buf[B_IN][i] = m.buf[B_OUT][i] = at(g, device(k, i));
+                    ringSl[i] = segs[device(k, i)][k];
+                }
+                for (uint32_t i = 0; i < D; i++) {
+                    Proc pr;
+                    pr.rank = i;
+                    ProgAllGatherRing(pr.prog, i, D, B_OUT, B_OUT, ringSl, ringSl);
+                    m.procs.push_back(std::move(pr));
+                }
+                int rc = m.Run();
+                if (rc != 0) {
+                    return rc;
+                }
+                moved += m.bytesTouched;
+            }
+        }
+        offset += bytes;
+        left -= cur;
+    }
+    if (touched != nullptr) {
+        *touched = moved;
+    }
+    return 0;
+}
+
 // Per-rank programs of ReduceRecursiveHalvingDoubling::RunAsync (TPL/temp_reduce/reduce_recursive_hd.cc:31-316) on the
 // machine's buffers of `bytes` bytes: input accumulates in place, the result ends in the root's output buffer.
 void AddReduceRhdProcs(Machine &m, uint32_t root, uint64_t bytes, uint64_t align)

@@ -86,6 +86,7 @@ def lib():
         L.orc_broadcast_star.restype = i32
         L.orc_allreduce_ring_pruned.argtypes = [u32, ctypes.POINTER(vp), ctypes.POINTER(vp), u64, i32, i32, ctypes.POINTER(u32), u32,
                                                 u64, u64, i32, i32]
+        L.orc_broadcast_two_level_ring.argtypes = [u32, u32, u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32, ctypes.POINTER(u64)]
         L.orc_broadcast_two_level.argtypes = [u32, u32, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32, ctypes.POINTER(u64)]
         L.orc_reduce_to_root_mesh.argtypes = [u32, ctypes.POINTER(vp), vp, u64, i32, i32, u32, u64, u64, i32, i32, i32]
         L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
@@ -361,6 +362,19 @@ def broadcast_hd_blocks_route(p, root):
     n = lib().orc_broadcast_hd_blocks_route(p, root, pairs, cap)
     assert 0 <= n <= cap
     return [(pairs[2 * i], pairs[2 * i + 1]) for i in range(n)]
+
+
+def broadcast_two_level_ring(bufs, dt, root, servers, rings=1, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1,
+                             return_touched=False):
+    """Two-level broadcast of the ring topologies (coll_broadcast_ring_executor.cc): ring scatter in the root's server over
+    one ring or the four rings of the 8-device topology, halving-doubling between the servers, ring all-gather in every
+    server.  bufs are written in place."""
+    touched = ctypes.c_uint64(0)
+    rc = lib().orc_broadcast_two_level_ring(servers, rings, len(bufs), _ptrs(bufs), bufs[0].size, dt, root, ccl_bytes, align,
+                                            flags, threads, ctypes.byref(touched))
+    if rc != 0:
+        raise RuntimeError("oracle two-level ring broadcast failed rc=%d" % rc)
+    return (bufs, touched.value) if return_touched else bufs
 
 
 def broadcast_two_level(bufs, dt, root, servers, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1,

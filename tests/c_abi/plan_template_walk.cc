@@ -84,7 +84,8 @@ int main(int argc, char **argv)
             }
         }
         const uint32_t perGroup = base.p / base.servers;
-        if ((base.coll == COLL_ALLREDUCE || base.coll == COLL_REDUCESCATTER || base.coll == COLL_ALLGATHER || base.coll == COLL_REDUCE) &&
+        if ((base.coll == COLL_ALLREDUCE || base.coll == COLL_REDUCESCATTER || base.coll == COLL_ALLGATHER || base.coll == COLL_REDUCE ||
+                base.coll == COLL_BROADCAST) &&
             Below(4) == 0 && (base.servers > 1 || perGroup == 8)) {
             base.level0Rings = (perGroup == 8 && Below(2)) ? 4 : (base.servers > 1 ? 1 : 0);
         }

@@ -1037,6 +1037,35 @@ def test_binary_block_broadcast(orc):
                 g.close()
 
 
+def test_two_level_ring_broadcast(orc):
+    # the ring topologies' broadcast: ring scatter in the root's group (one ring, or the four rings of a group of 8),
+    # halving-doubling between the groups, ring all-gather in every group; fused one launch, step by step one per phase
+    n = 70001
+    for servers, D, level0 in ((2, 4, "ring"), (3, 3, "ring"), (2, 8, "ring4"), (1, 8, "ring4")):
+        p = servers * D
+        for fuse in (1, 0):
+            g = gh.Group(p, algo="rhd", servers=servers, level0=level0, fuse=fuse, buffsize_bytes=1 << 17)
+            try:
+                for root in sorted({0, p - 1, (D + 1) % p}):
+                    print("two-level ring broadcast", servers, "x", D, level0, "fuse", fuse, "root", root, flush=True)
+                    bufs_np = _ins(INT32, p, n, 205 + p + root)
+                    want, touched = orc.broadcast_two_level_ring([x.copy() for x in bufs_np], INT32, root, servers,
+                                                                 rings=4 if level0 == "ring4" else 1, ccl_bytes=1 << 17,
+                                                                 return_touched=True)
+                    bufs = [gh.to_dev(x) for x in bufs_np]
+                    torch.cuda.synchronize()
+                    H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, INT32, root, g.stream_ptr)
+                    g.stream.synchronize()
+                    info = g.info()
+                    assert info["fused"] == fuse, info
+                    if not fuse:
+                        assert info["launches"] > (2 if servers > 1 else 1) and info["bytesWritten"] < touched // 2
+                    for r in range(p):
+                        assert np.array_equal(gh.to_host(bufs[r], INT32), want[r]), (servers, D, level0, fuse, root, r)
+            finally:
+                g.close()
+
+
 def test_allreduce_at_the_rank_limit(orc):
     # 64 ranks is the most a group holds: ring / uncut mesh = chains of 64 sources (the fused kernel's limit),
     # halving-doubling at 48 ranks = 32 leaves of which 16 are folded pairs, at 64 ranks = 32 leaves of two

@@ -782,6 +782,39 @@ def test_binary_block_broadcast_routes_and_bytes(orc):
             assert set(route) == tree, (p, root)
 
 
+@pytest.mark.parametrize("shape", [(2, 4, 1), (3, 3, 1), (4, 2, 1), (1, 5, 1), (5, 1, 1), (2, 8, 4), (1, 8, 4), (3, 8, 4)])
+def test_two_level_ring_broadcast_delivers_and_moves_the_closed_form_bytes(orc, shape):
+    # Definition: every rank ends with the root's bytes.  Structure: the bytes received over all ranks are those of the
+    # ring scatter in the root's group (a part that ends j positions behind the root is received j times), one
+    # halving-doubling broadcast per slice between the groups, and one ring all-gather per group and ring -- a mesh
+    # scatter, a flat broadcast or a scatter that started at another position would count differently.
+    servers, D, rings = shape
+    p = servers * D
+    for dt, n in ((INT32, 1), (INT32, 1000), (INT8, 100003), (INT64, 5000)):
+        unit = orc.dtype_size(dt)
+        for root in sorted({0, p - 1, p // 2, D - 1, min(D, p - 1)}):
+            for ccl in (200 << 20, 8192):
+                bufs = _inputs(dt, p, n, root + n)
+                src = bufs[root].copy()
+                bufs, touched = orc.broadcast_two_level_ring(bufs, dt, root, servers, rings=rings, ccl_bytes=ccl, return_touched=True)
+                assert all(np.array_equal(b, src) for b in bufs), (shape, dt, n, root, ccl)
+                received, left = 0, n
+                max_per = ccl // unit
+                while left > 0 and p > 1:
+                    cur = min(left, max_per)
+                    sl = cf.slice_plan(cur * unit, D, 128)
+                    for k in range(rings):
+                        order = list(cf.EIGHT_DEVICE_RINGS[k]) if rings == 4 else list(range(D))
+                        root_pos = order.index(root % D)
+                        for j in range(1, D):
+                            size = sl[order[(root_pos + j) % D]][1]
+                            parts = cf.slice_plan(size, rings, 128)
+                            received += j * parts[k][1]
+                    received += (servers - 1) * cur * unit + servers * (D - 1) * cur * unit
+                    left -= cur
+                assert touched == 2 * received, (shape, dt, n, root, ccl, touched, received)
+
+
 @pytest.mark.parametrize("shape", [(2, 4), (4, 2), (3, 2), (3, 4), (1, 4), (8, 1), (5, 3)])
 def test_two_level_broadcast_delivers_and_moves_the_closed_form_bytes(orc, shape):
     # Definition: every rank ends with the root's bytes.  Structure: the bytes received over all ranks are those of

@@ -880,6 +880,46 @@ def test_binary_block_broadcast_plan(orc):
                         assert np.array_equal(mem[r].view(np.int32), want[r]), (p, root, ccl, fused, r)
 
 
+@pytest.mark.parametrize("servers,D,rings", [(2, 4, 1), (3, 3, 1), (4, 2, 1), (2, 8, 4), (1, 8, 4), (3, 8, 4)])
+def test_two_level_ring_broadcast_plan(orc, servers, D, rings):
+    # ring scatter in the root's group, halving-doubling between the groups, ring all-gather in every group: results and
+    # bytes as the checker's (less what the all-gather would hand back to the root), and the route -- inside a group a
+    # part only moves to the next device of its ring, between groups only between equal positions
+    p = servers * D
+    n = 1003
+    rng = np.random.default_rng(650 + p)
+    orders = [list(o) for o in cf.EIGHT_DEVICE_RINGS] if rings == 4 else [list(range(D))]
+    nexts = {(o[i], o[(i + 1) % D]) for o in orders for i in range(D)}
+    for root in sorted({0, p - 1, (D + 1) % p}):
+        for ccl in (200 << 20, 1024):
+            bufs = [rng.integers(0, 1 << 30, n).astype(np.int32) for _ in range(p)]
+            want, touched = orc.broadcast_two_level_ring([b.copy() for b in bufs], INT32, root, servers, rings=rings, ccl_bytes=ccl,
+                                                         return_touched=True)
+            word = root | (RHD << 16) | (servers << 20) | ((1 << 29) if rings == 1 else (1 << 30))
+            plan = H.describe_plan(H.COLL_BROADCAST, word, p, n, INT32, ccl_bytes=ccl, in_place_mask=(1 << p) - 1)
+            assert plan["fusedOk"]
+            back = 0
+            for cur in ([n] if ccl >= n * 4 else [256] * (n // 256) + [n % 256]):
+                back += cur * 4 - cf.slice_plan(cur * 4, D, 128)[root % D][1]
+            assert plan["stepWritten"] == touched // 2 - back
+            for ph in plan["phases"]:
+                for st in ph:
+                    a, d = st["a"][0], st["dst"][0]
+                    assert d != root
+                    if a // D == d // D:
+                        assert (a % D, d % D) in nexts, (servers, D, rings, root, a, d)
+                    else:
+                        assert a % D == d % D, (servers, D, rings, root, a, d)
+            for fused in (False, True):
+                mem = _bytes(bufs)
+                (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, mem, mem, INT32, 0, in_place=True)
+                for r in range(p):
+                    assert np.array_equal(mem[r].view(np.int32), want[r]), (servers, D, rings, root, ccl, fused, r)
+    # four rings need groups of 8
+    with pytest.raises(H.HcclError):
+        H.describe_plan(H.COLL_BROADCAST, 0 | (RHD << 16) | (2 << 20) | (1 << 30), 8, n, INT32)
+
+
 @pytest.mark.parametrize("servers,D", [(2, 4), (4, 2), (3, 4), (5, 3), (6, 1), (2, 8)])
 def test_two_level_broadcast_plan(orc, servers, D):
     # scatter inside the root's group, halving-doubling between the groups, all-gather inside every group:
