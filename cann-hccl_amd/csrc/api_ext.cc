@@ -234,6 +234,7 @@ HcclResult HcclAmdDescribePlan(int32_t coll, int32_t algo, uint32_t nRanks, uint
         if (coll == COLL_SCATTER) {
             rq.algo = ((uint32_t(algo) >> 20) & 1u) ? ALGO_RING : ALGO_MESH;   // scatter: bit 20 = the ring schedule
             rq.servers = std::max(1u, (uint32_t(algo) >> 21) & 0xffu);         // bits 21..28 = rank groups (two levels, mesh only)
+            rq.level0Rings = ((uint32_t(algo) >> 29) & 1u) ? 1u : (((uint32_t(algo) >> 30) & 1u) ? 4u : 0u);   // as for the reduce
         }
         if (coll == COLL_BROADCAST) {
             rq.servers = std::max(1u, (uint32_t(algo) >> 20) & 0xffu);   // broadcast: bits 20..27 = rank groups (two levels)

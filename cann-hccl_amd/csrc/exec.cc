@@ -1012,8 +1012,10 @@ HcclResult Prepare(Group *g, int algo, std::unique_ptr<Prepared> *out, bool noAl
     }
     if (rq.coll == COLL_SCATTER && g->cfg.servers > 1 && g->p % g->cfg.servers == 0 && rq.algo != ALGO_RING) {
         // two levels (coll_scatter_mesh_executor.cc:40-110): ring scatter of the groups' runs between the sub-roots,
-        // mesh scatter inside every group; the flat ring when the ring is asked for by name
+        // mesh scatter inside every group, or the ring scatter when the groups are set up as rings
+        // (coll_scatter_ring_executor.cc:42-113); the flat ring when the ring is asked for by name
         rq.servers = g->cfg.servers;
+        rq.level0Rings = g->cfg.level0Rings == 4 ? (g->p / g->cfg.servers == 8 ? 4u : 1u) : g->cfg.level0Rings;
     }
     if (rq.coll == COLL_REDUCE && g->cfg.servers > 1 && g->p % g->cfg.servers == 0) {
         // two levels (coll_reduce_mesh_executor.cc:75-194, coll_reduce_ring_plus_hd_executor.cc:75-168): inside the

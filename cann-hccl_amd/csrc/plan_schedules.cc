@@ -1098,9 +1098,35 @@ int BuildVirtual(const PlanRequest &rq, VProgram *vp, std::string *err)
                     vp->workBytes[to] = std::max(vp->workBytes[to], uint64_t(dest + 1) * run);
                 }
             }
-            for (uint32_t r = 0; r < p; r++) {
+            for (uint32_t r = 0; r < p && rq.level0Rings == 0; r++) {
                 EmitCopy(*vp, size_t(S - 1), MkRef(r, BUF_RECV, 0), MkRef(r / D * D + rootLocal, BUF_SEND, uint64_t(r) * total), total);
                 vp->outBytes[r] = total;
+            }
+            // With rings inside a group (coll_scatter_ring_executor.cc:42-113) level 0 is the ring scatter from the
+            // sub-root instead, along the ranks in their order or, for groups of 8 set up as the four-ring topology,
+            // in the order of its ring 0 (PrepareScatterRingSliceData, :115-131).
+            for (uint32_t g = 0; g < S && rq.level0Rings != 0; g++) {
+                auto order = [&](uint32_t i) { return rq.level0Rings == 4 ? kRingOrders8[0][i] : i; };
+                uint32_t rootPos = 0;
+                for (uint32_t i = 0; i < D; i++) {
+                    rootPos = order(i) == rootLocal ? i : rootPos;
+                }
+                const uint32_t sub = g * D + rootLocal;
+                EmitCopy(*vp, size_t(S - 1), MkRef(sub, BUF_RECV, 0), MkRef(sub, BUF_SEND, uint64_t(sub) * total), total);
+                vp->outBytes[sub] = total;
+                for (uint32_t j = 1; j < D; j++) {            // j = hops from the sub-root to the block's owner
+                    const uint32_t dest = g * D + order((rootPos + j) % D);
+                    for (uint32_t h = 1; h <= j; h++) {
+                        const uint32_t from = g * D + order((rootPos + h - 1) % D), to = g * D + order((rootPos + h) % D);
+                        const Ref src = MkRef(from, BUF_SEND, uint64_t(dest) * total);
+                        const Ref dst = h == j ? MkRef(dest, BUF_RECV, 0) : MkRef(to, BUF_SEND, uint64_t(dest) * total);
+                        EmitCopy(*vp, size_t(S - 1) + size_t(D - j + h - 2), dst, src, total);
+                        if (h != j) {
+                            vp->workBytes[to] = std::max(vp->workBytes[to], uint64_t(dest + 1) * total);
+                        }
+                    }
+                    vp->outBytes[dest] = total;
+                }
             }
             return 0;
         }

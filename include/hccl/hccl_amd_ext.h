@@ -34,7 +34,7 @@ extern "C" {
  *                   inside the group, unless "algo" is "ring";
  *                   the all-to-all family then runs the staged schedule (gather inside a group into a workspace, pairwise
  *                   between the groups) unless "algo" is "pairwise"
- *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter / all-gather / reduce / broadcast: the mesh schedule
+ *   "level0"        "mesh" | "ring" | "ring4"   what runs inside a group of the two-level all-reduce / reduce-scatter / all-gather / reduce / broadcast / scatter: the mesh schedule
  *                                (default), one ring in rank order, or -- for groups of 8 ranks, for the all-reduce also with one group --
  *                                the four rings of the 8-device ring topology, each on a quarter of every slice
  *   "nic_ranks"     "all" | list of 1, 2 or 4 ranks, e.g. "0,4"   groups of 8 ranks only: the ranks that own a network port.
@@ -104,7 +104,7 @@ extern HcclResult HcclAmdGetLastOpInfo(HcclComm comm, HcclAmdOpInfo *info);
  * collectives (coll 4 broadcast, 5 reduce, 6 scatter) the algo argument carries the root rank in its low 16 bits and the
  * schedule in bits 16..19 (0 ring, 1 mesh, 2 rhd, 4 mesh without the piece cut, 5 star, 6 hd over blocks: broadcast only), for the reduce also the number of rank
  * groups of its two-level schedule in bits 20..27, bit 28 for the mesh level without the piece cut and bit 29 / bit 30 for
- * one ring / four rings inside a group, for the broadcast the number of rank groups in bits 20..27 and bit 29 / bit 30 the same way, for the scatter
+ * one ring / four rings inside a group, for the broadcast the number of rank groups in bits 20..27 and bit 29 / bit 30 the same way (the scatter takes these two bits too), for the scatter
  * bit 20 for the ring schedule instead of the mesh and the number of rank groups of the two-level mesh schedule in bits 21..28;
  * for the all-reduce (coll 0) bits 8..15 of algo
  * carry the number of rank groups of the two-level schedule (0 or 1: one level), bit 16 asks for its mesh level

@@ -3562,11 +3562,16 @@ int orc_scatter_ring(uint32_t p, const void *inRoot, void **out, uint64_t count,
 // (:72-101): mesh scatter inside every group from the sub-root over the group's run (scatter_mesh.cc:46-160, base
 // offset = the run's), again in place in the staging buffers; then every rank copies its block out (:103-106).
 // `touched` (optional) receives the bytes read + written by all ranks.
+// level0 = 1 / 2: CollScatterRingExecutor::KernelRun (EXE/coll_scatter/coll_scatter_ring_executor.cc:42-113) instead:
+// step 1 is the same, step 2 the ring scatter (scatter_ring.cc) inside every group from the sub-root, along the ranks
+// in their order (1) or in the order of ring 0 of the 8-device topology (2; PrepareScatterRingSliceData :115-131 puts
+// the blocks in that order).
 int orc_scatter_two_level(uint32_t servers, uint32_t p, const void *inRoot, void **out, uint64_t count, int dt,
-    uint32_t root, uint64_t cclBytes, uint64_t align, int flags, int threads, uint64_t *touched)
+    uint32_t root, uint64_t cclBytes, uint64_t align, int flags, int threads, uint64_t *touched, int level0)
 {
     const uint64_t unit = DtSize(dt);
-    if (unit == 0 || p == 0 || root >= p || servers == 0 || p % servers != 0 || align == 0) {
+    if (unit == 0 || p == 0 || root >= p || servers == 0 || p % servers != 0 || align == 0 || level0 < 0 || level0 > 2 ||
+        (level0 == 2 && p / servers != 8)) {
         return -20;
     }
     const uint64_t maxPer = cclBytes / p / align * align / unit;
@@ -3640,7 +3645,35 @@ int orc_scatter_two_level(uint32_t servers, uint32_t p, const void *inRoot, void
             for (uint32_t d = 0; d < D; d++) {
                 m.buf[B_IN][d] = m.buf[B_OUT][d] = stage[g * D + d].data() + cb * D * g;
             }
-            for (uint32_t d = 0; d < D; d++) {
+            if (level0 != 0) {
+                // machine rank i = ring position i = device order(i); block of a device at cb * device
+                auto order = [&](uint32_t i) { return level0 == 2 ? kEightDeviceRings[0][i] : i; };
+                uint32_t rootPos = 0;
+                for (uint32_t i = 0; i < D; i++) {
+                    m.buf[B_IN][i] = m.buf[B_OUT][i] = stage[g * D + order(i)].data() + cb * D * g;
+                    rootPos = order(i) == rootLocal ? i : rootPos;
+                }
+                for (uint32_t r = 0; r < D; r++) {
+                    Proc pr;
+                    pr.rank = r;
+                    const int lft = static_cast<int>((r + D - 1) % D), rgt = static_cast<int>((r + 1) % D);
+                    if (r == rootPos) {
+                        for (uint32_t i = 1; i < D; i++) {
+                            pr.prog.push_back(MkSend(rgt, 0, B_IN, cb * order((r + D - i) % D), cb));
+                        }
+                    } else {
+                        const uint32_t rounds = (rootPos + D - r) % D;
+                        for (uint32_t i = 1; i <= rounds; i++) {
+                            if (i != 1) {
+                                pr.prog.push_back(MkSend(rgt, 0, B_OUT, cb * order((r + rounds - i + 1) % D), cb));
+                            }
+                            pr.prog.push_back(MkRecvCopy(lft, 0, B_OUT, cb * order((r + rounds - i) % D), cb));
+                        }
+                    }
+                    m.procs.push_back(std::move(pr));
+                }
+            }
+            for (uint32_t d = 0; d < D && level0 == 0; d++) {
                 Proc pr;
                 pr.rank = d;
                 if (d == rootLocal) {

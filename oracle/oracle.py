@@ -92,7 +92,7 @@ def lib():
         L.orc_scatter.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
         L.orc_scatter_ring.argtypes = [u32, vp, ctypes.POINTER(vp), u64, i32, u32, i32, i32]
         L.orc_scatter_ring.restype = i32
-        L.orc_scatter_two_level.argtypes = [u32, u32, vp, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32, ctypes.POINTER(u64)]
+        L.orc_scatter_two_level.argtypes = [u32, u32, vp, ctypes.POINTER(vp), u64, i32, u32, u64, u64, i32, i32, ctypes.POINTER(u64), i32]
         L.orc_scatter_two_level.restype = i32
         L.orc_alltoallv.argtypes = [u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, u64, i32, i32]
         L.orc_alltoallv_staged.argtypes = [u32, u32, ctypes.POINTER(vp), pu64, pu64, ctypes.POINTER(vp), pu64, pu64, i32, i32, i32]
@@ -430,14 +430,15 @@ def scatter(src, p, dt, root, flags=0, threads=1, algo=MESH):
 
 
 def scatter_two_level(src, p, dt, root, servers, ccl_bytes=DEFAULT_CCL_BYTES, align=DEFAULT_ALIGN, flags=0, threads=1,
-                      return_touched=False):
+                      return_touched=False, level0="mesh"):
     """`servers` groups of consecutive ranks: ring scatter of the groups' runs among the ranks at the root's position,
-    then mesh scatter inside every group from that rank, under the staging buffer's chunk loop."""
+    then inside every group from that rank the mesh scatter, or the ring scatter along the ranks in their order ("ring")
+    or in the order of ring 0 of the 8-device topology ("ring4"), under the staging buffer's chunk loop."""
     n = src.size // p
     outs = [np.empty(n, dtype=src.dtype) for _ in range(p)]
     touched = ctypes.c_uint64(0)
     rc = lib().orc_scatter_two_level(servers, p, src.ctypes.data, _ptrs(outs), n, dt, root, ccl_bytes, align, flags, threads,
-                                     ctypes.byref(touched))
+                                     ctypes.byref(touched), {"mesh": 0, "ring": 1, "ring4": 2}[level0])
     if rc != 0:
         raise RuntimeError("oracle two-level scatter failed rc=%d" % rc)
     return (outs, touched.value) if return_touched else outs

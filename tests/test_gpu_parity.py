@@ -839,17 +839,19 @@ def test_ring_scatter(orc):
 
 def test_two_level_scatter(orc):
     # scatter over several groups: a group's run of blocks goes round the ring of the ranks at the root's position,
-    # then each of those hands the ranks of its group their blocks; step by step the runs rest in the workspace
+    # then each of those hands the ranks of its group their blocks (mesh), or sends them round the group's ring (rank
+    # order, or ring 0 of the 8-device topology); step by step the runs rest in the workspace
     n = 30011
-    for servers, D in ((2, 4), (3, 4), (4, 2), (5, 1)):
+    for servers, D, level0 in ((2, 4, "mesh"), (3, 4, "mesh"), (4, 2, "mesh"), (5, 1, "mesh"), (2, 4, "ring"), (3, 3, "ring"),
+                               (2, 8, "ring4")):
         p = servers * D
         for fuse in (1, 0):
-            g = gh.Group(p, servers=servers, fuse=fuse)
+            g = gh.Group(p, servers=servers, fuse=fuse, level0=level0)
             try:
                 for root in sorted({0, p - 1, (D + 1) % p}):
-                    print("two-level scatter", servers, D, "fuse", fuse, "root", root, flush=True)
+                    print("two-level scatter", servers, D, level0, "fuse", fuse, "root", root, flush=True)
                     src = (np.arange(n * p, dtype=np.int64) * 2654435761 % (1 << 31)).astype(np.int32)
-                    want, touched = orc.scatter_two_level(src, p, INT32, root, servers, return_touched=True)
+                    want, touched = orc.scatter_two_level(src, p, INT32, root, servers, return_touched=True, level0=level0)
                     sends = [gh.to_dev(src) if r == root else None for r in range(p)]
                     recvs = [gh.empty_dev(n * 4) for _ in range(p)]
                     torch.cuda.synchronize()
@@ -863,10 +865,10 @@ def test_two_level_scatter(orc):
                     else:
                         # what the launches wrote = what the checker's ranks moved, less the root's packing and the
                         # stop in the receivers' staging buffers (p - servers blocks), which the hand-over skips
-                        assert info["launches"] == servers
+                        assert info["launches"] == (servers if level0 == "mesh" else servers - 1 + D - 1)
                         assert info["bytesWritten"] == touched // 2 - (2 * p - servers) * n * 4
                     for r in range(p):
-                        assert np.array_equal(gh.to_host(recvs[r], INT32), want[r]), ("two-level scatter", servers, D, fuse, root, r)
+                        assert np.array_equal(gh.to_host(recvs[r], INT32), want[r]), ("two-level scatter", servers, D, level0, fuse, root, r)
                     assert np.array_equal(gh.to_host(sends[root], INT32), src)
             finally:
                 g.close()

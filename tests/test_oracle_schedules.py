@@ -873,6 +873,30 @@ def test_two_level_scatter_delivers_and_moves_the_closed_form_bytes(orc, shape):
                 assert touched == 2 * moved, (shape, dt, n, root, ccl)
 
 
+@pytest.mark.parametrize("shape", [(2, 4, "ring"), (3, 3, "ring"), (4, 2, "ring"), (1, 5, "ring"), (2, 8, "ring4"), (3, 8, "ring4")])
+def test_two_level_scatter_with_rings_inside_delivers_and_moves_the_closed_form_bytes(orc, shape):
+    # As above, but inside a group the blocks go round the ring from the sub-root: the block of the rank j positions
+    # behind it makes j hops, D (D - 1) / 2 block hops per group where the mesh hands out D - 1.
+    servers, D, level0 = shape
+    p = servers * D
+    for dt, n in ((INT32, 1), (INT32, 1000), (INT8, 10003)):
+        unit = orc.dtype_size(dt)
+        for root in sorted({0, p - 1, p // 2, D - 1, min(D, p - 1)}):
+            for ccl in (200 << 20, 8192):
+                src = _inputs(dt, 1, n * p, root + n)[0]
+                outs, touched = orc.scatter_two_level(src, p, dt, root, servers, ccl_bytes=ccl, return_touched=True, level0=level0)
+                for r in range(p):
+                    assert np.array_equal(outs[r], src[r * n:(r + 1) * n]), (shape, dt, n, root, ccl, r)
+                max_per = ccl // p // 128 * 128 // unit
+                moved, left = 0, n
+                while left > 0:
+                    cur = max_per if left * unit * p > ccl else left
+                    block = cur * unit
+                    moved += 2 * p * block + (servers * (servers - 1) // 2) * D * block + servers * (D * (D - 1) // 2) * block
+                    left -= cur
+                assert touched == 2 * moved, (shape, dt, n, root, ccl)
+
+
 PRUNED_PORTS = ([0], [5], [0, 4], [2, 3], [1, 6], [0, 2, 4, 6], [1, 2, 3, 7], [4, 5, 6, 7])
 
 

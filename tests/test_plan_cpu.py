@@ -1000,6 +1000,41 @@ def test_two_level_scatter_plan(orc, servers, D):
         assert sum(it["n"] for it in plan["fused"]) == n * 4 * p          # fused: every block moves once
 
 
+@pytest.mark.parametrize("servers,D,level0", [(2, 4, "ring"), (3, 3, "ring"), (4, 2, "ring"), (2, 8, "ring4"), (3, 8, "ring4")])
+def test_two_level_scatter_with_rings_inside_plan(orc, servers, D, level0):
+    # level 1 as the mesh variant; inside a group a block only moves from a rank to the next one of the ring (rank order,
+    # or ring 0 of the 8-device topology), starting at the rank at the root's position
+    p = servers * D
+    n = 1003
+    rng = np.random.default_rng(660 + p)
+    order = list(cf.EIGHT_DEVICE_RINGS[0]) if level0 == "ring4" else list(range(D))
+    nexts = {(order[i], order[(i + 1) % D]) for i in range(D)}
+    bit = (1 << 29) if level0 == "ring" else (1 << 30)
+    for root in sorted({0, p - 1, (D + 1) % p}):
+        src = rng.integers(0, 1 << 30, n * p).astype(np.int32)
+        plan = H.describe_plan(H.COLL_SCATTER, root | (servers << 21) | bit, p, n, INT32)
+        assert len(plan["phases"]) == (servers - 1) + (D - 1)
+        inside = 0
+        for k, ph in enumerate(plan["phases"]):
+            for st in ph:
+                a, d = st["a"][0], st["dst"][0]
+                if k < servers - 1 and a // D != d // D:
+                    assert a % D == d % D == root % D and d // D == (a // D + 1) % servers
+                elif a != d:
+                    assert a // D == d // D and (a % D, d % D) in nexts, (servers, D, level0, root, a, d)
+                    inside += 1
+        assert inside == servers * D * (D - 1) // 2
+        want, touched = orc.scatter_two_level(src, p, INT32, root, servers, return_touched=True, level0=level0)
+        assert plan["stepWritten"] == touched // 2 - (2 * p - servers) * n * 4, (servers, D, level0, root)
+        for fused in (False, True):
+            sends = [src.view(np.uint8).copy() if r == root else np.zeros(0, np.uint8) for r in range(p)]
+            recvs = [np.zeros(n * 4, np.uint8) for _ in range(p)]
+            (plan_interp.run_fused if fused else plan_interp.run_steps)(plan, sends, recvs, INT32, 0)
+            for r in range(p):
+                assert np.array_equal(recvs[r].view(np.int32), want[r]), (servers, D, level0, root, fused, r)
+        assert sum(it["n"] for it in plan["fused"]) == n * 4 * p          # fused: every block moves once
+
+
 PRUNED_PORTS = ([0], [5], [0, 4], [2, 3], [1, 6], [0, 2, 4, 6], [1, 2, 3, 7], [4, 5, 6, 7])
 
 
