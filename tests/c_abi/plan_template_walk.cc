@@ -143,13 +143,18 @@ int main(int argc, char **argv)
                 shouldRefuse = kind >= 8;
             } else {
                 const uint64_t kind = Below(10);
-                const uint64_t chunk = base.cclBytes / base.unit;
+                // one chunk of the executor's loop: the CCL buffer holds a count, or one block per rank
+                const bool perRank = base.coll == COLL_REDUCESCATTER || base.coll == COLL_ALLGATHER;
+                const uint64_t chunk = std::max<uint64_t>(1, base.cclBytes / base.unit / (perRank ? base.p : 1));
                 rq.count = kind < 4 ? (1 + Below(9)) * regular                       // whole slices
                     : kind < 7 ? (1 + Below(9)) * regular + 1 + Below(regular - 1)   // a ragged last slice
                     : kind < 8 ? 1 + Below(40)                                        // a few elements
                     : chunk + Below(2 * chunk);                                       // several chunks of the CCL buffer
                 if (rq.count > (96ull << 20)) {
                     rq.count = (96ull << 20) + Below(1000);        // keep the plans of many-rank requests small enough to compare
+                }
+                if (rq.count > 6 * chunk) {
+                    rq.count = 6 * chunk - Below(std::min<uint64_t>(chunk, 1000));   // and at most six rounds of the chunk loop
                 }
             }
             std::string err;
