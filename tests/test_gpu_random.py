@@ -182,8 +182,10 @@ def test_random_reducescatter_and_reduce_on_rank_groups(orc, seed):
     # two-level reduce-scatter and rooted reduce: random group shapes, types, sizes, misaligned buffers, both issue modes
     rng = np.random.default_rng(9400 + SEED_SHIFT + seed)
     for case in range(8):
-        p = int(rng.choice([4, 6, 8, 12, 16]))
+        p = int(rng.choice([4, 6, 8, 12, 16, 16, 24, 32]))
         servers = int(rng.choice([s for s in range(2, p + 1) if p % s == 0]))
+        if p >= 16 and p % 8 == 0 and int(rng.integers(0, 2)):
+            servers = p // 8                                  # servers of 8 devices: the four-ring topology is allowed
         level1 = int(rng.choice([RING, RHD]))
         det = int(rng.integers(0, 2))
         dt = int(rng.choice(ALL_TYPES))
@@ -201,7 +203,15 @@ def test_random_reducescatter_and_reduce_on_rank_groups(orc, seed):
         try:
             ins = [cf.random_input(dt, n * p, rng) for _ in range(p)]
             g.set(level0=level0)
-            want = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, atomic=atomic, level0=level0)
+            # four rings inside, a ring between the servers: on some cases only a few devices of a server have a network port
+            nic = ([[0, 4], [5], [1, 2, 3, 7], None][int(rng.integers(0, 4))]
+                   if level0 == "ring4" and level1 == RING and servers > 1 else None)
+            if nic is not None:
+                print("    network ports on devices", nic, flush=True)
+                g.set(nic_ranks=",".join(str(d) for d in nic))
+                want = orc.reducescatter_two_level_pruned([x.copy() for x in ins], dt, op, servers, nic)
+            else:
+                want = orc.reducescatter_two_level(ins, dt, op, servers, level1=level1, atomic=atomic, level0=level0)
             sends = [gh.to_dev(x, pad) for x in ins]
             recvs = [gh.empty_dev(n * unit, pad if r % 2 else 0) for r in range(p)]
             torch.cuda.synchronize()
@@ -210,6 +220,8 @@ def test_random_reducescatter_and_reduce_on_rank_groups(orc, seed):
             for r in range(p):
                 assert gh.same(dt, gh.to_host(recvs[r], dt), want[r]), (seed, case, "reduce-scatter", r)
                 assert np.array_equal(gh.to_host(sends[r], dt), ins[r]), (seed, case, "send buffer changed", r)
+            if nic is not None:
+                g.set(nic_ranks="all")
             want_root = orc.reduce_to_root_two_level(ins, dt, op, root, servers, level1=level1, atomic=atomic, level0=level0)
             outs = [gh.empty_dev(n * p * unit, 0 if r % 2 else pad, fill=0x33) for r in range(p)]
             torch.cuda.synchronize()
@@ -274,6 +286,44 @@ def test_random_alltoallv_flat_and_staged(orc, seed):
             g.close()
 
 
+@pytest.mark.parametrize("seed", range(2))
+def test_random_two_level_reducescatter_with_random_network_ports(orc, seed):
+    """Servers of 8 devices with four rings inside and a ring between them, 1, 2, 4 or all 8 devices of every server with a
+    network port, chosen at random: the branch that all-reduces inside a server first, against the checker, on random
+    types, reductions, counts, staging-buffer sizes and both issue modes."""
+    rng = np.random.default_rng(9700 + SEED_SHIFT + seed)
+    for case in range(6):
+        servers = int(rng.choice([2, 2, 3, 4]))
+        p = servers * 8
+        ports = int(rng.choice([1, 2, 4, 8]))
+        nic = sorted(int(d) for d in rng.choice(8, size=ports, replace=False))
+        dt = int(rng.choice(ALL_TYPES))
+        op = int(rng.integers(0, 4))
+        n = max(1, _size(rng) // (4 * p))
+        fuse = int(rng.integers(0, 2))
+        ccl = int(rng.choice([200 << 20, 1 << 18]))
+        unit = H.DTYPE_SIZE[dt]
+        pad = int(rng.choice([0, unit, 16]))
+        print("random pruned two-level seed", seed, "case", case, "servers", servers, "ports", nic, "type", dt, "op", op, "n", n,
+              "fuse", fuse, "buffer", ccl, "pad", pad, flush=True)
+        g = gh.Group(p, algo="ring", servers=servers, level0="ring4", fuse=fuse, buffsize_bytes=ccl)
+        try:
+            g.set(nic_ranks=",".join(str(d) for d in nic))
+            ins = [cf.random_input(dt, n * p, rng) for _ in range(p)]
+            want = (orc.reducescatter_two_level_pruned([x.copy() for x in ins], dt, op, servers, nic, ccl_bytes=ccl) if ports < 8
+                    else orc.reducescatter_two_level(ins, dt, op, servers, level1=RING, level0="ring4", ccl_bytes=ccl))
+            sends = [gh.to_dev(x, pad) for x in ins]
+            recvs = [gh.empty_dev(n * unit, pad if r % 2 else 0) for r in range(p)]
+            torch.cuda.synchronize()
+            H.reduce_scatter(g.comms, [t.data_ptr() for t in sends], [t.data_ptr() for t in recvs], n, dt, op, g.stream_ptr)
+            g.stream.synchronize()
+            for r in range(p):
+                assert gh.same(dt, gh.to_host(recvs[r], dt), want[r]), (seed, case, r)
+                assert np.array_equal(gh.to_host(sends[r], dt), ins[r]), (seed, case, "send buffer changed", r)
+        finally:
+            g.close()
+
+
 @pytest.mark.parametrize("seed", range(3))
 def test_random_scatter_and_broadcast_over_rank_groups(orc, seed):
     """Scatter and broadcast with random roots, rank groups and schedule settings (auto, ring, star, ...): whatever the route,
@@ -288,10 +338,12 @@ def test_random_scatter_and_broadcast_over_rank_groups(orc, seed):
         fuse = int(rng.integers(0, 2))
         root = int(rng.integers(0, p))
         ccl = int(rng.choice([200 << 20, 1 << 16]))
-        print("random scatter / broadcast seed", seed, "case", case, "p", p, "servers", servers, "algo", setting, "type", dt,
+        level0 = str(rng.choice(["mesh", "ring", "ring4"] if p // servers == 8 else ["mesh", "ring"]))
+        print("random scatter / broadcast seed", seed, "case", case, "p", p, "servers", servers, level0, "algo", setting, "type", dt,
               "n", n, "fuse", fuse, "root", root, "buffer", ccl, flush=True)
         g = gh.Group(p, algo=setting, fuse=fuse, servers=servers, buffsize_bytes=ccl)
         try:
+            g.set(level0=level0)
             src = cf.random_input(dt, n * p, rng)
             sends = [gh.to_dev(src) if r == root else None for r in range(p)]
             recvs = [gh.empty_dev(n * H.DTYPE_SIZE[dt], fill=0x33) for _ in range(p)]
