@@ -6,8 +6,10 @@
 // a time (measured on MI355X, 8 x 256 MiB read and 8 x 256 MiB written: 5.3 - 5.6 TB/s with reads and writes
 // interleaved per workgroup, 5.9 - 6.0 TB/s when the 32 workgroups of an XCD read together and then write together;
 // 1 read : 8 writes 4.9 against 5.9 TB/s).  So here the workgroups of one XCD form a team:
-//   read phase   every workgroup evaluates up to kTeamTiles tiles (a run of consecutive tiles; the team's runs follow
-//                each other, so an XCD works on one contiguous stretch of the tile space) and parks the results in LDS
+//   read phase   every workgroup evaluates up to kTeamTiles tiles (every 32nd tile of the team's region, so an XCD
+//                works on one contiguous stretch of the tile space) and parks the results in LDS.  A round of whole
+//                tiles of one item is read with all its loads issued together (a copy) or source by source with the
+//                partial results in LDS (a chain), see Round() below
 //   barrier      among the team's workgroups only; the other XCDs run on, in whatever phase they are
 //   write phase  every workgroup writes its parked tiles to their destinations, destination by destination
 // Workgroup b belongs to XCD b % 8 (workgroups are dealt to the XCDs round robin).  If they are not, or if the team is
@@ -191,7 +193,35 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
         FusedDesc d;
         uint32_t dEnd = 0;
         Eval eval;
-        for (uint32_t q = 0; q < n; q++) {
+        bool bySource = false;
+        if constexpr (Eval::kBySource) {
+            // All the round's tiles whole, vector-aligned and of one item: the team reads source by source (see
+            // TeamChainEval::Round).
+            if (n == kTeamTiles || n == kTeamTiles / 2) {
+                idx = ItemOfTile(items, nitems, first, tilesPerItem);
+                d = items[idx];
+                dEnd = d.tile0 + uint32_t((d.bytes + kTileBytes - 1) / kTileBytes);
+                const uint32_t lastTile = first + (n - 1) * teamSize;
+                bySource = d.mode == ACC_VEC16 && d.nsrc >= Eval::kRoundMinSrc && lastTile < dEnd &&
+                    uint64_t(lastTile - d.tile0 + 1) * kTileBytes <= d.bytes;
+            }
+            if (bySource) {
+                const uint64_t off = uint64_t(first - d.tile0) * kTileBytes;
+                const uint64_t stride = uint64_t(teamSize) * kTileBytes;
+                if (n == kTeamTiles) {
+                    Eval::template Round<kTeamTiles>(d, srcPool + d.srcBase, off, stride, park, slots + round, &seen);
+                } else {
+                    Eval::template Round<kTeamTiles / 2>(d, srcPool + d.srcBase, off, stride, park, slots + round, &seen);
+                }
+                maxDst = d.ndst;
+                if (threadIdx.x < n) {
+                    heldItem[threadIdx.x] = idx;
+                    heldTile[threadIdx.x] = first + threadIdx.x * teamSize;
+                    heldVec[threadIdx.x] = kTeamVecPerTile;
+                }
+            }
+        }
+        for (uint32_t q = 0; q < n && !bySource; q++) {
             const uint32_t tile = first + q * teamSize;
             if (q + 1 == n && threadIdx.x == 0) {
                 // a look at the slot of the next round, in flight together with the last tile's loads: a workgroup
@@ -263,6 +293,100 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
 
 // ---- what a tile's value is, per kernel family --------------------------------------------------------------------
 template <typename T, int OP> struct TeamChainEval {
+    static constexpr bool kBySource = true;
+    static constexpr uint32_t kRoundMinSrc = 2;
+    // A whole round at once: N whole tiles of one item, `stride` bytes apart from `off` on.  The team reads source by
+    // source -- at any moment its loads go to one stretch of N x 32 tiles of one buffer instead of 32 tiles of each of
+    // the item's buffers -- and the partial results rest in LDS, folded in the chain's order, so the bits are those of
+    // the tile-by-tile evaluation.  Two register sets of N x 4 vectors: while one source is folded, the next one's
+    // loads are in flight, and the one after that is requested as soon as the fold has freed its set (8 ranks x
+    // 256 MiB, stand-alone: 691 us this way, 770 us with one set, 705 us tile by tile).
+    // Straight-line code for a source count fixed at compile time, in which every wait is for exactly the loads it
+    // needs, measured the same and takes three times as long to build.
+    // `peek` is looked at (thread 0, into *seen) once the last loads are on their way.
+    template <uint32_t N>
+    static __device__ __forceinline__ void LoadSet(V4 (&v)[N][kVecPerLane], const void *base, uint64_t off, uint64_t stride)
+    {
+        const char *s = static_cast<const char *>(base) + off;
+#pragma unroll
+        for (uint32_t q = 0; q < N; q++) {
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerLane; u++) {
+                v[q][u] = Load16<ACC_VEC16>(s + q * stride + uint64_t(u) * kBlockThreads * 16, threadIdx.x * 16u);
+            }
+        }
+    }
+    // Source j into the partial results: source 0 starts them.  A tile's partial results are fetched from LDS together,
+    // so that their latencies overlap.
+    template <uint32_t N>
+    static __device__ __forceinline__ void FoldSet(const V4 (&v)[N][kVecPerLane], const FusedDesc &d, uint32_t j, LdsV4 *park)
+    {
+        const uint32_t tid = threadIdx.x;
+        if (j == 0) {
+#pragma unroll
+            for (uint32_t q = 0; q < N; q++) {
+#pragma unroll
+                for (uint32_t u = 0; u < kVecPerLane; u++) {
+                    park[q * kTeamVecPerTile + u * kBlockThreads + tid] = v[q][u];
+                }
+            }
+            return;
+        }
+        const bool accLeft = OrderMatters<T, OP>::value && ((d.accLeftMask >> j) & 1ull);
+#pragma unroll
+        for (uint32_t q = 0; q < N; q++) {
+            V4 a[kVecPerLane];
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerLane; u++) {
+                a[u] = park[q * kTeamVecPerTile + u * kBlockThreads + tid];
+            }
+            if (accLeft) {      // the same for the whole wave
+#pragma unroll
+                for (uint32_t u = 0; u < kVecPerLane; u++) {
+                    a[u] = Combine16<T, OP>(a[u], v[q][u]);
+                }
+            } else {
+#pragma unroll
+                for (uint32_t u = 0; u < kVecPerLane; u++) {
+                    a[u] = Combine16<T, OP>(v[q][u], a[u]);
+                }
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerLane; u++) {
+                park[q * kTeamVecPerTile + u * kBlockThreads + tid] = a[u];
+            }
+        }
+    }
+    template <uint32_t N>
+    static __device__ __forceinline__ void Round(const FusedDesc &d, const void *const *__restrict__ src, uint64_t off,
+        uint64_t stride, LdsV4 *park, const uint32_t *peek, uint32_t *seen)
+    {
+        const uint32_t nsrc = d.nsrc;
+        V4 va[N][kVecPerLane], vb[N][kVecPerLane];
+        LoadSet<N>(va, src[0], off, stride);
+        LoadSet<N>(vb, src[1], off, stride);
+        uint32_t j = 0;
+#pragma nounroll
+        for (; j + 4 <= nsrc; j += 2) {
+            FoldSet<N>(va, d, j, park);
+            LoadSet<N>(va, src[j + 2], off, stride);
+            FoldSet<N>(vb, d, j + 1, park);
+            LoadSet<N>(vb, src[j + 3], off, stride);
+        }
+        // two or three sources left, the first two of them loaded or on their way
+        const bool three = nsrc - j == 3;
+        FoldSet<N>(va, d, j, park);
+        if (three) {
+            LoadSet<N>(va, src[j + 2], off, stride);
+        }
+        if (threadIdx.x == 0) {
+            *seen = TeamLoad(peek);
+        }
+        FoldSet<N>(vb, d, j + 1, park);
+        if (three) {
+            FoldSet<N>(va, d, j + 2, park);
+        }
+    }
     // Up to kChainSrcBatch source pointers are kept in registers from tile to tile: fetched per tile they are a chain
     // of dependent loads in front of the tile's data, with nothing else on the CU to hide it.
     const void *sp[kChainSrcBatch];
@@ -313,6 +437,35 @@ template <typename T, int OP> struct TeamChainEval {
 };
 
 struct TeamCopyEval {
+    static constexpr bool kBySource = true;
+    static constexpr uint32_t kRoundMinSrc = 1;
+    // A whole round at once (see TeamChainEval::Round): the loads of all N tiles are issued before the first of them is
+    // parked, instead of tile after tile with an LDS write between them.
+    template <uint32_t N>
+    static __device__ __forceinline__ void Round(const FusedDesc &, const void *const *__restrict__ src, uint64_t off,
+        uint64_t stride, LdsV4 *park, const uint32_t *peek, uint32_t *seen)
+    {
+        const uint32_t tid = threadIdx.x;
+        const char *s = static_cast<const char *>(src[0]) + off;
+        V4 v[N][kVecPerLane];
+#pragma unroll
+        for (uint32_t q = 0; q < N; q++) {
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerLane; u++) {
+                v[q][u] = Load16<ACC_VEC16>(s + q * stride + uint64_t(u) * kBlockThreads * 16, tid * 16u);
+            }
+        }
+        if (tid == 0) {
+            *seen = TeamLoad(peek);
+        }
+#pragma unroll
+        for (uint32_t q = 0; q < N; q++) {
+#pragma unroll
+            for (uint32_t u = 0; u < kVecPerLane; u++) {
+                park[q * kTeamVecPerTile + u * kBlockThreads + tid] = v[q][u];
+            }
+        }
+    }
     const void *s;
     __device__ __forceinline__ void SetItem(const FusedDesc &d, const void *const *__restrict__ srcPool) { s = srcPool[d.srcBase]; }
     __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__, const void *, uint64_t off,
@@ -351,6 +504,7 @@ struct TeamCopyEval {
 };
 
 template <typename T, int OP> struct TeamTreeEval {
+    static constexpr bool kBySource = false;
     __device__ __forceinline__ void SetItem(const FusedDesc &, const void *const *__restrict__) {}
     __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__ srcPool, const void *,
         uint64_t off, uint32_t nvec, LdsV4 *park) const
@@ -366,6 +520,7 @@ template <typename T, int OP> struct TeamTreeEval {
 
 // extra = the launch's op words (they follow the item table)
 template <typename T, int OP> struct TeamStackEval {
+    static constexpr bool kBySource = false;
     __device__ __forceinline__ void SetItem(const FusedDesc &, const void *const *__restrict__) {}
     __device__ __forceinline__ void Vec(const FusedDesc &d, const void *const *__restrict__ srcPool, const void *extra,
         uint64_t off, uint32_t nvec, LdsV4 *park) const

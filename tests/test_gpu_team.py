@@ -68,6 +68,41 @@ def test_team_chain_in_place_and_unaligned(orc):
         g.close()
 
 
+def test_team_chain_whole_rounds_read_source_by_source(orc):
+    # Slices of 4 MiB and more: a workgroup's round is then 8 (in the tail of regions 4) whole tiles of one item, and
+    # the chain kernel reads such a round source by source with the partial results in LDS.  Even and odd numbers of
+    # sources, 2 and 3 of them, more than 8; element widths of 1 to 8 bytes; float max / min over NaNs with payloads,
+    # signed zeros, infinities and denormals, where a swapped operand in any fold changes the bits; in place.
+    specials = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.0, -1.0, 3.4e38], np.float32)
+    nan2 = np.array([0x7fc00001, 0xffc00002, 0x7fa00003], np.uint32).view(np.float32)
+    pool = np.concatenate([specials, nan2])
+    mib = 1 << 20
+    for p, dt, op, slice_bytes, special, in_place in ((8, FP32, MAX, 8 * mib, True, False), (8, FP32, MIN, 4 * mib, True, True),
+                                                      (7, FP16, SUM, 8 * mib, False, False), (5, INT8, SUM, 8 * mib, False, False),
+                                                      (4, INT64, PROD, 8 * mib, False, False), (16, FP32, SUM, 4 * mib, False, False),
+                                                      (3, BF16, MIN, 8 * mib, False, True), (2, FP32, MAX, 16 * mib, True, False),
+                                                      (6, BF16, SUM, 8 * mib, False, False)):
+        n = p * slice_bytes // H.DTYPE_SIZE[dt]
+        rng = np.random.default_rng(7300 + p + dt)
+        print("team chain by source p", p, "type", dt, "op", op, "slice", slice_bytes, "specials", special, "in place", in_place, flush=True)
+        ins = [rng.choice(pool, n).astype(np.float32) if special else cf.random_input(dt, n, rng) for _ in range(p)]
+        want = orc.allreduce([x.copy() for x in ins], dt, op, threads=8)
+        g = gh.Group(p, algo="ring", team=1)
+        try:
+            for rep in range(2):
+                outs, keep = gh.all_reduce(g, ins, dt, op, in_place=in_place)
+                info = g.info()
+                assert info["fused"] == 1 and info["teamLaunches"] >= 1, info
+                for r in range(p):
+                    if special:
+                        assert np.array_equal(outs[r].view(np.uint32), want[r].view(np.uint32)), (p, dt, op, rep, r)
+                    else:
+                        assert gh.same(dt, outs[r], want[r]), (p, dt, op, rep, r)
+                    assert in_place or np.array_equal(keep[r].view(np.uint8), ins[r].view(np.uint8))
+        finally:
+            g.close()
+
+
 @pytest.mark.parametrize("algo", [MESH, RHD])
 def test_team_mesh_and_tree_allreduce(orc, algo):
     # the halving-doubling schedule fuses into trees (TeamTreeKernel), with a fold for rank counts that are no power of
@@ -111,7 +146,8 @@ def test_team_copy_allgather_and_broadcast(orc):
     p = 8
     g = gh.Group(p, algo="ring", team=1)
     try:
-        for dt, n, pad in ((INT32, 1000003, 0), (INT8, 5 * 1024 * 1024 + 1, 0), (BF16, 700001, 6)):
+        # (the 16 MiB blocks give rounds of 8 whole tiles, which are read with all their loads issued at once)
+        for dt, n, pad in ((INT32, 1000003, 0), (INT8, 5 * 1024 * 1024 + 1, 0), (BF16, 700001, 6), (INT32, 4 * 1024 * 1024, 0)):
             print("team copy all-gather", dt, n, pad, flush=True)
             ins = _ins(dt, p, n, 7400 + dt)
             outs = gh.all_gather(g, ins, dt, pad=pad)
@@ -119,15 +155,16 @@ def test_team_copy_allgather_and_broadcast(orc):
             whole = np.concatenate(ins)
             for r in range(p):
                 assert np.array_equal(outs[r], whole), (dt, n, r)
-        n, root = 3 * 1024 * 1024 + 9, 5
-        bufs_np = _ins(INT32, p, n, 7450)
-        bufs = [gh.to_dev(x) for x in bufs_np]
-        torch.cuda.synchronize()
-        H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, INT32, root, g.stream_ptr)
-        g.stream.synchronize()
-        assert g.info()["teamLaunches"] >= 1
-        for r in range(p):
-            assert np.array_equal(gh.to_host(bufs[r], INT32), bufs_np[root]), r
+        for n, root in ((3 * 1024 * 1024 + 9, 5), (16 * 1024 * 1024, 2)):
+            print("team copy broadcast", n, root, flush=True)
+            bufs_np = _ins(INT32, p, n, 7450)
+            bufs = [gh.to_dev(x) for x in bufs_np]
+            torch.cuda.synchronize()
+            H.broadcast(g.comms, [t.data_ptr() for t in bufs], n, INT32, root, g.stream_ptr)
+            g.stream.synchronize()
+            assert g.info()["teamLaunches"] >= 1
+            for r in range(p):
+                assert np.array_equal(gh.to_host(bufs[r], INT32), bufs_np[root]), r
     finally:
         g.close()
 
