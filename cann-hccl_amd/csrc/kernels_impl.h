@@ -1136,6 +1136,11 @@ constexpr uint32_t kStackVecShallow = 4;
 constexpr uint32_t kStackVecDeep = 2;
 constexpr uint32_t kStackShallowDepth = 4;
 constexpr uint32_t kStackSrcBatch = 8;
+// The plain kernel issues the loads of 4 sources together: with 8 it needs every register a wave can have, one
+// workgroup fits a CU and nothing hides the table look-ups between its tiles (two-level reduce-scatter of 8 x 256 MiB
+// 426 -> 417 us, reduce 434 -> 415 us, all-reduce of 8 x 16 MiB 52 -> 47 us).  The team form, one workgroup per CU by
+// its LDS, keeps 8.
+constexpr uint32_t kStackPlainBatch = 4;
 
 template <uint32_t U> struct StackVal {
     V4 x[U];
@@ -1182,7 +1187,7 @@ template <uint32_t U> struct StackVal {
         }                                 \
     }
 
-template <typename T, int OP, uint32_t MODE, bool FULL, bool DEEP, bool PARK = false>
+template <typename T, int OP, uint32_t MODE, bool FULL, bool DEEP, bool PARK = false, uint32_t BATCH = kStackSrcBatch>
 __device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *const *__restrict__ src,
     const uint32_t *__restrict__ ops, void *const *__restrict__ dst, uint64_t off, uint32_t vecBase, uint32_t nvec,
     LdsV4 *park = nullptr)
@@ -1204,10 +1209,10 @@ __device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *con
     StackVal<U> b0 = top, b1 = top, b2 = top, b3 = top, b4 = top, b5 = top, b6 = top;
     uint32_t depth = 0;                  // values on the stack, the top one included
     const uint32_t nsrc = d.nsrc;
-    for (uint32_t j = 0; j < nsrc; j += kStackSrcBatch) {
-        StackVal<U> v[kStackSrcBatch];
+    for (uint32_t j = 0; j < nsrc; j += BATCH) {
+        StackVal<U> v[BATCH];
 #pragma unroll
-        for (uint32_t jj = 0; jj < kStackSrcBatch; jj++) {
+        for (uint32_t jj = 0; jj < BATCH; jj++) {
             if (j + jj < nsrc) {
                 const void *s = src[j + jj];
 #pragma unroll
@@ -1219,7 +1224,7 @@ __device__ __forceinline__ void StackVecPass(const FusedDesc &d, const void *con
             }
         }
 #pragma unroll
-        for (uint32_t jj = 0; jj < kStackSrcBatch; jj++) {
+        for (uint32_t jj = 0; jj < BATCH; jj++) {
             if (j + jj < nsrc) {
                 const uint32_t op = ops[j + jj];
                 if (depth > 0) {
@@ -1308,7 +1313,7 @@ __device__ __forceinline__ void StackElem(const FusedDesc &d, const void *const 
 }
 
 // All vector passes of one tile.
-template <typename T, int OP, bool PARK = false>
+template <typename T, int OP, bool PARK = false, uint32_t BATCH = kStackSrcBatch>
 __device__ __forceinline__ void StackTile(const FusedDesc &d, const void *const *__restrict__ src,
     const uint32_t *__restrict__ ops, void *const *__restrict__ dst, uint64_t off, uint32_t nvec, LdsV4 *park = nullptr)
 {
@@ -1318,18 +1323,18 @@ __device__ __forceinline__ void StackTile(const FusedDesc &d, const void *const 
         // d.nleaf: the stack depth the item needs
         if (d.nleaf <= kStackShallowDepth) {
             for (; base + kPassShallow <= nvec; base += kPassShallow) {
-                StackVecPass<T, OP, ACC_VEC16, true, false, PARK>(d, src, ops, dst, off, base, nvec, park);
+                StackVecPass<T, OP, ACC_VEC16, true, false, PARK, BATCH>(d, src, ops, dst, off, base, nvec, park);
             }
         }
         for (; base + kPassDeep <= nvec; base += kPassDeep) {
-            StackVecPass<T, OP, ACC_VEC16, true, true, PARK>(d, src, ops, dst, off, base, nvec, park);
+            StackVecPass<T, OP, ACC_VEC16, true, true, PARK, BATCH>(d, src, ops, dst, off, base, nvec, park);
         }
         if (base < nvec) {
-            StackVecPass<T, OP, ACC_VEC16, false, true, PARK>(d, src, ops, dst, off, base, nvec, park);
+            StackVecPass<T, OP, ACC_VEC16, false, true, PARK, BATCH>(d, src, ops, dst, off, base, nvec, park);
         }
     } else {
         for (; base < nvec; base += kPassDeep) {
-            StackVecPass<T, OP, ACC_VEC16_ANY, false, true, PARK>(d, src, ops, dst, off, base, nvec, park);
+            StackVecPass<T, OP, ACC_VEC16_ANY, false, true, PARK, BATCH>(d, src, ops, dst, off, base, nvec, park);
         }
     }
 }
@@ -1350,7 +1355,7 @@ __global__ void __launch_bounds__(kBlockThreads) StackKernel(const FusedDesc *__
         if (d.mode == ACC_ELEM) {
             StackElem<T, OP>(d, src, ops, dst, off, n);
         } else {
-            StackTile<T, OP>(d, src, ops, dst, off, n >> 4);
+            StackTile<T, OP, false, kStackPlainBatch>(d, src, ops, dst, off, n >> 4);
         }
     }
 }
