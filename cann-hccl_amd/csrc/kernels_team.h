@@ -292,8 +292,15 @@ __device__ __forceinline__ void TeamBody(const FusedDesc *__restrict__ items, ui
 }
 
 // ---- what a tile's value is, per kernel family --------------------------------------------------------------------
+// A bf16 combine is a dozen instructions per element pair (widen, combine, round); between a set's loads and the next
+// request for that set they cost more than the order of the reads gains (8 ranks x 256 MiB, source by source against
+// tile by tile: fp32 sum 0.708 / 0.719 ms, int32 0.705 / 0.720, int64 product 0.725 / 0.749, fp16 sum 0.716 / 0.720,
+// int8 the same, bf16 sum 0.737 / 0.734, bf16 max 0.762 / 0.753).
+template <typename T> struct ReadsBySource { static constexpr bool value = true; };
+template <> struct ReadsBySource<Bf16Bits> { static constexpr bool value = false; };
+
 template <typename T, int OP> struct TeamChainEval {
-    static constexpr bool kBySource = true;
+    static constexpr bool kBySource = ReadsBySource<T>::value;
     static constexpr uint32_t kRoundMinSrc = 2;
     // A whole round at once: N whole tiles of one item, `stride` bytes apart from `off` on.  The team reads source by
     // source -- at any moment its loads go to one stretch of N x 32 tiles of one buffer instead of 32 tiles of each of
