@@ -587,11 +587,13 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                     pl.rec.grid = g->numCu;
                     pl.rec.dynamicLds = kTeamDynamicLds;
                     // The regions the teams draw: roundTiles tiles per workgroup (fewer when that would leave an XCD
-                    // without a region); over the last quarter of the tiles the size is halved whenever fewer than 16
+                    // without a region); over the last quarter of the tiles the size is halved whenever fewer than 8
                     // regions of the current size are left.  The XCDs do not all move data at the same rate, and with
                     // regions that get smaller towards the end they finish together (measured, 8 x 256 MiB fp32
                     // all-reduce: 727 us with 64 equal regions dealt out in order, 714 us with the shrinking tail
-                    // drawn from the counter; shrinking earlier costs more than it brings, small regions run slower).
+                    // drawn from the counter; shrinking earlier costs more than it brings, small regions run slower --
+                    // the more so since rounds of 8 and 4 whole tiles are read in one piece: with "fewer than 16"
+                    // all-gather and broadcast took 2 % longer, the all-reduces 1 %).
                     const uint32_t perX = g->numCu / kTeamXcds;
                     std::vector<TeamRegion> regions;
                     uint32_t per = pl.rec.roundTiles;
@@ -601,7 +603,7 @@ HcclResult BuildTables(Group *g, Prepared *pp, bool reduceColl, int dtype, int o
                     for (uint32_t at = 0; at < tiles;) {
                         const uint32_t left = tiles - at;
                         if (uint64_t(at) * 4 >= uint64_t(tiles) * 3) {
-                            while (per > 1 && uint64_t(per) * perX * 16 > left) {
+                            while (per > 1 && uint64_t(per) * perX * 8 > left) {
                                 per /= 2;
                             }
                         }
